@@ -1,0 +1,340 @@
+"""Pins the CPU oracle against what the mathematics fixes, independently of its own formulas.
+
+Every check here uses a different formulation than the oracle's C code: exact rationals for the
+rounding modes, numpy int64 matmul for the GEMMs, python big ints for the integer softmax steps,
+closed forms / invariants / float references with explicit error bounds for the rest.
+"""
+
+import math
+from fractions import Fraction
+
+import numpy as np
+import pytest
+
+MODES = ['floor', 'ceil', 'positive_inf', 'negative_inf', 'symmetric_inf', 'symmetric_zero', 'conv_even',
+         'conv_odd']
+RANGE = {'int8': (-128, 127), 'uint8': (0, 255), 'int16': (-32768, 32767), 'int32': (-2**31, 2**31 - 1)}
+
+
+def exact_round(x: Fraction, mode: str) -> int:
+    """Textbook definition of each AIE rounding mode on an exact rational."""
+    lo = math.floor(x)
+    frac = x - lo
+    if mode == 'floor':
+        return lo
+    if mode == 'ceil':
+        return math.ceil(x)
+    if frac != Fraction(1, 2):
+        return lo + (1 if frac > Fraction(1, 2) else 0)
+    # exact tie between lo and lo+1
+    if mode == 'positive_inf':
+        return lo + 1
+    if mode == 'negative_inf':
+        return lo
+    if mode == 'symmetric_inf':
+        return lo + 1 if x > 0 else lo
+    if mode == 'symmetric_zero':
+        return lo if x > 0 else lo + 1
+    if mode == 'conv_even':
+        return lo if lo % 2 == 0 else lo + 1
+    if mode == 'conv_odd':
+        return lo if lo % 2 != 0 else lo + 1
+    raise AssertionError(mode)
+
+
+def exact_srs(acc: int, shift: int, mode: str, kind: str) -> int:
+    q = exact_round(Fraction(acc, 1 << shift), mode)
+    lo, hi = RANGE[kind]
+    return min(max(q, lo), hi)
+
+
+@pytest.mark.parametrize('mode', MODES)
+def test_srs_bruteforce_window(oracle, mode):
+    # every accumulator in a window around zero x every shift 0..12, plus extremes
+    accs = list(range(-1100, 1101)) + [2**31 - 1, -2**31, 2**31 - 2, -2**31 + 1, 2**30, -2**30, 12345678, -12345678]
+    for shift in list(range(0, 13)) + [15, 20, 31]:
+        for kind in ('int8', 'uint8', 'int16', 'int32'):
+            got = oracle.srs(np.array(accs), shift, mode, kind)
+            exp = [exact_srs(a, shift, mode, kind) for a in accs]
+            assert got.tolist() == exp, (mode, shift, kind)
+
+
+def test_srs_known_ties(oracle):
+    # 2.5 and -2.5 and 3.5 with shift 1
+    table = {
+        'floor': (2, -3, 3), 'ceil': (3, -2, 4), 'positive_inf': (3, -2, 4), 'negative_inf': (2, -3, 3),
+        'symmetric_inf': (3, -3, 4), 'symmetric_zero': (2, -2, 3), 'conv_even': (2, -2, 4),
+        'conv_odd': (3, -3, 3),
+    }
+    for mode, (p, n, q) in table.items():
+        assert oracle.srs(np.array([5, -5, 7]), 1, mode, 'int32').tolist() == [p, n, q], mode
+
+
+def _rng(seed):
+    return np.random.default_rng(seed)
+
+
+@pytest.mark.parametrize('a_dtype', [np.int8, np.uint8])
+@pytest.mark.parametrize('mode', ['floor', 'positive_inf', 'symmetric_inf', 'conv_even'])
+def test_dense_vs_int64_matmul(oracle, a_dtype, mode):
+    r = _rng(1)
+    M, K, N = 37, 83, 29
+    lo, hi = (0, 256) if a_dtype == np.uint8 else (-128, 128)
+    A = r.integers(lo, hi, (M, K)).astype(a_dtype)
+    W = r.integers(-128, 128, (K, N)).astype(np.int8)
+    bias = r.integers(-2**14, 2**14, N).astype(np.int32)
+    shifts = r.integers(4, 11, N).astype(np.int32)
+    acc = A.astype(np.int64) @ W.astype(np.int64) + bias
+    for relu in (False, True):
+        for out in ('int8', 'uint8', 'int16'):
+            exp = np.array([[exact_srs(int(acc[m, n]), int(shifts[n]), mode, out) for n in range(N)]
+                            for m in range(M)])
+            if relu:
+                exp = np.maximum(exp, 0)
+            got = oracle.dense(A, W, bias, shifts, mode, relu=relu, out=out)
+            assert np.array_equal(got.astype(np.int64), exp)
+    # scalar shift == vector of equal shifts (the per-channel extension reduces to the reference)
+    a = oracle.dense(A, W, bias, 7, mode)
+    b = oracle.dense(A, W, bias, np.full(N, 7), mode)
+    assert np.array_equal(a, b)
+
+
+def test_dense_special_cases(oracle):
+    r = _rng(2)
+    K = 16
+    A = r.integers(-128, 128, (8, K)).astype(np.int8)
+    eye = np.eye(K, dtype=np.int8)
+    # W = I, shift 0: identity
+    assert np.array_equal(oracle.dense(A, eye, None, 0, 'floor'), A)
+    # W = 0: out = srs(bias)
+    bias = np.array([64, -64, 63, -65, 192, -192, 2**31 - 1, -2**31] * 2, dtype=np.int32)
+    got = oracle.dense(A, np.zeros((K, K), np.int8), bias, 7, 'conv_even')
+    exp = [exact_srs(int(b), 7, 'conv_even', 'int8') for b in bias]
+    assert (got == np.array(exp, dtype=np.int8)).all()
+    # accumulator wraps modulo 2^32 (acc32), it does not saturate
+    A1 = np.full((1, 4), 127, np.int8)
+    W1 = np.full((4, 1), 127, np.int8)
+    big = np.array([2**31 - 1], np.int32)
+    wrapped = (4 * 127 * 127 + 2**31 - 1 + 2**31) % 2**32 - 2**31
+    assert oracle.dense(A1, W1, big, 0, 'floor', out='int32')[0, 0] == wrapped
+
+
+def test_matmul_batched_and_transposed(oracle):
+    r = _rng(3)
+    A = r.integers(-128, 128, (2, 3, 17, 24)).astype(np.int8)
+    B = r.integers(-128, 128, (2, 3, 24, 11)).astype(np.int8)
+    acc = A.astype(np.int64) @ B.astype(np.int64)
+    exp = np.vectorize(lambda v: exact_srs(int(v), 6, 'conv_even', 'int8'))(acc)
+    assert np.array_equal(oracle.matmul(A, B, 6, 'conv_even').astype(np.int64), exp)
+    Bt = np.ascontiguousarray(np.swapaxes(B, -1, -2))
+    assert np.array_equal(oracle.matmul(A, Bt, 6, 'conv_even', trans_b=True).astype(np.int64), exp)
+    # unsigned lhs (probabilities) x signed rhs
+    P = r.integers(0, 256, (2, 3, 17, 24)).astype(np.uint8)
+    acc = P.astype(np.int64) @ B.astype(np.int64)
+    exp = np.vectorize(lambda v: exact_srs(int(v), 8, 'symmetric_inf', 'int8'))(acc)
+    assert np.array_equal(oracle.matmul(P, B, 8, 'symmetric_inf').astype(np.int64), exp)
+
+
+def test_add_is_saturating(oracle):
+    a = np.arange(-128, 128, dtype=np.int8).repeat(256)
+    b = np.tile(np.arange(-128, 128, dtype=np.int8), 256)
+    exp = np.clip(a.astype(np.int32) + b.astype(np.int32), -128, 127).astype(np.int8)
+    assert np.array_equal(oracle.add(a, b), exp)
+    au, bu = a.view(np.uint8), b.view(np.uint8)
+    expu = np.clip(au.astype(np.int32) + bu.astype(np.int32), 0, 255).astype(np.uint8)
+    assert np.array_equal(oracle.add(au, bu), expu)
+    # shift 1 halves with the requested rounding
+    s = a.astype(np.int32) + b.astype(np.int32)
+    exp1 = np.array([exact_srs(int(v), 1, 'conv_even', 'int8') for v in s], dtype=np.int8)
+    assert np.array_equal(oracle.add(a, b, 1, 'conv_even'), exp1)
+
+
+# ---- integer exp softmax ---------------------------------------------------------------------
+
+def py_exp_score(d: int, kq: int) -> int:
+    """Python big-int restatement of the reference's exp_score16 steps (softmax.cpp:252-273)."""
+    z = min(d * kq, 32767)
+    zi, zf = z >> 8, z & 255
+    t = (zf * 2811) >> 8
+    e = (((t - 11004) * zf) >> 8) + 16384
+    for b in range(4):
+        if zi & (1 << b):
+            e >>= (1 << b)
+    return 0 if zi >= 16 else e
+
+
+def test_exp_score_exhaustive(oracle):
+    worst = 0.0
+    for kq in range(1, 129):
+        for d in range(256):
+            e = oracle.exp_score16(d, kq)
+            assert e == py_exp_score(d, kq), (d, kq)
+            # and it really is 2^(-d*kq/256) in Q14, within the 2nd-order polynomial's error
+            ideal = 16384.0 * 2.0 ** (-(d * kq) / 256.0)
+            worst = max(worst, abs(e - ideal))
+            assert abs(e - ideal) <= 40.0, (d, kq, e, ideal)
+    assert oracle.exp_score16(0, 23) == 16384
+    assert worst > 0.0
+
+
+def py_softmax_exp(row, kq, inv_shift=15):
+    m = max(row)
+    e = [py_exp_score(m - v, kq) for v in row]
+    inv = (255 << inv_shift) // max(sum(e), 1)
+    return [min(255, (x * inv) >> inv_shift) for x in e]
+
+
+def test_softmax_exp_rows(oracle):
+    r = _rng(4)
+    x = np.clip(np.rint(r.normal(0, 24, (64, 96))), -128, 127).astype(np.int8)
+    for kq in (1, 23, 46, 128):
+        got = oracle.softmax_exp(x, kq)
+        exp = np.array([py_softmax_exp(list(map(int, row)), kq) for row in x], dtype=np.uint8)
+        assert np.array_equal(got, exp), kq
+    # float softmax of the dequantised logits, frac 4 -> kq 23: within a few codes of 255*p
+    xf = x.astype(np.float64) / 16.0
+    p = np.exp(xf - xf.max(-1, keepdims=True))
+    p /= p.sum(-1, keepdims=True)
+    assert np.abs(oracle.softmax_exp(x, 23).astype(np.float64) - 255.0 * p).max() <= 3.0
+    # invariants: uniform row of C=512 -> inv = floor(510/512) = 0 -> all-zero probabilities
+    assert not oracle.softmax_exp(np.zeros((1, 512), np.int8), 23).any()
+    # uniform row of 32 -> inv = floor(255*2^15/(32*16384)) = 15 -> (16384*15)>>15 = 7
+    assert (oracle.softmax_exp(np.full((1, 32), 5, np.int8), 23) == 7).all()
+    # one-hot dominant row -> the max gets 255
+    one = np.full((1, 64), -128, np.int8)
+    one[0, 7] = 127
+    o = oracle.softmax_exp(one, 64)
+    assert o[0, 7] == 255 and o.sum() == 255
+
+
+def test_softmax_exp_int16_out(oracle):
+    r = _rng(5)
+    x = r.integers(-128, 128, (16, 64)).astype(np.int8)
+    got = oracle.softmax_exp(x, 23, out='int16')
+    for row, g in zip(x, got):
+        m = int(row.max())
+        e = [py_exp_score(m - int(v), 23) for v in row]
+        inv = 32767 // sum(e)
+        assert g.tolist() == [min(32767, v * inv) for v in e]
+
+
+def py_softmax_hccs(row, B, S, Dmax, inv_shift=15, out='uint8'):
+    m = max(row)
+    sc = [B - S * min(m - v, Dmax) for v in row]
+    if out == 'uint8':
+        inv = (255 << inv_shift) // sum(sc)
+        return [min(255, max(0, (s * inv) >> inv_shift)) for s in sc]
+    inv = 32767 // sum(sc)
+    return [min(32767, s * inv) for s in sc]
+
+
+def test_softmax_hccs_rows(oracle):
+    r = _rng(6)
+    x = np.clip(np.rint(r.normal(0, 24, (48, 512))), -128, 127).astype(np.int8)
+    for (B, S, Dmax) in [(60, 1, 59), (63, 2, 31), (40, 0, 0), (33, 1, 32)]:
+        got = oracle.softmax_hccs(x, B, S, Dmax)
+        exp = np.array([py_softmax_hccs(list(map(int, row)), B, S, Dmax) for row in x], dtype=np.uint8)
+        assert np.array_equal(got, exp)
+        got16 = oracle.softmax_hccs(x, B, S, Dmax, out='int16')
+        exp16 = np.array([py_softmax_hccs(list(map(int, row)), B, S, Dmax, out='int16') for row in x],
+                         dtype=np.int16)
+        assert np.array_equal(got16, exp16)
+    # S = 0 -> uniform: every output = floor(B * floor(255*2^15/(C*B)) / 2^15)
+    o = oracle.softmax_hccs(x[:1], 40, 0, 0)
+    inv = (255 << 15) // (512 * 40)
+    assert (o == ((40 * inv) >> 15)).all()
+    # sum of codes never exceeds 255 and is close to it for a peaked surrogate
+    o = oracle.softmax_hccs(x, 60, 1, 59).astype(np.int64).sum(-1)
+    assert (o <= 255).all()
+
+
+# ---- LayerNorm ---------------------------------------------------------------------------------
+
+def exact_rsqrt_q15(v: int) -> int:
+    """Nearest integer to 2^15/sqrt(v), by exact comparison of squares (independent of libm)."""
+    # q = floor(2^15/sqrt(v) + 1/2): largest q with (q - 1/2)^2 <= 2^30 / v
+    q = math.isqrt((1 << 32) // v) // 2  # coarse start, then fix up exactly
+    while Fraction(2 * q + 1, 2) ** 2 * v <= (1 << 30):
+        q += 1
+    while q > 0 and Fraction(2 * q - 1, 2) ** 2 * v > (1 << 30):
+        q -= 1
+    return min(q, 32767)
+
+
+def test_rsqrt_q15(oracle):
+    vals = list(range(1, 5000)) + [16384, 16385, 16383, 65535, 65536, 10**6, 2**30, 2**31 - 1]
+    vals += [int(v) for v in _rng(7).integers(1, 2**31 - 1, 2000)]
+    for v in vals:
+        assert oracle.rsqrt_q15(v) == exact_rsqrt_q15(v), v
+    assert oracle.rsqrt_q15(1) == 32767       # 32768 clamps
+    assert oracle.rsqrt_q15(4) == 16384
+    assert oracle.rsqrt_q15(16384) == 256
+
+
+def py_layernorm_row(x, gamma, beta, out_shift, mode, eps_q0=1):
+    C = len(x)
+    sx, sq = sum(x), sum(v * v for v in x)
+    mu = (sx + C // 2) // C
+    var = max(0, (sq - 2 * mu * sx + C * mu * mu) // C)
+    inv = exact_rsqrt_q15(var + eps_q0)
+    out = []
+    for v, g, b in zip(x, gamma, beta):
+        fs = exact_srs(inv * g, 7, mode, 'int16')
+        out.append(exact_srs((v - mu) * fs + b, 15 - out_shift, mode, 'int8'))
+    return out
+
+
+@pytest.mark.parametrize('cols', [32, 128, 1024, 768, 48])
+@pytest.mark.parametrize('mode', ['conv_even', 'symmetric_inf', 'floor'])
+def test_layernorm_rows(oracle, cols, mode):
+    r = _rng(8)
+    x = np.clip(np.rint(r.normal(3, 20, (24, cols))), -128, 127).astype(np.int8)
+    gamma = r.integers(32, 128, cols).astype(np.int16)
+    beta = (r.integers(-16, 17, cols) << 10).astype(np.int16)
+    for out_shift in (5, 4, 7):
+        got = oracle.layernorm(x, gamma, beta, out_shift, mode)
+        exp = np.array([py_layernorm_row(list(map(int, row)), gamma.tolist(), beta.tolist(), out_shift, mode)
+                        for row in x], dtype=np.int8)
+        assert np.array_equal(got, exp)
+
+
+def test_layernorm_invariants_and_float(oracle):
+    r = _rng(9)
+    cols = 256
+    gamma = r.integers(32, 128, cols).astype(np.int16)
+    beta = (r.integers(-16, 17, cols) << 10).astype(np.int16)
+    # constant row -> centred value 0 -> out = srs(beta, 15 - out_shift)
+    const = np.full((1, cols), 17, np.int8)
+    got = oracle.layernorm(const, gamma, beta, 5, 'conv_even')
+    assert got[0].tolist() == [exact_srs(int(b), 10, 'conv_even', 'int8') for b in beta]
+    # mean is rounded half-up: sum = C/2 -> mu = 1; sum = -C/2 -> mu = 0 (gamma large makes mu visible)
+    x = np.zeros((2, cols), np.int8)
+    x[0, :cols // 2] = 1
+    x[1, :cols // 2] = -1
+    g1 = np.full(cols, 128, np.int16)
+    b0 = np.zeros(cols, np.int16)
+    o = oracle.layernorm(x, g1, b0, 5, 'conv_even').astype(np.int64)
+    # row0: mu=1 -> centred {0 (x=1), -1 (x=0)}: var = (C/2)/C -> 0 -> inv = 32767 (eps=1), fs = sat16(32767)
+    assert o[0, 0] == 0 and o[0, -1] == exact_srs(-32767, 10, 'conv_even', 'int8')
+    assert o[1, 0] == exact_srs(-32767, 10, 'conv_even', 'int8') and o[1, -1] == 0
+    # against float LayerNorm: |error| <= 1.5 output LSB for well-conditioned rows
+    xs = np.clip(np.rint(r.normal(0, 25, (64, cols))), -128, 127).astype(np.int8)
+    out_shift = 5
+    got = oracle.layernorm(xs, gamma, beta, out_shift, 'conv_even').astype(np.float64)
+    xf = xs.astype(np.float64)
+    ref = (xf - xf.mean(-1, keepdims=True)) / np.sqrt(xf.var(-1, keepdims=True) + 1.0)
+    ref = ref * (gamma / 128.0) + beta / 32768.0
+    ref = np.clip(ref * (1 << out_shift), -128, 127)
+    assert np.abs(got - ref).max() <= 1.5
+
+
+def test_add_layernorm_is_composition(oracle):
+    r = _rng(10)
+    a = np.clip(np.rint(r.normal(0, 60, (32, 128))), -128, 127).astype(np.int8)
+    b = np.clip(np.rint(r.normal(0, 60, (32, 128))), -128, 127).astype(np.int8)
+    gamma = r.integers(32, 128, 128).astype(np.int16)
+    beta = (r.integers(-16, 17, 128) << 10).astype(np.int16)
+    s, out = oracle.add_layernorm(a, b, gamma, beta, 5, 'conv_even', return_sum=True)
+    s2 = oracle.add(a, b)
+    assert np.array_equal(s, s2)
+    assert np.array_equal(out, oracle.layernorm(s2, gamma, beta, 5, 'conv_even'))
