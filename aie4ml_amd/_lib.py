@@ -1,0 +1,106 @@
+"""ctypes loader for libaie4ml_gfx950.so — the only way the Python host reaches the HIP kernels.
+
+There is no CPU fallback: if the library is missing or a symbol cannot be bound, importing an operator
+raises, loudly.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / 'libaie4ml_gfx950.so'
+
+A4G_OK = 0
+A4G_ERR_INVALID_ARGUMENT = -1
+A4G_ERR_UNSUPPORTED = -2
+A4G_ERR_WORKSPACE = -3
+A4G_ERR_HIP = -4
+
+ROUNDING = {
+    'floor': 0,
+    'ceil': 1,
+    'positive_inf': 2,
+    'negative_inf': 3,
+    'symmetric_inf': 4,
+    'symmetric_zero': 5,
+    'conv_even': 6,
+    'conv_odd': 7,
+}
+KIND = {'int8': 0, 'uint8': 1, 'int16': 2, 'uint16': 3, 'int32': 4}
+
+_i64, _i32, _vp, _sz = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
+
+
+class MlpLayer(ctypes.Structure):
+    """Mirror of ``a4g_mlp_layer`` (include/aie4ml_gfx950.h)."""
+
+    _fields_ = [
+        ('wt', _vp),
+        ('ldwt', _i64),
+        ('colsum', _vp),
+        ('bias', _vp),
+        ('K', ctypes.c_int32),
+        ('N', ctypes.c_int32),
+        ('shift', ctypes.c_int32),
+        ('relu', ctypes.c_int32),
+        ('out_kind', ctypes.c_int32),
+    ]
+
+
+# name -> (restype, argtypes); must list every symbol the public header declares
+SIGNATURES = {
+    'a4g_version': (_i32, []),
+    'a4g_last_error': (ctypes.c_char_p, []),
+    'a4g_add': (_i32, [_vp, _vp, _vp, _i64, _i32, _i32, _i32, _vp]),
+    'a4g_packed_ld': (_i64, [_i64]),
+    'a4g_pack_weights_i8': (_i32, [_vp, _i64, _i64, _i64, _vp, _vp, _vp]),
+    'a4g_dense_i8': (_i32, [_vp, _i32, _i64, _vp, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _i64, _i64, _i64,
+                            _i64, _vp]),
+    'a4g_matmul_i8_workspace_bytes': (_sz, [_i64, _i64, _i64, _i64, _i32, _i32]),
+    'a4g_matmul_i8': (_i32, [_vp, _i32, _i64, _i64, _vp, _i64, _i64, _i32, _vp, _i64, _i64, _i64, _i64, _i64, _i64,
+                             _i32, _i32, _i32, _vp, _sz, _vp]),
+    'a4g_layernorm_i8': (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, ctypes.c_int32, _i32, _i32, _i32, _vp]),
+    'a4g_add_layernorm_i8': (_i32, [_vp, _vp, _i32, _i32, _vp, _vp, _vp, _vp, _i64, _i64, ctypes.c_int32, _i32, _i32,
+                                    _i32, _vp]),
+    'a4g_softmax_exp_i8': (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _i32, _vp]),
+    'a4g_softmax_hccs_i8': (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _vp]),
+    'a4g_mlp_i8': (_i32, [ctypes.POINTER(MlpLayer), _i32, _vp, _i32, _i64, _vp, _i64, _i64, _i32, _vp]),
+}
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Load the shared library and bind every entry point. Raises if anything is missing."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not LIB_PATH.exists():
+        raise RuntimeError(
+            f'{LIB_PATH} is missing: build it with `python -m aie4ml_amd.build` (hipcc, gfx950). '
+            'aie4ml_amd has no CPU fallback.'
+        )
+    lib = ctypes.CDLL(str(LIB_PATH))
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the symbol is not exported
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _lib = lib
+    return lib
+
+
+_EXC = {
+    A4G_ERR_INVALID_ARGUMENT: ValueError,
+    A4G_ERR_UNSUPPORTED: NotImplementedError,
+    A4G_ERR_WORKSPACE: RuntimeError,
+    A4G_ERR_HIP: RuntimeError,
+}
+
+
+def check(status: int) -> None:
+    """Translate a C status into the exception class the reference raises for the same condition."""
+    if status == A4G_OK:
+        return
+    msg = load().a4g_last_error().decode('utf-8', 'replace')
+    raise _EXC.get(status, RuntimeError)(msg)

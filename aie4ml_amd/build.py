@@ -1,0 +1,76 @@
+"""Builds libaie4ml_gfx950.so (the HIP kernels + C ABI) in-tree with hipcc for gfx950.
+
+Usage:  python -m aie4ml_amd.build [--force]
+"""
+
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+CSRC = Path(__file__).resolve().parent / 'csrc'
+LIB_PATH = Path(__file__).resolve().parent / 'libaie4ml_gfx950.so'
+SOURCES = ('abi.hip', 'rowops.hip', 'gemm.hip', 'mlp.hip')
+
+HIPCC_FLAGS = [
+    '--offload-arch=gfx950',
+    '-O3',
+    '-std=c++17',
+    '-fPIC',
+    '-fvisibility=hidden',
+    '-fvisibility-inlines-hidden',
+    '-Wall',
+    '-Wno-unused-function',
+    # packed-FP32 instruction selection is switched off for every kernel in this library
+    '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
+]
+
+
+def _hipcc() -> str:
+    rocm = os.environ.get('ROCM_PATH', '/opt/rocm')
+    cand = Path(rocm) / 'bin' / 'hipcc'
+    return str(cand) if cand.exists() else 'hipcc'
+
+
+def _stale() -> bool:
+    if not LIB_PATH.exists():
+        return True
+    t = LIB_PATH.stat().st_mtime
+    deps = [CSRC / s for s in SOURCES] + [CSRC / 'common.hpp', CSRC.parent.parent / 'include' / 'aie4ml_gfx950.h']
+    return any(d.stat().st_mtime > t for d in deps)
+
+
+def build(force: bool = False, verbose: bool = False) -> Path:
+    """Compile every HIP source for gfx950 and link the shared library. Returns its path."""
+    if not force and not _stale():
+        return LIB_PATH
+    objdir = CSRC / 'build'
+    objdir.mkdir(exist_ok=True)
+    hipcc = _hipcc()
+
+    def compile_one(src: str) -> Path:
+        obj = objdir / (Path(src).stem + '.o')
+        cmd = [hipcc, *HIPCC_FLAGS, '-c', str(CSRC / src), '-o', str(obj)]
+        res = subprocess.run(cmd, capture_output=True, text=True)
+        errs = '\n'.join(line for line in res.stderr.splitlines()
+                         if "is not a recognized feature" not in line)
+        if res.returncode != 0:
+            raise RuntimeError(f'hipcc failed on {src}:\n{errs}')
+        if verbose and errs.strip():
+            print(errs, file=sys.stderr)
+        return obj
+
+    with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as pool:
+        objs = list(pool.map(compile_one, SOURCES))
+    cmd = [hipcc, '--offload-arch=gfx950', '-shared', '-fPIC', '-o', str(LIB_PATH), *map(str, objs)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f'link failed:\n{res.stderr}')
+    return LIB_PATH
+
+
+if __name__ == '__main__':
+    print(build(force='--force' in sys.argv, verbose=True))

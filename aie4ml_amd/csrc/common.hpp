@@ -1,0 +1,169 @@
+// Shared device helpers: shift-round-saturate, storage kinds, wave-level reductions, error plumbing.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/aie4ml_gfx950.h"
+
+namespace a4g {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef short v2s __attribute__((ext_vector_type(2)));
+typedef unsigned short v2us __attribute__((ext_vector_type(2)));
+
+// ---- host-side error plumbing -------------------------------------------------------------------
+void set_error(const char* fmt, ...);
+int fail(int code, const char* fmt, ...);
+int check_hip(hipError_t e, const char* what);
+
+#define A4G_REQUIRE(cond, code, ...)                    \
+    do {                                                \
+        if (!(cond)) return ::a4g::fail(code, __VA_ARGS__); \
+    } while (0)
+
+static inline bool valid_round(int m) { return m >= 0 && m <= 7; }
+static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+static inline int kind_bytes(int kind) { return (kind == A4G_I8 || kind == A4G_U8) ? 1 : (kind == A4G_I32 ? 4 : 2); }
+
+// ---- rounding ---------------------------------------------------------------------------------------
+// round(acc / 2^s) for the eight aie::rounding_mode values; s in [0,31]. 32-bit only: the quotient
+// plus a 0/1 increment never overflows for s >= 1.
+template <int MODE>
+__device__ __forceinline__ int round_shift(int acc, int s) {
+    if (s == 0) return acc;
+    const int q = acc >> s;
+    if (MODE == A4G_RND_FLOOR) return q;
+    const unsigned mask = (1u << s) - 1u;
+    const unsigned r = static_cast<unsigned>(acc) & mask;
+    const unsigned h = 1u << (s - 1);
+    if (MODE == A4G_RND_CEIL) return q + (r != 0u);
+    if (MODE == A4G_RND_POSITIVE_INF) return q + (r >= h);
+    if (MODE == A4G_RND_NEGATIVE_INF) return q + (r > h);
+    if (MODE == A4G_RND_SYMMETRIC_INF) return q + ((r > h) | ((r == h) & (acc >= 0)));
+    if (MODE == A4G_RND_SYMMETRIC_ZERO) return q + ((r > h) | ((r == h) & (acc < 0)));
+    if (MODE == A4G_RND_CONV_EVEN) return q + ((r > h) | ((r == h) & (q & 1)));
+    /* conv_odd */ return q + ((r > h) | ((r == h) & ((q & 1) == 0)));
+}
+
+__device__ __forceinline__ int round_shift_rt(int acc, int s, int mode) {
+    switch (mode) {
+    case A4G_RND_FLOOR: return round_shift<A4G_RND_FLOOR>(acc, s);
+    case A4G_RND_CEIL: return round_shift<A4G_RND_CEIL>(acc, s);
+    case A4G_RND_POSITIVE_INF: return round_shift<A4G_RND_POSITIVE_INF>(acc, s);
+    case A4G_RND_NEGATIVE_INF: return round_shift<A4G_RND_NEGATIVE_INF>(acc, s);
+    case A4G_RND_SYMMETRIC_INF: return round_shift<A4G_RND_SYMMETRIC_INF>(acc, s);
+    case A4G_RND_SYMMETRIC_ZERO: return round_shift<A4G_RND_SYMMETRIC_ZERO>(acc, s);
+    case A4G_RND_CONV_EVEN: return round_shift<A4G_RND_CONV_EVEN>(acc, s);
+    default: return round_shift<A4G_RND_CONV_ODD>(acc, s);
+    }
+}
+
+// The same eight modes without a per-element switch: every mode is floor((acc + off) / 2^s) with
+// off = c0 + cx * bit, where bit is either the sign of acc or the parity of the floor quotient.
+// The offset is added to the remainder, not to acc, so nothing can overflow.
+struct RoundCfg {
+    int s;          // shift, 0..31
+    unsigned mask;  // 2^s - 1
+    int c0, cx;     // offset constants
+    int bs;         // which bit of acc feeds `bit`: 31 (sign) or s (quotient parity)
+};
+
+__host__ __device__ __forceinline__ RoundCfg make_round(int mode, int s) {
+    RoundCfg rc;
+    rc.s = s;
+    rc.mask = s > 0 ? ((1u << s) - 1u) : 0u;
+    rc.c0 = 0;
+    rc.cx = 0;
+    rc.bs = 31;
+    if (s <= 0) return rc;
+    const int h = 1 << (s - 1);
+    switch (mode) {
+    case A4G_RND_FLOOR: break;
+    case A4G_RND_CEIL: rc.c0 = static_cast<int>(rc.mask); break;
+    case A4G_RND_POSITIVE_INF: rc.c0 = h; break;
+    case A4G_RND_NEGATIVE_INF: rc.c0 = h - 1; break;
+    case A4G_RND_SYMMETRIC_INF: rc.c0 = h; rc.cx = -1; break;
+    case A4G_RND_SYMMETRIC_ZERO: rc.c0 = h - 1; rc.cx = 1; break;
+    case A4G_RND_CONV_EVEN: rc.c0 = h - 1; rc.cx = 1; rc.bs = s; break;
+    default: rc.c0 = h; rc.cx = -1; rc.bs = s; break;  // conv_odd
+    }
+    return rc;
+}
+
+__device__ __forceinline__ int apply_round(int acc, const RoundCfg& rc) {
+    const int q = acc >> rc.s;
+    const unsigned r = static_cast<unsigned>(acc) & rc.mask;
+    const int bit = (acc >> rc.bs) & 1;
+    const unsigned t = r + static_cast<unsigned>(rc.c0 + rc.cx * bit);
+    return q + static_cast<int>(t >> rc.s);
+}
+
+__device__ __forceinline__ int clamp_i(int v, int lo, int hi) { return min(max(v, lo), hi); }
+
+__device__ __forceinline__ int kind_lo(int kind) {
+    return kind == A4G_I8 ? -128 : (kind == A4G_I16 ? -32768 : (kind == A4G_I32 ? INT32_MIN : 0));
+}
+__device__ __forceinline__ int kind_hi(int kind) {
+    return kind == A4G_I8 ? 127 : (kind == A4G_U8 ? 255 : (kind == A4G_I16 ? 32767 : (kind == A4G_U16 ? 65535 : INT32_MAX)));
+}
+
+__device__ __forceinline__ int load_kind(const void* p, int64_t i, int kind) {
+    switch (kind) {
+    case A4G_I8: return static_cast<const int8_t*>(p)[i];
+    case A4G_U8: return static_cast<const uint8_t*>(p)[i];
+    case A4G_I16: return static_cast<const int16_t*>(p)[i];
+    case A4G_U16: return static_cast<const uint16_t*>(p)[i];
+    default: return static_cast<const int32_t*>(p)[i];
+    }
+}
+__device__ __forceinline__ void store_kind(void* p, int64_t i, int kind, int v) {
+    switch (kind) {
+    case A4G_I8: static_cast<int8_t*>(p)[i] = static_cast<int8_t>(v); break;
+    case A4G_U8: static_cast<uint8_t*>(p)[i] = static_cast<uint8_t>(v); break;
+    case A4G_I16: static_cast<int16_t*>(p)[i] = static_cast<int16_t>(v); break;
+    case A4G_U16: static_cast<uint16_t*>(p)[i] = static_cast<uint16_t>(v); break;
+    default: static_cast<int32_t*>(p)[i] = v; break;
+    }
+}
+
+// ---- cross-lane helpers (64-wide wavefront) -------------------------------------------------------------
+// xor-butterfly partner exchange. Masks 1,2 use DPP quad permutes, 4 and 8 the row mirrors (valid
+// as reduction steps once the lower levels are already combined), 16 ds_swizzle, 32 ds_bpermute.
+template <int MASK>
+__device__ __forceinline__ int lane_xor(int v) {
+    if (MASK == 1) return __builtin_amdgcn_mov_dpp(v, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
+    if (MASK == 2) return __builtin_amdgcn_mov_dpp(v, 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
+    if (MASK == 4) return __builtin_amdgcn_mov_dpp(v, 0x141, 0xF, 0xF, true); // row_half_mirror
+    if (MASK == 8) return __builtin_amdgcn_mov_dpp(v, 0x140, 0xF, 0xF, true); // row_mirror
+    if (MASK == 16) return __builtin_amdgcn_ds_swizzle(v, (0x10 << 10) | 0x1F);
+    return __builtin_amdgcn_ds_bpermute(((__lane_id() ^ 32) << 2), v);
+}
+
+struct OpAdd {
+    __device__ __forceinline__ int operator()(int a, int b) const { return a + b; }
+};
+struct OpMax {
+    __device__ __forceinline__ int operator()(int a, int b) const { return max(a, b); }
+};
+
+// All-reduce over aligned groups of L consecutive lanes (L a power of two, 1..64).
+template <int L, typename Op>
+__device__ __forceinline__ int group_allreduce(int v, Op op) {
+    if (L >= 2) v = op(v, lane_xor<1>(v));
+    if (L >= 4) v = op(v, lane_xor<2>(v));
+    if (L >= 8) v = op(v, lane_xor<4>(v));
+    if (L >= 16) v = op(v, lane_xor<8>(v));
+    if (L >= 32) v = op(v, lane_xor<16>(v));
+    if (L >= 64) v = op(v, lane_xor<32>(v));
+    return v;
+}
+
+__device__ __forceinline__ int64_t floordiv64(int64_t a, int64_t b) {
+    int64_t q = a / b, r = a % b;
+    return (r != 0 && ((r < 0) != (b < 0))) ? q - 1 : q;
+}
+
+}  // namespace a4g

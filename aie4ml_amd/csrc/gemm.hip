@@ -1,0 +1,522 @@
+// int8 x int8 -> int32 GEMM on the gfx950 matrix cores (v_mfma_i32_32x32x32_i8) with the fused
+// requantisation epilogue of the reference's Dense and MatMul kernels
+// (dense_bias_relu.cpp:112-163, matmul.cpp:80-115): bias, shift / round / saturate, ReLU.
+//
+// Operand layout ("NT"): A is [M][lda] and the right-hand side is [N][ldb], both with the
+// reduction axis contiguous, so every MFMA operand is one 16-byte read. Dense weights are packed to
+// that layout once (a4g_pack_weights_i8); a K x N activation operand is transposed by a pre-pass.
+// uint8 left operands are biased to int8 with x ^ 0x80 when fragments are read; the epilogue adds
+// back 128 * colsum[n] (exact in wrapping int32).
+#include <algorithm>
+#include <cstdlib>
+
+#include "common.hpp"
+
+namespace a4g {
+
+struct GemmArgs {
+    const int8_t* A;
+    const int8_t* Bt;
+    void* C;
+    const int32_t* bias;    // [N] or null
+    const int32_t* colsum;  // [batch][N] or null (only read when a_unsigned)
+    const int32_t* shifts;  // device shifts, entry n * shift_stride; null -> the scalar `shift`
+    int64_t lda, stride_a, ldb, stride_b, ldc, stride_c, stride_colsum;
+    int M, N, K;
+    int shift;
+    int shift_stride;  // 0: one device scalar for every column, 1: per output channel
+    int a_unsigned;
+    int relu;
+    int out_kind;
+    int mode;
+};
+
+__device__ __forceinline__ int column_shift(const GemmArgs& g, int n) {
+    const int s = g.shifts ? g.shifts[static_cast<int64_t>(n) * g.shift_stride] : g.shift;
+    return min(max(s, 0), 31);
+}
+
+// lo already includes the ReLU floor (max(lo, 0)) when the layer has one
+__device__ __forceinline__ int requant(int acc, const RoundCfg& rc, int lo, int hi) {
+    return clamp_i(apply_round(acc, rc), lo, hi);
+}
+
+// -----------------------------------------------------------------------------------------------------
+// Tiled MFMA kernel. Block tile BM x BN, K step BK, WAVES_M x WAVES_N waves; each wave owns a
+// (BM/WAVES_M) x (BN/WAVES_N) sub-tile as TM x TN blocks of 32x32 int32 accumulators.
+// Requirements checked by the host: K % 16 == 0, lda % 16 == 0, ldb % 16 == 0, 16-byte aligned bases.
+// -----------------------------------------------------------------------------------------------------
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
+struct GemmCfg {
+    static constexpr int NT = WAVES_M * WAVES_N * 64;
+    static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+    static constexpr int TM = WTM / 32, TN = WTN / 32;
+    static constexpr int CPR = BK / 16;          // 16-byte chunks per tile row
+    static constexpr int PITCH = BK + 16;        // LDS row pitch: breaks the power-of-two bank stride
+    static constexpr int A_CHUNKS = BM * CPR, B_CHUNKS = BN * CPR;
+    static constexpr int A_PER_T = A_CHUNKS / NT, B_PER_T = B_CHUNKS / NT;
+    static constexpr int LDS_BYTES = 2 * (BM + BN) * PITCH;
+    static_assert(A_CHUNKS % NT == 0 && B_CHUNKS % NT == 0, "tile loads must divide evenly over the threads");
+    static_assert(WTM % 32 == 0 && WTN % 32 == 0 && BK % 32 == 0, "wave tile must be whole 32x32x32 MFMA blocks");
+};
+
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_i8_nt_kernel(GemmArgs g) {
+    using Cfg = GemmCfg<BM, BN, BK, WAVES_M, WAVES_N>;
+    extern __shared__ __attribute__((aligned(16))) int8_t smem[];
+    constexpr int BUF = (BM + BN) * Cfg::PITCH;  // one stage: A tile then B tile
+    constexpr int B_OFF = BM * Cfg::PITCH;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+
+    // Workgroup -> tile mapping. Hardware deals consecutive workgroup ids round-robin over the 8
+    // XCDs, each with a private L2, so id % 8 names the XCD: give every XCD one contiguous range of
+    // tiles, and order that range in bands of GROUP_M tile rows (row index fastest inside a band) so
+    // that the tiles resident on an XCD at one time share both activation and weight panels.
+    const int tiles_m = (g.M + BM - 1) / BM;
+    const int tiles_n = (g.N + BN - 1) / BN;
+    const int tiles = tiles_m * tiles_n;
+    const int per_xcd = (tiles + 7) / 8;
+    const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    if (tile >= tiles) return;
+    constexpr int GROUP_M = 8;
+    const int band = tile / (GROUP_M * tiles_n);
+    const int band_rows = min(GROUP_M, tiles_m - band * GROUP_M);
+    const int in_band = tile % (GROUP_M * tiles_n);
+    const int m0 = (band * GROUP_M + in_band % band_rows) * BM;
+    const int n0 = (in_band / band_rows) * BN;
+    const int batch = blockIdx.y;
+
+    const int8_t* __restrict__ Ab = g.A + batch * g.stride_a;
+    const int8_t* __restrict__ Bb = g.Bt + batch * g.stride_b;
+
+    // global -> register staging of the next K tile
+    v4i ra[Cfg::A_PER_T], rb[Cfg::B_PER_T];
+    const int8_t* pa[Cfg::A_PER_T];
+    const int8_t* pb[Cfg::B_PER_T];
+    int ka[Cfg::A_PER_T], kb[Cfg::B_PER_T];
+    int offa[Cfg::A_PER_T], offb[Cfg::B_PER_T];
+#pragma unroll
+    for (int i = 0; i < Cfg::A_PER_T; ++i) {
+        const int c = tid + i * Cfg::NT;
+        const int row = c / Cfg::CPR, kc = c % Cfg::CPR;
+        const int gm = min(m0 + row, g.M - 1);
+        pa[i] = Ab + static_cast<int64_t>(gm) * g.lda + kc * 16;
+        ka[i] = kc * 16;
+        offa[i] = row * Cfg::PITCH + kc * 16;
+    }
+#pragma unroll
+    for (int i = 0; i < Cfg::B_PER_T; ++i) {
+        const int c = tid + i * Cfg::NT;
+        const int row = c / Cfg::CPR, kc = c % Cfg::CPR;
+        const int gn = min(n0 + row, g.N - 1);
+        pb[i] = Bb + static_cast<int64_t>(gn) * g.ldb + kc * 16;
+        kb[i] = kc * 16;
+        offb[i] = row * Cfg::PITCH + kc * 16;
+    }
+
+    auto load_tile = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < Cfg::A_PER_T; ++i)
+            ra[i] = (k0 + ka[i] < g.K) ? *reinterpret_cast<const v4i*>(pa[i] + k0) : v4i{0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < Cfg::B_PER_T; ++i)
+            rb[i] = (k0 + kb[i] < g.K) ? *reinterpret_cast<const v4i*>(pb[i] + k0) : v4i{0, 0, 0, 0};
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < Cfg::A_PER_T; ++i) *reinterpret_cast<v4i*>(smem + buf * BUF + offa[i]) = ra[i];
+#pragma unroll
+        for (int i = 0; i < Cfg::B_PER_T; ++i) *reinterpret_cast<v4i*>(smem + buf * BUF + B_OFF + offb[i]) = rb[i];
+    };
+
+    v16i acc[Cfg::TM][Cfg::TN];
+#pragma unroll
+    for (int i = 0; i < Cfg::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < Cfg::TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+    // fragment addressing: lane%32 picks the row of the operand block, lane/32 the 16-byte half of
+    // the 32-wide K step
+    const int frag_row = lane & 31;
+    const int frag_k = (lane >> 5) * 16;
+    const int a_frag_off = (wm * Cfg::WTM + frag_row) * Cfg::PITCH + frag_k;
+    const int b_frag_off = (wn * Cfg::WTN + frag_row) * Cfg::PITCH + frag_k;
+    const int xor_mask = g.a_unsigned ? static_cast<int>(0x80808080u) : 0;
+
+    const int ktiles = (g.K + BK - 1) / BK;
+    load_tile(0);
+    store_tile(0);
+    __syncthreads();
+
+    for (int kt = 0; kt < ktiles; ++kt) {
+        const int buf = kt & 1;
+        if (kt + 1 < ktiles) load_tile((kt + 1) * BK);
+#pragma unroll
+        for (int kk = 0; kk < BK / 32; ++kk) {
+            v4i af[Cfg::TM], bf[Cfg::TN];
+#pragma unroll
+            for (int i = 0; i < Cfg::TM; ++i) {
+                af[i] = *reinterpret_cast<const v4i*>(smem + buf * BUF + a_frag_off + i * 32 * Cfg::PITCH + kk * 32);
+                af[i] ^= xor_mask;
+            }
+#pragma unroll
+            for (int j = 0; j < Cfg::TN; ++j)
+                bf[j] = *reinterpret_cast<const v4i*>(smem + buf * BUF + B_OFF + b_frag_off + j * 32 * Cfg::PITCH + kk * 32);
+#pragma unroll
+            for (int i = 0; i < Cfg::TM; ++i)
+#pragma unroll
+                for (int j = 0; j < Cfg::TN; ++j)
+                    // operands swapped: the block's first index (registers) runs over n, lanes over m
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[i], acc[i][j], 0, 0, 0);
+        }
+        if (kt + 1 < ktiles) store_tile(buf ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: lane owns row m = lane%32 of each block and, per register quad q, the four
+    // consecutive columns 8q + 4*(lane/32) .. +3.
+    const int lo = g.relu ? max(kind_lo(g.out_kind), 0) : kind_lo(g.out_kind), hi = kind_hi(g.out_kind);
+    const int obytes = (g.out_kind == A4G_I16 || g.out_kind == A4G_U16) ? 2 : 1;
+    int8_t* Cb = static_cast<int8_t*>(g.C) + batch * g.stride_c * obytes;
+    const int32_t* cs = (g.a_unsigned && g.colsum) ? g.colsum + batch * g.stride_colsum : nullptr;
+    const bool vec_ok = (g.ldc % 4 == 0) && ((reinterpret_cast<uintptr_t>(Cb) & 7) == 0);
+#pragma unroll
+    for (int j = 0; j < Cfg::TN; ++j) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int n = n0 + wn * Cfg::WTN + j * 32 + 8 * q + 4 * (lane >> 5);
+            int add[4];
+            RoundCfg rc[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const int nn = min(n + t, g.N - 1);
+                int a = g.bias ? g.bias[nn] : 0;
+                if (cs) a += 128 * cs[nn];
+                add[t] = a;
+                rc[t] = make_round(g.mode, column_shift(g, nn));
+            }
+#pragma unroll
+            for (int i = 0; i < Cfg::TM; ++i) {
+                const int m = m0 + wm * Cfg::WTM + i * 32 + (lane & 31);
+                int y[4];
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    y[t] = requant(static_cast<int>(static_cast<unsigned>(acc[i][j][q * 4 + t]) + static_cast<unsigned>(add[t])),
+                                   rc[t], lo, hi);
+                int8_t* dst = Cb + (static_cast<int64_t>(m) * g.ldc + n) * obytes;
+                if (m >= g.M || n >= g.N) {
+                    // outside the matrix: nothing to store
+                } else if (n + 3 < g.N && vec_ok) {
+                    if (obytes == 1) {
+                        *reinterpret_cast<unsigned*>(dst) = (y[0] & 0xFF) | ((y[1] & 0xFF) << 8) | ((y[2] & 0xFF) << 16) |
+                                                            (static_cast<unsigned>(y[3]) << 24);
+                    } else {
+                        v2i o = {(y[0] & 0xFFFF) | (y[1] << 16), (y[2] & 0xFFFF) | (y[3] << 16)};
+                        *reinterpret_cast<v2i*>(dst) = o;
+                    }
+                } else {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        if (n + t < g.N) {
+                            if (obytes == 1) dst[t] = static_cast<int8_t>(y[t]);
+                            else reinterpret_cast<int16_t*>(dst)[t] = static_cast<int16_t>(y[t]);
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+// -----------------------------------------------------------------------------------------------------
+// Generic kernel: any shape / pitch / alignment; one thread per output element.
+// trans_b == 1: B is [N][ldb]; trans_b == 0: B is [K][ldb].
+// -----------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void gemm_generic_kernel(GemmArgs g, int trans_b) {
+    const int64_t total = static_cast<int64_t>(g.M) * g.N;
+    const int batch = blockIdx.y;
+    const int8_t* Ab = g.A + batch * g.stride_a;
+    const int8_t* Bb = g.Bt + batch * g.stride_b;
+    const int obytes = (g.out_kind == A4G_I16 || g.out_kind == A4G_U16) ? 2 : 1;
+    int8_t* Cb = static_cast<int8_t*>(g.C) + batch * g.stride_c * obytes;
+    const int lo = g.relu ? max(kind_lo(g.out_kind), 0) : kind_lo(g.out_kind), hi = kind_hi(g.out_kind);
+    for (int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; idx < total;
+         idx += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+        const int m = static_cast<int>(idx / g.N), n = static_cast<int>(idx % g.N);
+        unsigned acc = g.bias ? static_cast<unsigned>(g.bias[n]) : 0u;
+        const int8_t* ar = Ab + static_cast<int64_t>(m) * g.lda;
+        for (int k = 0; k < g.K; ++k) {
+            const int a = g.a_unsigned ? static_cast<int>(static_cast<uint8_t>(ar[k])) : static_cast<int>(ar[k]);
+            const int b = trans_b ? Bb[static_cast<int64_t>(n) * g.ldb + k] : Bb[static_cast<int64_t>(k) * g.ldb + n];
+            acc += static_cast<unsigned>(a * b);
+        }
+        const int y = requant(static_cast<int>(acc), make_round(g.mode, column_shift(g, n)), lo, hi);
+        if (obytes == 1) Cb[static_cast<int64_t>(m) * g.ldc + n] = static_cast<int8_t>(y);
+        else reinterpret_cast<int16_t*>(Cb)[static_cast<int64_t>(m) * g.ldc + n] = static_cast<int16_t>(y);
+    }
+}
+
+// -----------------------------------------------------------------------------------------------------
+// Right-hand-side preparation: [K][ldb] -> [N][ldt] (zero padded to ldt) and column sums.
+// -----------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void transpose_kn_kernel(const int8_t* __restrict__ B, int64_t ldb, int64_t stride_b,
+                                                            int8_t* __restrict__ Bt, int64_t ldt, int64_t stride_t, int K,
+                                                            int N) {
+    __shared__ int8_t tile[64][65];
+    const int batch = blockIdx.z;
+    const int k0 = blockIdx.x * 64, n0 = blockIdx.y * 64;
+    const int8_t* src = B + batch * stride_b;
+    int8_t* dst = Bt + batch * stride_t;
+    for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+        const int kk = i >> 6, nn = i & 63;
+        const int k = k0 + kk, n = n0 + nn;
+        tile[kk][nn] = (k < K && n < N) ? src[static_cast<int64_t>(k) * ldb + n] : static_cast<int8_t>(0);
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+        const int nn = i >> 6, kk = i & 63;
+        const int k = k0 + kk, n = n0 + nn;
+        if (n < N && k < ldt) dst[static_cast<int64_t>(n) * ldt + k] = tile[kk][nn];
+    }
+}
+
+// colsum[b][n] = sum_k rhs[k][n]; trans: rhs stored [N][ld] (sum along the contiguous axis).
+__global__ __launch_bounds__(256) void colsum_kernel(const int8_t* __restrict__ B, int64_t ld, int64_t stride_b, int trans,
+                                                      int32_t* __restrict__ colsum, int64_t stride_c, int K, int N) {
+    const int batch = blockIdx.y;
+    const int8_t* src = B + batch * stride_b;
+    const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    if (n >= N) return;
+    int s = 0;
+    if (trans) {
+        const int8_t* r = src + static_cast<int64_t>(n) * ld;
+        for (int k = 0; k < K; ++k) s += r[k];
+    } else {
+        for (int k = 0; k < K; ++k) s += src[static_cast<int64_t>(k) * ld + n];
+    }
+    colsum[batch * stride_c + n] = s;
+}
+
+static inline int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
+
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
+static hipError_t launch_tiled(const GemmArgs& g, int batch, hipStream_t stream) {
+    using Cfg = GemmCfg<BM, BN, BK, WAVES_M, WAVES_N>;
+    auto kern = gemm_i8_nt_kernel<BM, BN, BK, WAVES_M, WAVES_N>;
+    static bool attr_set = false;  // benign race: the attribute is idempotent
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           Cfg::LDS_BYTES);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    const int tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
+    const int grid_x = (tiles + 7) / 8 * 8;  // whole ranges for the 8 XCDs; surplus workgroups exit at once
+    hipLaunchKernelGGL(kern, dim3(grid_x, batch), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, g);
+    return hipGetLastError();
+}
+
+// Picks a tile shape for the problem. variant: 0 = automatic; >0 forces a shape (used by the tuning
+// harness through the A4G_GEMM_VARIANT environment variable).
+static hipError_t launch_gemm_nt(const GemmArgs& g, int batch, hipStream_t stream, int variant) {
+    if (variant == 0) {
+        const int64_t tiles256 = static_cast<int64_t>((g.M + 255) / 256) * ((g.N + 255) / 256) * batch;
+        if (g.N <= 64) variant = 3;
+        else if (g.M >= 256 && g.N >= 256 && tiles256 >= 128) variant = 1;
+        else variant = 2;
+    }
+    switch (variant) {
+    case 1: return launch_tiled<256, 256, 64, 2, 4>(g, batch, stream);
+    case 2: return launch_tiled<128, 128, 64, 2, 2>(g, batch, stream);
+    case 3: return launch_tiled<256, 64, 64, 4, 1>(g, batch, stream);
+    case 4: return launch_tiled<256, 256, 64, 2, 2>(g, batch, stream);
+    case 5: return launch_tiled<256, 128, 64, 2, 2>(g, batch, stream);
+    case 6: return launch_tiled<256, 256, 128, 2, 4>(g, batch, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+static int env_variant() {
+    static int v = -1;
+    if (v < 0) {
+        const char* e = getenv("A4G_GEMM_VARIANT");
+        v = e ? atoi(e) : 0;
+        if (v < 0) v = 0;
+    }
+    return v;
+}
+
+static bool out_kind_ok(int k) { return k == A4G_I8 || k == A4G_U8 || k == A4G_I16; }
+
+}  // namespace a4g
+
+using namespace a4g;
+
+extern "C" int64_t a4g_packed_ld(int64_t K) { return K <= 0 ? 16 : round_up(K, 16); }
+
+extern "C" int a4g_pack_weights_i8(const int8_t* W, int64_t ldw, int64_t K, int64_t N, int8_t* Wt, int32_t* colsum,
+                                   a4g_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    A4G_REQUIRE(W && Wt, A4G_ERR_INVALID_ARGUMENT, "a4g_pack_weights_i8: null pointer");
+    A4G_REQUIRE(K >= 1 && N >= 1 && K <= (1 << 24) && N <= (1 << 24) && ldw >= N, A4G_ERR_INVALID_ARGUMENT,
+                "a4g_pack_weights_i8: bad shape K=%lld N=%lld ldw=%lld", (long long)K, (long long)N, (long long)ldw);
+    const int64_t ldt = a4g_packed_ld(K);
+    dim3 grid(static_cast<unsigned>((ldt + 63) / 64), static_cast<unsigned>((N + 63) / 64), 1);
+    transpose_kn_kernel<<<grid, 256, 0, stream>>>(W, ldw, 0, Wt, ldt, 0, static_cast<int>(K), static_cast<int>(N));
+    if (colsum) {
+        colsum_kernel<<<dim3(static_cast<unsigned>((N + 255) / 256), 1), 256, 0, stream>>>(W, ldw, 0, 0, colsum, 0,
+                                                                                          static_cast<int>(K),
+                                                                                          static_cast<int>(N));
+    }
+    return check_hip(hipGetLastError(), "a4g_pack_weights_i8");
+}
+
+extern "C" int a4g_dense_i8(const void* A, int a_kind, int64_t lda, const int8_t* Wt, int64_t ldwt, const int32_t* colsum,
+                            const int32_t* bias, const int32_t* shifts, int n_shift, int round_mode, int relu, int out_kind,
+                            void* Y, int64_t ldy, int64_t M, int64_t N, int64_t K, a4g_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const char* who = "a4g_dense_i8";
+    A4G_REQUIRE(M >= 0 && N >= 1 && K >= 1 && M <= INT32_MAX && N <= (1 << 24) && K <= (1 << 24), A4G_ERR_INVALID_ARGUMENT,
+                "%s: bad shape M=%lld N=%lld K=%lld", who, (long long)M, (long long)N, (long long)K);
+    A4G_REQUIRE(a_kind == A4G_I8 || a_kind == A4G_U8, A4G_ERR_UNSUPPORTED, "%s: activations must be int8 or uint8 (kind %d)",
+                who, a_kind);
+    A4G_REQUIRE(out_kind_ok(out_kind), A4G_ERR_UNSUPPORTED, "%s: output kind %d is not int8/uint8/int16", who, out_kind);
+    A4G_REQUIRE(valid_round(round_mode), A4G_ERR_INVALID_ARGUMENT, "%s: unknown rounding mode %d", who, round_mode);
+    A4G_REQUIRE(n_shift == 1 || n_shift == N, A4G_ERR_INVALID_ARGUMENT, "%s: n_shift must be 1 or N=%lld, got %d", who,
+                (long long)N, n_shift);
+    A4G_REQUIRE(lda >= K && ldy >= N && ldwt >= K, A4G_ERR_INVALID_ARGUMENT, "%s: pitch smaller than the row", who);
+    if (M == 0) return A4G_OK;
+    A4G_REQUIRE(A && Wt && Y && shifts, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+    A4G_REQUIRE(a_kind != A4G_U8 || colsum, A4G_ERR_INVALID_ARGUMENT, "%s: uint8 activations need the packed colsum vector",
+                who);
+
+    GemmArgs g{};
+    g.A = static_cast<const int8_t*>(A);
+    g.Bt = Wt;
+    g.C = Y;
+    g.bias = bias;
+    g.colsum = colsum;
+    g.shifts = shifts;
+    g.lda = lda;
+    g.ldb = ldwt;
+    g.ldc = ldy;
+    g.M = static_cast<int>(M);
+    g.N = static_cast<int>(N);
+    g.K = static_cast<int>(K);
+    g.shift_stride = n_shift == 1 ? 0 : 1;
+    g.a_unsigned = a_kind == A4G_U8;
+    g.relu = relu != 0;
+    g.out_kind = out_kind;
+    g.mode = round_mode;
+
+    const bool tiled = K % 16 == 0 && lda % 16 == 0 && ldwt % 16 == 0 && aligned16(A) && aligned16(Wt);
+    hipError_t e;
+    if (tiled) {
+        e = launch_gemm_nt(g, 1, stream, env_variant());
+    } else {
+        const int64_t total = M * N;
+        const int grid = static_cast<int>(std::min<int64_t>((total + 255) / 256, 256 * 32));
+        gemm_generic_kernel<<<dim3(grid, 1), 256, 0, stream>>>(g, 1);
+        e = hipGetLastError();
+    }
+    return check_hip(e, who);
+}
+
+extern "C" size_t a4g_matmul_i8_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int trans_b, int a_kind) {
+    (void)M;
+    if (batch <= 0 || N <= 0 || K <= 0) return 0;
+    size_t bytes = 0;
+    if (!trans_b) bytes += static_cast<size_t>(round_up(batch * N * a4g_packed_ld(K), 256));
+    if (a_kind == A4G_U8) bytes += static_cast<size_t>(round_up(batch * N * 4, 256));
+    return bytes;
+}
+
+extern "C" int a4g_matmul_i8(const void* A, int a_kind, int64_t lda, int64_t stride_a, const int8_t* B, int64_t ldb,
+                             int64_t stride_b, int trans_b, void* C, int64_t ldc, int64_t stride_c, int64_t batch, int64_t M,
+                             int64_t N, int64_t K, int shift, int round_mode, int out_kind, void* workspace,
+                             size_t workspace_bytes, a4g_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const char* who = "a4g_matmul_i8";
+    A4G_REQUIRE(batch >= 0 && batch <= 65535 && M >= 0 && N >= 1 && K >= 1 && M <= INT32_MAX && N <= (1 << 24) &&
+                    K <= (1 << 24),
+                A4G_ERR_INVALID_ARGUMENT, "%s: bad shape batch=%lld M=%lld N=%lld K=%lld", who, (long long)batch,
+                (long long)M, (long long)N, (long long)K);
+    A4G_REQUIRE(a_kind == A4G_I8 || a_kind == A4G_U8, A4G_ERR_UNSUPPORTED, "%s: lhs must be int8 or uint8 (kind %d)", who,
+                a_kind);
+    A4G_REQUIRE(out_kind_ok(out_kind), A4G_ERR_UNSUPPORTED, "%s: output kind %d is not int8/uint8/int16", who, out_kind);
+    A4G_REQUIRE(valid_round(round_mode), A4G_ERR_INVALID_ARGUMENT, "%s: unknown rounding mode %d", who, round_mode);
+    A4G_REQUIRE(shift >= 0 && shift <= 31, A4G_ERR_INVALID_ARGUMENT,
+                "%s: accumulator output shift must be in [0,31], got %d", who, shift);
+    A4G_REQUIRE(lda >= K && ldc >= N && ldb >= (trans_b ? K : N), A4G_ERR_INVALID_ARGUMENT, "%s: pitch smaller than the row",
+                who);
+    if (batch == 0 || M == 0) return A4G_OK;
+    A4G_REQUIRE(A && B && C, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+    const size_t need = a4g_matmul_i8_workspace_bytes(batch, M, N, K, trans_b, a_kind);
+    A4G_REQUIRE(need == 0 || (workspace && workspace_bytes >= need), A4G_ERR_WORKSPACE,
+                "%s: workspace of %zu bytes required, got %zu", who, need, workspace ? workspace_bytes : (size_t)0);
+    A4G_REQUIRE(need == 0 || aligned16(workspace), A4G_ERR_WORKSPACE, "%s: workspace must be 16-byte aligned", who);
+
+    GemmArgs g{};
+    g.A = static_cast<const int8_t*>(A);
+    g.C = C;
+    g.lda = lda;
+    g.stride_a = stride_a;
+    g.ldc = ldc;
+    g.stride_c = stride_c;
+    g.M = static_cast<int>(M);
+    g.N = static_cast<int>(N);
+    g.K = static_cast<int>(K);
+    g.shift = shift;
+    g.shifts = nullptr;
+    g.a_unsigned = a_kind == A4G_U8;
+    g.out_kind = out_kind;
+    g.mode = round_mode;
+
+    int8_t* ws = static_cast<int8_t*>(workspace);
+    const int64_t ldt = a4g_packed_ld(K);
+    int32_t* colsum = nullptr;
+    if (g.a_unsigned) {
+        colsum = reinterpret_cast<int32_t*>(ws + (trans_b ? 0 : round_up(batch * N * ldt, 256)));
+        colsum_kernel<<<dim3(static_cast<unsigned>((N + 255) / 256), static_cast<unsigned>(batch)), 256, 0, stream>>>(
+            B, ldb, stride_b, trans_b, colsum, N, static_cast<int>(K), static_cast<int>(N));
+        g.colsum = colsum;
+        g.stride_colsum = N;
+    }
+
+    const bool a_ok = K % 16 == 0 && lda % 16 == 0 && stride_a % 16 == 0 && aligned16(A);
+    hipError_t e;
+    if (trans_b) {
+        g.Bt = B;
+        g.ldb = ldb;
+        g.stride_b = stride_b;
+        if (a_ok && ldb % 16 == 0 && stride_b % 16 == 0 && aligned16(B)) {
+            e = launch_gemm_nt(g, static_cast<int>(batch), stream, env_variant());
+        } else {
+            const int grid = static_cast<int>(std::min<int64_t>((M * N + 255) / 256, 256 * 32));
+            gemm_generic_kernel<<<dim3(grid, static_cast<unsigned>(batch)), 256, 0, stream>>>(g, 1);
+            e = hipGetLastError();
+        }
+    } else if (a_ok) {
+        dim3 tg(static_cast<unsigned>((ldt + 63) / 64), static_cast<unsigned>((N + 63) / 64), static_cast<unsigned>(batch));
+        transpose_kn_kernel<<<tg, 256, 0, stream>>>(B, ldb, stride_b, ws, ldt, N * ldt, static_cast<int>(K),
+                                                    static_cast<int>(N));
+        g.Bt = ws;
+        g.ldb = ldt;
+        g.stride_b = N * ldt;
+        e = launch_gemm_nt(g, static_cast<int>(batch), stream, env_variant());
+    } else {
+        g.Bt = B;
+        g.ldb = ldb;
+        g.stride_b = stride_b;
+        const int grid = static_cast<int>(std::min<int64_t>((M * N + 255) / 256, 256 * 32));
+        gemm_generic_kernel<<<dim3(grid, static_cast<unsigned>(batch)), 256, 0, stream>>>(g, 0);
+        e = hipGetLastError();
+    }
+    return check_hip(e, who);
+}

@@ -1,0 +1,270 @@
+"""Operator-level host API: torch device tensors in, torch device tensors out, HIP kernels underneath.
+
+Each function is a thin shim over one C-ABI entry point of ``libaie4ml_gfx950.so``; PyTorch only
+supplies device memory and the current stream. Argument meaning follows the reference's kernel
+configuration structs (templates/firmware/variants/*/parameters.h.jinja).
+"""
+
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass
+from typing import List, Optional, Sequence
+
+import torch
+
+from . import _lib
+from ._lib import KIND, ROUNDING, MlpLayer, check
+
+_TORCH_KIND = {torch.int8: 0, torch.uint8: 1, torch.int16: 2, torch.int32: 4}
+_KIND_TORCH = {0: torch.int8, 1: torch.uint8, 2: torch.int16, 4: torch.int32}
+
+
+def _mode(mode) -> int:
+    if isinstance(mode, str):
+        try:
+            return ROUNDING[mode]
+        except KeyError:
+            raise ValueError(f'Unsupported rounding mode {mode!r} for the GPU kernels.') from None
+    return int(mode)
+
+
+def _kind(kind) -> int:
+    return KIND[kind] if isinstance(kind, str) else int(kind)
+
+
+def _dev(t: torch.Tensor, name: str) -> torch.Tensor:
+    if not t.is_cuda:
+        raise ValueError(f'{name}: expected a tensor in GPU memory, got device {t.device}.')
+    return t
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def _stream() -> ctypes.c_void_p:
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _rows2d(t: torch.Tensor, name: str) -> torch.Tensor:
+    """View a tensor as [rows, cols] with a contiguous last axis."""
+    _dev(t, name)
+    if t.dim() < 1:
+        raise ValueError(f'{name}: need at least one axis.')
+    t2 = t.reshape(-1, t.shape[-1])
+    if t2.stride(-1) != 1 and t2.shape[-1] > 1:
+        t2 = t2.contiguous()
+    return t2
+
+
+def add(a: torch.Tensor, b: torch.Tensor, shift: int = 0, rounding='floor', out: Optional[torch.Tensor] = None):
+    """Saturating elementwise add of two tensors that share shape and storage type."""
+    _dev(a, 'a'), _dev(b, 'b')
+    if a.shape != b.shape:
+        raise ValueError(f'elementwise Add requires exact-shape inputs, got {tuple(a.shape)} and {tuple(b.shape)}.')
+    if a.dtype != b.dtype or a.dtype not in _TORCH_KIND:
+        raise ValueError('elementwise Add requires lhs/rhs/output to use the same storage type.')
+    a, b = a.contiguous(), b.contiguous()
+    if out is None:
+        out = torch.empty_like(a)
+    check(_lib.load().a4g_add(_ptr(a), _ptr(b), _ptr(out), a.numel(), _TORCH_KIND[a.dtype], int(shift), _mode(rounding),
+                              _stream()))
+    return out
+
+
+@dataclass
+class PackedDense:
+    """Device-resident Dense parameters in the layout the GEMM kernel consumes."""
+
+    wt: torch.Tensor       # [N, ldwt] int8, reduction axis contiguous, zero padded
+    colsum: torch.Tensor   # [N] int32
+    bias: Optional[torch.Tensor]  # [N] int32 or None
+    shifts: torch.Tensor   # [1] or [N] int32
+    K: int
+    N: int
+
+    @property
+    def ldwt(self) -> int:
+        return int(self.wt.shape[1])
+
+
+def pack_dense(weight: torch.Tensor, bias: Optional[torch.Tensor], shifts) -> PackedDense:
+    """weight: logical [K, N] int8 on the device; bias: [N] int32 or None; shifts: int or [N] ints."""
+    _dev(weight, 'weight')
+    if weight.dtype != torch.int8 or weight.dim() != 2:
+        raise ValueError('weight matrix must be a rank-2 int8 tensor')
+    weight = weight.contiguous()
+    K, N = int(weight.shape[0]), int(weight.shape[1])
+    L = _lib.load()
+    ldwt = int(L.a4g_packed_ld(K))
+    wt = torch.empty((N, ldwt), dtype=torch.int8, device=weight.device)
+    colsum = torch.empty((N,), dtype=torch.int32, device=weight.device)
+    check(L.a4g_pack_weights_i8(_ptr(weight), N, K, N, _ptr(wt), _ptr(colsum), _stream()))
+    if bias is not None:
+        bias = _dev(bias, 'bias').to(torch.int32).contiguous()
+        if bias.numel() != N:
+            raise ValueError(f'dense bias requires exactly {N} elements, got {bias.numel()}.')
+    sh = torch.as_tensor(shifts, dtype=torch.int32).reshape(-1)
+    if sh.numel() not in (1, N):
+        raise ValueError(f'shifts must hold 1 or {N} entries, got {sh.numel()}')
+    if int(sh.min()) < 0 or int(sh.max()) > 31:
+        raise ValueError(f'dense accumulator output shift must be in [0, 31], got [{int(sh.min())}, {int(sh.max())}].')
+    return PackedDense(wt=wt, colsum=colsum, bias=bias, shifts=sh.to(weight.device), K=K, N=N)
+
+
+def dense(x: torch.Tensor, p: PackedDense, rounding='floor', relu: bool = False, out_kind='int8',
+          out: Optional[torch.Tensor] = None):
+    """y = saturate(round((x @ W + bias) >> shift)), optionally ReLU. x: [..., K] int8/uint8."""
+    x2 = _rows2d(x, 'x')
+    if x2.dtype not in (torch.int8, torch.uint8):
+        raise NotImplementedError(f'dense activations must be int8 or uint8, got {x2.dtype}')
+    if x2.shape[1] != p.K:
+        raise ValueError(f'dense input has {x2.shape[1]} features, weights expect {p.K}')
+    M = int(x2.shape[0])
+    ok = _kind(out_kind)
+    if out is None:
+        out = torch.empty(tuple(x.shape[:-1]) + (p.N,), dtype=_KIND_TORCH[ok], device=x.device)
+    y2 = out.reshape(-1, p.N)
+    check(_lib.load().a4g_dense_i8(_ptr(x2), _TORCH_KIND[x2.dtype], x2.stride(0) if M > 0 else p.K, _ptr(p.wt), p.ldwt,
+                                   _ptr(p.colsum), _ptr(p.bias), _ptr(p.shifts), int(p.shifts.numel()), _mode(rounding),
+                                   int(bool(relu)), ok, _ptr(y2), y2.stride(0) if M > 0 else p.N, M, p.N, p.K, _stream()))
+    return out
+
+
+def matmul(a: torch.Tensor, b: torch.Tensor, shift: int, rounding='floor', trans_b: bool = False, out_kind='int8',
+           out: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None):
+    """Batched dynamic MatMul. a: [..., M, K] int8/uint8; b: [..., K, N] int8, or [..., N, K] when
+    ``trans_b`` (the operand is consumed through a last-two-axes transpose view)."""
+    _dev(a, 'a'), _dev(b, 'b')
+    if b.dtype != torch.int8:
+        raise ValueError('matmul RHS must use a signed integer precision.')
+    if a.dtype not in (torch.int8, torch.uint8):
+        raise NotImplementedError(f'matmul LHS must be int8 or uint8, got {a.dtype}')
+    if a.dim() < 2 or b.dim() < 2:
+        raise ValueError('matmul operands need rank >= 2')
+    a, b = a.contiguous(), b.contiguous()
+    M, K = int(a.shape[-2]), int(a.shape[-1])
+    N = int(b.shape[-2] if trans_b else b.shape[-1])
+    Kb = int(b.shape[-1] if trans_b else b.shape[-2])
+    if K != Kb:
+        raise ValueError(f'matmul reduction extents differ: {K} vs {Kb}')
+    lead = tuple(a.shape[:-2])
+    if tuple(b.shape[:-2]) != lead:
+        raise ValueError(f'matmul leading axes differ: {lead} vs {tuple(b.shape[:-2])}')
+    batch = 1
+    for d in lead:
+        batch *= int(d)
+    ok = _kind(out_kind)
+    if out is None:
+        out = torch.empty(lead + (M, N), dtype=_KIND_TORCH[ok], device=a.device)
+    L = _lib.load()
+    akind = _TORCH_KIND[a.dtype]
+    need = int(L.a4g_matmul_i8_workspace_bytes(batch, M, N, K, int(trans_b), akind))
+    if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
+        workspace = torch.empty((need,), dtype=torch.uint8, device=a.device)
+    ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    check(L.a4g_matmul_i8(_ptr(a), akind, K, M * K, _ptr(b), int(b.shape[-1]), K * N, int(bool(trans_b)), _ptr(out), N,
+                          M * N, batch, M, N, K, int(shift), _mode(rounding), ok, _ptr(workspace), ws_bytes, _stream()))
+    return out
+
+
+def layernorm(x: torch.Tensor, gamma_q7: torch.Tensor, beta_q15: torch.Tensor, out_shift: int, rounding='floor',
+              eps_q0: int = 1, gamma_shift: int = 7, out: Optional[torch.Tensor] = None):
+    """Integer LayerNorm over the last axis, int8 -> int8. gamma int16 Q7, beta int16 Q15."""
+    x2 = _rows2d(x, 'x').contiguous()
+    if x2.dtype != torch.int8:
+        raise NotImplementedError('integer LayerNorm needs signed 8-bit input and output')
+    cols = int(x2.shape[1])
+    g = _dev(gamma_q7, 'gamma').to(torch.int16).contiguous()
+    b = _dev(beta_q15, 'beta').to(torch.int16).contiguous()
+    if g.numel() != cols or b.numel() != cols:
+        raise ValueError(f'LayerNorm parameter length does not match full_inner={cols}.')
+    if out is None:
+        out = torch.empty_like(x2).reshape(x.shape)
+    check(_lib.load().a4g_layernorm_i8(_ptr(x2), _ptr(g), _ptr(b), _ptr(out), int(x2.shape[0]), cols, int(eps_q0),
+                                       int(gamma_shift), int(out_shift), _mode(rounding), _stream()))
+    return out
+
+
+def add_layernorm(a: torch.Tensor, b: torch.Tensor, gamma_q7: torch.Tensor, beta_q15: torch.Tensor, out_shift: int,
+                  rounding='floor', eps_q0: int = 1, gamma_shift: int = 7, add_shift: int = 0, add_rounding='floor',
+                  return_sum: bool = False):
+    """Residual add fused in front of the LayerNorm (same result as add() then layernorm())."""
+    if a.shape != b.shape or a.dtype != torch.int8 or b.dtype != torch.int8:
+        raise ValueError('add_layernorm requires two int8 tensors of one shape')
+    a2 = _rows2d(a, 'a').contiguous()
+    b2 = _rows2d(b, 'b').contiguous()
+    cols = int(a2.shape[1])
+    g = _dev(gamma_q7, 'gamma').to(torch.int16).contiguous()
+    bt = _dev(beta_q15, 'beta').to(torch.int16).contiguous()
+    if g.numel() != cols or bt.numel() != cols:
+        raise ValueError(f'LayerNorm parameter length does not match full_inner={cols}.')
+    out = torch.empty_like(a2).reshape(a.shape)
+    s = torch.empty_like(a2).reshape(a.shape) if return_sum else None
+    check(_lib.load().a4g_add_layernorm_i8(_ptr(a2), _ptr(b2), int(add_shift), _mode(add_rounding), _ptr(g), _ptr(bt),
+                                           _ptr(s), _ptr(out), int(a2.shape[0]), cols, int(eps_q0), int(gamma_shift),
+                                           int(out_shift), _mode(rounding), _stream()))
+    return (s, out) if return_sum else out
+
+
+def softmax_exp(x: torch.Tensor, exp_kq: int, inv_shift: int = 15, out_kind='uint8', out: Optional[torch.Tensor] = None):
+    """Accurate integer-exp Softmax over the last axis: int8 -> uint8 (scale 1/256) or int16."""
+    x2 = _rows2d(x, 'x').contiguous()
+    if x2.dtype != torch.int8:
+        raise NotImplementedError('integer Softmax needs int8 input')
+    ok = _kind(out_kind)
+    if out is None:
+        out = torch.empty(x.shape, dtype=_KIND_TORCH.get(ok, torch.uint8), device=x.device)
+    check(_lib.load().a4g_softmax_exp_i8(_ptr(x2), _ptr(out), int(x2.shape[0]), int(x2.shape[1]), int(exp_kq),
+                                         int(inv_shift), ok, _stream()))
+    return out
+
+
+def softmax_hccs(x: torch.Tensor, B: int, S: int, Dmax: int, inv_shift: int = 15, use_clb: bool = False,
+                 out_kind='uint8', out: Optional[torch.Tensor] = None):
+    """HCCS clipped-linear surrogate Softmax over the last axis."""
+    x2 = _rows2d(x, 'x').contiguous()
+    if x2.dtype != torch.int8:
+        raise NotImplementedError('integer Softmax needs int8 input')
+    ok = _kind(out_kind)
+    if out is None:
+        out = torch.empty(x.shape, dtype=_KIND_TORCH.get(ok, torch.uint8), device=x.device)
+    check(_lib.load().a4g_softmax_hccs_i8(_ptr(x2), _ptr(out), int(x2.shape[0]), int(x2.shape[1]), int(B), int(S),
+                                          int(Dmax), int(inv_shift), int(bool(use_clb)), ok, _stream()))
+    return out
+
+
+@dataclass
+class MlpLayerSpec:
+    params: PackedDense
+    shift: int
+    relu: bool
+    out_kind: str = 'int8'
+
+
+def mlp(x: torch.Tensor, layers: Sequence[MlpLayerSpec], rounding='floor', out: Optional[torch.Tensor] = None):
+    """Whole MLP in one launch (weights resident in LDS). x: [batch, K0] int8/uint8."""
+    x2 = _rows2d(x, 'x').contiguous()
+    n = len(layers)
+    arr = (MlpLayer * max(n, 1))()
+    keep: List[torch.Tensor] = []
+    for i, spec in enumerate(layers):
+        p = spec.params
+        arr[i].wt = p.wt.data_ptr()
+        arr[i].ldwt = p.ldwt
+        arr[i].colsum = p.colsum.data_ptr()
+        arr[i].bias = p.bias.data_ptr() if p.bias is not None else None
+        arr[i].K, arr[i].N = p.K, p.N
+        arr[i].shift = int(spec.shift)
+        arr[i].relu = int(bool(spec.relu))
+        arr[i].out_kind = _kind(spec.out_kind)
+        keep.append(p.wt)
+    last = layers[-1]
+    ok = _kind(last.out_kind)
+    if out is None:
+        out = torch.empty((x2.shape[0], last.params.N), dtype=_KIND_TORCH[ok], device=x.device)
+    check(_lib.load().a4g_mlp_i8(arr, n, _ptr(x2), _TORCH_KIND[x2.dtype], x2.stride(0) if x2.shape[0] else x2.shape[1],
+                                 _ptr(out), out.stride(0) if out.shape[0] else last.params.N, int(x2.shape[0]),
+                                 _mode(rounding), _stream()))
+    return out

@@ -1,0 +1,266 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized-operator hot path on one MI355X.
+
+Default workload: the single quantized Dense of the baseline configuration
+(M=8192 rows x K=4096 -> N=4096, int32 bias, per-output-channel shift in [8,12], round-to-nearest-even,
+saturate to int8, fused ReLU). One step = one pass of the operator over the whole synthetic batch,
+inputs already resident in HBM. Prints ONE JSON line.
+
+Other workloads (--workload c1_mlp | c3_softmax_exp | c3_softmax_hccs | c3_qk | c3_pv |
+c4_add_layernorm | c4_layernorm | c4_add) print the same line for that operator.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+import numpy as np
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, TOP/s
+PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
+
+
+def _time_gpu(torch, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    ev0 = torch.cuda.Event(enable_timing=True)
+    ev1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    ev0.record()
+    for _ in range(steps):
+        fn()
+    ev1.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return wall_ms / steps, ev0.elapsed_time(ev1) / steps
+
+
+def _time_cpu(fn, budget_s=12.0, min_runs=2):
+    fn()  # warm
+    times = []
+    t_start = time.perf_counter()
+    while len(times) < min_runs or (time.perf_counter() - t_start < budget_s and len(times) < 7):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    return float(np.median(times))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=50)
+    ap.add_argument('--warmup', type=int, default=10)
+    ap.add_argument('--workload', default='c2_dense')
+    ap.add_argument('--no-cpu-baseline', action='store_true')
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit('bench.py: this build runs on exactly one GPU (every operator is row-independent; '
+                 'see DESIGN.md for how it would shard). Use --gpus 1.')
+
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.exit('bench.py: no GPU visible')
+    from aie4ml_amd import ops, workloads
+    from oracle import oracle
+
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()  # noqa: E731
+    wl = args.workload
+    extra = {}
+    cpu_fn = None
+
+    if wl == 'c2_dense':
+        M, K, N = 8192, 4096, 4096
+        A, W, bias, shifts = workloads.c2_dense(M, K, N)
+        p = ops.pack_dense(dev(W), dev(bias), shifts)
+        dA = dev(A)
+        out = torch.empty((M, N), dtype=torch.int8, device='cuda')
+        fn = lambda: ops.dense(dA, p, 'conv_even', relu=True, out=out)  # noqa: E731
+        fn()
+        # bit-exact gate on a row subset (rows are independent)
+        rows = np.random.default_rng(0).choice(M, 96, replace=False)
+        exp = oracle.dense(A[rows], W, bias, shifts, 'conv_even', relu=True)
+        torch.cuda.synchronize()
+        bit_exact = bool(np.array_equal(out[torch.from_numpy(rows).cuda()].cpu().numpy(), exp))
+        work, unit_work, bound = 2.0 * M * N * K, 'op', 'mfma'
+        samples = M
+        config = {'workload': 'c2_dense: Dense 8192x4096 -> 4096, int8, bias, per-channel shift 8..12, conv_even, '
+                              'sat int8, ReLU'}
+        sample_rows = 256
+        cpu_desc = f'oracle Dense on the first {sample_rows} of {M} rows (same W/bias/shifts), scaled per op'
+        cpu_fn = lambda: oracle.dense(A[:sample_rows], W, bias, shifts, 'conv_even', relu=True)  # noqa: E731
+        cpu_work = 2.0 * sample_rows * N * K
+        metric, unit = 'int8_dense_tops', 'TOP/s'
+        kernel = 'gemm_i8_nt_kernel'
+    elif wl == 'c1_mlp':
+        x, layers = workloads.c1_mlp(1024)
+        specs = [ops.MlpLayerSpec(ops.pack_dense(dev(Wl), dev(b), s), s, relu, o) for (Wl, b, s, relu, o) in layers]
+        dx = dev(x)
+        out = torch.empty((1024, 5), dtype=torch.int8, device='cuda')
+        fn = lambda: ops.mlp(dx, specs, 'positive_inf', out=out)  # noqa: E731
+        fn()
+        torch.cuda.synchronize()
+        bit_exact = bool(np.array_equal(out.cpu().numpy(), oracle.mlp(x, layers, 'positive_inf')))
+        work, bound = 8512.0 * 1024, 'mfma'
+        samples = 1024
+        config = {'workload': 'c1_mlp: int8 MLP 16-64-32-32-5, batch 1024, shift 7, round half up, fused single launch'}
+        cpu_desc = 'oracle MLP (layer by layer) on the full batch of 1024'
+        cpu_fn = lambda: oracle.mlp(x, layers, 'positive_inf')  # noqa: E731
+        cpu_work = work
+        metric, unit = 'int8_mlp_samples_per_s', 'samples/s'
+        kernel = 'mlp_fused_kernel'
+    elif wl in ('c4_add_layernorm', 'c4_layernorm', 'c4_add'):
+        rows, cols = 16384, 1024
+        a, b, gamma, beta, prm = workloads.c4_add_layernorm(rows, cols)
+        da, db, dg, dbt = dev(a), dev(b), dev(gamma), dev(beta)
+        sub = slice(0, 512)
+        if wl == 'c4_add_layernorm':
+            fn = lambda: ops.add_layernorm(da, db, dg, dbt, prm['out_shift'], 'conv_even')  # noqa: E731
+            got = fn()
+            exp = oracle.add_layernorm(a[sub], b[sub], gamma, beta, prm['out_shift'], 'conv_even')
+            work = 3.0 * rows * cols
+            cpu_fn = lambda: oracle.add_layernorm(a, b, gamma, beta, prm['out_shift'], 'conv_even')  # noqa: E731
+            kernel = 'layernorm_wave_kernel'
+        elif wl == 'c4_layernorm':
+            fn = lambda: ops.layernorm(da, dg, dbt, prm['out_shift'], 'conv_even')  # noqa: E731
+            got = fn()
+            exp = oracle.layernorm(a[sub], gamma, beta, prm['out_shift'], 'conv_even')
+            work = 2.0 * rows * cols
+            cpu_fn = lambda: oracle.layernorm(a, gamma, beta, prm['out_shift'], 'conv_even')  # noqa: E731
+            kernel = 'layernorm_wave_kernel'
+        else:
+            fn = lambda: ops.add(da, db)  # noqa: E731
+            got = fn()
+            exp = oracle.add(a[sub], b[sub])
+            work = 3.0 * rows * cols
+            cpu_fn = lambda: oracle.add(a, b)  # noqa: E731
+            kernel = 'add_sat8_kernel'
+        torch.cuda.synchronize()
+        bit_exact = bool(np.array_equal(got[sub].cpu().numpy(), exp))
+        bound, samples = 'hbm', rows
+        cpu_work = work
+        cpu_desc = f'oracle {wl} on the full [{rows},{cols}] tensor'
+        config = {'workload': f'{wl}: [{rows},{cols}] int8, conv_even, out frac 5'}
+        metric, unit = f'{wl}_gbs', 'GB/s'
+    elif wl in ('c3_softmax_exp', 'c3_softmax_hccs', 'c3_qk', 'c3_pv'):
+        Bt, H, S, D = 32, 16, 512, 64
+        q, k, v, prm = workloads.c3_attention(Bt, H, S, D)
+        dq, dk, dv = dev(q), dev(k), dev(v)
+        logits = ops.matmul(dq, dk, prm['logit_shift'], 'conv_even', trans_b=True)
+        probs = ops.softmax_exp(logits, prm['exp_kq'])
+        torch.cuda.synchronize()
+        hb = (0, 3)  # one (batch, head) slice for the bit-exact gate
+        l_ref = oracle.matmul(q[hb], k[hb], prm['logit_shift'], 'conv_even', trans_b=True)
+        if wl == 'c3_qk':
+            out = torch.empty_like(logits)
+            fn = lambda: ops.matmul(dq, dk, prm['logit_shift'], 'conv_even', trans_b=True, out=out)  # noqa: E731
+            fn()
+            torch.cuda.synchronize()
+            bit_exact = bool(np.array_equal(out[hb].cpu().numpy(), l_ref))
+            work, bound = 2.0 * Bt * H * S * S * D, 'hbm'
+            bytes_ = Bt * H * (2 * S * D + S * S)
+            extra['tops'] = None
+            cpu_fn = lambda: oracle.matmul(q[0, :4], k[0, :4], prm['logit_shift'], 'conv_even', trans_b=True)  # noqa: E731
+            cpu_work = bytes_ * 4 / (Bt * H)
+            cpu_desc = 'oracle MatMul on 4 of 512 (batch, head) slices'
+            work = float(bytes_)
+            kernel = 'gemm_i8_nt_kernel'
+        elif wl == 'c3_pv':
+            ws = torch.empty((ops._lib.load().a4g_matmul_i8_workspace_bytes(Bt * H, S, D, S, 0, 1),), dtype=torch.uint8,
+                             device='cuda')
+            out = torch.empty((Bt, H, S, D), dtype=torch.int8, device='cuda')
+            fn = lambda: ops.matmul(probs, dv, prm['pv_shift'], 'conv_even', out=out, workspace=ws)  # noqa: E731
+            fn()
+            torch.cuda.synchronize()
+            p_ref = oracle.softmax_exp(l_ref, prm['exp_kq'])
+            bit_exact = bool(np.array_equal(out[hb].cpu().numpy(), oracle.matmul(p_ref, v[hb], prm['pv_shift'], 'conv_even')))
+            bytes_ = Bt * H * (S * S + 2 * S * D)
+            work, bound = float(bytes_), 'hbm'
+            pl = probs[0, :4].cpu().numpy()
+            cpu_fn = lambda: oracle.matmul(pl, v[0, :4], prm['pv_shift'], 'conv_even')  # noqa: E731
+            cpu_work = bytes_ * 4 / (Bt * H)
+            cpu_desc = 'oracle MatMul (uint8 x int8) on 4 of 512 (batch, head) slices'
+            kernel = 'gemm_i8_nt_kernel'
+        else:
+            out = torch.empty(logits.shape, dtype=torch.uint8, device='cuda')
+            hc = prm['hccs']
+            if wl == 'c3_softmax_exp':
+                fn = lambda: ops.softmax_exp(logits, prm['exp_kq'], out=out)  # noqa: E731
+                ref = oracle.softmax_exp(l_ref, prm['exp_kq'])
+                cpu1 = lambda x_: oracle.softmax_exp(x_, prm['exp_kq'])  # noqa: E731
+            else:
+                fn = lambda: ops.softmax_hccs(logits, hc['B'], hc['S'], hc['Dmax'], out=out)  # noqa: E731
+                ref = oracle.softmax_hccs(l_ref, hc['B'], hc['S'], hc['Dmax'])
+                cpu1 = lambda x_: oracle.softmax_hccs(x_, hc['B'], hc['S'], hc['Dmax'])  # noqa: E731
+            fn()
+            torch.cuda.synchronize()
+            bit_exact = bool(np.array_equal(out[hb].cpu().numpy(), ref))
+            work, bound = 2.0 * Bt * H * S * S, 'hbm'
+            lsub = logits[:2].cpu().numpy()
+            cpu_fn = lambda: cpu1(lsub)  # noqa: E731
+            cpu_work = 2.0 * 2 * H * S * S
+            cpu_desc = 'oracle softmax on 2 of 32 batches (16384 of 262144 rows)'
+            kernel = 'softmax_lut_kernel'
+        samples = Bt
+        config = {'workload': f'{wl}: attention core batch 32 x 16 heads, seq 512, head_dim 64'}
+        metric, unit = f'{wl}_gbs', 'GB/s'
+    else:
+        sys.exit(f'unknown workload {wl}')
+
+    ms_wall, ms_ev = _time_gpu(torch, fn, args.steps, args.warmup)
+    ms = max(ms_wall, ms_ev)
+    if bound == 'mfma':
+        achieved = work / (ms_ev * 1e-3) / 1e12
+        roof = {'bound': 'mfma', 'achieved': round(achieved, 3), 'peak': PEAK_INT8_TOPS, 'unit': 'TOP/s',
+                'frac': round(achieved / PEAK_INT8_TOPS, 4), 'traffic': None, 'kernel': kernel,
+                'kernel_ms': round(ms_ev, 5)}
+    else:
+        achieved = work / (ms_ev * 1e-3) / 1e9
+        roof = {'bound': 'hbm', 'achieved': round(achieved, 2), 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
+                'frac': round(achieved / PEAK_HBM_GBS, 4), 'traffic': None, 'kernel': kernel,
+                'kernel_ms': round(ms_ev, 5)}
+
+    if unit == 'TOP/s':
+        value = work / (ms * 1e-3) / 1e12
+    elif unit == 'GB/s':
+        value = work / (ms * 1e-3) / 1e9
+    else:
+        value = samples / (ms * 1e-3)
+
+    cpu = None
+    if cpu_fn is not None and not args.no_cpu_baseline:
+        t = _time_cpu(cpu_fn)
+        if unit == 'TOP/s':
+            v = cpu_work / t / 1e12
+        elif unit == 'GB/s':
+            v = cpu_work / t / 1e9
+        else:
+            v = samples / t
+        cpu = {'value': float(f'{v:.6g}'), 'unit': unit, 'cores': oracle.num_threads(), 'kind': 'port',
+               'sample': cpu_desc, 'host_cpus': os.cpu_count()}
+
+    line = {
+        'metric': metric, 'value': float(f'{value:.6g}'), 'unit': unit, 'n_gpus': 1, 'steps': args.steps,
+        'warmup': args.warmup, 'ms_per_step': round(ms, 5), 'higher_is_better': True, 'scaling': 'weak',
+        'vs_baseline': None, 'dtype': 'int8', 'data': 'synthetic', 'config': config,
+        'samples_per_s': float(f'{samples / (ms * 1e-3):.6g}'), 'bit_exact': bit_exact,
+        'roofline': roof, 'cpu_baseline': cpu,
+    }
+    line.update(extra)
+    print(json.dumps(line), flush=True)
+    if not bit_exact:
+        sys.exit('bench.py: GPU result differs from the oracle — throughput above is INVALID')
+
+
+if __name__ == '__main__':
+    main()

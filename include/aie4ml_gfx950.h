@@ -1,0 +1,183 @@
+/*
+ * aie4ml_gfx950.h — C ABI of libaie4ml_gfx950.so: the quantized operators aie4ml lowers
+ * (Dense/GEMM + ReLU, dynamic MatMul, elementwise Add, integer LayerNorm, integer Softmax in its
+ * accurate and HCCS-surrogate forms), executed on one AMD Instinct MI355X (gfx950).
+ *
+ * Conventions
+ *  - Every pointer is a DEVICE pointer owned by the caller unless the comment says "host".
+ *    The library never allocates, frees or copies to the host. Work is enqueued on `stream`
+ *    (a hipStream_t passed as void*; NULL = the default stream) and the call returns without
+ *    synchronising.
+ *  - Tensors are plain row-major; `ld*` are row pitches in ELEMENTS, `stride_*` batch pitches in
+ *    elements.
+ *  - Return value: A4G_OK (0) or a negative a4g_status. a4g_last_error() returns a host string
+ *    describing the last failure on the calling thread. Arguments are validated before any launch.
+ *  - Results are bit-exact restatements of the reference's AIE kernels under
+ *    aie::saturation_mode::saturate and the given aie::rounding_mode.
+ *
+ * The reference interface each entry point replaces is cited as file:line under
+ * src/aie4ml/ of dimdano/aie4ml.
+ */
+#ifndef AIE4ML_GFX950_H
+#define AIE4ML_GFX950_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define A4G_VERSION 100 /* major*10000 + minor*100 + patch */
+
+#if defined(__GNUC__)
+#define A4G_API __attribute__((visibility("default")))
+#else
+#define A4G_API
+#endif
+
+typedef void* a4g_stream_t; /* hipStream_t */
+
+enum a4g_status {
+    A4G_OK = 0,
+    A4G_ERR_INVALID_ARGUMENT = -1, /* the reference would raise ValueError */
+    A4G_ERR_UNSUPPORTED = -2,      /* the reference would raise NotImplementedError */
+    A4G_ERR_WORKSPACE = -3,        /* workspace missing or too small */
+    A4G_ERR_HIP = -4               /* a HIP runtime call failed (RuntimeError) */
+};
+
+/* aie::rounding_mode tokens, as produced by ROUNDING_TOKEN_MAP (op_impls/utils/precision.py:13-21).
+ * positive_inf ("round half up"), negative_inf and conv_odd are AIE-API modes the reference
+ * never emits; they are accepted for completeness. */
+enum a4g_rounding {
+    A4G_RND_FLOOR = 0,
+    A4G_RND_CEIL = 1,
+    A4G_RND_POSITIVE_INF = 2,
+    A4G_RND_NEGATIVE_INF = 3,
+    A4G_RND_SYMMETRIC_INF = 4,
+    A4G_RND_SYMMETRIC_ZERO = 5,
+    A4G_RND_CONV_EVEN = 6,
+    A4G_RND_CONV_ODD = 7
+};
+
+/* storage kinds (AIEDataType.format, aie_types.py:42-90) */
+enum a4g_kind { A4G_I8 = 0, A4G_U8 = 1, A4G_I16 = 2, A4G_U16 = 3, A4G_I32 = 4 };
+
+A4G_API int a4g_version(void);
+A4G_API const char* a4g_last_error(void);
+
+/* ---- Elementwise Add ---------------------------------------------------------------------------
+ * out[i] = srs(a[i] + b[i], shift, round_mode) saturated to `kind` (int8 / uint8 / int16).
+ * Replaces elementwise_add_kernel<Cfg>::run, templates/nnet_utils/elementwise_add/
+ * elementwise_add.cpp:12-37, configured by AddOpImplVariant.resolve
+ * (op_impls/families/elementwise/add.py:57-164: SHIFT, ROUNDING). */
+A4G_API int a4g_add(const void* a, const void* b, void* out, int64_t n, int kind, int shift, int round_mode,
+            a4g_stream_t stream);
+
+/* ---- Dense weights -----------------------------------------------------------------------------
+ * Packs a logical [K][N] int8 weight matrix (row pitch ldw) into the layout the GEMM consumes:
+ * Wt[N][ldwt] with the reduction axis contiguous and zero-padded to ldwt = a4g_packed_ld(K), plus
+ * colsum[n] = sum_k W[k][n] (needed when the activations are uint8). Device-side; replaces
+ * pack_mmul_rhs_matrix (op_impls/families/matmul/common.py:307-358), which lays the same matrix
+ * out in aie::mmul microtiles. */
+A4G_API int64_t a4g_packed_ld(int64_t K);
+A4G_API int a4g_pack_weights_i8(const int8_t* W, int64_t ldw, int64_t K, int64_t N, int8_t* Wt, int32_t* colsum,
+                        a4g_stream_t stream);
+
+/* ---- Dense (GEMM + bias + requantise + ReLU) ----------------------------------------------------
+ * acc32 = bias[n] + sum_k A[m][k] * W[k][n];  y = saturate(round(acc >> shift));  relu: y = max(y,0).
+ * Replaces dense_single/first/middle/last<Cfg>::run, templates/nnet_utils/dense_bias_relu/
+ * dense_bias_relu.cpp:66-430, configured by _DenseVariantBase.resolve
+ * (op_impls/families/matmul/dense.py:94-133) through variants/dense_bias_relu/parameters.h.jinja.
+ *   A       [M][lda]  int8 or uint8 (a_kind)
+ *   Wt      packed weights from a4g_pack_weights_i8, pitch ldwt
+ *   colsum  [N] from a4g_pack_weights_i8; required iff a_kind == A4G_U8, else may be NULL
+ *   bias    [N] int32 at accumulator scale, or NULL (USE_BIAS = false)
+ *   shifts  [n_shift] int32 on the device; n_shift == 1 (the reference's scalar SHIFT) or == N
+ *           (per-output-channel extension; identical to the reference when all entries are equal)
+ *   Y       [M][ldy]  out_kind in {A4G_I8, A4G_U8, A4G_I16} */
+A4G_API int a4g_dense_i8(const void* A, int a_kind, int64_t lda, const int8_t* Wt, int64_t ldwt,
+                 const int32_t* colsum, const int32_t* bias, const int32_t* shifts, int n_shift,
+                 int round_mode, int relu, int out_kind, void* Y, int64_t ldy, int64_t M, int64_t N,
+                 int64_t K, a4g_stream_t stream);
+
+/* ---- Dynamic MatMul (both operands activations) --------------------------------------------------
+ * C[b] = saturate(round((A[b] x B[b]) >> shift)), no bias, no ReLU, for b in [0, batch).
+ * Replaces matmul_single/first/middle/last<Cfg>::run, templates/nnet_utils/matmul/matmul.cpp:31-390,
+ * configured by _MatmulVariantBase.resolve (op_impls/families/matmul/matmul.py:47-98).
+ *   A  [batch][M][lda]  int8 or uint8 (a_kind; uint8 = softmax probabilities)
+ *   B  signed int8 (matmul.py:96-98). trans_b == 0: [batch][K][ldb] (logical K x N).
+ *      trans_b == 1: [batch][N][ldb] — the operand arrives as the last-two-axes transpose of the
+ *      producer tensor (io_view perm, matmul.py:86-95 / TRANSPOSE_B, matmul.cpp:70-76).
+ *   C  [batch][M][ldc]  out_kind in {A4G_I8, A4G_U8, A4G_I16}
+ * The reference accepts only batch == 1 for B (matmul/resolver.py:440-463); larger batches are
+ * independent per-slice products. `workspace` must hold a4g_matmul_i8_workspace_bytes(...) bytes
+ * (0 for some argument combinations, in which case it may be NULL). */
+A4G_API size_t a4g_matmul_i8_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int trans_b, int a_kind);
+A4G_API int a4g_matmul_i8(const void* A, int a_kind, int64_t lda, int64_t stride_a, const int8_t* B, int64_t ldb,
+                  int64_t stride_b, int trans_b, void* C, int64_t ldc, int64_t stride_c, int64_t batch,
+                  int64_t M, int64_t N, int64_t K, int shift, int round_mode, int out_kind, void* workspace,
+                  size_t workspace_bytes, a4g_stream_t stream);
+
+/* ---- Integer LayerNorm, int8 -> int8, over the last axis -------------------------------------------
+ * Replaces layernorm_i8<Cfg>::run / layernorm_i8_tiled<Cfg>::run and
+ * layernorm_base<Cfg>::row_statistics, templates/nnet_utils/layer_norm/layer_norm.cpp:14-231,
+ * configured by _LayerNormVariantBase.resolve (op_impls/families/layernorm/layer_norm.py:94-167).
+ *   gamma  [cols] int16 Q7, beta [cols] int16 Q15 (layernorm/common.py:19-20)
+ *   eps_q0 >= 1; gamma_shift = 7; out_shift in [0,15] = the output's fractional bits.
+ * cols need not be a power of two (the reference requires it): mean and variance use exact floor
+ * division, equal to the reference's shifts when cols is 2^k. */
+A4G_API int a4g_layernorm_i8(const int8_t* x, const int16_t* gamma, const int16_t* beta, int8_t* out, int64_t rows,
+                     int64_t cols, int32_t eps_q0, int gamma_shift, int out_shift, int round_mode,
+                     a4g_stream_t stream);
+
+/* Residual add fused in front of the LayerNorm: s = saturate_i8(round((a + b) >> add_shift));
+ * out = layernorm(s). sum_out (nullable) receives s. Equals a4g_add followed by a4g_layernorm_i8
+ * (the reference runs the two kernels back to back through a memory tile). */
+A4G_API int a4g_add_layernorm_i8(const int8_t* a, const int8_t* b, int add_shift, int add_round_mode,
+                         const int16_t* gamma, const int16_t* beta, int8_t* sum_out, int8_t* out, int64_t rows,
+                         int64_t cols, int32_t eps_q0, int gamma_shift, int out_shift, int round_mode,
+                         a4g_stream_t stream);
+
+/* ---- Integer Softmax over the last axis, int8 -> uint8 (scale 1/256) or int16 -----------------------
+ * Accurate form: 2nd-order integer exp. Replaces softmax_exp_i8<Cfg>::run /
+ * softmax_exp_i8_tiled<Cfg>::run, exp_score16 and softmax_base<Cfg>::batched_reciprocal,
+ * templates/nnet_utils/softmax/softmax.cpp:108-127,252-384, configured by
+ * _SoftmaxExpBase._resolve_params (op_impls/families/softmax/softmax.py:309-349).
+ *   exp_kq in [1,128]; inv_shift in [1,21] (the reference always uses 15). */
+A4G_API int a4g_softmax_exp_i8(const int8_t* x, void* out, int64_t rows, int64_t cols, int exp_kq, int inv_shift,
+                       int out_kind, a4g_stream_t stream);
+
+/* HCCS clipped-linear surrogate: score = B - S*min(max-x, Dmax). Replaces
+ * softmax_i8<Cfg>::softmax_row/run and softmax_i8_tiled<Cfg>::run,
+ * templates/nnet_utils/softmax/softmax.cpp:19-239, configured by _SoftmaxHccsBase._resolve_params
+ * (op_impls/families/softmax/softmax.py:258-283) under the constraints of validate_hccs_params
+ * (op_impls/families/softmax/common.py:59-89), which this call re-checks. inv_shift in [1,23]. */
+A4G_API int a4g_softmax_hccs_i8(const int8_t* x, void* out, int64_t rows, int64_t cols, int B, int S, int Dmax,
+                        int inv_shift, int use_clb, int out_kind, a4g_stream_t stream);
+
+/* ---- Fused multi-layer perceptron ---------------------------------------------------------------------
+ * A chain of Dense layers evaluated in one launch with every weight matrix resident in LDS; same
+ * arithmetic as calling a4g_dense_i8 per layer (scalar shift per layer). Replaces the chain of
+ * dense_bias_relu_graph instances the reference wires for an hls4ml MLP
+ * (templates/nnet_utils/dense_bias_relu/dense_bias_relu_graph.h:12-134).
+ * `layers` is a HOST array. Limits: n_layers <= 8, every K and N <= 256, packed weights <= 96 KiB in
+ * total; beyond them the call returns A4G_ERR_UNSUPPORTED and the caller runs layer by layer. */
+typedef struct a4g_mlp_layer {
+    const int8_t* wt;      /* packed weights (a4g_pack_weights_i8), pitch ldwt */
+    int64_t ldwt;
+    const int32_t* colsum; /* required iff the layer's input is uint8 */
+    const int32_t* bias;   /* nullable */
+    int32_t K, N;
+    int32_t shift;
+    int32_t relu;
+    int32_t out_kind;      /* A4G_I8 or A4G_U8; becomes the next layer's input kind */
+} a4g_mlp_layer;
+
+A4G_API int a4g_mlp_i8(const a4g_mlp_layer* layers, int n_layers, const void* X, int x_kind, int64_t ldx, void* Y,
+               int64_t ldy, int64_t batch, int round_mode, a4g_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AIE4ML_GFX950_H */

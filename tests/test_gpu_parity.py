@@ -1,0 +1,362 @@
+"""GPU parity: every operator, through the C ABI, bit-exact against the CPU oracle on seeded inputs.
+
+Sizes are chosen so the oracle finishes in seconds; the full benchmark shapes are covered by row
+subsets (every operator is row-independent) in test_gpu_configs.py.
+"""
+
+import numpy as np
+import pytest
+
+torch = pytest.importorskip('torch')
+
+pytestmark = pytest.mark.gpu
+
+MODES = ['floor', 'ceil', 'positive_inf', 'negative_inf', 'symmetric_inf', 'symmetric_zero', 'conv_even',
+         'conv_odd']
+REF_MODES = ['floor', 'symmetric_inf', 'conv_even', 'positive_inf']
+
+
+@pytest.fixture(scope='module')
+def ops():
+    if not torch.cuda.is_available():
+        pytest.skip('no GPU')
+    from aie4ml_amd import ops as _ops
+
+    return _ops
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+def gauss8(r, sigma, shape):
+    return np.clip(np.rint(r.normal(0, sigma, shape)), -128, 127).astype(np.int8)
+
+
+# ---- Add ------------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize('n', [0, 1, 15, 16, 4096 + 3, 1 << 20])
+@pytest.mark.parametrize('dtype', [np.int8, np.uint8])
+def test_add_saturating(ops, oracle, n, dtype):
+    r = rng(n + 1)
+    lo, hi = (0, 256) if dtype == np.uint8 else (-128, 128)
+    a = r.integers(lo, hi, n).astype(dtype)
+    b = r.integers(lo, hi, n).astype(dtype)
+    got = host(ops.add(dev(a), dev(b)))
+    assert np.array_equal(got, oracle.add(a, b))
+
+
+def test_add_exhaustive_pairs(ops, oracle):
+    a = np.arange(-128, 128, dtype=np.int8).repeat(256)
+    b = np.tile(np.arange(-128, 128, dtype=np.int8), 256)
+    assert np.array_equal(host(ops.add(dev(a), dev(b))), oracle.add(a, b))
+    au, bu = a.view(np.uint8), b.view(np.uint8)
+    assert np.array_equal(host(ops.add(dev(au), dev(bu))), oracle.add(au, bu))
+
+
+@pytest.mark.parametrize('mode', MODES)
+def test_add_shift_and_modes(ops, oracle, mode):
+    r = rng(3)
+    a = r.integers(-128, 128, 5000).astype(np.int8)
+    b = r.integers(-128, 128, 5000).astype(np.int8)
+    for shift in (1, 2):
+        assert np.array_equal(host(ops.add(dev(a), dev(b), shift, mode)), oracle.add(a, b, shift, mode))
+    a16 = r.integers(-32768, 32768, 3001).astype(np.int16)
+    b16 = r.integers(-32768, 32768, 3001).astype(np.int16)
+    assert np.array_equal(host(ops.add(dev(a16), dev(b16), 0, mode)), oracle.add(a16, b16, 0, mode))
+
+
+def test_add_unaligned_views(ops, oracle):
+    r = rng(4)
+    a = r.integers(-128, 128, 10007).astype(np.int8)
+    b = r.integers(-128, 128, 10007).astype(np.int8)
+    ta, tb = dev(a)[3:10003], dev(b)[5:10005]
+    got = host(ops.add(ta, tb))
+    assert np.array_equal(got, oracle.add(a[3:10003], b[5:10005]))
+
+
+# ---- Dense ----------------------------------------------------------------------------------------------
+
+def run_dense(ops, oracle, M, K, N, mode, a_dtype=np.int8, relu=True, per_channel=True, out='int8', bias=True,
+              seed=0):
+    r = rng(seed)
+    if a_dtype == np.uint8:
+        A = r.integers(0, 256, (M, K)).astype(np.uint8)
+    else:
+        A = gauss8(r, 40, (M, K))
+    W = gauss8(r, 30, (K, N))
+    b = r.integers(-2**14, 2**14, N).astype(np.int32) if bias else None
+    if per_channel:
+        shifts = r.integers(5, 11, N).astype(np.int32)
+    else:
+        shifts = np.array([7], dtype=np.int32)
+    p = ops.pack_dense(dev(W), dev(b) if bias else None, shifts)
+    got = host(ops.dense(dev(A), p, mode, relu=relu, out_kind=out))
+    exp = oracle.dense(A, W, b, shifts if per_channel else 7, mode, relu=relu, out=out)
+    assert got.dtype == exp.dtype
+    assert np.array_equal(got, exp), f'mismatch at {np.argwhere(got != exp)[:5]}'
+
+
+@pytest.mark.parametrize('shape', [(1, 16, 1), (7, 16, 5), (64, 64, 64), (130, 96, 70), (256, 256, 256),
+                                   (300, 128, 260), (33, 1024, 17), (512, 80, 384), (1024, 16, 64)])
+def test_dense_shapes_mfma_path(ops, oracle, shape):
+    M, K, N = shape
+    run_dense(ops, oracle, M, K, N, 'conv_even', seed=M + K + N)
+
+
+@pytest.mark.parametrize('shape', [(5, 3, 2), (64, 17, 33), (9, 100, 12), (128, 250, 64)])
+def test_dense_ragged_k_generic_path(ops, oracle, shape):
+    M, K, N = shape
+    run_dense(ops, oracle, M, K, N, 'symmetric_inf', seed=M * K + N)
+    run_dense(ops, oracle, M, K, N, 'conv_even', a_dtype=np.uint8, seed=M * K + N + 1)
+
+
+@pytest.mark.parametrize('mode', MODES)
+def test_dense_rounding_modes(ops, oracle, mode):
+    run_dense(ops, oracle, 96, 64, 96, mode, relu=False, seed=11)
+    run_dense(ops, oracle, 96, 64, 96, mode, relu=True, per_channel=False, seed=12)
+
+
+@pytest.mark.parametrize('out', ['int8', 'uint8', 'int16'])
+@pytest.mark.parametrize('a_dtype', [np.int8, np.uint8])
+def test_dense_kinds(ops, oracle, out, a_dtype):
+    run_dense(ops, oracle, 200, 128, 136, 'conv_even', a_dtype=a_dtype, relu=False, out=out, seed=21)
+    run_dense(ops, oracle, 200, 128, 136, 'floor', a_dtype=a_dtype, relu=True, out=out, bias=False, seed=22)
+
+
+def test_dense_ties_saturation_identity(ops, oracle):
+    K = 64
+    A = rng(5).integers(-128, 128, (32, K)).astype(np.int8)
+    eye = np.eye(K, dtype=np.int8)
+    p = ops.pack_dense(dev(eye), None, 0)
+    assert np.array_equal(host(ops.dense(dev(A), p, 'floor')), A)
+    # W = 0 -> out = srs(bias): exact ties +-2^(s-1), saturation at the int32 extremes
+    bias = np.array([64, -64, 63, -65, 192, -192, 2**31 - 1, -2**31] * 8, dtype=np.int32)
+    p = ops.pack_dense(dev(np.zeros((K, K), np.int8)), dev(bias), 7)
+    for mode in MODES:
+        got = host(ops.dense(dev(A), p, mode))
+        assert np.array_equal(got, oracle.dense(A, np.zeros((K, K), np.int8), bias, 7, mode)), mode
+
+
+def test_dense_accumulator_wraps(ops, oracle):
+    K, N = 4096, 64
+    A = np.full((40, K), 127, np.int8)
+    W = np.full((K, N), 127, np.int8)
+    bias = np.full(N, 2**31 - 1, np.int32)
+    p = ops.pack_dense(dev(W), dev(bias), 12)
+    got = host(ops.dense(dev(A), p, 'conv_even'))
+    assert np.array_equal(got, oracle.dense(A, W, bias, 12, 'conv_even'))
+
+
+def test_dense_nd_input_and_empty(ops, oracle):
+    r = rng(6)
+    A = gauss8(r, 30, (3, 5, 32))
+    W = gauss8(r, 30, (32, 48))
+    p = ops.pack_dense(dev(W), None, 6)
+    got = host(ops.dense(dev(A), p, 'conv_even'))
+    assert got.shape == (3, 5, 48)
+    assert np.array_equal(got.reshape(15, 48), oracle.dense(A.reshape(15, 32), W, None, 6, 'conv_even'))
+    empty = ops.dense(torch.empty((0, 32), dtype=torch.int8, device='cuda'), p, 'conv_even')
+    assert tuple(empty.shape) == (0, 48)
+
+
+# ---- MatMul ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize('trans_b', [True, False])
+@pytest.mark.parametrize('shape', [((2, 3), 64, 64, 64), ((4,), 128, 96, 32), ((), 130, 70, 48), ((2,), 50, 17, 24),
+                                   ((3,), 33, 64, 19)])
+def test_matmul_batched(ops, oracle, shape, trans_b):
+    lead, M, N, K = shape
+    r = rng(M + N + K)
+    A = gauss8(r, 24, lead + (M, K))
+    B = gauss8(r, 24, lead + ((N, K) if trans_b else (K, N)))
+    for mode in ('conv_even', 'symmetric_inf'):
+        got = host(ops.matmul(dev(A), dev(B), 6, mode, trans_b=trans_b))
+        assert np.array_equal(got, oracle.matmul(A, B, 6, mode, trans_b=trans_b))
+
+
+@pytest.mark.parametrize('trans_b', [True, False])
+def test_matmul_unsigned_lhs(ops, oracle, trans_b):
+    r = rng(9)
+    P = r.integers(0, 256, (2, 4, 96, 128)).astype(np.uint8)
+    V = gauss8(r, 24, (2, 4) + ((64, 128) if trans_b else (128, 64)))
+    for out in ('int8', 'int16'):
+        got = host(ops.matmul(dev(P), dev(V), 8, 'conv_even', trans_b=trans_b, out_kind=out))
+        assert np.array_equal(got, oracle.matmul(P, V, 8, 'conv_even', trans_b=trans_b, out=out))
+
+
+def test_matmul_rejects_bad_arguments(ops):
+    a = torch.zeros((2, 16, 16), dtype=torch.int8, device='cuda')
+    with pytest.raises(ValueError):
+        ops.matmul(a, a.to(torch.uint8), 0)  # RHS must be signed
+    with pytest.raises(ValueError):
+        ops.matmul(a, a, 40)  # shift out of range
+
+
+# ---- LayerNorm ------------------------------------------------------------------------------------------
+
+def ln_params(r, cols):
+    gamma = r.integers(32, 128, cols).astype(np.int16)
+    beta = (r.integers(-16, 17, cols).astype(np.int32) << 10).astype(np.int16)
+    return gamma, beta
+
+
+@pytest.mark.parametrize('cols', [16, 32, 128, 768, 1024, 2048, 4096, 48, 100, 8192])
+def test_layernorm_columns(ops, oracle, cols):
+    r = rng(cols)
+    rows = 37
+    x = gauss8(r, 20, (rows, cols)) + np.int8(3)
+    gamma, beta = ln_params(r, cols)
+    for mode in ('conv_even', 'symmetric_inf'):
+        got = host(ops.layernorm(dev(x), dev(gamma), dev(beta), 5, mode))
+        assert np.array_equal(got, oracle.layernorm(x, gamma, beta, 5, mode)), (cols, mode)
+
+
+@pytest.mark.parametrize('mode', MODES)
+def test_layernorm_modes_and_shifts(ops, oracle, mode):
+    r = rng(31)
+    x = gauss8(r, 35, (64, 256))
+    gamma = r.integers(-256, 256, 256).astype(np.int16)
+    beta = r.integers(-32768, 32768, 256).astype(np.int16)
+    for out_shift in (0, 4, 7, 15):
+        got = host(ops.layernorm(dev(x), dev(gamma), dev(beta), out_shift, mode, eps_q0=3))
+        assert np.array_equal(got, oracle.layernorm(x, gamma, beta, out_shift, mode, eps_q0=3)), (mode, out_shift)
+
+
+def test_layernorm_degenerate_rows(ops, oracle):
+    cols = 1024
+    r = rng(32)
+    gamma = np.full(cols, 32767, np.int16)  # forces the int16 saturation of inv_std * gamma
+    beta = r.integers(-32768, 32768, cols).astype(np.int16)
+    x = np.zeros((6, cols), np.int8)
+    x[0] = 17                      # constant row: variance 0
+    x[1, :cols // 2] = 1           # mean rounds half up
+    x[2, :cols // 2] = -1
+    x[3] = 127
+    x[4] = -128
+    x[5, ::2], x[5, 1::2] = 127, -128   # maximum variance
+    got = host(ops.layernorm(dev(x), dev(gamma), dev(beta), 5, 'conv_even'))
+    assert np.array_equal(got, oracle.layernorm(x, gamma, beta, 5, 'conv_even'))
+
+
+@pytest.mark.parametrize('cols', [64, 768, 1024, 100])
+def test_add_layernorm_fused(ops, oracle, cols):
+    r = rng(cols + 7)
+    a = gauss8(r, 60, (41, cols))
+    b = gauss8(r, 60, (41, cols))
+    gamma, beta = ln_params(r, cols)
+    s, out = ops.add_layernorm(dev(a), dev(b), dev(gamma), dev(beta), 5, 'conv_even', return_sum=True)
+    es, eo = oracle.add_layernorm(a, b, gamma, beta, 5, 'conv_even', return_sum=True)
+    assert np.array_equal(host(s), es)
+    assert np.array_equal(host(out), eo)
+    out2 = ops.add_layernorm(dev(a), dev(b), dev(gamma), dev(beta), 5, 'conv_even')
+    assert np.array_equal(host(out2), eo)
+
+
+# ---- Softmax --------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize('cols', [16, 32, 64, 128, 512, 1024, 2048, 4096, 48, 96, 100, 8192])
+def test_softmax_exp_columns(ops, oracle, cols):
+    r = rng(cols + 100)
+    x = gauss8(r, 24, (53, cols))
+    for kq in (23, 1, 128):
+        got = host(ops.softmax_exp(dev(x), kq))
+        assert np.array_equal(got, oracle.softmax_exp(x, kq)), (cols, kq)
+    got16 = host(ops.softmax_exp(dev(x), 23, out_kind='int16'))
+    assert np.array_equal(got16, oracle.softmax_exp(x, 23, out='int16'))
+
+
+def test_softmax_exp_every_gap_and_kq(ops, oracle):
+    # a row containing every gap 0..255, for every legal KQ: the whole exp table is exercised
+    base = np.arange(-128, 128, dtype=np.int8)
+    x = np.stack([np.roll(base, i) for i in range(8)])
+    for kq in range(1, 129):
+        got = host(ops.softmax_exp(dev(x), kq))
+        assert np.array_equal(got, oracle.softmax_exp(x, kq)), kq
+
+
+def test_softmax_exp_special_rows(ops, oracle):
+    x = np.zeros((4, 512), np.int8)
+    x[1] = -128
+    x[2, 7] = 127
+    x[2, :7] = -128
+    x[3] = 127
+    got = host(ops.softmax_exp(dev(x), 23))
+    assert np.array_equal(got, oracle.softmax_exp(x, 23))
+    assert not got[0].any()  # uniform row of 512: floor(510/512) = 0 -> all zero
+
+
+@pytest.mark.parametrize('cols,params', [(512, (60, 1, 59)), (512, (63, 2, 31)), (128, (255, 2, 127)),
+                                         (64, (400, 3, 100)), (96, (33, 1, 30)), (100, (300, 2, 127))])
+def test_softmax_hccs(ops, oracle, cols, params):
+    B, S, Dmax = params
+    r = rng(cols + B)
+    x = gauss8(r, 24, (77, cols))
+    for out in ('uint8', 'int16'):
+        for clb in (False, True):
+            got = host(ops.softmax_hccs(dev(x), B, S, Dmax, use_clb=clb, out_kind=out))
+            assert np.array_equal(got, oracle.softmax_hccs(x, B, S, Dmax, use_clb=clb, out=out)), (out, clb)
+    for inv_shift in (8, 12, 20):
+        got = host(ops.softmax_hccs(dev(x), B, S, Dmax, inv_shift=inv_shift))
+        assert np.array_equal(got, oracle.softmax_hccs(x, B, S, Dmax, inv_shift=inv_shift)), inv_shift
+
+
+def test_softmax_validation_errors(ops):
+    x = torch.zeros((4, 512), dtype=torch.int8, device='cuda')
+    with pytest.raises(ValueError, match='cols \\* B <= 32767'):
+        ops.softmax_hccs(x, 100, 1, 59)
+    with pytest.raises(ValueError, match='B - S\\*Dmax >= 0'):
+        ops.softmax_hccs(x, 10, 1, 59)
+    with pytest.raises(ValueError, match='EXP_KQ'):
+        ops.softmax_exp(x, 200)
+    with pytest.raises(ValueError, match='uint8 or int16'):
+        ops.softmax_exp(x, 23, out_kind='int8')
+
+
+# ---- fused MLP ------------------------------------------------------------------------------------------
+
+def make_mlp(ops, r, widths, relu_kind='int8'):
+    layers_np, specs = [], []
+    for i, (k, n) in enumerate(zip(widths[:-1], widths[1:])):
+        W = r.integers(-64, 64, (k, n)).astype(np.int8)
+        b = r.integers(-4096, 4097, n).astype(np.int32)
+        last = i == len(widths) - 2
+        relu = not last
+        out = relu_kind if relu else 'int8'
+        layers_np.append((W, b, 7, relu, out))
+        specs.append(ops.MlpLayerSpec(ops.pack_dense(dev(W), dev(b), 7), 7, relu, out))
+    return layers_np, specs
+
+
+@pytest.mark.parametrize('mode', ['positive_inf', 'symmetric_inf', 'conv_even', 'floor'])
+@pytest.mark.parametrize('batch', [1, 63, 1024, 5000])
+def test_mlp_fused_matches_layerwise_oracle(ops, oracle, mode, batch):
+    r = rng(17)
+    x = r.integers(-128, 128, (batch, 16)).astype(np.int8)
+    layers_np, specs = make_mlp(ops, r, [16, 64, 32, 32, 5])
+    got = host(ops.mlp(dev(x), specs, mode))
+    assert np.array_equal(got, oracle.mlp(x, layers_np, mode))
+
+
+def test_mlp_unsigned_hidden_activations_and_odd_widths(ops, oracle):
+    r = rng(18)
+    x = r.integers(-128, 128, (300, 23)).astype(np.int8)
+    layers_np, specs = make_mlp(ops, r, [23, 50, 7, 256, 3], relu_kind='uint8')
+    got = host(ops.mlp(dev(x), specs, 'conv_even'))
+    assert np.array_equal(got, oracle.mlp(x, layers_np, 'conv_even'))
+
+
+def test_mlp_limits(ops):
+    r = rng(19)
+    _, specs = make_mlp(ops, r, [16, 300, 4])
+    with pytest.raises(NotImplementedError):
+        ops.mlp(torch.zeros((4, 16), dtype=torch.int8, device='cuda'), specs, 'floor')
