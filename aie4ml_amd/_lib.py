@@ -76,6 +76,10 @@ def load() -> ctypes.CDLL:
     global _lib
     if _lib is not None:
         return _lib
+    # PyTorch's bundled HIP runtime must be the one this process initialises: load it first so that the
+    # library below binds to the same libamdhip64 that owns torch's device memory and streams.
+    import torch  # noqa: F401
+
     if not LIB_PATH.exists():
         raise RuntimeError(
             f'{LIB_PATH} is missing: build it with `python -m aie4ml_amd.build` (hipcc, gfx950). '

@@ -103,6 +103,19 @@ __device__ __forceinline__ int apply_round(int acc, const RoundCfg& rc) {
 
 __device__ __forceinline__ int clamp_i(int v, int lo, int hi) { return min(max(v, lo), hi); }
 
+// Low bytes of four ints -> one dword, through v_perm_b32. Shift-and-or packing of clamped shifts is
+// avoided on purpose: the compiler folds that shape into gfx950's v_ashr_pk_u8_i32 / _i8_i32 and then
+// treats the upper half of its result as zero, which the hardware does not guarantee.
+__device__ __forceinline__ unsigned pack4_bytes(int y0, int y1, int y2, int y3) {
+    const unsigned lo = __builtin_amdgcn_perm(static_cast<unsigned>(y1), static_cast<unsigned>(y0), 0x0c0c0400u);
+    const unsigned hi = __builtin_amdgcn_perm(static_cast<unsigned>(y3), static_cast<unsigned>(y2), 0x04000c0cu);
+    return lo | hi;
+}
+// Low halves of two ints -> one dword.
+__device__ __forceinline__ unsigned pack2_halves(int y0, int y1) {
+    return __builtin_amdgcn_perm(static_cast<unsigned>(y1), static_cast<unsigned>(y0), 0x05040100u);
+}
+
 __device__ __forceinline__ int kind_lo(int kind) {
     return kind == A4G_I8 ? -128 : (kind == A4G_I16 ? -32768 : (kind == A4G_I32 ? INT32_MIN : 0));
 }

@@ -214,10 +214,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_i8_nt_kernel(GemmA
                     // outside the matrix: nothing to store
                 } else if (n + 3 < g.N && vec_ok) {
                     if (obytes == 1) {
-                        *reinterpret_cast<unsigned*>(dst) = (y[0] & 0xFF) | ((y[1] & 0xFF) << 8) | ((y[2] & 0xFF) << 16) |
-                                                            (static_cast<unsigned>(y[3]) << 24);
+                        *reinterpret_cast<unsigned*>(dst) = pack4_bytes(y[0], y[1], y[2], y[3]);
                     } else {
-                        v2i o = {(y[0] & 0xFFFF) | (y[1] << 16), (y[2] & 0xFFFF) | (y[3] << 16)};
+                        v2i o = {static_cast<int>(pack2_halves(y[0], y[1])), static_cast<int>(pack2_halves(y[2], y[3]))};
                         *reinterpret_cast<v2i*>(dst) = o;
                     }
                 } else {

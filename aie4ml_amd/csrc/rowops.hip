@@ -213,7 +213,7 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const int8_t* __res
             v4i o;
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
-                unsigned packed = 0;
+                int y4[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const int e = w * 4 + j;  // element within the chunk
@@ -224,10 +224,9 @@ __global__ __launch_bounds__(256) void layernorm_wave_kernel(const int8_t* __res
                     const int vd = sext8(xv[i][w], j) - st.mu;
                     const int fs = clamp_i(round_shift<MODE>(st.inv * gam, gamma_shift), -32768, 32767);
                     const int acc = vd * fs + bet;
-                    const int y = clamp_i(round_shift<MODE>(acc, final_shift), -128, 127);
-                    packed |= static_cast<unsigned>(y & 0xFF) << (8 * j);
+                    y4[j] = clamp_i(round_shift<MODE>(acc, final_shift), -128, 127);
                 }
-                o[w] = static_cast<int>(packed);
+                o[w] = static_cast<int>(pack4_bytes(y4[0], y4[1], y4[2], y4[3]));
             }
             __builtin_nontemporal_store(o, reinterpret_cast<v4i*>(out + base + col0));
         }
@@ -486,7 +485,7 @@ __global__ __launch_bounds__(256) void softmax_lut_kernel(const int8_t* __restri
                 for (int k = 0; k < 8; ++k) {
                     const int y0 = sat16((e[i][2 * k] * inv) >> p.out_shift);
                     const int y1 = sat16((e[i][2 * k + 1] * inv) >> p.out_shift);
-                    o[k >> 2][k & 3] = (y0 & 0xFFFF) | (y1 << 16);
+                    o[k >> 2][k & 3] = static_cast<int>(pack2_halves(y0, y1));
                 }
                 v4i* dst = reinterpret_cast<v4i*>(static_cast<int16_t*>(out) + base + col0);
                 __builtin_nontemporal_store(o[0], dst);
@@ -495,14 +494,13 @@ __global__ __launch_bounds__(256) void softmax_lut_kernel(const int8_t* __restri
                 v4i o;
 #pragma unroll
                 for (int w = 0; w < 4; ++w) {
-                    unsigned packed = 0;
+                    int y4[4];
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        int y = (e[i][w * 4 + j] * inv) >> p.out_shift;
-                        if (!NOCLAMP_U8) y = clamp_i(y, 0, 255);
-                        packed |= static_cast<unsigned>(y) << (8 * j);
+                        y4[j] = (e[i][w * 4 + j] * inv) >> p.out_shift;
+                        if (!NOCLAMP_U8) y4[j] = clamp_i(y4[j], 0, 255);
                     }
-                    o[w] = static_cast<int>(packed);
+                    o[w] = static_cast<int>(pack4_bytes(y4[0], y4[1], y4[2], y4[3]));
                 }
                 __builtin_nontemporal_store(o, reinterpret_cast<v4i*>(static_cast<uint8_t*>(out) + base + col0));
             }
