@@ -9,6 +9,7 @@
 // back 128 * colsum[n] (exact in wrapping int32).
 #include <algorithm>
 #include <cstdlib>
+#include <type_traits>
 
 #include "common.hpp"
 
@@ -234,6 +235,527 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_i8_nt_kernel(GemmA
 }
 
 // -----------------------------------------------------------------------------------------------------
+// Pipelined MFMA kernel (K % BK == 0). Tiles go global -> LDS directly (global_load_lds, 16 bytes per
+// lane, no register staging) into a ring of STAGES buffers; fragments are read with ds_read_b128 one
+// K step (32) ahead of the MFMAs that consume them, one read issued behind each MFMA, so LDS latency
+// and the per-wave LDS issue rate hide behind the matrix pipe. One workgroup barrier per K tile,
+// placed before the tile's last K step.
+//
+// LDS layout of one operand tile: rows of BK bytes = CPR 16-byte chunks, unpadded (a wave-wide direct
+// load writes 64 consecutive chunks). Chunk c of row r lives at slot r*CPR + (c ^ swz(r)) with
+// swz(r) = (r>>2)&3 for BK = 64 and (r>>1)&7 for BK = 128: the 16 lanes that read one chunk column of
+// 16 consecutive rows then touch 16 distinct 16-byte bank groups. The swizzle is applied on the
+// global side: lane l of wave-load j fetches the chunk that belongs in slot j*64 + l. With BK = 128
+// every row segment is one whole 128-byte cache line.
+// -----------------------------------------------------------------------------------------------------
+typedef __attribute__((address_space(1))) const void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
+
+struct TileCoord {
+    int m0, n0, batch;
+    bool valid;
+};
+
+// Workgroup -> tile mapping. Hardware deals consecutive workgroup ids round-robin over the 8 XCDs,
+// each with a private L2, so id % 8 names the XCD: every XCD gets one contiguous range of tiles, and
+// that range is ordered in bands of GROUP_M tile rows (row index fastest inside a band) so that the
+// tiles resident on an XCD at one time share both activation and weight panels.
+template <int BM, int BN>
+__device__ __forceinline__ TileCoord tile_coord(const GemmArgs& g) {
+    TileCoord tc;
+    const int tiles_m = (g.M + BM - 1) / BM;
+    const int tiles_n = (g.N + BN - 1) / BN;
+    const int tiles = tiles_m * tiles_n;
+    const int per_xcd = (tiles + 7) / 8;
+    const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    tc.valid = tile < tiles;
+    constexpr int GROUP_M = 8;
+    const int band = tile / (GROUP_M * tiles_n);
+    const int band_rows = min(GROUP_M, tiles_m - band * GROUP_M);
+    const int in_band = tile % (GROUP_M * tiles_n);
+    tc.m0 = (band * GROUP_M + in_band % max(band_rows, 1)) * BM;
+    tc.n0 = (in_band / max(band_rows, 1)) * BN;
+    tc.batch = blockIdx.y;
+    return tc;
+}
+
+// Per-column epilogue parameters, 5 ints per tile column in LDS: add (bias + 128*colsum), shift, and
+// the rounding constants c0, cx, bs of RoundCfg.
+template <int BN>
+struct ColParams {
+    int* add;
+    int* s;
+    int* c0;
+    int* cx;
+    int* bs;
+    __device__ __forceinline__ explicit ColParams(int8_t* base)
+        : add(reinterpret_cast<int*>(base)), s(add + BN), c0(s + BN), cx(c0 + BN), bs(cx + BN) {}
+    static constexpr int BYTES = 5 * 4 * BN;
+};
+
+// Issues the global loads of this thread's column parameters (threads tid < BN own one column each).
+template <int BN, bool A_UNSIGNED>
+__device__ __forceinline__ void fetch_col_params(const GemmArgs& g, const TileCoord& tc, int tid, int& col_add, int& col_shift) {
+    col_add = 0;
+    col_shift = 0;
+    if (tid < BN) {
+        const int nn = min(tc.n0 + tid, g.N - 1);
+        col_add = g.bias ? g.bias[nn] : 0;
+        if (A_UNSIGNED && g.colsum) col_add += 128 * g.colsum[tc.batch * g.stride_colsum + nn];
+        col_shift = column_shift(g, nn);
+    }
+}
+
+// Parks them in LDS; returns true (workgroup-uniform) when some shift exceeds 15. Contains a barrier.
+template <int BN>
+__device__ __forceinline__ bool park_col_params(const GemmArgs& g, const ColParams<BN>& cp, int tid, int col_add, int col_shift) {
+    int big_shift = 0;
+    if (tid < BN) {
+        const RoundCfg rc = make_round(g.mode, col_shift);
+        cp.add[tid] = col_add;
+        cp.s[tid] = rc.s;
+        cp.c0[tid] = rc.c0;
+        cp.cx[tid] = rc.cx;
+        cp.bs[tid] = rc.bs;
+        big_shift = rc.s > 15;
+    }
+    return __syncthreads_or(big_shift) != 0;
+}
+
+// Epilogue shared by the pipelined kernels: requantise the accumulators into an LDS image of the
+// output tile (row pitch BN*obytes + 16), then store whole rows with coalesced 16-byte writes.
+// Rounding: floor((acc + off) / 2^s), off = c0 + cx*bit (see RoundCfg). With every shift <= 15 the
+// offset is added with a saturating add: a sum that would overflow lies far above any output range
+// either way, so the clamp gives the same value. Larger shifts take the overflow-free form.
+// The caller has made sure that no tile load is in flight and that all waves are past the main loop.
+template <int BM, int BN, int WTM, int WTN, int NT>
+__device__ __forceinline__ void epilogue_store(const GemmArgs& g, const TileCoord& tc, v16i (&acc)[WTM / 32][WTN / 32],
+                                               int8_t* smem, const ColParams<BN>& cp, bool slow_round, int wm, int wn, int lane,
+                                               int tid) {
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    const int lo = g.relu ? max(kind_lo(g.out_kind), 0) : kind_lo(g.out_kind), hi = kind_hi(g.out_kind);
+    const int obytes = (g.out_kind == A4G_I16 || g.out_kind == A4G_U16) ? 2 : 1;
+    const int cpitch = BN * obytes + 16;
+    int8_t* Cb = static_cast<int8_t*>(g.C) + tc.batch * g.stride_c * obytes;
+    auto requantise = [&](auto slow_tag) {
+        constexpr bool SLOW = decltype(slow_tag)::value;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int nl = wn * WTN + j * 32 + 8 * q + 4 * (lane >> 5);  // column inside the tile
+                const v4i add4 = *reinterpret_cast<const v4i*>(cp.add + nl);
+                const v4i s4 = *reinterpret_cast<const v4i*>(cp.s + nl);
+                const v4i c04 = *reinterpret_cast<const v4i*>(cp.c0 + nl);
+                const v4i cx4 = *reinterpret_cast<const v4i*>(cp.cx + nl);
+                const v4i bs4 = *reinterpret_cast<const v4i*>(cp.bs + nl);
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+                    const int ml = wm * WTM + i * 32 + (lane & 31);
+                    int y[4];
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const int a = static_cast<int>(static_cast<unsigned>(acc[i][j][q * 4 + t]) + static_cast<unsigned>(add4[t]));
+                        if (!SLOW) {
+                            const int bit = (a >> bs4[t]) & 1;
+                            const int sum = __builtin_elementwise_add_sat(a, c04[t] + cx4[t] * bit);
+                            y[t] = clamp_i(sum >> s4[t], lo, hi);
+                        } else {
+                            RoundCfg rc;
+                            rc.s = s4[t];
+                            rc.mask = (1u << s4[t]) - 1u;
+                            rc.c0 = c04[t];
+                            rc.cx = cx4[t];
+                            rc.bs = bs4[t];
+                            y[t] = clamp_i(apply_round(a, rc), lo, hi);
+                        }
+                    }
+                    if (obytes == 1) {
+                        *reinterpret_cast<unsigned*>(smem + ml * cpitch + nl) = pack4_bytes(y[0], y[1], y[2], y[3]);
+                    } else {
+                        v2i o = {static_cast<int>(pack2_halves(y[0], y[1])), static_cast<int>(pack2_halves(y[2], y[3]))};
+                        *reinterpret_cast<v2i*>(smem + ml * cpitch + nl * 2) = o;
+                    }
+                }
+            }
+        }
+    };
+    if (slow_round) requantise(std::true_type{});
+    else requantise(std::false_type{});
+    __syncthreads();
+    const int cpr = BN * obytes / 16;  // 16-byte chunks per tile row
+    const bool vec_ok = ((g.ldc * obytes) % 16 == 0) && ((reinterpret_cast<uintptr_t>(Cb) & 15) == 0);
+    for (int idx = tid; idx < BM * cpr; idx += NT) {
+        const int row = idx / cpr, ch = idx % cpr;
+        const int m = tc.m0 + row;
+        const int nb = tc.n0 * obytes + ch * 16;  // byte column in the output row
+        if (m >= g.M || nb >= g.N * obytes) continue;
+        const v4i v = *reinterpret_cast<const v4i*>(smem + row * cpitch + ch * 16);
+        int8_t* dst = Cb + static_cast<int64_t>(m) * g.ldc * obytes + nb;
+        if (vec_ok && nb + 16 <= g.N * obytes) {
+            *reinterpret_cast<v4i*>(dst) = v;
+        } else {
+            const int nbytes = min(16, g.N * obytes - nb);
+            const int8_t* srcb = smem + row * cpitch + ch * 16;
+            for (int b = 0; b < nbytes; ++b) dst[b] = srcb[b];
+        }
+    }
+}
+
+template <int BM, int BN, int BK_, int WAVES_M, int WAVES_N, int STAGES>
+struct DtlCfg {
+    static constexpr int BK = BK_;
+    static constexpr int CPR = BK / 16;    // chunks per row
+    static constexpr int KSTEPS = BK / 32; // MFMA K steps per tile
+    static constexpr int NW = WAVES_M * WAVES_N;
+    static constexpr int NT = NW * 64;
+    static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+    static constexpr int TM = WTM / 32, TN = WTN / 32;
+    static constexpr int A_WL = BM * CPR / 64, B_WL = BN * CPR / 64;  // wave-wide loads per tile (64 chunks each)
+    static constexpr int A_PER_W = A_WL / NW, B_PER_W = B_WL / NW;
+    static constexpr int LOADS = A_PER_W + B_PER_W;  // per thread per K tile
+    static constexpr int STAGE_BYTES = (BM + BN) * BK;
+    static constexpr int C_PITCH1 = BN + 16, C_PITCH2 = 2 * BN + 16;
+    static constexpr int EPI_BYTES = BM * C_PITCH2;
+    // per-column epilogue parameters (5 ints per column) live behind the stages / output image
+    static constexpr int PARAM_OFF = STAGES * STAGE_BYTES > EPI_BYTES ? STAGES * STAGE_BYTES : EPI_BYTES;
+    static constexpr int LDS_BYTES = PARAM_OFF + ColParams<BN>::BYTES;
+    static_assert(BK == 64 || BK == 128, "BK is 64 or 128");
+    static_assert(A_WL % NW == 0 && B_WL % NW == 0, "every wave must issue the same number of tile loads");
+    static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be whole 32x32 MFMA blocks");
+    static_assert(TM >= TN, "fragment read order assumes TM >= TN");
+    static_assert(TM * TN >= TM + TN, "one fragment read is issued behind each MFMA");
+    static_assert(STAGES >= 2 && STAGES <= 4, "2..4 stages");
+    static_assert(LOADS * (STAGES - 1) < 64, "vmcnt is a 6-bit counter");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
+    __host__ __device__ static constexpr int swz(int r) { return BK == 64 ? ((r >> 2) & 3) : ((r >> 1) & 7); }
+};
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    // s_waitcnt vmcnt(N) only (lgkmcnt / expcnt left at their maxima); gfx9 encoding:
+    // vmcnt[3:0] = simm16[3:0], vmcnt[5:4] = simm16[15:14], expcnt = [6:4], lgkmcnt = [11:8]
+    __builtin_amdgcn_s_waitcnt(((N & 0xF) | ((N >> 4) << 14)) | (0x7 << 4) | (0xF << 8));
+}
+__device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xC07F); }
+
+template <int BM, int BN, int BK_, int WAVES_M, int WAVES_N, int STAGES, bool A_UNSIGNED>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_i8_dtl_kernel(GemmArgs g) {
+    using Cfg = DtlCfg<BM, BN, BK_, WAVES_M, WAVES_N, STAGES>;
+    constexpr int BK = Cfg::BK, CPR = Cfg::CPR, KSTEPS = Cfg::KSTEPS;
+    extern __shared__ __attribute__((aligned(16))) int8_t smem[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+
+    const TileCoord tc = tile_coord<BM, BN>(g);
+    if (!tc.valid) return;
+    const int m0 = tc.m0, n0 = tc.n0, batch = tc.batch;
+
+    const int8_t* __restrict__ Ab = g.A + batch * g.stride_a;
+    const int8_t* __restrict__ Bb = g.Bt + batch * g.stride_b;
+
+    // per-column epilogue parameters: fetched first, parked in LDS once the tile loads are in flight
+    const ColParams<BN> cp(smem + Cfg::PARAM_OFF);
+    int col_add, col_shift;
+    fetch_col_params<BN, A_UNSIGNED>(g, tc, tid, col_add, col_shift);
+
+    // ---- global -> LDS assignment: wave-load j covers chunk slots [j*64, j*64+64) of the tile
+    const int8_t* pa[Cfg::A_PER_W];
+    const int8_t* pb[Cfg::B_PER_W];
+#pragma unroll
+    for (int i = 0; i < Cfg::A_PER_W; ++i) {
+        const int slot = (wave + i * Cfg::NW) * 64 + lane;
+        const int r = slot / CPR, c = (slot % CPR) ^ Cfg::swz(r);
+        pa[i] = Ab + static_cast<int64_t>(min(m0 + r, g.M - 1)) * g.lda + c * 16;
+    }
+#pragma unroll
+    for (int i = 0; i < Cfg::B_PER_W; ++i) {
+        const int slot = (wave + i * Cfg::NW) * 64 + lane;
+        const int r = slot / CPR, c = (slot % CPR) ^ Cfg::swz(r);
+        pb[i] = Bb + static_cast<int64_t>(min(n0 + r, g.N - 1)) * g.ldb + c * 16;
+    }
+    auto issue_tile = [&](int kt, int stage) {
+        int8_t* base = smem + stage * Cfg::STAGE_BYTES + wave * 1024;
+#pragma unroll
+        for (int i = 0; i < Cfg::A_PER_W; ++i)
+            __builtin_amdgcn_global_load_lds((gptr_t)(pa[i] + static_cast<int64_t>(kt) * BK),
+                                             (lptr_t)(base + i * Cfg::NW * 1024), 16, 0, 0);
+#pragma unroll
+        for (int i = 0; i < Cfg::B_PER_W; ++i)
+            __builtin_amdgcn_global_load_lds((gptr_t)(pb[i] + static_cast<int64_t>(kt) * BK),
+                                             (lptr_t)(base + BM * BK + i * Cfg::NW * 1024), 16, 0, 0);
+    };
+
+    const int ktiles = g.K / BK;
+    // prologue: fill every stage. Tiles past the end are still issued (the last tile again, into a
+    // stage nobody reads any more) so that the outstanding-load count stays a compile-time constant.
+#pragma unroll
+    for (int st = 0; st < STAGES; ++st) issue_tile(min(st, ktiles - 1), st);
+
+    const bool slow_round = park_col_params<BN>(g, cp, tid, col_add, col_shift);
+
+    // ---- fragment addressing: row = lane%32 of the block, 16-byte half of the 32-wide K step = lane/32
+    const int frow = lane & 31;
+    int koff[KSTEPS];
+#pragma unroll
+    for (int kk = 0; kk < KSTEPS; ++kk) koff[kk] = ((kk * 2 + (lane >> 5)) ^ Cfg::swz(frow)) * 16;
+    const int a_off = (wm * Cfg::WTM + frow) * BK;
+    const int b_off = BM * BK + (wn * Cfg::WTN + frow) * BK;
+
+    v16i acc[Cfg::TM][Cfg::TN];
+#pragma unroll
+    for (int i = 0; i < Cfg::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < Cfg::TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+    v4i af[2][Cfg::TM], bf[2][Cfg::TN];
+    constexpr int NR = Cfg::TM + Cfg::TN, NM = Cfg::TM * Cfg::TN;
+    auto read_one = [&](int set, const int8_t* base, int kk, int idx) {
+        // order B0, A0, B1, A1, ... so that the first MFMA of the next step can start early
+        if (idx < 2 * Cfg::TN) {
+            if (idx & 1) af[set][idx >> 1] = *reinterpret_cast<const v4i*>(base + a_off + (idx >> 1) * 32 * BK + koff[kk]);
+            else bf[set][idx >> 1] = *reinterpret_cast<const v4i*>(base + b_off + (idx >> 1) * 32 * BK + koff[kk]);
+        } else {
+            const int i = idx - Cfg::TN;
+            af[set][i] = *reinterpret_cast<const v4i*>(base + a_off + i * 32 * BK + koff[kk]);
+        }
+    };
+    // MFMAs of the fragment set `cur`, with the reads of set `nxt` threaded between them
+    auto step = [&](int cur, int nxt, const int8_t* next_base, int next_kk) {
+#pragma unroll
+        for (int m = 0; m < NM; ++m) {
+            const int i = m / Cfg::TN, j = m % Cfg::TN;
+            if (A_UNSIGNED && j == 0) af[cur][i] ^= static_cast<int>(0x80808080u);
+            // operands swapped: the block's first index (registers) runs over n, lanes over m
+            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[cur][j], af[cur][i], acc[i][j], 0, 0, 0);
+            if (m < NR) read_one(nxt, next_base, next_kk, m);
+        }
+#pragma unroll
+        for (int m = 0; m < NM; ++m) {
+            if (A_UNSIGNED && m % Cfg::TN == 0) __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // operand fix-up
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                      // one MFMA
+            if (m < NR) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                          // one LDS read
+        }
+    };
+
+    wait_vmcnt<Cfg::LOADS*(STAGES - 1)>();
+    __syncthreads();  // tile 0 visible to every wave
+#pragma unroll
+    for (int r = 0; r < NR; ++r) read_one(0, smem, 0, r);
+
+    for (int kt = 0; kt < ktiles; ++kt) {
+        const int8_t* cur_base = smem + (kt % STAGES) * Cfg::STAGE_BYTES;
+        const int8_t* nxt_base = smem + ((kt + 1) % STAGES) * Cfg::STAGE_BYTES;
+#pragma unroll
+        for (int kk = 0; kk < KSTEPS - 1; ++kk) {
+            step(kk & 1, (kk + 1) & 1, cur_base, kk + 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // every read of tile kt has been issued; once they have returned its stage can be refilled
+        wait_vmcnt<Cfg::LOADS*(STAGES - 2)>();  // this wave's share of tile kt+1 has landed
+        wait_lgkmcnt0();
+        __builtin_amdgcn_s_barrier();            // ... and everyone's; nobody reads stage kt%S any more
+        __builtin_amdgcn_sched_barrier(0);
+        issue_tile(min(kt + STAGES, ktiles - 1), kt % STAGES);
+        step((KSTEPS - 1) & 1, KSTEPS & 1, nxt_base, 0);  // after the last tile this reads a stale stage: unused
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // drain the direct loads still in flight before the stages are reused as the output tile
+    wait_vmcnt<0>();
+    __syncthreads();
+
+    epilogue_store<BM, BN, Cfg::WTM, Cfg::WTN, Cfg::NT>(g, tc, acc, smem, cp, slow_round, wm, wn, lane, tid);
+}
+
+// -----------------------------------------------------------------------------------------------------
+// Register-staged pipelined MFMA kernel (K % 128 == 0) — the kernel for large GEMMs.
+//
+// Measured on this part, 16-byte global loads into registers that cover whole 128-byte lines sustain
+// about 1.75x the L2 throughput of the direct-to-LDS path, so tiles take the classic route: global ->
+// VGPR (one K tile ahead) -> ds_write_b128 -> LDS (two stages) -> ds_read_b128 -> MFMA. BK = 128 makes
+// every row segment one cache line. LDS layout and swizzle as in the direct-load kernel (BK = 128).
+//
+// Per K tile kt and wave, four K steps of TM*TN MFMAs each; the memory work is threaded between them:
+//   step 0: MFMAs(kt,0) | reads(kt,1) | ds_write of the registers holding tile kt+1 -> stage (kt+1)%2
+//   step 1: MFMAs(kt,1) | reads(kt,2) | global loads of tile kt+2 -> the same registers
+//   step 2: MFMAs(kt,2) | reads(kt,3)
+//   lgkmcnt(0); barrier        (tile kt+1 complete in LDS; nobody reads stage kt%2 after this point)
+//   step 3: MFMAs(kt,3) | reads(kt+1,0)
+// -----------------------------------------------------------------------------------------------------
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+struct RsCfg {
+    static constexpr int BK = 128, CPR = 8, KSTEPS = 4;
+    static constexpr int NW = WAVES_M * WAVES_N;
+    static constexpr int NT = NW * 64;
+    static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+    static constexpr int TM = WTM / 32, TN = WTN / 32;
+    static constexpr int ROWS_PER_PASS = NT / CPR;  // tile rows covered by one load per thread
+    static constexpr int A_LOADS = BM / ROWS_PER_PASS, B_LOADS = BN / ROWS_PER_PASS;
+    static constexpr int LOADS = A_LOADS + B_LOADS;
+    static constexpr int STAGE_BYTES = (BM + BN) * BK;
+    static constexpr int EPI_BYTES = BM * (2 * BN + 16);
+    static constexpr int PARAM_OFF = 2 * STAGE_BYTES > EPI_BYTES ? 2 * STAGE_BYTES : EPI_BYTES;
+    static constexpr int LDS_BYTES = PARAM_OFF + ColParams<BN>::BYTES;
+    static_assert(BM % ROWS_PER_PASS == 0 && BN % ROWS_PER_PASS == 0, "tile rows must divide over the threads");
+    static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be whole 32x32 MFMA blocks");
+    static_assert(TM >= TN && TM * TN >= TM + TN, "one fragment read is issued behind each MFMA");
+    static constexpr int EPM = (LOADS + TM * TN - 1) / (TM * TN);  // staging writes / global loads behind each MFMA
+    static_assert(ROWS_PER_PASS % 16 == 0, "the swizzle term must not depend on the pass");
+    static_assert((BM + BN) * BK <= 65536, "ds_write immediate offsets are 16 bits");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
+};
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool A_UNSIGNED, bool EARLY = false>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_i8_rs_kernel(GemmArgs g) {
+    using Cfg = RsCfg<BM, BN, WAVES_M, WAVES_N>;
+    constexpr int BK = Cfg::BK, KSTEPS = Cfg::KSTEPS;
+    extern __shared__ __attribute__((aligned(16))) int8_t smem[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+
+    const TileCoord tc = tile_coord<BM, BN>(g);
+    if (!tc.valid) return;
+    const int m0 = tc.m0, n0 = tc.n0;
+
+    const ColParams<BN> cp(smem + Cfg::PARAM_OFF);
+    int col_add, col_shift;
+    fetch_col_params<BN, A_UNSIGNED>(g, tc, tid, col_add, col_shift);
+
+    // ---- global -> register staging: thread t owns chunk t%8 of rows t/8 + pass*ROWS_PER_PASS
+    const int lrow = tid / Cfg::CPR, lchunk = tid % Cfg::CPR;
+    const int8_t* __restrict__ Abase = g.A + tc.batch * g.stride_a + static_cast<int64_t>(m0) * g.lda;
+    const int8_t* __restrict__ Bbase = g.Bt + tc.batch * g.stride_b + static_cast<int64_t>(n0) * g.ldb;
+    int offa[Cfg::A_LOADS], offb[Cfg::B_LOADS];  // 32-bit offsets from the tile's first row
+#pragma unroll
+    for (int i = 0; i < Cfg::A_LOADS; ++i)
+        offa[i] = min(lrow + i * Cfg::ROWS_PER_PASS, g.M - 1 - m0) * static_cast<int>(g.lda) + lchunk * 16;
+#pragma unroll
+    for (int i = 0; i < Cfg::B_LOADS; ++i)
+        offb[i] = min(lrow + i * Cfg::ROWS_PER_PASS, g.N - 1 - n0) * static_cast<int>(g.ldb) + lchunk * 16;
+    // LDS slot of that chunk; the swizzle term (row>>1)&7 is the same for every pass
+    const int st_off = lrow * BK + ((lchunk ^ ((lrow >> 1) & 7)) * 16);
+
+    v4i ra[Cfg::A_LOADS], rb[Cfg::B_LOADS];
+    auto load_one = [&](int kt, int idx) {
+        if (idx < Cfg::A_LOADS) ra[idx] = *reinterpret_cast<const v4i*>(Abase + offa[idx] + static_cast<int64_t>(kt) * BK);
+        else rb[idx - Cfg::A_LOADS] = *reinterpret_cast<const v4i*>(Bbase + offb[idx - Cfg::A_LOADS] + static_cast<int64_t>(kt) * BK);
+    };
+    auto store_one = [&](int8_t* stage, int idx) {
+        if (idx < Cfg::A_LOADS) *reinterpret_cast<v4i*>(stage + st_off + idx * Cfg::ROWS_PER_PASS * BK) = ra[idx];
+        else *reinterpret_cast<v4i*>(stage + BM * BK + st_off + (idx - Cfg::A_LOADS) * Cfg::ROWS_PER_PASS * BK) = rb[idx - Cfg::A_LOADS];
+    };
+
+    const int ktiles = g.K / BK;
+#pragma unroll
+    for (int i = 0; i < Cfg::LOADS; ++i) load_one(0, i);
+
+    const bool slow_round = park_col_params<BN>(g, cp, tid, col_add, col_shift);
+
+    // ---- fragment addressing: row = lane%32 of the block, 16-byte half of the 32-wide K step = lane/32
+    const int frow = lane & 31;
+    int koff[KSTEPS];
+#pragma unroll
+    for (int kk = 0; kk < KSTEPS; ++kk) koff[kk] = ((kk * 2 + (lane >> 5)) ^ ((frow >> 1) & 7)) * 16;
+    const int a_off = (wm * Cfg::WTM + frow) * BK;
+    const int b_off = BM * BK + (wn * Cfg::WTN + frow) * BK;
+
+    v16i acc[Cfg::TM][Cfg::TN];
+#pragma unroll
+    for (int i = 0; i < Cfg::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < Cfg::TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+
+    v4i af[2][Cfg::TM], bf[2][Cfg::TN];
+    constexpr int NR = Cfg::TM + Cfg::TN, NM = Cfg::TM * Cfg::TN;
+    auto read_one = [&](int set, const int8_t* base, int kk, int idx) {
+        if (idx < 2 * Cfg::TN) {
+            if (idx & 1) af[set][idx >> 1] = *reinterpret_cast<const v4i*>(base + a_off + (idx >> 1) * 32 * BK + koff[kk]);
+            else bf[set][idx >> 1] = *reinterpret_cast<const v4i*>(base + b_off + (idx >> 1) * 32 * BK + koff[kk]);
+        } else {
+            const int i = idx - Cfg::TN;
+            af[set][i] = *reinterpret_cast<const v4i*>(base + a_off + i * 32 * BK + koff[kk]);
+        }
+    };
+    // EXTRA: 0 = nothing, 1 = staging writes into `stage_w`, 2 = global loads of tile `kt_load`
+    auto step = [&](int cur, int nxt, const int8_t* next_base, int next_kk, auto extra_tag, int8_t* stage_w, int kt_load) {
+        constexpr int EXTRA = decltype(extra_tag)::value;
+#pragma unroll
+        for (int m = 0; m < NM; ++m) {
+            const int i = m / Cfg::TN, j = m % Cfg::TN;
+            if (A_UNSIGNED && j == 0) af[cur][i] ^= static_cast<int>(0x80808080u);
+            // operands swapped: the block's first index (registers) runs over n, lanes over m
+            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[cur][j], af[cur][i], acc[i][j], 0, 0, 0);
+            if (m < NR) read_one(nxt, next_base, next_kk, m);
+#pragma unroll
+            for (int e = m * Cfg::EPM; e < (m + 1) * Cfg::EPM && e < Cfg::LOADS; ++e) {
+                if (EXTRA == 1 || EXTRA == 3) store_one(stage_w, e);
+                if (EXTRA == 2 || EXTRA == 3) load_one(kt_load, e);
+            }
+        }
+#pragma unroll
+        for (int m = 0; m < NM; ++m) {
+            if (A_UNSIGNED && m % Cfg::TN == 0) __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // operand fix-up
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                      // one MFMA
+            if (m < NR) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                          // one LDS read
+#pragma unroll
+            for (int e = m * Cfg::EPM; e < (m + 1) * Cfg::EPM && e < Cfg::LOADS; ++e) {
+                if (EXTRA == 1 || EXTRA == 3) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // one LDS write
+                if (EXTRA == 2 || EXTRA == 3) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global load
+            }
+        }
+    };
+    using Tag0 = std::integral_constant<int, 0>;
+    using Tag1 = std::integral_constant<int, 1>;
+    using Tag2 = std::integral_constant<int, 2>;
+    using Tag3 = std::integral_constant<int, 3>;
+
+    // prologue: tile 0 -> stage 0, tile 1 -> registers, first fragments
+#pragma unroll
+    for (int i = 0; i < Cfg::LOADS; ++i) store_one(smem, i);
+#pragma unroll
+    for (int i = 0; i < Cfg::LOADS; ++i) load_one(min(1, ktiles - 1), i);
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < NR; ++r) read_one(0, smem, 0, r);
+
+    for (int kt = 0; kt < ktiles; ++kt) {
+        int8_t* cur_base = smem + (kt & 1) * Cfg::STAGE_BYTES;
+        int8_t* nxt_base = smem + ((kt + 1) & 1) * Cfg::STAGE_BYTES;
+        if (EARLY) {
+            step(0, 1, cur_base, 1, Tag3{}, nxt_base, min(kt + 2, ktiles - 1));
+            __builtin_amdgcn_sched_barrier(0);
+            step(1, 0, cur_base, 2, Tag0{}, nullptr, 0);
+        } else {
+            step(0, 1, cur_base, 1, Tag1{}, nxt_base, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            step(1, 0, cur_base, 2, Tag2{}, nullptr, min(kt + 2, ktiles - 1));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        step(0, 1, cur_base, 3, Tag0{}, nullptr, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        wait_lgkmcnt0();               // own staging writes and fragment reads have completed
+        __builtin_amdgcn_s_barrier();  // tile kt+1 complete in LDS; stage kt%2 is dead from here on
+        __builtin_amdgcn_sched_barrier(0);
+        step(1, 0, nxt_base, 0, Tag0{}, nullptr, 0);  // after the last tile this reads a stale stage: unused
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    __syncthreads();  // every wave is past its last fragment read before the stages become the output image
+
+    epilogue_store<BM, BN, Cfg::WTM, Cfg::WTN, Cfg::NT>(g, tc, acc, smem, cp, slow_round, wm, wn, lane, tid);
+}
+
+// -----------------------------------------------------------------------------------------------------
 // Generic kernel: any shape / pitch / alignment; one thread per output element.
 // trans_b == 1: B is [N][ldb]; trans_b == 0: B is [K][ldb].
 // -----------------------------------------------------------------------------------------------------
@@ -321,22 +843,85 @@ static hipError_t launch_tiled(const GemmArgs& g, int batch, hipStream_t stream)
     return hipGetLastError();
 }
 
-// Picks a tile shape for the problem. variant: 0 = automatic; >0 forces a shape (used by the tuning
-// harness through the A4G_GEMM_VARIANT environment variable).
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES, bool A_UNSIGNED>
+static hipError_t launch_dtl_u(const GemmArgs& g, int batch, hipStream_t stream) {
+    using Cfg = DtlCfg<BM, BN, BK, WAVES_M, WAVES_N, STAGES>;
+    auto kern = gemm_i8_dtl_kernel<BM, BN, BK, WAVES_M, WAVES_N, STAGES, A_UNSIGNED>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           Cfg::LDS_BYTES);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    const int tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
+    const int grid_x = (tiles + 7) / 8 * 8;
+    hipLaunchKernelGGL(kern, dim3(grid_x, batch), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, g);
+    return hipGetLastError();
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool A_UNSIGNED, bool EARLY = false>
+static hipError_t launch_rs_u(const GemmArgs& g, int batch, hipStream_t stream) {
+    using Cfg = RsCfg<BM, BN, WAVES_M, WAVES_N>;
+    auto kern = gemm_i8_rs_kernel<BM, BN, WAVES_M, WAVES_N, A_UNSIGNED, EARLY>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           Cfg::LDS_BYTES);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    const int tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
+    const int grid_x = (tiles + 7) / 8 * 8;
+    hipLaunchKernelGGL(kern, dim3(grid_x, batch), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, g);
+    return hipGetLastError();
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+static hipError_t launch_rs(const GemmArgs& g, int batch, hipStream_t stream) {
+    return g.a_unsigned ? launch_rs_u<BM, BN, WAVES_M, WAVES_N, true>(g, batch, stream)
+                        : launch_rs_u<BM, BN, WAVES_M, WAVES_N, false>(g, batch, stream);
+}
+
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, int STAGES>
+static hipError_t launch_dtl(const GemmArgs& g, int batch, hipStream_t stream) {
+    return g.a_unsigned ? launch_dtl_u<BM, BN, BK, WAVES_M, WAVES_N, STAGES, true>(g, batch, stream)
+                        : launch_dtl_u<BM, BN, BK, WAVES_M, WAVES_N, STAGES, false>(g, batch, stream);
+}
+
+// Picks a kernel and tile shape for the problem. variant: 0 = automatic; > 0 forces one (tuning only,
+// through the A4G_GEMM_VARIANT environment variable; a forced kernel whose K granularity does not
+// divide K falls back to the next finer one).
 static hipError_t launch_gemm_nt(const GemmArgs& g, int batch, hipStream_t stream, int variant) {
     if (variant == 0) {
+        // 256 x 256 tiles halve the L2 traffic per MAC but cost a long fill / drain per workgroup:
+        // they pay off only for deep reductions with enough tiles to keep 256 CUs busy. Everything
+        // else (attention-sized batches, short K, narrow N) measured faster with 128 x 128.
         const int64_t tiles256 = static_cast<int64_t>((g.M + 255) / 256) * ((g.N + 255) / 256) * batch;
-        if (g.N <= 64) variant = 3;
-        else if (g.M >= 256 && g.N >= 256 && tiles256 >= 128) variant = 1;
-        else variant = 2;
+        variant = (g.M >= 256 && g.N >= 256 && g.K >= 512 && tiles256 >= 192) ? 1 : 2;
     }
+    const bool k128 = g.K % 128 == 0, k64 = g.K % 64 == 0;
     switch (variant) {
-    case 1: return launch_tiled<256, 256, 64, 2, 4>(g, batch, stream);
-    case 2: return launch_tiled<128, 128, 64, 2, 2>(g, batch, stream);
-    case 3: return launch_tiled<256, 64, 64, 4, 1>(g, batch, stream);
-    case 4: return launch_tiled<256, 256, 64, 2, 2>(g, batch, stream);
-    case 5: return launch_tiled<256, 128, 64, 2, 2>(g, batch, stream);
-    case 6: return launch_tiled<256, 256, 128, 2, 4>(g, batch, stream);
+    case 1:  // 256 x 256
+        if (k128) return g.a_unsigned ? launch_rs_u<256, 256, 2, 4, true, true>(g, batch, stream)
+                                      : launch_rs_u<256, 256, 2, 4, false, true>(g, batch, stream);
+        if (k64) return launch_dtl<256, 256, 64, 2, 4, 4>(g, batch, stream);
+        return launch_tiled<256, 256, 64, 2, 4>(g, batch, stream);
+    case 2:  // 128 x 128
+        if (k128) return launch_rs<128, 128, 2, 2>(g, batch, stream);
+        if (k64) return launch_dtl<128, 128, 64, 2, 2, 4>(g, batch, stream);
+        return launch_tiled<128, 128, 64, 2, 2>(g, batch, stream);
+    case 3:  // 256 x 64
+        if (k64) return launch_dtl<256, 64, 64, 4, 1, 4>(g, batch, stream);
+        return launch_tiled<256, 64, 64, 4, 1>(g, batch, stream);
+    // ---- tuning alternatives
+    case 4: return launch_tiled<256, 256, 64, 2, 4>(g, batch, stream);
+    case 5: return launch_tiled<128, 128, 64, 2, 2>(g, batch, stream);
+    case 6: return k64 ? launch_dtl<256, 256, 64, 2, 4, 4>(g, batch, stream) : launch_tiled<256, 256, 64, 2, 4>(g, batch, stream);
+    case 7: return k128 ? launch_rs<256, 256, 2, 4>(g, batch, stream) : launch_tiled<256, 256, 64, 2, 4>(g, batch, stream);
+    case 8: return k128 ? launch_rs<256, 64, 4, 1>(g, batch, stream) : launch_tiled<256, 64, 64, 4, 1>(g, batch, stream);
+    case 9: return k64 ? launch_dtl<128, 128, 64, 2, 2, 4>(g, batch, stream) : launch_tiled<128, 128, 64, 2, 2>(g, batch, stream);
+    case 10: return k128 ? launch_rs<256, 128, 2, 2>(g, batch, stream) : launch_tiled<256, 256, 64, 2, 4>(g, batch, stream);
     default: return hipErrorInvalidValue;
     }
 }
