@@ -1,0 +1,15 @@
+"""aie4ml_amd — an MI355X (gfx950) executor for the quantized operators aie4ml lowers.
+
+Public surface:
+  ops            torch-tensor operator API over the HIP kernels (C ABI underneath)
+  GPUModel       runtime object with the reference's compile() / predict() contract
+  GraphBuilder   programmatic construction of the operator IR
+"""
+
+from .aie_types import AIEDataType, QuantIntent, RoundingMode, SaturationMode
+from .frontends.builder import GraphBuilder, qint
+from .model import GPUModel
+
+__version__ = '0.1.0'
+__all__ = ['AIEDataType', 'QuantIntent', 'RoundingMode', 'SaturationMode', 'GraphBuilder', 'GPUModel', 'qint',
+           '__version__']

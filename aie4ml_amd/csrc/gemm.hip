@@ -898,7 +898,9 @@ static hipError_t launch_gemm_nt(const GemmArgs& g, int batch, hipStream_t strea
         // they pay off only for deep reductions with enough tiles to keep 256 CUs busy. Everything
         // else (attention-sized batches, short K, narrow N) measured faster with 128 x 128.
         const int64_t tiles256 = static_cast<int64_t>((g.M + 255) / 256) * ((g.N + 255) / 256) * batch;
-        variant = (g.M >= 256 && g.N >= 256 && g.K >= 512 && tiles256 >= 192) ? 1 : 2;
+        const int64_t rounds256 = (tiles256 + 255) / 256;  // one workgroup per CU at a time
+        const bool fills = tiles256 * 100 >= rounds256 * 256 * 85;
+        variant = (g.M >= 256 && g.N >= 256 && g.K >= 512 && fills) ? 1 : 2;
     }
     const bool k128 = g.K % 128 == 0, k64 = g.K % 64 == 0;
     switch (variant) {

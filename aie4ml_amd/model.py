@@ -1,0 +1,200 @@
+"""Runtime object of the GPU backend: the counterpart of the reference's AIEModel
+(src/aie4ml/model.py:29-153) whose predict() runs the graph on the MI355X instead of writing text
+files and shelling out to the Vitis simulator.
+
+I/O contract of predict() (src/aie4ml/simulation.py:157-196, 248-269; model.py:137-147):
+  * X is an array (single graph input) or a dict tensor-name -> array;
+  * each array has the input tensor's shape, or (1, *shape), or (iterations, *shape);
+  * quantize_in=True: floats are scaled by 2^frac, rounded with the tensor's rounding mode and
+    overflow-handled with its saturation mode; integer arrays pass through with a dtype cast;
+    quantize_in=False requires integer arrays;
+  * the result is int64 raw values, or float64 value / 2^frac with dequantize_out=True; a leading
+    iteration axis is folded into the batch axis; one output -> ndarray, several -> dict by name.
+"""
+
+from __future__ import annotations
+
+import logging
+from typing import Any, Dict, List, Optional
+
+import numpy as np
+
+from .ir import CONTEXT_ATTR, BackendContext, get_backend_context, input_tensor_for_role
+from .op_impls.precision import resolve_exact_storage_dtype
+from .passes import GPU_PIPELINE, run_aie_passes
+from .quant_utils import dequantize_output, dtype_for_precision, quantize_input
+
+log = logging.getLogger(__name__)
+
+
+class GPUModel:
+    """Owns a backend context; compile() resolves + packs, predict() executes."""
+
+    def __init__(self, ctx: BackendContext, source_model: Optional[Any] = None):
+        setattr(self, CONTEXT_ATTR, ctx)
+        self.source_model = source_model
+        self._compiled = False
+
+    @classmethod
+    def from_context(cls, ctx: BackendContext, source_model: Optional[Any] = None) -> 'GPUModel':
+        return cls(ctx, source_model=source_model)
+
+    @property
+    def context(self) -> BackendContext:
+        return get_backend_context(self)
+
+    def run_pipeline(self) -> 'GPUModel':
+        run_aie_passes(self.context, [cls() for cls in GPU_PIPELINE])
+        return self
+
+    def write(self) -> 'GPUModel':
+        """Nothing is emitted for the GPU (no firmware project); kept so call sites written for the
+        reference's write() / compile() / predict() sequence work unchanged."""
+        return self.run_pipeline()
+
+    def compile(self) -> int:
+        """Load the HIP library (raises if it was never built), resolve every node, upload parameters."""
+        from . import _lib
+
+        _lib.load()
+        self.run_pipeline()
+        self._compiled = True
+        return 0
+
+    build = compile
+
+    # ---- I/O boundary -------------------------------------------------------------------------------
+    def _io_dtype(self, tensor, namespace: str):
+        if tensor.precision is None:
+            raise RuntimeError(f'{tensor.name}: graph {namespace} has no precision; every activation must carry a '
+                               'QuantIntent.')
+        return resolve_exact_storage_dtype(tensor.precision, namespace=namespace, layer_name=tensor.name)
+
+    def prepare_inputs(self, X, quantize: bool = True) -> Dict[str, np.ndarray]:
+        graph = self.context.ir.logical
+        inputs = graph.graph_inputs()
+        iterations = int(self.context.config.get('Iterations', 1))
+        if len(inputs) == 1 and not isinstance(X, dict):
+            X = {inputs[0].name: X}
+        prepared = {}
+        for t in inputs:
+            expected = tuple(int(d) for d in t.shape)
+            if t.name not in X:
+                raise KeyError(f'{t.name}: missing graph input.')
+            arr = np.asarray(X[t.name])
+            if tuple(arr.shape) == expected:
+                arr = arr[np.newaxis, ...]
+            elif not (arr.ndim == len(expected) + 1 and tuple(arr.shape[1:]) == expected):
+                raise ValueError(f'{t.name}: expected shape {expected}, (1, *{expected}) or ({iterations}, *{expected}); '
+                                 f'got {tuple(arr.shape)}')
+            dtype = self._io_dtype(t, 'input')
+            if quantize:
+                prepared[t.name] = quantize_input(arr, dtype)
+            else:
+                if not np.issubdtype(arr.dtype, np.integer):
+                    raise ValueError(f'{t.name}: quantize=False requires integer inputs')
+                prepared[t.name] = arr.astype(dtype_for_precision(dtype.width, dtype.signed), copy=False)
+        return prepared
+
+    def predict(self, X, simulator: str = 'gpu', *, quantize_in: bool = True, dequantize_out: bool = True):
+        if simulator.lower() not in ('gpu', 'mi355x', 'gfx950'):
+            raise ValueError(f'Unknown simulator "{simulator}". Expected one of: gpu.')
+        if not self._compiled:
+            self.compile()
+        import torch
+
+        prepared = self.prepare_inputs(X, quantize=quantize_in)
+        graph = self.context.ir.logical
+        # the iteration axis and the tensors' own leading (batch) axis are one batch axis on the GPU
+        dev_inputs = {}
+        for name, arr in prepared.items():
+            merged = arr.reshape((arr.shape[0] * arr.shape[1],) + tuple(arr.shape[2:])) if arr.ndim >= 2 else arr
+            dev_inputs[name] = torch.from_numpy(np.ascontiguousarray(merged)).cuda()
+        iters = next(iter(prepared.values())).shape[0]
+        dev_out = self.execute(dev_inputs, batch_scale=iters)
+        torch.cuda.synchronize()
+        results = {}
+        for t in graph.graph_outputs():
+            raw = dev_out[t.name].cpu().numpy().astype(np.int64)
+            results[t.name] = dequantize_output(raw, self._io_dtype(t, 'output').frac) if dequantize_out else raw
+        if len(results) == 1:
+            return next(iter(results.values()))
+        return results
+
+    # ---- executor -------------------------------------------------------------------------------------
+    def execute(self, inputs: Dict[str, Any], batch_scale: int = 1) -> Dict[str, Any]:
+        """Run the resolved graph on device tensors. `inputs`: graph-input name -> integer device tensor
+        whose leading axis may be `batch_scale` times the declared one. Returns every graph output."""
+        from . import ops
+
+        ctx = self.context
+        graph, execution = ctx.ir.logical, ctx.ir.execution
+        plan = ctx.config.get('gpu_fusion_plan') or {'add_layernorm': {}, 'mlp_chains': []}
+        values: Dict[str, Any] = dict(inputs)
+        fused_ln = {v['layer_norm'] for v in plan['add_layernorm'].values()}
+        chain_head = {c[0]: c for c in plan['mlp_chains']}
+        chain_rest = {n for c in plan['mlp_chains'] for n in c[1:]}
+
+        for node in graph.nodes:
+            if node.is_placeholder:
+                self._run_view(node, values)
+                continue
+            if node.name in chain_rest or node.name in fused_ln:
+                continue  # executed as part of a fused launch
+            inst = execution.get(node.name)
+            if inst is None:
+                raise RuntimeError(f'{node.name}: node was never resolved; run compile() first.')
+            if node.name in chain_head:
+                self._run_mlp(chain_head[node.name], values, ops)
+            elif node.name in plan['add_layernorm']:
+                # launched at the add's position: everything that reads the sum comes later in the order
+                info = plan['add_layernorm'][node.name]
+                self._run_add_layernorm((node.name, info), execution.get(info['layer_norm']), values, ops)
+            else:
+                args = {t.name: values[t.name] for t in node.inputs if not t.is_parameter}
+                values.update(inst.variant.run(inst, args))
+        return {name: values[name] for name in graph.output_tensor_names}
+
+    def _run_view(self, node, values) -> None:
+        import torch
+
+        sv, cv = node.traits.get('slice_view'), node.traits.get('concat_view')
+        if sv is not None:
+            src = values[sv.data['source']]
+            for item in sv.data['slices']:
+                values[item['output']] = src.narrow(int(sv.data['axis']), int(item['start']), int(item['extent']))
+        elif cv is not None:
+            values[cv.data['output']] = torch.cat([values[i['input']] for i in cv.data['slices']], dim=int(cv.data['axis']))
+        elif node.op_type == 'input':
+            pass  # hls4ml-style input placeholder
+        else:
+            raise NotImplementedError(f'{node.name}: placeholder of type {node.op_type!r} has no view trait.')
+
+    def _run_add_layernorm(self, fused, ln_inst, values, ops) -> None:
+        add_name, info = fused
+        add_inst = self.context.ir.execution.get(add_name)
+        add_node, ln_node, cfg = add_inst.node, ln_inst.node, ln_inst.config
+        a = values[input_tensor_for_role(add_node, 'lhs').name]
+        b = values[input_tensor_for_role(add_node, 'rhs').name]
+        res = ops.add_layernorm(a, b, ln_inst.artifacts['packed_gamma'], ln_inst.artifacts['packed_beta'], cfg.out_shift,
+                                cfg.rounding_mode, eps_q0=cfg.eps_q0, gamma_shift=cfg.gamma_shift,
+                                add_shift=add_inst.config.shift, add_rounding=add_inst.config.rounding_mode,
+                                return_sum=bool(info['keep_sum']))
+        if info['keep_sum']:
+            values[add_node.outputs[0].name], values[ln_node.outputs[0].name] = res
+        else:
+            values[ln_node.outputs[0].name] = res
+
+    def _run_mlp(self, chain: List[str], values, ops) -> None:
+        execution = self.context.ir.execution
+        insts = [execution.get(n) for n in chain]
+        specs = [ops.MlpLayerSpec(i.artifacts['packed_weights'], i.config.shift, i.config.flags.use_relu,
+                                  i.config.precision['output'].format) for i in insts]
+        x = values[input_tensor_for_role(insts[0].node, 'lhs').name]
+        lead = tuple(x.shape[:-1])
+        y = ops.mlp(x.reshape(-1, x.shape[-1]), specs, insts[0].config.rounding_mode)
+        values[insts[-1].node.outputs[0].name] = y.reshape(lead + (y.shape[-1],))
+
+
+def from_context(ctx: BackendContext) -> GPUModel:
+    return GPUModel.from_context(ctx)

@@ -1,0 +1,369 @@
+"""Graph passes of the GPU backend.
+
+The fold / fuse passes decide what each kernel fuses and restate the reference's passes of the same
+names (src/aie4ml/passes/fold_bias.py, fold_scale.py, fuse_activation.py, fold_views.py); Resolve and
+PackKernelArtifacts restate passes/resolve.py:48-95 and passes/pack.py:20-37 without the AIE contract /
+staging propagation. Everything the reference runs after packing (transport, placement, memory plan)
+is AIE-physical and has no counterpart here. PlanGpuFusion is the GPU-only addition.
+"""
+
+from __future__ import annotations
+
+from typing import Iterable
+
+import numpy as np
+
+from ..ir import TraitInstance, get_backend_context
+from ..op_impls import get_family_resolver_registry
+from ..op_impls.base import OpImplVariant
+
+
+class AIEPass:
+    """Base class: transform(model_or_ctx) -> True when the IR changed."""
+
+    name: str = ''
+
+    def transform(self, model_or_ctx) -> bool:
+        raise NotImplementedError
+
+
+def run_aie_passes(ctx, passes: Iterable[AIEPass]) -> None:
+    ctx.ir.logical.verify()
+    for p in passes:
+        p.transform(ctx)
+
+
+class FoldBias(AIEPass):
+    """add(dense_output, constant) -> the dense's bias input."""
+
+    name = 'fold_bias'
+
+    def transform(self, model_or_ctx) -> bool:
+        graph = get_backend_context(model_or_ctx).ir.logical
+        changed = False
+        for add in list(graph.nodes):
+            if add.op_type != 'add' or len(add.inputs) != 2 or len(add.outputs) != 1:
+                continue
+            a, b = add.inputs
+            if self._biasless_dense(a) and b.is_parameter:
+                dense_out, bias = a, b
+            elif self._biasless_dense(b) and a.is_parameter:
+                dense_out, bias = b, a
+            else:
+                continue
+            dense = dense_out.producer
+            n_out = int(dense.metadata['n_out'])
+            size = int(np.asarray(bias.data).size)
+            if size != n_out:
+                raise ValueError(f'{add.name}: dense bias Add requires exactly {n_out} elements, got {size}.')
+            if len(dense_out.consumers) != 1:
+                raise ValueError(f'{add.name}: cannot fold bias because dense output {dense_out.name!r} '
+                                 f'has {len(dense_out.consumers)} consumers.')
+            y = add.outputs[0]
+            dense.inputs.append(bias)
+            bias.consumers = [c for c in bias.consumers if c is not add] + [dense]
+            dense.metadata['use_bias'] = True
+            dense.metadata['input_roles'] = ['lhs', 'rhs', 'bias']
+            dense.roles[bias.name] = 'bias'
+            dense.outputs = [y]
+            y.producer = dense
+            graph.tensors.pop(dense_out.name, None)
+            graph.nodes.remove(add)
+            add.inputs, add.outputs = [], []
+            changed = True
+        return changed
+
+    @staticmethod
+    def _biasless_dense(t) -> bool:
+        p = t.producer
+        return p is not None and p.op_type == 'dense' and not p.metadata.get('use_bias')
+
+
+# which op absorbs a constant scale, and on which side
+_SCALE_ABSORBERS = {'dense': 'output_scale', 'matmul': 'output_scale', 'softmax': 'input_scale'}
+
+
+class FoldScale(AIEPass):
+    """Constant `scale` nodes fold into a following softmax (temperature) or a preceding dense / matmul
+    (extra output shift). There is no standalone scale kernel."""
+
+    name = 'fold_scale'
+
+    def transform(self, model_or_ctx) -> bool:
+        graph = get_backend_context(model_or_ctx).ir.logical
+        changed = False
+        for node in list(graph.nodes):
+            if node.op_type != 'scale':
+                continue
+            if len(node.inputs) != 1 or len(node.outputs) != 1:
+                raise ValueError(f'{node.name}: scale must have exactly one input and one output.')
+            scale = float(node.metadata['scale'])
+            if scale <= 0.0:
+                raise ValueError(f'{node.name}: scale must be positive, got {scale}.')
+            src = node.inputs[0]
+            consumers = list(node.outputs[0].consumers)
+            producer = src.producer
+            consumer = consumers[0] if len(consumers) == 1 else None
+            if consumer is not None and _SCALE_ABSORBERS.get(consumer.op_type) == 'input_scale':
+                self._accumulate(consumer, 'input_scale', scale)
+                graph.remove_node(node, mode='bypass')
+            elif producer is not None and _SCALE_ABSORBERS.get(producer.op_type) == 'output_scale':
+                if len(src.consumers) != 1:
+                    raise NotImplementedError(f'{node.name}: cannot fold output scale because {src.name!r} '
+                                              f'has {len(src.consumers)} consumers.')
+                self._accumulate(producer, 'output_scale', scale)
+                graph.remove_node(node, mode='contract')
+            else:
+                raise NotImplementedError(
+                    f'{node.name}: no adjacent op absorbs this scale (producer='
+                    f'{producer.op_type if producer else None}, consumers={[c.op_type for c in consumers]}); '
+                    'there is no standalone scale kernel.')
+            changed = True
+        return changed
+
+    @staticmethod
+    def _accumulate(node, trait_name: str, scale: float) -> None:
+        prev = node.traits.get(trait_name)
+        node.add_trait(TraitInstance(trait_name, {'scale': scale * float(prev.data['scale']) if prev else scale}))
+
+
+class FuseActivationCasts(AIEPass):
+    """relu after a dense becomes the dense's fused_activation trait; linear activations disappear."""
+
+    name = 'fuse_activation_casts'
+
+    def transform(self, model_or_ctx) -> bool:
+        graph = get_backend_context(model_or_ctx).ir.logical
+        changed = False
+        for act in list(graph.nodes):
+            if act.op_type != 'activation' or len(act.inputs) != 1 or len(act.outputs) != 1:
+                continue
+            kind = (act.metadata.get('activation', '') or '').lower()
+            if kind == 'relu':
+                producer = act.inputs[0].producer
+                if producer is None or producer.op_type != 'dense' or len(producer.outputs) != 1:
+                    continue  # stays an activation node: Resolve will refuse it (no standalone kernel)
+                producer.add_trait(TraitInstance('fused_activation', {'activation': 'relu'}))
+                graph.remove_node(act, mode='contract')
+                changed = True
+            elif kind in ('linear', ''):
+                graph.remove_node(act, mode='contract')
+                changed = True
+        return changed
+
+
+class FoldViewOps(AIEPass):
+    """Transpose -> io_view permutation on its consumers; Split / Slice / Concat -> placeholder nodes
+    carrying slice_view / concat_view traits."""
+
+    name = 'fold_view_ops'
+
+    def transform(self, model_or_ctx) -> bool:
+        graph = get_backend_context(model_or_ctx).ir.logical
+        changed = False
+        for node in list(graph.nodes):
+            if node.op_type == 'transpose':
+                changed = self._transpose(graph, node) or changed
+            elif node.op_type == 'concat':
+                changed = self._concat(node) or changed
+            elif node.op_type in ('slice', 'split'):
+                changed = self._slice(node) or changed
+        return changed
+
+    @staticmethod
+    def _view(node):
+        trait = node.traits.get('io_view')
+        if trait is None:
+            trait = TraitInstance('io_view', {'inputs': {}, 'outputs': {}})
+            node.add_trait(trait)
+        trait.data.setdefault('inputs', {})
+        trait.data.setdefault('outputs', {})
+        return trait.data
+
+    def _transpose(self, graph, node) -> bool:
+        src, dst = node.inputs[0], node.outputs[0]
+        perm = node.metadata.get('perm')
+        if perm is None:
+            raise ValueError(f'{node.name}: missing transpose permutation metadata.')
+        perm = [int(p) for p in perm]
+        rank = len(src.shape)
+        if len(dst.shape) != rank:
+            raise ValueError(f'{node.name}: transpose rank mismatch between input and output.')
+        if sorted(perm) != list(range(rank)):
+            raise ValueError(f'{node.name}: invalid permutation {perm} for rank {rank}.')
+        for consumer in dst.consumers:
+            view = self._view(consumer)
+            view['inputs'][src.name] = {'perm': list(perm)}
+            view['inputs'].pop(dst.name, None)
+        graph.remove_node(node, mode='bypass')
+        return True
+
+    @staticmethod
+    def _concat(node) -> bool:
+        if len(node.outputs) != 1:
+            raise ValueError(f'{node.name}: concat must have exactly one output.')
+        if not node.inputs:
+            raise ValueError(f'{node.name}: concat must have at least one input.')
+        out = node.outputs[0]
+        rank = len(out.shape)
+        axis = int(node.metadata.get('axis', -1))
+        axis = axis + rank if axis < 0 else axis
+        if not 0 <= axis < rank:
+            raise ValueError(f'{node.name}: concat axis {node.metadata.get("axis")} is out of range for rank {rank}.')
+        offset, slices = 0, []
+        for t in node.inputs:
+            if len(t.shape) != rank:
+                raise ValueError(f'{node.name}: concat input {t.name!r} rank does not match output rank.')
+            extent = int(t.shape[axis])
+            slices.append({'input': t.name, 'start': offset, 'extent': extent})
+            offset += extent
+        if int(out.shape[axis]) != offset:
+            raise ValueError(f'{node.name}: concat output axis extent {out.shape[axis]} does not match input sum {offset}.')
+        node.add_trait(TraitInstance('concat_view', {'kind': 'concat', 'axis': axis, 'output': out.name, 'slices': slices}))
+        node.is_placeholder = True
+        return True
+
+    @staticmethod
+    def _slice(node) -> bool:
+        if len(node.inputs) != 1:
+            raise ValueError(f'{node.name}: {node.op_type} view must have exactly one input.')
+        if not node.outputs:
+            raise ValueError(f'{node.name}: {node.op_type} view must have at least one output.')
+        src = node.inputs[0]
+        rank = len(src.shape)
+        axis = int(node.metadata['axis'])
+        axis = axis + rank if axis < 0 else axis
+        if not 0 <= axis < rank:
+            raise ValueError(f'{node.name}: {node.op_type} axis {axis} is out of range for rank {rank}.')
+        items = list(node.metadata.get('slices', ()))
+        if len(items) != len(node.outputs):
+            raise ValueError(f'{node.name}: {node.op_type} slice metadata does not match output count.')
+        norm = []
+        for out, item in zip(node.outputs, items):
+            start, extent = int(item['start']), int(item['extent'])
+            if start < 0 or extent <= 0 or start + extent > int(src.shape[axis]):
+                raise ValueError(f'{node.name}: invalid {node.op_type} range [{start}, {start + extent}).')
+            if int(out.shape[axis]) != extent:
+                raise ValueError(f'{node.name}: {node.op_type} output {out.name!r} extent mismatch.')
+            norm.append({'output': out.name, 'start': start, 'extent': extent})
+        node.add_trait(TraitInstance('slice_view', {'kind': node.op_type, 'axis': axis, 'source': src.name, 'slices': norm}))
+        node.is_placeholder = True
+        return True
+
+
+class Resolve(AIEPass):
+    """Bind every non-placeholder node to an operator variant and its resolved constants."""
+
+    name = 'resolve'
+
+    def transform(self, model_or_ctx) -> bool:
+        ctx = get_backend_context(model_or_ctx)
+        ctx.ir.logical.verify()
+        registry = get_family_resolver_registry()
+        changed, visited = False, set()
+        for node in ctx.ir.logical:
+            if node.is_placeholder:
+                continue
+            resolver = registry.get(node.op_type)  # NotImplementedError for e.g. a stray activation
+            config, variant = resolver.resolve(node, ctx.device, dict(node.directives or {}))
+            variant.validate_config(node, config, ctx.device)
+            inst = ctx.ir.execution.get(node.name)
+            if inst is None or inst.variant is not variant or inst.config != config:
+                ctx.ir.execution.register(node, variant, config)
+                changed = True
+            visited.add(node.name)
+        return ctx.ir.execution.prune(visited) or changed
+
+
+class PackKernelArtifacts(AIEPass):
+    """Quantise and upload kernel-resident parameters (weights, bias, gamma, beta)."""
+
+    name = 'pack_kernel_artifacts'
+
+    def transform(self, model_or_ctx) -> bool:
+        ctx = get_backend_context(model_or_ctx)
+        changed = False
+        for inst in ctx.ir.execution:
+            if type(inst.variant).pack is OpImplVariant.pack or inst.artifacts:
+                continue
+            packed = inst.variant.pack(inst)
+            if packed:
+                inst.artifacts.update(packed)
+                changed = True
+        return changed
+
+
+class PlanGpuFusion(AIEPass):
+    """GPU-only: mark node groups the executor runs as one launch.
+
+    * add -> layer_norm: the residual add is computed inside the LayerNorm kernel (the sum is written out
+      only if something else reads it).
+    * a chain of dense nodes whose whole weight set fits LDS: one fused-MLP launch.
+    Both are exact: the fused kernels perform the same integer operations in the same order.
+    """
+
+    name = 'plan_gpu_fusion'
+    MLP_MAX_WIDTH = 256
+    MLP_MAX_WEIGHT_BYTES = 96 * 1024
+
+    def transform(self, model_or_ctx) -> bool:
+        ctx = get_backend_context(model_or_ctx)
+        graph, execution = ctx.ir.logical, ctx.ir.execution
+        plan = {'add_layernorm': {}, 'mlp_chains': []}
+        outputs = set(graph.output_tensor_names)
+        for node in graph.nodes:
+            if node.op_type != 'add' or execution.get(node.name) is None:
+                continue
+            cfg = execution.get(node.name).config
+            s = node.outputs[0]
+            lns = [c for c in s.consumers if c.op_type == 'layer_norm']
+            if len(lns) == 1 and cfg.shift == 0 and cfg.precision['output'].format == 'int8' \
+                    and not lns[0].traits.get('io_view'):
+                keep_sum = len(s.consumers) > 1 or s.name in outputs
+                plan['add_layernorm'][node.name] = {'layer_norm': lns[0].name, 'keep_sum': keep_sum}
+        # dense chains: every link a dense with a single consumer that is the next dense
+        used = set()
+        for node in graph.nodes:
+            if node.op_type != 'dense' or node.name in used or execution.get(node.name) is None:
+                continue
+            prev = node.inputs[0].producer
+            if prev is not None and prev.op_type == 'dense' and len(node.inputs[0].consumers) == 1 \
+                    and node.inputs[0].name not in outputs:
+                continue  # not a chain head
+            chain, cur = [node], node
+            while True:
+                out = cur.outputs[0]
+                nxt = out.consumers[0] if len(out.consumers) == 1 and out.name not in outputs else None
+                if nxt is None or nxt.op_type != 'dense' or nxt.inputs[0] is not out or execution.get(nxt.name) is None:
+                    break
+                chain.append(nxt)
+                cur = nxt
+            if len(chain) >= 2 and self._fits(chain, execution):
+                plan['mlp_chains'].append([n.name for n in chain])
+                used.update(n.name for n in chain)
+        changed = ctx.config.get('gpu_fusion_plan') != plan
+        ctx.config['gpu_fusion_plan'] = plan
+        return changed
+
+    def _fits(self, chain, execution) -> bool:
+        if len(chain) > 8:
+            return False
+        total, mode = 0, None
+        for i, n in enumerate(chain):
+            cfg = execution.get(n.name).config
+            if cfg.n_in > self.MLP_MAX_WIDTH or cfg.n_out > self.MLP_MAX_WIDTH or cfg.flags.transpose_lhs:
+                return False
+            if cfg.shift_per_channel is not None or n.traits.get('io_view'):
+                return False
+            last = i + 1 == len(chain)
+            fmt = cfg.precision['output'].format
+            if fmt not in ('int8', 'uint8') and not (last and fmt == 'int16'):
+                return False
+            mode = mode or cfg.rounding_mode
+            if cfg.rounding_mode != mode:
+                return False
+            total += cfg.n_out * ((cfg.n_in + 15) // 16 * 16)
+        return total <= self.MLP_MAX_WEIGHT_BYTES
+
+
+GPU_PIPELINE = (FoldBias, FoldScale, FuseActivationCasts, FoldViewOps, Resolve, PackKernelArtifacts, PlanGpuFusion)

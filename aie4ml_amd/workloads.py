@@ -58,3 +58,85 @@ def c4_add_layernorm(rows: int = 16384, cols: int = 1024):
     out_frac = 5
     beta = (r.integers(-16, 17, cols).astype(np.int32) << (15 - out_frac)).astype(np.int16)
     return a, b, gamma, beta, {'out_shift': out_frac, 'eps_q0': 1}
+
+
+def c5_encoder_block(batch: int = 64, seq: int = 128, hidden: int = 768, heads: int = 12, ffn: int = 3072,
+                     softmax: str = 'hccs', seed: int = 17 + 5):
+    """Full int8 transformer encoder block as an operator graph (the structure an ONNX Q/DQ export of
+    the block lowers to: no Reshape, heads expressed with Split / Transpose / Concat).
+
+    QKV Dense hidden->3*hidden, Split, per head: Q.K^T (Transpose folded into the MatMul), integer
+    Softmax, P.V; Concat; output Dense; Add + LayerNorm; FFN Dense+ReLU, Dense; Add + LayerNorm.
+    Weights int8 from clipped N(0,16); every tensor has a per-tensor power-of-two scale.
+    Returns (model, x_int8) with x the seeded int8 input [batch, seq, hidden].
+    """
+    from .frontends.builder import GraphBuilder, qint
+
+    r = np.random.default_rng(seed)
+    hd = hidden // heads
+    act = qint(8, 4)            # activations: int8, scale 2^-4
+    wq = qint(8, 7)             # weights: int8, scale 2^-7
+    bq = qint(32, 11)           # bias at accumulator scale 2^-(4+7)
+    prob = qint(8, 8, signed=False)  # softmax probabilities: uint8, scale 1/256
+
+    def weights(k, n):
+        return _gauss8(r, 16.0, (k, n)).astype(np.float64) / 128.0
+
+    def bias(n):
+        return r.integers(-(1 << 10), (1 << 10) + 1, n).astype(np.float64) / 2048.0
+
+    gb = GraphBuilder(config={'Iterations': 1})
+    x = gb.input('x', (batch, seq, hidden), act)
+    qkv = gb.dense(x, weights(hidden, 3 * hidden), wq, act, bias=bias(3 * hidden), bias_precision=bq, name='qkv')
+    q, k, v = gb.split(qkv, -1, [hidden] * 3, name='qkv_split')
+    qs = gb.split(q, -1, [hd] * heads, name='q_heads')
+    ks = gb.split(k, -1, [hd] * heads, name='k_heads')
+    vs = gb.split(v, -1, [hd] * heads, name='v_heads')
+    ctx_heads = []
+    directives = None
+    if softmax == 'hccs':
+        # legal for cols = seq: seq*B <= 32767 and seq*(B - S*Dmax) >= 256
+        B = min(255, 32767 // seq)
+        directives = {'approximation': 'hccs', 'hccs': {'B': B, 'S': 4, 'Dmax': (B - max(1, -(-256 // seq))) // 4}}
+    for h in range(heads):
+        kt = gb.transpose(ks[h], (0, 2, 1), name=f'k_t{h}')
+        # Q.K^T has a standard deviation of a few 10^4 at these scales: keep the top bits (shift 11)
+        logits = gb.matmul(qs[h], kt, qint(8, -3), name=f'qk{h}')
+        if softmax == 'exp':
+            # temperature 1/32, absorbed by the Softmax: EXP_KQ = round(log2(e) * 2^3 / 32 * 256) = 92
+            logits = gb.scale(logits, 1.0 / 32.0, name=f'qk_scale{h}')
+        p = gb.softmax(logits, prob, name=f'softmax{h}', directives=directives)
+        ctx_heads.append(gb.matmul(p, vs[h], act, name=f'pv{h}'))
+    attn = gb.concat(ctx_heads, -1, name='heads_concat')
+    proj = gb.dense(attn, weights(hidden, hidden), wq, act, bias=bias(hidden), bias_precision=bq, name='attn_out')
+    res1 = gb.add(x, proj, act, name='residual1')
+    gamma1 = r.integers(32, 128, hidden).astype(np.float64) / 128.0
+    beta1 = r.integers(-15, 16, hidden).astype(np.float64) / 16.0
+    ln1 = gb.layer_norm(res1, gamma1, beta1, act, eps_q0=1, name='ln1')
+    h1 = gb.dense(ln1, weights(hidden, ffn), wq, act, bias=bias(ffn), bias_precision=bq, relu=True, name='ffn1')
+    h2 = gb.dense(h1, weights(ffn, hidden), wq, act, bias=bias(hidden), bias_precision=bq, name='ffn2')
+    res2 = gb.add(ln1, h2, act, name='residual2')
+    gamma2 = r.integers(32, 128, hidden).astype(np.float64) / 128.0
+    beta2 = r.integers(-15, 16, hidden).astype(np.float64) / 16.0
+    out = gb.layer_norm(res2, gamma2, beta2, act, eps_q0=1, name='ln2')
+    gb.output(out)
+    x_int = _gauss8(r, 24.0, (batch, seq, hidden))
+    return gb.build(), x_int
+
+
+def c1_mlp_model(batch: int = 1024, rounding=None):
+    """The C1 MLP as an operator graph (hls4ml-style: Dense + ReLU layers, shift 7 everywhere)."""
+    from .aie_types import RoundingMode
+    from .frontends.builder import GraphBuilder, qint
+
+    rounding = rounding or RoundingMode.RND
+    x, layers = c1_mlp(batch)
+    # activations int8 frac 0; weights frac 7 -> acc frac 7 -> shift 7 to an int8 frac-0 output
+    act = qint(8, 0, rounding=rounding)
+    gb = GraphBuilder(config={'Iterations': 1})
+    t = gb.input('x', (batch, x.shape[1]), act)
+    for i, (W, b, _shift, relu, _kind) in enumerate(layers):
+        t = gb.dense(t, W.astype(np.float64) / 128.0, qint(8, 7), act, bias=b.astype(np.float64) / 128.0,
+                     bias_precision=qint(32, 7), relu=relu, name=f'fc{i}')
+    gb.output(t)
+    return gb.build(), x, layers

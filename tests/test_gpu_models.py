@@ -1,0 +1,142 @@
+"""GPU tests of the operator-graph executor: graphs built through the front end, lowered by the pass
+pipeline, run with GPUModel.predict on the MI355X and compared bit for bit with the CPU oracle evaluating
+the same resolved graph node by node."""
+
+import numpy as np
+import pytest
+
+from aie4ml_amd import GraphBuilder, qint, workloads
+from aie4ml_amd.aie_types import RoundingMode
+
+from ir_oracle import run_graph
+
+pytestmark = pytest.mark.gpu
+
+
+def _graph_check(model, oracle, inputs):
+    model.compile()
+    got = model.predict(inputs if len(inputs) > 1 else next(iter(inputs.values())), simulator='gpu',
+                        quantize_in=False, dequantize_out=False)
+    vals = run_graph(model, oracle, inputs)
+    outs = model.context.ir.logical.output_tensor_names
+    if len(outs) == 1:
+        got = {outs[0]: got}
+    for name in outs:
+        want = vals[name].astype(np.int64)
+        assert got[name].shape[-want.ndim:] == want.shape or got[name].size == want.size
+        np.testing.assert_array_equal(got[name].reshape(want.shape), want, err_msg=name)
+    return got
+
+
+@pytest.mark.parametrize('rounding', [RoundingMode.RND, RoundingMode.RND_CONV, RoundingMode.TRN])
+def test_c1_mlp_graph(oracle, rounding):
+    model, x, layers = workloads.c1_mlp_model(batch=256, rounding=rounding)
+    model.compile()
+    assert model.context.config['gpu_fusion_plan']['mlp_chains'] == [['fc0_aie', 'fc1_aie', 'fc2_aie', 'fc3_aie']]
+    y = model.predict(x, quantize_in=False, dequantize_out=False)
+    mode = {RoundingMode.RND: 'symmetric_inf', RoundingMode.RND_CONV: 'conv_even', RoundingMode.TRN: 'floor'}[rounding]
+    want = x
+    for W, b, shift, relu, kind in layers:
+        want = oracle.dense(want, W, b, shift, mode, relu=relu, out=kind)
+    np.testing.assert_array_equal(y, want.astype(np.int64))
+    # float inputs on the grid quantise to the same integers; dequantised output is value / 2^frac
+    yf = model.predict(x.astype(np.float64))
+    np.testing.assert_array_equal(yf, want.astype(np.float64))
+    assert yf.dtype == np.float64
+
+
+def test_mlp_graph_unfused_matches_fused(oracle):
+    model, x, layers = workloads.c1_mlp_model(batch=128)
+    model.compile()
+    fused = model.predict(x, quantize_in=False, dequantize_out=False)
+    model.context.config['gpu_fusion_plan'] = {'add_layernorm': {}, 'mlp_chains': []}
+    unfused = model.predict(x, quantize_in=False, dequantize_out=False)
+    np.testing.assert_array_equal(fused, unfused)
+
+
+def test_iteration_axis_folds_into_batch(oracle):
+    model, x, layers = workloads.c1_mlp_model(batch=64)
+    xs = np.stack([x, x[::-1], x])                      # (iterations, batch, features)
+    y = model.predict(xs, quantize_in=False, dequantize_out=False)
+    assert y.shape == (3 * 64, layers[-1][0].shape[1])
+    one = model.predict(x, quantize_in=False, dequantize_out=False)
+    np.testing.assert_array_equal(y[:64], one)
+    np.testing.assert_array_equal(y[64:128], one[::-1])
+
+
+def test_float_quantisation_at_the_boundary(oracle):
+    gb = GraphBuilder()
+    x = gb.input('x', (32, 64), qint(8, 4, rounding=RoundingMode.RND_CONV))
+    r = np.random.default_rng(3)
+    W = r.integers(-100, 100, (64, 48)) / 128.0
+    bias = r.integers(-64, 64, 48) / 8.0
+    y = gb.dense(x, W, qint(8, 7), qint(8, 2, rounding=RoundingMode.RND), bias=bias, bias_precision=qint(32, 11),
+                 name='fc')
+    gb.output(y)
+    model = gb.build()
+    xf = r.normal(0, 3, (32, 64))                        # off-grid floats, some beyond +-8 (saturate)
+    got = model.predict(xf)
+    xq = np.clip(np.round(xf * 16), -128, 127)           # numpy's round is ties-to-even = RND_CONV
+    want = oracle.dense(xq.astype(np.int8), np.round(W * 128).astype(np.int8), np.round(bias * 2048).astype(np.int32),
+                        4 + 7 - 2, 'symmetric_inf')
+    np.testing.assert_array_equal(got, want / 4.0)
+
+
+@pytest.mark.parametrize('approx', ['exp', 'hccs'])
+def test_attention_core_graph(oracle, approx):
+    r = np.random.default_rng(11)
+    gb = GraphBuilder()
+    q = gb.input('q', (3, 128, 64), qint(8, 4))
+    k = gb.input('k', (3, 128, 64), qint(8, 4))
+    v = gb.input('v', (3, 128, 64), qint(8, 4))
+    kt = gb.transpose(k, (0, 2, 1))
+    logits = gb.matmul(q, kt, qint(8, 0), name='qk')
+    d = None
+    if approx == 'exp':
+        logits = gb.scale(logits, 0.125, name='temp')
+    else:
+        d = {'approximation': 'hccs', 'hccs': {'B': 255, 'S': 3, 'Dmax': 84}}
+    p = gb.softmax(logits, qint(8, 8, signed=False), name='sm', directives=d)
+    o = gb.matmul(p, v, qint(8, 4), name='pv')
+    gb.output(o)
+    gb.output(p)
+    model = gb.build()
+    ins = {n: np.clip(r.normal(0, 20, (3, 128, 64)), -128, 127).astype(np.int8) for n in 'qkv'}
+    got = _graph_check(model, oracle, ins)
+    assert len(got) == 2                                 # several outputs come back as a dict by name
+
+
+@pytest.mark.parametrize('keep_sum', [False, True])
+def test_add_layernorm_graph(oracle, keep_sum):
+    r = np.random.default_rng(5)
+    gb = GraphBuilder()
+    a = gb.input('a', (4, 96, 768), qint(8, 4))
+    b = gb.input('b', (4, 96, 768), qint(8, 4))
+    s = gb.add(a, b, qint(8, 4), name='res')
+    y = gb.layer_norm(s, r.integers(32, 128, 768) / 128.0, r.integers(-15, 16, 768) / 16.0, qint(8, 4), eps_q0=1,
+                      name='ln')
+    gb.output(y)
+    if keep_sum:
+        gb.output(s)
+    model = gb.build()
+    model.compile()
+    assert model.context.config['gpu_fusion_plan']['add_layernorm']['res_aie']['keep_sum'] is keep_sum
+    ins = {n: np.clip(r.normal(0, 30, (4, 96, 768)), -128, 127).astype(np.int8) for n in 'ab'}
+    _graph_check(model, oracle, ins)
+
+
+@pytest.mark.parametrize('softmax', ['exp', 'hccs'])
+def test_encoder_block_small(oracle, softmax):
+    model, x = workloads.c5_encoder_block(batch=2, seq=64, hidden=128, heads=2, ffn=256, softmax=softmax)
+    got = _graph_check(model, oracle, {'x': x})
+    out = next(iter(got.values()))
+    assert len(np.unique(out)) > 32        # a live signal, not a saturated or constant tensor
+
+
+def test_encoder_block_c5_shape(oracle):
+    """BERT-base geometry (hidden 768, 12 heads of 64, FFN 3072, seq 128) on a batch the oracle finishes
+    in seconds; the full batch of 64 differs only in the number of independent sequences."""
+    model, x = workloads.c5_encoder_block(batch=2, seq=128, hidden=768, heads=12, ffn=3072, softmax='hccs')
+    got = _graph_check(model, oracle, {'x': x})
+    out = next(iter(got.values()))
+    assert out.shape[-1] == 768 and len(np.unique(out)) > 64

@@ -1,0 +1,363 @@
+"""CPU tests of the host side: fixed-point helpers, graph passes, numeric resolution, error behaviour.
+No kernels run; the pipeline is driven up to Resolve (packing uploads to the GPU)."""
+
+import numpy as np
+import pytest
+
+from aie4ml_amd import GraphBuilder, qint
+from aie4ml_amd.aie_types import AIEDataType, RoundingMode, SaturationMode
+from aie4ml_amd.ir import get_backend_context
+from aie4ml_amd.passes import (FoldBias, FoldScale, FoldViewOps, FuseActivationCasts, PlanGpuFusion, Resolve,
+                               run_aie_passes)
+from aie4ml_amd.quant_utils import (apply_rounding, dequantize_output, handle_overflow, quantize_input,
+                                    quantize_to_int, wrap_to_width)
+
+FRONT = (FoldBias, FoldScale, FuseActivationCasts, FoldViewOps, Resolve)
+
+
+def lower(gb, passes=FRONT):
+    ctx = gb.ctx
+    run_aie_passes(ctx, [p() for p in passes])
+    return ctx
+
+
+# ---- fixed-point helpers (values fixed by the definition of each mode) ---------------------------------
+
+def test_apply_rounding_ties():
+    v = np.array([-2.5, -1.5, -0.5, 0.5, 1.5, 2.5, 2.4, -2.6])
+    assert apply_rounding(v, RoundingMode.TRN).tolist() == [-3, -2, -1, 0, 1, 2, 2, -3]
+    assert apply_rounding(v, RoundingMode.RND_MIN_INF).tolist() == [-3, -2, -1, 0, 1, 2, 2, -3]
+    assert apply_rounding(v, RoundingMode.TRN_ZERO).tolist() == [-2, -1, -0.0, 0, 1, 2, 2, -2]
+    assert apply_rounding(v, RoundingMode.RND_INF).tolist() == [-2, -1, -0.0, 1, 2, 3, 3, -2]
+    assert apply_rounding(v, RoundingMode.RND_CONV).tolist() == [-2, -2, -0.0, 0, 2, 2, 2, -3]
+    assert apply_rounding(v, RoundingMode.RND).tolist() == [-3, -2, -1, 1, 2, 3, 2, -3]
+
+
+def test_overflow_modes():
+    v = np.array([-300, -129, -128, 127, 128, 300])
+    assert handle_overflow(v, 8, True, SaturationMode.SAT).tolist() == [-128, -128, -128, 127, 127, 127]
+    assert handle_overflow(v, 8, True, SaturationMode.SAT_SYM).tolist() == [-127, -127, -127, 127, 127, 127]
+    assert handle_overflow(v, 8, True, SaturationMode.SAT_ZERO).tolist() == [0, 0, 0, 127, 127, 127]
+    assert handle_overflow(v, 8, True, SaturationMode.WRAP).tolist() == [-44, 127, -128, 127, -128, 44]
+    assert handle_overflow(v, 8, False, SaturationMode.SAT).tolist() == [0, 0, 0, 127, 128, 255]
+    assert wrap_to_width(np.array([256, 255, -1]), 8, False).tolist() == [0, 255, 255]
+
+
+def test_quantize_input_and_dequantize():
+    dt = AIEDataType('int8', frac=4, rounding=RoundingMode.RND_CONV, saturation=SaturationMode.SAT)
+    x = np.array([0.03125, 0.09375, -0.09375, 7.99, -9.0, 1.0])
+    assert quantize_input(x, dt).tolist() == [0, 2, -2, 127, -128, 16]   # 0.5 -> 0, 1.5 -> 2 (ties to even)
+    assert quantize_input(x, dt).dtype == np.int8
+    # integer arrays pass through untouched (cast only)
+    assert quantize_input(np.array([300, -5], dtype=np.int64), dt).tolist() == [44, -5]
+    du = AIEDataType('uint8', frac=8, rounding=RoundingMode.TRN, saturation=SaturationMode.WRAP)
+    assert quantize_input(np.array([0.999, 1.0, -1 / 256]), du).tolist() == [255, 0, 255]
+    assert dequantize_output(np.array([16, -8]), 4).tolist() == [1.0, -0.5]
+    assert dequantize_output(np.array([3]), 0).dtype == np.float64
+    w = quantize_to_int(np.array([0.5, -1.0, 0.996]), 7, 8, True, RoundingMode.RND, SaturationMode.SAT)
+    assert w.tolist() == [64, -128, 127] and w.dtype == np.int8
+
+
+# ---- passes ---------------------------------------------------------------------------------------------
+
+def small_mlp(relu_on_last=False):
+    gb = GraphBuilder()
+    x = gb.input('x', (4, 16), qint(8, 4))
+    r = np.random.default_rng(0)
+    h = gb.dense(x, r.integers(-64, 64, (16, 32)) / 128.0, qint(8, 7), qint(8, 4), bias=r.integers(-8, 8, 32) / 16.0,
+                 bias_precision=qint(32, 11), relu=True, name='fc0')
+    y = gb.dense(h, r.integers(-64, 64, (32, 8)) / 128.0, qint(8, 7), qint(8, 3), bias=np.zeros(8),
+                 bias_precision=qint(32, 11), relu=relu_on_last, name='fc1')
+    gb.output(y)
+    return gb
+
+
+def test_fold_bias_fuse_relu_and_resolve_constants():
+    gb = small_mlp()
+    assert [n.op_type for n in gb.graph.nodes] == ['dense', 'add', 'activation', 'dense', 'add']
+    ctx = lower(gb)
+    assert [n.op_type for n in ctx.ir.logical.nodes] == ['dense', 'dense']
+    fc0, fc1 = ctx.ir.logical.nodes
+    assert fc0.metadata['use_bias'] and fc0.roles[fc0.inputs[2].name] == 'bias'
+    assert fc0.traits['fused_activation'].data == {'activation': 'relu'}
+    c0, c1 = ctx.ir.execution.get(fc0.name).config, ctx.ir.execution.get(fc1.name).config
+    assert c0.shift == 4 + 7 - 4 and c1.shift == 4 + 7 - 3
+    assert c0.rounding_mode == 'conv_even' and c0.accumulator_tag == 'acc32'
+    assert c0.flags.use_relu and c0.flags.use_bias and not c1.flags.use_relu
+    assert c0.precision['bias'].format == 'int32' and c0.precision['bias'].frac == 11
+    assert c0.precision['acc'].frac == 11 and c0.precision['output'].format == 'int8'
+    # weights and bias quantise exactly as the reference packs them: bias at 2^(in_frac + w_frac)
+    inst = ctx.ir.execution.get(fc0.name)
+    W, b = inst.variant.quantize_weight_bias(inst)
+    r = np.random.default_rng(0)
+    assert np.array_equal(W, r.integers(-64, 64, (16, 32)))
+    assert np.array_equal(b, r.integers(-8, 8, 32) * 128) and b.dtype == np.int32
+
+
+def test_rounding_token_map():
+    from aie4ml_amd.op_impls.precision import aie_rounding_token
+
+    want = {RoundingMode.TRN: 'floor', RoundingMode.RND_MIN_INF: 'floor', RoundingMode.RND_INF: 'ceil',
+            RoundingMode.RND: 'symmetric_inf', RoundingMode.TRN_ZERO: 'symmetric_zero',
+            RoundingMode.RND_ZERO: 'symmetric_zero', RoundingMode.RND_CONV: 'conv_even'}
+    for mode, token in want.items():
+        assert aie_rounding_token(qint(8, 0, rounding=mode)) == token
+
+
+def test_relu_without_dense_has_no_kernel():
+    gb = GraphBuilder()
+    a = gb.input('a', (4, 32), qint(8, 4))
+    b = gb.input('b', (4, 32), qint(8, 4))
+    s = gb.add(a, b, qint(8, 4))
+    (y,) = gb._emit('activation', 'lonely_relu', [s], [('y', s.shape, qint(8, 4))], ['lhs'], {'activation': 'relu'})
+    gb.output(y)
+    with pytest.raises(NotImplementedError, match='No family resolver'):
+        lower(gb)
+
+
+def attention_graph(scale=0.125, approx=None, hccs=None, frac=4):
+    gb = GraphBuilder()
+    q = gb.input('q', (2, 64, 32), qint(8, frac))
+    k = gb.input('k', (2, 64, 32), qint(8, frac))
+    v = gb.input('v', (2, 64, 32), qint(8, frac))
+    kt = gb.transpose(k, (0, 2, 1))
+    logits = gb.matmul(q, kt, qint(8, frac), name='qk')
+    if scale is not None:
+        logits = gb.scale(logits, scale, qint(8, frac), name='qk_scale')
+    d = {}
+    if approx:
+        d['approximation'] = approx
+    if hccs:
+        d['hccs'] = hccs
+    p = gb.softmax(logits, qint(8, 8, signed=False), name='sm', directives=d or None)
+    o = gb.matmul(p, v, qint(8, frac), name='pv')
+    gb.output(o)
+    return gb
+
+
+def test_transpose_folds_into_matmul_and_scale_prefers_softmax():
+    # a Scale between MatMul and Softmax is absorbed by the Softmax (as in the reference: the consumer
+    # is tried first), so the MatMul keeps its plain alignment shift and EXP_KQ carries the 1/8
+    ctx = lower(attention_graph())
+    kinds = [n.op_type for n in ctx.ir.logical.nodes]
+    assert kinds == ['matmul', 'softmax', 'matmul']
+    qk, sm, pv = ctx.ir.logical.nodes
+    assert qk.traits['io_view'].data['inputs']['k'] == {'perm': [0, 2, 1]}
+    assert 'output_scale' not in qk.traits and sm.traits['input_scale'].data['scale'] == 0.125
+    c = ctx.ir.execution.get(qk.name).config
+    assert c.flags.transpose_rhs and not c.flags.transpose_lhs
+    assert c.shift == 4 + 4 - 4
+    cs = ctx.ir.execution.get(sm.name).config
+    assert cs.approximation == 'exp' and cs.exp_kq == 3    # round(log2(e) * 2^-4 / 8 * 256)
+    assert cs.inv_shift == 15 and cs.rounding_mode == 'floor' and cs.precision['output'].format == 'uint8'
+    cp = ctx.ir.execution.get(pv.name).config
+    assert cp.precision['lhs'].format == 'uint8' and cp.shift == 8 + 4 - 4
+    assert ctx.ir.execution.get('sm_aie') is not None
+    assert lower(attention_graph(scale=None)).ir.execution.get('sm_aie').config.exp_kq == 23
+
+
+def test_scale_after_matmul_folds_into_its_shift():
+    gb = GraphBuilder()
+    a = gb.input('a', (2, 16, 32), qint(8, 4))
+    b = gb.input('b', (2, 32, 16), qint(8, 4))
+    y = gb.scale(gb.matmul(a, b, qint(8, 4), name='mm'), 0.125, qint(8, 4))
+    gb.output(y)
+    ctx = lower(gb)
+    (mm,) = ctx.ir.logical.nodes
+    assert mm.traits['output_scale'].data['scale'] == 0.125
+    c = ctx.ir.execution.get(mm.name).config
+    assert c.shift == (4 + 4 - 4) + 3 and not c.flags.transpose_rhs   # alignment + log2(1/scale)
+
+
+def test_scale_before_softmax_becomes_temperature():
+    gb = GraphBuilder()
+    x = gb.input('x', (8, 64), qint(8, 4))
+    s = gb.scale(x, 0.5, qint(8, 4))
+    p = gb.softmax(s, qint(8, 8, signed=False), name='sm')
+    gb.output(p)
+    ctx = lower(gb)
+    (sm,) = ctx.ir.logical.nodes
+    assert sm.traits['input_scale'].data['scale'] == 0.5
+    assert ctx.ir.execution.get(sm.name).config.exp_kq == round(1.4426950408889634 * 2 ** -4 * 0.5 * 256)
+
+
+def matmul_scale_graph(scale):
+    gb = GraphBuilder()
+    a = gb.input('a', (2, 16, 32), qint(8, 4))
+    b = gb.input('b', (2, 32, 16), qint(8, 4))
+    gb.output(gb.scale(gb.matmul(a, b, qint(8, 4), name='mm'), scale, qint(8, 4)))
+    return gb
+
+
+def test_scale_errors():
+    with pytest.raises(NotImplementedError, match='not a power of two'):
+        lower(matmul_scale_graph(0.3))
+    with pytest.raises(ValueError, match=r'range \(0, 1\]'):
+        lower(matmul_scale_graph(2.0))
+    gb = GraphBuilder()
+    x = gb.input('x', (4, 32), qint(8, 4))
+    y = gb.scale(x, 0.5)
+    gb.output(gb.add(y, x, qint(8, 4)))
+    with pytest.raises(NotImplementedError, match='no adjacent op absorbs this scale'):
+        lower(gb)
+
+
+def test_softmax_variants_and_hccs_validation():
+    ok = {'B': 100, 'S': 1, 'Dmax': 90}
+    ctx = lower(attention_graph(scale=None, approx='hccs', hccs=ok))
+    cfg = ctx.ir.execution.get('sm_aie').config
+    assert cfg.approximation == 'hccs' and cfg.hccs == ok and cfg.param_sets == 1 and not cfg.use_clb
+    with pytest.raises(ValueError, match='directives missing S, Dmax'):
+        lower(attention_graph(scale=None, approx='hccs', hccs={'B': 10}))
+    with pytest.raises(ValueError, match=r'cols \* B <= 32767'):
+        lower(attention_graph(scale=None, approx='hccs', hccs={'B': 600, 'S': 1, 'Dmax': 5}))
+    with pytest.raises(ValueError, match=r'B - S\*Dmax >= 0'):
+        lower(attention_graph(scale=None, approx='hccs', hccs={'B': 50, 'S': 1, 'Dmax': 60}))
+    with pytest.raises(ValueError, match='>= 256 for reciprocal range'):
+        lower(attention_graph(scale=None, approx='hccs', hccs={'B': 60, 'S': 1, 'Dmax': 59}))  # 64 * 1 < 256
+    with pytest.raises(ValueError, match="'S' must be in"):
+        lower(attention_graph(scale=None, approx='hccs', hccs={'B': 300, 'S': 200, 'Dmax': 1}))
+    with pytest.raises(ValueError, match='cannot apply a runtime input_scale'):
+        gb = GraphBuilder()
+        x = gb.input('x', (8, 64), qint(8, 4))
+        gb.output(gb.softmax(gb.scale(x, 0.5), qint(8, 8, signed=False), name='sm',
+                             directives={'approximation': 'hccs', 'hccs': ok}))
+        lower(gb)
+    # exp needs the logit scale in range: frac 12 -> KQ rounds to 0
+    with pytest.raises(ValueError, match='1 <= EXP_KQ'):
+        lower(attention_graph(scale=None, frac=12))
+    # int8 output is not a softmax output type
+    gb = GraphBuilder()
+    x = gb.input('x', (8, 64), qint(8, 4))
+    gb.output(gb.softmax(x, qint(8, 7), name='sm'))
+    with pytest.raises(ValueError, match='requires uint8 or int16 output'):
+        lower(gb)
+
+
+def test_matmul_rules():
+    gb = GraphBuilder()
+    a = gb.input('a', (2, 16, 32), qint(8, 4))
+    b = gb.input('b', (2, 32, 16), qint(8, 4, signed=False))
+    gb.output(gb.matmul(a, b, qint(8, 4)))
+    with pytest.raises(ValueError, match='RHS must use a signed integer precision'):
+        lower(gb)
+    gb = GraphBuilder()
+    a = gb.input('a', (2, 16, 32), qint(8, 4))
+    b = gb.input('b', (2, 16, 32), qint(8, 4))
+    bt = gb.transpose(b, (1, 0, 2))
+    gb.output(gb.matmul(a, bt, qint(8, 4)))
+    with pytest.raises(ValueError):
+        lower(gb)
+    gb = GraphBuilder()
+    a = gb.input('a', (2, 16, 32), qint(16, 4))
+    gb.output(gb.dense(a, np.zeros((32, 8)), qint(8, 7), qint(8, 4)))
+    with pytest.raises(ValueError, match='no dense variant matches'):
+        lower(gb)
+
+
+def ln_graph(cols=64, eps=None, eps_q0=None, gamma=None, out_frac=5):
+    gb = GraphBuilder()
+    a = gb.input('a', (8, cols), qint(8, 4))
+    b = gb.input('b', (8, cols), qint(8, 4))
+    s = gb.add(a, b, qint(8, 4), name='res')
+    y = gb.layer_norm(s, np.ones(cols) * 0.75 if gamma is None else gamma, np.zeros(cols), qint(8, out_frac), epsilon=eps,
+                      eps_q0=eps_q0, name='ln')
+    gb.output(y)
+    return gb
+
+
+def test_layernorm_resolution_and_errors():
+    ctx = lower(ln_graph(eps=2.0 ** -8))
+    cfg = ctx.ir.execution.get('ln_aie').config
+    assert cfg.eps_q0 == 1 and cfg.out_shift == 5 and cfg.gamma_shift == 7 and cfg.cols == 64 and cfg.rows == 8
+    assert cfg.precision['gamma'].frac == 7 and cfg.precision['beta'].frac == 15 and cfg.power_of_two_cols
+    assert ctx.ir.execution.get('res_aie').config.shift == 0
+    assert lower(ln_graph(eps_q0=3)).ir.execution.get('ln_aie').config.eps_q0 == 3
+    assert not lower(ln_graph(cols=48)).ir.execution.get('ln_aie').config.power_of_two_cols  # extension
+    with pytest.raises(ValueError, match='not exactly representable'):
+        lower(ln_graph(eps=1e-5))
+    with pytest.raises(ValueError, match='positive variance floor'):
+        lower(ln_graph(eps=0.0))
+    with pytest.raises(ValueError, match=r'out_shift=20 must be in \[0, 15\]'):
+        lower(ln_graph(out_frac=20))
+    from aie4ml_amd.op_impls.layernorm import pack_layernorm_param
+
+    assert pack_layernorm_param([0.5, -1.0, 0.996], name='gamma', full_inner=3, frac=7).tolist() == [64, -128, 127]
+    with pytest.raises(ValueError, match='cannot be represented as signed int16 Q7'):
+        pack_layernorm_param([300.0], name='gamma', full_inner=1, frac=7)
+    with pytest.raises(ValueError, match='does not match full_inner'):
+        pack_layernorm_param([1.0, 2.0], name='beta', full_inner=3, frac=15)
+
+
+def test_add_requires_one_storage_type():
+    gb = GraphBuilder()
+    a = gb.input('a', (8, 64), qint(8, 4))
+    b = gb.input('b', (8, 64), qint(8, 5))
+    gb.output(gb.add(a, b, qint(8, 4)))
+    with pytest.raises(ValueError, match='same storage type'):
+        lower(gb)
+    gb = GraphBuilder()
+    a = gb.input('a', (8, 64), qint(8, 4))
+    b = gb.input('b', (8, 32), qint(8, 4))
+    gb.output(gb.add(a, b, qint(8, 4)))
+    with pytest.raises(ValueError, match='exact-shape inputs'):
+        lower(gb)
+
+
+def test_split_concat_become_view_placeholders():
+    gb = GraphBuilder()
+    x = gb.input('x', (4, 8, 96), qint(8, 4))
+    a, b, c = gb.split(x, -1, [32, 32, 32], name='sp')
+    y = gb.concat([c, a], -1, name='cat')
+    gb.output(gb.add(y, gb.concat([a, b], -1, name='cat2'), qint(8, 4)))
+    ctx = lower(gb)
+    sp = next(n for n in ctx.ir.logical.nodes if n.name == 'sp_aie')
+    assert sp.is_placeholder and sp.traits['slice_view'].data['axis'] == 2
+    assert [s['start'] for s in sp.traits['slice_view'].data['slices']] == [0, 32, 64]
+    cat = next(n for n in ctx.ir.logical.nodes if n.name == 'cat_aie')
+    assert cat.is_placeholder and [s['start'] for s in cat.traits['concat_view'].data['slices']] == [0, 32]
+    assert ctx.ir.execution.get('sp_aie') is None
+
+
+def test_gpu_fusion_plan():
+    ctx = lower(small_mlp(), FRONT + (PlanGpuFusion,))
+    assert ctx.config['gpu_fusion_plan']['mlp_chains'] == [['fc0_aie', 'fc1_aie']]
+    ctx = lower(ln_graph(), FRONT + (PlanGpuFusion,))
+    assert ctx.config['gpu_fusion_plan']['add_layernorm'] == {'res_aie': {'layer_norm': 'ln_aie', 'keep_sum': False}}
+
+
+def test_encoder_block_graph_lowers():
+    from aie4ml_amd import workloads
+
+    model, x = workloads.c5_encoder_block(batch=2, seq=32, hidden=64, heads=2, ffn=128)
+    ctx = lower(GraphHolder(model), FRONT + (PlanGpuFusion,))
+    kinds = [n.op_type for n in ctx.ir.logical.nodes if not n.is_placeholder]
+    assert kinds.count('dense') == 4 and kinds.count('matmul') == 4 and kinds.count('softmax') == 2
+    assert kinds.count('layer_norm') == 2 and kinds.count('add') == 2
+    plan = ctx.config['gpu_fusion_plan']
+    assert plan['add_layernorm']['residual1_aie'] == {'layer_norm': 'ln1_aie', 'keep_sum': False}
+    assert plan['mlp_chains'] == [['ffn1_aie', 'ffn2_aie']]   # widths 64/128/64 fit the fused-MLP kernel
+    assert x.shape == (2, 32, 64) and x.dtype == np.int8
+
+
+class GraphHolder:
+    """Adapts a model to the `gb.ctx` attribute lower() expects."""
+
+    def __init__(self, model):
+        self.ctx = get_backend_context(model)
+
+
+def test_predict_input_contract_without_gpu():
+    gb = small_mlp()
+    model = gb.build()
+    with pytest.raises(ValueError, match='Unknown simulator'):
+        model.predict(np.zeros((4, 16)), simulator='x86')
+    good = model.prepare_inputs(np.zeros((4, 16)))
+    assert good['x'].shape == (1, 4, 16) and good['x'].dtype == np.int8
+    assert model.prepare_inputs(np.zeros((3, 4, 16)))['x'].shape == (3, 4, 16)
+    assert model.prepare_inputs({'x': np.zeros((1, 4, 16))})['x'].shape == (1, 4, 16)
+    with pytest.raises(ValueError, match='expected shape'):
+        model.prepare_inputs(np.zeros((4, 15)))
+    with pytest.raises(ValueError, match='quantize=False requires integer inputs'):
+        model.prepare_inputs(np.zeros((4, 16)), quantize=False)
+    assert model.prepare_inputs(np.full((4, 16), 1.0))['x'][0, 0, 0] == 16   # 1.0 * 2^4
