@@ -7,7 +7,9 @@ saturate to int8, fused ReLU). One step = one pass of the operator over the whol
 inputs already resident in HBM. Prints ONE JSON line.
 
 Other workloads (--workload c1_mlp | c3_softmax_exp | c3_softmax_hccs | c3_qk | c3_pv |
-c4_add_layernorm | c4_layernorm | c4_add) print the same line for that operator.
+c4_add_layernorm | c4_layernorm | c4_add | c5_encoder) print the same line for that operator or graph;
+--workload calib_copy runs a plain 256 MiB elementwise copy, the known-size kernel the HBM traffic
+counters are scaled against.
 """
 
 from __future__ import annotations
@@ -26,6 +28,15 @@ sys.path.insert(0, str(ROOT))
 
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, TOP/s
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
+
+# HBM bytes per launch of each workload's dominant kernel, from hardware counters (FETCH_SIZE and
+# WRITE_SIZE, one counter run each, scaled by what the same counter reads for calib_copy).
+# None = not measured.
+MEASURED_TRAFFIC = {
+    'c2_dense': 215313495, 'c1_mlp': 115929, 'c4_add': 46997271, 'c4_layernorm': 31996938,
+    'c4_add_layernorm': 47107737, 'c3_softmax_exp': 255051182, 'c3_softmax_hccs': 255049600,
+    'c3_qk': 225000660, 'c3_pv': 198540800, 'calib_copy': 536870912,
+}
 
 
 def _time_gpu(torch, fn, steps, warmup):
@@ -78,6 +89,7 @@ def main():
     wl = args.workload
     extra = {}
     cpu_fn = None
+    cpu_samples = None
 
     if wl == 'c2_dense':
         M, K, N = 8192, 4096, 4096
@@ -101,7 +113,7 @@ def main():
         cpu_fn = lambda: oracle.dense(A[:sample_rows], W, bias, shifts, 'conv_even', relu=True)  # noqa: E731
         cpu_work = 2.0 * sample_rows * N * K
         metric, unit = 'int8_dense_tops', 'TOP/s'
-        kernel = 'gemm_i8_nt_kernel'
+        kernel = 'gemm_i8_rs_kernel'
     elif wl == 'c1_mlp':
         x, layers = workloads.c1_mlp(1024)
         specs = [ops.MlpLayerSpec(ops.pack_dense(dev(Wl), dev(b), s), s, relu, o) for (Wl, b, s, relu, o) in layers]
@@ -174,7 +186,7 @@ def main():
             cpu_work = bytes_ * 4 / (Bt * H)
             cpu_desc = 'oracle MatMul on 4 of 512 (batch, head) slices'
             work = float(bytes_)
-            kernel = 'gemm_i8_nt_kernel'
+            kernel = 'gemm_i8_dtl_kernel'
         elif wl == 'c3_pv':
             ws = torch.empty((ops._lib.load().a4g_matmul_i8_workspace_bytes(Bt * H, S, D, S, 0, 1),), dtype=torch.uint8,
                              device='cuda')
@@ -190,7 +202,7 @@ def main():
             cpu_fn = lambda: oracle.matmul(pl, v[0, :4], prm['pv_shift'], 'conv_even')  # noqa: E731
             cpu_work = bytes_ * 4 / (Bt * H)
             cpu_desc = 'oracle MatMul (uint8 x int8) on 4 of 512 (batch, head) slices'
-            kernel = 'gemm_i8_nt_kernel'
+            kernel = 'gemm_i8_rs_kernel'
         else:
             out = torch.empty(logits.shape, dtype=torch.uint8, device='cuda')
             hc = prm['hccs']
@@ -214,6 +226,45 @@ def main():
         samples = Bt
         config = {'workload': f'{wl}: attention core batch 32 x 16 heads, seq 512, head_dim 64'}
         metric, unit = f'{wl}_gbs', 'GB/s'
+    elif wl == 'c5_encoder':
+        from oracle.graph import run_graph
+
+        batch, seq, hidden, heads, ffn = 64, 128, 768, 12, 3072
+        model, x = workloads.c5_encoder_block(batch, seq, hidden, heads, ffn, softmax='hccs')
+        model.compile()
+        dx = {'x': dev(x)}
+        out_name = model.context.ir.logical.output_tensor_names[0]
+        fn = lambda: model.execute(dx)  # noqa: E731
+        got = fn()[out_name]
+        torch.cuda.synchronize()
+        nsub = 2
+        ref = run_graph(model, oracle, {'x': x[:nsub]})[out_name]
+        bit_exact = bool(np.array_equal(got[:nsub].cpu().numpy(), ref))
+        rows = batch * seq
+        gemm_ops = 2.0 * rows * (hidden * 3 * hidden + hidden * hidden + 2 * hidden * ffn)
+        attn_ops = 2 * 2.0 * batch * heads * seq * seq * (hidden // heads)
+        work, bound = gemm_ops + attn_ops, 'mfma'
+        samples = batch
+        config = {'workload': f'c5_encoder: int8 encoder block, hidden {hidden}, {heads} heads, FFN {ffn}, seq {seq}, '
+                              f'batch {batch}, HCCS softmax, LayerNorm over {hidden} columns, through the graph executor'}
+        cpu_fn = lambda: run_graph(model, oracle, {'x': x[:nsub]})  # noqa: E731
+        cpu_work = work * nsub / batch
+        cpu_desc = f'oracle graph interpreter on {nsub} of {batch} sequences'
+        metric, unit = 'int8_encoder_sequences_per_s', 'samples/s'
+        kernel = 'whole graph (GEMM kernels dominate)'
+        cpu_samples = nsub
+    elif wl == 'calib_copy':
+        n = 256 << 20
+        src = torch.randint(-128, 127, (n,), dtype=torch.int8, device='cuda')
+        dst = torch.empty_like(src)
+        fn = lambda: torch.add(src, 0, out=dst)  # noqa: E731
+        fn()
+        torch.cuda.synchronize()
+        bit_exact = bool(torch.equal(src, dst))
+        work, bound, samples = 2.0 * n, 'hbm', 1
+        config = {'workload': 'calib_copy: 256 MiB read + 256 MiB write, one elementwise kernel'}
+        metric, unit = 'copy_gbs', 'GB/s'
+        kernel = 'elementwise_kernel'
     else:
         sys.exit(f'unknown workload {wl}')
 
@@ -222,12 +273,12 @@ def main():
     if bound == 'mfma':
         achieved = work / (ms_ev * 1e-3) / 1e12
         roof = {'bound': 'mfma', 'achieved': round(achieved, 3), 'peak': PEAK_INT8_TOPS, 'unit': 'TOP/s',
-                'frac': round(achieved / PEAK_INT8_TOPS, 4), 'traffic': None, 'kernel': kernel,
+                'frac': round(achieved / PEAK_INT8_TOPS, 4), 'traffic': MEASURED_TRAFFIC.get(wl), 'kernel': kernel,
                 'kernel_ms': round(ms_ev, 5)}
     else:
         achieved = work / (ms_ev * 1e-3) / 1e9
         roof = {'bound': 'hbm', 'achieved': round(achieved, 2), 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
-                'frac': round(achieved / PEAK_HBM_GBS, 4), 'traffic': None, 'kernel': kernel,
+                'frac': round(achieved / PEAK_HBM_GBS, 4), 'traffic': MEASURED_TRAFFIC.get(wl), 'kernel': kernel,
                 'kernel_ms': round(ms_ev, 5)}
 
     if unit == 'TOP/s':
@@ -245,7 +296,7 @@ def main():
         elif unit == 'GB/s':
             v = cpu_work / t / 1e9
         else:
-            v = samples / t
+            v = (cpu_samples or samples) / t
         cpu = {'value': float(f'{v:.6g}'), 'unit': unit, 'cores': oracle.num_threads(), 'kind': 'port',
                'sample': cpu_desc, 'host_cpus': os.cpu_count()}
 

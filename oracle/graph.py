@@ -1,4 +1,4 @@
-"""Test-only graph interpreter: walks a resolved operator graph and evaluates every node with the CPU
+"""Checker-only graph interpreter (test infrastructure, never on the product path): walks a resolved operator graph and evaluates every node with the CPU
 oracle. It shares the graph and the resolved constants with the GPU executor, but none of its arithmetic."""
 
 import numpy as np

@@ -8,7 +8,7 @@ import pytest
 from aie4ml_amd import GraphBuilder, qint, workloads
 from aie4ml_amd.aie_types import RoundingMode
 
-from ir_oracle import run_graph
+from oracle.graph import run_graph
 
 pytestmark = pytest.mark.gpu
 
