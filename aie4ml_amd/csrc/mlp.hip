@@ -2,17 +2,16 @@
 // resident in LDS, activations never leaving the CU. Same arithmetic, layer by layer, as the Dense
 // kernel (dense_bias_relu.cpp:112-163): acc32 = bias + sum a*w; srs; ReLU.
 //
-// A workgroup of 256 threads owns 64 samples. Lane l of every wave works on sample l; the four waves
-// split the output neurons of a layer between them. Weights are read from LDS as wave-uniform
-// (broadcast) dwords, activations as per-lane dwords from a padded LDS row, and four MACs retire per
-// v_dot4_i32_i8. uint8 activations are biased to int8 with x ^ 0x80 and corrected by 128 * colsum.
+// A workgroup of 256 threads owns 64 (or, for small batches, 16) samples. A lane works on one sample
+// and four output neurons at a time; weights are read from LDS as (mostly) wave-uniform dwords,
+// activations as per-lane dwords from a padded LDS row, and four MACs retire per v_dot4_i32_i8.
+// uint8 activations are biased to int8 with x ^ 0x80 and corrected by 128 * colsum.
 #include "common.hpp"
 
 namespace a4g {
 
 constexpr int MLP_MAX_LAYERS = 8;
 constexpr int MLP_MAX_WIDTH = 256;
-constexpr int MLP_SAMPLES = 64;                      // per workgroup
 constexpr int MLP_ACT_PITCH = MLP_MAX_WIDTH + 4;     // bytes; 65 dwords -> conflict-free lane stride
 constexpr int MLP_MAX_WEIGHT_BYTES = 96 * 1024;
 
@@ -24,6 +23,7 @@ struct MlpLayerDev {
     int K, N;
     int shift, relu, out_kind;
     int w_off;  // byte offset of this layer's weights in LDS
+    int b_off;  // byte offset of this layer's effective bias (int32 per neuron) in LDS
 };
 
 struct MlpArgs {
@@ -36,33 +36,80 @@ struct MlpArgs {
     int x_unsigned;
     int mode;
     int weight_bytes;
+    int total_chunks;  // 16-byte chunks of packed weights over all layers
 };
 
+// SPW = samples per workgroup (64 or 16). A wave holds SPW samples x 64/SPW neuron slots: lane l works on
+// sample l % SPW and, in each pass, on four neurons of its slot. Small batches use SPW = 16 so that the
+// work spreads over four times as many CUs and each wave's serial chain is four times shorter.
+template <int SPW>
 __global__ __launch_bounds__(256) void mlp_fused_kernel(MlpArgs a) {
     extern __shared__ __attribute__((aligned(16))) int8_t smem[];
     int8_t* sW = smem;
     int8_t* sAct0 = smem + a.weight_bytes;
-    int8_t* sAct1 = sAct0 + MLP_SAMPLES * MLP_ACT_PITCH;
+    int8_t* sAct1 = sAct0 + SPW * MLP_ACT_PITCH;
+    constexpr int SLOTS = 64 / SPW;   // neuron slots per wave
+    constexpr int NPW = 4 * SLOTS;    // neurons in flight per workgroup and pass step
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int smp = lane % SPW, slot = lane / SPW;
 
-    // stage all weights once (16-byte copies; rows are already zero padded to a multiple of 16)
-    for (int l = 0; l < a.n_layers; ++l) {
-        const MlpLayerDev& L = a.layer[l];
-        const int chunks = L.N * L.ldwt / 16;
-        for (int c = tid; c < chunks; c += 256)
-            *reinterpret_cast<v4i*>(sW + L.w_off + c * 16) = *reinterpret_cast<const v4i*>(L.wt + static_cast<int64_t>(c) * 16);
+    // Stage every layer's weights (16-byte chunks, LDS image = concatenation in layer order) and the
+    // per-neuron accumulator start value: bias, plus 128 * column sum when the layer's input is uint8.
+    // All global loads of a batch of chunks are issued before the first LDS store.
+    for (int c0 = tid; c0 < a.total_chunks; c0 += 256 * 4) {
+        v4i r[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = c0 + 256 * j;
+            r[j] = v4i{0, 0, 0, 0};
+            if (c < a.total_chunks) {
+                int l = 0;
+                while (l + 1 < a.n_layers && c * 16 >= a.layer[l + 1].w_off) ++l;
+                r[j] = *reinterpret_cast<const v4i*>(a.layer[l].wt + (static_cast<int64_t>(c) * 16 - a.layer[l].w_off));
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = c0 + 256 * j;
+            if (c < a.total_chunks) *reinterpret_cast<v4i*>(sW + c * 16) = r[j];
+        }
+    }
+    {
+        int in_u = a.x_unsigned;
+        for (int l = 0; l < a.n_layers; ++l) {
+            const MlpLayerDev& L = a.layer[l];
+            int* sb = reinterpret_cast<int*>(sW + L.b_off);
+            for (int n = tid; n < L.N; n += 256) {
+                int b = L.bias ? L.bias[n] : 0;
+                if (in_u) b += 128 * L.colsum[n];
+                sb[n] = b;
+            }
+            in_u = L.out_kind == A4G_U8;
+        }
     }
 
-    for (int s0 = blockIdx.x * MLP_SAMPLES; s0 < a.batch; s0 += gridDim.x * MLP_SAMPLES) {
+    const int K0 = a.layer[0].K, K0p = a.layer[0].ldwt;
+    const bool vec_in = (K0 & 15) == 0 && (a.ldx & 15) == 0 && (reinterpret_cast<uintptr_t>(a.X) & 15) == 0;
+    for (int s0 = blockIdx.x * SPW; s0 < a.batch; s0 += gridDim.x * SPW) {
         // input rows -> LDS, zero padded to the first layer's packed K
-        const int K0 = a.layer[0].K, K0p = a.layer[0].ldwt;
         __syncthreads();
-        for (int i = tid; i < MLP_SAMPLES * K0p; i += 256) {
-            const int s = i / K0p, k = i % K0p;
-            int8_t v = 0;
-            if (k < K0 && s0 + s < a.batch) v = a.X[static_cast<int64_t>(s0 + s) * a.ldx + k];
-            sAct0[s * MLP_ACT_PITCH + k] = v;
+        if (vec_in) {
+            const int cpr = K0 >> 4;  // 16-byte chunks per row
+            for (int i = tid; i < SPW * cpr; i += 256) {
+                const int s = i / cpr, c = i % cpr;
+                v4i v{0, 0, 0, 0};
+                if (s0 + s < a.batch) v = *reinterpret_cast<const v4i*>(a.X + static_cast<int64_t>(s0 + s) * a.ldx + c * 16);
+                int* d = reinterpret_cast<int*>(sAct0 + s * MLP_ACT_PITCH + c * 16);  // pitch is 4-byte aligned only
+                d[0] = v[0]; d[1] = v[1]; d[2] = v[2]; d[3] = v[3];
+            }
+        } else {
+            for (int i = tid; i < SPW * K0p; i += 256) {
+                const int s = i / K0p, k = i % K0p;
+                int8_t v = 0;
+                if (k < K0 && s0 + s < a.batch) v = a.X[static_cast<int64_t>(s0 + s) * a.ldx + k];
+                sAct0[s * MLP_ACT_PITCH + k] = v;
+            }
         }
         __syncthreads();
 
@@ -76,28 +123,45 @@ __global__ __launch_bounds__(256) void mlp_fused_kernel(MlpArgs a) {
             const int lo = L.relu ? max(kind_lo(L.out_kind), 0) : kind_lo(L.out_kind), hi = kind_hi(L.out_kind);
             const RoundCfg rc = make_round(a.mode, L.shift);
             const int xm = in_unsigned ? static_cast<int>(0x80808080u) : 0;
-            const int* arow = reinterpret_cast<const int*>(in + lane * MLP_ACT_PITCH);
+            const int* arow = reinterpret_cast<const int*>(in + smp * MLP_ACT_PITCH);
             const int next_kp = last ? 0 : a.layer[l + 1].ldwt;
-            for (int n = wave; n < L.N; n += 4) {
-                const int* wrow = reinterpret_cast<const int*>(sW + L.w_off + n * L.ldwt);
-                int acc = L.bias ? L.bias[n] : 0;
-                if (in_unsigned) acc += 128 * L.colsum[n];
-                for (int k4 = 0; k4 < k4n; ++k4) acc = __builtin_amdgcn_sdot4(arow[k4] ^ xm, wrow[k4], acc, false);
-                const int y = clamp_i(apply_round(acc, rc), lo, hi);
-                if (last) {
-                    if (s0 + lane < a.batch) {
-                        if (L.out_kind == A4G_I16)
-                            static_cast<int16_t*>(a.Y)[static_cast<int64_t>(s0 + lane) * a.ldy + n] = static_cast<int16_t>(y);
-                        else
-                            static_cast<int8_t*>(a.Y)[static_cast<int64_t>(s0 + lane) * a.ldy + n] = static_cast<int8_t>(y);
+            const int* sb = reinterpret_cast<const int*>(sW + L.b_off);
+            // four neurons per lane and pass: one activation read feeds four dot products
+            for (int n0 = wave * SLOTS + slot; n0 < L.N; n0 += 4 * NPW) {
+                int acc[4];
+                const int* wrow[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int n = min(n0 + NPW * j, L.N - 1);
+                    wrow[j] = reinterpret_cast<const int*>(sW + L.w_off + n * L.ldwt);
+                    acc[j] = sb[n];
+                }
+#pragma unroll 4
+                for (int k4 = 0; k4 < k4n; ++k4) {
+                    const int av = arow[k4] ^ xm;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_sdot4(av, wrow[j][k4], acc[j], false);
+                }
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int n = n0 + NPW * j;
+                    if (n >= L.N) break;
+                    const int y = clamp_i(apply_round(acc[j], rc), lo, hi);
+                    if (last) {
+                        if (s0 + smp < a.batch) {
+                            if (L.out_kind == A4G_I16)
+                                static_cast<int16_t*>(a.Y)[static_cast<int64_t>(s0 + smp) * a.ldy + n] = static_cast<int16_t>(y);
+                            else
+                                static_cast<int8_t*>(a.Y)[static_cast<int64_t>(s0 + smp) * a.ldy + n] = static_cast<int8_t>(y);
+                        }
+                    } else {
+                        out[smp * MLP_ACT_PITCH + n] = static_cast<int8_t>(y);
                     }
-                } else {
-                    out[lane * MLP_ACT_PITCH + n] = static_cast<int8_t>(y);
                 }
             }
             if (!last) {
                 // zero the padding columns the next layer's dot products will touch
-                for (int n = L.N + wave; n < next_kp; n += 4) out[lane * MLP_ACT_PITCH + n] = 0;
+                for (int n = L.N + wave * SLOTS + slot; n < next_kp; n += NPW) out[smp * MLP_ACT_PITCH + n] = 0;
                 __syncthreads();
                 int8_t* t = in;
                 in = out;
@@ -156,8 +220,14 @@ extern "C" int a4g_mlp_i8(const a4g_mlp_layer* layers, int n_layers, const void*
         off += d.N * d.ldwt;
         in_kind = s.out_kind;
     }
-    A4G_REQUIRE(off <= MLP_MAX_WEIGHT_BYTES, A4G_ERR_UNSUPPORTED, "%s: %d bytes of packed weights exceed the LDS budget of %d",
-                who, off, MLP_MAX_WEIGHT_BYTES);
+    const int weights_only = off;
+    for (int l = 0; l < n_layers; ++l) {
+        off = (off + 15) / 16 * 16;
+        a.layer[l].b_off = off;
+        off += a.layer[l].N * 4;
+    }
+    A4G_REQUIRE(weights_only <= MLP_MAX_WEIGHT_BYTES, A4G_ERR_UNSUPPORTED,
+                "%s: %d bytes of packed weights exceed the LDS budget of %d", who, weights_only, MLP_MAX_WEIGHT_BYTES);
     if (batch == 0) return A4G_OK;
     A4G_REQUIRE(X && Y, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
     A4G_REQUIRE(ldx >= layers[0].K && ldy >= layers[n_layers - 1].N, A4G_ERR_INVALID_ARGUMENT, "%s: pitch smaller than the row",
@@ -172,16 +242,26 @@ extern "C" int a4g_mlp_i8(const a4g_mlp_layer* layers, int n_layers, const void*
     a.mode = round_mode;
     a.weight_bytes = (off + 15) / 16 * 16;
 
-    const int lds = a.weight_bytes + 2 * MLP_SAMPLES * MLP_ACT_PITCH;
+    a.total_chunks = weights_only / 16;
+
     static bool attr_set = false;
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(mlp_fused_kernel),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(mlp_fused_kernel<64>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e == hipSuccess)
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(mlp_fused_kernel<16>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return check_hip(e, who);
         attr_set = true;
     }
-    int grid = static_cast<int>((batch + MLP_SAMPLES - 1) / MLP_SAMPLES);
+    // 64 samples per workgroup once that fills the chip (2 workgroups per CU), 16 below
+    const int spw = batch >= 64 * 512 ? 64 : 16;
+    const int lds = a.weight_bytes + 2 * spw * MLP_ACT_PITCH;
+    int grid = static_cast<int>((batch + spw - 1) / spw);
     if (grid > 256 * 4) grid = 256 * 4;
-    hipLaunchKernelGGL(mlp_fused_kernel, dim3(grid), dim3(256), lds, stream, a);
+    if (spw == 64)
+        hipLaunchKernelGGL(mlp_fused_kernel<64>, dim3(grid), dim3(256), lds, stream, a);
+    else
+        hipLaunchKernelGGL(mlp_fused_kernel<16>, dim3(grid), dim3(256), lds, stream, a);
     return check_hip(hipGetLastError(), who);
 }

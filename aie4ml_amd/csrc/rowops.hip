@@ -109,17 +109,36 @@ namespace a4g {
 // Integer LayerNorm                                 (reference: layer_norm.cpp:14-121)
 // =====================================================================================================
 
-// Nearest Q15 of 1/sqrt(v), v >= 1, clamped to 32767: float seed, exact integer correction
-// ((2q-1)^2 v <= 2^32 < (2q+1)^2 v).
-__device__ __forceinline__ int rsqrt_q15(int v) {
-    if (v < 1) v = 1;
-    long long q = static_cast<long long>(32768.0f * __frsqrt_rn(static_cast<float>(v)) + 0.5f);
-    if (q < 1) q = 1;
-    const unsigned long long two32 = 1ull << 32;
-    const unsigned long long uv = static_cast<unsigned long long>(v);
-    while (q > 0 && static_cast<unsigned long long>((2 * q - 1) * (2 * q - 1)) * uv > two32) --q;
-    while (static_cast<unsigned long long>((2 * q + 1) * (2 * q + 1)) * uv <= two32) ++q;
-    return static_cast<int>(q > 32767 ? 32767 : q);
+// Nearest Q15 of 1/sqrt(v), v >= 1, clamped to 32767: the answer is the largest q with
+// (2q-1)^2 * v <= 2^32. A float seed is within one of it (relative error of v_rsq_f32 and of the
+// int->float conversion are ~2^-22, q < 2^15), so testing the seed and its successor decides.
+__device__ __forceinline__ bool rsqrt_q15_fits(unsigned q, unsigned v) {
+    const unsigned a = (2u * q - 1u) * (2u * q - 1u);  // q <= 23172 here: no overflow
+    const unsigned lo = a * v, hi = __umulhi(a, v);
+    return hi == 0u || (hi == 1u && lo == 0u);
+}
+__device__ __forceinline__ int rsqrt_q15(int vi) {
+    const unsigned v = vi < 1 ? 1u : static_cast<unsigned>(vi);
+    if (v < 2u) return 32767;  // exact value 32768 saturates
+    unsigned q = static_cast<unsigned>(32768.0f * __frsqrt_rn(static_cast<float>(v)) + 0.5f);
+    if (q < 1u) q = 1u;
+    const bool t0 = rsqrt_q15_fits(q, v), t1 = rsqrt_q15_fits(q + 1u, v);
+    q = t0 ? (t1 ? q + 1u : q) : q - 1u;
+    if (q < 1u) q = 1u;
+    return static_cast<int>(q);
+}
+
+// floor(n / d) for any int32 n and 1 <= d <= 65536: float quotient (within one of the answer,
+// |n|/d * 2^-23 < 1), then exact remainder fix-up.
+__device__ __forceinline__ int floordiv_small(int n, int d) {
+    int q = static_cast<int>(floorf(static_cast<float>(n) / static_cast<float>(d)));
+    int r = n - q * d;  // |r| < 3d: no overflow
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        if (r < 0) { r += d; --q; }
+        if (r >= d) { r -= d; ++q; }
+    }
+    return q;
 }
 
 struct RowStats {
@@ -138,10 +157,10 @@ __device__ __forceinline__ RowStats row_stats(int sx, int sq, int cols, int log2
                                          static_cast<unsigned>(cols) * static_cast<unsigned>(mu) * static_cast<unsigned>(mu));
         var = csq >> log2c;
     } else {
-        mu = static_cast<int>(floordiv64(static_cast<int64_t>(sx) + (cols >> 1), cols));
+        mu = floordiv_small(sx + (cols >> 1), cols);
         const int csq = static_cast<int>(static_cast<unsigned>(sq) - 2u * static_cast<unsigned>(mu) * static_cast<unsigned>(sx) +
                                          static_cast<unsigned>(cols) * static_cast<unsigned>(mu) * static_cast<unsigned>(mu));
-        var = static_cast<int>(floordiv64(csq, cols));
+        var = floordiv_small(csq, cols);
     }
     if (var < 0) var = 0;
     st.mu = static_cast<int16_t>(mu);
@@ -151,84 +170,154 @@ __device__ __forceinline__ RowStats row_stats(int sx, int sq, int cols, int log2
 
 __device__ __forceinline__ int sext8(unsigned w, int j) { return static_cast<int>(w << (24 - 8 * j)) >> 24; }
 
-// One wave per row; lane l owns the 16-byte chunks l, l+64, ... (NCH of them). gamma/beta for those
-// columns stay in registers across the rows a wave processes.
-template <int NCH, int MODE, bool FUSE_ADD>
-__global__ __launch_bounds__(256) void layernorm_wave_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ x2,
+// Rounding of the two requantisations in the row kernel. Every mode is (acc + c0 + bit) >> s with bit
+// taken from acc itself; BIT selects where: 0 none, 1 minus the sign bit (symmetric_inf), 2 plus the
+// sign bit (symmetric_zero), 3 plus the parity of acc >> s (conv_even), 4 minus it (conv_odd).
+// w is the extracted field's width: 1, or 0 when s == 0 (then c0 == 0 too and acc passes unchanged).
+// |acc| < 2^30 here, so the additions cannot overflow.
+struct LnRound {
+    int s, c0, w;
+};
+static LnRound make_ln_round(int mode, int s, int* bit_kind) {
+    LnRound r{s, 0, s > 0 ? 1 : 0};
+    const int h = s > 0 ? (1 << (s - 1)) : 0;
+    int kind = 0;
+    switch (mode) {
+    case A4G_RND_FLOOR: break;
+    case A4G_RND_CEIL: r.c0 = s > 0 ? (1 << s) - 1 : 0; break;
+    case A4G_RND_POSITIVE_INF: r.c0 = h; break;
+    case A4G_RND_NEGATIVE_INF: r.c0 = s > 0 ? h - 1 : 0; break;
+    case A4G_RND_SYMMETRIC_INF: r.c0 = h; kind = 1; break;
+    case A4G_RND_SYMMETRIC_ZERO: r.c0 = s > 0 ? h - 1 : 0; kind = 2; break;
+    case A4G_RND_CONV_EVEN: r.c0 = s > 0 ? h - 1 : 0; kind = 3; break;
+    default: r.c0 = h; kind = 4; break;
+    }
+    *bit_kind = kind;
+    return r;
+}
+template <int BIT>
+__device__ __forceinline__ int ln_round(int acc, const LnRound& r) {
+    int bit = 0;
+    if (BIT == 1) bit = __builtin_amdgcn_sbfe(acc, 31, r.w);
+    if (BIT == 2) bit = static_cast<int>(__builtin_amdgcn_ubfe(static_cast<unsigned>(acc), 31, r.w));
+    if (BIT == 3) bit = static_cast<int>(__builtin_amdgcn_ubfe(static_cast<unsigned>(acc), r.s, r.w));
+    if (BIT == 4) bit = __builtin_amdgcn_sbfe(acc, r.s, r.w);
+    return (acc + r.c0 + bit) >> r.s;
+}
+
+// L lanes per row, 64/L rows per wave at a time; a lane owns the 16-byte chunks l, l+L, ... (NCH of
+// them) of its row. gamma/beta are widened to int32 once per block and kept in LDS, quad-major
+// ([4][nchunks][4] ints) so that the lanes of a group read consecutive 16-byte words. x is read from
+// HBM once: the statistics and the normalisation both work from registers, and the next rows' loads
+// are issued before the current rows are normalised.
+template <int L, int NCH, int BIT, bool FUSE_ADD>
+__global__ __launch_bounds__(256, 2) void layernorm_rows_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ x2,
                                                               const int16_t* __restrict__ gamma,
                                                               const int16_t* __restrict__ beta, int8_t* __restrict__ sum_out,
                                                               int8_t* __restrict__ out, int rows, int cols, int log2c,
-                                                              int eps_q0, int gamma_shift, int final_shift) {
+                                                              int eps_q0, LnRound rg, LnRound ro) {
+    extern __shared__ int ln_lds[];
+    const int nchunks = cols >> 4;
+    int* lg = ln_lds;
+    int* lb = ln_lds + nchunks * 16;
+
+    constexpr int G = 64 / L;  // rows per wave and iteration
     const int lane = threadIdx.x & 63;
+    const int grp = lane / L, sub = lane % L;
     const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
     const int nwaves = (gridDim.x * blockDim.x) >> 6;
 
     bool valid[NCH];
-    v4i g[NCH][2], bt[NCH][2];
+    int chunk_of[NCH];
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-        const int col0 = (lane + 64 * i) * 16;
-        valid[i] = col0 < cols;
-        if (valid[i]) {
-            g[i][0] = *reinterpret_cast<const v4i*>(gamma + col0);
-            g[i][1] = *reinterpret_cast<const v4i*>(gamma + col0 + 8);
-            bt[i][0] = *reinterpret_cast<const v4i*>(beta + col0);
-            bt[i][1] = *reinterpret_cast<const v4i*>(beta + col0 + 8);
-        } else {
-            g[i][0] = g[i][1] = bt[i][0] = bt[i][1] = v4i{0, 0, 0, 0};
-        }
+        const int chunk = sub + L * i;
+        valid[i] = chunk < nchunks;
+        chunk_of[i] = valid[i] ? chunk : 0;
     }
 
-    for (int row = wave; row < rows; row += nwaves) {
+    v4i nx[NCH], nx2[NCH];
+    auto fetch = [&](int row) {
+        const bool live = row < rows;
+        const int64_t base = static_cast<int64_t>(row) * cols;
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            nx[i] = v4i{0, 0, 0, 0};
+            if (FUSE_ADD) nx2[i] = v4i{0, 0, 0, 0};
+            if (live && valid[i]) {
+                nx[i] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(x + base + chunk_of[i] * 16));
+                if (FUSE_ADD)
+                    nx2[i] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(x2 + base + chunk_of[i] * 16));
+            }
+        }
+    };
+
+    // the first rows are requested before the parameters are staged, so both latencies overlap
+    int row0 = wave * G;
+    if (row0 < rows) fetch(row0 + grp);
+
+    // 8 int16 parameters per load; half-chunk hc = 8 columns = quads 2*(hc&1), 2*(hc&1)+1 of chunk hc>>1
+    for (int hc = threadIdx.x; hc < 4 * nchunks; hc += blockDim.x) {
+        const bool is_beta = hc >= 2 * nchunks;
+        const int h = is_beta ? hc - 2 * nchunks : hc;
+        const v4i raw = *reinterpret_cast<const v4i*>((is_beta ? beta : gamma) + h * 8);
+        int* dst = is_beta ? lb : lg;
+        const int chunk = h >> 1, q0 = (h & 1) * 2;
+        v4i lo, hi;
+        lo[0] = static_cast<int16_t>(raw[0]); lo[1] = raw[0] >> 16; lo[2] = static_cast<int16_t>(raw[1]); lo[3] = raw[1] >> 16;
+        hi[0] = static_cast<int16_t>(raw[2]); hi[1] = raw[2] >> 16; hi[2] = static_cast<int16_t>(raw[3]); hi[3] = raw[3] >> 16;
+        *reinterpret_cast<v4i*>(dst + ((q0 * nchunks + chunk) << 2)) = lo;
+        *reinterpret_cast<v4i*>(dst + (((q0 + 1) * nchunks + chunk) << 2)) = hi;
+    }
+    __syncthreads();
+
+    for (; row0 < rows; row0 += nwaves * G) {
+        const int row = row0 + grp;
+        const bool live = row < rows;
         const int64_t base = static_cast<int64_t>(row) * cols;
         v4i xv[NCH];
         int sx = 0, sq = 0;
 #pragma unroll
         for (int i = 0; i < NCH; ++i) {
-            const int col0 = (lane + 64 * i) * 16;
-            xv[i] = v4i{0, 0, 0, 0};
-            if (valid[i]) {
-                xv[i] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(x + base + col0));
-                if (FUSE_ADD) {
-                    const v4i o = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(x2 + base + col0));
+            xv[i] = nx[i];
+            if (FUSE_ADD) {
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) xv[i][j] = static_cast<int>(sat_add_i8x4(xv[i][j], o[j]));
-                    if (sum_out) __builtin_nontemporal_store(xv[i], reinterpret_cast<v4i*>(sum_out + base + col0));
-                }
+                for (int j = 0; j < 4; ++j) xv[i][j] = static_cast<int>(sat_add_i8x4(xv[i][j], nx2[i][j]));
+                if (sum_out && live && valid[i])
+                    __builtin_nontemporal_store(xv[i], reinterpret_cast<v4i*>(sum_out + base + chunk_of[i] * 16));
             }
+        }
+        if (row0 + nwaves * G < rows) fetch(row + nwaves * G);
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 sx = __builtin_amdgcn_sdot4(xv[i][j], 0x01010101, sx, false);
                 sq = __builtin_amdgcn_sdot4(xv[i][j], xv[i][j], sq, false);
             }
         }
-        sx = group_allreduce<64>(sx, OpAdd());
-        sq = group_allreduce<64>(sq, OpAdd());
+        sx = group_allreduce<L>(sx, OpAdd());
+        sq = group_allreduce<L>(sq, OpAdd());
         const RowStats st = row_stats(sx, sq, cols, log2c, eps_q0);
 
 #pragma unroll
         for (int i = 0; i < NCH; ++i) {
-            if (!valid[i]) continue;
-            const int col0 = (lane + 64 * i) * 16;
             v4i o;
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
+                const int at = (w * nchunks + chunk_of[i]) << 2;
+                const v4i g4 = *reinterpret_cast<const v4i*>(lg + at);
+                const v4i b4 = *reinterpret_cast<const v4i*>(lb + at);
                 int y4[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const int e = w * 4 + j;  // element within the chunk
-                    const int gw = g[i][e >> 3][(e & 7) >> 1];
-                    const int bw = bt[i][e >> 3][(e & 7) >> 1];
-                    const int gam = (e & 1) ? (gw >> 16) : static_cast<int>(static_cast<int16_t>(gw));
-                    const int bet = (e & 1) ? (bw >> 16) : static_cast<int>(static_cast<int16_t>(bw));
                     const int vd = sext8(xv[i][w], j) - st.mu;
-                    const int fs = clamp_i(round_shift<MODE>(st.inv * gam, gamma_shift), -32768, 32767);
-                    const int acc = vd * fs + bet;
-                    y4[j] = clamp_i(round_shift<MODE>(acc, final_shift), -128, 127);
+                    const int fs = clamp_i(ln_round<BIT>(__mul24(st.inv, g4[j]), rg), -32768, 32767);
+                    y4[j] = clamp_i(ln_round<BIT>(__mul24(vd, fs) + b4[j], ro), -128, 127);
                 }
                 o[w] = static_cast<int>(pack4_bytes(y4[0], y4[1], y4[2], y4[3]));
             }
-            __builtin_nontemporal_store(o, reinterpret_cast<v4i*>(out + base + col0));
+            if (live && valid[i]) __builtin_nontemporal_store(o, reinterpret_cast<v4i*>(out + base + chunk_of[i] * 16));
         }
     }
 }
@@ -276,19 +365,20 @@ __global__ __launch_bounds__(256) void layernorm_generic_kernel(const int8_t* __
     }
 }
 
-template <int NCH, bool FUSE>
-static void launch_ln_wave(int mode, int grid, hipStream_t stream, const int8_t* x, const int8_t* x2, const int16_t* gamma,
-                           const int16_t* beta, int8_t* sum_out, int8_t* out, int rows, int cols, int log2c, int eps_q0,
-                           int gamma_shift, int final_shift) {
-#define A4G_LN_CASE(M)                                                                                                  \
-    case M:                                                                                                             \
-        layernorm_wave_kernel<NCH, M, FUSE><<<grid, 256, 0, stream>>>(x, x2, gamma, beta, sum_out, out, rows, cols, log2c, \
-                                                                        eps_q0, gamma_shift, final_shift);               \
+template <int L, int NCH>
+static void launch_ln_rows(int bit_kind, bool fuse, int grid, size_t lds, hipStream_t stream, const int8_t* x,
+                           const int8_t* x2, const int16_t* gamma, const int16_t* beta, int8_t* sum_out, int8_t* out,
+                           int rows, int cols, int log2c, int eps_q0, const LnRound& rg, const LnRound& ro) {
+#define A4G_LN_CASE(B)                                                                                                   \
+    case B:                                                                                                              \
+        if (fuse)                                                                                                        \
+            layernorm_rows_kernel<L, NCH, B, true><<<grid, 256, lds, stream>>>(x, x2, gamma, beta, sum_out, out, rows,   \
+                                                                               cols, log2c, eps_q0, rg, ro);             \
+        else                                                                                                             \
+            layernorm_rows_kernel<L, NCH, B, false><<<grid, 256, lds, stream>>>(x, nullptr, gamma, beta, nullptr, out,   \
+                                                                                rows, cols, log2c, eps_q0, rg, ro);      \
         break;
-    switch (mode) {
-        A4G_LN_CASE(0) A4G_LN_CASE(1) A4G_LN_CASE(2) A4G_LN_CASE(3) A4G_LN_CASE(4) A4G_LN_CASE(5) A4G_LN_CASE(6)
-        A4G_LN_CASE(7)
-    }
+    switch (bit_kind) { A4G_LN_CASE(0) A4G_LN_CASE(1) A4G_LN_CASE(2) A4G_LN_CASE(3) A4G_LN_CASE(4) }
 #undef A4G_LN_CASE
 }
 
@@ -320,23 +410,24 @@ static int layernorm_dispatch(const int8_t* a, const int8_t* b, int add_shift, i
     const bool fast = cols % 16 == 0 && cols <= 4096 && aligned16(a) && aligned16(out) && (!fuse || aligned16(b)) &&
                       (!sum_out || aligned16(sum_out)) && aligned16(gamma) && aligned16(beta) && (!fuse || add_shift == 0);
     if (fast) {
-        const int nch = static_cast<int>((cols / 16 + 63) / 64);
-        const int grid = grid_for(rows, 4, 256 * 8);
-#define A4G_LN_NCH(N)                                                                                                        \
-    if (fuse)                                                                                                                \
-        launch_ln_wave<N, true>(mode, grid, stream, a, b, gamma, beta, sum_out, out, (int)rows, (int)cols, log2c, eps_q0,    \
-                                gamma_shift, final_shift);                                                                   \
-    else                                                                                                                     \
-        launch_ln_wave<N, false>(mode, grid, stream, a, nullptr, gamma, beta, nullptr, out, (int)rows, (int)cols, log2c,     \
-                                 eps_q0, gamma_shift, final_shift);
-        if (nch <= 1) {
-            A4G_LN_NCH(1)
-        } else if (nch <= 2) {
-            A4G_LN_NCH(2)
-        } else {
-            A4G_LN_NCH(4)
-        }
-#undef A4G_LN_NCH
+        const int nchunks = static_cast<int>(cols / 16);
+        int bit_kind = 0, unused = 0;
+        const LnRound rg = make_ln_round(mode, gamma_shift, &bit_kind);
+        const LnRound ro = make_ln_round(mode, final_shift, &unused);
+        const size_t lds = static_cast<size_t>(cols) * 8;
+        // The kernel is bound by its integer arithmetic (about 16 VALU instructions per element), not by
+        // HBM: a grid of 8 blocks per CU keeps every SIMD supplied with ready waves.
+        const int max_grid = 256 * 8;
+#define A4G_LN_GO(L, NCH)                                                                                                \
+    launch_ln_rows<L, NCH>(bit_kind, fuse, grid_for(rows, 4 * (64 / L), max_grid), lds, stream, a, b, gamma, beta, sum_out, \
+                           out, (int)rows, (int)cols, log2c, eps_q0, rg, ro)
+        if (nchunks <= 16) A4G_LN_GO(8, 2);
+        else if (nchunks <= 32) A4G_LN_GO(16, 2);
+        else if (nchunks <= 48) A4G_LN_GO(16, 3);
+        else if (nchunks <= 64) A4G_LN_GO(32, 2);
+        else if (nchunks <= 128) A4G_LN_GO(64, 2);
+        else A4G_LN_GO(64, 4);
+#undef A4G_LN_GO
     } else {
         const int grid = grid_for(rows, 1, 256 * 8);
         layernorm_generic_kernel<<<grid, 256, 0, stream>>>(a, b, add_shift, add_mode, gamma, beta, sum_out, out, (int)rows,

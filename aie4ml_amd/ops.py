@@ -189,7 +189,7 @@ def layernorm(x: torch.Tensor, gamma_q7: torch.Tensor, beta_q15: torch.Tensor, o
 
 def add_layernorm(a: torch.Tensor, b: torch.Tensor, gamma_q7: torch.Tensor, beta_q15: torch.Tensor, out_shift: int,
                   rounding='floor', eps_q0: int = 1, gamma_shift: int = 7, add_shift: int = 0, add_rounding='floor',
-                  return_sum: bool = False):
+                  return_sum: bool = False, out: Optional[torch.Tensor] = None, sum_out: Optional[torch.Tensor] = None):
     """Residual add fused in front of the LayerNorm (same result as add() then layernorm())."""
     if a.shape != b.shape or a.dtype != torch.int8 or b.dtype != torch.int8:
         raise ValueError('add_layernorm requires two int8 tensors of one shape')
@@ -200,8 +200,15 @@ def add_layernorm(a: torch.Tensor, b: torch.Tensor, gamma_q7: torch.Tensor, beta
     bt = _dev(beta_q15, 'beta').to(torch.int16).contiguous()
     if g.numel() != cols or bt.numel() != cols:
         raise ValueError(f'LayerNorm parameter length does not match full_inner={cols}.')
-    out = torch.empty_like(a2).reshape(a.shape)
-    s = torch.empty_like(a2).reshape(a.shape) if return_sum else None
+    if out is None:
+        out = torch.empty_like(a2).reshape(a.shape)
+    elif out.shape != a.shape or out.dtype != torch.int8 or not out.is_contiguous():
+        raise ValueError('add_layernorm: out must be a contiguous int8 tensor of the input shape')
+    s = None
+    if return_sum:
+        s = sum_out if sum_out is not None else torch.empty_like(a2).reshape(a.shape)
+        if s.shape != a.shape or s.dtype != torch.int8 or not s.is_contiguous():
+            raise ValueError('add_layernorm: sum_out must be a contiguous int8 tensor of the input shape')
     check(_lib.load().a4g_add_layernorm_i8(_ptr(a2), _ptr(b2), int(add_shift), _mode(add_rounding), _ptr(g), _ptr(bt),
                                            _ptr(s), _ptr(out), int(a2.shape[0]), cols, int(eps_q0), int(gamma_shift),
                                            int(out_shift), _mode(rounding), _stream()))
