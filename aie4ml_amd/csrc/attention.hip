@@ -1,0 +1,293 @@
+// Fused attention core: O = srs( softmax_int( srs(Q K^T) ) V ) for every (batch, head), in ONE launch.
+// It performs exactly the integer operations of the three reference kernels it replaces, in the same
+// order — MatMul (matmul.cpp:80-115) with the K operand transposed, Softmax in either form
+// (softmax.cpp:19-127 / 252-384), MatMul with a uint8 left operand — so the result is bit-identical to
+// running them one after another; the int8 logits and uint8 probabilities simply never leave the CU.
+//
+// A wave owns 32 query rows. With the MFMA operands swapped (lanes = rows), lane (m, half) ends each
+// 32x32 logit tile with 16 values of row m: columns 32t + 8g + 4*half + i. They are requantised and packed
+// to four dwords per tile and stay in registers: the row maximum and the score sum are in-lane reductions
+// plus one exchange between the two lanes of a row. The probabilities are then fed to the second MFMA
+// straight from those registers: integer dot products do not care about the order of k, so step t uses the
+// k-set a lane already holds, and V^T is laid out in LDS in the matching order.
+#include "common.hpp"
+#include "softmax_common.hpp"
+
+namespace a4g {
+
+struct FastRound {  // (acc + c0 + cx * bit) >> s, bit = one bit of acc at `pos` (width w = 0 disables it)
+    int s, c0, pos, w, cx;
+};
+
+static FastRound make_fast_round(int mode, int s) {
+    FastRound r{s, 0, 31, 0, 0};
+    if (s <= 0) return r;
+    const int h = 1 << (s - 1);
+    switch (mode) {
+    case A4G_RND_FLOOR: break;
+    case A4G_RND_CEIL: r.c0 = (1 << s) - 1; break;
+    case A4G_RND_POSITIVE_INF: r.c0 = h; break;
+    case A4G_RND_NEGATIVE_INF: r.c0 = h - 1; break;
+    case A4G_RND_SYMMETRIC_INF: r.c0 = h; r.cx = -1; r.w = 1; break;
+    case A4G_RND_SYMMETRIC_ZERO: r.c0 = h - 1; r.cx = 1; r.w = 1; break;
+    case A4G_RND_CONV_EVEN: r.c0 = h - 1; r.cx = 1; r.w = 1; r.pos = s; break;
+    default: r.c0 = h; r.cx = -1; r.w = 1; r.pos = s; break;  // conv_odd
+    }
+    return r;
+}
+
+// |acc| stays far below 2^30 in this kernel (at most 512 products of 8-bit values), so nothing overflows.
+__device__ __forceinline__ int fast_round(int acc, const FastRound& r) {
+    const int bit = static_cast<int>(__builtin_amdgcn_ubfe(static_cast<unsigned>(acc), r.pos, r.w));
+    return (acc + r.c0 + __mul24(bit, r.cx)) >> r.s;
+}
+
+struct AttnArgs {
+    const int8_t* Q;
+    const int8_t* K;
+    const int8_t* V;
+    int8_t* O;
+    int64_t q_sb, q_sh, q_ss;  // byte strides: batch, head, row (the feature axis is contiguous)
+    int64_t k_sb, k_sh, k_ss;
+    int64_t v_sb, v_sh, v_ss;
+    int64_t o_sb, o_sh, o_ss;
+    int heads, sq;
+    FastRound lr, orr;  // logits and output requantisation
+    SoftmaxParams sm;
+    int noclamp;
+};
+
+// 4x4 byte transpose: in a[i] byte j  ->  out c[j] byte i.
+__device__ __forceinline__ void transpose4x4(const unsigned a[4], unsigned c[4]) {
+    const unsigned lo01 = __builtin_amdgcn_perm(a[1], a[0], 0x05010400u);
+    const unsigned hi01 = __builtin_amdgcn_perm(a[1], a[0], 0x07030602u);
+    const unsigned lo23 = __builtin_amdgcn_perm(a[3], a[2], 0x05010400u);
+    const unsigned hi23 = __builtin_amdgcn_perm(a[3], a[2], 0x07030602u);
+    c[0] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);
+    c[1] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
+    c[2] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);
+    c[3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
+}
+
+// NT = key/value rows / 32, DT = head dimension / 32. 256 threads = 4 waves = 128 query rows of one head.
+template <int NT, int DT>
+__global__ __launch_bounds__(256, 2) void attention_kernel(AttnArgs a) {
+    constexpr int SK = NT * 32, D = DT * 32, PITCH = SK + 16;
+    extern __shared__ __attribute__((aligned(16))) int8_t attn_smem[];
+    int8_t* vt = attn_smem;                                        // V^T, k-permuted: [D][PITCH]
+    int* table = reinterpret_cast<int*>(attn_smem + D * PITCH);    // score of a gap d in [0,255]
+    int* colsum = table + 256;                                     // sum_k V[k][n]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int m = lane & 31, half = lane >> 5;
+    const int nblk = (a.sq + 127) >> 7;
+    const int bh = blockIdx.x / nblk, rb = blockIdx.x % nblk;
+    const int b = bh / a.heads, h = bh % a.heads;
+    const int8_t* Qp = a.Q + b * a.q_sb + h * a.q_sh;
+    const int8_t* Kp = a.K + b * a.k_sb + h * a.k_sh;
+    const int8_t* Vp = a.V + b * a.v_sb + h * a.v_sh;
+    int8_t* Op = a.O + b * a.o_sb + h * a.o_sh;
+    const int row = rb * 128 + wave * 32 + m;
+    const bool row_ok = row < a.sq;
+    const int rowc = row_ok ? row : a.sq - 1;
+
+    // operand fragments straight from global memory: lane (m, half) holds bytes [16*half, 16*half+16) of
+    // each 32-wide k step of its row
+    v4i qf[DT], kf[2][DT];
+#pragma unroll
+    for (int ks = 0; ks < DT; ++ks) {
+        qf[ks] = *reinterpret_cast<const v4i*>(Qp + rowc * a.q_ss + ks * 32 + half * 16);
+        kf[0][ks] = *reinterpret_cast<const v4i*>(Kp + m * a.k_ss + ks * 32 + half * 16);
+    }
+
+    table[tid] = table_entry(a.sm, tid);
+    if (tid < D) colsum[tid] = 0;
+    __syncthreads();
+
+    // V -> LDS, transposed in 4x4 byte blocks. Within each group of 32 k, position 16*half + 4*g + i holds
+    // k = 8*g + 4*half + i: the order in which a lane's probability registers run.
+    {
+        constexpr int NB = (SK / 4) * (D / 4);
+        const int n0 = (tid % (D / 4)) * 4;  // 256 % (D/4) == 0: a thread keeps its four columns
+        int part[4] = {0, 0, 0, 0};
+        for (int blk = tid; blk < NB; blk += 256) {
+            const int k0 = (blk / (D / 4)) * 4;
+            unsigned av[4], cv[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) av[i] = *reinterpret_cast<const unsigned*>(Vp + (k0 + i) * a.v_ss + n0);
+            transpose4x4(av, cv);
+            const int kk = k0 & 31;
+            const int pos = (k0 & ~31) + ((kk >> 2) & 1) * 16 + (kk >> 3) * 4;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                *reinterpret_cast<unsigned*>(vt + (n0 + j) * PITCH + pos) = cv[j];
+                part[j] = __builtin_amdgcn_sdot4(static_cast<int>(cv[j]), 0x01010101, part[j], false);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) atomicAdd(&colsum[n0 + j], part[j]);
+    }
+
+    // ---- pass A: logits = srs(Q K^T), packed int8 in registers; running row maximum -----------------
+    unsigned lg[NT][4];
+    int mx = -128;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        if (t + 1 < NT) {
+#pragma unroll
+            for (int ks = 0; ks < DT; ++ks)
+                kf[(t + 1) & 1][ks] =
+                    *reinterpret_cast<const v4i*>(Kp + ((t + 1) * 32 + m) * a.k_ss + ks * 32 + half * 16);
+        }
+        v16i acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int ks = 0; ks < DT; ++ks)
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[t & 1][ks], qf[ks], acc, 0, 0, 0);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            int y[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) y[i] = clamp_i(fast_round(acc[4 * g + i], a.lr), -128, 127);
+            mx = max(max(mx, y[0]), max(y[1], max(y[2], y[3])));
+            lg[t][g] = pack4_bytes(y[0], y[1], y[2], y[3]);
+        }
+    }
+    mx = max(mx, lane_xor<32>(mx));  // lanes m and m+32 share a row
+
+    __syncthreads();  // V^T, column sums and the score table are complete
+
+    // ---- pass B: scores by table lookup on the gap to the maximum; row sum ----------------------------
+    const unsigned mrep = static_cast<unsigned>((mx ^ 0x80) & 0xFF) * 0x01010101u;
+    unsigned ep[NT][8];  // two 16-bit scores per register
+    int sum = 0;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const unsigned d4 = mrep - (lg[t][g] ^ 0x80808080u);  // per byte, never borrows
+            const int e0 = table[d4 & 0xFF], e1 = table[(d4 >> 8) & 0xFF];
+            const int e2 = table[(d4 >> 16) & 0xFF], e3 = table[d4 >> 24];
+            sum += (e0 + e1) + (e2 + e3);
+            ep[t][2 * g] = pack2_halves(e0, e1);
+            ep[t][2 * g + 1] = pack2_halves(e2, e3);
+        }
+    }
+    sum += lane_xor<32>(sum);
+    const int inv = row_inverse(a.sm, sum);
+
+    // ---- pass C: probabilities (uint8, read as int8 after ^0x80) feed the second MFMA from registers ----
+    v16i oacc[DT];
+#pragma unroll
+    for (int u = 0; u < DT; ++u) oacc[u] = v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+        v4i pf;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            int p[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const unsigned pair = ep[t][2 * g + (i >> 1)];
+                const int e = (i & 1) ? static_cast<int>(pair >> 16) : static_cast<int>(pair & 0xFFFFu);
+                p[i] = __mul24(e, inv) >> a.sm.out_shift;
+                if (!a.noclamp) p[i] = clamp_i(p[i], 0, 255);
+            }
+            pf[g] = static_cast<int>(pack4_bytes(p[0], p[1], p[2], p[3]) ^ 0x80808080u);
+        }
+#pragma unroll
+        for (int u = 0; u < DT; ++u) {
+            const v4i vf = *reinterpret_cast<const v4i*>(vt + (32 * u + m) * PITCH + t * 32 + half * 16);
+            oacc[u] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf, pf, oacc[u], 0, 0, 0);
+        }
+    }
+
+    // ---- epilogue: + 128 * colsum (undoes the ^0x80), requantise, 16 contiguous bytes per lane ---------
+#pragma unroll
+    for (int u = 0; u < DT; ++u) {
+        unsigned ow[4];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const v4i cs = *reinterpret_cast<const v4i*>(colsum + 32 * u + 8 * g + 4 * half);
+            int y[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) y[i] = clamp_i(fast_round(oacc[u][4 * g + i] + 128 * cs[i], a.orr), -128, 127);
+            ow[g] = pack4_bytes(y[0], y[1], y[2], y[3]);
+        }
+        // lane m holds dwords 0,2,4,6 of the row's 32 bytes, lane m+32 dwords 1,3,5,7: two half-wave swaps
+        // give lane m bytes 0-15 and lane m+32 bytes 16-31
+        const auto s02 = __builtin_amdgcn_permlane32_swap(ow[0], ow[2], false, false);
+        const auto s13 = __builtin_amdgcn_permlane32_swap(ow[1], ow[3], false, false);
+        const v4i o = {static_cast<int>(s02[0]), static_cast<int>(s02[1]), static_cast<int>(s13[0]),
+                       static_cast<int>(s13[1])};
+        if (row_ok) *reinterpret_cast<v4i*>(Op + row * a.o_ss + 32 * u + 16 * half) = o;
+    }
+}
+
+template <int DT>
+static int launch_attention(int nt, int grid, hipStream_t stream, const AttnArgs& a) {
+    const size_t lds = static_cast<size_t>(DT * 32) * (nt * 32 + 16) + 256 * 4 + DT * 32 * 4;
+    switch (nt) {
+    case 1: attention_kernel<1, DT><<<grid, 256, lds, stream>>>(a); break;
+    case 2: attention_kernel<2, DT><<<grid, 256, lds, stream>>>(a); break;
+    case 4: attention_kernel<4, DT><<<grid, 256, lds, stream>>>(a); break;
+    case 8: attention_kernel<8, DT><<<grid, 256, lds, stream>>>(a); break;
+    case 16: attention_kernel<16, DT><<<grid, 256, lds, stream>>>(a); break;
+    default: return 1;
+    }
+    return 0;
+}
+
+}  // namespace a4g
+
+using namespace a4g;
+
+extern "C" int a4g_attention_i8(const int8_t* Q, const int8_t* K, const int8_t* V, int8_t* O, int64_t batch, int64_t heads,
+                                int64_t sq, int64_t sk, int64_t d, const int64_t* strides, int logit_shift,
+                                int logit_round_mode, int softmax_kind, int exp_kq, int hccs_B, int hccs_S, int hccs_Dmax,
+                                int inv_shift, int use_clb, int out_shift, int out_round_mode, a4g_stream_t stream_) {
+    const char* who = "a4g_attention_i8";
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    A4G_REQUIRE(batch >= 0 && heads >= 1 && sq >= 1 && sk >= 1 && d >= 1, A4G_ERR_INVALID_ARGUMENT,
+                "%s: bad shape batch=%lld heads=%lld sq=%lld sk=%lld d=%lld", who, (long long)batch, (long long)heads,
+                (long long)sq, (long long)sk, (long long)d);
+    A4G_REQUIRE(valid_round(logit_round_mode) && valid_round(out_round_mode), A4G_ERR_INVALID_ARGUMENT,
+                "%s: unknown rounding mode", who);
+    A4G_REQUIRE(logit_shift >= 0 && logit_shift <= 24 && out_shift >= 0 && out_shift <= 24, A4G_ERR_INVALID_ARGUMENT,
+                "%s: accumulator output shift must be in [0,24], got %d and %d", who, logit_shift, out_shift);
+    A4G_REQUIRE(softmax_kind == 0 || softmax_kind == 1, A4G_ERR_INVALID_ARGUMENT, "%s: softmax_kind must be 0 (exp) or 1 (hccs)",
+                who);
+    AttnArgs a{};
+    bool noclamp = false;
+    if (softmax_kind == 0) {
+        if (int rc = make_exp_params(who, exp_kq, inv_shift, A4G_U8, &a.sm, &noclamp)) return rc;
+    } else {
+        if (int rc = make_hccs_params(who, sk, hccs_B, hccs_S, hccs_Dmax, inv_shift, use_clb, A4G_U8, &a.sm, &noclamp))
+            return rc;
+    }
+    const bool pow2_tiles = sk % 32 == 0 && sk <= 512 && ((sk / 32) & (sk / 32 - 1)) == 0;
+    A4G_REQUIRE(d == 64 && pow2_tiles, A4G_ERR_UNSUPPORTED,
+                "%s: fused path covers head_dim 64 and 32/64/128/256/512 keys, got d=%lld sk=%lld", who, (long long)d,
+                (long long)sk);
+    A4G_REQUIRE(batch * heads * ((sq + 127) / 128) <= INT32_MAX && sq <= (1 << 24), A4G_ERR_UNSUPPORTED, "%s: too many rows", who);
+    if (batch == 0) return A4G_OK;
+    A4G_REQUIRE(Q && K && V && O && strides, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+    bool ok = aligned16(Q) && aligned16(K) && aligned16(V) && aligned16(O);
+    for (int i = 0; i < 12; ++i) ok = ok && strides[i] % 16 == 0 && strides[i] >= 0;
+    A4G_REQUIRE(ok, A4G_ERR_UNSUPPORTED, "%s: pointers and strides must be multiples of 16 bytes", who);
+    A4G_REQUIRE(strides[2] >= d && strides[5] >= d && strides[8] >= d && strides[11] >= d, A4G_ERR_INVALID_ARGUMENT,
+                "%s: row stride smaller than the head dimension", who);
+    a.Q = Q; a.K = K; a.V = V; a.O = O;
+    a.q_sb = strides[0]; a.q_sh = strides[1]; a.q_ss = strides[2];
+    a.k_sb = strides[3]; a.k_sh = strides[4]; a.k_ss = strides[5];
+    a.v_sb = strides[6]; a.v_sh = strides[7]; a.v_ss = strides[8];
+    a.o_sb = strides[9]; a.o_sh = strides[10]; a.o_ss = strides[11];
+    a.heads = static_cast<int>(heads);
+    a.sq = static_cast<int>(sq);
+    a.lr = make_fast_round(logit_round_mode, logit_shift);
+    a.orr = make_fast_round(out_round_mode, out_shift);
+    a.noclamp = noclamp;
+    const int grid = static_cast<int>(batch * heads * ((sq + 127) / 128));
+    if (launch_attention<2>(static_cast<int>(sk / 32), grid, stream, a))
+        return fail(A4G_ERR_UNSUPPORTED, "%s: no kernel for sk=%lld", who, (long long)sk);
+    return check_hip(hipGetLastError(), who);
+}

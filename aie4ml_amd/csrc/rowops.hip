@@ -5,6 +5,7 @@
 // lane (fully coalesced: 64 lanes x 16 B = 1 KiB per wave-load), keep the row in registers between
 // the reduction and the normalisation, and reduce across lanes with DPP / ds_swizzle butterflies.
 #include "common.hpp"
+#include "softmax_common.hpp"
 
 namespace a4g {
 
@@ -462,51 +463,6 @@ namespace a4g {
 // Both forms score an element from its gap d = max - x in [0,255] only, so the score is a 256-entry
 // table built once per block in LDS: exp -> exp_score16(d, KQ); HCCS -> B - S*min(d, Dmax).
 
-__device__ __forceinline__ int sat16(int v) { return clamp_i(v, -32768, 32767); }
-
-// softmax.cpp:252-273 under rounding_mode::floor.
-__device__ __forceinline__ int exp_score16(int d, int kq) {
-    const int z = sat16(d * kq);
-    const int zint = z >> 8;
-    const int zfrac = z & 255;
-    const int t = sat16((zfrac * 2811) >> 8);
-    const int inner = sat16(t - 11004);
-    const int t2 = sat16((inner * zfrac) >> 8);
-    int e = static_cast<int16_t>(t2 + 16384);
-    e = e >> (zint & 15);
-    return zint >= 16 ? 0 : e;
-}
-
-struct SoftmaxParams {
-    int is_hccs;
-    int exp_kq;
-    int B, S, Dmax;
-    int numer;      // 255 << inv_shift, or 32767
-    int inv_shift;  // for the use_clb branch
-    int use_clb;
-    int out_shift;
-    int out_i16;
-};
-
-__device__ __forceinline__ int table_entry(const SoftmaxParams& p, int d) {
-    if (p.is_hccs) return sat16(p.B - p.S * min(d, p.Dmax));
-    return exp_score16(d, p.exp_kq);
-}
-
-// softmax.cpp:62-79 (HCCS) / :108-127 (exact floor(NUMER/sum)); the int16 narrowing is the
-// broadcast<int16>(inv_q0) of softmax.cpp:79 and the (int16_t) cast of :375.
-__device__ __forceinline__ int row_inverse(const SoftmaxParams& p, int sum) {
-    const int s = sum > 0 ? sum : 1;
-    int inv;
-    if (p.use_clb) {
-        const int k = 31 - __builtin_clz(static_cast<unsigned>(s));
-        inv = p.out_i16 ? (32767 >> k) : (k <= p.inv_shift ? (255 << (p.inv_shift - k)) : 0);
-    } else {
-        inv = static_cast<int>(static_cast<unsigned>(p.numer) / static_cast<unsigned>(s));
-    }
-    return static_cast<int16_t>(inv);
-}
-
 // Byte-wise max of four packed int8 as a scalar.
 __device__ __forceinline__ int max_i8x4(unsigned w) {
     return max(max(sext8(w, 0), sext8(w, 1)), max(sext8(w, 2), sext8(w, 3)));
@@ -685,22 +641,10 @@ extern "C" int a4g_softmax_exp_i8(const int8_t* x, void* out, int64_t rows, int6
     const char* who = "a4g_softmax_exp_i8";
     A4G_REQUIRE(rows >= 0 && cols >= 1 && cols <= 65536 && rows <= INT32_MAX, A4G_ERR_INVALID_ARGUMENT,
                 "%s: bad shape rows=%lld cols=%lld", who, (long long)rows, (long long)cols);
-    A4G_REQUIRE(out_kind == A4G_U8 || out_kind == A4G_I16, A4G_ERR_INVALID_ARGUMENT,
-                "%s: requires uint8 or int16 output, got kind %d", who, out_kind);
-    A4G_REQUIRE(exp_kq >= 1 && exp_kq <= 128, A4G_ERR_INVALID_ARGUMENT, "%s: exp Softmax needs 1 <= EXP_KQ <= 128, got %d",
-                who, exp_kq);
-    A4G_REQUIRE(inv_shift >= 1 && inv_shift <= 21, A4G_ERR_INVALID_ARGUMENT, "%s: inv_shift %d outside [1,21]", who,
-                inv_shift);
     SoftmaxParams p{};
-    p.is_hccs = 0;
-    p.exp_kq = exp_kq;
-    p.out_i16 = out_kind == A4G_I16;
-    p.numer = p.out_i16 ? 32767 : (255 << inv_shift);
-    p.inv_shift = inv_shift;
-    p.use_clb = 0;
-    p.out_shift = p.out_i16 ? 0 : inv_shift;
-    // every score <= sum and inv = floor(numer/sum) fits int16, so score*inv >> shift <= 255
-    return softmax_dispatch(x, out, rows, cols, p, /*noclamp=*/true, static_cast<hipStream_t>(stream), who);
+    bool noclamp = false;
+    if (int rc = make_exp_params(who, exp_kq, inv_shift, out_kind, &p, &noclamp)) return rc;
+    return softmax_dispatch(x, out, rows, cols, p, noclamp, static_cast<hipStream_t>(stream), who);
 }
 
 extern "C" int a4g_softmax_hccs_i8(const int8_t* x, void* out, int64_t rows, int64_t cols, int B, int S, int Dmax,
@@ -708,31 +652,8 @@ extern "C" int a4g_softmax_hccs_i8(const int8_t* x, void* out, int64_t rows, int
     const char* who = "a4g_softmax_hccs_i8";
     A4G_REQUIRE(rows >= 0 && cols >= 1 && cols <= 65536 && rows <= INT32_MAX, A4G_ERR_INVALID_ARGUMENT,
                 "%s: bad shape rows=%lld cols=%lld", who, (long long)rows, (long long)cols);
-    A4G_REQUIRE(out_kind == A4G_U8 || out_kind == A4G_I16, A4G_ERR_INVALID_ARGUMENT,
-                "%s: requires uint8 or int16 output, got kind %d", who, out_kind);
-    A4G_REQUIRE(B >= 0 && B <= 32767, A4G_ERR_INVALID_ARGUMENT, "%s: HCCS Softmax parameter 'B' must be in [0, 32767]", who);
-    A4G_REQUIRE(S >= 0 && S <= 127, A4G_ERR_INVALID_ARGUMENT, "%s: HCCS Softmax parameter 'S' must be in [0, 127]", who);
-    A4G_REQUIRE(Dmax >= 0 && Dmax <= 127, A4G_ERR_INVALID_ARGUMENT, "%s: HCCS Softmax parameter 'Dmax' must be in [0, 127]",
-                who);
-    A4G_REQUIRE(B - S * Dmax >= 0, A4G_ERR_INVALID_ARGUMENT, "%s: HCCS Softmax requires B - S*Dmax >= 0, got %d", who,
-                B - S * Dmax);
-    A4G_REQUIRE(static_cast<int64_t>(B - S * Dmax) * cols >= 256, A4G_ERR_INVALID_ARGUMENT,
-                "%s: HCCS Softmax requires cols * (B - S*Dmax) >= 256 for reciprocal range, got %lld", who,
-                (long long)(static_cast<int64_t>(B - S * Dmax) * cols));
-    A4G_REQUIRE(static_cast<int64_t>(B) * cols <= 32767, A4G_ERR_INVALID_ARGUMENT,
-                "%s: HCCS Softmax requires cols * B <= 32767 so score sum fits int16 range", who);
-    A4G_REQUIRE(inv_shift >= 1 && inv_shift <= 23, A4G_ERR_INVALID_ARGUMENT, "%s: inv_shift %d outside [1,23]", who,
-                inv_shift);
     SoftmaxParams p{};
-    p.is_hccs = 1;
-    p.B = B;
-    p.S = S;
-    p.Dmax = Dmax;
-    p.out_i16 = out_kind == A4G_I16;
-    p.numer = p.out_i16 ? 32767 : (255 << inv_shift);
-    p.inv_shift = inv_shift;
-    p.use_clb = use_clb != 0;
-    p.out_shift = p.out_i16 ? 0 : inv_shift;
-    const bool noclamp = !p.use_clb && inv_shift <= 15;
+    bool noclamp = false;
+    if (int rc = make_hccs_params(who, cols, B, S, Dmax, inv_shift, use_clb, out_kind, &p, &noclamp)) return rc;
     return softmax_dispatch(x, out, rows, cols, p, noclamp, static_cast<hipStream_t>(stream), who);
 }

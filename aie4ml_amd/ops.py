@@ -275,3 +275,48 @@ def mlp(x: torch.Tensor, layers: Sequence[MlpLayerSpec], rounding='floor', out: 
                                  _ptr(out), out.stride(0) if out.shape[0] else last.params.N, int(x2.shape[0]),
                                  _mode(rounding), _stream()))
     return out
+
+
+def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, logit_shift: int, logit_rounding, softmax: dict,
+              out_shift: int, out_rounding, out: Optional[torch.Tensor] = None):
+    """Fused attention core: srs(softmax(srs(q k^T)) v) per (batch, head), one launch.
+
+    q: [..., sq, d], k and v: [..., sk, d] int8 with up to two leading axes (batch, head); any strides with a
+    contiguous last axis (head slices of a packed projection are fine). `softmax` is
+    {'kind': 'exp', 'exp_kq': .., 'inv_shift': 15} or {'kind': 'hccs', 'B': .., 'S': .., 'Dmax': .., 'inv_shift': 15,
+    'use_clb': False}. Bit-identical to matmul(trans_b) -> softmax_* -> matmul. Raises NotImplementedError for
+    shapes the fused kernel does not cover (head_dim != 64, sk not in 32/64/128/256/512, unaligned views).
+    """
+    for name, t in (('q', q), ('k', k), ('v', v)):
+        _dev(t, name)
+        if t.dtype != torch.int8 or t.dim() < 2 or t.dim() > 4 or t.stride(-1) != 1:
+            raise ValueError(f'attention: {name} must be int8 with 2..4 axes and a contiguous last axis')
+    if k.shape != v.shape or q.shape[:-2] != k.shape[:-2] or q.shape[-1] != k.shape[-1]:
+        raise ValueError(f'attention: incompatible shapes {tuple(q.shape)}, {tuple(k.shape)}, {tuple(v.shape)}')
+    lead = tuple(q.shape[:-2])
+    sq, d, sk = int(q.shape[-2]), int(q.shape[-1]), int(k.shape[-2])
+    if out is None:
+        out = torch.empty(lead + (sq, d), dtype=torch.int8, device=q.device)
+    elif out.shape != lead + (sq, d) or out.dtype != torch.int8 or out.stride(-1) != 1:
+        raise ValueError('attention: out must be int8 of shape [..., sq, d] with a contiguous last axis')
+
+    def strides3(t):  # (batch, head, row) byte strides with missing leading axes as 0
+        st = [0] * (4 - t.dim()) + [int(x) for x in t.stride()]
+        return st[0], st[1], st[2]
+
+    batch = int(lead[0]) if len(lead) >= 1 else 1
+    heads = int(lead[1]) if len(lead) == 2 else 1
+    if len(lead) == 1:  # [batch, s, d]: one head
+        flat = [(int(t.stride(0)), 0, int(t.stride(1))) for t in (q, k, v, out)]
+    else:
+        flat = [strides3(t) for t in (q, k, v, out)]
+    arr = (ctypes.c_int64 * 12)(*[x for trip in flat for x in trip])
+    kind = softmax.get('kind', 'exp')
+    if kind not in ('exp', 'hccs'):
+        raise ValueError(f"attention: unknown softmax kind {kind!r}")
+    check(_lib.load().a4g_attention_i8(_ptr(q), _ptr(k), _ptr(v), _ptr(out), batch, heads, sq, sk, d, arr, int(logit_shift),
+                                       _mode(logit_rounding), 0 if kind == 'exp' else 1, int(softmax.get('exp_kq', 1)),
+                                       int(softmax.get('B', 0)), int(softmax.get('S', 0)), int(softmax.get('Dmax', 0)),
+                                       int(softmax.get('inv_shift', 15)), int(bool(softmax.get('use_clb', False))),
+                                       int(out_shift), _mode(out_rounding), _stream()))
+    return out

@@ -7,7 +7,7 @@ saturate to int8, fused ReLU). One step = one pass of the operator over the whol
 inputs already resident in HBM. Prints ONE JSON line.
 
 Other workloads (--workload c1_mlp | c3_softmax_exp | c3_softmax_hccs | c3_qk | c3_pv |
-c4_add_layernorm | c4_layernorm | c4_add | c5_encoder) print the same line for that operator or graph;
+c3_attention_exp | c3_attention_hccs | c4_add_layernorm | c4_layernorm | c4_add | c5_encoder) print the same line for that operator or graph;
 --workload calib_copy runs a plain 256 MiB elementwise copy, the known-size kernel the HBM traffic
 counters are scaled against.
 """
@@ -255,6 +255,38 @@ def main():
         samples = Bt
         config = {'workload': f'{wl}: attention core batch 32 x 16 heads, seq 512, head_dim 64'}
         metric, unit = f'{wl}_gbs', 'GB/s'
+    elif wl in ('c3_attention_exp', 'c3_attention_hccs'):
+        Bt, H, S, D = 32, 16, 512, 64
+        q, k, v, prm = workloads.c3_attention(Bt, H, S, D)
+        dq, dk, dv = dev(q), dev(k), dev(v)
+        if wl.endswith('exp'):
+            sm = {'kind': 'exp', 'exp_kq': prm['exp_kq']}
+            sm_ref = lambda x_: oracle.softmax_exp(x_, prm['exp_kq'])  # noqa: E731
+        else:
+            sm = dict(prm['hccs'], kind='hccs')
+            sm_ref = lambda x_: oracle.softmax_hccs(x_, sm['B'], sm['S'], sm['Dmax'])  # noqa: E731
+        out = torch.empty_like(dq)
+        fn = lambda: ops.attention(dq, dk, dv, prm['logit_shift'], 'conv_even', sm, prm['pv_shift'], 'conv_even',  # noqa: E731
+                                   out=out)
+        fn()
+        torch.cuda.synchronize()
+
+        def ref_heads(qs, ks, vs):
+            lg = oracle.matmul(qs, ks, prm['logit_shift'], 'conv_even', trans_b=True)
+            return oracle.matmul(sm_ref(lg), vs, prm['pv_shift'], 'conv_even')
+
+        hb = (5, slice(2, 6))
+        bit_exact = bool(np.array_equal(out[hb].cpu().numpy(), ref_heads(q[hb], k[hb], v[hb])))
+        work, bound = 2 * 2.0 * Bt * H * S * S * D, 'mfma'
+        samples = Bt
+        config = {'workload': f'{wl}: fused attention core (QK^T shift {prm["logit_shift"]} -> softmax -> PV), batch 32 x 16 '
+                              'heads, seq 512, head_dim 64, one launch'}
+        cpu_fn = lambda: ref_heads(q[0, :4], k[0, :4], v[0, :4])  # noqa: E731
+        cpu_work = work * 4 / (Bt * H)
+        cpu_samples = 4 / H
+        cpu_desc = 'oracle MatMul -> Softmax -> MatMul on 4 of 512 (batch, head) slices'
+        metric, unit = 'int8_attention_tops', 'TOP/s'
+        kernel = 'attention_kernel'
     elif wl == 'c5_encoder':
         from oracle.graph import run_graph
 

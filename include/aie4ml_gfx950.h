@@ -177,6 +177,25 @@ typedef struct a4g_mlp_layer {
 A4G_API int a4g_mlp_i8(const a4g_mlp_layer* layers, int n_layers, const void* X, int x_kind, int64_t ldx, void* Y,
                int64_t ldy, int64_t batch, int round_mode, a4g_stream_t stream);
 
+/* ---- Fused attention core -----------------------------------------------------------------------------
+ * O[b,h] = srs( softmax( srs(Q[b,h] x K[b,h]^T, logit_shift) ) x V[b,h], out_shift ) in one launch: the
+ * chain MatMul (TRANSPOSE_B, matmul.cpp:70-115) -> Softmax (softmax.cpp:19-127 or 252-384) -> MatMul with
+ * a uint8 left operand that the reference builds from three kernels (the graph of
+ * scripts/check_onnx_bit_exact.py's attention models after fold_views.py / fold_scale.py). Same integer
+ * operations in the same order as a4g_matmul_i8 -> a4g_softmax_*_i8 -> a4g_matmul_i8; the int8 logits and
+ * the uint8 probabilities are never written to memory.
+ *   Q [batch][heads][sq][d], K and V [batch][heads][sk][d], O [batch][heads][sq][d], all int8, feature
+ *   axis contiguous. strides: 12 byte strides {batch, head, row} for Q, K, V, O in that order, so head
+ *   slices of a packed QKV projection and a concatenated output need no copies.
+ *   softmax_kind 0: accurate exp (exp_kq, inv_shift); 1: HCCS (hccs_B, hccs_S, hccs_Dmax, inv_shift,
+ *   use_clb), same parameter rules as the stand-alone entries; probabilities are uint8.
+ * Covered shapes: d == 64, sk in {32, 64, 128, 256, 512}, pointers and strides multiples of 16 bytes;
+ * anything else returns A4G_ERR_UNSUPPORTED and the caller runs the three operators separately. */
+A4G_API int a4g_attention_i8(const int8_t* Q, const int8_t* K, const int8_t* V, int8_t* O, int64_t batch, int64_t heads,
+                     int64_t sq, int64_t sk, int64_t d, const int64_t* strides, int logit_shift,
+                     int logit_round_mode, int softmax_kind, int exp_kq, int hccs_B, int hccs_S, int hccs_Dmax,
+                     int inv_shift, int use_clb, int out_shift, int out_round_mode, a4g_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

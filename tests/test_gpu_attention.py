@@ -1,0 +1,119 @@
+"""GPU parity of the fused attention core against the oracle's three separate operators
+(MatMul with transposed K -> integer Softmax -> MatMul with a uint8 left operand)."""
+
+import numpy as np
+import pytest
+import torch
+
+from aie4ml_amd import ops
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def reference(oracle, q, k, v, lshift, lmode, sm, oshift, omode):
+    logits = oracle.matmul(q, k, lshift, lmode, trans_b=True)
+    if sm['kind'] == 'exp':
+        p = oracle.softmax_exp(logits, sm['exp_kq'], sm.get('inv_shift', 15))
+    else:
+        p = oracle.softmax_hccs(logits, sm['B'], sm['S'], sm['Dmax'], sm.get('inv_shift', 15), sm.get('use_clb', False))
+    return oracle.matmul(p, v, oshift, omode)
+
+
+def qkv(seed, shape_q, shape_k, sigma=24.0):
+    r = np.random.default_rng(seed)
+    g = lambda s: np.clip(np.rint(r.normal(0, sigma, s)), -128, 127).astype(np.int8)  # noqa: E731
+    return g(shape_q), g(shape_k), g(shape_k)
+
+
+HCCS = {32: (255, 4, 60), 64: (255, 3, 80), 128: (255, 2, 126), 256: (127, 1, 126), 512: (60, 1, 59)}
+
+
+@pytest.mark.parametrize('sk', [32, 64, 128, 256, 512])
+@pytest.mark.parametrize('kind', ['exp', 'hccs'])
+def test_attention_matches_three_operators(oracle, sk, kind):
+    q, k, v = qkv(sk, (2, 3, sk, 64), (2, 3, sk, 64))
+    if kind == 'exp':
+        sm = {'kind': 'exp', 'exp_kq': 23}
+    else:
+        B, S, D = HCCS[sk]
+        sm = {'kind': 'hccs', 'B': B, 'S': S, 'Dmax': D}
+    got = ops.attention(dev(q), dev(k), dev(v), 6, 'conv_even', sm, 7, 'conv_even').cpu().numpy()
+    want = reference(oracle, q, k, v, 6, 'conv_even', sm, 7, 'conv_even')
+    np.testing.assert_array_equal(got, want)
+    assert len(np.unique(got)) > 16
+
+
+@pytest.mark.parametrize('mode', ['floor', 'ceil', 'positive_inf', 'negative_inf', 'symmetric_inf', 'symmetric_zero',
+                                  'conv_even', 'conv_odd'])
+def test_attention_rounding_modes(oracle, mode):
+    q, k, v = qkv(7, (4, 128, 64), (4, 128, 64), sigma=40.0)
+    sm = {'kind': 'exp', 'exp_kq': 40}
+    got = ops.attention(dev(q), dev(k), dev(v), 5, mode, sm, 6, mode).cpu().numpy()
+    np.testing.assert_array_equal(got, reference(oracle, q, k, v, 5, mode, sm, 6, mode))
+
+
+@pytest.mark.parametrize('sq', [1, 31, 100, 129, 300])
+def test_attention_ragged_query_count(oracle, sq):
+    q, k, v = qkv(sq, (2, 2, sq, 64), (2, 2, 128, 64))
+    sm = {'kind': 'hccs', 'B': 255, 'S': 2, 'Dmax': 126, 'use_clb': True}
+    got = ops.attention(dev(q), dev(k), dev(v), 6, 'symmetric_inf', sm, 8, 'floor').cpu().numpy()
+    np.testing.assert_array_equal(got, reference(oracle, q, k, v, 6, 'symmetric_inf', sm, 8, 'floor'))
+
+
+def test_attention_zero_shift_and_saturation(oracle):
+    # shift 0 on the logits saturates most of them; shift 0 on the output saturates everything
+    q, k, v = qkv(3, (2, 64, 64), (2, 64, 64), sigma=60.0)
+    sm = {'kind': 'exp', 'exp_kq': 128}
+    got = ops.attention(dev(q), dev(k), dev(v), 0, 'conv_even', sm, 0, 'conv_even').cpu().numpy()
+    np.testing.assert_array_equal(got, reference(oracle, q, k, v, 0, 'conv_even', sm, 0, 'conv_even'))
+    got = ops.attention(dev(q), dev(k), dev(v), 10, 'conv_even', sm, 3, 'conv_even').cpu().numpy()
+    np.testing.assert_array_equal(got, reference(oracle, q, k, v, 10, 'conv_even', sm, 3, 'conv_even'))
+
+
+def test_attention_on_head_slices_of_a_packed_projection(oracle):
+    """Q, K, V as strided views of one [batch, seq, 3*hidden] tensor, output written into the head's
+    columns of a [batch, seq, hidden] tensor: the layout of an encoder block, no copies."""
+    batch, seq, heads, hd = 3, 128, 4, 64
+    hidden = heads * hd
+    r = np.random.default_rng(12)
+    qkv_np = np.clip(np.rint(r.normal(0, 30, (batch, seq, 3 * hidden))), -128, 127).astype(np.int8)
+    t = dev(qkv_np)
+    out = torch.zeros((batch, seq, hidden), dtype=torch.int8, device='cuda')
+    sm = {'kind': 'hccs', 'B': 255, 'S': 4, 'Dmax': 62}
+    for h in range(heads):
+        qs = t[:, :, h * hd:(h + 1) * hd]
+        ks = t[:, :, hidden + h * hd:hidden + (h + 1) * hd]
+        vs = t[:, :, 2 * hidden + h * hd:2 * hidden + (h + 1) * hd]
+        ops.attention(qs, ks, vs, 7, 'conv_even', sm, 7, 'conv_even', out=out[:, :, h * hd:(h + 1) * hd])
+    got = out.cpu().numpy()
+    for h in range(heads):
+        sl = lambda o: np.ascontiguousarray(qkv_np[:, :, o + h * hd:o + (h + 1) * hd])  # noqa: E731
+        want = reference(oracle, sl(0), sl(hidden), sl(2 * hidden), 7, 'conv_even', sm, 7, 'conv_even')
+        np.testing.assert_array_equal(got[:, :, h * hd:(h + 1) * hd], want, err_msg=f'head {h}')
+    # all heads in one launch: [batch, heads, seq, hd] views with head stride hd
+    q4 = t[:, :, :hidden].view(batch, seq, heads, hd).permute(0, 2, 1, 3)
+    k4 = t[:, :, hidden:2 * hidden].view(batch, seq, heads, hd).permute(0, 2, 1, 3)
+    v4 = t[:, :, 2 * hidden:].view(batch, seq, heads, hd).permute(0, 2, 1, 3)
+    out2 = torch.zeros((batch, seq, hidden), dtype=torch.int8, device='cuda')
+    ops.attention(q4, k4, v4, 7, 'conv_even', sm, 7, 'conv_even', out=out2.view(batch, seq, heads, hd).permute(0, 2, 1, 3))
+    np.testing.assert_array_equal(out2.cpu().numpy(), got)
+
+
+def test_attention_uncovered_shapes_and_bad_parameters():
+    q = torch.zeros((2, 64, 32), dtype=torch.int8, device='cuda')
+    with pytest.raises(NotImplementedError, match='fused path covers head_dim 64'):
+        ops.attention(q, q, q, 6, 'floor', {'kind': 'exp', 'exp_kq': 23}, 7, 'floor')
+    q = torch.zeros((2, 96, 64), dtype=torch.int8, device='cuda')
+    with pytest.raises(NotImplementedError, match='fused path covers'):
+        ops.attention(q, q, q, 6, 'floor', {'kind': 'exp', 'exp_kq': 23}, 7, 'floor')
+    q = torch.zeros((2, 64, 64), dtype=torch.int8, device='cuda')
+    with pytest.raises(ValueError, match='1 <= EXP_KQ <= 128'):
+        ops.attention(q, q, q, 6, 'floor', {'kind': 'exp', 'exp_kq': 0}, 7, 'floor')
+    with pytest.raises(ValueError, match=r'cols \* B <= 32767'):
+        ops.attention(q, q, q, 6, 'floor', {'kind': 'hccs', 'B': 600, 'S': 1, 'Dmax': 5}, 7, 'floor')
+    with pytest.raises(ValueError, match='incompatible shapes'):
+        ops.attention(q, q[:, :32], q, 6, 'floor', {'kind': 'exp', 'exp_kq': 23}, 7, 'floor')
