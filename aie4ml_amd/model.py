@@ -129,18 +129,34 @@ class GPUModel:
 
         ctx = self.context
         graph, execution = ctx.ir.logical, ctx.ir.execution
-        plan = ctx.config.get('gpu_fusion_plan') or {'add_layernorm': {}, 'mlp_chains': []}
+        plan = ctx.config.get('gpu_fusion_plan') or {}
+        plan = {'add_layernorm': plan.get('add_layernorm', {}), 'mlp_chains': plan.get('mlp_chains', []),
+                'attention': plan.get('attention', [])}
         values: Dict[str, Any] = dict(inputs)
         fused_ln = {v['layer_norm'] for v in plan['add_layernorm'].values()}
         chain_head = {c[0]: c for c in plan['mlp_chains']}
         chain_rest = {n for c in plan['mlp_chains'] for n in c[1:]}
+        attn_at, attn_skip = {}, set()
+        order = {n.name: i for i, n in enumerate(graph.nodes)}
+        for grp in plan['attention']:
+            members = [tr[k] for tr in grp['heads'] for k in ('qk', 'softmax', 'pv')]
+            first = min((tr['qk'] for tr in grp['heads']), key=order.get)
+            attn_at[first] = grp
+            attn_skip.update(m for m in members if m != first)
+            if grp.get('concat'):
+                attn_skip.add(grp['concat'])
 
         for node in graph.nodes:
+            if node.name in attn_skip:
+                continue
             if node.is_placeholder:
                 self._run_view(node, values)
                 continue
             if node.name in chain_rest or node.name in fused_ln:
                 continue  # executed as part of a fused launch
+            if node.name in attn_at:
+                self._run_attention(attn_at[node.name], values, ops)
+                continue
             inst = execution.get(node.name)
             if inst is None:
                 raise RuntimeError(f'{node.name}: node was never resolved; run compile() first.')
@@ -184,6 +200,37 @@ class GPUModel:
             values[add_node.outputs[0].name], values[ln_node.outputs[0].name] = res
         else:
             values[ln_node.outputs[0].name] = res
+
+    def _run_attention(self, grp, values, ops) -> None:
+        """One fused launch for a matmul -> softmax -> matmul triple, or for all heads of a merged group
+        (operands become [batch, heads, seq, head_dim] strided views, the result lands in the concat output)."""
+        import torch
+
+        execution = self.context.ir.execution
+        tr0 = grp['heads'][0]
+        c1, c2, c3 = (execution.get(tr0[k]).config for k in ('qk', 'softmax', 'pv'))
+        if c2.approximation == 'exp':
+            sm = {'kind': 'exp', 'exp_kq': c2.exp_kq, 'inv_shift': c2.inv_shift}
+        else:
+            sm = {'kind': 'hccs', 'B': int(c2.hccs['B']), 'S': int(c2.hccs['S']), 'Dmax': int(c2.hccs['Dmax']),
+                  'inv_shift': c2.inv_shift, 'use_clb': c2.use_clb}
+        if grp.get('concat'):
+            nh, d = len(grp['heads']), int(self.context.ir.logical.tensors[tr0['q']].shape[-1])
+
+            def heads_view(t, base):  # [batch, seq, H*d] slice -> [batch, H, seq, d] view
+                t = t.narrow(-1, base, nh * d)
+                return t.unflatten(-1, (nh, d)).permute(0, 2, 1, 3)
+
+            q = heads_view(values[grp['q_src']], grp['q_base'])
+            k = heads_view(values[grp['k_src']], grp['k_base'])
+            v = heads_view(values[grp['v_src']], grp['v_base'])
+            out = torch.empty((q.shape[0], q.shape[2], nh * d), dtype=torch.int8, device=q.device)
+            ops.attention(q, k, v, c1.shift, c1.rounding_mode, sm, c3.shift, c3.rounding_mode,
+                          out=out.unflatten(-1, (nh, d)).permute(0, 2, 1, 3))
+            values[grp['out']] = out
+        else:
+            values[grp['out']] = ops.attention(values[tr0['q']], values[tr0['k']], values[tr0['v']], c1.shift, c1.rounding_mode,
+                                               sm, c3.shift, c3.rounding_mode)
 
     def _run_mlp(self, chain: List[str], values, ops) -> None:
         execution = self.context.ir.execution

@@ -13,7 +13,7 @@ from typing import Iterable
 
 import numpy as np
 
-from ..ir import TraitInstance, get_backend_context
+from ..ir import TraitInstance, get_backend_context, input_tensor_for_role
 from ..op_impls import get_family_resolver_registry
 from ..op_impls.base import OpImplVariant
 
@@ -299,7 +299,10 @@ class PlanGpuFusion(AIEPass):
     * add -> layer_norm: the residual add is computed inside the LayerNorm kernel (the sum is written out
       only if something else reads it).
     * a chain of dense nodes whose whole weight set fits LDS: one fused-MLP launch.
-    Both are exact: the fused kernels perform the same integer operations in the same order.
+    * matmul(Q, K^T) -> softmax -> matmul(P, V) whose logits and probabilities have no other reader: one
+      fused-attention launch; triples that read per-head slices of the same three tensors and feed one
+      concat are merged into a single launch over all heads that writes the concat's output directly.
+    All are exact: the fused kernels perform the same integer operations in the same order.
     """
 
     name = 'plan_gpu_fusion'
@@ -309,8 +312,9 @@ class PlanGpuFusion(AIEPass):
     def transform(self, model_or_ctx) -> bool:
         ctx = get_backend_context(model_or_ctx)
         graph, execution = ctx.ir.logical, ctx.ir.execution
-        plan = {'add_layernorm': {}, 'mlp_chains': []}
+        plan = {'add_layernorm': {}, 'mlp_chains': [], 'attention': []}
         outputs = set(graph.output_tensor_names)
+        plan['attention'] = self._plan_attention(graph, execution, outputs)
         for node in graph.nodes:
             if node.op_type != 'add' or execution.get(node.name) is None:
                 continue
@@ -344,6 +348,108 @@ class PlanGpuFusion(AIEPass):
         changed = ctx.config.get('gpu_fusion_plan') != plan
         ctx.config['gpu_fusion_plan'] = plan
         return changed
+
+    # ---- attention -------------------------------------------------------------------------------------
+    ATTN_HEAD_DIM = 64
+    ATTN_KEYS = (32, 64, 128, 256, 512)
+
+    def _plan_attention(self, graph, execution, outputs):
+        triples = []
+        for qk in graph.nodes:
+            if qk.op_type != 'matmul' or execution.get(qk.name) is None:
+                continue
+            c1 = execution.get(qk.name).config
+            logits = qk.outputs[0]
+            if not c1.flags.transpose_rhs or c1.flags.transpose_lhs or logits.name in outputs or len(logits.consumers) != 1:
+                continue
+            sm = logits.consumers[0]
+            if sm.op_type != 'softmax' or execution.get(sm.name) is None or sm.traits.get('io_view'):
+                continue
+            probs = sm.outputs[0]
+            if probs.name in outputs or len(probs.consumers) != 1:
+                continue
+            pv = probs.consumers[0]
+            if pv.op_type != 'matmul' or execution.get(pv.name) is None or input_tensor_for_role(pv, 'lhs') is not probs:
+                continue
+            c2, c3 = execution.get(sm.name).config, execution.get(pv.name).config
+            q, k = input_tensor_for_role(qk, 'lhs'), input_tensor_for_role(qk, 'rhs')
+            v = input_tensor_for_role(pv, 'rhs')
+            if k.is_parameter or v.is_parameter or c3.flags.transpose_rhs or c3.flags.transpose_lhs:
+                continue
+            if c1.precision['output'].format != 'int8' or c2.precision['output'].format != 'uint8' \
+                    or c3.precision['output'].format != 'int8' or c1.precision['lhs'].format != 'int8':
+                continue
+            if len(q.shape) != len(k.shape) or len(k.shape) != len(v.shape) or tuple(k.shape) != tuple(v.shape) \
+                    or tuple(q.shape[:-2]) != tuple(k.shape[:-2]) or len(q.shape) not in (2, 3, 4):
+                continue
+            if int(q.shape[-1]) != self.ATTN_HEAD_DIM or int(k.shape[-2]) not in self.ATTN_KEYS:
+                continue
+            triples.append({'qk': qk.name, 'softmax': sm.name, 'pv': pv.name, 'q': q.name, 'k': k.name, 'v': v.name,
+                            'out': pv.outputs[0].name})
+        groups, used = [], set()
+        by_name = {n.name: n for n in graph.nodes}
+        # merge per-head triples: operands are last-axis slices of three common tensors, results feed one concat
+        def slice_of(tname):
+            prod = None
+            for n in graph.nodes:
+                if n.is_placeholder and n.traits.get('slice_view') is not None:
+                    for it in n.traits['slice_view'].data['slices']:
+                        if it['output'] == tname:
+                            prod = (n, it)
+            if prod is None:
+                return None
+            n, it = prod
+            sv = n.traits['slice_view'].data
+            src = n.inputs[0]
+            ax = int(sv['axis'])
+            if ax not in (-1, len(src.shape) - 1):
+                return None
+            return sv['source'], int(it['start']), int(it['extent'])
+
+        cand = {}
+        for tr in triples:
+            out_t = by_name[tr['pv']].outputs[0]
+            if out_t.name in outputs or len(out_t.consumers) != 1:
+                continue
+            cat = out_t.consumers[0]
+            cv = cat.traits.get('concat_view')
+            if not cat.is_placeholder or cv is None:
+                continue
+            cat_out = cat.outputs[0]
+            if int(cv.data['axis']) not in (-1, len(cat_out.shape) - 1) or len(cat_out.shape) != 3:
+                continue
+            sq, sk_, sv_ = slice_of(tr['q']), slice_of(tr['k']), slice_of(tr['v'])
+            if not (sq and sk_ and sv_):
+                continue
+            o_start = next(int(it['start']) for it in cv.data['slices'] if it['input'] == out_t.name)
+            key = (sq[0], sk_[0], sv_[0], cat.name)
+            cand.setdefault(key, []).append((o_start, sq[1], sk_[1], sv_[1], tr))
+        for (qs, ks, vs, cat_name), items in cand.items():
+            items.sort(key=lambda x: x[0])
+            d = self.ATTN_HEAD_DIM
+            cat = by_name[cat_name]
+            regular = len(items) == len(cat.traits['concat_view'].data['slices']) and len(items) >= 2
+            for h, (o, a, b, c, tr) in enumerate(items):
+                regular = regular and o == h * d and a == items[0][1] + h * d and b == items[0][2] + h * d \
+                    and c == items[0][3] + h * d
+            ref = [self._attn_signature(execution, items[0][4])]
+            regular = regular and all(self._attn_signature(execution, it[4]) == ref[0] for it in items)
+            if not regular:
+                continue
+            groups.append({'heads': [it[4] for it in items], 'q_src': qs, 'k_src': ks, 'v_src': vs,
+                           'q_base': items[0][1], 'k_base': items[0][2], 'v_base': items[0][3], 'concat': cat_name,
+                           'out': cat.outputs[0].name})
+            used.update(it[4]['qk'] for it in items)
+        for tr in triples:
+            if tr['qk'] not in used:
+                groups.append({'heads': [tr], 'concat': None, 'out': tr['out']})
+        return groups
+
+    @staticmethod
+    def _attn_signature(execution, tr):
+        c1, c2, c3 = (execution.get(tr[k]).config for k in ('qk', 'softmax', 'pv'))
+        return (c1.shift, c1.rounding_mode, c2.approximation, c2.exp_kq, tuple(sorted((c2.hccs or {}).items())), c2.inv_shift,
+                c2.use_clb, c3.shift, c3.rounding_mode)
 
     def _fits(self, chain, execution) -> bool:
         if len(chain) > 8:

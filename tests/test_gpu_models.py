@@ -82,8 +82,9 @@ def test_float_quantisation_at_the_boundary(oracle):
     np.testing.assert_array_equal(got, want / 4.0)
 
 
+@pytest.mark.parametrize('probs_out', [True, False])
 @pytest.mark.parametrize('approx', ['exp', 'hccs'])
-def test_attention_core_graph(oracle, approx):
+def test_attention_core_graph(oracle, approx, probs_out):
     r = np.random.default_rng(11)
     gb = GraphBuilder()
     q = gb.input('q', (3, 128, 64), qint(8, 4))
@@ -99,11 +100,15 @@ def test_attention_core_graph(oracle, approx):
     p = gb.softmax(logits, qint(8, 8, signed=False), name='sm', directives=d)
     o = gb.matmul(p, v, qint(8, 4), name='pv')
     gb.output(o)
-    gb.output(p)
+    if probs_out:
+        gb.output(p)
     model = gb.build()
+    model.compile()
+    # with the probabilities as a graph output the three operators run separately, otherwise as one launch
+    assert (len(model.context.config['gpu_fusion_plan']['attention']) == 0) is probs_out
     ins = {n: np.clip(r.normal(0, 20, (3, 128, 64)), -128, 127).astype(np.int8) for n in 'qkv'}
     got = _graph_check(model, oracle, ins)
-    assert len(got) == 2                                 # several outputs come back as a dict by name
+    assert len(got) == (2 if probs_out else 1)           # several outputs come back as a dict by name
 
 
 @pytest.mark.parametrize('keep_sum', [False, True])
@@ -128,7 +133,12 @@ def test_add_layernorm_graph(oracle, keep_sum):
 @pytest.mark.parametrize('softmax', ['exp', 'hccs'])
 def test_encoder_block_small(oracle, softmax):
     model, x = workloads.c5_encoder_block(batch=2, seq=64, hidden=128, heads=2, ffn=256, softmax=softmax)
+    model.compile()
+    (grp,) = model.context.config['gpu_fusion_plan']['attention']
+    assert len(grp['heads']) == 2 and grp['concat']     # both heads in one fused-attention launch
     got = _graph_check(model, oracle, {'x': x})
+    model.context.config['gpu_fusion_plan'] = {}        # and the same graph operator by operator
+    _graph_check(model, oracle, {'x': x})
     out = next(iter(got.values()))
     assert len(np.unique(out)) > 32        # a live signal, not a saturated or constant tensor
 

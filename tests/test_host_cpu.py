@@ -338,6 +338,33 @@ def test_encoder_block_graph_lowers():
     assert plan['add_layernorm']['residual1_aie'] == {'layer_norm': 'ln1_aie', 'keep_sum': False}
     assert plan['mlp_chains'] == [['ffn1_aie', 'ffn2_aie']]   # widths 64/128/64 fit the fused-MLP kernel
     assert x.shape == (2, 32, 64) and x.dtype == np.int8
+    assert plan['attention'] == []          # head_dim 32 is outside the fused attention kernel's range
+
+
+def test_attention_plan_merges_heads():
+    from aie4ml_amd import workloads
+
+    model, _ = workloads.c5_encoder_block(batch=2, seq=32, hidden=192, heads=3, ffn=128)
+    ctx = lower(GraphHolder(model), FRONT + (PlanGpuFusion,))
+    (grp,) = ctx.config['gpu_fusion_plan']['attention']
+    assert [tr['qk'] for tr in grp['heads']] == ['qk0_aie', 'qk1_aie', 'qk2_aie']
+    assert grp['concat'] == 'heads_concat_aie' and (grp['q_base'], grp['k_base'], grp['v_base']) == (0, 0, 0)
+    # a lone triple (its probabilities are also a graph output in the second graph: not fusable)
+    gb = attention_graph(scale=None)
+    ctx = lower(gb, FRONT + (PlanGpuFusion,))
+    assert ctx.config['gpu_fusion_plan']['attention'] == []     # head_dim 32
+    gb = GraphBuilder()
+    q = gb.input('q', (2, 64, 64), qint(8, 4))
+    k = gb.input('k', (2, 64, 64), qint(8, 4))
+    v = gb.input('v', (2, 64, 64), qint(8, 4))
+    p = gb.softmax(gb.matmul(q, gb.transpose(k, (0, 2, 1)), qint(8, 4), name='qk'), qint(8, 8, signed=False), name='sm')
+    gb.output(gb.matmul(p, v, qint(8, 4), name='pv'))
+    ctx = lower(gb, FRONT + (PlanGpuFusion,))
+    (grp,) = ctx.config['gpu_fusion_plan']['attention']
+    assert grp['concat'] is None and grp['heads'][0]['softmax'] == 'sm_aie'
+    gb.output(p)
+    ctx = lower(gb, FRONT + (PlanGpuFusion,))
+    assert ctx.config['gpu_fusion_plan']['attention'] == []
 
 
 class GraphHolder:
