@@ -15,33 +15,6 @@
 
 namespace a4g {
 
-struct FastRound {  // (acc + c0 + cx * bit) >> s, bit = one bit of acc at `pos` (width w = 0 disables it)
-    int s, c0, pos, w, cx;
-};
-
-static FastRound make_fast_round(int mode, int s) {
-    FastRound r{s, 0, 31, 0, 0};
-    if (s <= 0) return r;
-    const int h = 1 << (s - 1);
-    switch (mode) {
-    case A4G_RND_FLOOR: break;
-    case A4G_RND_CEIL: r.c0 = (1 << s) - 1; break;
-    case A4G_RND_POSITIVE_INF: r.c0 = h; break;
-    case A4G_RND_NEGATIVE_INF: r.c0 = h - 1; break;
-    case A4G_RND_SYMMETRIC_INF: r.c0 = h; r.cx = -1; r.w = 1; break;
-    case A4G_RND_SYMMETRIC_ZERO: r.c0 = h - 1; r.cx = 1; r.w = 1; break;
-    case A4G_RND_CONV_EVEN: r.c0 = h - 1; r.cx = 1; r.w = 1; r.pos = s; break;
-    default: r.c0 = h; r.cx = -1; r.w = 1; r.pos = s; break;  // conv_odd
-    }
-    return r;
-}
-
-// |acc| stays far below 2^30 in this kernel (at most 512 products of 8-bit values), so nothing overflows.
-__device__ __forceinline__ int fast_round(int acc, const FastRound& r) {
-    const int bit = static_cast<int>(__builtin_amdgcn_ubfe(static_cast<unsigned>(acc), r.pos, r.w));
-    return (acc + r.c0 + __mul24(bit, r.cx)) >> r.s;
-}
-
 struct AttnArgs {
     const int8_t* Q;
     const int8_t* K;
@@ -70,7 +43,7 @@ __device__ __forceinline__ void transpose4x4(const unsigned a[4], unsigned c[4])
 }
 
 // NT = key/value rows / 32, DT = head dimension / 32. 256 threads = 4 waves = 128 query rows of one head.
-template <int NT, int DT>
+template <int NT, int DT, int BIT>
 __global__ __launch_bounds__(256, 2) void attention_kernel(AttnArgs a) {
     constexpr int SK = NT * 32, D = DT * 32, PITCH = SK + 16;
     extern __shared__ __attribute__((aligned(16))) int8_t attn_smem[];
@@ -147,7 +120,7 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(AttnArgs a) {
         for (int g = 0; g < 4; ++g) {
             int y[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) y[i] = clamp_i(fast_round(acc[4 * g + i], a.lr), -128, 127);
+            for (int i = 0; i < 4; ++i) y[i] = clamp_i(fast_round_k<BIT>(acc[4 * g + i], a.lr), -128, 127);
             mx = max(max(mx, y[0]), max(y[1], max(y[2], y[3])));
             lg[t][g] = pack4_bytes(y[0], y[1], y[2], y[3]);
         }
@@ -223,15 +196,24 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(AttnArgs a) {
     }
 }
 
+template <int NT, int DT>
+static void launch_attention_nt(int grid, size_t lds, hipStream_t stream, const AttnArgs& a) {
+    switch (fast_round_kind(a.lr)) {
+    case 0: attention_kernel<NT, DT, 0><<<grid, 256, lds, stream>>>(a); break;
+    case 1: attention_kernel<NT, DT, 1><<<grid, 256, lds, stream>>>(a); break;
+    default: attention_kernel<NT, DT, 2><<<grid, 256, lds, stream>>>(a); break;
+    }
+}
+
 template <int DT>
 static int launch_attention(int nt, int grid, hipStream_t stream, const AttnArgs& a) {
     const size_t lds = static_cast<size_t>(DT * 32) * (nt * 32 + 16) + 256 * 4 + DT * 32 * 4;
     switch (nt) {
-    case 1: attention_kernel<1, DT><<<grid, 256, lds, stream>>>(a); break;
-    case 2: attention_kernel<2, DT><<<grid, 256, lds, stream>>>(a); break;
-    case 4: attention_kernel<4, DT><<<grid, 256, lds, stream>>>(a); break;
-    case 8: attention_kernel<8, DT><<<grid, 256, lds, stream>>>(a); break;
-    case 16: attention_kernel<16, DT><<<grid, 256, lds, stream>>>(a); break;
+    case 1: launch_attention_nt<1, DT>(grid, lds, stream, a); break;
+    case 2: launch_attention_nt<2, DT>(grid, lds, stream, a); break;
+    case 4: launch_attention_nt<4, DT>(grid, lds, stream, a); break;
+    case 8: launch_attention_nt<8, DT>(grid, lds, stream, a); break;
+    case 16: launch_attention_nt<16, DT>(grid, lds, stream, a); break;
     default: return 1;
     }
     return 0;

@@ -101,6 +101,45 @@ __device__ __forceinline__ int apply_round(int acc, const RoundCfg& rc) {
     return q + static_cast<int>(t >> rc.s);
 }
 
+// Cheaper form for accumulators of bounded magnitude: three VALU instructions per value.
+struct FastRound {  // (acc + c0 + cx * bit) >> s, bit = one bit of acc at `pos` (width w = 0 disables it)
+    int s, c0, pos, w, cx;
+};
+
+static inline FastRound make_fast_round(int mode, int s) {
+    FastRound r{s, 0, 31, 0, 0};
+    if (s <= 0) return r;
+    const int h = 1 << (s - 1);
+    switch (mode) {
+    case A4G_RND_FLOOR: break;
+    case A4G_RND_CEIL: r.c0 = (1 << s) - 1; break;
+    case A4G_RND_POSITIVE_INF: r.c0 = h; break;
+    case A4G_RND_NEGATIVE_INF: r.c0 = h - 1; break;
+    case A4G_RND_SYMMETRIC_INF: r.c0 = h; r.cx = -1; r.w = 1; break;
+    case A4G_RND_SYMMETRIC_ZERO: r.c0 = h - 1; r.cx = 1; r.w = 1; break;
+    case A4G_RND_CONV_EVEN: r.c0 = h - 1; r.cx = 1; r.w = 1; r.pos = s; break;
+    default: r.c0 = h; r.cx = -1; r.w = 1; r.pos = s; break;  // conv_odd
+    }
+    return r;
+}
+
+// Callers guarantee |acc| + 2^s < 2^31 (short reductions of 8-bit products, s <= 24), so nothing overflows.
+__device__ __forceinline__ int fast_round(int acc, const FastRound& r) {
+    const int bit = static_cast<int>(__builtin_amdgcn_ubfe(static_cast<unsigned>(acc), r.pos, r.w));
+    return (acc + r.c0 + __mul24(bit, r.cx)) >> r.s;
+}
+
+// The same with the bit's sign fixed at compile time: BIT 0 no bit, 1 add it, 2 subtract it (kind from
+// fast_round_kind). Two or three VALU instructions per value.
+static inline int fast_round_kind(const FastRound& r) { return r.w == 0 || r.cx == 0 ? 0 : (r.cx > 0 ? 1 : 2); }
+template <int BIT>
+__device__ __forceinline__ int fast_round_k(int acc, const FastRound& r) {
+    int bit = 0;
+    if (BIT == 1) bit = static_cast<int>(__builtin_amdgcn_ubfe(static_cast<unsigned>(acc), r.pos, 1));
+    if (BIT == 2) bit = __builtin_amdgcn_sbfe(acc, r.pos, 1);
+    return (acc + r.c0 + bit) >> r.s;
+}
+
 __device__ __forceinline__ int clamp_i(int v, int lo, int hi) { return min(max(v, lo), hi); }
 
 // Low bytes of four ints -> one dword, through v_perm_b32. Shift-and-or packing of clamped shifts is

@@ -12,6 +12,7 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "matmul_lean.hpp"
 
 namespace a4g {
 
@@ -1043,6 +1044,23 @@ extern "C" int a4g_matmul_i8(const void* A, int a_kind, int64_t lda, int64_t str
                 who);
     if (batch == 0 || M == 0) return A4G_OK;
     A4G_REQUIRE(A && B && C, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+
+    // the two attention shapes have kernels of their own that need neither workspace nor K-loop barriers
+    if (out_kind != A4G_I16 && env_variant() == 0) {
+        LeanArgs la{};
+        la.A = static_cast<const int8_t*>(A);
+        la.B = B;
+        la.C = static_cast<int8_t*>(C);
+        la.lda = lda; la.stride_a = stride_a; la.ldb = ldb; la.stride_b = stride_b; la.ldc = ldc; la.stride_c = stride_c;
+        la.M = static_cast<int>(M); la.N = static_cast<int>(N); la.K = static_cast<int>(K); la.batch = static_cast<int>(batch);
+        la.a_unsigned = a_kind == A4G_U8;
+        la.lo = out_kind == A4G_I8 ? -128 : 0;
+        la.hi = out_kind == A4G_I8 ? 127 : 255;
+        la.fr = make_fast_round(round_mode, shift);
+        if (trans_b && lean_nt_applicable(la)) return check_hip(launch_lean_nt(la, stream), who);
+        if (!trans_b && lean_nn_applicable(la)) return check_hip(launch_lean_nn(la, stream), who);
+    }
+
     const size_t need = a4g_matmul_i8_workspace_bytes(batch, M, N, K, trans_b, a_kind);
     A4G_REQUIRE(need == 0 || (workspace && workspace_bytes >= need), A4G_ERR_WORKSPACE,
                 "%s: workspace of %zu bytes required, got %zu", who, need, workspace ? workspace_bytes : (size_t)0);

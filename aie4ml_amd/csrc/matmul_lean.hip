@@ -1,0 +1,256 @@
+// See matmul_lean.hpp. Arithmetic is that of matmul.cpp:80-115: int32 accumulation, shift / round /
+// saturate; a uint8 left operand is read as int8 after ^0x80 and corrected by 128 * column sum.
+//
+// Shared conventions (MFMA operands swapped, so lanes are rows): lane (m, half) supplies bytes
+// [16*half, 16*half+16) of each 32-wide k step of row m, and receives 16 results of row m. The lane that
+// supplies column j of the right operand may load any actual column: it loads column
+// 16*h' + 4*g + i for j = 8*g + 4*h' + i, which makes a lane's 16 results 16 CONTIGUOUS output bytes.
+#include "matmul_lean.hpp"
+
+namespace a4g {
+
+__device__ __forceinline__ int lean_col(int j) { return ((j >> 2) & 1) * 16 + (j >> 3) * 4 + (j & 3); }
+
+// ---- A x B^T, short K ----------------------------------------------------------------------------------
+// grid: (row blocks of 128, column chunks of 512, batch); 4 waves x 32 rows; A fragments live in registers.
+// Columns are processed in groups of TG tiles of 32. Within a group the lane that supplies MFMA column
+// j = 8*g + 4*h' + i of tile T loads actual column (16*TG)*h' + 16*T + 4*g + i, so that lane (m, half) ends
+// the group with 16*TG contiguous output bytes of row m (a whole 128-byte line per row for TG = 4).
+template <int DT, int TG>
+__device__ __forceinline__ void lean_nt_load(const LeanArgs& a, const int8_t* Bp, v4i (&bf)[TG][DT], int col0, int m, int half) {
+    const int g = m >> 3, hp = (m >> 2) & 1, i = m & 3;
+#pragma unroll
+    for (int T = 0; T < TG; ++T) {
+        const int col = col0 + 16 * TG * hp + 16 * T + 4 * g + i;
+#pragma unroll
+        for (int ks = 0; ks < DT; ++ks)
+            bf[T][ks] = *reinterpret_cast<const v4i*>(Bp + static_cast<int64_t>(col) * a.ldb + ks * 32 + half * 16);
+    }
+}
+
+template <int DT, int TG, int RB, int BIT, bool UOUT>
+__device__ __forceinline__ void lean_nt_compute(const LeanArgs& a, int8_t* Cp, const v4i (&af)[RB][DT], const v4i (&bf)[TG][DT],
+                                                int col0, int half, const int (&row)[RB], const bool (&row_ok)[RB]) {
+#pragma unroll
+    for (int T = 0; T < TG; ++T) {
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+            v16i acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+            for (int ks = 0; ks < DT; ++ks) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[T][ks], af[rb][ks], acc, 0, 0, 0);
+            v4i o;
+#pragma unroll
+            for (int gg = 0; gg < 4; ++gg) {
+                int y[4];
+#pragma unroll
+                for (int ii = 0; ii < 4; ++ii)
+                    y[ii] = UOUT ? clamp_i(fast_round_k<BIT>(acc[4 * gg + ii], a.fr), 0, 255)
+                                 : clamp_i(fast_round_k<BIT>(acc[4 * gg + ii], a.fr), -128, 127);
+                o[gg] = static_cast<int>(pack4_bytes(y[0], y[1], y[2], y[3]));
+            }
+            if (row_ok[rb])
+                *reinterpret_cast<v4i*>(Cp + static_cast<int64_t>(row[rb]) * a.ldc + col0 + 16 * TG * half + 16 * T) = o;
+        }
+    }
+}
+
+// RB = 32-row blocks per wave: 2 (256 rows per workgroup) halves how often B is re-read.
+template <int DT, int RB, int BIT, bool UOUT>
+__global__ __launch_bounds__(256, 2) void matmul_lean_nt_kernel(LeanArgs a) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int m = lane & 31, half = lane >> 5;
+    const int8_t* Ap = a.A + blockIdx.z * a.stride_a;
+    const int8_t* Bp = a.B + blockIdx.z * a.stride_b;
+    int8_t* Cp = a.C + blockIdx.z * a.stride_c;
+    const int c0 = blockIdx.y * 512, c1 = min(c0 + 512, a.N);
+
+    int row[RB];
+    bool row_ok[RB];
+    v4i af[RB][DT];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+        row[rb] = blockIdx.x * (128 * RB) + (wave * RB + rb) * 32 + m;
+        row_ok[rb] = row[rb] < a.M;
+        const int64_t rowc = row_ok[rb] ? row[rb] : a.M - 1;
+#pragma unroll
+        for (int ks = 0; ks < DT; ++ks) af[rb][ks] = *reinterpret_cast<const v4i*>(Ap + rowc * a.lda + ks * 32 + half * 16);
+    }
+    int col = c0;
+    if (col + 128 <= c1) {
+        v4i bf[4][DT], nbf[4][DT];
+        lean_nt_load<DT, 4>(a, Bp, bf, col, m, half);
+        for (; col + 128 <= c1; col += 128) {
+            const bool more = col + 256 <= c1;
+            if (more) lean_nt_load<DT, 4>(a, Bp, nbf, col + 128, m, half);  // in flight during the arithmetic below
+            lean_nt_compute<DT, 4, RB, BIT, UOUT>(a, Cp, af, bf, col, half, row, row_ok);
+            if (more) {
+#pragma unroll
+                for (int T = 0; T < 4; ++T)
+#pragma unroll
+                    for (int ks = 0; ks < DT; ++ks) bf[T][ks] = nbf[T][ks];
+            }
+        }
+    }
+    for (; col < c1; col += 32) {
+        v4i bf[1][DT];
+        lean_nt_load<DT, 1>(a, Bp, bf, col, m, half);
+        lean_nt_compute<DT, 1, RB, BIT, UOUT>(a, Cp, af, bf, col, half, row, row_ok);
+    }
+}
+
+// ---- A x B, narrow N -----------------------------------------------------------------------------------
+// grid: (row blocks of 128, batch); B^T is staged once per workgroup in LDS ([N][K + 16] bytes, natural k
+// order); a lane streams 64 contiguous bytes of its A row per group of 128 k (k order inside a group is
+// permuted identically for both operands, which an integer dot product cannot see).
+template <int NTL>
+__global__ __launch_bounds__(256, 2) void matmul_lean_nn_kernel(LeanArgs a) {
+    extern __shared__ __attribute__((aligned(16))) int8_t lean_smem[];
+    constexpr int N = NTL * 32;
+    const int pitch = a.K + 16;
+    int8_t* bt = lean_smem;
+    int* colsum = reinterpret_cast<int*>(lean_smem + N * pitch);
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int m = lane & 31, half = lane >> 5;
+    const int8_t* Ap = a.A + blockIdx.y * a.stride_a;
+    const int8_t* Bp = a.B + blockIdx.y * a.stride_b;
+    int8_t* Cp = a.C + blockIdx.y * a.stride_c;
+    const int row = blockIdx.x * 128 + wave * 32 + m;
+    const bool row_ok = row < a.M;
+    const int8_t* arow = Ap + static_cast<int64_t>(row_ok ? row : a.M - 1) * a.lda + half * 64;
+
+    v4i af[2][4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) af[0][s] = *reinterpret_cast<const v4i*>(arow + s * 16);
+
+    if (tid < N) colsum[tid] = 0;
+    __syncthreads();
+    {
+        // 4x4 byte blocks of B transposed through registers; 256 % (N/4) == 0 keeps a thread on its columns
+        const int nb = (a.K >> 2) * (N / 4);
+        const int n0 = (tid % (N / 4)) * 4;
+        int part[4] = {0, 0, 0, 0};
+        for (int blk = tid; blk < nb; blk += 256) {
+            const int k0 = (blk / (N / 4)) * 4;
+            unsigned av[4], cv[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) av[i] = *reinterpret_cast<const unsigned*>(Bp + static_cast<int64_t>(k0 + i) * a.ldb + n0);
+            const unsigned lo01 = __builtin_amdgcn_perm(av[1], av[0], 0x05010400u);
+            const unsigned hi01 = __builtin_amdgcn_perm(av[1], av[0], 0x07030602u);
+            const unsigned lo23 = __builtin_amdgcn_perm(av[3], av[2], 0x05010400u);
+            const unsigned hi23 = __builtin_amdgcn_perm(av[3], av[2], 0x07030602u);
+            cv[0] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);
+            cv[1] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
+            cv[2] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);
+            cv[3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                *reinterpret_cast<unsigned*>(bt + (n0 + j) * pitch + k0) = cv[j];
+                part[j] = __builtin_amdgcn_sdot4(static_cast<int>(cv[j]), 0x01010101, part[j], false);
+            }
+        }
+        if (a.a_unsigned) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) atomicAdd(&colsum[n0 + j], part[j]);
+        }
+    }
+    __syncthreads();
+
+    v16i acc[NTL];
+#pragma unroll
+    for (int u = 0; u < NTL; ++u) acc[u] = v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    const int xm = a.a_unsigned ? static_cast<int>(0x80808080u) : 0;
+    const int8_t* brow = bt + lean_col(m) * pitch + half * 64;
+    const int groups = a.K >> 7;
+    for (int G = 0; G < groups; ++G) {
+        const int cur = G & 1;
+        if (G + 1 < groups) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) af[cur ^ 1][s] = *reinterpret_cast<const v4i*>(arow + (G + 1) * 128 + s * 16);
+        }
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            v4i av = af[cur][s];
+            av[0] ^= xm; av[1] ^= xm; av[2] ^= xm; av[3] ^= xm;
+#pragma unroll
+            for (int u = 0; u < NTL; ++u) {
+                const v4i bv = *reinterpret_cast<const v4i*>(brow + u * 32 * pitch + G * 128 + s * 16);
+                acc[u] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bv, av, acc[u], 0, 0, 0);
+            }
+        }
+    }
+
+#pragma unroll
+    for (int u = 0; u < NTL; ++u) {
+        v4i o;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const v4i cs = *reinterpret_cast<const v4i*>(colsum + 32 * u + 16 * half + 4 * g);
+            int y[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) y[i] = clamp_i(fast_round(acc[u][4 * g + i] + 128 * cs[i], a.fr), a.lo, a.hi);
+            o[g] = static_cast<int>(pack4_bytes(y[0], y[1], y[2], y[3]));
+        }
+        if (row_ok) *reinterpret_cast<v4i*>(Cp + static_cast<int64_t>(row) * a.ldc + 32 * u + 16 * half) = o;
+    }
+}
+
+static bool lean_common_ok(const LeanArgs& a) {
+    return aligned16(a.A) && aligned16(a.B) && aligned16(a.C) && a.lda % 16 == 0 && a.ldb % 16 == 0 && a.ldc % 16 == 0 &&
+           a.stride_a % 16 == 0 && a.stride_b % 16 == 0 && a.stride_c % 16 == 0 && a.fr.s <= 24 && a.batch <= 65535 && a.M >= 1;
+}
+
+bool lean_nt_applicable(const LeanArgs& a) {
+    return lean_common_ok(a) && !a.a_unsigned && a.K % 32 == 0 && a.K <= 128 && a.N % 32 == 0 && a.N <= 512 * 65535;
+}
+
+template <int DT, int RB>
+static void launch_lean_nt_cfg(const LeanArgs& a, dim3 grid, hipStream_t stream) {
+    const int bit = fast_round_kind(a.fr);
+    const bool uo = a.lo == 0;
+#define A4G_NT(B)                                                                          \
+    if (uo)                                                                                \
+        matmul_lean_nt_kernel<DT, RB, B, true><<<grid, 256, 0, stream>>>(a);               \
+    else                                                                                   \
+        matmul_lean_nt_kernel<DT, RB, B, false><<<grid, 256, 0, stream>>>(a);
+    if (bit == 0) { A4G_NT(0) } else if (bit == 1) { A4G_NT(1) } else { A4G_NT(2) }
+#undef A4G_NT
+}
+
+template <int RB>
+static void launch_lean_nt_rb(const LeanArgs& a, hipStream_t stream) {
+    const dim3 grid(static_cast<unsigned>((a.M + 128 * RB - 1) / (128 * RB)), static_cast<unsigned>((a.N + 511) / 512),
+                    static_cast<unsigned>(a.batch));
+    switch (a.K / 32) {
+    case 1: launch_lean_nt_cfg<1, RB>(a, grid, stream); break;
+    case 2: launch_lean_nt_cfg<2, RB>(a, grid, stream); break;
+    case 3: launch_lean_nt_cfg<3, RB>(a, grid, stream); break;
+    default: launch_lean_nt_cfg<4, RB>(a, grid, stream); break;
+    }
+}
+
+hipError_t launch_lean_nt(const LeanArgs& a, hipStream_t stream) {
+    if (a.M > 128)
+        launch_lean_nt_rb<2>(a, stream);
+    else
+        launch_lean_nt_rb<1>(a, stream);
+    return hipGetLastError();
+}
+
+bool lean_nn_applicable(const LeanArgs& a) {
+    return lean_common_ok(a) && (a.N == 32 || a.N == 64 || a.N == 128) && a.K % 128 == 0 &&
+           static_cast<int64_t>(a.N) * (a.K + 16) + a.N * 4 <= 60 * 1024;
+}
+
+hipError_t launch_lean_nn(const LeanArgs& a, hipStream_t stream) {
+    const dim3 grid(static_cast<unsigned>((a.M + 127) / 128), static_cast<unsigned>(a.batch));
+    const size_t lds = static_cast<size_t>(a.N) * (a.K + 16) + a.N * 4;
+    switch (a.N / 32) {
+    case 1: matmul_lean_nn_kernel<1><<<grid, 256, lds, stream>>>(a); break;
+    case 2: matmul_lean_nn_kernel<2><<<grid, 256, lds, stream>>>(a); break;
+    default: matmul_lean_nn_kernel<4><<<grid, 256, lds, stream>>>(a); break;
+    }
+    return hipGetLastError();
+}
+
+}  // namespace a4g

@@ -194,6 +194,41 @@ def test_matmul_unsigned_lhs(ops, oracle, trans_b):
         assert np.array_equal(got, oracle.matmul(P, V, 8, 'conv_even', trans_b=trans_b, out=out))
 
 
+MODES8 = ('floor', 'ceil', 'positive_inf', 'negative_inf', 'symmetric_inf', 'symmetric_zero', 'conv_even', 'conv_odd')
+
+
+@pytest.mark.parametrize('shape', [((2, 3), 200, 96, 32), ((5,), 129, 544, 64), ((2,), 31, 1056, 96), ((), 512, 512, 128),
+                                   ((3,), 1, 32, 64)])
+def test_matmul_short_reduction_transposed_rhs(ops, oracle, shape):
+    """Q.K^T shapes (K <= 128, right operand transposed): the register-resident kernel, all rounding modes,
+    ragged row counts, more than one 512-column chunk, uint8 output."""
+    lead, M, N, K = shape
+    r = rng(M + N + K)
+    A = gauss8(r, 30, lead + (M, K))
+    B = gauss8(r, 30, lead + (N, K))
+    for i, mode in enumerate(MODES8):
+        shift = (0, 3, 6, 9)[i % 4]
+        got = host(ops.matmul(dev(A), dev(B), shift, mode, trans_b=True))
+        assert np.array_equal(got, oracle.matmul(A, B, shift, mode, trans_b=True)), (mode, shift)
+    got = host(ops.matmul(dev(A), dev(B), 5, 'conv_even', trans_b=True, out_kind='uint8'))
+    assert np.array_equal(got, oracle.matmul(A, B, 5, 'conv_even', trans_b=True, out='uint8'))
+
+
+@pytest.mark.parametrize('unsigned', [True, False])
+@pytest.mark.parametrize('shape', [((2, 2), 200, 64, 512), ((3,), 129, 32, 128), ((), 300, 128, 256), ((2,), 7, 64, 384)])
+def test_matmul_narrow_result(ops, oracle, shape, unsigned):
+    """P.V shapes (N in 32/64/128, K a multiple of 128, right operand [K][N]): the kernel that transposes
+    V into LDS itself, with int8 and uint8 left operands."""
+    lead, M, N, K = shape
+    r = rng(M + N + K + unsigned)
+    A = r.integers(0, 256, lead + (M, K)).astype(np.uint8) if unsigned else gauss8(r, 30, lead + (M, K))
+    B = gauss8(r, 30, lead + (K, N))
+    for i, mode in enumerate(MODES8):
+        shift = (8, 11, 0, 14)[i % 4]
+        got = host(ops.matmul(dev(A), dev(B), shift, mode))
+        assert np.array_equal(got, oracle.matmul(A, B, shift, mode)), (mode, shift)
+
+
 def test_matmul_rejects_bad_arguments(ops):
     a = torch.zeros((2, 16, 16), dtype=torch.int8, device='cuda')
     with pytest.raises(ValueError):
