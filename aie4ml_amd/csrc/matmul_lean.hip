@@ -28,17 +28,26 @@ __device__ __forceinline__ void lean_nt_load(const LeanArgs& a, const int8_t* Bp
     }
 }
 
+// A group of four tiles (128 columns) leaves lane (m, half) with bytes [64*half, 64*half + 64) of row m. Stored
+// as they are, every 16-byte piece is a write request of its own to L2; a round trip through a wave-private
+// LDS patch (32 rows x 128 bytes, rows padded to 144 for conflict-free access) regroups them so that eight
+// consecutive lanes write one whole 128-byte line.
+constexpr int LEAN_PATCH_PITCH = 144;
+constexpr int LEAN_PATCH_BYTES = 32 * LEAN_PATCH_PITCH;
+
 template <int DT, int TG, int RB, int BIT, bool UOUT>
 __device__ __forceinline__ void lean_nt_compute(const LeanArgs& a, int8_t* Cp, const v4i (&af)[RB][DT], const v4i (&bf)[TG][DT],
-                                                int col0, int half, const int (&row)[RB], const bool (&row_ok)[RB]) {
+                                                int col0, int lane, const int (&row)[RB], const bool (&row_ok)[RB],
+                                                int8_t* patch, int row_base) {
+    const int m = lane & 31, half = lane >> 5;
 #pragma unroll
-    for (int T = 0; T < TG; ++T) {
+    for (int rb = 0; rb < RB; ++rb) {
+        v4i o[TG];
 #pragma unroll
-        for (int rb = 0; rb < RB; ++rb) {
+        for (int T = 0; T < TG; ++T) {
             v16i acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
             for (int ks = 0; ks < DT; ++ks) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[T][ks], af[rb][ks], acc, 0, 0, 0);
-            v4i o;
 #pragma unroll
             for (int gg = 0; gg < 4; ++gg) {
                 int y[4];
@@ -46,10 +55,25 @@ __device__ __forceinline__ void lean_nt_compute(const LeanArgs& a, int8_t* Cp, c
                 for (int ii = 0; ii < 4; ++ii)
                     y[ii] = UOUT ? clamp_i(fast_round_k<BIT>(acc[4 * gg + ii], a.fr), 0, 255)
                                  : clamp_i(fast_round_k<BIT>(acc[4 * gg + ii], a.fr), -128, 127);
-                o[gg] = static_cast<int>(pack4_bytes(y[0], y[1], y[2], y[3]));
+                o[T][gg] = static_cast<int>(pack4_bytes(y[0], y[1], y[2], y[3]));
             }
-            if (row_ok[rb])
-                *reinterpret_cast<v4i*>(Cp + static_cast<int64_t>(row[rb]) * a.ldc + col0 + 16 * TG * half + 16 * T) = o;
+        }
+        if (TG == 4) {
+#pragma unroll
+            for (int T = 0; T < TG; ++T)
+                *reinterpret_cast<v4i*>(patch + m * LEAN_PATCH_PITCH + 64 * half + 16 * T) = o[T];
+            const int r0 = row_base + rb * 32;
+#pragma unroll
+            for (int s4 = 0; s4 < 4; ++s4) {
+                const int r = 8 * s4 + (lane >> 3), c = lane & 7;
+                const v4i v = *reinterpret_cast<const v4i*>(patch + r * LEAN_PATCH_PITCH + 16 * c);
+                if (r0 + r < a.M) *reinterpret_cast<v4i*>(Cp + static_cast<int64_t>(r0 + r) * a.ldc + col0 + 16 * c) = v;
+            }
+        } else {
+#pragma unroll
+            for (int T = 0; T < TG; ++T)
+                if (row_ok[rb])
+                    *reinterpret_cast<v4i*>(Cp + static_cast<int64_t>(row[rb]) * a.ldc + col0 + 16 * TG * half + 16 * T) = o[T];
         }
     }
 }
@@ -59,6 +83,9 @@ template <int DT, int RB, int BIT, bool UOUT>
 __global__ __launch_bounds__(256, 2) void matmul_lean_nt_kernel(LeanArgs a) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int m = lane & 31, half = lane >> 5;
+    __shared__ __attribute__((aligned(16))) int8_t patches[4 * LEAN_PATCH_BYTES];
+    int8_t* patch = patches + wave * LEAN_PATCH_BYTES;
+    const int row_base = blockIdx.x * (128 * RB) + wave * RB * 32;
     const int8_t* Ap = a.A + blockIdx.z * a.stride_a;
     const int8_t* Bp = a.B + blockIdx.z * a.stride_b;
     int8_t* Cp = a.C + blockIdx.z * a.stride_c;
@@ -82,7 +109,7 @@ __global__ __launch_bounds__(256, 2) void matmul_lean_nt_kernel(LeanArgs a) {
         for (; col + 128 <= c1; col += 128) {
             const bool more = col + 256 <= c1;
             if (more) lean_nt_load<DT, 4>(a, Bp, nbf, col + 128, m, half);  // in flight during the arithmetic below
-            lean_nt_compute<DT, 4, RB, BIT, UOUT>(a, Cp, af, bf, col, half, row, row_ok);
+            lean_nt_compute<DT, 4, RB, BIT, UOUT>(a, Cp, af, bf, col, lane, row, row_ok, patch, row_base);
             if (more) {
 #pragma unroll
                 for (int T = 0; T < 4; ++T)
@@ -94,7 +121,7 @@ __global__ __launch_bounds__(256, 2) void matmul_lean_nt_kernel(LeanArgs a) {
     for (; col < c1; col += 32) {
         v4i bf[1][DT];
         lean_nt_load<DT, 1>(a, Bp, bf, col, m, half);
-        lean_nt_compute<DT, 1, RB, BIT, UOUT>(a, Cp, af, bf, col, half, row, row_ok);
+        lean_nt_compute<DT, 1, RB, BIT, UOUT>(a, Cp, af, bf, col, lane, row, row_ok, patch, row_base);
     }
 }
 
