@@ -43,7 +43,9 @@ __device__ __forceinline__ void transpose4x4(const unsigned a[4], unsigned c[4])
 }
 
 // NT = key/value rows / 32, DT = head dimension / 32. 256 threads = 4 waves = 128 query rows of one head.
-template <int NT, int DT, int BIT>
+// BIT: rounding kind of the logits (fast_round_kind). FASTP: the probabilities need no clamp and their shift is
+// at most 16, so p = (e * inv) >> shift is read as byte 2 of e * (inv << (16 - shift)).
+template <int NT, int DT, int BIT, bool FASTP>
 __global__ __launch_bounds__(256, 2) void attention_kernel(AttnArgs a) {
     constexpr int SK = NT * 32, D = DT * 32, PITCH = SK + 16;
     extern __shared__ __attribute__((aligned(16))) int8_t attn_smem[];
@@ -152,20 +154,32 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(AttnArgs a) {
     v16i oacc[DT];
 #pragma unroll
     for (int u = 0; u < DT; ++u) oacc[u] = v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    const unsigned inv16 = static_cast<unsigned>(inv) << (16 - a.sm.out_shift);  // FASTP only: 0 <= inv, shift <= 16
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
         v4i pf;
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-            int p[4];
+            if (FASTP) {
+                unsigned q[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const unsigned pair = ep[t][2 * g + (i >> 1)];
-                const int e = (i & 1) ? static_cast<int>(pair >> 16) : static_cast<int>(pair & 0xFFFFu);
-                p[i] = __mul24(e, inv) >> a.sm.out_shift;
-                if (!a.noclamp) p[i] = clamp_i(p[i], 0, 255);
+                for (int i = 0; i < 4; ++i) {
+                    const unsigned pair = ep[t][2 * g + (i >> 1)];
+                    q[i] = __umul24((i & 1) ? (pair >> 16) : (pair & 0xFFFFu), inv16);  // p in bits 16..23, nothing above
+                }
+                const unsigned lo = __builtin_amdgcn_perm(q[1], q[0], 0x0c0c0602u);
+                const unsigned hi = __builtin_amdgcn_perm(q[3], q[2], 0x06020c0cu);
+                pf[g] = static_cast<int>((lo | hi) ^ 0x80808080u);
+            } else {
+                int p[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const unsigned pair = ep[t][2 * g + (i >> 1)];
+                    const int e = (i & 1) ? static_cast<int>(pair >> 16) : static_cast<int>(pair & 0xFFFFu);
+                    p[i] = clamp_i(__mul24(e, inv) >> a.sm.out_shift, 0, 255);
+                }
+                pf[g] = static_cast<int>(pack4_bytes(p[0], p[1], p[2], p[3]) ^ 0x80808080u);
             }
-            pf[g] = static_cast<int>(pack4_bytes(p[0], p[1], p[2], p[3]) ^ 0x80808080u);
         }
 #pragma unroll
         for (int u = 0; u < DT; ++u) {
@@ -198,11 +212,18 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(AttnArgs a) {
 
 template <int NT, int DT>
 static void launch_attention_nt(int grid, size_t lds, hipStream_t stream, const AttnArgs& a) {
+    const bool fastp = a.noclamp && a.sm.out_shift <= 16;
+#define A4G_ATTN(B)                                                              \
+    if (fastp)                                                                   \
+        attention_kernel<NT, DT, B, true><<<grid, 256, lds, stream>>>(a);        \
+    else                                                                         \
+        attention_kernel<NT, DT, B, false><<<grid, 256, lds, stream>>>(a);
     switch (fast_round_kind(a.lr)) {
-    case 0: attention_kernel<NT, DT, 0><<<grid, 256, lds, stream>>>(a); break;
-    case 1: attention_kernel<NT, DT, 1><<<grid, 256, lds, stream>>>(a); break;
-    default: attention_kernel<NT, DT, 2><<<grid, 256, lds, stream>>>(a); break;
+    case 0: A4G_ATTN(0) break;
+    case 1: A4G_ATTN(1) break;
+    default: A4G_ATTN(2) break;
     }
+#undef A4G_ATTN
 }
 
 template <int DT>
