@@ -126,6 +126,7 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(AttnArgs a) {
             mx = max(max(mx, y[0]), max(y[1], max(y[2], y[3])));
             lg[t][g] = pack4_bytes(y[0], y[1], y[2], y[3]);
         }
+        if (NT >= 16) __builtin_amdgcn_sched_barrier(0);  // one tile of K fragments in flight, not all sixteen
     }
     mx = max(mx, lane_xor<32>(mx));  // lanes m and m+32 share a row
 
@@ -146,6 +147,8 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(AttnArgs a) {
             ep[t][2 * g] = pack2_halves(e0, e1);
             ep[t][2 * g + 1] = pack2_halves(e2, e3);
         }
+        // keep the scheduler from hoisting many tiles' lookups at once (their results would spill)
+        if (NT >= 16 && (t & 1)) __builtin_amdgcn_sched_barrier(0);
     }
     sum += lane_xor<32>(sum);
     const int inv = row_inverse(a.sm, sum);
@@ -186,6 +189,7 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(AttnArgs a) {
             const v4i vf = *reinterpret_cast<const v4i*>(vt + (32 * u + m) * PITCH + t * 32 + half * 16);
             oacc[u] = __builtin_amdgcn_mfma_i32_32x32x32_i8(vf, pf, oacc[u], 0, 0, 0);
         }
+        if (NT >= 16 && (t & 1)) __builtin_amdgcn_sched_barrier(0);  // products of later tiles stay packed until needed
     }
 
     // ---- epilogue: + 128 * colsum (undoes the ^0x80), requantise, 16 contiguous bytes per lane ---------

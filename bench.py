@@ -33,9 +33,10 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
 # WRITE_SIZE, one counter run each, scaled by what the same counter reads for calib_copy).
 # None = not measured.
 MEASURED_TRAFFIC = {
-    'c2_dense': 215313495, 'c1_mlp': 115929, 'c4_add': 46997271, 'c4_layernorm': 31996938,
-    'c4_add_layernorm': 47107737, 'c3_softmax_exp': 255051182, 'c3_softmax_hccs': 255049600,
-    'c3_qk': 225000660, 'c3_pv': 198540800, 'calib_copy': 536870912,
+    'c2_dense': 222877251, 'c1_mlp': 163162, 'c4_add': 48256768, 'c4_layernorm': 32630962,
+    'c4_add_layernorm': 48358174, 'c3_softmax_exp': 260086260, 'c3_softmax_hccs': 260086154,
+    'c3_qk': 181584228, 'c3_pv': 205590134, 'c3_attention_exp': 200697313, 'c3_attention_hccs': 200417715,
+    'calib_copy': 536870912,
 }
 
 
