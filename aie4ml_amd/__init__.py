@@ -4,12 +4,14 @@ Public surface:
   ops            torch-tensor operator API over the HIP kernels (C ABI underneath)
   GPUModel       runtime object with the reference's compile() / predict() contract
   GraphBuilder   programmatic construction of the operator IR
+  from_onnx      ONNX Q/DQ model (path / bytes) -> GPUModel, no onnx package needed
 """
 
 from .aie_types import AIEDataType, QuantIntent, RoundingMode, SaturationMode
 from .frontends.builder import GraphBuilder, qint
+from .frontends.onnx_import import from_onnx
 from .model import GPUModel
 
 __version__ = '0.1.0'
-__all__ = ['AIEDataType', 'QuantIntent', 'RoundingMode', 'SaturationMode', 'GraphBuilder', 'GPUModel', 'qint',
+__all__ = ['AIEDataType', 'QuantIntent', 'RoundingMode', 'SaturationMode', 'GraphBuilder', 'GPUModel', 'from_onnx', 'qint',
            '__version__']

@@ -925,6 +925,10 @@ static hipError_t launch_gemm_nt(const GemmArgs& g, int batch, hipStream_t strea
     case 8: return k128 ? launch_rs<256, 64, 4, 1>(g, batch, stream) : launch_tiled<256, 64, 64, 4, 1>(g, batch, stream);
     case 9: return k64 ? launch_dtl<128, 128, 64, 2, 2, 4>(g, batch, stream) : launch_tiled<128, 128, 64, 2, 2>(g, batch, stream);
     case 10: return k128 ? launch_rs<256, 128, 2, 2>(g, batch, stream) : launch_tiled<256, 256, 64, 2, 4>(g, batch, stream);
+    case 11: return k64 ? launch_dtl<128, 128, 64, 2, 2, 2>(g, batch, stream) : launch_tiled<128, 128, 64, 2, 2>(g, batch, stream);
+    case 12: return k64 ? launch_dtl<128, 128, 64, 2, 2, 3>(g, batch, stream) : launch_tiled<128, 128, 64, 2, 2>(g, batch, stream);
+    case 13: return k64 ? launch_dtl<256, 128, 64, 2, 2, 3>(g, batch, stream) : launch_tiled<128, 128, 64, 2, 2>(g, batch, stream);
+    case 14: return k64 ? launch_dtl<256, 128, 64, 2, 2, 2>(g, batch, stream) : launch_tiled<128, 128, 64, 2, 2>(g, batch, stream);
     default: return hipErrorInvalidValue;
     }
 }

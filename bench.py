@@ -292,7 +292,10 @@ def main():
         from oracle.graph import run_graph
 
         batch, seq, hidden, heads, ffn = 64, 128, 768, 12, 3072
-        model, x = workloads.c5_encoder_block(batch, seq, hidden, heads, ffn, softmax='hccs')
+        from aie4ml_amd import from_onnx
+
+        onnx_bytes, onnx_cfg, x = workloads.c5_encoder_block_onnx(batch, seq, hidden, heads, ffn, softmax='hccs')
+        model = from_onnx(onnx_bytes, onnx_cfg)   # the block as an ONNX Q/DQ model, read by the built-in importer
         model.compile()
         dx = {'x': dev(x)}
         out_name = model.context.ir.logical.output_tensor_names[0]
@@ -308,7 +311,7 @@ def main():
         work, bound = gemm_ops + attn_ops, 'mfma'
         samples = batch
         config = {'workload': f'c5_encoder: int8 encoder block, hidden {hidden}, {heads} heads, FFN {ffn}, seq {seq}, '
-                              f'batch {batch}, HCCS softmax, LayerNorm over {hidden} columns, through the graph executor'}
+                              f'batch {batch}, HCCS softmax, LayerNorm over {hidden} columns, imported from ONNX Q/DQ, through the graph executor'}
         cpu_fn = lambda: run_graph(model, oracle, {'x': x[:nsub]})  # noqa: E731
         cpu_work = work * nsub / batch
         cpu_desc = f'oracle graph interpreter on {nsub} of {batch} sequences'

@@ -150,3 +150,23 @@ def test_encoder_block_c5_shape(oracle):
     got = _graph_check(model, oracle, {'x': x})
     out = next(iter(got.values()))
     assert out.shape[-1] == 768 and len(np.unique(out)) > 64
+
+
+@pytest.mark.parametrize('softmax', ['exp', 'hccs'])
+def test_encoder_block_from_onnx_file(oracle, softmax, tmp_path):
+    """The block written as an ONNX Q/DQ file, read back without the onnx package, run on float inputs: equals the
+    builder-made graph on the same parameters, and the oracle evaluating the imported graph."""
+    from aie4ml_amd import from_onnx
+
+    shape = (2, 64, 128, 2, 256)
+    data, cfg, x = workloads.c5_encoder_block_onnx(*shape, softmax=softmax)
+    path = tmp_path / 'encoder_block.onnx'
+    path.write_bytes(data)
+    model = from_onnx(str(path), cfg)
+    y = model.predict(x.astype(np.float32) / 16.0)                       # float in, float out (value / 2^4)
+    ref_model, x2 = workloads.c5_encoder_block(*shape, softmax=softmax)
+    want = ref_model.predict(x2, quantize_in=False, dequantize_out=False)
+    np.testing.assert_array_equal(y * 16.0, want)
+    name = model.context.ir.logical.output_tensor_names[0]
+    np.testing.assert_array_equal(want, run_graph(model, oracle, {'x': x})[name].astype(np.int64))
+    assert len(model.context.config['gpu_fusion_plan']['attention']) == 1
