@@ -890,9 +890,9 @@ static hipError_t launch_dtl(const GemmArgs& g, int batch, hipStream_t stream) {
                         : launch_dtl_u<BM, BN, BK, WAVES_M, WAVES_N, STAGES, false>(g, batch, stream);
 }
 
-// Picks a kernel and tile shape for the problem. variant: 0 = automatic; > 0 forces one (tuning only,
-// through the A4G_GEMM_VARIANT environment variable; a forced kernel whose K granularity does not
-// divide K falls back to the next finer one).
+// Picks a kernel and tile shape for the problem. variant: 0 = automatic; 1..3 force a tile shape (tuning only,
+// through the A4G_GEMM_VARIANT environment variable; a forced shape whose kernel's K granularity does not
+// divide K falls back to the next finer kernel).
 static hipError_t launch_gemm_nt(const GemmArgs& g, int batch, hipStream_t stream, int variant) {
     if (variant == 0) {
         // 256 x 256 tiles halve the L2 traffic per MAC but cost a long fill / drain per workgroup:
@@ -917,18 +917,6 @@ static hipError_t launch_gemm_nt(const GemmArgs& g, int batch, hipStream_t strea
     case 3:  // 256 x 64
         if (k64) return launch_dtl<256, 64, 64, 4, 1, 4>(g, batch, stream);
         return launch_tiled<256, 64, 64, 4, 1>(g, batch, stream);
-    // ---- tuning alternatives
-    case 4: return launch_tiled<256, 256, 64, 2, 4>(g, batch, stream);
-    case 5: return launch_tiled<128, 128, 64, 2, 2>(g, batch, stream);
-    case 6: return k64 ? launch_dtl<256, 256, 64, 2, 4, 4>(g, batch, stream) : launch_tiled<256, 256, 64, 2, 4>(g, batch, stream);
-    case 7: return k128 ? launch_rs<256, 256, 2, 4>(g, batch, stream) : launch_tiled<256, 256, 64, 2, 4>(g, batch, stream);
-    case 8: return k128 ? launch_rs<256, 64, 4, 1>(g, batch, stream) : launch_tiled<256, 64, 64, 4, 1>(g, batch, stream);
-    case 9: return k64 ? launch_dtl<128, 128, 64, 2, 2, 4>(g, batch, stream) : launch_tiled<128, 128, 64, 2, 2>(g, batch, stream);
-    case 10: return k128 ? launch_rs<256, 128, 2, 2>(g, batch, stream) : launch_tiled<256, 256, 64, 2, 4>(g, batch, stream);
-    case 11: return k64 ? launch_dtl<128, 128, 64, 2, 2, 2>(g, batch, stream) : launch_tiled<128, 128, 64, 2, 2>(g, batch, stream);
-    case 12: return k64 ? launch_dtl<128, 128, 64, 2, 2, 3>(g, batch, stream) : launch_tiled<128, 128, 64, 2, 2>(g, batch, stream);
-    case 13: return k64 ? launch_dtl<256, 128, 64, 2, 2, 3>(g, batch, stream) : launch_tiled<128, 128, 64, 2, 2>(g, batch, stream);
-    case 14: return k64 ? launch_dtl<256, 128, 64, 2, 2, 2>(g, batch, stream) : launch_tiled<128, 128, 64, 2, 2>(g, batch, stream);
     default: return hipErrorInvalidValue;
     }
 }
