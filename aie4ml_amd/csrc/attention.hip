@@ -134,6 +134,8 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(AttnArgs a) {
 
     // ---- pass B: scores by table lookup on the gap to the maximum; row sum ----------------------------
     const unsigned mrep = static_cast<unsigned>((mx ^ 0x80) & 0xFF) * 0x01010101u;
+    const char* tbytes = reinterpret_cast<const char*>(table);
+    const unsigned two = 2;
     unsigned ep[NT][8];  // two 16-bit scores per register
     int sum = 0;
 #pragma unroll
@@ -141,8 +143,10 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(AttnArgs a) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             const unsigned d4 = mrep - (lg[t][g] ^ 0x80808080u);  // per byte, never borrows
-            const int e0 = table[d4 & 0xFF], e1 = table[(d4 >> 8) & 0xFF];
-            const int e2 = table[(d4 >> 16) & 0xFF], e3 = table[d4 >> 24];
+            const int e0 = *reinterpret_cast<const int*>(tbytes + byte_x4<0>(d4, two));
+            const int e1 = *reinterpret_cast<const int*>(tbytes + byte_x4<1>(d4, two));
+            const int e2 = *reinterpret_cast<const int*>(tbytes + byte_x4<2>(d4, two));
+            const int e3 = *reinterpret_cast<const int*>(tbytes + byte_x4<3>(d4, two));
             sum += (e0 + e1) + (e2 + e3);
             ep[t][2 * g] = pack2_halves(e0, e1);
             ep[t][2 * g + 1] = pack2_halves(e2, e3);

@@ -470,7 +470,9 @@ __device__ __forceinline__ int max_i8x4(unsigned w) {
 
 // L consecutive lanes share one row (64/L rows per wave pass); lane l of the group owns chunks
 // l, l+L, ... (NCH of them), 16 int8 each.
-template <int L, int NCH, bool NOCLAMP_U8>
+// FASTP: uint8 output that needs no clamp with a shift of at most 16: the probability is read as byte 2 of
+// score * (inv << (16 - shift)), which saves the shift. FULL: cols == L * NCH * 16, no chunk is ever masked.
+template <int L, int NCH, bool FASTP, bool FULL>
 __global__ __launch_bounds__(256) void softmax_lut_kernel(const int8_t* __restrict__ x, void* __restrict__ out, int rows,
                                                            int cols, SoftmaxParams p) {
     __shared__ int table[256];
@@ -482,6 +484,8 @@ __global__ __launch_bounds__(256) void softmax_lut_kernel(const int8_t* __restri
     const int grp = lane / L, l = lane % L;
     const int wave = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
     const int nwaves = (gridDim.x * blockDim.x) >> 6;
+    const char* tbytes = reinterpret_cast<const char*>(table);
+    const unsigned two = 2;
 
     for (int row0 = wave * RPW; row0 < rows; row0 += nwaves * RPW) {
         const int row = row0 + grp;
@@ -493,7 +497,7 @@ __global__ __launch_bounds__(256) void softmax_lut_kernel(const int8_t* __restri
 #pragma unroll
         for (int i = 0; i < NCH; ++i) {
             const int col0 = (l + L * i) * 16;
-            valid[i] = row_ok && col0 < cols;
+            valid[i] = row_ok && (FULL || col0 < cols);
             xv[i] = v4i{(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
             if (valid[i]) xv[i] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(x + base + col0));
 #pragma unroll
@@ -510,10 +514,14 @@ __global__ __launch_bounds__(256) void softmax_lut_kernel(const int8_t* __restri
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
                 const unsigned d4 = mrep - (static_cast<unsigned>(xv[i][w]) ^ 0x80808080u);
+                int s4[4];
+                s4[0] = *reinterpret_cast<const int*>(tbytes + byte_x4<0>(d4, two));
+                s4[1] = *reinterpret_cast<const int*>(tbytes + byte_x4<1>(d4, two));
+                s4[2] = *reinterpret_cast<const int*>(tbytes + byte_x4<2>(d4, two));
+                s4[3] = *reinterpret_cast<const int*>(tbytes + byte_x4<3>(d4, two));
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const int d = (d4 >> (8 * j)) & 0xFF;
-                    const int s = valid[i] ? table[d] : 0;
+                    const int s = (FULL || valid[i]) ? s4[j] : 0;
                     e[i][w * 4 + j] = s;
                     sum += s;
                 }
@@ -521,6 +529,7 @@ __global__ __launch_bounds__(256) void softmax_lut_kernel(const int8_t* __restri
         }
         sum = group_allreduce<L>(sum, OpAdd());
         const int inv = row_inverse(p, sum);
+        const unsigned inv16 = static_cast<unsigned>(inv) << (16 - p.out_shift);  // FASTP only
 
 #pragma unroll
         for (int i = 0; i < NCH; ++i) {
@@ -530,8 +539,8 @@ __global__ __launch_bounds__(256) void softmax_lut_kernel(const int8_t* __restri
                 v4i o[2];
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
-                    const int y0 = sat16((e[i][2 * k] * inv) >> p.out_shift);
-                    const int y1 = sat16((e[i][2 * k + 1] * inv) >> p.out_shift);
+                    const int y0 = sat16(__mul24(e[i][2 * k], inv) >> p.out_shift);
+                    const int y1 = sat16(__mul24(e[i][2 * k + 1], inv) >> p.out_shift);
                     o[k >> 2][k & 3] = static_cast<int>(pack2_halves(y0, y1));
                 }
                 v4i* dst = reinterpret_cast<v4i*>(static_cast<int16_t*>(out) + base + col0);
@@ -541,13 +550,18 @@ __global__ __launch_bounds__(256) void softmax_lut_kernel(const int8_t* __restri
                 v4i o;
 #pragma unroll
                 for (int w = 0; w < 4; ++w) {
-                    int y4[4];
+                    if (FASTP) {
+                        unsigned q[4];
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        y4[j] = (e[i][w * 4 + j] * inv) >> p.out_shift;
-                        if (!NOCLAMP_U8) y4[j] = clamp_i(y4[j], 0, 255);
+                        for (int j = 0; j < 4; ++j) q[j] = __umul24(static_cast<unsigned>(e[i][w * 4 + j]), inv16);
+                        o[w] = static_cast<int>(__builtin_amdgcn_perm(q[1], q[0], 0x0c0c0602u) |
+                                                __builtin_amdgcn_perm(q[3], q[2], 0x06020c0cu));
+                    } else {
+                        int y4[4];
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) y4[j] = clamp_i(__mul24(e[i][w * 4 + j], inv) >> p.out_shift, 0, 255);
+                        o[w] = static_cast<int>(pack4_bytes(y4[0], y4[1], y4[2], y4[3]));
                     }
-                    o[w] = static_cast<int>(pack4_bytes(y4[0], y4[1], y4[2], y4[3]));
                 }
                 __builtin_nontemporal_store(o, reinterpret_cast<v4i*>(static_cast<uint8_t*>(out) + base + col0));
             }
@@ -593,10 +607,16 @@ __global__ __launch_bounds__(256) void softmax_generic_kernel(const int8_t* __re
 template <int L, int NCH>
 static void launch_softmax(bool noclamp, int grid, hipStream_t stream, const int8_t* x, void* out, int rows, int cols,
                            const SoftmaxParams& p) {
-    if (noclamp)
-        softmax_lut_kernel<L, NCH, true><<<grid, 256, 0, stream>>>(x, out, rows, cols, p);
+    const bool fastp = noclamp && !p.out_i16 && p.out_shift <= 16;
+    const bool full = cols == L * NCH * 16;
+    if (fastp && full)
+        softmax_lut_kernel<L, NCH, true, true><<<grid, 256, 0, stream>>>(x, out, rows, cols, p);
+    else if (fastp)
+        softmax_lut_kernel<L, NCH, true, false><<<grid, 256, 0, stream>>>(x, out, rows, cols, p);
+    else if (full)
+        softmax_lut_kernel<L, NCH, false, true><<<grid, 256, 0, stream>>>(x, out, rows, cols, p);
     else
-        softmax_lut_kernel<L, NCH, false><<<grid, 256, 0, stream>>>(x, out, rows, cols, p);
+        softmax_lut_kernel<L, NCH, false, false><<<grid, 256, 0, stream>>>(x, out, rows, cols, p);
 }
 
 static int softmax_dispatch(const int8_t* x, void* out, int64_t rows, int64_t cols, const SoftmaxParams& p, bool noclamp,

@@ -52,6 +52,17 @@ __device__ __forceinline__ int row_inverse(const SoftmaxParams& p, int sum) {
 }
 
 
+// (byte n of w) * 4 in one instruction: the LDS byte offset of a table entry.
+template <int N>
+__device__ __forceinline__ unsigned byte_x4(unsigned w, unsigned two) {
+    unsigned r;
+    if (N == 0) asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_0" : "=v"(r) : "v"(two), "v"(w));
+    if (N == 1) asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_1" : "=v"(r) : "v"(two), "v"(w));
+    if (N == 2) asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_2" : "=v"(r) : "v"(two), "v"(w));
+    if (N == 3) asm("v_lshlrev_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:BYTE_3" : "=v"(r) : "v"(two), "v"(w));
+    return r;
+}
+
 // Parameter checks of the two Softmax forms (softmax.py:339-349, softmax/common.py:59-89); both fill
 // `p` and say whether the final clamp to [0,255] can be skipped.
 static inline int make_exp_params(const char* who, int exp_kq, int inv_shift, int out_kind, SoftmaxParams* p,
