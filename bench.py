@@ -104,8 +104,8 @@ def main():
     ap.add_argument('--eager', action='store_true', help='time eager launches instead of a replayed HIP graph')
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit('bench.py: this build runs on exactly one GPU (every operator is row-independent; '
-                 'see DESIGN.md for how it would shard). Use --gpus 1.')
+        sys.exit('bench.py: this build runs on exactly one GPU (every operator is row-independent, so more GPUs '
+                 'would each take a slice of the batch with the weights replicated). Use --gpus 1.')
 
     import torch
 
