@@ -243,5 +243,45 @@ class GPUModel:
         values[insts[-1].node.outputs[0].name] = y.reshape(lead + (y.shape[-1],))
 
 
+class CapturedExecution:
+    """A whole-graph execution recorded once into a HIP graph: replaying it costs one launch on the host
+    instead of one Python round trip per operator. Inputs are copied into fixed device buffers, outputs live
+    in fixed device buffers that the next call overwrites."""
+
+    def __init__(self, model: 'GPUModel', example_inputs: Dict[str, Any]):
+        import torch
+
+        self._inputs = {k: v.clone() for k, v in example_inputs.items()}
+        # warm up on a side stream (allocator pools, lazily built kernel attributes), then record
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            model.execute(self._inputs)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        self._graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self._graph):
+            self._outputs = model.execute(self._inputs)
+
+    def __call__(self, inputs: Dict[str, Any]) -> Dict[str, Any]:
+        for name, buf in self._inputs.items():
+            src = inputs[name]
+            if tuple(src.shape) != tuple(buf.shape) or src.dtype != buf.dtype:
+                raise ValueError(f'{name}: captured for {tuple(buf.shape)} {buf.dtype}, got {tuple(src.shape)} {src.dtype}')
+            buf.copy_(src)
+        self._graph.replay()
+        return self._outputs
+
+
+def _capture(self: GPUModel, example_inputs: Dict[str, Any]) -> CapturedExecution:
+    """Record execute() on inputs of these shapes into a HIP graph; see CapturedExecution."""
+    if not self._compiled:
+        self.compile()
+    return CapturedExecution(self, example_inputs)
+
+
+GPUModel.capture = _capture
+
+
 def from_context(ctx: BackendContext) -> GPUModel:
     return GPUModel.from_context(ctx)

@@ -170,3 +170,27 @@ def test_encoder_block_from_onnx_file(oracle, softmax, tmp_path):
     name = model.context.ir.logical.output_tensor_names[0]
     np.testing.assert_array_equal(want, run_graph(model, oracle, {'x': x})[name].astype(np.int64))
     assert len(model.context.config['gpu_fusion_plan']['attention']) == 1
+
+
+def test_captured_execution_replays_match_eager(oracle):
+    """The whole encoder block recorded into a HIP graph: every replay, with eager work and synchronisations in
+    between and fresh inputs each time, equals the eager result."""
+    import torch
+
+    model, x = workloads.c5_encoder_block(4, 64, 128, 2, 256, softmax='exp')
+    model.compile()
+    name = model.context.ir.logical.output_tensor_names[0]
+    dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()  # noqa: E731
+    captured = model.capture({'x': dev(x)})
+    r = np.random.default_rng(2)
+    for i in range(4):
+        xi = np.roll(x, i, axis=0) if i < 3 else np.clip(np.rint(r.normal(0, 30, x.shape)), -128, 127).astype(np.int8)
+        eager = model.execute({'x': dev(xi)})[name].clone()
+        torch.cuda.synchronize()
+        junk = torch.randint(-128, 127, (1 << 20,), dtype=torch.int8, device='cuda').add_(1)   # unrelated eager work
+        replay = captured({'x': dev(xi)})[name]
+        torch.cuda.synchronize()
+        assert torch.equal(replay, eager), f'replay {i}'
+        del junk
+    with pytest.raises(ValueError, match='captured for'):
+        captured({'x': dev(x[:2])})
