@@ -105,6 +105,10 @@ def _resolve_output_scale_shift(node) -> int:
     return shift
 
 
+# (lhs, rhs) storage widths; (16, 8) for Dense only (the reference's list also has (16, 16), with a 64-bit accumulator)
+_SUPPORTED_INT_WIDTH_COMBOS = frozenset({(8, 8), (16, 8)})
+
+
 def _bitwidths_supported(node, device) -> bool:
     if not is_gpu(device):
         return False
@@ -113,7 +117,7 @@ def _bitwidths_supported(node, device) -> bool:
         return False
     lw = resolve_exact_storage_dtype(lhs.precision, namespace='lhs', layer_name=node.name).width
     rw = resolve_exact_storage_dtype(rhs.precision, namespace='rhs', layer_name=node.name).width
-    return (lw, rw) == (8, 8)
+    return (lw, rw) in _SUPPORTED_INT_WIDTH_COMBOS and (node.op_type == 'dense' or lw == 8)
 
 
 def _check_out_format(node, fmt: str) -> None:

@@ -115,10 +115,10 @@ def pack_dense(weight: torch.Tensor, bias: Optional[torch.Tensor], shifts) -> Pa
 
 def dense(x: torch.Tensor, p: PackedDense, rounding='floor', relu: bool = False, out_kind='int8',
           out: Optional[torch.Tensor] = None):
-    """y = saturate(round((x @ W + bias) >> shift)), optionally ReLU. x: [..., K] int8/uint8."""
+    """y = saturate(round((x @ W + bias) >> shift)), optionally ReLU. x: [..., K] int8 / uint8 / int16."""
     x2 = _rows2d(x, 'x')
-    if x2.dtype not in (torch.int8, torch.uint8):
-        raise NotImplementedError(f'dense activations must be int8 or uint8, got {x2.dtype}')
+    if x2.dtype not in (torch.int8, torch.uint8, torch.int16):
+        raise NotImplementedError(f'dense activations must be int8, uint8 or int16, got {x2.dtype}')
     if x2.shape[1] != p.K:
         raise ValueError(f'dense input has {x2.shape[1]} features, weights expect {p.K}')
     M = int(x2.shape[0])
@@ -126,6 +126,11 @@ def dense(x: torch.Tensor, p: PackedDense, rounding='floor', relu: bool = False,
     if out is None:
         out = torch.empty(tuple(x.shape[:-1]) + (p.N,), dtype=_KIND_TORCH[ok], device=x.device)
     y2 = out.reshape(-1, p.N)
+    if x2.dtype == torch.int16:
+        check(_lib.load().a4g_dense_i16(_ptr(x2), x2.stride(0) if M > 0 else p.K, _ptr(p.wt), p.ldwt, _ptr(p.colsum),
+                                        _ptr(p.bias), _ptr(p.shifts), int(p.shifts.numel()), _mode(rounding),
+                                        int(bool(relu)), ok, _ptr(y2), y2.stride(0) if M > 0 else p.N, M, p.N, p.K, _stream()))
+        return out
     check(_lib.load().a4g_dense_i8(_ptr(x2), _TORCH_KIND[x2.dtype], x2.stride(0) if M > 0 else p.K, _ptr(p.wt), p.ldwt,
                                    _ptr(p.colsum), _ptr(p.bias), _ptr(p.shifts), int(p.shifts.numel()), _mode(rounding),
                                    int(bool(relu)), ok, _ptr(y2), y2.stride(0) if M > 0 else p.N, M, p.N, p.K, _stream()))

@@ -6,7 +6,7 @@ Default workload: the single quantized Dense of the baseline configuration
 saturate to int8, fused ReLU). One step = one pass of the operator over the whole synthetic batch,
 inputs already resident in HBM. Prints ONE JSON line.
 
-Other workloads (--workload c1_mlp | c3_softmax_exp | c3_softmax_hccs | c3_qk | c3_pv |
+Other workloads (--workload c2_dense_i16 | c1_mlp | c3_softmax_exp | c3_softmax_hccs | c3_qk | c3_pv |
 c3_attention_exp | c3_attention_hccs | c4_add_layernorm | c4_layernorm | c4_add | c5_encoder) print the same line for that operator or graph;
 --workload calib_copy runs a plain 256 MiB elementwise copy, the known-size kernel the HBM traffic
 counters are scaled against.
@@ -143,6 +143,31 @@ def main():
         cpu_work = 2.0 * sample_rows * N * K
         metric, unit = 'int8_dense_tops', 'TOP/s'
         kernel = 'gemm_i8_rs_kernel'
+    elif wl == 'c2_dense_i16':
+        # the (16, 8) width combination on the C2 shape: int16 activations, int8 weights, int16 output
+        M, K, N = 8192, 4096, 4096
+        _, W, bias, shifts = workloads.c2_dense(M, K, N)
+        A = np.random.default_rng(19).integers(-32768, 32768, (M, K)).astype(np.int16)
+        shifts = shifts + 6
+        p = ops.pack_dense(dev(W), dev(bias), shifts)
+        dA = dev(A)
+        out = torch.empty((M, N), dtype=torch.int16, device='cuda')
+        fn = lambda: ops.dense(dA, p, 'conv_even', relu=True, out_kind='int16', out=out)  # noqa: E731
+        fn()
+        rows = np.random.default_rng(0).choice(M, 64, replace=False)
+        exp = oracle.dense(A[rows], W, bias, shifts, 'conv_even', relu=True, out='int16')
+        torch.cuda.synchronize()
+        bit_exact = bool(np.array_equal(out[torch.from_numpy(rows).cuda()].cpu().numpy(), exp))
+        work, bound = 2.0 * M * N * K, 'mfma'
+        samples = M
+        config = {'workload': 'c2_dense_i16: Dense 8192x4096 -> 4096, int16 activations x int8 weights (acc32), bias, '
+                              'per-channel shift, conv_even, sat int16, ReLU'}
+        sample_rows = 256
+        cpu_desc = f'oracle Dense (int16 activations) on the first {sample_rows} of {M} rows, scaled per op'
+        cpu_fn = lambda: oracle.dense(A[:sample_rows], W, bias, shifts, 'conv_even', relu=True, out='int16')  # noqa: E731
+        cpu_work = 2.0 * sample_rows * N * K
+        metric, unit = 'int16x8_dense_tops', 'TOP/s'
+        kernel = 'gemm_i16i8_kernel'
     elif wl == 'c1_mlp':
         x, layers = workloads.c1_mlp(1024)
         specs = [ops.MlpLayerSpec(ops.pack_dense(dev(Wl), dev(b), s), s, relu, o) for (Wl, b, s, relu, o) in layers]
@@ -368,7 +393,7 @@ def main():
     line = {
         'metric': metric, 'value': float(f'{value:.6g}'), 'unit': unit, 'n_gpus': 1, 'steps': args.steps,
         'warmup': args.warmup, 'ms_per_step': round(ms, 5), 'higher_is_better': True, 'scaling': 'weak',
-        'vs_baseline': None, 'dtype': 'int8', 'data': 'synthetic', 'config': config,
+        'vs_baseline': None, 'dtype': 'int16' if wl == 'c2_dense_i16' else 'int8', 'data': 'synthetic', 'config': config,
         'samples_per_s': float(f'{samples / (ms * 1e-3):.6g}'), 'bit_exact': bit_exact,
         'roofline': roof, 'cpu_baseline': cpu, 'launch': 'hip_graph' if graphed else 'eager',
     }

@@ -101,6 +101,15 @@ A4G_API int a4g_dense_i8(const void* A, int a_kind, int64_t lda, const int8_t* W
                  int round_mode, int relu, int out_kind, void* Y, int64_t ldy, int64_t M, int64_t N,
                  int64_t K, a4g_stream_t stream);
 
+/* Dense with int16 activations and int8 weights: the reference's (16, 8) width combination
+ * (op_impls/families/matmul/common.py:52), accumulated in acc32 like the 8-bit case
+ * (op_impls/utils/precision.py:120-121). Same arguments as a4g_dense_i8 with A [M][lda] int16 (lda in
+ * elements); colsum (from a4g_pack_weights_i8) is always required: the low bytes of A are fed to the
+ * matrix cores biased by 128. */
+A4G_API int a4g_dense_i16(const int16_t* A, int64_t lda, const int8_t* Wt, int64_t ldwt, const int32_t* colsum,
+                  const int32_t* bias, const int32_t* shifts, int n_shift, int round_mode, int relu, int out_kind,
+                  void* Y, int64_t ldy, int64_t M, int64_t N, int64_t K, a4g_stream_t stream);
+
 /* ---- Dynamic MatMul (both operands activations) --------------------------------------------------
  * C[b] = saturate(round((A[b] x B[b]) >> shift)), no bias, no ReLU, for b in [0, batch).
  * Replaces matmul_single/first/middle/last<Cfg>::run, templates/nnet_utils/matmul/matmul.cpp:31-390,

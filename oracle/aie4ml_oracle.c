@@ -146,7 +146,9 @@ A4O_EXPORT int a4o_dense_i8(const void* A, int a_kind, int64_t lda,
                             int mode, int relu, int out_kind,
                             void* Y, int64_t ldy,
                             int64_t M, int64_t N, int64_t K) {
-    if (!(a_kind == A4O_I8 || a_kind == A4O_U8)) return -1;
+    /* int16 activations: the reference's (16, 8) combination, also accumulated in acc32
+     * (op_impls/families/matmul/common.py:52, op_impls/utils/precision.py:120-121) */
+    if (!(a_kind == A4O_I8 || a_kind == A4O_U8 || a_kind == A4O_I16)) return -1;
     if (!(n_shift == 1 || n_shift == N)) return -1;
     /* transpose W once so the inner loop streams */
 #pragma omp parallel for schedule(static)

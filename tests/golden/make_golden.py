@@ -153,6 +153,10 @@ def main():
     big = np.full(20, 2**31 - 5, dtype=np.int64)  # accumulator wraps to negative
     d['bias_wrap'] = big.astype(np.int32)
     d['y__wrap'] = dense(np.abs(A), np.abs(W), big, np.full(20, 10), 'floor', False, 'int8')
+    A16 = r.integers(-32768, 32768, (12, 40)).astype(np.int16)
+    d['A16'] = A16
+    d['y__i16in__conv_even__i16'] = dense(A16, W, bias, np.full(20, 9), 'conv_even', False, 'int16')
+    d['y__i16in__symmetric_inf__i8relu'] = dense(A16, W, bias, shifts + 8, 'symmetric_inf', True, 'int8')
     np.savez_compressed(HERE / 'dense.npz', **d)
 
     # ---- matmul (batched, both operand orders, uint8 left operand) -------------------------------------

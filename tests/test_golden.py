@@ -40,6 +40,9 @@ def test_oracle_dense_matmul_add(oracle):
                                   g['y__u8out__symmetric_inf'])
     np.testing.assert_array_equal(oracle.dense(g['A'], g['W'], g['bias'], 2, 'conv_even', out='int16'), g['y__i16out__conv_even'])
     np.testing.assert_array_equal(oracle.dense(np.abs(g['A']), np.abs(g['W']), g['bias_wrap'], 10, 'floor'), g['y__wrap'])
+    np.testing.assert_array_equal(oracle.dense(g['A16'], g['W'], g['bias'], 9, 'conv_even', out='int16'), g['y__i16in__conv_even__i16'])
+    np.testing.assert_array_equal(oracle.dense(g['A16'], g['W'], g['bias'], g['shifts'] + 8, 'symmetric_inf', relu=True),
+                                  g['y__i16in__symmetric_inf__i8relu'])
     m = load('matmul')
     for mode in ('conv_even', 'symmetric_inf', 'floor'):
         np.testing.assert_array_equal(oracle.matmul(m['Aq'], m['Bk'], 5, mode, trans_b=True), m[f'qk__{mode}'])
@@ -102,6 +105,10 @@ def test_gpu_dense_matmul_add():
                                   g['y__i16out__conv_even'])
     wrap = ops.pack_dense(_dev(np.abs(g['W'])), _dev(g['bias_wrap']), 10)
     np.testing.assert_array_equal(_host(ops.dense(_dev(np.abs(g['A'])), wrap, 'floor')), g['y__wrap'])
+    np.testing.assert_array_equal(_host(ops.dense(_dev(g['A16']), ops.pack_dense(W, bias, 9), 'conv_even', out_kind='int16')),
+                                  g['y__i16in__conv_even__i16'])
+    np.testing.assert_array_equal(_host(ops.dense(_dev(g['A16']), ops.pack_dense(W, bias, g['shifts'] + 8), 'symmetric_inf', relu=True)),
+                                  g['y__i16in__symmetric_inf__i8relu'])
     m = load('matmul')
     for mode in ('conv_even', 'symmetric_inf', 'floor'):
         np.testing.assert_array_equal(_host(ops.matmul(_dev(m['Aq']), _dev(m['Bk']), 5, mode, trans_b=True)), m[f'qk__{mode}'])

@@ -194,3 +194,22 @@ def test_captured_execution_replays_match_eager(oracle):
         del junk
     with pytest.raises(ValueError, match='captured for'):
         captured({'x': dev(x[:2])})
+
+
+def test_int16_activation_mlp_graph(oracle):
+    """An MLP with 16-bit activations and 8-bit weights (the (16, 8) combination hls4ml models use): the dense
+    variant accepts it, the fused-MLP kernel (8-bit only) is not chosen, results equal the oracle."""
+    r = np.random.default_rng(23)
+    gb = GraphBuilder()
+    t = gb.input('x', (64, 48), qint(16, 8))
+    dims = [48, 96, 64, 10]
+    for i in range(3):
+        W = r.integers(-100, 100, (dims[i], dims[i + 1])) / 128.0
+        b = r.integers(-512, 512, dims[i + 1]) / 32768.0
+        t = gb.dense(t, W, qint(8, 7), qint(16, 8), bias=b, bias_precision=qint(32, 15), relu=i < 2, name=f'fc{i}')
+    gb.output(t)
+    model = gb.build()
+    model.compile()
+    assert model.context.config['gpu_fusion_plan']['mlp_chains'] == []
+    x = r.integers(-32768, 32768, (64, 48)).astype(np.int16)
+    _graph_check(model, oracle, {'x': x})

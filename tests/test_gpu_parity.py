@@ -194,6 +194,27 @@ def test_matmul_unsigned_lhs(ops, oracle, trans_b):
         assert np.array_equal(got, oracle.matmul(P, V, 8, 'conv_even', trans_b=trans_b, out=out))
 
 
+@pytest.mark.parametrize('shape', [(300, 200, 256), (128, 128, 64), (33, 17, 48), (70, 130, 1000), (5, 9, 23), (1024, 512, 512)])
+def test_dense_int16_activations(ops, oracle, shape):
+    """(16, 8) Dense: int16 activations split into byte planes on the matrix cores, acc32 semantics; aligned shapes take
+    the tiled kernel, the others the generic one; int16 / int8 / uint8 outputs, ReLU, per-channel shifts, a wrapping bias."""
+    M, N, K = shape
+    r = rng(M + N + K)
+    A = r.integers(-32768, 32768, (M, K)).astype(np.int16)
+    A[0, :] = 32767
+    A[-1, :] = -32768
+    W = gauss8(r, 40, (K, N))
+    bias = r.integers(-2**24, 2**24, N).astype(np.int32)
+    shifts = r.integers(10, 16, N).astype(np.int32)
+    p = ops.pack_dense(dev(W), dev(bias), shifts)
+    for mode, relu, kind in (('conv_even', False, 'int16'), ('symmetric_inf', True, 'int8'), ('floor', False, 'uint8')):
+        got = host(ops.dense(dev(A), p, mode, relu=relu, out_kind=kind))
+        assert np.array_equal(got, oracle.dense(A, W, bias, shifts, mode, relu=relu, out=kind)), (mode, kind)
+    big = np.full(N, 2**31 - 77, dtype=np.int32)      # the 32-bit accumulator wraps, as acc32 does
+    got = host(ops.dense(dev(np.abs(A)), ops.pack_dense(dev(np.abs(W)), dev(big), 16), 'conv_even', out_kind='int16'))
+    assert np.array_equal(got, oracle.dense(np.abs(A), np.abs(W), big, 16, 'conv_even', out='int16'))
+
+
 MODES8 = ('floor', 'ceil', 'positive_inf', 'negative_inf', 'symmetric_inf', 'symmetric_zero', 'conv_even', 'conv_odd')
 
 

@@ -249,9 +249,21 @@ def test_matmul_rules():
     with pytest.raises(ValueError):
         lower(gb)
     gb = GraphBuilder()
-    a = gb.input('a', (2, 16, 32), qint(16, 4))
+    a = gb.input('a', (2, 16, 32), qint(32, 4))
     gb.output(gb.dense(a, np.zeros((32, 8)), qint(8, 7), qint(8, 4)))
     with pytest.raises(ValueError, match='no dense variant matches'):
+        lower(gb)
+    # 16-bit activations with 8-bit weights are a Dense combination (acc32), not a MatMul one
+    gb = GraphBuilder()
+    a = gb.input('a', (2, 16, 32), qint(16, 8))
+    gb.output(gb.dense(a, np.zeros((32, 8)), qint(8, 7), qint(16, 8), name='fc'))
+    cfg = lower(gb).ir.execution.get('fc_aie').config
+    assert cfg.precision['lhs'].format == 'int16' and cfg.shift == 8 + 7 - 8 and cfg.accumulator_tag == 'acc32'
+    gb = GraphBuilder()
+    a = gb.input('a', (2, 16, 32), qint(16, 8))
+    b = gb.input('b', (2, 32, 16), qint(8, 4))
+    gb.output(gb.matmul(a, b, qint(8, 4)))
+    with pytest.raises(ValueError, match='no matmul variant matches'):
         lower(gb)
 
 

@@ -99,6 +99,19 @@ def test_dense_vs_int64_matmul(oracle, a_dtype, mode):
     assert np.array_equal(a, b)
 
 
+def test_dense_int16_activations_vs_int64_matmul(oracle):
+    """(16, 8) Dense: int64 numpy product wrapped to 32 bits, then the exact srs; includes a wrapping bias."""
+    r = _rng(61)
+    A = r.integers(-32768, 32768, (9, 70)).astype(np.int16)
+    W = r.integers(-128, 128, (70, 11)).astype(np.int8)
+    for bias in (r.integers(-2**20, 2**20, 11).astype(np.int32), np.full(11, 2**31 - 1000, dtype=np.int32)):
+        acc = A.astype(np.int64) @ W.astype(np.int64) + bias.astype(np.int64)
+        acc = ((acc + 2**31) % 2**32) - 2**31
+        for mode, shift, kind in (('conv_even', 9, 'int16'), ('symmetric_inf', 14, 'int8'), ('floor', 0, 'int16')):
+            want = np.array([[exact_srs(int(v), shift, mode, kind) for v in row] for row in acc])
+            np.testing.assert_array_equal(oracle.dense(A, W, bias, shift, mode, out=kind), want)
+
+
 def test_dense_special_cases(oracle):
     r = _rng(2)
     K = 16
