@@ -34,9 +34,9 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
 # None = not measured.
 MEASURED_TRAFFIC = {
     'c2_dense': 222877251, 'c1_mlp': 163162, 'c4_add': 48256768, 'c4_layernorm': 32630962,
-    'c4_add_layernorm': 48358174, 'c3_softmax_exp': 260086260, 'c3_softmax_hccs': 260086154,
-    'c3_qk': 181584228, 'c3_pv': 205590134, 'c3_attention_exp': 200697313, 'c3_attention_hccs': 200417715,
-    'calib_copy': 536870912,
+    'c4_add_layernorm': 48358174, 'c3_softmax_exp': 260085316, 'c3_softmax_hccs': 260085793,
+    'c3_qk': 181584228, 'c3_pv': 205590134, 'c3_attention_exp': 195232175, 'c3_attention_hccs': 195226688,
+    'calib_copy': 536870912, 'c2_dense_i16': 697146376,
 }
 
 
