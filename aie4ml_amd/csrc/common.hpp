@@ -142,6 +142,14 @@ __device__ __forceinline__ int fast_round_k(int acc, const FastRound& r) {
 
 __device__ __forceinline__ int clamp_i(int v, int lo, int hi) { return min(max(v, lo), hi); }
 
+// clamp_i as one instruction for bounds that are only known at run time (callers guarantee lo <= hi,
+// which the compiler would have to prove before it forms the median by itself).
+__device__ __forceinline__ int clamp_med3(int v, int lo, int hi) {
+    int y;
+    asm("v_med3_i32 %0, %1, %2, %3" : "=v"(y) : "v"(v), "v"(lo), "v"(hi));
+    return y;
+}
+
 // Low bytes of four ints -> one dword, through v_perm_b32. Shift-and-or packing of clamped shifts is
 // avoided on purpose: the compiler folds that shape into gfx950's v_ashr_pk_u8_i32 / _i8_i32 and then
 // treats the upper half of its result as zero, which the hardware does not guarantee.

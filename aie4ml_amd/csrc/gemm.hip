@@ -14,6 +14,20 @@
 #include "common.hpp"
 #include "matmul_lean.hpp"
 
+// Phase stamps for tuning builds (-DA4G_TIMING): thread 0 of every workgroup records the 100 MHz
+// real-time counter at a few points of the pipelined kernel. Compiled out of the library.
+#ifdef A4G_TIMING
+__device__ unsigned long long a4g_stamps[8 * 65536];
+#define A4G_STAMP(i)                                                                                  \
+    do {                                                                                              \
+        if (threadIdx.x == 0 && blockIdx.x < 65536) a4g_stamps[blockIdx.x * 8 + (i)] = __builtin_amdgcn_s_memrealtime(); \
+    } while (0)
+#else
+#define A4G_STAMP(i) \
+    do {             \
+    } while (0)
+#endif
+
 namespace a4g {
 
 struct GemmArgs {
@@ -307,10 +321,12 @@ __device__ __forceinline__ void fetch_col_params(const GemmArgs& g, const TileCo
     }
 }
 
-// Parks them in LDS; returns true (workgroup-uniform) when some shift exceeds 15. Contains a barrier.
+// Parks them in LDS; returns (workgroup-uniform) which requantisation path the tile takes: 0 = every
+// shift is within 1..15 (or the mode needs no tie bit), 1 = some shift is 0, 2 = some shift exceeds 15.
+// Contains barriers.
 template <int BN>
-__device__ __forceinline__ bool park_col_params(const GemmArgs& g, const ColParams<BN>& cp, int tid, int col_add, int col_shift) {
-    int big_shift = 0;
+__device__ __forceinline__ int park_col_params(const GemmArgs& g, const ColParams<BN>& cp, int tid, int col_add, int col_shift) {
+    int big_shift = 0, zero_shift = 0;
     if (tid < BN) {
         const RoundCfg rc = make_round(g.mode, col_shift);
         cp.add[tid] = col_add;
@@ -319,8 +335,10 @@ __device__ __forceinline__ bool park_col_params(const GemmArgs& g, const ColPara
         cp.cx[tid] = rc.cx;
         cp.bs[tid] = rc.bs;
         big_shift = rc.s > 15;
+        zero_shift = rc.s <= 0;
     }
-    return __syncthreads_or(big_shift) != 0;
+    if (__syncthreads_or(big_shift) != 0) return 2;
+    return __syncthreads_or(zero_shift) != 0 ? 1 : 0;
 }
 
 // Epilogue shared by the pipelined kernels: requantise the accumulators into an LDS image of the
@@ -331,13 +349,22 @@ __device__ __forceinline__ bool park_col_params(const GemmArgs& g, const ColPara
 // The caller has made sure that no tile load is in flight and that all waves are past the main loop.
 template <int BM, int BN, int WTM, int WTN, int NT>
 __device__ __forceinline__ void epilogue_store(const GemmArgs& g, const TileCoord& tc, v16i (&acc)[WTM / 32][WTN / 32],
-                                               int8_t* smem, const ColParams<BN>& cp, bool slow_round, int wm, int wn, int lane,
+                                               int8_t* smem, const ColParams<BN>& cp, int round_path, int wm, int wn, int lane,
                                                int tid) {
     constexpr int TM = WTM / 32, TN = WTN / 32;
     const int lo = g.relu ? max(kind_lo(g.out_kind), 0) : kind_lo(g.out_kind), hi = kind_hi(g.out_kind);
     const int obytes = (g.out_kind == A4G_I16 || g.out_kind == A4G_U16) ? 2 : 1;
     const int cpitch = BN * obytes + 16;
     int8_t* Cb = static_cast<int8_t*>(g.C) + tc.batch * g.stride_c * obytes;
+    auto store_quad = [&](int ml, int nl, const int (&y)[4]) {
+        if (obytes == 1) {
+            *reinterpret_cast<unsigned*>(smem + ml * cpitch + nl) = pack4_bytes(y[0], y[1], y[2], y[3]);
+        } else {
+            v2i o = {static_cast<int>(pack2_halves(y[0], y[1])), static_cast<int>(pack2_halves(y[2], y[3]))};
+            *reinterpret_cast<v2i*>(smem + ml * cpitch + nl * 2) = o;
+        }
+    };
+    // General forms: PATH 1 multiplies the tie bit by its per-column sign, PATH 2 is the overflow-free one.
     auto requantise = [&](auto slow_tag) {
         constexpr bool SLOW = decltype(slow_tag)::value;
 #pragma unroll
@@ -371,19 +398,54 @@ __device__ __forceinline__ void epilogue_store(const GemmArgs& g, const TileCoor
                             y[t] = clamp_i(apply_round(a, rc), lo, hi);
                         }
                     }
-                    if (obytes == 1) {
-                        *reinterpret_cast<unsigned*>(smem + ml * cpitch + nl) = pack4_bytes(y[0], y[1], y[2], y[3]);
-                    } else {
-                        v2i o = {static_cast<int>(pack2_halves(y[0], y[1])), static_cast<int>(pack2_halves(y[2], y[3]))};
-                        *reinterpret_cast<v2i*>(smem + ml * cpitch + nl * 2) = o;
-                    }
+                    store_quad(ml, nl, y);
                 }
             }
         }
     };
-    if (slow_round) requantise(std::true_type{});
-    else requantise(std::false_type{});
+    // Shifts within 1..15: the sign of the tie bit (BIT 0 none, 1 added, 2 subtracted) and where it sits
+    // (CONV: bit s of the sum, else its sign) are compile-time facts of the rounding mode, which leaves
+    // add, bit extract, add, saturating add, shift and one median per value.
+    auto requantise_fast = [&](auto bit_tag, auto conv_tag) {
+        constexpr int BIT = decltype(bit_tag)::value;
+        constexpr bool CONV = decltype(conv_tag)::value;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int nl = wn * WTN + j * 32 + 8 * q + 4 * (lane >> 5);
+                const v4i add4 = *reinterpret_cast<const v4i*>(cp.add + nl);
+                const v4i s4 = *reinterpret_cast<const v4i*>(cp.s + nl);
+                const v4i c04 = *reinterpret_cast<const v4i*>(cp.c0 + nl);
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+                    const int ml = wm * WTM + i * 32 + (lane & 31);
+                    int y[4];
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const int a = static_cast<int>(static_cast<unsigned>(acc[i][j][q * 4 + t]) + static_cast<unsigned>(add4[t]));
+                        int off = c04[t];
+                        if (BIT == 1) off += static_cast<int>(__builtin_amdgcn_ubfe(static_cast<unsigned>(a), CONV ? s4[t] : 31, 1));
+                        if (BIT == 2) off += __builtin_amdgcn_sbfe(a, CONV ? s4[t] : 31, 1);
+                        y[t] = clamp_med3(__builtin_elementwise_add_sat(a, off) >> s4[t], lo, hi);
+                    }
+                    store_quad(ml, nl, y);
+                }
+            }
+        }
+    };
+    using B0 = std::integral_constant<int, 0>;
+    using B1 = std::integral_constant<int, 1>;
+    using B2 = std::integral_constant<int, 2>;
+    if (round_path == 2) requantise(std::true_type{});
+    else if (g.mode <= A4G_RND_NEGATIVE_INF) requantise_fast(B0{}, std::false_type{});
+    else if (round_path == 1) requantise(std::false_type{});
+    else if (g.mode == A4G_RND_SYMMETRIC_INF) requantise_fast(B2{}, std::false_type{});
+    else if (g.mode == A4G_RND_SYMMETRIC_ZERO) requantise_fast(B1{}, std::false_type{});
+    else if (g.mode == A4G_RND_CONV_EVEN) requantise_fast(B1{}, std::true_type{});
+    else requantise_fast(B2{}, std::true_type{});
     __syncthreads();
+    A4G_STAMP(4);
     const int cpr = BN * obytes / 16;  // 16-byte chunks per tile row
     const bool vec_ok = ((g.ldc * obytes) % 16 == 0) && ((reinterpret_cast<uintptr_t>(Cb) & 15) == 0);
     for (int idx = tid; idx < BM * cpr; idx += NT) {
@@ -496,7 +558,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_i8_dtl_kernel(Gemm
 #pragma unroll
     for (int st = 0; st < STAGES; ++st) issue_tile(min(st, ktiles - 1), st);
 
-    const bool slow_round = park_col_params<BN>(g, cp, tid, col_add, col_shift);
+    const int round_path = park_col_params<BN>(g, cp, tid, col_add, col_shift);
 
     // ---- fragment addressing: row = lane%32 of the block, 16-byte half of the 32-wide K step = lane/32
     const int frow = lane & 31;
@@ -518,12 +580,16 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_i8_dtl_kernel(Gemm
     constexpr int NR = Cfg::TM + Cfg::TN, NM = Cfg::TM * Cfg::TN;
     auto read_one = [&](int set, const int8_t* base, int kk, int idx) {
         // order B0, A0, B1, A1, ... so that the first MFMA of the next step can start early
-        if (idx < 2 * Cfg::TN) {
+        constexpr int TMIN = Cfg::TM < Cfg::TN ? Cfg::TM : Cfg::TN;
+        if (idx < 2 * TMIN) {
             if (idx & 1) af[set][idx >> 1] = *reinterpret_cast<const v4i*>(base + a_off + (idx >> 1) * 32 * BK + koff[kk]);
             else bf[set][idx >> 1] = *reinterpret_cast<const v4i*>(base + b_off + (idx >> 1) * 32 * BK + koff[kk]);
-        } else {
-            const int i = idx - Cfg::TN;
+        } else if (Cfg::TM > Cfg::TN) {
+            const int i = idx - TMIN;
             af[set][i] = *reinterpret_cast<const v4i*>(base + a_off + i * 32 * BK + koff[kk]);
+        } else {
+            const int j = idx - TMIN;
+            bf[set][j] = *reinterpret_cast<const v4i*>(base + b_off + j * 32 * BK + koff[kk]);
         }
     };
     // MFMAs of the fragment set `cur`, with the reads of set `nxt` threaded between them
@@ -571,7 +637,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_i8_dtl_kernel(Gemm
     wait_vmcnt<0>();
     __syncthreads();
 
-    epilogue_store<BM, BN, Cfg::WTM, Cfg::WTN, Cfg::NT>(g, tc, acc, smem, cp, slow_round, wm, wn, lane, tid);
+    epilogue_store<BM, BN, Cfg::WTM, Cfg::WTN, Cfg::NT>(g, tc, acc, smem, cp, round_path, wm, wn, lane, tid);
 }
 
 // -----------------------------------------------------------------------------------------------------
@@ -605,7 +671,7 @@ struct RsCfg {
     static constexpr int LDS_BYTES = PARAM_OFF + ColParams<BN>::BYTES;
     static_assert(BM % ROWS_PER_PASS == 0 && BN % ROWS_PER_PASS == 0, "tile rows must divide over the threads");
     static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be whole 32x32 MFMA blocks");
-    static_assert(TM >= TN && TM * TN >= TM + TN, "one fragment read is issued behind each MFMA");
+    static_assert(TM * TN >= TM + TN, "one fragment read is issued behind each MFMA");
     static constexpr int EPM = (LOADS + TM * TN - 1) / (TM * TN);  // staging writes / global loads behind each MFMA
     static_assert(ROWS_PER_PASS % 16 == 0, "the swizzle term must not depend on the pass");
     static_assert((BM + BN) * BK <= 65536, "ds_write immediate offsets are 16 bits");
@@ -623,6 +689,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_i8_rs_kernel(GemmA
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 
+    A4G_STAMP(0);
     const TileCoord tc = tile_coord<BM, BN>(g);
     if (!tc.valid) return;
     const int m0 = tc.m0, n0 = tc.n0;
@@ -659,7 +726,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_i8_rs_kernel(GemmA
 #pragma unroll
     for (int i = 0; i < Cfg::LOADS; ++i) load_one(0, i);
 
-    const bool slow_round = park_col_params<BN>(g, cp, tid, col_add, col_shift);
+    const int round_path = park_col_params<BN>(g, cp, tid, col_add, col_shift);
+    A4G_STAMP(1);
 
     // ---- fragment addressing: row = lane%32 of the block, 16-byte half of the 32-wide K step = lane/32
     const int frow = lane & 31;
@@ -680,12 +748,16 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_i8_rs_kernel(GemmA
     v4i af[2][Cfg::TM], bf[2][Cfg::TN];
     constexpr int NR = Cfg::TM + Cfg::TN, NM = Cfg::TM * Cfg::TN;
     auto read_one = [&](int set, const int8_t* base, int kk, int idx) {
-        if (idx < 2 * Cfg::TN) {
+        constexpr int TMIN = Cfg::TM < Cfg::TN ? Cfg::TM : Cfg::TN;
+        if (idx < 2 * TMIN) {
             if (idx & 1) af[set][idx >> 1] = *reinterpret_cast<const v4i*>(base + a_off + (idx >> 1) * 32 * BK + koff[kk]);
             else bf[set][idx >> 1] = *reinterpret_cast<const v4i*>(base + b_off + (idx >> 1) * 32 * BK + koff[kk]);
-        } else {
-            const int i = idx - Cfg::TN;
+        } else if (Cfg::TM > Cfg::TN) {
+            const int i = idx - TMIN;
             af[set][i] = *reinterpret_cast<const v4i*>(base + a_off + i * 32 * BK + koff[kk]);
+        } else {
+            const int j = idx - TMIN;
+            bf[set][j] = *reinterpret_cast<const v4i*>(base + b_off + j * 32 * BK + koff[kk]);
         }
     };
     // EXTRA: 0 = nothing, 1 = staging writes into `stage_w`, 2 = global loads of tile `kt_load`
@@ -729,6 +801,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_i8_rs_kernel(GemmA
     __syncthreads();
 #pragma unroll
     for (int r = 0; r < NR; ++r) read_one(0, smem, 0, r);
+    A4G_STAMP(2);
 
     for (int kt = 0; kt < ktiles; ++kt) {
         int8_t* cur_base = smem + (kt & 1) * Cfg::STAGE_BYTES;
@@ -752,8 +825,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_i8_rs_kernel(GemmA
         __builtin_amdgcn_sched_barrier(0);
     }
     __syncthreads();  // every wave is past its last fragment read before the stages become the output image
+    A4G_STAMP(3);
 
-    epilogue_store<BM, BN, Cfg::WTM, Cfg::WTN, Cfg::NT>(g, tc, acc, smem, cp, slow_round, wm, wn, lane, tid);
+    epilogue_store<BM, BN, Cfg::WTM, Cfg::WTN, Cfg::NT>(g, tc, acc, smem, cp, round_path, wm, wn, lane, tid);
+    A4G_STAMP(5);
 }
 
 // -----------------------------------------------------------------------------------------------------
@@ -890,7 +965,7 @@ static hipError_t launch_dtl(const GemmArgs& g, int batch, hipStream_t stream) {
                         : launch_dtl_u<BM, BN, BK, WAVES_M, WAVES_N, STAGES, false>(g, batch, stream);
 }
 
-// Picks a kernel and tile shape for the problem. variant: 0 = automatic; 1..3 force a tile shape (tuning only,
+// Picks a kernel and tile shape for the problem. variant: 0 = automatic; 1..4 force a tile shape (tuning only,
 // through the A4G_GEMM_VARIANT environment variable; a forced shape whose kernel's K granularity does not
 // divide K falls back to the next finer kernel).
 static hipError_t launch_gemm_nt(const GemmArgs& g, int batch, hipStream_t stream, int variant) {
@@ -902,6 +977,10 @@ static hipError_t launch_gemm_nt(const GemmArgs& g, int batch, hipStream_t strea
         const int64_t rounds256 = (tiles256 + 255) / 256;  // one workgroup per CU at a time
         const bool fills = tiles256 * 100 >= rounds256 * 256 * 85;
         variant = (g.M >= 256 && g.N >= 256 && g.K >= 512 && fills) ? 1 : 2;
+        // Widths that are multiples of 192 but not of 256 (768 = 3 * 256 columns on 256 CUs): 128 x 192
+        // tiles that make exactly one round of workgroups measured 5-15 % faster than 128 x 128.
+        const int64_t tiles192 = static_cast<int64_t>((g.M + 127) / 128) * ((g.N + 191) / 192) * batch;
+        if (variant == 2 && g.N % 192 == 0 && g.K % 128 == 0 && tiles192 <= 256 && tiles192 >= 224) variant = 4;
     }
     const bool k128 = g.K % 128 == 0, k64 = g.K % 64 == 0;
     switch (variant) {
@@ -914,6 +993,10 @@ static hipError_t launch_gemm_nt(const GemmArgs& g, int batch, hipStream_t strea
         if (k128) return launch_rs<128, 128, 2, 2>(g, batch, stream);
         if (k64) return launch_dtl<128, 128, 64, 2, 2, 4>(g, batch, stream);
         return launch_tiled<128, 128, 64, 2, 2>(g, batch, stream);
+    case 4:  // 128 x 192
+        if (k128) return g.a_unsigned ? launch_rs_u<128, 192, 2, 2, true, true>(g, batch, stream)
+                                      : launch_rs_u<128, 192, 2, 2, false, true>(g, batch, stream);
+        return launch_gemm_nt(g, batch, stream, 2);
     case 3:  // 256 x 64
         if (k64) return launch_dtl<256, 64, 64, 4, 1, 4>(g, batch, stream);
         return launch_tiled<256, 64, 64, 4, 1>(g, batch, stream);

@@ -157,6 +157,37 @@ def test_dense_accumulator_wraps(ops, oracle):
     assert np.array_equal(got, oracle.dense(A, W, bias, 12, 'conv_even'))
 
 
+@pytest.mark.parametrize('mode', MODES)
+@pytest.mark.parametrize('shift_set', ['1..15', 'with zero', 'beyond 15'])
+def test_dense_requantisation_paths_with_extreme_accumulators(ops, oracle, mode, shift_set):
+    # the tiled kernels choose their requantisation form from the shifts of a tile: all within 1..15, some
+    # zero, some above 15; the bias puts accumulators next to both int32 extremes and on exact ties
+    r = rng(31)
+    M, K, N = 160, 128, 192
+    A = gauss8(r, 40, (M, K))
+    W = gauss8(r, 30, (K, N))
+    W[:, ::3] = 0  # those columns give srs(bias) exactly
+    lo, hi = {'1..15': (1, 16), 'with zero': (0, 16), 'beyond 15': (0, 25)}[shift_set]
+    shifts = r.integers(lo, hi, N).astype(np.int32)
+    shifts[:hi - lo] = np.arange(lo, hi)
+    bias = r.integers(-2**20, 2**20, N).astype(np.int64)
+    bias[0::12] = 2**31 - 1 - r.integers(0, 70000, len(bias[0::12]))
+    bias[3::12] = -2**31 + r.integers(0, 70000, len(bias[3::12]))
+    bias[6::12] = (1 << shifts[6::12].astype(np.int64)) // 2 * r.choice([-3, -1, 1, 3], len(bias[6::12]))
+    bias = bias.astype(np.int32)
+    p = ops.pack_dense(dev(W), dev(bias), shifts)
+    for out, relu in (('int8', False), ('uint8', False), ('int16', True)):
+        got = host(ops.dense(dev(A), p, mode, relu=relu, out_kind=out))
+        exp = oracle.dense(A, W, bias, shifts, mode, relu=relu, out=out)
+        assert np.array_equal(got, exp), (out, np.argwhere(got != exp)[:5])
+
+
+def test_dense_width_multiple_of_192(ops, oracle):
+    # 56 x 4 = 224 tiles of 128 x 192: the tile shape picked for widths such as 768 on 256 CUs
+    run_dense(ops, oracle, 7168, 128, 768, 'conv_even', seed=41)
+    run_dense(ops, oracle, 7100, 256, 768, 'symmetric_inf', a_dtype=np.uint8, out='int16', seed=42)
+
+
 def test_dense_nd_input_and_empty(ops, oracle):
     r = rng(6)
     A = gauss8(r, 30, (3, 5, 32))
