@@ -28,6 +28,7 @@ ROUNDING = {
     'conv_odd': 7,
 }
 KIND = {'int8': 0, 'uint8': 1, 'int16': 2, 'uint16': 3, 'int32': 4}
+FLOAT_FORMAT = {'bfloat16': 16, 'float32': 17}
 
 _i64, _i32, _vp, _sz = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
 
@@ -69,6 +70,13 @@ SIGNATURES = {
     'a4g_dense_i16': (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _i64, _i64, _i64, _i64, _vp]),
     'a4g_attention_i8': (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, ctypes.POINTER(ctypes.c_int64), _i32, _i32,
                                 _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp]),
+    'a4g_packed_ld_f': (_i64, [_i64, _i32]),
+    'a4g_pack_weights_f': (_i32, [_vp, _i32, _i64, _i64, _i64, _vp, _vp]),
+    'a4g_dense_f': (_i32, [_vp, _i32, _i64, _vp, _i64, _vp, _i32, _vp, _i64, _i64, _i64, _i64, _vp]),
+    'a4g_matmul_f_workspace_bytes': (_sz, [_i64, _i64, _i64, _i32, _i32]),
+    'a4g_matmul_f': (_i32, [_vp, _i32, _i64, _i64, _vp, _i64, _i64, _i32, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _sz,
+                            _vp]),
+    'a4g_add_f': (_i32, [_vp, _vp, _vp, _i64, _i32, _vp]),
 }
 
 _lib = None

@@ -2,8 +2,9 @@
 
 Mirrors the names and meaning of the reference's ``aie4ml.aie_types`` (RoundingMode /
 SaturationMode / QuantIntent / AIEDataType, src/aie4ml/aie_types.py:9-178) so that tensors built by the
-reference's frontends and tensors built here are interchangeable by attribute access. Only the integer
-formats the GPU kernels execute are modelled.
+reference's frontends and tensors built here are interchangeable by attribute access. The float side
+(FloatFormat / FloatIntent, src/aie4ml/aie_types.py:20-25, 85-98) covers the formats of the reference's
+float compute path.
 """
 
 from __future__ import annotations
@@ -29,6 +30,23 @@ class SaturationMode(Enum):
     SAT_SYM = 'SAT_SYM'
 
 
+class FloatFormat(Enum):
+    BF16 = 'bfloat16'
+    FP32 = 'float32'
+    FP8_E4M3 = 'fp8_e4m3'
+
+
+FLOAT_FORMATS = frozenset(f.value for f in FloatFormat)
+
+
+@dataclass(frozen=True)
+class FloatIntent:
+    """What a tensor of the float compute path holds (no fractional-bit bookkeeping)."""
+
+    width: int
+    format: FloatFormat
+
+
 @dataclass(frozen=True)
 class QuantIntent:
     """What a tensor is meant to hold: `width`-bit fixed point with `frac` fractional bits."""
@@ -41,8 +59,10 @@ class QuantIntent:
 
 
 _INT_WIDTHS = {'int8': 8, 'uint8': 8, 'int16': 16, 'uint16': 16, 'int32': 32, 'uint32': 32, 'int64': 64}
+_INT_WIDTHS.update({'bfloat16': 16, 'float32': 32, 'fp8_e4m3': 8, 'accfloat': 32})
 _C_TYPES = {'int8': 'int8_t', 'uint8': 'uint8_t', 'int16': 'int16_t', 'uint16': 'uint16_t', 'int32': 'int32_t',
-            'uint32': 'uint32_t', 'int64': 'int64_t'}
+            'uint32': 'uint32_t', 'int64': 'int64_t', 'bfloat16': 'bfloat16', 'float32': 'float', 'fp8_e4m3': 'float8',
+            'accfloat': 'accfloat'}
 
 
 @dataclass(frozen=True)
@@ -67,10 +87,14 @@ class AIEDataType:
         return not self.format.startswith('u')
 
     @property
+    def is_float(self) -> bool:
+        return self.format in FLOAT_FORMATS or self.format == 'accfloat'
+
+    @property
     def c_type(self) -> str:
         return _C_TYPES[self.format]
 
 
 def is_float_intent(precision) -> bool:
-    """True for the reference's FloatIntent (bf16 / fp32 / fp8 tensors): no GPU integer kernel takes them."""
+    """True for a FloatIntent, this package's or the reference's (bf16 / fp32 / fp8 tensors)."""
     return precision is not None and not hasattr(precision, 'frac') and hasattr(precision, 'format')

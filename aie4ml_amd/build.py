@@ -13,7 +13,7 @@ from pathlib import Path
 
 CSRC = Path(__file__).resolve().parent / 'csrc'
 LIB_PATH = Path(__file__).resolve().parent / 'libaie4ml_gfx950.so'
-SOURCES = ('abi.hip', 'rowops.hip', 'gemm.hip', 'mlp.hip', 'attention.hip', 'matmul_lean.hip', 'gemm_i16.hip')
+SOURCES = ('abi.hip', 'rowops.hip', 'gemm.hip', 'mlp.hip', 'attention.hip', 'matmul_lean.hip', 'gemm_i16.hip', 'gemm_float.hip')
 
 HIPCC_FLAGS = [
     '--offload-arch=gfx950',
@@ -39,7 +39,7 @@ def _stale() -> bool:
     if not LIB_PATH.exists():
         return True
     t = LIB_PATH.stat().st_mtime
-    deps = [CSRC / s for s in SOURCES] + [CSRC / 'common.hpp', CSRC / 'softmax_common.hpp', CSRC / 'matmul_lean.hpp', CSRC.parent.parent / 'include' / 'aie4ml_gfx950.h']
+    deps = [CSRC / s for s in SOURCES] + [CSRC / 'common.hpp', CSRC / 'softmax_common.hpp', CSRC / 'matmul_lean.hpp', CSRC / 'gemm_rs.hpp', CSRC.parent.parent / 'include' / 'aie4ml_gfx950.h']
     return any(d.stat().st_mtime > t for d in deps)
 
 

@@ -12,40 +12,11 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "gemm_rs.hpp"
 #include "matmul_lean.hpp"
 
-// Phase stamps for tuning builds (-DA4G_TIMING): thread 0 of every workgroup records the 100 MHz
-// real-time counter at a few points of the pipelined kernel. Compiled out of the library.
-#ifdef A4G_TIMING
-__device__ unsigned long long a4g_stamps[8 * 65536];
-#define A4G_STAMP(i)                                                                                  \
-    do {                                                                                              \
-        if (threadIdx.x == 0 && blockIdx.x < 65536) a4g_stamps[blockIdx.x * 8 + (i)] = __builtin_amdgcn_s_memrealtime(); \
-    } while (0)
-#else
-#define A4G_STAMP(i) \
-    do {             \
-    } while (0)
-#endif
 
 namespace a4g {
-
-struct GemmArgs {
-    const int8_t* A;
-    const int8_t* Bt;
-    void* C;
-    const int32_t* bias;    // [N] or null
-    const int32_t* colsum;  // [batch][N] or null (only read when a_unsigned)
-    const int32_t* shifts;  // device shifts, entry n * shift_stride; null -> the scalar `shift`
-    int64_t lda, stride_a, ldb, stride_b, ldc, stride_c, stride_colsum;
-    int M, N, K;
-    int shift;
-    int shift_stride;  // 0: one device scalar for every column, 1: per output channel
-    int a_unsigned;
-    int relu;
-    int out_kind;
-    int mode;
-};
 
 __device__ __forceinline__ int column_shift(const GemmArgs& g, int n) {
     const int s = g.shifts ? g.shifts[static_cast<int64_t>(n) * g.shift_stride] : g.shift;
@@ -266,34 +237,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_i8_nt_kernel(GemmA
 typedef __attribute__((address_space(1))) const void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
 
-struct TileCoord {
-    int m0, n0, batch;
-    bool valid;
-};
-
-// Workgroup -> tile mapping. Hardware deals consecutive workgroup ids round-robin over the 8 XCDs,
-// each with a private L2, so id % 8 names the XCD: every XCD gets one contiguous range of tiles, and
-// that range is ordered in bands of GROUP_M tile rows (row index fastest inside a band) so that the
-// tiles resident on an XCD at one time share both activation and weight panels.
-template <int BM, int BN>
-__device__ __forceinline__ TileCoord tile_coord(const GemmArgs& g) {
-    TileCoord tc;
-    const int tiles_m = (g.M + BM - 1) / BM;
-    const int tiles_n = (g.N + BN - 1) / BN;
-    const int tiles = tiles_m * tiles_n;
-    const int per_xcd = (tiles + 7) / 8;
-    const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
-    tc.valid = tile < tiles;
-    constexpr int GROUP_M = 8;
-    const int band = tile / (GROUP_M * tiles_n);
-    const int band_rows = min(GROUP_M, tiles_m - band * GROUP_M);
-    const int in_band = tile % (GROUP_M * tiles_n);
-    tc.m0 = (band * GROUP_M + in_band % max(band_rows, 1)) * BM;
-    tc.n0 = (in_band / max(band_rows, 1)) * BN;
-    tc.batch = blockIdx.y;
-    return tc;
-}
-
 // Per-column epilogue parameters, 5 ints per tile column in LDS: add (bias + 128*colsum), shift, and
 // the rounding constants c0, cx, bs of RoundCfg.
 template <int BN>
@@ -355,7 +298,6 @@ __device__ __forceinline__ void epilogue_store(const GemmArgs& g, const TileCoor
     const int lo = g.relu ? max(kind_lo(g.out_kind), 0) : kind_lo(g.out_kind), hi = kind_hi(g.out_kind);
     const int obytes = (g.out_kind == A4G_I16 || g.out_kind == A4G_U16) ? 2 : 1;
     const int cpitch = BN * obytes + 16;
-    int8_t* Cb = static_cast<int8_t*>(g.C) + tc.batch * g.stride_c * obytes;
     auto store_quad = [&](int ml, int nl, const int (&y)[4]) {
         if (obytes == 1) {
             *reinterpret_cast<unsigned*>(smem + ml * cpitch + nl) = pack4_bytes(y[0], y[1], y[2], y[3]);
@@ -446,24 +388,40 @@ __device__ __forceinline__ void epilogue_store(const GemmArgs& g, const TileCoor
     else requantise_fast(B2{}, std::true_type{});
     __syncthreads();
     A4G_STAMP(4);
-    const int cpr = BN * obytes / 16;  // 16-byte chunks per tile row
-    const bool vec_ok = ((g.ldc * obytes) % 16 == 0) && ((reinterpret_cast<uintptr_t>(Cb) & 15) == 0);
-    for (int idx = tid; idx < BM * cpr; idx += NT) {
-        const int row = idx / cpr, ch = idx % cpr;
-        const int m = tc.m0 + row;
-        const int nb = tc.n0 * obytes + ch * 16;  // byte column in the output row
-        if (m >= g.M || nb >= g.N * obytes) continue;
-        const v4i v = *reinterpret_cast<const v4i*>(smem + row * cpitch + ch * 16);
-        int8_t* dst = Cb + static_cast<int64_t>(m) * g.ldc * obytes + nb;
-        if (vec_ok && nb + 16 <= g.N * obytes) {
-            *reinterpret_cast<v4i*>(dst) = v;
-        } else {
-            const int nbytes = min(16, g.N * obytes - nb);
-            const int8_t* srcb = smem + row * cpitch + ch * 16;
-            for (int b = 0; b < nbytes; ++b) dst[b] = srcb[b];
-        }
-    }
+    store_tile_image<BM, BN, NT>(g, tc, smem, obytes, tid);
 }
+
+// What the shared pipelined kernel needs to know about int8 operands with an integer epilogue.
+template <bool A_UNSIGNED>
+struct I8Policy {
+    using acc_t = v16i;
+    static constexpr int MMAS = 1;
+    static constexpr bool FIX_A = A_UNSIGNED;
+    static constexpr int MAX_OUT_BYTES = 2;
+    template <int BN>
+    static constexpr int param_bytes() { return ColParams<BN>::BYTES; }
+    struct ColRegs {
+        int add, shift;
+    };
+    __device__ static __forceinline__ void fix_a(v4i& a) { a ^= static_cast<int>(0x80808080u); }
+    __device__ static __forceinline__ v16i mma(const v4i& b, const v4i& a, const v16i& c) {
+        return __builtin_amdgcn_mfma_i32_32x32x32_i8(b, a, c, 0, 0, 0);
+    }
+    template <int BN>
+    __device__ static __forceinline__ void fetch_params(const GemmArgs& g, const TileCoord& tc, int tid, ColRegs& r) {
+        fetch_col_params<BN, A_UNSIGNED>(g, tc, tid, r.add, r.shift);
+    }
+    template <int BN>
+    __device__ static __forceinline__ int park_params(const GemmArgs& g, int8_t* lds, int tid, const ColRegs& r) {
+        return park_col_params<BN>(g, ColParams<BN>(lds), tid, r.add, r.shift);
+    }
+    template <int BM, int BN, int WTM, int WTN, int NT>
+    __device__ static __forceinline__ void epilogue(const GemmArgs& g, const TileCoord& tc, v16i (&acc)[WTM / 32][WTN / 32],
+                                                    int8_t* smem, int8_t* lds_params, int path, int wm, int wn, int lane,
+                                                    int tid) {
+        epilogue_store<BM, BN, WTM, WTN, NT>(g, tc, acc, smem, ColParams<BN>(lds_params), path, wm, wn, lane, tid);
+    }
+};
 
 template <int BM, int BN, int BK_, int WAVES_M, int WAVES_N, int STAGES>
 struct DtlCfg {
@@ -500,7 +458,6 @@ __device__ __forceinline__ void wait_vmcnt() {
     // vmcnt[3:0] = simm16[3:0], vmcnt[5:4] = simm16[15:14], expcnt = [6:4], lgkmcnt = [11:8]
     __builtin_amdgcn_s_waitcnt(((N & 0xF) | ((N >> 4) << 14)) | (0x7 << 4) | (0xF << 8));
 }
-__device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xC07F); }
 
 template <int BM, int BN, int BK_, int WAVES_M, int WAVES_N, int STAGES, bool A_UNSIGNED>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_i8_dtl_kernel(GemmArgs g) {
@@ -640,196 +597,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_i8_dtl_kernel(Gemm
     epilogue_store<BM, BN, Cfg::WTM, Cfg::WTN, Cfg::NT>(g, tc, acc, smem, cp, round_path, wm, wn, lane, tid);
 }
 
-// -----------------------------------------------------------------------------------------------------
-// Register-staged pipelined MFMA kernel (K % 128 == 0) — the kernel for large GEMMs.
-//
-// Measured on this part, 16-byte global loads into registers that cover whole 128-byte lines sustain
-// about 1.75x the L2 throughput of the direct-to-LDS path, so tiles take the classic route: global ->
-// VGPR (one K tile ahead) -> ds_write_b128 -> LDS (two stages) -> ds_read_b128 -> MFMA. BK = 128 makes
-// every row segment one cache line. LDS layout and swizzle as in the direct-load kernel (BK = 128).
-//
-// Per K tile kt and wave, four K steps of TM*TN MFMAs each; the memory work is threaded between them:
-//   step 0: MFMAs(kt,0) | reads(kt,1) | ds_write of the registers holding tile kt+1 -> stage (kt+1)%2
-//   step 1: MFMAs(kt,1) | reads(kt,2) | global loads of tile kt+2 -> the same registers
-//   step 2: MFMAs(kt,2) | reads(kt,3)
-//   lgkmcnt(0); barrier        (tile kt+1 complete in LDS; nobody reads stage kt%2 after this point)
-//   step 3: MFMAs(kt,3) | reads(kt+1,0)
-// -----------------------------------------------------------------------------------------------------
-template <int BM, int BN, int WAVES_M, int WAVES_N>
-struct RsCfg {
-    static constexpr int BK = 128, CPR = 8, KSTEPS = 4;
-    static constexpr int NW = WAVES_M * WAVES_N;
-    static constexpr int NT = NW * 64;
-    static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
-    static constexpr int TM = WTM / 32, TN = WTN / 32;
-    static constexpr int ROWS_PER_PASS = NT / CPR;  // tile rows covered by one load per thread
-    static constexpr int A_LOADS = BM / ROWS_PER_PASS, B_LOADS = BN / ROWS_PER_PASS;
-    static constexpr int LOADS = A_LOADS + B_LOADS;
-    static constexpr int STAGE_BYTES = (BM + BN) * BK;
-    static constexpr int EPI_BYTES = BM * (2 * BN + 16);
-    static constexpr int PARAM_OFF = 2 * STAGE_BYTES > EPI_BYTES ? 2 * STAGE_BYTES : EPI_BYTES;
-    static constexpr int LDS_BYTES = PARAM_OFF + ColParams<BN>::BYTES;
-    static_assert(BM % ROWS_PER_PASS == 0 && BN % ROWS_PER_PASS == 0, "tile rows must divide over the threads");
-    static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be whole 32x32 MFMA blocks");
-    static_assert(TM * TN >= TM + TN, "one fragment read is issued behind each MFMA");
-    static constexpr int EPM = (LOADS + TM * TN - 1) / (TM * TN);  // staging writes / global loads behind each MFMA
-    static_assert(ROWS_PER_PASS % 16 == 0, "the swizzle term must not depend on the pass");
-    static_assert((BM + BN) * BK <= 65536, "ds_write immediate offsets are 16 bits");
-    static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
-};
-
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool A_UNSIGNED, bool EARLY = false>
-__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_i8_rs_kernel(GemmArgs g) {
-    using Cfg = RsCfg<BM, BN, WAVES_M, WAVES_N>;
-    constexpr int BK = Cfg::BK, KSTEPS = Cfg::KSTEPS;
-    extern __shared__ __attribute__((aligned(16))) int8_t smem[];
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
-
-    A4G_STAMP(0);
-    const TileCoord tc = tile_coord<BM, BN>(g);
-    if (!tc.valid) return;
-    const int m0 = tc.m0, n0 = tc.n0;
-
-    const ColParams<BN> cp(smem + Cfg::PARAM_OFF);
-    int col_add, col_shift;
-    fetch_col_params<BN, A_UNSIGNED>(g, tc, tid, col_add, col_shift);
-
-    // ---- global -> register staging: thread t owns chunk t%8 of rows t/8 + pass*ROWS_PER_PASS
-    const int lrow = tid / Cfg::CPR, lchunk = tid % Cfg::CPR;
-    const int8_t* __restrict__ Abase = g.A + tc.batch * g.stride_a + static_cast<int64_t>(m0) * g.lda;
-    const int8_t* __restrict__ Bbase = g.Bt + tc.batch * g.stride_b + static_cast<int64_t>(n0) * g.ldb;
-    int offa[Cfg::A_LOADS], offb[Cfg::B_LOADS];  // 32-bit offsets from the tile's first row
-#pragma unroll
-    for (int i = 0; i < Cfg::A_LOADS; ++i)
-        offa[i] = min(lrow + i * Cfg::ROWS_PER_PASS, g.M - 1 - m0) * static_cast<int>(g.lda) + lchunk * 16;
-#pragma unroll
-    for (int i = 0; i < Cfg::B_LOADS; ++i)
-        offb[i] = min(lrow + i * Cfg::ROWS_PER_PASS, g.N - 1 - n0) * static_cast<int>(g.ldb) + lchunk * 16;
-    // LDS slot of that chunk; the swizzle term (row>>1)&7 is the same for every pass
-    const int st_off = lrow * BK + ((lchunk ^ ((lrow >> 1) & 7)) * 16);
-
-    v4i ra[Cfg::A_LOADS], rb[Cfg::B_LOADS];
-    auto load_one = [&](int kt, int idx) {
-        if (idx < Cfg::A_LOADS) ra[idx] = *reinterpret_cast<const v4i*>(Abase + offa[idx] + static_cast<int64_t>(kt) * BK);
-        else rb[idx - Cfg::A_LOADS] = *reinterpret_cast<const v4i*>(Bbase + offb[idx - Cfg::A_LOADS] + static_cast<int64_t>(kt) * BK);
-    };
-    auto store_one = [&](int8_t* stage, int idx) {
-        if (idx < Cfg::A_LOADS) *reinterpret_cast<v4i*>(stage + st_off + idx * Cfg::ROWS_PER_PASS * BK) = ra[idx];
-        else *reinterpret_cast<v4i*>(stage + BM * BK + st_off + (idx - Cfg::A_LOADS) * Cfg::ROWS_PER_PASS * BK) = rb[idx - Cfg::A_LOADS];
-    };
-
-    const int ktiles = g.K / BK;
-#pragma unroll
-    for (int i = 0; i < Cfg::LOADS; ++i) load_one(0, i);
-
-    const int round_path = park_col_params<BN>(g, cp, tid, col_add, col_shift);
-    A4G_STAMP(1);
-
-    // ---- fragment addressing: row = lane%32 of the block, 16-byte half of the 32-wide K step = lane/32
-    const int frow = lane & 31;
-    int koff[KSTEPS];
-#pragma unroll
-    for (int kk = 0; kk < KSTEPS; ++kk) koff[kk] = ((kk * 2 + (lane >> 5)) ^ ((frow >> 1) & 7)) * 16;
-    const int a_off = (wm * Cfg::WTM + frow) * BK;
-    const int b_off = BM * BK + (wn * Cfg::WTN + frow) * BK;
-
-    v16i acc[Cfg::TM][Cfg::TN];
-#pragma unroll
-    for (int i = 0; i < Cfg::TM; ++i)
-#pragma unroll
-        for (int j = 0; j < Cfg::TN; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
-
-    v4i af[2][Cfg::TM], bf[2][Cfg::TN];
-    constexpr int NR = Cfg::TM + Cfg::TN, NM = Cfg::TM * Cfg::TN;
-    auto read_one = [&](int set, const int8_t* base, int kk, int idx) {
-        constexpr int TMIN = Cfg::TM < Cfg::TN ? Cfg::TM : Cfg::TN;
-        if (idx < 2 * TMIN) {
-            if (idx & 1) af[set][idx >> 1] = *reinterpret_cast<const v4i*>(base + a_off + (idx >> 1) * 32 * BK + koff[kk]);
-            else bf[set][idx >> 1] = *reinterpret_cast<const v4i*>(base + b_off + (idx >> 1) * 32 * BK + koff[kk]);
-        } else if (Cfg::TM > Cfg::TN) {
-            const int i = idx - TMIN;
-            af[set][i] = *reinterpret_cast<const v4i*>(base + a_off + i * 32 * BK + koff[kk]);
-        } else {
-            const int j = idx - TMIN;
-            bf[set][j] = *reinterpret_cast<const v4i*>(base + b_off + j * 32 * BK + koff[kk]);
-        }
-    };
-    // EXTRA: 0 = nothing, 1 = staging writes into `stage_w`, 2 = global loads of tile `kt_load`
-    auto step = [&](int cur, int nxt, const int8_t* next_base, int next_kk, auto extra_tag, int8_t* stage_w, int kt_load) {
-        constexpr int EXTRA = decltype(extra_tag)::value;
-#pragma unroll
-        for (int m = 0; m < NM; ++m) {
-            const int i = m / Cfg::TN, j = m % Cfg::TN;
-            if (A_UNSIGNED && j == 0) af[cur][i] ^= static_cast<int>(0x80808080u);
-            // operands swapped: the block's first index (registers) runs over n, lanes over m
-            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[cur][j], af[cur][i], acc[i][j], 0, 0, 0);
-            if (m < NR) read_one(nxt, next_base, next_kk, m);
-#pragma unroll
-            for (int e = m * Cfg::EPM; e < (m + 1) * Cfg::EPM && e < Cfg::LOADS; ++e) {
-                if (EXTRA == 1 || EXTRA == 3) store_one(stage_w, e);
-                if (EXTRA == 2 || EXTRA == 3) load_one(kt_load, e);
-            }
-        }
-#pragma unroll
-        for (int m = 0; m < NM; ++m) {
-            if (A_UNSIGNED && m % Cfg::TN == 0) __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // operand fix-up
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                      // one MFMA
-            if (m < NR) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                          // one LDS read
-#pragma unroll
-            for (int e = m * Cfg::EPM; e < (m + 1) * Cfg::EPM && e < Cfg::LOADS; ++e) {
-                if (EXTRA == 1 || EXTRA == 3) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // one LDS write
-                if (EXTRA == 2 || EXTRA == 3) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global load
-            }
-        }
-    };
-    using Tag0 = std::integral_constant<int, 0>;
-    using Tag1 = std::integral_constant<int, 1>;
-    using Tag2 = std::integral_constant<int, 2>;
-    using Tag3 = std::integral_constant<int, 3>;
-
-    // prologue: tile 0 -> stage 0, tile 1 -> registers, first fragments
-#pragma unroll
-    for (int i = 0; i < Cfg::LOADS; ++i) store_one(smem, i);
-#pragma unroll
-    for (int i = 0; i < Cfg::LOADS; ++i) load_one(min(1, ktiles - 1), i);
-    __syncthreads();
-#pragma unroll
-    for (int r = 0; r < NR; ++r) read_one(0, smem, 0, r);
-    A4G_STAMP(2);
-
-    for (int kt = 0; kt < ktiles; ++kt) {
-        int8_t* cur_base = smem + (kt & 1) * Cfg::STAGE_BYTES;
-        int8_t* nxt_base = smem + ((kt + 1) & 1) * Cfg::STAGE_BYTES;
-        if (EARLY) {
-            step(0, 1, cur_base, 1, Tag3{}, nxt_base, min(kt + 2, ktiles - 1));
-            __builtin_amdgcn_sched_barrier(0);
-            step(1, 0, cur_base, 2, Tag0{}, nullptr, 0);
-        } else {
-            step(0, 1, cur_base, 1, Tag1{}, nxt_base, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            step(1, 0, cur_base, 2, Tag2{}, nullptr, min(kt + 2, ktiles - 1));
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        step(0, 1, cur_base, 3, Tag0{}, nullptr, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        wait_lgkmcnt0();               // own staging writes and fragment reads have completed
-        __builtin_amdgcn_s_barrier();  // tile kt+1 complete in LDS; stage kt%2 is dead from here on
-        __builtin_amdgcn_sched_barrier(0);
-        step(1, 0, nxt_base, 0, Tag0{}, nullptr, 0);  // after the last tile this reads a stale stage: unused
-        __builtin_amdgcn_sched_barrier(0);
-    }
-    __syncthreads();  // every wave is past its last fragment read before the stages become the output image
-    A4G_STAMP(3);
-
-    epilogue_store<BM, BN, Cfg::WTM, Cfg::WTN, Cfg::NT>(g, tc, acc, smem, cp, round_path, wm, wn, lane, tid);
-    A4G_STAMP(5);
-}
 
 // -----------------------------------------------------------------------------------------------------
 // Generic kernel: any shape / pitch / alignment; one thread per output element.
@@ -938,19 +705,7 @@ static hipError_t launch_dtl_u(const GemmArgs& g, int batch, hipStream_t stream)
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool A_UNSIGNED, bool EARLY = false>
 static hipError_t launch_rs_u(const GemmArgs& g, int batch, hipStream_t stream) {
-    using Cfg = RsCfg<BM, BN, WAVES_M, WAVES_N>;
-    auto kern = gemm_i8_rs_kernel<BM, BN, WAVES_M, WAVES_N, A_UNSIGNED, EARLY>;
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                           Cfg::LDS_BYTES);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
-    const int tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
-    const int grid_x = (tiles + 7) / 8 * 8;
-    hipLaunchKernelGGL(kern, dim3(grid_x, batch), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, g);
-    return hipGetLastError();
+    return launch_rs_policy<I8Policy<A_UNSIGNED>, BM, BN, WAVES_M, WAVES_N, EARLY>(g, batch, stream);
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N>

@@ -1,0 +1,290 @@
+// Floating-point Dense / MatMul / Add: the reference's float compute path (bfloat16 or float32 operands,
+// float32 accumulation, result rounded to the operand format with round-to-nearest-even).
+//   Dense   templates/nnet_utils/dense_bias_relu/dense_bias_relu.cpp:66-166 with acc_scalar_t = accfloat
+//           (dense.py:105-127: shift 0, rounding conv_even, float32 bias as the accumulator's start value)
+//   MatMul  templates/nnet_utils/matmul/matmul.cpp:31-118, same accumulator
+//   Add     templates/nnet_utils/elementwise_add/elementwise_add.cpp:12-37
+// The tiled path is the shared pipelined MFMA kernel with a float policy: a 16-byte fragment is eight
+// bfloat16 (one v_mfma_f32_32x32x16_bf16) or four float32 (four v_mfma_f32_32x32x2_f32); the order of the
+// additions inside a dot product therefore differs from any sequential loop, as it does on the AI Engine.
+#include <algorithm>
+
+#include "gemm_rs.hpp"
+
+namespace a4g {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ unsigned f32_to_bf16_bits(float f) {  // round to nearest even; NaN stays NaN
+    const unsigned u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+__device__ __forceinline__ float bf16_bits_to_f32(unsigned h) { return __uint_as_float(h << 16); }
+
+__device__ __forceinline__ float load_float(const void* p, int64_t i, int fmt) {
+    return fmt == A4G_F32 ? static_cast<const float*>(p)[i] : bf16_bits_to_f32(static_cast<const uint16_t*>(p)[i]);
+}
+__device__ __forceinline__ void store_float(void* p, int64_t i, int fmt, float v) {
+    if (fmt == A4G_F32) static_cast<float*>(p)[i] = v;
+    else static_cast<uint16_t*>(p)[i] = static_cast<uint16_t>(f32_to_bf16_bits(v));
+}
+static inline int fmt_bytes(int fmt) { return fmt == A4G_F32 ? 4 : 2; }
+static inline bool fmt_ok(int fmt) { return fmt == A4G_F32 || fmt == A4G_BF16; }
+
+template <int FMT>
+struct FloatPolicy {
+    using acc_t = v16f;
+    static constexpr int ES = FMT == A4G_F32 ? 4 : 2;
+    static constexpr int MMAS = FMT == A4G_F32 ? 4 : 1;
+    static constexpr bool FIX_A = false;
+    static constexpr int MAX_OUT_BYTES = ES;
+    template <int BN>
+    static constexpr int param_bytes() { return 4 * BN; }
+    struct ColRegs {
+        float bias;
+    };
+    __device__ static __forceinline__ void fix_a(v4i&) {}
+    __device__ static __forceinline__ v16f mma(const v4i& b, const v4i& a, v16f c) {
+        if (FMT == A4G_F32) {
+            const v4f bf = __builtin_bit_cast(v4f, b), af = __builtin_bit_cast(v4f, a);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) c = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[t], af[t], c, 0, 0, 0);
+            return c;
+        }
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, b), __builtin_bit_cast(v8bf, a), c, 0, 0, 0);
+    }
+    template <int BN>
+    __device__ static __forceinline__ void fetch_params(const GemmArgs& g, const TileCoord& tc, int tid, ColRegs& r) {
+        r.bias = 0.f;
+        if (tid < BN && g.bias) r.bias = reinterpret_cast<const float*>(g.bias)[min(tc.n0 + tid, g.N - 1)];
+    }
+    template <int BN>
+    __device__ static __forceinline__ int park_params(const GemmArgs&, int8_t* lds, int tid, const ColRegs& r) {
+        if (tid < BN) reinterpret_cast<float*>(lds)[tid] = r.bias;
+        __syncthreads();
+        return 0;
+    }
+    // acc + bias -> ReLU -> operand format, through an LDS image of the tile, then whole-row stores
+    template <int BM, int BN, int WTM, int WTN, int NT>
+    __device__ static __forceinline__ void epilogue(const GemmArgs& g, const TileCoord& tc, v16f (&acc)[WTM / 32][WTN / 32],
+                                                    int8_t* smem, int8_t* lds_params, int, int wm, int wn, int lane, int tid) {
+        constexpr int TM = WTM / 32, TN = WTN / 32;
+        constexpr int cpitch = BN * ES + 16;
+        const float* bias = reinterpret_cast<const float*>(lds_params);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int nl = wn * WTN + j * 32 + 8 * q + 4 * (lane >> 5);  // column inside the tile
+                const v4f b4 = *reinterpret_cast<const v4f*>(bias + nl);
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+                    const int ml = wm * WTM + i * 32 + (lane & 31);
+                    float y[4];
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        y[t] = acc[i][j][q * 4 + t] + b4[t];
+                        if (g.relu) y[t] = fmaxf(y[t], 0.f);
+                    }
+                    if (FMT == A4G_F32) {
+                        const v4f o = {y[0], y[1], y[2], y[3]};
+                        *reinterpret_cast<v4f*>(smem + ml * cpitch + nl * 4) = o;
+                    } else {
+                        v2i o;
+                        o[0] = static_cast<int>(f32_to_bf16_bits(y[0]) | (f32_to_bf16_bits(y[1]) << 16));
+                        o[1] = static_cast<int>(f32_to_bf16_bits(y[2]) | (f32_to_bf16_bits(y[3]) << 16));
+                        *reinterpret_cast<v2i*>(smem + ml * cpitch + nl * 2) = o;
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        store_tile_image<BM, BN, NT>(g, tc, smem, ES, tid);
+    }
+};
+
+// Any shape / pitch / alignment: one thread per output element, float32 accumulation in k order starting
+// from the bias. lda / ldb / K here are in elements. trans_b == 1: B is [N][ldb]; 0: B is [K][ldb].
+struct FloatGenericArgs {
+    const void *A, *B;
+    void* C;
+    const float* bias;
+    int64_t lda, stride_a, ldb, stride_b, ldc, stride_c;
+    int M, N, K, relu, fmt, trans_b;
+};
+
+__global__ __launch_bounds__(256) void gemm_float_generic_kernel(FloatGenericArgs g) {
+    const int64_t total = static_cast<int64_t>(g.M) * g.N;
+    const int batch = blockIdx.y;
+    const int es = g.fmt == A4G_F32 ? 4 : 2;
+    const char* A = static_cast<const char*>(g.A) + batch * g.stride_a * es;
+    const char* B = static_cast<const char*>(g.B) + batch * g.stride_b * es;
+    char* C = static_cast<char*>(g.C) + batch * g.stride_c * es;
+    for (int64_t idx = blockIdx.x * 256ll + threadIdx.x; idx < total; idx += static_cast<int64_t>(gridDim.x) * 256) {
+        const int m = static_cast<int>(idx / g.N), n = static_cast<int>(idx % g.N);
+        float acc = g.bias ? g.bias[n] : 0.f;
+        for (int k = 0; k < g.K; ++k) {
+            const float a = load_float(A, static_cast<int64_t>(m) * g.lda + k, g.fmt);
+            const float b = g.trans_b ? load_float(B, static_cast<int64_t>(n) * g.ldb + k, g.fmt)
+                                      : load_float(B, static_cast<int64_t>(k) * g.ldb + n, g.fmt);
+            acc = fmaf(a, b, acc);
+        }
+        if (g.relu) acc = fmaxf(acc, 0.f);
+        store_float(C, static_cast<int64_t>(m) * g.ldc + n, g.fmt, acc);
+    }
+}
+
+// [K][ldb] -> [N][ldt] for 2- or 4-byte elements, 32 x 32 tiles through LDS; columns K..ldt-1 are zero filled.
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_elems_kernel(const T* __restrict__ B, int64_t ldb, int64_t stride_b,
+                                                              T* __restrict__ Bt, int64_t ldt, int64_t stride_t, int K, int N) {
+    __shared__ T tile[32][33];
+    const T* src = B + blockIdx.z * stride_b;
+    T* dst = Bt + blockIdx.z * stride_t;
+    const int k0 = blockIdx.x * 32, n0 = blockIdx.y * 32;
+    const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+    for (int r = ty; r < 32; r += 8) {
+        const int k = k0 + r, n = n0 + tx;
+        tile[r][tx] = (k < K && n < N) ? src[static_cast<int64_t>(k) * ldb + n] : T(0);
+    }
+    __syncthreads();
+    for (int r = ty; r < 32; r += 8) {
+        const int n = n0 + r, k = k0 + tx;
+        if (n < N && k < ldt) dst[static_cast<int64_t>(n) * ldt + k] = tile[tx][r];
+    }
+}
+
+__global__ __launch_bounds__(256) void add_float_kernel(const void* a, const void* b, void* out, int64_t n, int fmt) {
+    for (int64_t i = blockIdx.x * 256ll + threadIdx.x; i < n; i += static_cast<int64_t>(gridDim.x) * 256)
+        store_float(out, i, fmt, load_float(a, i, fmt) + load_float(b, i, fmt));
+}
+
+static inline int64_t round_up64(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
+
+// A is [batch][M][lda], Bt is [batch][N][ldb], both K-contiguous, element counts; C [batch][M][ldc].
+static hipError_t launch_float_nt(const void* A, int64_t lda, int64_t stride_a, const void* Bt, int64_t ldb, int64_t stride_b,
+                                  const float* bias, int relu, void* C, int64_t ldc, int64_t stride_c, int batch, int M, int N,
+                                  int K, int fmt, hipStream_t stream) {
+    const int es = fmt_bytes(fmt);
+    const bool tiled = (static_cast<int64_t>(K) * es) % 128 == 0 && (lda * es) % 16 == 0 && (ldb * es) % 16 == 0 &&
+                       (stride_a * es) % 16 == 0 && (stride_b * es) % 16 == 0 && aligned16(A) && aligned16(Bt);
+    if (!tiled) {
+        FloatGenericArgs ga{A, Bt, C, bias, lda, stride_a, ldb, stride_b, ldc, stride_c, M, N, K, relu, fmt, 1};
+        const int64_t total = static_cast<int64_t>(M) * N;
+        const int grid = static_cast<int>(std::min<int64_t>((total + 255) / 256, 256 * 32));
+        gemm_float_generic_kernel<<<dim3(grid, batch), 256, 0, stream>>>(ga);
+        return hipGetLastError();
+    }
+    GemmArgs g{};
+    g.A = static_cast<const int8_t*>(A);
+    g.Bt = static_cast<const int8_t*>(Bt);
+    g.C = C;
+    g.bias = reinterpret_cast<const int32_t*>(bias);
+    g.lda = lda * es;
+    g.stride_a = stride_a * es;
+    g.ldb = ldb * es;
+    g.stride_b = stride_b * es;
+    g.ldc = ldc;
+    g.stride_c = stride_c;
+    g.M = M;
+    g.N = N;
+    g.K = K * es;
+    g.relu = relu != 0;
+    if (fmt == A4G_F32) return launch_rs_policy<FloatPolicy<A4G_F32>, 128, 128, 2, 2>(g, batch, stream);
+    const int64_t tiles256 = static_cast<int64_t>((M + 255) / 256) * ((N + 255) / 256) * batch;
+    const int64_t rounds256 = (tiles256 + 255) / 256;
+    const bool big = M >= 256 && N >= 256 && K >= 256 && tiles256 * 100 >= rounds256 * 256 * 85;
+    if (big) return launch_rs_policy<FloatPolicy<A4G_BF16>, 256, 256, 2, 4, true>(g, batch, stream);
+    return launch_rs_policy<FloatPolicy<A4G_BF16>, 128, 128, 2, 2>(g, batch, stream);
+}
+
+template <typename T>
+static hipError_t launch_transpose(const void* B, int64_t ldb, int64_t stride_b, void* Bt, int64_t ldt, int64_t stride_t, int batch,
+                                   int K, int N, hipStream_t stream) {
+    dim3 grid(static_cast<unsigned>((ldt + 31) / 32), static_cast<unsigned>((N + 31) / 32), static_cast<unsigned>(batch));
+    transpose_elems_kernel<T><<<grid, 256, 0, stream>>>(static_cast<const T*>(B), ldb, stride_b, static_cast<T*>(Bt), ldt, stride_t, K,
+                                                        N);
+    return hipGetLastError();
+}
+
+}  // namespace a4g
+
+using namespace a4g;
+
+extern "C" int64_t a4g_packed_ld_f(int64_t K, int fmt) {
+    const int es = fmt == A4G_F32 ? 4 : 2;
+    return K <= 0 ? 16 / es : round_up64(K * es, 16) / es;
+}
+
+extern "C" int a4g_pack_weights_f(const void* W, int fmt, int64_t ldw, int64_t K, int64_t N, void* Wt, a4g_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const char* who = "a4g_pack_weights_f";
+    A4G_REQUIRE(fmt_ok(fmt), A4G_ERR_UNSUPPORTED, "%s: format %d is not bfloat16 / float32", who, fmt);
+    A4G_REQUIRE(W && Wt, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+    A4G_REQUIRE(K >= 1 && N >= 1 && K <= (1 << 24) && N <= (1 << 24) && ldw >= N, A4G_ERR_INVALID_ARGUMENT,
+                "%s: bad shape K=%lld N=%lld ldw=%lld", who, (long long)K, (long long)N, (long long)ldw);
+    const int64_t ldt = a4g_packed_ld_f(K, fmt);
+    const hipError_t e = fmt == A4G_F32 ? launch_transpose<uint32_t>(W, ldw, 0, Wt, ldt, 0, 1, (int)K, (int)N, stream)
+                                        : launch_transpose<uint16_t>(W, ldw, 0, Wt, ldt, 0, 1, (int)K, (int)N, stream);
+    return check_hip(e, who);
+}
+
+extern "C" int a4g_dense_f(const void* A, int fmt, int64_t lda, const void* Wt, int64_t ldwt, const float* bias, int relu, void* Y,
+                           int64_t ldy, int64_t M, int64_t N, int64_t K, a4g_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const char* who = "a4g_dense_f";
+    A4G_REQUIRE(fmt_ok(fmt), A4G_ERR_UNSUPPORTED, "%s: format %d is not bfloat16 / float32", who, fmt);
+    A4G_REQUIRE(M >= 0 && N >= 1 && K >= 1 && M <= INT32_MAX && N <= (1 << 24) && K <= (1 << 24), A4G_ERR_INVALID_ARGUMENT,
+                "%s: bad shape M=%lld N=%lld K=%lld", who, (long long)M, (long long)N, (long long)K);
+    A4G_REQUIRE(lda >= K && ldy >= N && ldwt >= K, A4G_ERR_INVALID_ARGUMENT, "%s: pitch smaller than the row", who);
+    if (M == 0) return A4G_OK;
+    A4G_REQUIRE(A && Wt && Y, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+    return check_hip(launch_float_nt(A, lda, 0, Wt, ldwt, 0, bias, relu, Y, ldy, 0, 1, (int)M, (int)N, (int)K, fmt, stream), who);
+}
+
+extern "C" size_t a4g_matmul_f_workspace_bytes(int64_t batch, int64_t N, int64_t K, int trans_b, int fmt) {
+    if (trans_b || batch <= 0 || N <= 0 || K <= 0) return 0;
+    return static_cast<size_t>(batch) * N * a4g_packed_ld_f(K, fmt) * (fmt == A4G_F32 ? 4 : 2);
+}
+
+extern "C" int a4g_matmul_f(const void* A, int fmt, int64_t lda, int64_t stride_a, const void* B, int64_t ldb, int64_t stride_b,
+                            int trans_b, void* C, int64_t ldc, int64_t stride_c, int64_t batch, int64_t M, int64_t N, int64_t K,
+                            void* workspace, size_t workspace_bytes, a4g_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const char* who = "a4g_matmul_f";
+    A4G_REQUIRE(fmt_ok(fmt), A4G_ERR_UNSUPPORTED, "%s: format %d is not bfloat16 / float32", who, fmt);
+    A4G_REQUIRE(batch >= 0 && batch <= 65535 && M >= 0 && N >= 1 && K >= 1 && M <= INT32_MAX && N <= (1 << 24) && K <= (1 << 24),
+                A4G_ERR_INVALID_ARGUMENT, "%s: bad shape batch=%lld M=%lld N=%lld K=%lld", who, (long long)batch, (long long)M,
+                (long long)N, (long long)K);
+    A4G_REQUIRE(lda >= K && ldc >= N && ldb >= (trans_b ? K : N), A4G_ERR_INVALID_ARGUMENT, "%s: pitch smaller than the row", who);
+    if (M == 0 || batch == 0) return A4G_OK;
+    A4G_REQUIRE(A && B && C, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+    if (trans_b)
+        return check_hip(launch_float_nt(A, lda, stride_a, B, ldb, stride_b, nullptr, 0, C, ldc, stride_c, (int)batch, (int)M, (int)N,
+                                         (int)K, fmt, stream), who);
+    const size_t need = a4g_matmul_f_workspace_bytes(batch, N, K, 0, fmt);
+    A4G_REQUIRE(workspace && workspace_bytes >= need && aligned16(workspace), A4G_ERR_WORKSPACE,
+                "%s: needs a 16-byte aligned workspace of %zu bytes (a4g_matmul_f_workspace_bytes)", who, need);
+    const int64_t ldt = a4g_packed_ld_f(K, fmt);
+    hipError_t e = fmt == A4G_F32
+                       ? launch_transpose<uint32_t>(B, ldb, stride_b, workspace, ldt, N * ldt, (int)batch, (int)K, (int)N, stream)
+                       : launch_transpose<uint16_t>(B, ldb, stride_b, workspace, ldt, N * ldt, (int)batch, (int)K, (int)N, stream);
+    if (e != hipSuccess) return check_hip(e, who);
+    return check_hip(launch_float_nt(A, lda, stride_a, workspace, ldt, N * ldt, nullptr, 0, C, ldc, stride_c, (int)batch, (int)M, (int)N,
+                                     (int)K, fmt, stream), who);
+}
+
+extern "C" int a4g_add_f(const void* a, const void* b, void* out, int64_t n, int fmt, a4g_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const char* who = "a4g_add_f";
+    A4G_REQUIRE(fmt_ok(fmt), A4G_ERR_UNSUPPORTED, "%s: format %d is not bfloat16 / float32", who, fmt);
+    A4G_REQUIRE(n >= 0, A4G_ERR_INVALID_ARGUMENT, "%s: negative length", who);
+    if (n == 0) return A4G_OK;
+    A4G_REQUIRE(a && b && out, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+    const int grid = static_cast<int>(std::min<int64_t>((n + 255) / 256, 256 * 16));
+    add_float_kernel<<<grid, 256, 0, stream>>>(a, b, out, n, fmt);
+    return check_hip(hipGetLastError(), who);
+}

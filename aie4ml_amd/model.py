@@ -9,7 +9,9 @@ I/O contract of predict() (src/aie4ml/simulation.py:157-196, 248-269; model.py:1
     overflow-handled with its saturation mode; integer arrays pass through with a dtype cast;
     quantize_in=False requires integer arrays;
   * the result is int64 raw values, or float64 value / 2^frac with dequantize_out=True; a leading
-    iteration axis is folded into the batch axis; one output -> ndarray, several -> dict by name.
+    iteration axis is folded into the batch axis; one output -> ndarray, several -> dict by name;
+  * tensors of the float compute path (FloatIntent) take float32 arrays as they are (simulation.py:184-185)
+    and come back as float64 (simulation.py:235, 253-254), whatever the two flags say.
 """
 
 from __future__ import annotations
@@ -20,6 +22,7 @@ from typing import Any, Dict, List, Optional
 import numpy as np
 
 from .ir import CONTEXT_ATTR, BackendContext, get_backend_context, input_tensor_for_role
+from .op_impls.float_ops import pack_as_float, to_device_float
 from .op_impls.precision import resolve_exact_storage_dtype
 from .passes import GPU_PIPELINE, run_aie_passes
 from .quant_utils import dequantize_output, dtype_for_precision, quantize_input
@@ -88,7 +91,9 @@ class GPUModel:
                 raise ValueError(f'{t.name}: expected shape {expected}, (1, *{expected}) or ({iterations}, *{expected}); '
                                  f'got {tuple(arr.shape)}')
             dtype = self._io_dtype(t, 'input')
-            if quantize:
+            if dtype.is_float:
+                prepared[t.name] = np.asarray(arr, dtype=np.float32)  # simulation.py:184-185
+            elif quantize:
                 prepared[t.name] = quantize_input(arr, dtype)
             else:
                 if not np.issubdtype(arr.dtype, np.integer):
@@ -109,14 +114,23 @@ class GPUModel:
         dev_inputs = {}
         for name, arr in prepared.items():
             merged = arr.reshape((arr.shape[0] * arr.shape[1],) + tuple(arr.shape[2:])) if arr.ndim >= 2 else arr
-            dev_inputs[name] = torch.from_numpy(np.ascontiguousarray(merged)).cuda()
+            dtype = self._io_dtype(graph.tensors[name], 'input')
+            if dtype.is_float:
+                # float32 values enter the device format the way parameters do (pack_as_float truncates to bfloat16)
+                dev_inputs[name] = to_device_float(pack_as_float(merged, dtype.format), dtype.format)
+            else:
+                dev_inputs[name] = torch.from_numpy(np.ascontiguousarray(merged)).cuda()
         iters = next(iter(prepared.values())).shape[0]
         dev_out = self.execute(dev_inputs, batch_scale=iters)
         torch.cuda.synchronize()
         results = {}
         for t in graph.graph_outputs():
+            dtype = self._io_dtype(t, 'output')
+            if dtype.is_float:
+                results[t.name] = dev_out[t.name].float().cpu().numpy().astype(np.float64)  # simulation.py:235, 253-254
+                continue
             raw = dev_out[t.name].cpu().numpy().astype(np.int64)
-            results[t.name] = dequantize_output(raw, self._io_dtype(t, 'output').frac) if dequantize_out else raw
+            results[t.name] = dequantize_output(raw, dtype.frac) if dequantize_out else raw
         if len(results) == 1:
             return next(iter(results.values()))
         return results

@@ -39,7 +39,10 @@ class AddFamilyResolver(FamilyResolver):
         if any(t.precision is None for t in tensors):
             raise ValueError(f'{node.name}: missing precision metadata for add.')
         if any(is_float_intent(t.precision) for t in tensors):
-            raise NotImplementedError(f'{node.name}: float Add has no GPU variant.')
+            # float Add: all three tensors float (elementwise/resolver.py:26-28); the float variant checks formats
+            if not all(is_float_intent(t.precision) for t in tensors):
+                raise ValueError(f'{node.name}: elementwise Add requires lhs/rhs/output to use the same storage type.')
+            return
         kinds = [resolve_exact_storage_dtype(t.precision, namespace=ns, layer_name=node.name)
                  for t, ns in zip(tensors, ('lhs', 'rhs', 'output'))]
         if kinds[0] != kinds[1] or kinds[0] != kinds[2]:
@@ -52,8 +55,9 @@ class AddGpuVariant(OpImplVariant):
     op_type = 'add'
     plevel = 10
 
-    def matches(self, _node, device) -> bool:
-        return is_gpu(device)
+    def matches(self, node, device) -> bool:
+        lhs = input_tensor_for_role(node, 'lhs')
+        return is_gpu(device) and not is_float_intent(lhs.precision)
 
     def resolve(self, node, _device, _directives=None) -> AddConfig:
         lhs, rhs = input_tensor_for_role(node, 'lhs'), input_tensor_for_role(node, 'rhs')

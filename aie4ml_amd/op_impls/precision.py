@@ -39,8 +39,17 @@ def to_quant_intent(precision: Any) -> QuantIntent:
                        rounding=_mode_key(precision.rounding), saturation=precision.saturation)
 
 
+def float_format_name(precision: Any) -> str:
+    """'bfloat16' / 'float32' / 'fp8_e4m3' of a FloatIntent (this package's or the reference's enum)."""
+    fmt = precision.format
+    return str(getattr(fmt, 'value', fmt))
+
+
 def resolve_exact_storage_dtype(precision: Any, *, namespace: str, layer_name: str) -> AIEDataType:
-    """Round the intent's width up to a storage width (4 -> 8, 8, 16, 32), keeping signedness and frac."""
+    """Round the intent's width up to a storage width (4 -> 8, 8, 16, 32), keeping signedness and frac;
+    a FloatIntent maps to its own format (precision.py:64-71)."""
+    if is_float_intent(precision):
+        return AIEDataType(format=float_format_name(precision))
     q = to_quant_intent(precision)
     if q.width <= 0:
         raise ValueError(f'{layer_name}: invalid {namespace} width {q.width}.')

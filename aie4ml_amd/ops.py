@@ -325,3 +325,112 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, logit_shift: in
                                        int(softmax.get('inv_shift', 15)), int(bool(softmax.get('use_clb', False))),
                                        int(out_shift), _mode(out_rounding), _stream()))
     return out
+
+
+# ---- floating-point compute path (bfloat16 / float32 operands, float32 accumulation) ---------------------------
+
+_TORCH_FLOAT = {torch.bfloat16: 16, torch.float32: 17}
+
+
+def _float_format(t: torch.Tensor, name: str) -> int:
+    try:
+        return _TORCH_FLOAT[t.dtype]
+    except KeyError:
+        raise NotImplementedError(f'{name}: the float path takes bfloat16 or float32 tensors, got {t.dtype}') from None
+
+
+@dataclass
+class PackedDenseFloat:
+    """Device-resident float Dense parameters: weights [N, ldwt] with the reduction axis contiguous."""
+
+    wt: torch.Tensor
+    bias: Optional[torch.Tensor]  # [N] float32 or None
+    K: int
+    N: int
+
+    @property
+    def ldwt(self) -> int:
+        return int(self.wt.shape[1])
+
+
+def pack_dense_float(weight: torch.Tensor, bias: Optional[torch.Tensor]) -> PackedDenseFloat:
+    """weight: logical [K, N] bfloat16 / float32 on the device; bias: [N] (kept in float32) or None."""
+    _dev(weight, 'weight')
+    fmt = _float_format(weight, 'weight')
+    if weight.dim() != 2:
+        raise ValueError('weight matrix must be a rank-2 tensor')
+    weight = weight.contiguous()
+    K, N = int(weight.shape[0]), int(weight.shape[1])
+    L = _lib.load()
+    wt = torch.empty((N, int(L.a4g_packed_ld_f(K, fmt))), dtype=weight.dtype, device=weight.device)
+    check(L.a4g_pack_weights_f(_ptr(weight), fmt, N, K, N, _ptr(wt), _stream()))
+    if bias is not None:
+        bias = _dev(bias, 'bias').to(torch.float32).contiguous()
+        if bias.numel() != N:
+            raise ValueError(f'dense bias requires exactly {N} elements, got {bias.numel()}.')
+    return PackedDenseFloat(wt=wt, bias=bias, K=K, N=N)
+
+
+def dense_float(x: torch.Tensor, p: PackedDenseFloat, relu: bool = False, out: Optional[torch.Tensor] = None):
+    """y = fmt(relu?(bias + x @ W)) with float32 accumulation; x: [..., K] in the weights' format."""
+    x2 = _rows2d(x, 'x')
+    fmt = _float_format(x2, 'x')
+    if x2.dtype != p.wt.dtype:
+        raise ValueError(f'float dense requires lhs/rhs/output to share float precision, got {x2.dtype} and {p.wt.dtype}.')
+    if x2.shape[1] != p.K:
+        raise ValueError(f'dense input has {x2.shape[1]} features, weights expect {p.K}')
+    M = int(x2.shape[0])
+    if out is None:
+        out = torch.empty(tuple(x.shape[:-1]) + (p.N,), dtype=x.dtype, device=x.device)
+    y2 = out.reshape(-1, p.N)
+    check(_lib.load().a4g_dense_f(_ptr(x2), fmt, x2.stride(0) if M > 0 else p.K, _ptr(p.wt), p.ldwt, _ptr(p.bias),
+                                  int(bool(relu)), _ptr(y2), y2.stride(0) if M > 0 else p.N, M, p.N, p.K, _stream()))
+    return out
+
+
+def matmul_float(a: torch.Tensor, b: torch.Tensor, trans_b: bool = False, out: Optional[torch.Tensor] = None,
+                 workspace: Optional[torch.Tensor] = None):
+    """Batched float MatMul. a: [..., M, K]; b: [..., K, N], or [..., N, K] when ``trans_b``."""
+    _dev(a, 'a'), _dev(b, 'b')
+    fmt = _float_format(a, 'a')
+    if a.dtype != b.dtype:
+        raise ValueError(f'float matmul requires lhs/rhs/output to share float precision, got {a.dtype} and {b.dtype}.')
+    if a.dim() < 2 or b.dim() < 2:
+        raise ValueError('matmul operands need rank >= 2')
+    a, b = a.contiguous(), b.contiguous()
+    M, K = int(a.shape[-2]), int(a.shape[-1])
+    N = int(b.shape[-2] if trans_b else b.shape[-1])
+    Kb = int(b.shape[-1] if trans_b else b.shape[-2])
+    if K != Kb:
+        raise ValueError(f'matmul reduction extents differ: {K} vs {Kb}')
+    lead = tuple(a.shape[:-2])
+    if tuple(b.shape[:-2]) != lead:
+        raise ValueError(f'matmul leading axes differ: {lead} vs {tuple(b.shape[:-2])}')
+    batch = 1
+    for d in lead:
+        batch *= int(d)
+    if out is None:
+        out = torch.empty(lead + (M, N), dtype=a.dtype, device=a.device)
+    L = _lib.load()
+    need = int(L.a4g_matmul_f_workspace_bytes(batch, N, K, int(trans_b), fmt))
+    if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
+        workspace = torch.empty((need,), dtype=torch.uint8, device=a.device)
+    ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    check(L.a4g_matmul_f(_ptr(a), fmt, K, M * K, _ptr(b), int(b.shape[-1]), K * N, int(bool(trans_b)), _ptr(out), N, M * N,
+                         batch, M, N, K, _ptr(workspace), ws_bytes, _stream()))
+    return out
+
+
+def add_float(a: torch.Tensor, b: torch.Tensor, out: Optional[torch.Tensor] = None):
+    """Elementwise a + b in float32, rounded to the operands' format."""
+    _dev(a, 'a'), _dev(b, 'b')
+    if a.shape != b.shape:
+        raise ValueError(f'elementwise Add requires exact-shape inputs, got {tuple(a.shape)} and {tuple(b.shape)}.')
+    if a.dtype != b.dtype:
+        raise ValueError('elementwise Add requires lhs/rhs/output to use the same storage type.')
+    fmt = _float_format(a, 'a')
+    a, b = a.contiguous(), b.contiguous()
+    if out is None:
+        out = torch.empty_like(a)
+    check(_lib.load().a4g_add_f(_ptr(a), _ptr(b), _ptr(out), a.numel(), fmt, _stream()))
+    return out

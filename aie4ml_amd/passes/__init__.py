@@ -4,7 +4,8 @@ The fold / fuse passes decide what each kernel fuses and restate the reference's
 names (src/aie4ml/passes/fold_bias.py, fold_scale.py, fuse_activation.py, fold_views.py); Resolve and
 PackKernelArtifacts restate passes/resolve.py:48-95 and passes/pack.py:20-37 without the AIE contract /
 staging propagation. Everything the reference runs after packing (transport, placement, memory plan)
-is AIE-physical and has no counterpart here. PlanGpuFusion is the GPU-only addition.
+is AIE-physical and has no counterpart here. PlanGpuFusion is the GPU-only addition; ForceFloatMode restates
+passes/force_float_mode.py.
 """
 
 from __future__ import annotations
@@ -13,6 +14,7 @@ from typing import Iterable
 
 import numpy as np
 
+from ..aie_types import FloatFormat, FloatIntent, is_float_intent
 from ..ir import TraitInstance, get_backend_context, input_tensor_for_role
 from ..op_impls import get_family_resolver_registry
 from ..op_impls.base import OpImplVariant
@@ -31,6 +33,31 @@ def run_aie_passes(ctx, passes: Iterable[AIEPass]) -> None:
     ctx.ir.logical.verify()
     for p in passes:
         p.transform(ctx)
+
+
+class ForceFloatMode(AIEPass):
+    """Replace every QuantIntent of the logical IR with a FloatIntent when the run configuration names a
+    ComputeDtype ('bfloat16', 'float32' or 'float'): the reference's way of exercising its float path on a
+    quantised model (src/aie4ml/passes/force_float_mode.py:15-46)."""
+
+    name = 'force_float_mode'
+    FORMATS = {'bfloat16': (FloatFormat.BF16, 16), 'float32': (FloatFormat.FP32, 32), 'float': (FloatFormat.FP32, 32)}
+
+    def transform(self, model_or_ctx) -> bool:
+        ctx = get_backend_context(model_or_ctx)
+        fmt_str = str(ctx.config.get('ComputeDtype') or '').lower()
+        if not fmt_str:
+            return False
+        if fmt_str not in self.FORMATS:
+            raise ValueError(f'ComputeDtype={fmt_str!r} is not recognised. Use one of: {list(self.FORMATS)}')
+        fmt, width = self.FORMATS[fmt_str]
+        intent = FloatIntent(width=width, format=fmt)
+        changed = False
+        for tv in ctx.ir.logical.tensors.values():
+            if tv.precision is not None and not is_float_intent(tv.precision):
+                tv.precision = intent
+                changed = True
+        return changed
 
 
 class FoldBias(AIEPass):
@@ -454,6 +481,8 @@ class PlanGpuFusion(AIEPass):
     def _fits(self, chain, execution) -> bool:
         if len(chain) > 8:
             return False
+        if any(execution.get(n.name).config.accumulator_tag != 'acc32' for n in chain):
+            return False  # the fused MLP kernel is the int8 one
         total, mode = 0, None
         for i, n in enumerate(chain):
             cfg = execution.get(n.name).config
@@ -472,4 +501,4 @@ class PlanGpuFusion(AIEPass):
         return total <= self.MLP_MAX_WEIGHT_BYTES
 
 
-GPU_PIPELINE = (FoldBias, FoldScale, FuseActivationCasts, FoldViewOps, Resolve, PackKernelArtifacts, PlanGpuFusion)
+GPU_PIPELINE = (ForceFloatMode, FoldBias, FoldScale, FuseActivationCasts, FoldViewOps, Resolve, PackKernelArtifacts, PlanGpuFusion)

@@ -6,7 +6,7 @@ Default workload: the single quantized Dense of the baseline configuration
 saturate to int8, fused ReLU). One step = one pass of the operator over the whole synthetic batch,
 inputs already resident in HBM. Prints ONE JSON line.
 
-Other workloads (--workload c2_dense_i16 | c1_mlp | c3_softmax_exp | c3_softmax_hccs | c3_qk | c3_pv |
+Other workloads (--workload c2_dense_i16 | c2_dense_bf16 | c1_mlp | c3_softmax_exp | c3_softmax_hccs | c3_qk | c3_pv |
 c3_attention_exp | c3_attention_hccs | c4_add_layernorm | c4_layernorm | c4_add | c5_encoder) print the same line for that operator or graph;
 --workload calib_copy runs a plain 256 MiB elementwise copy, the known-size kernel the HBM traffic
 counters are scaled against.
@@ -27,6 +27,7 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, TOP/s
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, TFLOP/s
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
 
 # HBM bytes per launch of each workload's dominant kernel, from hardware counters (FETCH_SIZE and
@@ -119,6 +120,7 @@ def main():
     extra = {}
     cpu_fn = None
     cpu_samples = None
+    peak_mfma, mfma_unit = PEAK_INT8_TOPS, 'TOP/s'
 
     if wl == 'c2_dense':
         M, K, N = 8192, 4096, 4096
@@ -142,7 +144,7 @@ def main():
         cpu_fn = lambda: oracle.dense(A[:sample_rows], W, bias, shifts, 'conv_even', relu=True)  # noqa: E731
         cpu_work = 2.0 * sample_rows * N * K
         metric, unit = 'int8_dense_tops', 'TOP/s'
-        kernel = 'gemm_i8_rs_kernel'
+        kernel = 'gemm_rs_kernel'
     elif wl == 'c2_dense_i16':
         # the (16, 8) width combination on the C2 shape: int16 activations, int8 weights, int16 output
         M, K, N = 8192, 4096, 4096
@@ -168,6 +170,37 @@ def main():
         cpu_work = 2.0 * sample_rows * N * K
         metric, unit = 'int16x8_dense_tops', 'TOP/s'
         kernel = 'gemm_i16i8_kernel'
+    elif wl == 'c2_dense_bf16':
+        # the reference's float compute path on the C2 shape: bfloat16 operands, float32 accumulation and bias
+        M, K, N = 8192, 4096, 4096
+        r = np.random.default_rng(23)
+        A = oracle.bf16_truncate(r.normal(0, 1.0, (M, K)).astype(np.float32))
+        W = oracle.bf16_truncate(r.normal(0, 0.02, (K, N)).astype(np.float32))
+        bias = r.normal(0, 0.1, N).astype(np.float32)
+        p = ops.pack_dense_float(torch.from_numpy(W).cuda().to(torch.bfloat16), torch.from_numpy(bias).cuda())
+        dA = torch.from_numpy(A).cuda().to(torch.bfloat16)
+        out = torch.empty((M, N), dtype=torch.bfloat16, device='cuda')
+        fn = lambda: ops.dense_float(dA, p, relu=True, out=out)  # noqa: E731
+        fn()
+        rows = r.choice(M, 64, replace=False)
+        exp = oracle.dense_float(A[rows], W, bias, relu=True, fmt='bfloat16')
+        torch.cuda.synchronize()
+        got = out[torch.from_numpy(rows).cuda()].float().cpu().numpy()
+        # float path: no bit-exactness across summation orders; the reference's own tolerance (rtol 1e-2, atol 5e-2)
+        bit_exact = bool(np.allclose(got, exp, rtol=1e-2, atol=5e-2))
+        extra['parity'] = 'within rtol 1e-2 / atol 5e-2 of the exact-accumulation oracle (float path)'
+        extra['max_abs_err'] = float(np.max(np.abs(got - exp)))
+        work, bound = 2.0 * M * N * K, 'mfma'
+        peak_mfma, mfma_unit = PEAK_BF16_TFLOPS, 'TFLOP/s'
+        samples = M
+        config = {'workload': 'c2_dense_bf16: Dense 8192x4096 -> 4096, bfloat16 operands, float32 accumulate + bias, ReLU, '
+                              'bfloat16 out (round to nearest even)'}
+        sample_rows = 256
+        cpu_desc = f'oracle float Dense (float64 numpy matmul) on the first {sample_rows} of {M} rows, scaled per op'
+        cpu_fn = lambda: oracle.dense_float(A[:sample_rows], W, bias, relu=True, fmt='bfloat16')  # noqa: E731
+        cpu_work = 2.0 * sample_rows * N * K
+        metric, unit = 'bf16_dense_tflops', 'TFLOP/s'
+        kernel = 'gemm_rs_kernel'
     elif wl == 'c1_mlp':
         x, layers = workloads.c1_mlp(1024)
         specs = [ops.MlpLayerSpec(ops.pack_dense(dev(Wl), dev(b), s), s, relu, o) for (Wl, b, s, relu, o) in layers]
@@ -257,7 +290,7 @@ def main():
             cpu_fn = lambda: oracle.matmul(pl, v[0, :4], prm['pv_shift'], 'conv_even')  # noqa: E731
             cpu_work = bytes_ * 4 / (Bt * H)
             cpu_desc = 'oracle MatMul (uint8 x int8) on 4 of 512 (batch, head) slices'
-            kernel = 'gemm_i8_rs_kernel'
+            kernel = 'gemm_rs_kernel'
         else:
             out = torch.empty(logits.shape, dtype=torch.uint8, device='cuda')
             hc = prm['hccs']
@@ -362,8 +395,8 @@ def main():
     ms = max(ms_wall, ms_ev)
     if bound == 'mfma':
         achieved = work / (ms_ev * 1e-3) / 1e12
-        roof = {'bound': 'mfma', 'achieved': round(achieved, 3), 'peak': PEAK_INT8_TOPS, 'unit': 'TOP/s',
-                'frac': round(achieved / PEAK_INT8_TOPS, 4), 'traffic': MEASURED_TRAFFIC.get(wl), 'kernel': kernel,
+        roof = {'bound': 'mfma', 'achieved': round(achieved, 3), 'peak': peak_mfma, 'unit': mfma_unit,
+                'frac': round(achieved / peak_mfma, 4), 'traffic': MEASURED_TRAFFIC.get(wl), 'kernel': kernel,
                 'kernel_ms': round(ms_ev, 5)}
     else:
         achieved = work / (ms_ev * 1e-3) / 1e9
@@ -371,7 +404,7 @@ def main():
                 'frac': round(achieved / PEAK_HBM_GBS, 4), 'traffic': MEASURED_TRAFFIC.get(wl), 'kernel': kernel,
                 'kernel_ms': round(ms_ev, 5)}
 
-    if unit == 'TOP/s':
+    if unit in ('TOP/s', 'TFLOP/s'):
         value = work / (ms * 1e-3) / 1e12
     elif unit == 'GB/s':
         value = work / (ms * 1e-3) / 1e9
@@ -381,7 +414,7 @@ def main():
     cpu = None
     if cpu_fn is not None and not args.no_cpu_baseline:
         t = _time_cpu(cpu_fn)
-        if unit == 'TOP/s':
+        if unit in ('TOP/s', 'TFLOP/s'):
             v = cpu_work / t / 1e12
         elif unit == 'GB/s':
             v = cpu_work / t / 1e9
@@ -393,7 +426,7 @@ def main():
     line = {
         'metric': metric, 'value': float(f'{value:.6g}'), 'unit': unit, 'n_gpus': 1, 'steps': args.steps,
         'warmup': args.warmup, 'ms_per_step': round(ms, 5), 'higher_is_better': True, 'scaling': 'weak',
-        'vs_baseline': None, 'dtype': 'int16' if wl == 'c2_dense_i16' else 'int8', 'data': 'synthetic', 'config': config,
+        'vs_baseline': None, 'dtype': {'c2_dense_i16': 'int16', 'c2_dense_bf16': 'bf16'}.get(wl, 'int8'), 'data': 'synthetic', 'config': config,
         'samples_per_s': float(f'{samples / (ms * 1e-3):.6g}'), 'bit_exact': bit_exact,
         'roofline': roof, 'cpu_baseline': cpu, 'launch': 'hip_graph' if graphed else 'eager',
     }

@@ -205,6 +205,35 @@ A4G_API int a4g_attention_i8(const int8_t* Q, const int8_t* K, const int8_t* V, 
                      int logit_round_mode, int softmax_kind, int exp_kq, int hccs_B, int hccs_S, int hccs_Dmax,
                      int inv_shift, int use_clb, int out_shift, int out_round_mode, a4g_stream_t stream);
 
+/* ---- Floating-point compute path ------------------------------------------------------------------
+ * The reference's float mode (FloatIntent tensors, passes/force_float_mode.py): bfloat16 or float32
+ * operands, float32 accumulation (acc_scalar_t = accfloat), results rounded to the operand format with
+ * round-to-nearest-even (dense.py:105-127: shift 0, rounding_mode 'conv_even'). Operands, weights and
+ * results of one call share one format (resolver.py:125-129). Sizes and pitches count elements. */
+enum a4g_float_format { A4G_BF16 = 16, A4G_F32 = 17 };
+
+/* Row pitch (elements) of a packed float weight matrix: rows start 16-byte aligned. */
+A4G_API int64_t a4g_packed_ld_f(int64_t K, int fmt);
+/* W [K][ldw] (the reference's [n_in][n_out], after pack_as_float, matmul/common.py:253-284)
+ * -> Wt [N][a4g_packed_ld_f(K, fmt)], padding zero filled. */
+A4G_API int a4g_pack_weights_f(const void* W, int fmt, int64_t ldw, int64_t K, int64_t N, void* Wt, a4g_stream_t stream);
+/* Y = fmt(relu?(bias + A x W)). Replaces dense_single<Cfg>::run with float types,
+ * templates/nnet_utils/dense_bias_relu/dense_bias_relu.cpp:66-166 (the bias is the accumulator's start
+ * value, :112-124). A [M][lda], Wt packed, bias float32 [N] or null, Y [M][ldy]. */
+A4G_API int a4g_dense_f(const void* A, int fmt, int64_t lda, const void* Wt, int64_t ldwt, const float* bias, int relu, void* Y,
+                int64_t ldy, int64_t M, int64_t N, int64_t K, a4g_stream_t stream);
+/* C[b] = fmt(A[b] x B[b]). Replaces matmul_single<Cfg>::run with float types,
+ * templates/nnet_utils/matmul/matmul.cpp:31-118. trans_b != 0: B is [batch][N][ldb] (the io_view swap of
+ * matmul.py:84-98); otherwise B is [batch][K][ldb] and a workspace of a4g_matmul_f_workspace_bytes()
+ * holds its transpose. */
+A4G_API size_t a4g_matmul_f_workspace_bytes(int64_t batch, int64_t N, int64_t K, int trans_b, int fmt);
+A4G_API int a4g_matmul_f(const void* A, int fmt, int64_t lda, int64_t stride_a, const void* B, int64_t ldb, int64_t stride_b,
+                 int trans_b, void* C, int64_t ldc, int64_t stride_c, int64_t batch, int64_t M, int64_t N, int64_t K,
+                 void* workspace, size_t workspace_bytes, a4g_stream_t stream);
+/* out[i] = fmt(a[i] + b[i]). Replaces elementwise_add_kernel<Cfg>::run with float types,
+ * templates/nnet_utils/elementwise_add/elementwise_add.cpp:12-37. */
+A4G_API int a4g_add_f(const void* a, const void* b, void* out, int64_t n, int fmt, a4g_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -209,3 +209,56 @@ def num_threads():
 
 def set_num_threads(n):
     lib().a4o_set_num_threads(int(n))
+
+
+# ---- floating-point compute path ---------------------------------------------------------------------------------
+# The reference's float mode multiplies bfloat16 (or float32) operands into a float32 accumulator that starts at
+# the bias and rounds the result to the operand format with conv_even (dense.py:105-127,
+# dense_bias_relu.cpp:112-163). The AI Engine's order of additions is not visible from the sources, so the
+# restatement below accumulates exactly (float64 on operands that are exact in their format) and rounds once:
+# every float32 summation order stays within the usual forward error bound of it. Parity with the AI Engine
+# itself is unpinned beyond the tolerances of the reference's own test (tests/test_float_sim.py:81-87:
+# rtol 1e-2 / atol 5e-2 for bfloat16, 1e-3 / 1e-3 for float32).
+
+def bf16_truncate(x):
+    """float -> nearest-toward-zero bfloat16 value, as float32 (pack_as_float, matmul/common.py:272-274,
+    and _bf16_like of tests/test_float_sim.py:59-61)."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    return ((u >> 16) << 16).view(np.float32)
+
+
+def bf16_round(x):
+    """float -> bfloat16 with round-to-nearest-even (the conv_even of the kernels' to_vector), as float32."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    r = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16
+    out = r.astype(np.uint32).view(np.float32)
+    return np.where(np.isnan(x), np.float32(np.nan), out)
+
+
+def to_float_format(x, fmt):
+    if fmt == 'bfloat16':
+        return bf16_round(np.asarray(x, dtype=np.float64).astype(np.float32))
+    if fmt == 'float32':
+        return np.asarray(x, dtype=np.float64).astype(np.float32)
+    raise ValueError(f'unknown float format {fmt!r}')
+
+
+def dense_float(A, W, bias, relu=False, fmt='bfloat16'):
+    """A [M,K], W [K,N] (values exact in `fmt`), bias float32 [N] or None -> float32 array of `fmt` values."""
+    acc = np.asarray(A, dtype=np.float64) @ np.asarray(W, dtype=np.float64)
+    if bias is not None:
+        acc = acc + np.asarray(bias, dtype=np.float32).astype(np.float64)
+    if relu:
+        acc = np.maximum(acc, 0.0)
+    return to_float_format(acc, fmt)
+
+
+def matmul_float(A, B, trans_b=False, fmt='bfloat16'):
+    B = np.asarray(B, dtype=np.float64)
+    if trans_b:
+        B = np.swapaxes(B, -1, -2)
+    return to_float_format(np.asarray(A, dtype=np.float64) @ B, fmt)
+
+
+def add_float(a, b, fmt='bfloat16'):
+    return to_float_format(np.asarray(a, dtype=np.float64) + np.asarray(b, dtype=np.float64), fmt)

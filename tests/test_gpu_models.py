@@ -213,3 +213,63 @@ def test_int16_activation_mlp_graph(oracle):
     assert model.context.config['gpu_fusion_plan']['mlp_chains'] == []
     x = r.integers(-32768, 32768, (64, 48)).astype(np.int16)
     _graph_check(model, oracle, {'x': x})
+
+
+# ---- float compute path through the graph executor ----------------------------------------------------------------
+
+def _float_net(compute_dtype, batch, n_in=32, n_h=32, n_out=16, seed=0):
+    r = np.random.default_rng(seed)
+    q = qint(16, 13)
+    w0, b0 = r.normal(0, 0.05, (n_in, n_h)), r.normal(0, 0.05, n_h)
+    w1, b1 = r.normal(0, 0.05, (n_h, n_out)), r.normal(0, 0.05, n_out)
+    gb = GraphBuilder({'ComputeDtype': compute_dtype})
+    x = gb.input('x', (batch, n_in), q)
+    h = gb.dense(x, w0, q, q, bias=b0, bias_precision=q, relu=True, name='dense0')
+    gb.output(gb.dense(h, w1, q, q, bias=b1, bias_precision=q, name='dense1'))
+    return gb.build(), (w0, b0, w1, b1)
+
+
+@pytest.mark.parametrize('compute_dtype,rtol,atol', [('bfloat16', 1e-2, 5e-2), ('float', 1e-3, 1e-3)])
+@pytest.mark.parametrize('batch,width', [(4, 32), (512, 256)])
+def test_forced_float_mode_mlp(oracle, compute_dtype, rtol, atol, batch, width):
+    """The reference's float test (tests/test_float_sim.py:113-149): a quantised two-layer network forced into
+    float mode must match the plain float network within rtol / atol. The comparison model is that test's
+    _float_reference: bfloat16 by truncation of the input, the weights and the hidden activations, float32
+    bias, float32 matmuls. Width 256 takes the tiled matrix-core kernel, width 32 the generic one."""
+    model, (w0, b0, w1, b1) = _float_net(compute_dtype, batch, n_in=width, n_h=width)
+    x = np.random.default_rng(42).uniform(-2.0, 2.0, (batch, width)).astype(np.float32)
+    y = model.predict(x)
+    assert y.dtype == np.float64 and y.shape == (batch, 16)
+    cast = oracle.bf16_truncate if compute_dtype == 'bfloat16' else (lambda a: np.asarray(a, dtype=np.float32))
+    h = cast(x) @ cast(w0) + b0.astype(np.float32)
+    h = np.maximum(h, 0.0).astype(np.float32)
+    ref = cast(h) @ cast(w1) + b1.astype(np.float32)
+    np.testing.assert_allclose(y, ref, rtol=rtol, atol=atol)
+    # and against the layer-by-layer oracle (exact accumulation, one rounding per layer): at most one unit in
+    # the last place of the output format per layer, carried through the second layer
+    fmt = 'bfloat16' if compute_dtype == 'bfloat16' else 'float32'
+    h_o = oracle.dense_float(cast(x), cast(w0), b0, relu=True, fmt=fmt)
+    y_o = oracle.dense_float(h_o, cast(w1), b1, fmt=fmt)
+    ulp = 2.0 ** -7 if fmt == 'bfloat16' else 2.0 ** -22
+    slack = ulp * (np.abs(h_o).astype(np.float64) @ np.abs(cast(w1)).astype(np.float64) + np.abs(y_o) + np.abs(b1))
+    assert np.all(np.abs(y - y_o) <= slack)
+
+
+def test_float_graph_with_matmul_and_add(oracle):
+    from aie4ml_amd.aie_types import FloatFormat, FloatIntent
+
+    bf = FloatIntent(16, FloatFormat.BF16)
+    r = np.random.default_rng(7)
+    gb = GraphBuilder()
+    a = gb.input('a', (2, 64, 32), bf)
+    b = gb.input('b', (2, 64, 32), bf)
+    s = gb.add(a, b, bf, name='sum')
+    gb.output(gb.matmul(s, gb.transpose(b, (0, 2, 1)), bf, name='mm'))
+    model = gb.build()
+    A = oracle.bf16_truncate(r.normal(0, 1, (2, 64, 32)))
+    B = oracle.bf16_truncate(r.normal(0, 1, (2, 64, 32)))
+    y = model.predict({'a': A, 'b': B})
+    s_o = oracle.add_float(A, B, 'bfloat16')
+    y_o = oracle.matmul_float(s_o, B, trans_b=True, fmt='bfloat16')
+    bound = 2.0 ** -7 * np.abs(y_o) + 34 * 2.0 ** -24 * (np.abs(s_o).astype(np.float64) @ np.abs(np.swapaxes(B, -1, -2)))
+    assert np.all(np.abs(y - y_o) <= bound)

@@ -400,3 +400,72 @@ def test_predict_input_contract_without_gpu():
     with pytest.raises(ValueError, match='quantize=False requires integer inputs'):
         model.prepare_inputs(np.zeros((4, 16)), quantize=False)
     assert model.prepare_inputs(np.full((4, 16), 1.0))['x'][0, 0, 0] == 16   # 1.0 * 2^4
+
+
+# ---- float compute path (host side) -----------------------------------------------------------------------
+
+def _float_mlp(config=None, in_prec=None, w_prec=None):
+    # the network of the reference's float test (tests/test_float_sim.py:77-78: 32 -> 32 -> 16, batch 4)
+    r = np.random.default_rng(0)
+    q = qint(16, 13)
+    gb = GraphBuilder(config or {})
+    x = gb.input('x', (4, 32), in_prec or q)
+    h = gb.dense(x, r.normal(0, 0.05, (32, 32)), w_prec or q, in_prec or q, bias=r.normal(0, 0.05, 32),
+                 bias_precision=w_prec or q, relu=True, name='dense0')
+    y = gb.dense(h, r.normal(0, 0.05, (32, 16)), w_prec or q, in_prec or q, bias=r.normal(0, 0.05, 16),
+                 bias_precision=w_prec or q, name='dense1')
+    gb.output(y)
+    return gb
+
+
+@pytest.mark.parametrize('compute_dtype,fmt', [('bfloat16', 'bfloat16'), ('float', 'float32'), ('float32', 'float32')])
+def test_force_float_mode_resolves_float_variants(compute_dtype, fmt):
+    from aie4ml_amd.passes import ForceFloatMode
+
+    gb = _float_mlp({'ComputeDtype': compute_dtype})
+    ctx = lower(gb, (ForceFloatMode,) + FRONT)
+    for name, relu in (('dense0_aie', True), ('dense1_aie', False)):
+        inst = ctx.ir.execution.get(name)
+        assert inst.variant.variant_id == 'dense.b.r.float.gfx950.v1'
+        cfg = inst.config
+        assert cfg.shift == 0 and cfg.accumulator_tag == 'accfloat' and cfg.rounding_mode == 'conv_even'
+        assert cfg.flags.use_relu is relu and cfg.flags.use_bias is True
+        assert {cfg.precision[k].format for k in ('lhs', 'rhs', 'output')} == {fmt}
+        assert cfg.precision['bias'].format == 'float32' and cfg.precision['acc'].format == 'accfloat'
+    assert [n.op_type for n in ctx.ir.logical.nodes] == ['dense', 'dense']  # bias and ReLU folded as in integer mode
+    # the fused int8 MLP kernel must not claim a float chain
+    PlanGpuFusion().transform(ctx)
+    assert ctx.config['gpu_fusion_plan']['mlp_chains'] == []
+
+
+def test_float_mode_rules():
+    from aie4ml_amd.aie_types import FloatFormat, FloatIntent
+    from aie4ml_amd.op_impls.float_ops import pack_as_float
+    from aie4ml_amd.passes import ForceFloatMode
+
+    with pytest.raises(ValueError, match='is not recognised'):
+        lower(_float_mlp({'ComputeDtype': 'float16'}), (ForceFloatMode,) + FRONT)
+    bf, f32 = FloatIntent(16, FloatFormat.BF16), FloatIntent(32, FloatFormat.FP32)
+    # mixed float / fixed point, and mixed float formats, are rejected as in the reference's _resolve_numeric
+    with pytest.raises(ValueError):
+        lower(_float_mlp(in_prec=bf, w_prec=qint(8, 6)))
+    with pytest.raises(ValueError, match='share float precision'):
+        lower(_float_mlp(in_prec=bf, w_prec=f32))
+    with pytest.raises(NotImplementedError, match='no GPU kernel'):
+        lower(_float_mlp(in_prec=FloatIntent(8, FloatFormat.FP8_E4M3), w_prec=FloatIntent(8, FloatFormat.FP8_E4M3)))
+    # a power-of-two scale cannot fold into a float dense
+    gb = GraphBuilder()
+    x = gb.input('x', (4, 32), bf)
+    gb.output(gb.scale(gb.dense(x, np.zeros((32, 8)), bf, bf, name='fc'), 0.5, bf))
+    with pytest.raises(NotImplementedError, match='not implemented for float'):
+        lower(gb)
+    # LayerNorm and Softmax have no float variant
+    gb = GraphBuilder()
+    x = gb.input('x', (4, 32), bf)
+    gb.output(gb.softmax(x, bf))
+    with pytest.raises((ValueError, NotImplementedError)):
+        lower(gb)
+    # parameters reach bfloat16 by truncation
+    v = np.array([1.0, 1.00390625, 1.0078125, -1.00390625, 3.14159], dtype=np.float32)
+    assert pack_as_float(v, 'bfloat16').tolist() == [1.0, 1.0, 1.0078125, -1.0, 3.140625]
+    assert pack_as_float(v, 'float32').tolist() == v.tolist()

@@ -351,3 +351,39 @@ def test_add_layernorm_is_composition(oracle):
     s2 = oracle.add(a, b)
     assert np.array_equal(s, s2)
     assert np.array_equal(out, oracle.layernorm(s2, gamma, beta, 5, 'conv_even'))
+
+
+# ---- float path: the conversions are checked against an independent library routine (torch's CPU casts) ----------
+
+def test_bf16_conversions_against_torch_cpu(oracle):
+    torch = pytest.importorskip('torch')
+    r = np.random.default_rng(3)
+    x = np.concatenate([r.normal(0, 1, 20000), r.normal(0, 1e-3, 2000), r.normal(0, 1e4, 2000),
+                        [0.0, -0.0, 1.0, -1.0, 3.0e38, -3.0e38, 1e-40, np.inf, -np.inf]]).astype(np.float32)
+    # exact ties: odd bfloat16 neighbours' midpoints, where round-to-nearest-even and half-up differ
+    base = (r.integers(0x3000, 0x4800, 4000).astype(np.uint32) << 16) | 0x8000
+    x = np.concatenate([x, base.view(np.float32), (base | 0x80000000).view(np.float32)])
+    want = torch.from_numpy(x).to(torch.bfloat16).float().numpy()
+    assert np.array_equal(oracle.bf16_round(x).view(np.uint32), want.view(np.uint32))
+    t = oracle.bf16_truncate(x)
+    assert np.all((t.view(np.uint32) & 0xFFFF) == 0)
+    fin = np.isfinite(x)
+    assert np.all(np.abs(t[fin]) <= np.abs(x[fin]))                       # toward zero
+    up = ((t.view(np.uint32) + 0x10000).view(np.float32))                  # next bfloat16 away from zero
+    assert np.all(np.abs(x[fin]) < np.abs(up[fin]))                        # and less than one step away
+
+
+def test_float_dense_oracle_against_float64_identity_and_linearity(oracle):
+    r = np.random.default_rng(4)
+    A = oracle.bf16_truncate(r.normal(0, 1, (9, 40)))
+    W = oracle.bf16_truncate(r.normal(0, 1, (40, 7)))
+    b = r.normal(0, 1, 7).astype(np.float32)
+    y = oracle.dense_float(A, W, b, relu=False, fmt='float32')
+    want = np.array([[sum(float(A[m, k]) * float(W[k, n]) for k in range(40)) + float(b[n]) for n in range(7)]
+                     for m in range(9)])
+    assert np.allclose(y, want, rtol=2.0 ** -23, atol=0)
+    yb = oracle.dense_float(A, W, b, relu=True, fmt='bfloat16')
+    assert np.array_equal(yb, oracle.bf16_round(np.maximum(want, 0).astype(np.float32)))
+    assert np.array_equal(oracle.dense_float(A, np.eye(40, dtype=np.float32), None, fmt='bfloat16'), A)
+    assert np.array_equal(oracle.matmul_float(A, W.T.copy(), trans_b=True, fmt='float32'),
+                          oracle.matmul_float(A, W, fmt='float32'))
