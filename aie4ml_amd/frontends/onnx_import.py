@@ -5,8 +5,8 @@ same handler registry (`@onnx_handler(*op_types)` -> `fn(ctx, node, node_name, d
 frontends/onnx/registry.py:12-34), the same lowering of QuantizeLinear / DequantizeLinear pairs to per-tensor
 power-of-two QuantIntents (frontends/onnx/quantize.py), the same node kinds, roles and metadata, and the same
 error messages. Differences: the file is decoded by onnx_proto (no protobuf dependency), static shapes come
-from the small inference table below instead of onnx.shape_inference, float tensors are rejected (the GPU
-build covers the integer path), and the result is a GPUModel.
+from the small inference table below instead of onnx.shape_inference, of the float element types FLOAT and
+BFLOAT16 are taken (the formats with a GPU kernel), and the result is a GPUModel.
 """
 
 from __future__ import annotations
@@ -15,7 +15,7 @@ from typing import Any, Callable, Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
 
-from ..aie_types import QuantIntent, RoundingMode, SaturationMode
+from ..aie_types import FloatFormat, FloatIntent, QuantIntent, RoundingMode, SaturationMode, is_float_intent
 from ..ir import BackendContext, LogicalIR, OpNode, TensorVar, set_input_roles
 from . import onnx_proto as op
 
@@ -202,6 +202,13 @@ def build_shape_table(model: op.Model, initializers: Dict[str, np.ndarray], inpu
 
 # ---- import state (frontends/onnx/context.py) -----------------------------------------------------------------
 
+# ONNX elem_type of a bare (not Q/DQ wrapped) graph input -> intent (frontends/onnx/context.py:18-24)
+_FLOAT_INPUT_INTENT = {
+    op.FLOAT: FloatIntent(width=32, format=FloatFormat.FP32),
+    op.BFLOAT16: FloatIntent(width=16, format=FloatFormat.BF16),
+}
+
+
 class OnnxImportContext:
     """Mutable state threaded through the handler dispatch."""
 
@@ -218,6 +225,7 @@ class OnnxImportContext:
         self.value_tensors: Dict[str, TensorVar] = {}   # ONNX value name -> lowered tensor
         self.q_aliases: Dict[str, Tuple[str, Any, QuantIntent, Tuple[int, ...]]] = {}  # Quantize output awaiting its Dequantize
         self.precision_mirrors: List[Tuple[str, str]] = []
+        self.bfloat16_initializers: set = set()  # names of initializers the file stores as BFLOAT16
 
     def mirror_precision(self, target: str, source: str) -> None:
         self.precision_mirrors.append((target, source))
@@ -262,8 +270,14 @@ class OnnxImportContext:
         if name in self.value_tensors:
             return self.value_tensors[name]
         if name in self.input_shapes:
-            raise ValueError(f'{node_name}: graph input "{name}" has ONNX elem_type {self.input_dtypes.get(name)} and is used '
-                             'without QDQ wrapping; only the integer path is supported. Use QDQ wrapping for integer inputs.')
+            # a bare float graph input belongs to the float compute path (frontends/onnx/context.py:18-24, 131-143)
+            intent = _FLOAT_INPUT_INTENT.get(self.input_dtypes.get(name))
+            if intent is None:
+                raise ValueError(f'{node_name}: graph input "{name}" has unsupported ONNX elem_type '
+                                 f'{self.input_dtypes.get(name)}. Use QDQ wrapping for integer inputs.')
+            tensor = self.graph_input_tensor(name, self.input_shapes[name], intent)
+            self.bind(name, tensor)
+            return tensor
         raise ValueError(f'{node_name}: unsupported input {name}. Expected a dequantized activation tensor.')
 
     def parameter_source_for(self, name: str, node_name: str) -> TensorVar:
@@ -278,8 +292,10 @@ class OnnxImportContext:
             if data.dtype not in (np.dtype(np.float32), np.dtype(np.float64)):
                 raise ValueError(f'{node_name}: direct initializer inputs must be float32, or quantized via DequantizeLinear; '
                                  f'got {data.dtype}.')
-            # a float constant (LayerNormalization scale / bias): the consuming operator quantises it itself
-            return self.param_tensor(name, data, None)
+            # a float constant: LayerNormalization scale / bias (the operator quantises those itself, whatever the
+            # intent says) or a parameter of the float compute path (intent_from_initializer, utils.py:229-241)
+            fmt = FloatFormat.BF16 if name in self.bfloat16_initializers else FloatFormat.FP32
+            return self.param_tensor(name, data, FloatIntent(width=16 if fmt is FloatFormat.BF16 else 32, format=fmt))
         raise ValueError(f'{node_name}: parameter input {name} must be a constant initializer.')
 
     def any_source_for(self, name: str, node_name: str) -> TensorVar:
@@ -432,12 +448,13 @@ def _matmul_gemm(ctx: OnnxImportContext, node: op.Node, node_name: str, directiv
         raise ValueError(f'{node_name}: activation input cannot be constant.')
     out_name = node.outputs[0]
     out_shape = ctx.output_shape(out_name, node_name)
+    out_precision = lhs.precision if is_float_intent(lhs.precision) else None  # handlers/matmul.py:51
 
     if not rhs_const:
         rhs = ctx.source_for(rhs_name, node_name)
         rs = ctx.output_shape(rhs_name, node_name)
         n_in, n_out = int(rs[0] if len(rs) == 1 else rs[-2]), int(1 if len(rs) == 1 else rs[-1])
-        ctx.emit('matmul', node_name, inputs=[lhs, rhs], outputs=[(out_name, out_shape, None)], roles=['lhs', 'rhs'],
+        ctx.emit('matmul', node_name, inputs=[lhs, rhs], outputs=[(out_name, out_shape, out_precision)], roles=['lhs', 'rhs'],
                  metadata=_mm_meta('MatMul', 'MatMul', n_in, n_out, node_name), directives=directives)
         return
 
@@ -450,19 +467,19 @@ def _matmul_gemm(ctx: OnnxImportContext, node: op.Node, node_name: str, directiv
             raise ValueError(f'{node_name}: ONNX Gemm weight matrix must be rank-2.')
         n_in, n_out = int(data.shape[0] if data.ndim == 1 else data.shape[-2]), int(1 if data.ndim == 1 else data.shape[-1])
         ctx.emit('matmul', node_name, inputs=[lhs, ctx.param_tensor(f'{node_name}_rhs', data, rhs.precision)],
-                 outputs=[(out_name, out_shape, None)], roles=['lhs', 'rhs'],
+                 outputs=[(out_name, out_shape, out_precision)], roles=['lhs', 'rhs'],
                  metadata=_mm_meta('MatMul', 'MatMul', n_in, n_out, node_name), directives=directives)
         return
     n_in, n_out = int(data.shape[0]), int(data.shape[1])
     weight = ctx.param_tensor(f'{node_name}_weight', data, rhs.precision)
     if bias_name is None:
-        ctx.emit('dense', node_name, inputs=[lhs, weight], outputs=[(out_name, out_shape, None)], roles=['lhs', 'rhs'],
+        ctx.emit('dense', node_name, inputs=[lhs, weight], outputs=[(out_name, out_shape, out_precision)], roles=['lhs', 'rhs'],
                  metadata=_mm_meta('Dense', kind, n_in, n_out, node_name), directives=directives)
         return
     # Gemm with bias: dense -> add(bias); the bias-folding pass re-fuses the add into the dense
     prebias = f'{node_name}_prebias'
     ctx.mirror_precision(prebias, out_name)
-    ctx.emit('dense', node_name, inputs=[lhs, weight], outputs=[(prebias, out_shape, None)], roles=['lhs', 'rhs'],
+    ctx.emit('dense', node_name, inputs=[lhs, weight], outputs=[(prebias, out_shape, out_precision)], roles=['lhs', 'rhs'],
              metadata=_mm_meta('Dense', kind, n_in, n_out, node_name), directives=directives)
     bias = ctx.parameter_source_for(bias_name, node_name)
     bias_data = np.asarray(bias.data, dtype=np.float64).reshape(-1)
@@ -470,7 +487,7 @@ def _matmul_gemm(ctx: OnnxImportContext, node: op.Node, node_name: str, directiv
         raise ValueError(f'{node_name}: Gemm bias must contain exactly {n_out} elements.')
     ctx.emit('add', f'{node_name}_bias', inputs=[ctx.value_tensors[prebias], ctx.param_tensor(f'{node_name}_bias', bias_data,
                                                                                              bias.precision)],
-             outputs=[(out_name, out_shape, None)], roles=['lhs', 'rhs'],
+             outputs=[(out_name, out_shape, out_precision)], roles=['lhs', 'rhs'],
              metadata={'layer_class': 'Add', 'source_class': 'Gemm', 'source_layer': node_name}, directives={})
 
 
@@ -517,7 +534,8 @@ def _add(ctx: OnnxImportContext, node: op.Node, node_name: str, directives: dict
         ls, rs = ctx.output_shape(lhs_name, node_name), ctx.output_shape(rhs_name, node_name)
         if ls != rs:
             raise ValueError(f'{node_name}: generic Add only supports exact-shape elementwise inputs; got {ls} and {rs}.')
-    ctx.emit('add', node_name, inputs=[lhs, rhs], outputs=[(out_name, ctx.output_shape(out_name, node_name), None)],
+    out_precision = lhs.precision if is_float_intent(lhs.precision) else None  # handlers/elementwise.py:61
+    ctx.emit('add', node_name, inputs=[lhs, rhs], outputs=[(out_name, ctx.output_shape(out_name, node_name), out_precision)],
              roles=['lhs', 'rhs'], metadata={'layer_class': 'Add', 'source_class': 'Add', 'source_layer': node_name},
              directives=directives)
 
@@ -672,6 +690,7 @@ def lower_onnx_model(model_or_path, config: Optional[Dict[str, Any]] = None) -> 
     backend = BackendContext(config=config)
     graph = backend.ir.logical
     initializers = {t.name: np.asarray(t.array) for t in model.graph.initializers}
+    bfloat16_initializers = {t.name for t in model.graph.initializers if t.bfloat16}
     input_shapes: Dict[str, Tuple[int, ...]] = {}
     input_dtypes: Dict[str, int] = {}
     for vi in model.graph.inputs:
@@ -692,6 +711,7 @@ def lower_onnx_model(model_or_path, config: Optional[Dict[str, Any]] = None) -> 
     ctx = OnnxImportContext(backend, initializers=initializers, input_shapes=input_shapes, input_dtypes=input_dtypes,
                             shape_of=build_shape_table(model, initializers, input_shapes),
                             layer_directives=dict(config.get('LayerDirectives', {}) or {}))
+    ctx.bfloat16_initializers = bfloat16_initializers
     for index, node in enumerate(model.graph.nodes):
         name = node_name_of(node, index)
         dispatch(ctx, node, name, ctx.take_directives(name))

@@ -18,6 +18,7 @@ import numpy as np
 
 # TensorProto.DataType
 FLOAT, UINT8, INT8, UINT16, INT16, INT32, INT64, BOOL, FLOAT16, DOUBLE = 1, 2, 3, 4, 5, 6, 7, 9, 10, 11
+BFLOAT16 = 16  # no numpy dtype: such tensors are held as float32 arrays and flagged (Tensor.bfloat16)
 NP_OF = {FLOAT: np.float32, UINT8: np.uint8, INT8: np.int8, UINT16: np.uint16, INT16: np.int16, INT32: np.int32,
          INT64: np.int64, BOOL: np.bool_, FLOAT16: np.float16, DOUBLE: np.float64}
 ONNX_OF = {np.dtype(v): k for k, v in NP_OF.items()}
@@ -27,6 +28,7 @@ ONNX_OF = {np.dtype(v): k for k, v in NP_OF.items()}
 class Tensor:
     name: str
     array: np.ndarray
+    bfloat16: bool = False  # the file stores (or shall store) the values as ONNX BFLOAT16
 
 
 @dataclass
@@ -157,6 +159,13 @@ def _parse_tensor(buf: bytes) -> Tensor:
             _ints(wt, val, u64)
         elif num == 13 and len(val):
             raise NotImplementedError(f'tensor {name!r}: external data is not supported')
+    if dtype == BFLOAT16:  # 16-bit patterns in raw_data or int32_data; widened to float32 (exact)
+        bits = np.frombuffer(raw, dtype='<u2') if raw is not None else np.array(i32, dtype=np.int64)
+        arr = (bits.astype(np.uint32) << 16).view(np.float32)
+        count = int(np.prod(dims)) if dims else 1
+        if arr.size != count:
+            raise ValueError(f'tensor {name!r}: {arr.size} values for shape {tuple(dims)}')
+        return Tensor(name, arr.reshape(tuple(dims)), bfloat16=True)
     if dtype not in NP_OF:
         raise NotImplementedError(f'tensor {name!r}: ONNX data type {dtype} is not supported')
     npdt = np.dtype(NP_OF[dtype])
@@ -343,6 +352,12 @@ def _packed_ints(num: int, values) -> bytes:
 
 def _ser_tensor(t: Tensor) -> bytes:
     arr = np.ascontiguousarray(t.array)
+    if t.bfloat16:
+        bits = np.ascontiguousarray(arr, dtype=np.float32).view(np.uint32)
+        if np.any(bits & 0xFFFF):
+            raise ValueError(f'tensor {t.name!r}: values are not exact in bfloat16')
+        out = _packed_ints(1, arr.shape) + _vi(2, BFLOAT16) + _ld(8, t.name.encode())
+        return out + _ld(9, (bits >> 16).astype('<u2').tobytes())
     if arr.dtype not in ONNX_OF:
         raise NotImplementedError(f'tensor {t.name!r}: dtype {arr.dtype} has no ONNX type here')
     out = _packed_ints(1, arr.shape) + _vi(2, ONNX_OF[arr.dtype]) + _ld(8, t.name.encode())

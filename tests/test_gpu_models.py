@@ -273,3 +273,28 @@ def test_float_graph_with_matmul_and_add(oracle):
     y_o = oracle.matmul_float(s_o, B, trans_b=True, fmt='bfloat16')
     bound = 2.0 ** -7 * np.abs(y_o) + 34 * 2.0 ** -24 * (np.abs(s_o).astype(np.float64) @ np.abs(np.swapaxes(B, -1, -2)))
     assert np.all(np.abs(y - y_o) <= bound)
+
+
+@pytest.mark.parametrize('bf', [False, True])
+def test_float_onnx_model_predicts(oracle, bf):
+    from aie4ml_amd import from_onnx
+    from aie4ml_amd.frontends import onnx_proto as op
+
+    r = np.random.default_rng(1)
+    cast = oracle.bf16_truncate if bf else (lambda a: np.asarray(a, dtype=np.float32))
+    elem = op.BFLOAT16 if bf else op.FLOAT
+    w0, b0, w1 = cast(r.normal(0, 0.1, (64, 128))), cast(r.normal(0, 0.1, 128)), cast(r.normal(0, 0.1, (128, 32)))
+    g = op.Graph(name='float_mlp')
+    g.inputs.append(op.ValueInfo('x', elem, (8, 64)))
+    g.initializers += [op.Tensor('w0', w0, bfloat16=bf), op.Tensor('b0', b0, bfloat16=bf), op.Tensor('w1', w1, bfloat16=bf)]
+    g.nodes += [op.Node('Gemm', ['x', 'w0', 'b0'], ['h'], 'fc0', {}), op.Node('Relu', ['h'], ['hr'], 'relu0', {}),
+                op.Node('MatMul', ['hr', 'w1'], ['y'], 'fc1', {})]
+    g.outputs.append(op.ValueInfo('y', elem, (8, 32)))
+    model = from_onnx(op.serialize_model(op.Model(graph=g, opset={'': 17}, producer_name='test')))
+    x = cast(r.uniform(-2, 2, (8, 64)))
+    y = model.predict(x)
+    fmt = 'bfloat16' if bf else 'float32'
+    h_o = oracle.dense_float(x, w0, b0, relu=True, fmt=fmt)
+    y_o = oracle.dense_float(h_o, w1, None, fmt=fmt)
+    rtol, atol = (1e-2, 5e-2) if bf else (1e-3, 1e-3)  # the reference's float tolerances (tests/test_float_sim.py:81-87)
+    np.testing.assert_allclose(y, y_o, rtol=rtol, atol=atol)

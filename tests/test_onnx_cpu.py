@@ -146,3 +146,38 @@ def test_gemm_bias_relu_and_slice():
     assert W.shape == (32, 16) and np.all(W == 32) and b.tolist() == list(range(16))
     cut = next(n for n in ctx.ir.logical.nodes if n.is_placeholder)
     assert cut.traits['slice_view'].data['slices'] == [{'output': 'cut_out', 'start': 4, 'extent': 8}]
+
+
+def test_float_onnx_graph_imports_with_float_intents():
+    """A graph without Q/DQ nodes is a float graph: bare FLOAT / BFLOAT16 inputs and initializers carry a
+    FloatIntent (frontends/onnx/context.py:18-24, utils.py:229-241) and matmul-family outputs inherit it."""
+    from aie4ml_amd.aie_types import FloatFormat, is_float_intent
+    from aie4ml_amd.frontends import onnx_proto as op
+    from aie4ml_amd.frontends.onnx_import import lower_onnx_model
+    from aie4ml_amd.passes import FoldBias, FoldScale, FoldViewOps, FuseActivationCasts, Resolve, run_aie_passes
+
+    r = np.random.default_rng(0)
+    for elem, bf in ((op.FLOAT, False), (op.BFLOAT16, True)):
+        def cast(a):
+            a = np.asarray(a, dtype=np.float32)
+            return ((a.view(np.uint32) >> 16) << 16).view(np.float32) if bf else a
+
+        g = op.Graph(name='float_mlp')
+        g.inputs.append(op.ValueInfo('x', elem, (4, 32)))
+        g.initializers += [op.Tensor('w0', cast(r.normal(0, 0.1, (32, 32))), bfloat16=bf),
+                           op.Tensor('b0', cast(r.normal(0, 0.1, 32)), bfloat16=bf),
+                           op.Tensor('w1', cast(r.normal(0, 0.1, (32, 16))), bfloat16=bf)]
+        g.nodes += [op.Node('Gemm', ['x', 'w0', 'b0'], ['h'], 'fc0', {}), op.Node('Relu', ['h'], ['hr'], 'relu0', {}),
+                    op.Node('MatMul', ['hr', 'w1'], ['y'], 'fc1', {})]
+        g.outputs.append(op.ValueInfo('y', elem, (4, 16)))
+        blob = op.serialize_model(op.Model(graph=g, opset={'': 17}, producer_name='test'))
+        back = op.parse_model(blob)
+        assert [t.bfloat16 for t in back.graph.initializers] == [bf] * 3
+        assert np.array_equal(back.graph.initializers[0].array, g.initializers[0].array)
+        ctx = lower_onnx_model(blob, {})
+        fmt = FloatFormat.BF16 if bf else FloatFormat.FP32
+        assert all(is_float_intent(t.precision) and t.precision.format is fmt for t in ctx.ir.logical.tensors.values())
+        run_aie_passes(ctx, [p() for p in (FoldBias, FoldScale, FuseActivationCasts, FoldViewOps, Resolve)])
+        assert [n.op_type for n in ctx.ir.logical.nodes] == ['dense', 'dense']
+        cfg = ctx.ir.execution.get(ctx.ir.logical.nodes[0].name).config
+        assert cfg.accumulator_tag == 'accfloat' and cfg.flags.use_relu and cfg.flags.use_bias
