@@ -101,16 +101,12 @@ class GPUModel:
                 prepared[t.name] = arr.astype(dtype_for_precision(dtype.width, dtype.signed), copy=False)
         return prepared
 
-    def predict(self, X, simulator: str = 'gpu', *, quantize_in: bool = True, dequantize_out: bool = True):
-        if simulator.lower() not in ('gpu', 'mi355x', 'gfx950'):
-            raise ValueError(f'Unknown simulator "{simulator}". Expected one of: gpu.')
-        if not self._compiled:
-            self.compile()
+    def to_device(self, prepared: Dict[str, np.ndarray]) -> Dict[str, Any]:
+        """Prepared host arrays -> device tensors; the iteration axis and the tensors' own leading (batch)
+        axis become one batch axis on the GPU."""
         import torch
 
-        prepared = self.prepare_inputs(X, quantize=quantize_in)
         graph = self.context.ir.logical
-        # the iteration axis and the tensors' own leading (batch) axis are one batch axis on the GPU
         dev_inputs = {}
         for name, arr in prepared.items():
             merged = arr.reshape((arr.shape[0] * arr.shape[1],) + tuple(arr.shape[2:])) if arr.ndim >= 2 else arr
@@ -120,6 +116,24 @@ class GPUModel:
                 dev_inputs[name] = to_device_float(pack_as_float(merged, dtype.format), dtype.format)
             else:
                 dev_inputs[name] = torch.from_numpy(np.ascontiguousarray(merged)).cuda()
+        return dev_inputs
+
+    def report(self, X=None, repeats: int = 10):
+        """Per-launch timing report on the GPU (the counterpart of the reference's report())."""
+        from .report import report
+
+        return report(self, X=X, repeats=repeats)
+
+    def predict(self, X, simulator: str = 'gpu', *, quantize_in: bool = True, dequantize_out: bool = True):
+        if simulator.lower() not in ('gpu', 'mi355x', 'gfx950'):
+            raise ValueError(f'Unknown simulator "{simulator}". Expected one of: gpu.')
+        if not self._compiled:
+            self.compile()
+        import torch
+
+        prepared = self.prepare_inputs(X, quantize=quantize_in)
+        graph = self.context.ir.logical
+        dev_inputs = self.to_device(prepared)
         iters = next(iter(prepared.values())).shape[0]
         dev_out = self.execute(dev_inputs, batch_scale=iters)
         torch.cuda.synchronize()
@@ -136,9 +150,11 @@ class GPUModel:
         return results
 
     # ---- executor -------------------------------------------------------------------------------------
-    def execute(self, inputs: Dict[str, Any], batch_scale: int = 1) -> Dict[str, Any]:
+    def execute(self, inputs: Dict[str, Any], batch_scale: int = 1, trace: Optional[List[dict]] = None) -> Dict[str, Any]:
         """Run the resolved graph on device tensors. `inputs`: graph-input name -> integer device tensor
-        whose leading axis may be `batch_scale` times the declared one. Returns every graph output."""
+        whose leading axis may be `batch_scale` times the declared one. Returns every graph output.
+        With `trace` (a list), every launch group is bracketed by two events and appended to it as
+        {'name', 'kind', 'nodes', 'events'} (used by report())."""
         from . import ops
 
         ctx = self.context
@@ -160,6 +176,18 @@ class GPUModel:
             if grp.get('concat'):
                 attn_skip.add(grp['concat'])
 
+        def launch(label, kind, members, fn):
+            if trace is None:
+                fn()
+                return
+            import torch
+
+            ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            ev0.record()
+            fn()
+            ev1.record()
+            trace.append({'name': label, 'kind': kind, 'nodes': list(members), 'events': (ev0, ev1)})
+
         for node in graph.nodes:
             if node.name in attn_skip:
                 continue
@@ -169,20 +197,24 @@ class GPUModel:
             if node.name in chain_rest or node.name in fused_ln:
                 continue  # executed as part of a fused launch
             if node.name in attn_at:
-                self._run_attention(attn_at[node.name], values, ops)
+                grp = attn_at[node.name]
+                members = [tr[k] for tr in grp['heads'] for k in ('qk', 'softmax', 'pv')]
+                launch(node.name, 'attention', members, lambda: self._run_attention(grp, values, ops))
                 continue
             inst = execution.get(node.name)
             if inst is None:
                 raise RuntimeError(f'{node.name}: node was never resolved; run compile() first.')
             if node.name in chain_head:
-                self._run_mlp(chain_head[node.name], values, ops)
+                chain = chain_head[node.name]
+                launch(node.name, 'mlp', chain, lambda: self._run_mlp(chain, values, ops))
             elif node.name in plan['add_layernorm']:
                 # launched at the add's position: everything that reads the sum comes later in the order
                 info = plan['add_layernorm'][node.name]
-                self._run_add_layernorm((node.name, info), execution.get(info['layer_norm']), values, ops)
+                launch(node.name, 'add_layer_norm', [node.name, info['layer_norm']],
+                       lambda: self._run_add_layernorm((node.name, info), execution.get(info['layer_norm']), values, ops))
             else:
                 args = {t.name: values[t.name] for t in node.inputs if not t.is_parameter}
-                values.update(inst.variant.run(inst, args))
+                launch(node.name, node.op_type, [node.name], lambda: values.update(inst.variant.run(inst, args)))
         return {name: values[name] for name in graph.output_tensor_names}
 
     def _run_view(self, node, values) -> None:

@@ -298,3 +298,27 @@ def test_float_onnx_model_predicts(oracle, bf):
     y_o = oracle.dense_float(h_o, w1, None, fmt=fmt)
     rtol, atol = (1e-2, 5e-2) if bf else (1e-3, 1e-3)  # the reference's float tolerances (tests/test_float_sim.py:81-87)
     np.testing.assert_allclose(y, y_o, rtol=rtol, atol=atol)
+
+
+def test_report_times_every_launch(oracle):
+    """report(): one entry per launch group of the executor, operation count by the reference's convention
+    (2 * n_in * n_out per row, dense and matmul only; src/aie4ml/report.py:133-155)."""
+    model, x, _layers = workloads.c1_mlp_model(batch=256)
+    rep = model.report(x, repeats=3)
+    assert rep['design']['launches'] == 1 and rep['kernels'][0]['kind'] == 'mlp'      # four dense nodes, one fused launch
+    assert rep['design']['ops'] == 2 * 256 * (16 * 64 + 64 * 32 + 32 * 32 + 32 * 5)
+    assert rep['latency']['graph_replay_us'] > 0 and rep['bottleneck']['name'] == rep['kernels'][0]['name']
+    text = str(rep)
+    assert 'GPU execution report' in text and 'Bottleneck' in text
+
+    onnx_bytes, config, x_int = workloads.c5_encoder_block_onnx(batch=2, seq=32, hidden=128, heads=2, ffn=256, softmax='hccs')
+    from aie4ml_amd import from_onnx
+
+    enc = from_onnx(onnx_bytes, config)
+    rep = enc.report(repeats=3)
+    kinds = [k['kind'] for k in rep['kernels']]
+    # QKV and output projections, all heads in one attention launch, both residual adds inside their LayerNorm,
+    # and an FFN this small runs as one fused-MLP launch
+    assert kinds == ['dense', 'attention', 'dense', 'add_layer_norm', 'mlp', 'add_layer_norm']
+    assert abs(sum(k['pct'] for k in rep['kernels']) - 100.0) < 1.0
+    assert all(k['time_us'] > 0 for k in rep['kernels'])
