@@ -28,7 +28,7 @@ ROUNDING = {
     'conv_odd': 7,
 }
 KIND = {'int8': 0, 'uint8': 1, 'int16': 2, 'uint16': 3, 'int32': 4}
-FLOAT_FORMAT = {'bfloat16': 16, 'float32': 17}
+FLOAT_FORMAT = {'bfloat16': 16, 'float32': 17, 'fp8_e4m3': 18}
 
 _i64, _i32, _vp, _sz = ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t
 

@@ -1,12 +1,14 @@
-// Floating-point Dense / MatMul / Add: the reference's float compute path (bfloat16 or float32 operands,
-// float32 accumulation, result rounded to the operand format with round-to-nearest-even).
+// Floating-point Dense / MatMul / Add: the reference's float compute path (bfloat16, float32 or fp8 e4m3
+// operands, float32 accumulation, result converted to the operand format: round-to-nearest-even for bfloat16
+// and float32, the conversion of the reference's own fp8 packer for fp8).
 //   Dense   templates/nnet_utils/dense_bias_relu/dense_bias_relu.cpp:66-166 with acc_scalar_t = accfloat
 //           (dense.py:105-127: shift 0, rounding conv_even, float32 bias as the accumulator's start value)
 //   MatMul  templates/nnet_utils/matmul/matmul.cpp:31-118, same accumulator
 //   Add     templates/nnet_utils/elementwise_add/elementwise_add.cpp:12-37
 // The tiled path is the shared pipelined MFMA kernel with a float policy: a 16-byte fragment is eight
-// bfloat16 (one v_mfma_f32_32x32x16_bf16) or four float32 (four v_mfma_f32_32x32x2_f32); the order of the
-// additions inside a dot product therefore differs from any sequential loop, as it does on the AI Engine.
+// bfloat16 (one v_mfma_f32_32x32x16_bf16), four float32 (four v_mfma_f32_32x32x2_f32) or sixteen fp8 (two
+// v_mfma_f32_32x32x16_fp8_fp8); the order of the additions inside a dot product therefore differs from any
+// sequential loop, as it does on the AI Engine.
 #include <algorithm>
 
 #include "gemm_rs.hpp"
@@ -24,21 +26,44 @@ __device__ __forceinline__ unsigned f32_to_bf16_bits(float f) {  // round to nea
 }
 __device__ __forceinline__ float bf16_bits_to_f32(unsigned h) { return __uint_as_float(h << 16); }
 
+// float32 -> fp8 e4m3 code, the integer recipe of the reference's packer (_float32_to_fp8_scalar,
+// op_impls/families/matmul/common.py:262-276): round half away from zero at mantissa bit 20, exponent bias 7,
+// gradual underflow below 2^-6, magnitudes from 480 up map to the code 0x7f.
+__host__ __device__ __forceinline__ unsigned f32_bits_to_fp8(unsigned bits) {
+    const unsigned h = bits + 0x00080000u;
+    const unsigned e = (h & 0x7F800000u) >> 23, m = h & 0x007FFFFFu, sign = (h & 0x80000000u) >> 24;
+    if (e > 135u) return sign | 0x7Fu;
+    if (e > 120u) return sign | (((e - 120u) << 3) & 0x78u) | (m >> 20);
+    if (e > 116u) return sign | ((((0x00780000u + m) >> (140u - e)) + 1u) >> 1);
+    return sign;
+}
+__device__ __forceinline__ unsigned f32_to_fp8_bits(float f) { return f32_bits_to_fp8(__float_as_uint(f)) & 0xFFu; }
+// fp8 e4m3 (OCP "fn": bias 7, no infinities, 0x7f / 0xff are NaN) -> float32, exact
+__device__ __forceinline__ float fp8_bits_to_f32(unsigned c) {
+    const unsigned sign = (c & 0x80u) << 24, e = (c >> 3) & 0xFu, m = c & 7u;
+    if (e == 15u && m == 7u) return __uint_as_float(sign | 0x7FC00000u);
+    if (e == 0u) return __uint_as_float(sign) + (sign ? -1.f : 1.f) * static_cast<float>(m) * 0.001953125f;  // m * 2^-9
+    return __uint_as_float(sign | ((e + 120u) << 23) | (m << 20));
+}
+
 __device__ __forceinline__ float load_float(const void* p, int64_t i, int fmt) {
-    return fmt == A4G_F32 ? static_cast<const float*>(p)[i] : bf16_bits_to_f32(static_cast<const uint16_t*>(p)[i]);
+    if (fmt == A4G_F32) return static_cast<const float*>(p)[i];
+    if (fmt == A4G_FP8) return fp8_bits_to_f32(static_cast<const uint8_t*>(p)[i]);
+    return bf16_bits_to_f32(static_cast<const uint16_t*>(p)[i]);
 }
 __device__ __forceinline__ void store_float(void* p, int64_t i, int fmt, float v) {
     if (fmt == A4G_F32) static_cast<float*>(p)[i] = v;
+    else if (fmt == A4G_FP8) static_cast<uint8_t*>(p)[i] = static_cast<uint8_t>(f32_to_fp8_bits(v));
     else static_cast<uint16_t*>(p)[i] = static_cast<uint16_t>(f32_to_bf16_bits(v));
 }
-static inline int fmt_bytes(int fmt) { return fmt == A4G_F32 ? 4 : 2; }
-static inline bool fmt_ok(int fmt) { return fmt == A4G_F32 || fmt == A4G_BF16; }
+static inline int fmt_bytes(int fmt) { return fmt == A4G_F32 ? 4 : (fmt == A4G_FP8 ? 1 : 2); }
+static inline bool fmt_ok(int fmt) { return fmt == A4G_F32 || fmt == A4G_BF16 || fmt == A4G_FP8; }
 
 template <int FMT>
 struct FloatPolicy {
     using acc_t = v16f;
-    static constexpr int ES = FMT == A4G_F32 ? 4 : 2;
-    static constexpr int MMAS = FMT == A4G_F32 ? 4 : 1;
+    static constexpr int ES = FMT == A4G_F32 ? 4 : (FMT == A4G_FP8 ? 1 : 2);
+    static constexpr int MMAS = FMT == A4G_F32 ? 4 : (FMT == A4G_FP8 ? 2 : 1);
     static constexpr bool FIX_A = false;
     static constexpr int MAX_OUT_BYTES = ES;
     template <int BN>
@@ -53,6 +78,12 @@ struct FloatPolicy {
 #pragma unroll
             for (int t = 0; t < 4; ++t) c = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[t], af[t], c, 0, 0, 0);
             return c;
+        }
+        if (FMT == A4G_FP8) {
+            typedef long v2l __attribute__((ext_vector_type(2)));
+            const v2l bl = __builtin_bit_cast(v2l, b), al = __builtin_bit_cast(v2l, a);
+            c = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(bl[0], al[0], c, 0, 0, 0);
+            return __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(bl[1], al[1], c, 0, 0, 0);
         }
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, b), __builtin_bit_cast(v8bf, a), c, 0, 0, 0);
     }
@@ -92,6 +123,10 @@ struct FloatPolicy {
                     if (FMT == A4G_F32) {
                         const v4f o = {y[0], y[1], y[2], y[3]};
                         *reinterpret_cast<v4f*>(smem + ml * cpitch + nl * 4) = o;
+                    } else if (FMT == A4G_FP8) {
+                        *reinterpret_cast<unsigned*>(smem + ml * cpitch + nl) =
+                            f32_to_fp8_bits(y[0]) | (f32_to_fp8_bits(y[1]) << 8) | (f32_to_fp8_bits(y[2]) << 16) |
+                            (f32_to_fp8_bits(y[3]) << 24);
                     } else {
                         v2i o;
                         o[0] = static_cast<int>(f32_to_bf16_bits(y[0]) | (f32_to_bf16_bits(y[1]) << 16));
@@ -119,7 +154,7 @@ struct FloatGenericArgs {
 __global__ __launch_bounds__(256) void gemm_float_generic_kernel(FloatGenericArgs g) {
     const int64_t total = static_cast<int64_t>(g.M) * g.N;
     const int batch = blockIdx.y;
-    const int es = g.fmt == A4G_F32 ? 4 : 2;
+    const int es = g.fmt == A4G_F32 ? 4 : (g.fmt == A4G_FP8 ? 1 : 2);
     const char* A = static_cast<const char*>(g.A) + batch * g.stride_a * es;
     const char* B = static_cast<const char*>(g.B) + batch * g.stride_b * es;
     char* C = static_cast<char*>(g.C) + batch * g.stride_c * es;
@@ -196,7 +231,11 @@ static hipError_t launch_float_nt(const void* A, int64_t lda, int64_t stride_a, 
     if (fmt == A4G_F32) return launch_rs_policy<FloatPolicy<A4G_F32>, 128, 128, 2, 2>(g, batch, stream);
     const int64_t tiles256 = static_cast<int64_t>((M + 255) / 256) * ((N + 255) / 256) * batch;
     const int64_t rounds256 = (tiles256 + 255) / 256;
-    const bool big = M >= 256 && N >= 256 && K >= 256 && tiles256 * 100 >= rounds256 * 256 * 85;
+    const bool big = M >= 256 && N >= 256 && K * es >= 512 && tiles256 * 100 >= rounds256 * 256 * 85;
+    if (fmt == A4G_FP8) {
+        if (big) return launch_rs_policy<FloatPolicy<A4G_FP8>, 256, 256, 2, 4, true>(g, batch, stream);
+        return launch_rs_policy<FloatPolicy<A4G_FP8>, 128, 128, 2, 2>(g, batch, stream);
+    }
     if (big) return launch_rs_policy<FloatPolicy<A4G_BF16>, 256, 256, 2, 4, true>(g, batch, stream);
     return launch_rs_policy<FloatPolicy<A4G_BF16>, 128, 128, 2, 2>(g, batch, stream);
 }
@@ -210,33 +249,38 @@ static hipError_t launch_transpose(const void* B, int64_t ldb, int64_t stride_b,
     return hipGetLastError();
 }
 
+static hipError_t launch_transpose_fmt(int fmt, const void* B, int64_t ldb, int64_t stride_b, void* Bt, int64_t ldt,
+                                       int64_t stride_t, int batch, int K, int N, hipStream_t stream) {
+    if (fmt == A4G_F32) return launch_transpose<uint32_t>(B, ldb, stride_b, Bt, ldt, stride_t, batch, K, N, stream);
+    if (fmt == A4G_FP8) return launch_transpose<uint8_t>(B, ldb, stride_b, Bt, ldt, stride_t, batch, K, N, stream);
+    return launch_transpose<uint16_t>(B, ldb, stride_b, Bt, ldt, stride_t, batch, K, N, stream);
+}
+
 }  // namespace a4g
 
 using namespace a4g;
 
 extern "C" int64_t a4g_packed_ld_f(int64_t K, int fmt) {
-    const int es = fmt == A4G_F32 ? 4 : 2;
+    const int es = fmt_bytes(fmt);
     return K <= 0 ? 16 / es : round_up64(K * es, 16) / es;
 }
 
 extern "C" int a4g_pack_weights_f(const void* W, int fmt, int64_t ldw, int64_t K, int64_t N, void* Wt, a4g_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const char* who = "a4g_pack_weights_f";
-    A4G_REQUIRE(fmt_ok(fmt), A4G_ERR_UNSUPPORTED, "%s: format %d is not bfloat16 / float32", who, fmt);
+    A4G_REQUIRE(fmt_ok(fmt), A4G_ERR_UNSUPPORTED, "%s: format %d is not bfloat16 / float32 / fp8 e4m3", who, fmt);
     A4G_REQUIRE(W && Wt, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
     A4G_REQUIRE(K >= 1 && N >= 1 && K <= (1 << 24) && N <= (1 << 24) && ldw >= N, A4G_ERR_INVALID_ARGUMENT,
                 "%s: bad shape K=%lld N=%lld ldw=%lld", who, (long long)K, (long long)N, (long long)ldw);
     const int64_t ldt = a4g_packed_ld_f(K, fmt);
-    const hipError_t e = fmt == A4G_F32 ? launch_transpose<uint32_t>(W, ldw, 0, Wt, ldt, 0, 1, (int)K, (int)N, stream)
-                                        : launch_transpose<uint16_t>(W, ldw, 0, Wt, ldt, 0, 1, (int)K, (int)N, stream);
-    return check_hip(e, who);
+    return check_hip(launch_transpose_fmt(fmt, W, ldw, 0, Wt, ldt, 0, 1, (int)K, (int)N, stream), who);
 }
 
 extern "C" int a4g_dense_f(const void* A, int fmt, int64_t lda, const void* Wt, int64_t ldwt, const float* bias, int relu, void* Y,
                            int64_t ldy, int64_t M, int64_t N, int64_t K, a4g_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const char* who = "a4g_dense_f";
-    A4G_REQUIRE(fmt_ok(fmt), A4G_ERR_UNSUPPORTED, "%s: format %d is not bfloat16 / float32", who, fmt);
+    A4G_REQUIRE(fmt_ok(fmt), A4G_ERR_UNSUPPORTED, "%s: format %d is not bfloat16 / float32 / fp8 e4m3", who, fmt);
     A4G_REQUIRE(M >= 0 && N >= 1 && K >= 1 && M <= INT32_MAX && N <= (1 << 24) && K <= (1 << 24), A4G_ERR_INVALID_ARGUMENT,
                 "%s: bad shape M=%lld N=%lld K=%lld", who, (long long)M, (long long)N, (long long)K);
     A4G_REQUIRE(lda >= K && ldy >= N && ldwt >= K, A4G_ERR_INVALID_ARGUMENT, "%s: pitch smaller than the row", who);
@@ -247,7 +291,7 @@ extern "C" int a4g_dense_f(const void* A, int fmt, int64_t lda, const void* Wt, 
 
 extern "C" size_t a4g_matmul_f_workspace_bytes(int64_t batch, int64_t N, int64_t K, int trans_b, int fmt) {
     if (trans_b || batch <= 0 || N <= 0 || K <= 0) return 0;
-    return static_cast<size_t>(batch) * N * a4g_packed_ld_f(K, fmt) * (fmt == A4G_F32 ? 4 : 2);
+    return static_cast<size_t>(batch) * N * a4g_packed_ld_f(K, fmt) * fmt_bytes(fmt);
 }
 
 extern "C" int a4g_matmul_f(const void* A, int fmt, int64_t lda, int64_t stride_a, const void* B, int64_t ldb, int64_t stride_b,
@@ -255,7 +299,7 @@ extern "C" int a4g_matmul_f(const void* A, int fmt, int64_t lda, int64_t stride_
                             void* workspace, size_t workspace_bytes, a4g_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const char* who = "a4g_matmul_f";
-    A4G_REQUIRE(fmt_ok(fmt), A4G_ERR_UNSUPPORTED, "%s: format %d is not bfloat16 / float32", who, fmt);
+    A4G_REQUIRE(fmt_ok(fmt), A4G_ERR_UNSUPPORTED, "%s: format %d is not bfloat16 / float32 / fp8 e4m3", who, fmt);
     A4G_REQUIRE(batch >= 0 && batch <= 65535 && M >= 0 && N >= 1 && K >= 1 && M <= INT32_MAX && N <= (1 << 24) && K <= (1 << 24),
                 A4G_ERR_INVALID_ARGUMENT, "%s: bad shape batch=%lld M=%lld N=%lld K=%lld", who, (long long)batch, (long long)M,
                 (long long)N, (long long)K);
@@ -269,9 +313,7 @@ extern "C" int a4g_matmul_f(const void* A, int fmt, int64_t lda, int64_t stride_
     A4G_REQUIRE(workspace && workspace_bytes >= need && aligned16(workspace), A4G_ERR_WORKSPACE,
                 "%s: needs a 16-byte aligned workspace of %zu bytes (a4g_matmul_f_workspace_bytes)", who, need);
     const int64_t ldt = a4g_packed_ld_f(K, fmt);
-    hipError_t e = fmt == A4G_F32
-                       ? launch_transpose<uint32_t>(B, ldb, stride_b, workspace, ldt, N * ldt, (int)batch, (int)K, (int)N, stream)
-                       : launch_transpose<uint16_t>(B, ldb, stride_b, workspace, ldt, N * ldt, (int)batch, (int)K, (int)N, stream);
+    hipError_t e = launch_transpose_fmt(fmt, B, ldb, stride_b, workspace, ldt, N * ldt, (int)batch, (int)K, (int)N, stream);
     if (e != hipSuccess) return check_hip(e, who);
     return check_hip(launch_float_nt(A, lda, stride_a, workspace, ldt, N * ldt, nullptr, 0, C, ldc, stride_c, (int)batch, (int)M, (int)N,
                                      (int)K, fmt, stream), who);
@@ -280,7 +322,7 @@ extern "C" int a4g_matmul_f(const void* A, int fmt, int64_t lda, int64_t stride_
 extern "C" int a4g_add_f(const void* a, const void* b, void* out, int64_t n, int fmt, a4g_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const char* who = "a4g_add_f";
-    A4G_REQUIRE(fmt_ok(fmt), A4G_ERR_UNSUPPORTED, "%s: format %d is not bfloat16 / float32", who, fmt);
+    A4G_REQUIRE(fmt_ok(fmt), A4G_ERR_UNSUPPORTED, "%s: format %d is not bfloat16 / float32 / fp8 e4m3", who, fmt);
     A4G_REQUIRE(n >= 0, A4G_ERR_INVALID_ARGUMENT, "%s: negative length", who);
     if (n == 0) return A4G_OK;
     A4G_REQUIRE(a && b && out, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);

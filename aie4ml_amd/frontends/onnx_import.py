@@ -5,8 +5,7 @@ same handler registry (`@onnx_handler(*op_types)` -> `fn(ctx, node, node_name, d
 frontends/onnx/registry.py:12-34), the same lowering of QuantizeLinear / DequantizeLinear pairs to per-tensor
 power-of-two QuantIntents (frontends/onnx/quantize.py), the same node kinds, roles and metadata, and the same
 error messages. Differences: the file is decoded by onnx_proto (no protobuf dependency), static shapes come
-from the small inference table below instead of onnx.shape_inference, of the float element types FLOAT and
-BFLOAT16 are taken (the formats with a GPU kernel), and the result is a GPUModel.
+from the small inference table below instead of onnx.shape_inference, and the result is a GPUModel.
 """
 
 from __future__ import annotations
@@ -206,6 +205,7 @@ def build_shape_table(model: op.Model, initializers: Dict[str, np.ndarray], inpu
 _FLOAT_INPUT_INTENT = {
     op.FLOAT: FloatIntent(width=32, format=FloatFormat.FP32),
     op.BFLOAT16: FloatIntent(width=16, format=FloatFormat.BF16),
+    op.FLOAT8E4M3FN: FloatIntent(width=8, format=FloatFormat.FP8_E4M3),
 }
 
 
@@ -225,7 +225,7 @@ class OnnxImportContext:
         self.value_tensors: Dict[str, TensorVar] = {}   # ONNX value name -> lowered tensor
         self.q_aliases: Dict[str, Tuple[str, Any, QuantIntent, Tuple[int, ...]]] = {}  # Quantize output awaiting its Dequantize
         self.precision_mirrors: List[Tuple[str, str]] = []
-        self.bfloat16_initializers: set = set()  # names of initializers the file stores as BFLOAT16
+        self.narrow_float_initializers: Dict[str, FloatFormat] = {}  # initializers the file stores as BFLOAT16 / FLOAT8E4M3FN
 
     def mirror_precision(self, target: str, source: str) -> None:
         self.precision_mirrors.append((target, source))
@@ -294,8 +294,9 @@ class OnnxImportContext:
                                  f'got {data.dtype}.')
             # a float constant: LayerNormalization scale / bias (the operator quantises those itself, whatever the
             # intent says) or a parameter of the float compute path (intent_from_initializer, utils.py:229-241)
-            fmt = FloatFormat.BF16 if name in self.bfloat16_initializers else FloatFormat.FP32
-            return self.param_tensor(name, data, FloatIntent(width=16 if fmt is FloatFormat.BF16 else 32, format=fmt))
+            fmt = self.narrow_float_initializers.get(name, FloatFormat.FP32)
+            width = {FloatFormat.BF16: 16, FloatFormat.FP8_E4M3: 8}.get(fmt, 32)
+            return self.param_tensor(name, data, FloatIntent(width=width, format=fmt))
         raise ValueError(f'{node_name}: parameter input {name} must be a constant initializer.')
 
     def any_source_for(self, name: str, node_name: str) -> TensorVar:
@@ -690,7 +691,8 @@ def lower_onnx_model(model_or_path, config: Optional[Dict[str, Any]] = None) -> 
     backend = BackendContext(config=config)
     graph = backend.ir.logical
     initializers = {t.name: np.asarray(t.array) for t in model.graph.initializers}
-    bfloat16_initializers = {t.name for t in model.graph.initializers if t.bfloat16}
+    narrow = {t.name: (FloatFormat.BF16 if t.bfloat16 else FloatFormat.FP8_E4M3) for t in model.graph.initializers
+              if t.bfloat16 or t.float8}
     input_shapes: Dict[str, Tuple[int, ...]] = {}
     input_dtypes: Dict[str, int] = {}
     for vi in model.graph.inputs:
@@ -711,7 +713,7 @@ def lower_onnx_model(model_or_path, config: Optional[Dict[str, Any]] = None) -> 
     ctx = OnnxImportContext(backend, initializers=initializers, input_shapes=input_shapes, input_dtypes=input_dtypes,
                             shape_of=build_shape_table(model, initializers, input_shapes),
                             layer_directives=dict(config.get('LayerDirectives', {}) or {}))
-    ctx.bfloat16_initializers = bfloat16_initializers
+    ctx.narrow_float_initializers = narrow
     for index, node in enumerate(model.graph.nodes):
         name = node_name_of(node, index)
         dispatch(ctx, node, name, ctx.take_directives(name))

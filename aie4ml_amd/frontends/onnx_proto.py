@@ -18,7 +18,7 @@ import numpy as np
 
 # TensorProto.DataType
 FLOAT, UINT8, INT8, UINT16, INT16, INT32, INT64, BOOL, FLOAT16, DOUBLE = 1, 2, 3, 4, 5, 6, 7, 9, 10, 11
-BFLOAT16 = 16  # no numpy dtype: such tensors are held as float32 arrays and flagged (Tensor.bfloat16)
+BFLOAT16, FLOAT8E4M3FN = 16, 17  # no numpy dtype: held as float32 arrays and flagged (Tensor.bfloat16 / .float8)
 NP_OF = {FLOAT: np.float32, UINT8: np.uint8, INT8: np.int8, UINT16: np.uint16, INT16: np.int16, INT32: np.int32,
          INT64: np.int64, BOOL: np.bool_, FLOAT16: np.float16, DOUBLE: np.float64}
 ONNX_OF = {np.dtype(v): k for k, v in NP_OF.items()}
@@ -29,6 +29,7 @@ class Tensor:
     name: str
     array: np.ndarray
     bfloat16: bool = False  # the file stores (or shall store) the values as ONNX BFLOAT16
+    float8: bool = False    # ... as ONNX FLOAT8E4M3FN
 
 
 @dataclass
@@ -166,6 +167,13 @@ def _parse_tensor(buf: bytes) -> Tensor:
         if arr.size != count:
             raise ValueError(f'tensor {name!r}: {arr.size} values for shape {tuple(dims)}')
         return Tensor(name, arr.reshape(tuple(dims)), bfloat16=True)
+    if dtype == FLOAT8E4M3FN:  # codes in raw_data or int32_data; decoded to float32 (exact)
+        codes = np.frombuffer(raw, dtype=np.uint8) if raw is not None else np.array(i32, dtype=np.int64).astype(np.uint8)
+        arr = _fp8_decode(codes)
+        count = int(np.prod(dims)) if dims else 1
+        if arr.size != count:
+            raise ValueError(f'tensor {name!r}: {arr.size} values for shape {tuple(dims)}')
+        return Tensor(name, arr.reshape(tuple(dims)), float8=True)
     if dtype not in NP_OF:
         raise NotImplementedError(f'tensor {name!r}: ONNX data type {dtype} is not supported')
     npdt = np.dtype(NP_OF[dtype])
@@ -350,6 +358,31 @@ def _packed_ints(num: int, values) -> bytes:
     return _ld(num, b''.join(_enc_varint(int(v)) for v in values)) if len(values) else b''
 
 
+def _fp8_decode(codes: np.ndarray) -> np.ndarray:
+    """FLOAT8E4M3FN codes -> float32: bias 7, subnormals m * 2^-9, no infinities, S.1111.111 is NaN."""
+    c = codes.astype(np.int64)
+    e, m = (c >> 3) & 0xF, c & 7
+    mag = np.where(e == 0, m * 2.0 ** -9, (1.0 + m / 8.0) * np.exp2(e - 7.0))
+    mag = np.where((e == 15) & (m == 7), np.nan, mag)
+    return np.where(c & 0x80, -mag, mag).astype(np.float32)
+
+
+_FP8_VALUES = None
+
+
+def _fp8_encode_exact(values: np.ndarray, name: str) -> np.ndarray:
+    """Values that are exact in FLOAT8E4M3FN -> their codes (table lookup; anything else is an error)."""
+    global _FP8_VALUES
+    if _FP8_VALUES is None:
+        table = _fp8_decode(np.arange(256, dtype=np.uint8))
+        _FP8_VALUES = {float(v): c for c, v in enumerate(table.tolist()) if v == v and not (c == 0x80)}
+    flat = values.reshape(-1).tolist()
+    try:
+        return np.array([_FP8_VALUES[float(v) + 0.0] for v in flat], dtype=np.uint8)
+    except KeyError as exc:
+        raise ValueError(f'tensor {name!r}: value {exc.args[0]} is not exact in float8 e4m3') from None
+
+
 def _ser_tensor(t: Tensor) -> bytes:
     arr = np.ascontiguousarray(t.array)
     if t.bfloat16:
@@ -358,6 +391,9 @@ def _ser_tensor(t: Tensor) -> bytes:
             raise ValueError(f'tensor {t.name!r}: values are not exact in bfloat16')
         out = _packed_ints(1, arr.shape) + _vi(2, BFLOAT16) + _ld(8, t.name.encode())
         return out + _ld(9, (bits >> 16).astype('<u2').tobytes())
+    if t.float8:
+        codes = _fp8_encode_exact(np.ascontiguousarray(arr, dtype=np.float32), t.name)
+        return _packed_ints(1, arr.shape) + _vi(2, FLOAT8E4M3FN) + _ld(8, t.name.encode()) + _ld(9, codes.tobytes())
     if arr.dtype not in ONNX_OF:
         raise NotImplementedError(f'tensor {t.name!r}: dtype {arr.dtype} has no ONNX type here')
     out = _packed_ints(1, arr.shape) + _vi(2, ONNX_OF[arr.dtype]) + _ld(8, t.name.encode())

@@ -1,4 +1,4 @@
-"""GPU variants of the reference's float compute path: Dense, MatMul and Add on bfloat16 or float32 tensors.
+"""GPU variants of the reference's float compute path: Dense, MatMul and Add on bfloat16, float32 or fp8 e4m3 tensors.
 
 In the reference the same variant classes serve both paths and branch on FloatIntent
 (_DenseVariantBase.resolve, src/aie4ml/op_impls/families/matmul/dense.py:94-133: shift 0, accumulator
@@ -21,7 +21,7 @@ from .base import OpImplVariant, is_gpu, register_variant
 from .dense import DenseFlags, MatmulFlags
 from .precision import float_format_name, is_identity, is_last_two_swap, view_perm
 
-GPU_FLOAT_FORMATS = ('bfloat16', 'float32')
+GPU_FLOAT_FORMATS = ('bfloat16', 'float32', 'fp8_e4m3')
 
 
 @dataclass(frozen=True)
@@ -61,27 +61,54 @@ class FloatAddConfig:
         return id(self)
 
 
+def float32_to_fp8_codes(array) -> np.ndarray:
+    """float32 -> fp8 e4m3 codes (uint8), the integer recipe of the reference's _float32_to_fp8_scalar
+    (matmul/common.py:262-276): round half away from zero at mantissa bit 20, bias 7, gradual underflow,
+    magnitudes from 480 up give the code 0x7f."""
+    bits = np.ascontiguousarray(np.asarray(array, dtype=np.float32)).view(np.uint32).astype(np.int64)
+    h = (bits + 0x00080000) & 0xFFFFFFFF
+    e, m, sign = (h & 0x7F800000) >> 23, h & 0x007FFFFF, (h & 0x80000000) >> 24
+    normal = sign | (((e - 120) << 3) & 0x78) | (m >> 20)
+    sub = sign | ((((0x00780000 + m) >> np.clip(140 - e, 0, 62)) + 1) >> 1)
+    out = np.where(e > 135, sign | 0x7F, np.where(e > 120, normal, np.where(e > 116, sub, sign)))
+    return (out & 0xFF).astype(np.uint8)
+
+
+def fp8_codes_to_float32(codes) -> np.ndarray:
+    """fp8 e4m3 codes -> float32 (bias 7, subnormals m * 2^-9, 0x7f / 0xff are NaN), exact."""
+    c = np.asarray(codes, dtype=np.uint8).astype(np.int64)
+    e, m = (c >> 3) & 0xF, c & 7
+    mag = np.where(e == 0, m * 2.0 ** -9, (1.0 + m / 8.0) * np.exp2(e - 7.0))
+    mag = np.where((e == 15) & (m == 7), np.nan, mag)
+    return np.where(c & 0x80, -mag, mag).astype(np.float32)
+
+
 def pack_as_float(array, fmt: str) -> np.ndarray:
     """Parameter data -> values of the storage format, as float32 (pack_as_float, matmul/common.py:253-284:
-    bfloat16 keeps the upper 16 bits of the float32 pattern, i.e. truncates)."""
+    bfloat16 keeps the upper 16 bits of the float32 pattern, i.e. truncates; fp8 goes through the packer's
+    integer recipe)."""
     f32 = np.ascontiguousarray(np.asarray(array, dtype=np.float32))
     if fmt == 'bfloat16':
         return ((f32.view(np.uint32) >> 16) << 16).view(np.float32)
     if fmt == 'float32':
         return f32
-    raise NotImplementedError(f'float format {fmt!r} has no GPU kernel (bfloat16 and float32 do).')
+    if fmt == 'fp8_e4m3':
+        return fp8_codes_to_float32(float32_to_fp8_codes(f32))
+    raise NotImplementedError(f'float format {fmt!r} has no GPU kernel (bfloat16, float32 and fp8_e4m3 do).')
 
 
 def _torch_dtype(fmt: str):
     import torch
 
-    return {'bfloat16': torch.bfloat16, 'float32': torch.float32}[fmt]
+    return {'bfloat16': torch.bfloat16, 'float32': torch.float32, 'fp8_e4m3': torch.float8_e4m3fn}[fmt]
 
 
 def to_device_float(array, fmt: str):
     """float32 host values that are exact in `fmt` -> device tensor of that format."""
     import torch
 
+    if fmt == 'fp8_e4m3':  # by code, so that the packer's recipe (not the library's cast) decides every bit
+        return torch.from_numpy(float32_to_fp8_codes(array)).cuda().view(torch.float8_e4m3fn)
     return torch.from_numpy(np.ascontiguousarray(array, dtype=np.float32)).cuda().to(_torch_dtype(fmt))
 
 
@@ -95,7 +122,7 @@ def _float_precision(node, tensors) -> Dict[str, AIEDataType]:
         raise ValueError(f'{node.name}: float {node.op_type} requires lhs/rhs/output to share float precision.')
     fmt = fmts['lhs']
     if fmt not in GPU_FLOAT_FORMATS:
-        raise NotImplementedError(f'{node.name}: float format {fmt!r} has no GPU kernel (bfloat16 and float32 do).')
+        raise NotImplementedError(f'{node.name}: float format {fmt!r} has no GPU kernel.')
     precision = {k: AIEDataType(format=fmt) for k in tensors}
     precision['acc'] = AIEDataType(format='accfloat')
     return precision

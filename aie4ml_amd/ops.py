@@ -329,14 +329,14 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, logit_shift: in
 
 # ---- floating-point compute path (bfloat16 / float32 operands, float32 accumulation) ---------------------------
 
-_TORCH_FLOAT = {torch.bfloat16: 16, torch.float32: 17}
+_TORCH_FLOAT = {torch.bfloat16: 16, torch.float32: 17, torch.float8_e4m3fn: 18}
 
 
 def _float_format(t: torch.Tensor, name: str) -> int:
     try:
         return _TORCH_FLOAT[t.dtype]
     except KeyError:
-        raise NotImplementedError(f'{name}: the float path takes bfloat16 or float32 tensors, got {t.dtype}') from None
+        raise NotImplementedError(f'{name}: the float path takes bfloat16, float32 or float8_e4m3fn tensors, got {t.dtype}') from None
 
 
 @dataclass

@@ -6,7 +6,7 @@ Default workload: the single quantized Dense of the baseline configuration
 saturate to int8, fused ReLU). One step = one pass of the operator over the whole synthetic batch,
 inputs already resident in HBM. Prints ONE JSON line.
 
-Other workloads (--workload c2_dense_i16 | c2_dense_bf16 | c1_mlp | c3_softmax_exp | c3_softmax_hccs | c3_qk | c3_pv |
+Other workloads (--workload c2_dense_i16 | c2_dense_bf16 | c2_dense_fp8 | c1_mlp | c3_softmax_exp | c3_softmax_hccs | c3_qk | c3_pv |
 c3_attention_exp | c3_attention_hccs | c4_add_layernorm | c4_layernorm | c4_add | c5_encoder) print the same line for that operator or graph;
 --workload calib_copy runs a plain 256 MiB elementwise copy, the known-size kernel the HBM traffic
 counters are scaled against.
@@ -28,6 +28,7 @@ sys.path.insert(0, str(ROOT))
 
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, TOP/s
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, TFLOP/s
+PEAK_FP8_TFLOPS = 5000.0   # MI355X dense fp8 MFMA, TFLOP/s
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
 
 # HBM bytes per launch of each workload's dominant kernel, from hardware counters (FETCH_SIZE and
@@ -170,36 +171,45 @@ def main():
         cpu_work = 2.0 * sample_rows * N * K
         metric, unit = 'int16x8_dense_tops', 'TOP/s'
         kernel = 'gemm_i16i8_kernel'
-    elif wl == 'c2_dense_bf16':
-        # the reference's float compute path on the C2 shape: bfloat16 operands, float32 accumulation and bias
+    elif wl in ('c2_dense_bf16', 'c2_dense_fp8'):
+        # the reference's float compute path on the C2 shape: bfloat16 / fp8 e4m3 operands, float32 accumulation and bias
         M, K, N = 8192, 4096, 4096
+        fp8 = wl == 'c2_dense_fp8'
+        fmt, tdt = ('fp8_e4m3', torch.float8_e4m3fn) if fp8 else ('bfloat16', torch.bfloat16)
         r = np.random.default_rng(23)
-        A = oracle.bf16_truncate(r.normal(0, 1.0, (M, K)).astype(np.float32))
-        W = oracle.bf16_truncate(r.normal(0, 0.02, (K, N)).astype(np.float32))
+        A32 = r.normal(0, 1.0, (M, K)).astype(np.float32)
+        W32 = r.normal(0, 0.02, (K, N)).astype(np.float32)
         bias = r.normal(0, 0.1, N).astype(np.float32)
-        p = ops.pack_dense_float(torch.from_numpy(W).cuda().to(torch.bfloat16), torch.from_numpy(bias).cuda())
-        dA = torch.from_numpy(A).cuda().to(torch.bfloat16)
-        out = torch.empty((M, N), dtype=torch.bfloat16, device='cuda')
+        if fp8:  # the library's device cast makes the operands (round to nearest even); what it made is what both sides use
+            dA = torch.from_numpy(A32).cuda().to(tdt)
+            dW = torch.from_numpy(W32).cuda().to(tdt)
+            A, W = dA.float().cpu().numpy(), dW.float().cpu().numpy()
+        else:
+            A, W = oracle.bf16_truncate(A32), oracle.bf16_truncate(W32)
+            dA, dW = torch.from_numpy(A).cuda().to(tdt), torch.from_numpy(W).cuda().to(tdt)
+        p = ops.pack_dense_float(dW, torch.from_numpy(bias).cuda())
+        out = torch.empty((M, N), dtype=tdt, device='cuda')
         fn = lambda: ops.dense_float(dA, p, relu=True, out=out)  # noqa: E731
         fn()
-        rows = r.choice(M, 64, replace=False)
-        exp = oracle.dense_float(A[rows], W, bias, relu=True, fmt='bfloat16')
+        rows = r.choice(M, 16 if fp8 else 64, replace=False)
+        exp = oracle.dense_float(A[rows], W, bias, relu=True, fmt=fmt)
         torch.cuda.synchronize()
         got = out[torch.from_numpy(rows).cuda()].float().cpu().numpy()
-        # float path: no bit-exactness across summation orders; the reference's own tolerance (rtol 1e-2, atol 5e-2)
-        bit_exact = bool(np.allclose(got, exp, rtol=1e-2, atol=5e-2))
-        extra['parity'] = 'within rtol 1e-2 / atol 5e-2 of the exact-accumulation oracle (float path)'
+        # float path: no bit-exactness across summation orders. bfloat16: the reference's own tolerance; fp8 (no
+        # reference test): one unit in the last place of the output format
+        rtol, atol = (2.0 ** -3, 2.0 ** -9) if fp8 else (1e-2, 5e-2)
+        bit_exact = bool(np.allclose(got, exp, rtol=rtol, atol=atol))
+        extra['parity'] = f'within rtol {rtol:g} / atol {atol:g} of the exact-accumulation oracle (float path)'
         extra['max_abs_err'] = float(np.max(np.abs(got - exp)))
         work, bound = 2.0 * M * N * K, 'mfma'
-        peak_mfma, mfma_unit = PEAK_BF16_TFLOPS, 'TFLOP/s'
+        peak_mfma, mfma_unit = (PEAK_FP8_TFLOPS if fp8 else PEAK_BF16_TFLOPS), 'TFLOP/s'
         samples = M
-        config = {'workload': 'c2_dense_bf16: Dense 8192x4096 -> 4096, bfloat16 operands, float32 accumulate + bias, ReLU, '
-                              'bfloat16 out (round to nearest even)'}
-        sample_rows = 256
+        config = {'workload': f'{wl}: Dense 8192x4096 -> 4096, {fmt} operands, float32 accumulate + bias, ReLU, {fmt} out'}
+        sample_rows = 64 if fp8 else 256
         cpu_desc = f'oracle float Dense (float64 numpy matmul) on the first {sample_rows} of {M} rows, scaled per op'
-        cpu_fn = lambda: oracle.dense_float(A[:sample_rows], W, bias, relu=True, fmt='bfloat16')  # noqa: E731
+        cpu_fn = lambda: oracle.dense_float(A[:sample_rows], W, bias, relu=True, fmt=fmt)  # noqa: E731
         cpu_work = 2.0 * sample_rows * N * K
-        metric, unit = 'bf16_dense_tflops', 'TFLOP/s'
+        metric, unit = ('fp8_dense_tflops' if fp8 else 'bf16_dense_tflops'), 'TFLOP/s'
         kernel = 'gemm_rs_kernel'
     elif wl == 'c1_mlp':
         x, layers = workloads.c1_mlp(1024)
@@ -426,7 +436,7 @@ def main():
     line = {
         'metric': metric, 'value': float(f'{value:.6g}'), 'unit': unit, 'n_gpus': 1, 'steps': args.steps,
         'warmup': args.warmup, 'ms_per_step': round(ms, 5), 'higher_is_better': True, 'scaling': 'weak',
-        'vs_baseline': None, 'dtype': {'c2_dense_i16': 'int16', 'c2_dense_bf16': 'bf16'}.get(wl, 'int8'), 'data': 'synthetic', 'config': config,
+        'vs_baseline': None, 'dtype': {'c2_dense_i16': 'int16', 'c2_dense_bf16': 'bf16', 'c2_dense_fp8': 'fp8'}.get(wl, 'int8'), 'data': 'synthetic', 'config': config,
         'samples_per_s': float(f'{samples / (ms * 1e-3):.6g}'), 'bit_exact': bit_exact,
         'roofline': roof, 'cpu_baseline': cpu, 'launch': 'hip_graph' if graphed else 'eager',
     }

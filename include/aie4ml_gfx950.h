@@ -206,11 +206,12 @@ A4G_API int a4g_attention_i8(const int8_t* Q, const int8_t* K, const int8_t* V, 
                      int inv_shift, int use_clb, int out_shift, int out_round_mode, a4g_stream_t stream);
 
 /* ---- Floating-point compute path ------------------------------------------------------------------
- * The reference's float mode (FloatIntent tensors, passes/force_float_mode.py): bfloat16 or float32
- * operands, float32 accumulation (acc_scalar_t = accfloat), results rounded to the operand format with
- * round-to-nearest-even (dense.py:105-127: shift 0, rounding_mode 'conv_even'). Operands, weights and
+ * The reference's float mode (FloatIntent tensors, passes/force_float_mode.py): bfloat16, float32 or fp8
+ * e4m3 operands, float32 accumulation (acc_scalar_t = accfloat), results converted to the operand format:
+ * round-to-nearest-even for bfloat16 / float32 (dense.py:105-127: shift 0, rounding_mode 'conv_even'), the
+ * integer recipe of the reference's own packer for fp8 (matmul/common.py:262-276). Operands, weights and
  * results of one call share one format (resolver.py:125-129). Sizes and pitches count elements. */
-enum a4g_float_format { A4G_BF16 = 16, A4G_F32 = 17 };
+enum a4g_float_format { A4G_BF16 = 16, A4G_F32 = 17, A4G_FP8 = 18 /* e4m3, bias 7, as the matrix cores read it */ };
 
 /* Row pitch (elements) of a packed float weight matrix: rows start 16-byte aligned. */
 A4G_API int64_t a4g_packed_ld_f(int64_t K, int fmt);

@@ -235,7 +235,45 @@ def bf16_round(x):
     return np.where(np.isnan(x), np.float32(np.nan), out)
 
 
+def fp8_encode(x):
+    """float32 -> fp8 e4m3 codes by the reference's packer recipe (_float32_to_fp8_scalar,
+    matmul/common.py:262-276), one value at a time as written there."""
+    flat = np.ascontiguousarray(x, dtype=np.float32).reshape(-1)
+    out = np.empty(flat.size, dtype=np.uint8)
+    for i, bits in enumerate(flat.view(np.uint32).tolist()):
+        h = (bits + 0x00080000) & 0xFFFFFFFF
+        e = (h & 0x7F800000) >> 23
+        m = h & 0x007FFFFF
+        sign = (h & 0x80000000) >> 24
+        if e > 135:
+            r = sign | 0x7F
+        elif e > 120:
+            r = sign | (((e - 120) << 3) & 0x78) | (m >> 20)
+        elif e > 116:
+            r = sign | (((0x00780000 + m) >> (140 - e)) + 1) >> 1
+        else:
+            r = sign
+        out[i] = r & 0xFF
+    return out.reshape(np.shape(x))
+
+
+def fp8_decode(codes):
+    """fp8 e4m3 codes -> float32: bias 7, subnormals m * 2^-9, no infinities, 0x7f / 0xff NaN."""
+    c = np.asarray(codes, dtype=np.uint8).astype(np.int64)
+    e, m = (c >> 3) & 0xF, c & 7
+    mag = np.where(e == 0, m * 2.0 ** -9, (1.0 + m / 8.0) * np.exp2(e - 7.0))
+    mag = np.where((e == 15) & (m == 7), np.nan, mag)
+    return np.where(c & 0x80, -mag, mag).astype(np.float32)
+
+
+def fp8_quantize(x):
+    """float -> nearest fp8 e4m3 value by the packer recipe, as float32."""
+    return fp8_decode(fp8_encode(np.asarray(x, dtype=np.float32)))
+
+
 def to_float_format(x, fmt):
+    if fmt == 'fp8_e4m3':
+        return fp8_quantize(np.asarray(x, dtype=np.float64).astype(np.float32))
     if fmt == 'bfloat16':
         return bf16_round(np.asarray(x, dtype=np.float64).astype(np.float32))
     if fmt == 'float32':

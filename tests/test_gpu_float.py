@@ -13,9 +13,11 @@ torch = pytest.importorskip('torch')
 
 pytestmark = pytest.mark.gpu
 
-REF_TOL = {'bfloat16': (1e-2, 5e-2), 'float32': (1e-3, 1e-3)}
-TORCH_DT = {'bfloat16': torch.bfloat16, 'float32': torch.float32}
-HALF_ULP = {'bfloat16': 2.0 ** -8, 'float32': 2.0 ** -24}
+# fp8: the reference has no fp8 test; the bar is one unit in the last place (relative 2^-3) of the output format
+REF_TOL = {'bfloat16': (1e-2, 5e-2), 'float32': (1e-3, 1e-3), 'fp8_e4m3': (2.0 ** -3, 2.0 ** -9)}
+TORCH_DT = {'bfloat16': torch.bfloat16, 'float32': torch.float32, 'fp8_e4m3': torch.float8_e4m3fn}
+HALF_ULP = {'bfloat16': 2.0 ** -8, 'float32': 2.0 ** -24, 'fp8_e4m3': 2.0 ** -4}
+FORMATS = ['bfloat16', 'float32', 'fp8_e4m3']
 
 
 @pytest.fixture(scope='module')
@@ -29,10 +31,15 @@ def ops():
 
 def operand(r, shape, fmt, oracle, scale=1.0):
     x = (r.normal(0, scale, shape)).astype(np.float32)
+    if fmt == 'fp8_e4m3':
+        return oracle.fp8_quantize(x)
     return oracle.bf16_truncate(x) if fmt == 'bfloat16' else x
 
 
 def dev(a, fmt):
+    if fmt == 'fp8_e4m3':  # by code: the values are exact in the format, the codes are the oracle's
+        from oracle import oracle as o
+        return torch.from_numpy(o.fp8_encode(np.ascontiguousarray(a, dtype=np.float32))).cuda().view(torch.float8_e4m3fn)
     return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).cuda().to(TORCH_DT[fmt])
 
 
@@ -47,10 +54,12 @@ def check(got, exp, fmt, k, abs_products):
     # float32 accumulation of k terms, any order: |err| <= k * 2^-24 * sum|a||w|; then one rounding of the
     # result (half an ulp), which can land on the neighbouring value when the two sums straddle a tie
     bound = 2.0 * HALF_ULP[fmt] * np.abs(exp) + (k + 2) * 2.0 ** -24 * abs_products + 1e-30
+    if fmt == 'fp8_e4m3':
+        bound = bound + 2.0 ** -9  # one step of the subnormal range
     assert np.all(np.abs(got.astype(np.float64) - exp.astype(np.float64)) <= bound)
 
 
-@pytest.mark.parametrize('fmt', ['bfloat16', 'float32'])
+@pytest.mark.parametrize('fmt', FORMATS)
 @pytest.mark.parametrize('shape', [(4, 32, 32), (4, 32, 16), (7, 19, 5), (130, 96, 70), (256, 256, 256), (300, 128, 260),
                                    (512, 1024, 384), (1024, 64, 64)])
 def test_dense_float(ops, oracle, fmt, shape):
@@ -68,12 +77,13 @@ def test_dense_float(ops, oracle, fmt, shape):
     check(host(ops.dense_float(dev(A, fmt), p0)), oracle.dense_float(A, W, None, fmt=fmt), fmt, K, absprod)
 
 
-@pytest.mark.parametrize('fmt', ['bfloat16', 'float32'])
+@pytest.mark.parametrize('fmt', FORMATS)
 def test_dense_float_exact_cases(ops, oracle, fmt):
     # small integers: every product and partial sum is exact in float32, so any order gives the same bits
     r = np.random.default_rng(5)
-    A = r.integers(-8, 9, (200, 128)).astype(np.float32)
-    W = r.integers(-4, 5, (128, 192)).astype(np.float32)
+    amax, wmax = (2, 1) if fmt == 'fp8_e4m3' else (8, 4)  # fp8: keep every sum below the largest value, 448
+    A = r.integers(-amax, amax + 1, (200, 128)).astype(np.float32)
+    W = r.integers(-wmax, wmax + 1, (128, 192)).astype(np.float32)
     b = r.integers(-16, 17, 192).astype(np.float32)
     p = ops.pack_dense_float(dev(W, fmt), torch.from_numpy(b).cuda())
     got = host(ops.dense_float(dev(A, fmt), p, relu=True))
@@ -87,7 +97,7 @@ def test_dense_float_exact_cases(ops, oracle, fmt):
     assert tuple(empty.shape) == (0, 64)
 
 
-@pytest.mark.parametrize('fmt', ['bfloat16', 'float32'])
+@pytest.mark.parametrize('fmt', FORMATS)
 @pytest.mark.parametrize('trans_b', [True, False])
 @pytest.mark.parametrize('shape', [((2, 3), 64, 64, 64), ((4,), 128, 96, 32), ((), 130, 70, 48), ((2,), 50, 17, 24),
                                    ((3,), 256, 128, 256)])
@@ -102,7 +112,7 @@ def test_matmul_float(ops, oracle, fmt, trans_b, shape):
     check(got, oracle.matmul_float(A, B, trans_b=trans_b, fmt=fmt), fmt, K, absprod)
 
 
-@pytest.mark.parametrize('fmt', ['bfloat16', 'float32'])
+@pytest.mark.parametrize('fmt', FORMATS)
 def test_add_float(ops, oracle, fmt):
     r = np.random.default_rng(9)
     a = operand(r, (5, 1001), fmt, oracle, 3.0)

@@ -451,8 +451,14 @@ def test_float_mode_rules():
         lower(_float_mlp(in_prec=bf, w_prec=qint(8, 6)))
     with pytest.raises(ValueError, match='share float precision'):
         lower(_float_mlp(in_prec=bf, w_prec=f32))
-    with pytest.raises(NotImplementedError, match='no GPU kernel'):
-        lower(_float_mlp(in_prec=FloatIntent(8, FloatFormat.FP8_E4M3), w_prec=FloatIntent(8, FloatFormat.FP8_E4M3)))
+    f8 = FloatIntent(8, FloatFormat.FP8_E4M3)
+    cfg = lower(_float_mlp(in_prec=f8, w_prec=f8)).ir.execution.get('dense0_aie').config
+    assert cfg.precision['lhs'].format == 'fp8_e4m3' and cfg.precision['bias'].format == 'float32'
+    # the fp8 packer: ties away from zero, bias 7, 0x7f from 480 up (matmul/common.py:262-276)
+    from aie4ml_amd.op_impls.float_ops import float32_to_fp8_codes, fp8_codes_to_float32
+    assert float32_to_fp8_codes([0.0, 1.0, -1.0, 1.0625, 448.0, 464.0, 2.0 ** -9, 0.3]).tolist() == \
+        [0x00, 0x38, 0xB8, 0x39, 0x7E, 0x7F, 0x01, 0x2A]
+    assert fp8_codes_to_float32([0x38, 0x7E, 0x01, 0x2A, 0xB9]).tolist() == [1.0, 448.0, 2.0 ** -9, 0.3125, -1.125]
     # a power-of-two scale cannot fold into a float dense
     gb = GraphBuilder()
     x = gb.input('x', (4, 32), bf)

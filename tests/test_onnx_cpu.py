@@ -159,7 +159,7 @@ def test_float_onnx_graph_imports_with_float_intents():
     r = np.random.default_rng(0)
     for elem, bf in ((op.FLOAT, False), (op.BFLOAT16, True)):
         def cast(a):
-            a = np.asarray(a, dtype=np.float32)
+            a = np.ascontiguousarray(a, dtype=np.float32)
             return ((a.view(np.uint32) >> 16) << 16).view(np.float32) if bf else a
 
         g = op.Graph(name='float_mlp')
@@ -181,3 +181,25 @@ def test_float_onnx_graph_imports_with_float_intents():
         assert [n.op_type for n in ctx.ir.logical.nodes] == ['dense', 'dense']
         cfg = ctx.ir.execution.get(ctx.ir.logical.nodes[0].name).config
         assert cfg.accumulator_tag == 'accfloat' and cfg.flags.use_relu and cfg.flags.use_bias
+
+
+def test_float8_onnx_tensors_round_trip_and_import():
+    from aie4ml_amd.aie_types import FloatFormat
+    from aie4ml_amd.frontends import onnx_proto as op
+    from aie4ml_amd.frontends.onnx_import import lower_onnx_model
+    from aie4ml_amd.op_impls.float_ops import pack_as_float
+
+    w = pack_as_float(np.random.default_rng(2).normal(0, 0.5, (16, 8)), 'fp8_e4m3')
+    g = op.Graph(name='f8')
+    g.inputs.append(op.ValueInfo('x', op.FLOAT8E4M3FN, (4, 16)))
+    g.initializers.append(op.Tensor('w', w, float8=True))
+    g.nodes.append(op.Node('MatMul', ['x', 'w'], ['y'], 'fc', {}))
+    g.outputs.append(op.ValueInfo('y', op.FLOAT8E4M3FN, (4, 8)))
+    blob = op.serialize_model(op.Model(graph=g, opset={'': 19}, producer_name='test'))
+    back = op.parse_model(blob).graph.initializers[0]
+    assert back.float8 and np.array_equal(back.array, w)
+    ctx = lower_onnx_model(blob, {})
+    assert {t.precision.format for t in ctx.ir.logical.tensors.values()} == {FloatFormat.FP8_E4M3}
+    with pytest.raises(ValueError, match='not exact in float8'):
+        op.serialize_model(op.Model(graph=op.Graph(name='bad', initializers=[op.Tensor('w', np.float32([0.3]), float8=True)]),
+                                    opset={'': 19}, producer_name='test'))

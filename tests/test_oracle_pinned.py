@@ -387,3 +387,25 @@ def test_float_dense_oracle_against_float64_identity_and_linearity(oracle):
     assert np.array_equal(oracle.dense_float(A, np.eye(40, dtype=np.float32), None, fmt='bfloat16'), A)
     assert np.array_equal(oracle.matmul_float(A, W.T.copy(), trans_b=True, fmt='float32'),
                           oracle.matmul_float(A, W, fmt='float32'))
+
+
+def test_fp8_e4m3_codec_against_torch_cpu(oracle):
+    torch = pytest.importorskip('torch')
+    codes = np.arange(256, dtype=np.uint8)
+    want = torch.from_numpy(codes).view(torch.float8_e4m3fn).float().numpy()      # independent decoder
+    got = oracle.fp8_decode(codes)
+    assert np.array_equal(np.isnan(got), np.isnan(want)) and np.array_equal(got[~np.isnan(got)], want[~np.isnan(want)])
+    fin = ~np.isnan(got)
+    assert np.array_equal(oracle.fp8_encode(got[fin]), codes[fin])               # every value encodes to its own code
+    # away from ties and below the largest value both round to nearest: the recipe must agree with torch's cast
+    r = np.random.default_rng(8)
+    x = np.concatenate([r.normal(0, 1, 20000), r.normal(0, 30, 5000), r.normal(0, 0.01, 5000)]).astype(np.float32)
+    x = x[np.abs(x) < 440]
+    t = torch.from_numpy(x).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    mine = oracle.fp8_encode(x)
+    lo, hi = np.minimum(oracle.fp8_decode(mine), oracle.fp8_decode(t)), np.maximum(oracle.fp8_decode(mine), oracle.fp8_decode(t))
+    tie = (lo != hi) & (np.abs((lo.astype(np.float64) + hi) / 2 - x) == 0)
+    assert np.all((mine == t) | tie | ((mine & 0x7F) == 0) & ((t & 0x7F) == 0))   # +-0 may differ in sign handling
+    # ties go away from zero (the recipe adds half a step to the magnitude), overflow gives 0x7f
+    assert oracle.fp8_encode(np.float32([1.0625, -1.0625, 464.0, 480.0, 1e9, 2.0 ** -10, 2.0 ** -9])).tolist() == \
+        [0x39, 0xB9, 0x7F, 0x7F, 0x7F, 0x01, 0x01]
