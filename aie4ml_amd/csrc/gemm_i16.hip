@@ -166,6 +166,216 @@ __global__ __launch_bounds__(256) void gemm_i16i8_generic_kernel(Gemm16Args g) {
     }
 }
 
+// -----------------------------------------------------------------------------------------------------
+// Dense with int16 activations and int16 weights: the reference's (16, 16) combination, whose accumulator is
+// acc64 (op_impls/utils/precision.py:122-123). Both operands are split into byte planes, both low planes are
+// fed biased by 128:  a = a' + 128, w = w' + 128 with a' = 256 ah + al', w' = 256 wh + wl', so
+//   sum a w = 65536 sum(ah wh) + 256 (sum(ah wl') + sum(al' wh)) + sum(al' wl')
+//             + 128 sum_k a'[m,k] + 128 sum_k w'[k,n] + 16384 K.
+// Four int32 accumulator sets per output block (each exact for K <= 32768), the column term from the packed
+// weights, the row term from the A fragments the lanes hold anyway (v_dot4 against ones), all combined in
+// 64-bit arithmetic in the epilogue.
+// -----------------------------------------------------------------------------------------------------
+struct Gemm16x16Args {
+    const int16_t* A;
+    const int8_t *Wh, *Wl;    // [N][ldwt] planes: signed high bytes, low bytes ^ 0x80
+    const int32_t* colsum;    // [N] sum_k (w[k][n] - 128)
+    const int32_t* bias;      // [N] or null
+    const int32_t* shifts;
+    void* Y;
+    int64_t lda, ldwt, ldy;
+    int M, N, K;
+    int shift_stride, relu, out_kind, mode;
+};
+
+__device__ __forceinline__ long long round_shift64(long long v, int s, int mode) {
+    if (s <= 0) return v;
+    const long long q = v >> s;
+    const unsigned long long r = static_cast<unsigned long long>(v) & ((1ull << s) - 1ull), h = 1ull << (s - 1);
+    switch (mode) {
+    case A4G_RND_FLOOR: return q;
+    case A4G_RND_CEIL: return q + (r != 0ull);
+    case A4G_RND_POSITIVE_INF: return q + (r >= h);
+    case A4G_RND_NEGATIVE_INF: return q + (r > h);
+    case A4G_RND_SYMMETRIC_INF: return q + ((r > h) | ((r == h) & (v >= 0)));
+    case A4G_RND_SYMMETRIC_ZERO: return q + ((r > h) | ((r == h) & (v < 0)));
+    case A4G_RND_CONV_EVEN: return q + ((r > h) | ((r == h) & ((q & 1) != 0)));
+    default: return q + ((r > h) | ((r == h) & ((q & 1) == 0)));
+    }
+}
+
+__device__ __forceinline__ int requant64(long long v, int s, int mode, int lo, int hi) {
+    const long long y = round_shift64(v, s, mode);
+    return static_cast<int>(y < lo ? lo : (y > hi ? hi : y));
+}
+
+// 64 x 128 output tile, K step 64, 4 waves (2 x 2) of 32 x 64, double-buffered LDS with the two byte planes
+// of both operands. Requires K % 16 == 0, 16-byte aligned rows.
+__global__ __launch_bounds__(256) void gemm_i16i16_kernel(Gemm16x16Args g) {
+    constexpr int BM = 64, BN = 128, BK = 64, PITCH = BK + 16;
+    constexpr int APLANE = BM * PITCH, WPLANE = BN * PITCH, STAGE = 2 * APLANE + 2 * WPLANE;
+    __shared__ __attribute__((aligned(16))) int8_t smem[2 * STAGE];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int tiles_n = (g.N + BN - 1) / BN;
+    const int m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN;
+
+    // staging: A tile = 64 rows x 8 chunks of 8 int16 (2 per thread); each W plane = 128 rows x 4 chunks (2 per thread)
+    v4i ra[2], rh[2], rl[2];
+    auto load_tile = [&](int k0) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int c = tid + i * 256, row = c >> 3, kc = (c & 7) * 8;
+            const int gm = min(m0 + row, g.M - 1);
+            ra[i] = (k0 + kc < g.K) ? *reinterpret_cast<const v4i*>(g.A + static_cast<int64_t>(gm) * g.lda + k0 + kc)
+                                    : v4i{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int c = tid + i * 256, row = c >> 2, kc = (c & 3) * 16;
+            const int gn = min(n0 + row, g.N - 1);
+            const bool in = k0 + kc < g.K;
+            // past the end of K the planes must contribute nothing: (0, 0) pairs with the zeroed A planes below
+            rh[i] = in ? *reinterpret_cast<const v4i*>(g.Wh + static_cast<int64_t>(gn) * g.ldwt + k0 + kc) : v4i{0, 0, 0, 0};
+            rl[i] = in ? *reinterpret_cast<const v4i*>(g.Wl + static_cast<int64_t>(gn) * g.ldwt + k0 + kc) : v4i{0, 0, 0, 0};
+        }
+    };
+    auto store_tile = [&](int buf, int k0) {
+        int8_t* st = smem + buf * STAGE;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int c = tid + i * 256, row = c >> 3, kc = (c & 7) * 8;
+            const unsigned w0 = ra[i][0], w1 = ra[i][1], w2 = ra[i][2], w3 = ra[i][3];
+            const bool in = k0 + kc < g.K;
+            const unsigned flip = in ? 0x80808080u : 0u;  // beyond K: both planes zero, so the row sums stay exact
+            v2i hi = {static_cast<int>(__builtin_amdgcn_perm(w1, w0, 0x07050301u)), static_cast<int>(__builtin_amdgcn_perm(w3, w2, 0x07050301u))};
+            v2i lo = {static_cast<int>(__builtin_amdgcn_perm(w1, w0, 0x06040200u) ^ flip),
+                      static_cast<int>(__builtin_amdgcn_perm(w3, w2, 0x06040200u) ^ flip)};
+            *reinterpret_cast<v2i*>(st + row * PITCH + kc) = hi;
+            *reinterpret_cast<v2i*>(st + APLANE + row * PITCH + kc) = lo;
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int c = tid + i * 256, row = c >> 2, kc = (c & 3) * 16;
+            *reinterpret_cast<v4i*>(st + 2 * APLANE + row * PITCH + kc) = rh[i];
+            *reinterpret_cast<v4i*>(st + 2 * APLANE + WPLANE + row * PITCH + kc) = rl[i];
+        }
+    };
+
+    v16i acc_hh[2], acc_hl[2], acc_lh[2], acc_ll[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc_hh[j][r] = acc_hl[j][r] = acc_lh[j][r] = acc_ll[j][r] = 0;
+    int rs_hi = 0, rs_lo = 0;  // this lane's share of sum_k ah[m,k] and sum_k al'[m,k] for row m = lane % 32
+
+    const int frow = lane & 31, fk = (lane >> 5) * 16;
+    const int a_off = (wm * 32 + frow) * PITCH + fk, b_off = 2 * APLANE + (wn * 64 + frow) * PITCH + fk;
+    const int ktiles = (g.K + BK - 1) / BK;
+    load_tile(0);
+    store_tile(0, 0);
+    __syncthreads();
+    for (int kt = 0; kt < ktiles; ++kt) {
+        const int8_t* st = smem + (kt & 1) * STAGE;
+        if (kt + 1 < ktiles) load_tile((kt + 1) * BK);
+#pragma unroll
+        for (int kk = 0; kk < BK / 32; ++kk) {
+            const v4i ah = *reinterpret_cast<const v4i*>(st + a_off + kk * 32);
+            const v4i al = *reinterpret_cast<const v4i*>(st + APLANE + a_off + kk * 32);
+            v4i bh[2], bl[2];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                bh[j] = *reinterpret_cast<const v4i*>(st + b_off + j * 32 * PITCH + kk * 32);
+                bl[j] = *reinterpret_cast<const v4i*>(st + WPLANE + b_off + j * 32 * PITCH + kk * 32);
+            }
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                rs_hi = __builtin_amdgcn_sdot4(ah[t], 0x01010101, rs_hi, false);
+                rs_lo = __builtin_amdgcn_sdot4(al[t], 0x01010101, rs_lo, false);
+            }
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                acc_hh[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bh[j], ah, acc_hh[j], 0, 0, 0);
+                acc_hl[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bl[j], ah, acc_hl[j], 0, 0, 0);
+                acc_lh[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bh[j], al, acc_lh[j], 0, 0, 0);
+                acc_ll[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bl[j], al, acc_ll[j], 0, 0, 0);
+            }
+        }
+        if (kt + 1 < ktiles) store_tile((kt + 1) & 1, (kt + 1) * BK);
+        __syncthreads();
+    }
+    // the other half of the row's k range sits in lane ^ 32
+    rs_hi += __shfl_xor(rs_hi, 32);
+    rs_lo += __shfl_xor(rs_lo, 32);
+    const long long row_term = 128ll * (256ll * rs_hi + rs_lo) + 16384ll * g.K;
+
+    const int lo_b = g.relu ? max(kind_lo(g.out_kind), 0) : kind_lo(g.out_kind), hi_b = kind_hi(g.out_kind);
+    const int obytes = (g.out_kind == A4G_I16 || g.out_kind == A4G_U16) ? 2 : 1;
+    int8_t* Yb = static_cast<int8_t*>(g.Y);
+    const int m = m0 + wm * 32 + (lane & 31);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int n = n0 + wn * 64 + j * 32 + 8 * q + 4 * (lane >> 5);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                if (m >= g.M || n + t >= g.N) continue;
+                const int nn = n + t;
+                const long long v = (static_cast<long long>(acc_hh[j][q * 4 + t]) << 16) +
+                                    ((static_cast<long long>(acc_hl[j][q * 4 + t]) + acc_lh[j][q * 4 + t]) << 8) +
+                                    acc_ll[j][q * 4 + t] + row_term + 128ll * g.colsum[nn] + (g.bias ? g.bias[nn] : 0);
+                const int s = min(max(g.shifts[static_cast<int64_t>(nn) * g.shift_stride], 0), 62);
+                const int y = requant64(v, s, g.mode, lo_b, hi_b);
+                const int64_t at = static_cast<int64_t>(m) * g.ldy + nn;
+                if (obytes == 1) Yb[at] = static_cast<int8_t>(y);
+                else reinterpret_cast<int16_t*>(Yb)[at] = static_cast<int16_t>(y);
+            }
+        }
+    }
+}
+
+// Any K / alignment: one thread per output element, straight from the planes (w = 256 wh + (wl ^ 0x80 as unsigned)).
+__global__ __launch_bounds__(256) void gemm_i16i16_generic_kernel(Gemm16x16Args g) {
+    const int64_t total = static_cast<int64_t>(g.M) * g.N;
+    const int lo_b = g.relu ? max(kind_lo(g.out_kind), 0) : kind_lo(g.out_kind), hi_b = kind_hi(g.out_kind);
+    for (int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; idx < total;
+         idx += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+        const int m = static_cast<int>(idx / g.N), n = static_cast<int>(idx % g.N);
+        long long acc = g.bias ? g.bias[n] : 0;
+        const int16_t* ar = g.A + static_cast<int64_t>(m) * g.lda;
+        const int8_t* wh = g.Wh + static_cast<int64_t>(n) * g.ldwt;
+        const int8_t* wl = g.Wl + static_cast<int64_t>(n) * g.ldwt;
+        for (int k = 0; k < g.K; ++k) {
+            const int w = 256 * static_cast<int>(wh[k]) + static_cast<int>(static_cast<uint8_t>(wl[k]) ^ 0x80u);
+            acc += static_cast<long long>(ar[k]) * w;
+        }
+        const int s = min(max(g.shifts[static_cast<int64_t>(n) * g.shift_stride], 0), 62);
+        store_kind(g.Y, static_cast<int64_t>(m) * g.ldy + n, g.out_kind, requant64(acc, s, g.mode, lo_b, hi_b));
+    }
+}
+
+// W [K][ldw] int16 -> planes [N][ldt] (signed high byte; low byte ^ 0x80), zero padding, and colsum[n] = sum_k (w - 128).
+__global__ __launch_bounds__(256) void pack_planes_i16_kernel(const int16_t* __restrict__ W, int64_t ldw, int8_t* __restrict__ Wh,
+                                                              int8_t* __restrict__ Wl, int64_t ldt, int32_t* __restrict__ colsum,
+                                                              int K, int N) {
+    const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    if (n >= N) return;
+    int sum = 0;
+    for (int k = 0; k < K; ++k) {
+        const int w = W[static_cast<int64_t>(k) * ldw + n];
+        Wh[static_cast<int64_t>(n) * ldt + k] = static_cast<int8_t>(w >> 8);
+        Wl[static_cast<int64_t>(n) * ldt + k] = static_cast<int8_t>((w & 0xFF) ^ 0x80);
+        sum += w - 128;
+    }
+    for (int k = K; k < ldt; ++k) {
+        Wh[static_cast<int64_t>(n) * ldt + k] = 0;
+        Wl[static_cast<int64_t>(n) * ldt + k] = 0;
+    }
+    colsum[n] = sum;
+}
+
 }  // namespace a4g
 
 using namespace a4g;
@@ -202,6 +412,55 @@ extern "C" int a4g_dense_i16(const int16_t* A, int64_t lda, const int8_t* Wt, in
     } else {
         const int grid = static_cast<int>(std::min<int64_t>((M * N + 255) / 256, 256 * 32));
         gemm_i16i8_generic_kernel<<<grid, 256, 0, stream>>>(g);
+    }
+    return check_hip(hipGetLastError(), who);
+}
+
+extern "C" int a4g_pack_weights_i16(const int16_t* W, int64_t ldw, int64_t K, int64_t N, int8_t* Wt_hi, int8_t* Wt_lo,
+                                    int32_t* colsum, a4g_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const char* who = "a4g_pack_weights_i16";
+    A4G_REQUIRE(W && Wt_hi && Wt_lo && colsum, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+    A4G_REQUIRE(K >= 1 && N >= 1 && K <= 32768 && N <= (1 << 24) && ldw >= N, A4G_ERR_INVALID_ARGUMENT,
+                "%s: bad shape K=%lld (at most 32768) N=%lld ldw=%lld", who, (long long)K, (long long)N, (long long)ldw);
+    const int64_t ldt = K <= 0 ? 16 : (K + 15) / 16 * 16;
+    pack_planes_i16_kernel<<<static_cast<unsigned>((N + 255) / 256), 256, 0, stream>>>(W, ldw, Wt_hi, Wt_lo, ldt, colsum,
+                                                                                      static_cast<int>(K), static_cast<int>(N));
+    return check_hip(hipGetLastError(), who);
+}
+
+extern "C" int a4g_dense_i16x16(const int16_t* A, int64_t lda, const int8_t* Wt_hi, const int8_t* Wt_lo, int64_t ldwt,
+                                const int32_t* colsum, const int32_t* bias, const int32_t* shifts, int n_shift, int round_mode,
+                                int relu, int out_kind, void* Y, int64_t ldy, int64_t M, int64_t N, int64_t K,
+                                a4g_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const char* who = "a4g_dense_i16x16";
+    A4G_REQUIRE(M >= 0 && N >= 1 && K >= 1 && M <= INT32_MAX && N <= (1 << 24) && K <= 32768, A4G_ERR_INVALID_ARGUMENT,
+                "%s: bad shape M=%lld N=%lld K=%lld (K at most 32768)", who, (long long)M, (long long)N, (long long)K);
+    A4G_REQUIRE(out_kind == A4G_I8 || out_kind == A4G_U8 || out_kind == A4G_I16, A4G_ERR_UNSUPPORTED,
+                "%s: output kind %d is not int8/uint8/int16", who, out_kind);
+    A4G_REQUIRE(valid_round(round_mode), A4G_ERR_INVALID_ARGUMENT, "%s: unknown rounding mode %d", who, round_mode);
+    A4G_REQUIRE(n_shift == 1 || n_shift == N, A4G_ERR_INVALID_ARGUMENT, "%s: n_shift must be 1 or N=%lld, got %d", who,
+                (long long)N, n_shift);
+    A4G_REQUIRE(lda >= K && ldy >= N && ldwt >= K, A4G_ERR_INVALID_ARGUMENT, "%s: pitch smaller than the row", who);
+    if (M == 0) return A4G_OK;
+    A4G_REQUIRE(A && Wt_hi && Wt_lo && Y && shifts && colsum, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+    Gemm16x16Args g{};
+    g.A = A; g.Wh = Wt_hi; g.Wl = Wt_lo; g.colsum = colsum; g.bias = bias; g.shifts = shifts; g.Y = Y;
+    g.lda = lda; g.ldwt = ldwt; g.ldy = ldy;
+    g.M = static_cast<int>(M); g.N = static_cast<int>(N); g.K = static_cast<int>(K);
+    g.shift_stride = n_shift == 1 ? 0 : 1;
+    g.relu = relu != 0;
+    g.out_kind = out_kind;
+    g.mode = round_mode;
+    const bool tiled = K % 16 == 0 && lda % 8 == 0 && ldwt % 16 == 0 && aligned16(A) && aligned16(Wt_hi) && aligned16(Wt_lo);
+    if (tiled) {
+        const int64_t tiles = ((M + 63) / 64) * ((N + 127) / 128);
+        A4G_REQUIRE(tiles <= INT32_MAX, A4G_ERR_UNSUPPORTED, "%s: too many tiles", who);
+        gemm_i16i16_kernel<<<static_cast<unsigned>(tiles), 256, 0, stream>>>(g);
+    } else {
+        const int grid = static_cast<int>(std::min<int64_t>((M * N + 255) / 256, 256 * 32));
+        gemm_i16i16_generic_kernel<<<grid, 256, 0, stream>>>(g);
     }
     return check_hip(hipGetLastError(), who);
 }

@@ -77,8 +77,9 @@ def _resolve_numeric(node) -> Dict[str, AIEDataType]:
     if resolved['lhs'].width <= 8 and resolved['rhs'].width > 8:
         raise RuntimeError(f'{node.name}: unsupported int8 x int16 precision mix for AIE implementations; '
                            'no implementation variant available.')
-    # 8 x 8 accumulates in 32 bits (infer_accumulator_tag, precision.py:116-119)
-    resolved['acc'] = AIEDataType(format='int32', frac=int(resolved['lhs'].frac + resolved['rhs'].frac))
+    # 8 x 8 and 16 x 8 accumulate in 32 bits, 16 x 16 in 64 (infer_accumulator_tag, precision.py:116-123)
+    wide = resolved['lhs'].width > 8 and resolved['rhs'].width > 8
+    resolved['acc'] = AIEDataType(format='int64' if wide else 'int32', frac=int(resolved['lhs'].frac + resolved['rhs'].frac))
     return resolved
 
 
@@ -105,8 +106,8 @@ def _resolve_output_scale_shift(node) -> int:
     return shift
 
 
-# (lhs, rhs) storage widths; (16, 8) for Dense only (the reference's list also has (16, 16), with a 64-bit accumulator)
-_SUPPORTED_INT_WIDTH_COMBOS = frozenset({(8, 8), (16, 8)})
+# (lhs, rhs) storage widths (matmul/common.py:52); the 16-bit ones for Dense only (dynamic MatMul kernels are int8)
+_SUPPORTED_INT_WIDTH_COMBOS = frozenset({(8, 8), (16, 8), (16, 16)})
 
 
 def _bitwidths_supported(node, device) -> bool:
@@ -187,7 +188,7 @@ class DenseGpuVariant(OpImplVariant):
             precision=precision,
             shift=int(shift),
             shift_per_channel=per_channel,
-            accumulator_tag='acc32',
+            accumulator_tag='acc64' if precision['acc'].format == 'int64' else 'acc32',
             rounding_mode=aie_rounding_token(precision['output']),
             flags=DenseFlags(use_relu=use_relu,
                              transpose_lhs=bool(lhs_perm is not None and lhs_perm[-1] != len(lhs_perm) - 1),
@@ -199,14 +200,16 @@ class DenseGpuVariant(OpImplVariant):
     def validate_config(self, node, config: DenseConfig, _device) -> None:
         if config.shift < 0:
             raise ValueError(f'{node.name}: dense accumulator output shift must be non-negative, got {config.shift}.')
-        if config.shift > 31:
-            raise ValueError(f'{node.name}: dense accumulator output shift {config.shift} exceeds the 32-bit accumulator.')
+        top = 62 if config.accumulator_tag == 'acc64' else 31
+        if config.shift > top:
+            raise ValueError(f'{node.name}: dense accumulator output shift {config.shift} exceeds the '
+                             f'{top + 1 if top == 31 else 64}-bit accumulator.')
         if config.shift_per_channel is not None:
             if len(config.shift_per_channel) != config.n_out:
                 raise ValueError(f'{node.name}: shift_per_channel needs {config.n_out} entries, got '
                                  f'{len(config.shift_per_channel)}.')
-            if min(config.shift_per_channel) < 0 or max(config.shift_per_channel) > 31:
-                raise ValueError(f'{node.name}: per-channel shifts must be in [0, 31].')
+            if min(config.shift_per_channel) < 0 or max(config.shift_per_channel) > top:
+                raise ValueError(f'{node.name}: per-channel shifts must be in [0, {top}].')
         _check_out_format(node, config.precision['output'].format)
         lhs_perm = view_perm(node, input_tensor_for_role(node, 'lhs'), 'inputs')
         if not (is_identity(lhs_perm) or is_last_two_swap(lhs_perm)):
@@ -229,6 +232,8 @@ class DenseGpuVariant(OpImplVariant):
                                    signed=bi.signed if bi else True,
                                    rounding_mode=bi.rounding if bi else inst.config.precision['bias'].rounding,
                                    saturation_mode=b.precision.saturation if bi else inst.config.precision['bias'].saturation)
+        if wi.width > 8:
+            return W.astype(np.int16 if wi.signed else np.uint16), bias
         return W.astype(np.int8 if wi.signed else np.uint8), bias
 
     def pack(self, inst) -> Dict[str, Any]:
@@ -237,7 +242,7 @@ class DenseGpuVariant(OpImplVariant):
         from .. import ops
 
         W, bias = self.quantize_weight_bias(inst)
-        if W.dtype != np.int8:
+        if W.dtype not in (np.int8, np.int16):
             raise ValueError(f'{inst.name}: dense weights must use a signed integer precision.')
         cfg = inst.config
         shifts = cfg.shift_per_channel if cfg.shift_per_channel is not None else cfg.shift

@@ -77,12 +77,13 @@ def add(a: torch.Tensor, b: torch.Tensor, shift: int = 0, rounding='floor', out:
 class PackedDense:
     """Device-resident Dense parameters in the layout the GEMM kernel consumes."""
 
-    wt: torch.Tensor       # [N, ldwt] int8, reduction axis contiguous, zero padded
+    wt: torch.Tensor       # [N, ldwt] int8, reduction axis contiguous, zero padded (int16 weights: their high bytes)
     colsum: torch.Tensor   # [N] int32
     bias: Optional[torch.Tensor]  # [N] int32 or None
     shifts: torch.Tensor   # [1] or [N] int32
     K: int
     N: int
+    wt_lo: Optional[torch.Tensor] = None  # int16 weights only: the low-byte plane (bytes ^ 0x80)
 
     @property
     def ldwt(self) -> int:
@@ -92,15 +93,20 @@ class PackedDense:
 def pack_dense(weight: torch.Tensor, bias: Optional[torch.Tensor], shifts) -> PackedDense:
     """weight: logical [K, N] int8 on the device; bias: [N] int32 or None; shifts: int or [N] ints."""
     _dev(weight, 'weight')
-    if weight.dtype != torch.int8 or weight.dim() != 2:
-        raise ValueError('weight matrix must be a rank-2 int8 tensor')
+    if weight.dtype not in (torch.int8, torch.int16) or weight.dim() != 2:
+        raise ValueError('weight matrix must be a rank-2 int8 (or int16) tensor')
     weight = weight.contiguous()
     K, N = int(weight.shape[0]), int(weight.shape[1])
     L = _lib.load()
     ldwt = int(L.a4g_packed_ld(K))
     wt = torch.empty((N, ldwt), dtype=torch.int8, device=weight.device)
     colsum = torch.empty((N,), dtype=torch.int32, device=weight.device)
-    check(L.a4g_pack_weights_i8(_ptr(weight), N, K, N, _ptr(wt), _ptr(colsum), _stream()))
+    wt_lo = None
+    if weight.dtype == torch.int16:
+        wt_lo = torch.empty((N, ldwt), dtype=torch.int8, device=weight.device)
+        check(L.a4g_pack_weights_i16(_ptr(weight), N, K, N, _ptr(wt), _ptr(wt_lo), _ptr(colsum), _stream()))
+    else:
+        check(L.a4g_pack_weights_i8(_ptr(weight), N, K, N, _ptr(wt), _ptr(colsum), _stream()))
     if bias is not None:
         bias = _dev(bias, 'bias').to(torch.int32).contiguous()
         if bias.numel() != N:
@@ -108,9 +114,10 @@ def pack_dense(weight: torch.Tensor, bias: Optional[torch.Tensor], shifts) -> Pa
     sh = torch.as_tensor(shifts, dtype=torch.int32).reshape(-1)
     if sh.numel() not in (1, N):
         raise ValueError(f'shifts must hold 1 or {N} entries, got {sh.numel()}')
-    if int(sh.min()) < 0 or int(sh.max()) > 31:
-        raise ValueError(f'dense accumulator output shift must be in [0, 31], got [{int(sh.min())}, {int(sh.max())}].')
-    return PackedDense(wt=wt, colsum=colsum, bias=bias, shifts=sh.to(weight.device), K=K, N=N)
+    top = 62 if wt_lo is not None else 31
+    if int(sh.min()) < 0 or int(sh.max()) > top:
+        raise ValueError(f'dense accumulator output shift must be in [0, {top}], got [{int(sh.min())}, {int(sh.max())}].')
+    return PackedDense(wt=wt, colsum=colsum, bias=bias, shifts=sh.to(weight.device), K=K, N=N, wt_lo=wt_lo)
 
 
 def dense(x: torch.Tensor, p: PackedDense, rounding='floor', relu: bool = False, out_kind='int8',
@@ -126,6 +133,15 @@ def dense(x: torch.Tensor, p: PackedDense, rounding='floor', relu: bool = False,
     if out is None:
         out = torch.empty(tuple(x.shape[:-1]) + (p.N,), dtype=_KIND_TORCH[ok], device=x.device)
     y2 = out.reshape(-1, p.N)
+    if p.wt_lo is not None:
+        if x2.dtype != torch.int16:
+            raise RuntimeError('unsupported int8 x int16 precision mix for AIE implementations; no implementation variant '
+                               'available.')
+        check(_lib.load().a4g_dense_i16x16(_ptr(x2), x2.stride(0) if M > 0 else p.K, _ptr(p.wt), _ptr(p.wt_lo), p.ldwt,
+                                           _ptr(p.colsum), _ptr(p.bias), _ptr(p.shifts), int(p.shifts.numel()), _mode(rounding),
+                                           int(bool(relu)), ok, _ptr(y2), y2.stride(0) if M > 0 else p.N, M, p.N, p.K,
+                                           _stream()))
+        return out
     if x2.dtype == torch.int16:
         check(_lib.load().a4g_dense_i16(_ptr(x2), x2.stride(0) if M > 0 else p.K, _ptr(p.wt), p.ldwt, _ptr(p.colsum),
                                         _ptr(p.bias), _ptr(p.shifts), int(p.shifts.numel()), _mode(rounding),

@@ -110,6 +110,17 @@ A4G_API int a4g_dense_i16(const int16_t* A, int64_t lda, const int8_t* Wt, int64
                   const int32_t* bias, const int32_t* shifts, int n_shift, int round_mode, int relu, int out_kind,
                   void* Y, int64_t ldy, int64_t M, int64_t N, int64_t K, a4g_stream_t stream);
 
+/* Dense with int16 activations and int16 weights: the reference's (16, 16) combination, accumulated in acc64
+ * (op_impls/families/matmul/common.py:52, op_impls/utils/precision.py:122-123), bias int32 at the accumulator
+ * scale. a4g_pack_weights_i16 turns W [K][ldw] int16 into two byte planes [N][ld] (ld = K rounded up to 16:
+ * signed high bytes; low bytes ^ 0x80) and colsum[n] = sum_k (W[k][n] - 128); K <= 32768 keeps every partial
+ * sum exact. Shifts up to 62. Other arguments as a4g_dense_i8. */
+A4G_API int a4g_pack_weights_i16(const int16_t* W, int64_t ldw, int64_t K, int64_t N, int8_t* Wt_hi, int8_t* Wt_lo,
+                         int32_t* colsum, a4g_stream_t stream);
+A4G_API int a4g_dense_i16x16(const int16_t* A, int64_t lda, const int8_t* Wt_hi, const int8_t* Wt_lo, int64_t ldwt,
+                     const int32_t* colsum, const int32_t* bias, const int32_t* shifts, int n_shift, int round_mode,
+                     int relu, int out_kind, void* Y, int64_t ldy, int64_t M, int64_t N, int64_t K, a4g_stream_t stream);
+
 /* ---- Dynamic MatMul (both operands activations) --------------------------------------------------
  * C[b] = saturate(round((A[b] x B[b]) >> shift)), no bias, no ReLU, for b in [0, batch).
  * Replaces matmul_single/first/middle/last<Cfg>::run, templates/nnet_utils/matmul/matmul.cpp:31-390,

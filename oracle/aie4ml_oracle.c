@@ -174,6 +174,26 @@ A4O_EXPORT int a4o_dense_i8(const void* A, int a_kind, int64_t lda,
     return 0;
 }
 
+/* Dense with int16 activations and int16 weights: the (16, 16) width combination, accumulated in acc64
+ * (op_impls/families/matmul/common.py:52, op_impls/utils/precision.py:122-123); bias stays int32 at the
+ * accumulator scale (matmul/resolver.py:147-157). Same kernel text as above, wider accumulator. */
+A4O_EXPORT int a4o_dense_i16x16(const int16_t* A, int64_t lda, const int16_t* W, int64_t ldw, const int32_t* bias,
+                                const int32_t* shifts, int n_shift, int mode, int relu, int out_kind, void* Y, int64_t ldy,
+                                int64_t M, int64_t N, int64_t K) {
+    if (!(n_shift == 1 || n_shift == N)) return -1;
+#pragma omp parallel for schedule(static)
+    for (int64_t m = 0; m < M; ++m) {
+        for (int64_t n = 0; n < N; ++n) {
+            int64_t acc = bias ? bias[n] : 0;
+            for (int64_t k = 0; k < K; ++k) acc += (int64_t)A[m * lda + k] * (int64_t)W[k * ldw + n];
+            int64_t y = srs(acc, shifts[n_shift == 1 ? 0 : n], mode, out_kind);
+            if (relu && y < 0) y = 0;
+            store_kind(Y, (size_t)(m * ldy + n), out_kind, y);
+        }
+    }
+    return 0;
+}
+
 /* MatMul: c = srs(wrap32(sum_k a[m,k]*b[k,n]), SHIFT); no bias, no ReLU. matmul.cpp:80-115.
  * trans_b: B is given as [N][K] (the last-two-axes transpose of the logical [K][N] operand, the
  * io_view perm of matmul.py:86-95 / TRANSPOSE_B matmul.cpp:70-76). batch > 1 = independent rank-2

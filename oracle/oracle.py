@@ -49,6 +49,7 @@ def lib():
         _lib.a4o_srs.argtypes = [ctypes.c_int32, i32, i32, i32]
         _lib.a4o_srs.restype = ctypes.c_int32
         _lib.a4o_dense_i8.argtypes = [vp, i32, i64, vp, i64, vp, vp, i32, i32, i32, i32, vp, i64, i64, i64, i64]
+        _lib.a4o_dense_i16x16.argtypes = [vp, i64, vp, i64, vp, vp, i32, i32, i32, i32, vp, i64, i64, i64, i64]
         _lib.a4o_matmul_i8.argtypes = [vp, i32, i64, i64, vp, i64, i64, i32, vp, i64, i64, i64, i64, i64, i64,
                                        i32, i32, i32]
         _lib.a4o_add.argtypes = [vp, vp, vp, i64, i32, i32, i32]
@@ -95,15 +96,23 @@ def srs(acc, shift, mode, kind='int8'):
 
 
 def dense(A, W, bias, shifts, mode, relu=False, out='int8'):
-    """A [M,K] int8/uint8, W [K,N] int8, bias [N] int32 or None, shifts scalar or [N]."""
+    """A [M,K] int8/uint8/int16, W [K,N] int8 (or int16 with int16 A: 64-bit accumulator), bias [N] int32 or None,
+    shifts scalar or [N]."""
     A = _c(A)
-    W = _c(W, np.int8)
+    wide = np.asarray(W).dtype == np.int16  # (16, 16): int16 weights, 64-bit accumulator
+    W = _c(W, np.int16 if wide else np.int8)
     M, K = A.shape
     K2, N = W.shape
     assert K == K2
     b = _c(bias, np.int32) if bias is not None else None
     sh = _c(np.atleast_1d(shifts), np.int32)
     Y = np.empty((M, N), dtype=_KIND_NP[KIND[out]])
+    if wide:
+        assert A.dtype == np.int16
+        rc = lib().a4o_dense_i16x16(_ptr(A), K, _ptr(W), N, _ptr(b), _ptr(sh), sh.size, _mode(mode), int(bool(relu)),
+                                    KIND[out], _ptr(Y), N, M, N, K)
+        _check(rc, 'dense 16x16')
+        return Y
     rc = lib().a4o_dense_i8(_ptr(A), _NP_KIND[A.dtype], K, _ptr(W), N, _ptr(b), _ptr(sh), sh.size, _mode(mode),
                             int(bool(relu)), KIND[out], _ptr(Y), N, M, N, K)
     _check(rc, 'dense')

@@ -45,14 +45,17 @@ def wrap32(v: int) -> int:
     return v - (1 << 32) if v >= (1 << 31) else v
 
 
-def dense(A, W, bias, shifts, mode, relu, kind):
-    """dense_bias_relu.cpp:112-163."""
+def dense(A, W, bias, shifts, mode, relu, kind, acc64=False):
+    """dense_bias_relu.cpp:112-163. acc64: the (16, 16) width combination, whose accumulator does not wrap at
+    32 bits (precision.py:122-123)."""
     M, K = A.shape
     N = W.shape[1]
     out = np.zeros((M, N), dtype=NPDT[kind])
     for m in range(M):
         for n in range(N):
-            acc = wrap32(int(bias[n]) + sum(int(A[m, k]) * int(W[k, n]) for k in range(K)))
+            acc = int(bias[n]) + sum(int(A[m, k]) * int(W[k, n]) for k in range(K))
+            if not acc64:
+                acc = wrap32(acc)
             y = srs(acc, int(shifts[n]), mode, kind)
             out[m, n] = max(y, 0) if relu else y
     return out
@@ -158,6 +161,22 @@ def main():
     d['y__i16in__conv_even__i16'] = dense(A16, W, bias, np.full(20, 9), 'conv_even', False, 'int16')
     d['y__i16in__symmetric_inf__i8relu'] = dense(A16, W, bias, shifts + 8, 'symmetric_inf', True, 'int8')
     np.savez_compressed(HERE / 'dense.npz', **d)
+
+    # ---- dense, int16 x int16 with a 64-bit accumulator (its own generator: the vectors above stay as they are) ---
+    r16 = np.random.default_rng(20250301)
+    A16b = r16.integers(-32768, 32768, (10, 48)).astype(np.int16)
+    W16 = r16.integers(-32768, 32768, (48, 12)).astype(np.int16)
+    A16b[0, :], W16[:, 0] = -32768, -32768          # the largest products: 48 * 2^30 needs more than 32 bits
+    A16b[1, :], W16[:, 1] = 32767, -32768
+    bias16 = r16.integers(-2**31, 2**31, 12).astype(np.int64)
+    d16 = {'A': A16b, 'W': W16, 'bias': bias16.astype(np.int32)}
+    sh16 = r16.integers(14, 30, 12).astype(np.int32)
+    d16['shifts'] = sh16
+    for mode in MODES:
+        d16[f'y__{mode}__i16'] = dense(A16b, W16, bias16, sh16, mode, False, 'int16', acc64=True)
+    d16['y__conv_even__i8relu__s24'] = dense(A16b, W16, bias16, np.full(12, 24), 'conv_even', True, 'int8', acc64=True)
+    d16['y__floor__i16__s36'] = dense(A16b, W16, bias16, np.full(12, 36), 'floor', False, 'int16', acc64=True)
+    np.savez_compressed(HERE / 'dense16.npz', **d16)
 
     # ---- matmul (batched, both operand orders, uint8 left operand) -------------------------------------
     Aq = gauss8(r, 30, (2, 10, 32))

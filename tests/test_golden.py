@@ -43,6 +43,12 @@ def test_oracle_dense_matmul_add(oracle):
     np.testing.assert_array_equal(oracle.dense(g['A16'], g['W'], g['bias'], 9, 'conv_even', out='int16'), g['y__i16in__conv_even__i16'])
     np.testing.assert_array_equal(oracle.dense(g['A16'], g['W'], g['bias'], g['shifts'] + 8, 'symmetric_inf', relu=True),
                                   g['y__i16in__symmetric_inf__i8relu'])
+    g16 = load('dense16')
+    for mode in MODES:
+        np.testing.assert_array_equal(oracle.dense(g16['A'], g16['W'], g16['bias'], g16['shifts'], mode, out='int16'),
+                                      g16[f'y__{mode}__i16'])
+    np.testing.assert_array_equal(oracle.dense(g16['A'], g16['W'], g16['bias'], 24, 'conv_even', relu=True), g16['y__conv_even__i8relu__s24'])
+    np.testing.assert_array_equal(oracle.dense(g16['A'], g16['W'], g16['bias'], 36, 'floor', out='int16'), g16['y__floor__i16__s36'])
     m = load('matmul')
     for mode in ('conv_even', 'symmetric_inf', 'floor'):
         np.testing.assert_array_equal(oracle.matmul(m['Aq'], m['Bk'], 5, mode, trans_b=True), m[f'qk__{mode}'])
@@ -109,6 +115,14 @@ def test_gpu_dense_matmul_add():
                                   g['y__i16in__conv_even__i16'])
     np.testing.assert_array_equal(_host(ops.dense(_dev(g['A16']), ops.pack_dense(W, bias, g['shifts'] + 8), 'symmetric_inf', relu=True)),
                                   g['y__i16in__symmetric_inf__i8relu'])
+    g16 = load('dense16')
+    for mode in MODES:
+        p16 = ops.pack_dense(_dev(g16['W']), _dev(g16['bias']), g16['shifts'])
+        np.testing.assert_array_equal(_host(ops.dense(_dev(g16['A']), p16, mode, out_kind='int16')), g16[f'y__{mode}__i16'])
+    np.testing.assert_array_equal(_host(ops.dense(_dev(g16['A']), ops.pack_dense(_dev(g16['W']), _dev(g16['bias']), 24), 'conv_even',
+                                                  relu=True)), g16['y__conv_even__i8relu__s24'])
+    np.testing.assert_array_equal(_host(ops.dense(_dev(g16['A']), ops.pack_dense(_dev(g16['W']), _dev(g16['bias']), 36), 'floor',
+                                                  out_kind='int16')), g16['y__floor__i16__s36'])
     m = load('matmul')
     for mode in ('conv_even', 'symmetric_inf', 'floor'):
         np.testing.assert_array_equal(_host(ops.matmul(_dev(m['Aq']), _dev(m['Bk']), 5, mode, trans_b=True)), m[f'qk__{mode}'])

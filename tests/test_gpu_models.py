@@ -215,6 +215,27 @@ def test_int16_activation_mlp_graph(oracle):
     _graph_check(model, oracle, {'x': x})
 
 
+def test_int16_weight_mlp_graph(oracle):
+    """16-bit activations and 16-bit weights (hls4ml's default ap_fixed<16, 6> everywhere): the (16, 16)
+    combination with its 64-bit accumulator, through the graph executor."""
+    r = np.random.default_rng(29)
+    gb = GraphBuilder()
+    t = gb.input('x', (32, 48), qint(16, 10))
+    dims = [48, 80, 10]
+    for i in range(2):
+        W = r.integers(-32768, 32768, (dims[i], dims[i + 1])) / 2.0 ** 14
+        b = r.integers(-2 ** 20, 2 ** 20, dims[i + 1]) / 2.0 ** 24
+        t = gb.dense(t, W, qint(16, 14), qint(16, 10), bias=b, bias_precision=qint(32, 24), relu=i < 1, name=f'fc{i}')
+    gb.output(t)
+    model = gb.build()
+    model.compile()
+    cfg = model.context.ir.execution.get('fc0_aie').config
+    assert cfg.accumulator_tag == 'acc64' and cfg.shift == 14
+    assert model.context.config['gpu_fusion_plan']['mlp_chains'] == []
+    x = r.integers(-32768, 32768, (32, 48)).astype(np.int16)
+    _graph_check(model, oracle, {'x': x})
+
+
 # ---- float compute path through the graph executor ----------------------------------------------------------------
 
 def _float_net(compute_dtype, batch, n_in=32, n_h=32, n_out=16, seed=0):

@@ -249,6 +249,30 @@ def test_dense_int16_activations(ops, oracle, shape):
 MODES8 = ('floor', 'ceil', 'positive_inf', 'negative_inf', 'symmetric_inf', 'symmetric_zero', 'conv_even', 'conv_odd')
 
 
+@pytest.mark.parametrize('shape', [(300, 200, 256), (64, 128, 64), (33, 17, 48), (70, 130, 1000), (5, 9, 23), (512, 384, 512),
+                                   (65, 129, 4096)])
+def test_dense_int16_activations_int16_weights(ops, oracle, shape):
+    # the (16, 16) width combination: 64-bit accumulator, byte-plane matrix-core kernel or the generic one
+    M, N, K = shape
+    r = rng(M + N + K)
+    A = r.integers(-32768, 32768, (M, K)).astype(np.int16)
+    W = r.integers(-32768, 32768, (K, N)).astype(np.int16)
+    A[0, :], W[:, 0] = -32768, -32768
+    if M > 1 and N > 1:
+        A[1, :], W[:, 1] = 32767, -32768
+    bias = r.integers(-2**31, 2**31, N).astype(np.int32)
+    shifts = r.integers(14, 32, N).astype(np.int32)
+    p = ops.pack_dense(dev(W), dev(bias), shifts)
+    for mode in MODES:
+        got = host(ops.dense(dev(A), p, mode, out_kind='int16'))
+        assert np.array_equal(got, oracle.dense(A, W, bias, shifts, mode, out='int16')), mode
+    p2 = ops.pack_dense(dev(W), None, 40)
+    assert np.array_equal(host(ops.dense(dev(A), p2, 'conv_even', relu=True, out_kind='int8')),
+                          oracle.dense(A, W, None, 40, 'conv_even', relu=True, out='int8'))
+    with pytest.raises(RuntimeError, match='int8 x int16'):
+        ops.dense(dev(A.astype(np.int8)), p, 'floor')
+
+
 @pytest.mark.parametrize('shape', [((2, 3), 200, 96, 32), ((5,), 129, 544, 64), ((2,), 31, 1056, 96), ((), 512, 512, 128),
                                    ((3,), 1, 32, 64)])
 def test_matmul_short_reduction_transposed_rhs(ops, oracle, shape):

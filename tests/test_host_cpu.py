@@ -259,6 +259,18 @@ def test_matmul_rules():
     gb.output(gb.dense(a, np.zeros((32, 8)), qint(8, 7), qint(16, 8), name='fc'))
     cfg = lower(gb).ir.execution.get('fc_aie').config
     assert cfg.precision['lhs'].format == 'int16' and cfg.shift == 8 + 7 - 8 and cfg.accumulator_tag == 'acc32'
+    # 16 x 16 accumulates in 64 bits (precision.py:122-123); 8-bit activations with 16-bit weights have no variant
+    gb = GraphBuilder()
+    a = gb.input('a', (2, 16, 32), qint(16, 8))
+    gb.output(gb.dense(a, np.zeros((32, 8)), qint(16, 14), qint(16, 8), name='fc'))
+    cfg = lower(gb).ir.execution.get('fc_aie').config
+    assert cfg.precision['rhs'].format == 'int16' and cfg.accumulator_tag == 'acc64' and cfg.shift == 14
+    assert cfg.precision['acc'].format == 'int64' and cfg.precision['bias'].format == 'int32'
+    gb = GraphBuilder()
+    a = gb.input('a', (2, 16, 32), qint(8, 4))
+    gb.output(gb.dense(a, np.zeros((32, 8)), qint(16, 14), qint(16, 8), name='fc'))
+    with pytest.raises((RuntimeError, ValueError)):
+        lower(gb)
     gb = GraphBuilder()
     a = gb.input('a', (2, 16, 32), qint(16, 8))
     b = gb.input('b', (2, 32, 16), qint(8, 4))

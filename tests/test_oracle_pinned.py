@@ -409,3 +409,17 @@ def test_fp8_e4m3_codec_against_torch_cpu(oracle):
     # ties go away from zero (the recipe adds half a step to the magnitude), overflow gives 0x7f
     assert oracle.fp8_encode(np.float32([1.0625, -1.0625, 464.0, 480.0, 1e9, 2.0 ** -10, 2.0 ** -9])).tolist() == \
         [0x39, 0xB9, 0x7F, 0x7F, 0x7F, 0x01, 0x01]
+
+
+def test_dense_int16x16_against_python_integers(oracle):
+    r = np.random.default_rng(12)
+    A = r.integers(-32768, 32768, (6, 50)).astype(np.int16)
+    W = r.integers(-32768, 32768, (50, 7)).astype(np.int16)
+    A[0, :], W[:, 0] = -32768, -32768     # 50 * 2^30: the 64-bit accumulator must not wrap at 32 bits
+    bias = r.integers(-2**31, 2**31, 7).astype(np.int32)
+    for mode, s in (('floor', 20), ('conv_even', 17), ('symmetric_inf', 33), ('ceil', 0)):
+        got = oracle.dense(A, W, bias, s, mode, out='int16')
+        for m in range(6):
+            for n in range(7):
+                acc = int(bias[n]) + sum(int(A[m, k]) * int(W[k, n]) for k in range(50))
+                assert got[m, n] == exact_srs(acc, s, mode, 'int16'), (mode, m, n)
