@@ -421,6 +421,18 @@ def test_softmax_hccs(ops, oracle, cols, params):
         assert np.array_equal(got, oracle.softmax_hccs(x, B, S, Dmax, inv_shift=inv_shift)), inv_shift
 
 
+@pytest.mark.parametrize('cols', [512, 256, 1024, 2048])
+def test_softmax_large_inputs(ops, oracle, cols):
+    # 2^24 elements: every workgroup makes many passes over its rows
+    rows = (1 << 24) // cols + 37
+    x = gauss8(rng(cols), 30, (rows, cols))
+    x[5, :] = 7                       # uniform row
+    x[6, :], x[6, 3] = -128, 127      # widest gap
+    assert np.array_equal(host(ops.softmax_exp(dev(x), 23)), oracle.softmax_exp(x, 23))
+    if cols == 512:
+        assert np.array_equal(host(ops.softmax_hccs(dev(x), 60, 1, 59)), oracle.softmax_hccs(x, 60, 1, 59))
+
+
 def test_softmax_validation_errors(ops):
     x = torch.zeros((4, 512), dtype=torch.int8, device='cuda')
     with pytest.raises(ValueError, match='cols \\* B <= 32767'):
