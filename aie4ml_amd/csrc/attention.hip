@@ -48,10 +48,12 @@ __device__ __forceinline__ void transpose4x4(const unsigned a[4], unsigned c[4])
 template <int NT, int DT, int BIT, bool FASTP>
 __global__ __launch_bounds__(256, 2) void attention_kernel(AttnArgs a) {
     constexpr int SK = NT * 32, D = DT * 32, PITCH = SK + 16;
+    // The score table is a static array: its LDS address is then a compile-time constant that folds into the
+    // offset field of the gathers (an array inside the dynamic block costs one address add per gather).
+    __shared__ int table[256];                                     // score of a gap d in [0,255]
     extern __shared__ __attribute__((aligned(16))) int8_t attn_smem[];
     int8_t* vt = attn_smem;                                        // V^T, k-permuted: [D][PITCH]
-    int* table = reinterpret_cast<int*>(attn_smem + D * PITCH);    // score of a gap d in [0,255]
-    int* colsum = table + 256;                                     // sum_k V[k][n]
+    int* colsum = reinterpret_cast<int*>(attn_smem + D * PITCH);   // sum_k V[k][n]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int m = lane & 31, half = lane >> 5;
@@ -236,7 +238,7 @@ static void launch_attention_nt(int grid, size_t lds, hipStream_t stream, const 
 
 template <int DT>
 static int launch_attention(int nt, int grid, hipStream_t stream, const AttnArgs& a) {
-    const size_t lds = static_cast<size_t>(DT * 32) * (nt * 32 + 16) + 256 * 4 + DT * 32 * 4;
+    const size_t lds = static_cast<size_t>(DT * 32) * (nt * 32 + 16) + DT * 32 * 4;  // V^T + column sums
     switch (nt) {
     case 1: launch_attention_nt<1, DT>(grid, lds, stream, a); break;
     case 2: launch_attention_nt<2, DT>(grid, lds, stream, a); break;
