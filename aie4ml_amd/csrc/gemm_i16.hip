@@ -8,6 +8,7 @@
 // per output block then give  a.w = 256 * sum(hi.w) + sum((lo-128).w) + 128 * sum(w),  all in wrapping
 // 32-bit arithmetic, which is exactly the acc32 the reference computes.
 #include "common.hpp"
+#include "gemm_rs.hpp"  // tile_coord: the XCD-aware workgroup -> tile mapping shared with the int8 kernels
 
 namespace a4g {
 
@@ -32,8 +33,12 @@ __global__ __launch_bounds__(256) void gemm_i16i8_kernel(Gemm16Args g) {
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int tiles_n = (g.N + BN - 1) / BN;
-    const int m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN;
+    GemmArgs shape{};
+    shape.M = g.M;
+    shape.N = g.N;
+    const TileCoord tc = tile_coord<BM, BN>(shape);
+    if (!tc.valid) return;
+    const int m0 = tc.m0, n0 = tc.n0;
 
     // staging: A tile = 128 rows x 8 chunks of 8 int16 (4 per thread), W tile = 128 rows x 4 chunks of 16 int8 (2 per thread)
     v4i ra[4], rb[2];
@@ -218,8 +223,12 @@ __global__ __launch_bounds__(256) void gemm_i16i16_kernel(Gemm16x16Args g) {
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int tiles_n = (g.N + BN - 1) / BN;
-    const int m0 = (blockIdx.x / tiles_n) * BM, n0 = (blockIdx.x % tiles_n) * BN;
+    GemmArgs shape{};
+    shape.M = g.M;
+    shape.N = g.N;
+    const TileCoord tc = tile_coord<BM, BN>(shape);
+    if (!tc.valid) return;
+    const int m0 = tc.m0, n0 = tc.n0;
 
     // staging: A tile = 64 rows x 8 chunks of 8 int16 (2 per thread); each W plane = 128 rows x 4 chunks (2 per thread)
     v4i ra[2], rh[2], rl[2];
@@ -408,7 +417,7 @@ extern "C" int a4g_dense_i16(const int16_t* A, int64_t lda, const int8_t* Wt, in
     if (tiled) {
         const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
         A4G_REQUIRE(tiles <= INT32_MAX, A4G_ERR_UNSUPPORTED, "%s: too many tiles", who);
-        gemm_i16i8_kernel<<<static_cast<unsigned>(tiles), 256, 0, stream>>>(g);
+        gemm_i16i8_kernel<<<static_cast<unsigned>((tiles + 7) / 8 * 8), 256, 0, stream>>>(g);  // whole ranges for the 8 XCDs
     } else {
         const int grid = static_cast<int>(std::min<int64_t>((M * N + 255) / 256, 256 * 32));
         gemm_i16i8_generic_kernel<<<grid, 256, 0, stream>>>(g);
@@ -457,7 +466,7 @@ extern "C" int a4g_dense_i16x16(const int16_t* A, int64_t lda, const int8_t* Wt_
     if (tiled) {
         const int64_t tiles = ((M + 63) / 64) * ((N + 127) / 128);
         A4G_REQUIRE(tiles <= INT32_MAX, A4G_ERR_UNSUPPORTED, "%s: too many tiles", who);
-        gemm_i16i16_kernel<<<static_cast<unsigned>(tiles), 256, 0, stream>>>(g);
+        gemm_i16i16_kernel<<<static_cast<unsigned>((tiles + 7) / 8 * 8), 256, 0, stream>>>(g);
     } else {
         const int grid = static_cast<int>(std::min<int64_t>((M * N + 255) / 256, 256 * 32));
         gemm_i16i16_generic_kernel<<<grid, 256, 0, stream>>>(g);
