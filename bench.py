@@ -35,10 +35,10 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
 # WRITE_SIZE, one counter run each, scaled by what the same counter reads for calib_copy).
 # None = not measured.
 MEASURED_TRAFFIC = {
-    'c2_dense': 222877251, 'c1_mlp': 163162, 'c4_add': 48256768, 'c4_layernorm': 32630962,
-    'c4_add_layernorm': 48358174, 'c3_softmax_exp': 260085316, 'c3_softmax_hccs': 260085793,
-    'c3_qk': 181584228, 'c3_pv': 205590134, 'c3_attention_exp': 195232175, 'c3_attention_hccs': 195226688,
-    'calib_copy': 536870912, 'c2_dense_i16': 697146376,
+    'c2_dense': 222949836, 'c1_mlp': 163145, 'c4_add': 48253451, 'c4_layernorm': 32619260,
+    'c4_add_layernorm': 48370373, 'c3_softmax_exp': 260085460, 'c3_softmax_hccs': 260085096,
+    'c3_qk': 181587792, 'c3_pv': 205589019, 'c3_attention_exp': 195074307, 'c3_attention_hccs': 194983774,
+    'calib_copy': 536870912, 'c2_dense_i16': 697020280, 'c2_dense_bf16': 445182204, 'c2_dense_fp8': 223038951,
 }
 
 
