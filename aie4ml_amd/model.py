@@ -10,6 +10,8 @@ I/O contract of predict() (src/aie4ml/simulation.py:157-196, 248-269; model.py:1
     quantize_in=False requires integer arrays;
   * the result is int64 raw values, or float64 value / 2^frac with dequantize_out=True; a leading
     iteration axis is folded into the batch axis; one output -> ndarray, several -> dict by name;
+  * with the run-configuration key 'HipGraph' set, predict() records the whole graph into a HIP graph per input
+    signature and replays it on later calls (one launch on the host instead of one per operator);
   * tensors of the float compute path (FloatIntent) take float32 arrays as they are (simulation.py:184-185)
     and come back as float64 (simulation.py:235, 253-254), whatever the two flags say.
 """
@@ -37,6 +39,7 @@ class GPUModel:
         setattr(self, CONTEXT_ATTR, ctx)
         self.source_model = source_model
         self._compiled = False
+        self._captured: Dict[Any, Any] = {}  # input signature -> CapturedExecution (config key 'HipGraph')
 
     @classmethod
     def from_context(cls, ctx: BackendContext, source_model: Optional[Any] = None) -> 'GPUModel':
@@ -135,7 +138,15 @@ class GPUModel:
         graph = self.context.ir.logical
         dev_inputs = self.to_device(prepared)
         iters = next(iter(prepared.values())).shape[0]
-        dev_out = self.execute(dev_inputs, batch_scale=iters)
+        if self.context.config.get('HipGraph'):
+            # serving loops: one HIP graph per input signature, recorded at the first call and replayed afterwards
+            key = tuple((n, tuple(t.shape), str(t.dtype)) for n, t in sorted(dev_inputs.items()))
+            captured = self._captured.get(key)
+            if captured is None:
+                captured = self._captured[key] = CapturedExecution(self, dev_inputs)
+            dev_out = captured(dev_inputs)
+        else:
+            dev_out = self.execute(dev_inputs, batch_scale=iters)
         torch.cuda.synchronize()
         results = {}
         for t in graph.graph_outputs():

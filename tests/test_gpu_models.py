@@ -343,3 +343,20 @@ def test_report_times_every_launch(oracle):
     assert kinds == ['dense', 'attention', 'dense', 'add_layer_norm', 'mlp', 'add_layer_norm']
     assert abs(sum(k['pct'] for k in rep['kernels']) - 100.0) < 1.0
     assert all(k['time_us'] > 0 for k in rep['kernels'])
+
+
+def test_predict_with_hip_graph_replay(oracle):
+    """Config key 'HipGraph': predict() records one HIP graph per input signature and replays it; every call must
+    equal the eager result, also after a call with another batch size in between."""
+    data, cfg, x = workloads.c5_encoder_block_onnx(batch=4, seq=32, hidden=128, heads=2, ffn=256, softmax='exp')
+    from aie4ml_amd import from_onnx
+
+    eager = from_onnx(data, cfg)
+    graphed = from_onnx(data, dict(cfg, HipGraph=True))
+    r = np.random.default_rng(3)
+    for i in range(4):
+        xi = r.integers(-128, 128, x.shape).astype(np.int8)
+        want = eager.predict(xi, quantize_in=False, dequantize_out=False)
+        got = graphed.predict(xi, quantize_in=False, dequantize_out=False)
+        assert np.array_equal(got, want), i
+    assert len(graphed._captured) == 1
