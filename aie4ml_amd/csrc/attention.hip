@@ -45,26 +45,32 @@ __device__ __forceinline__ void transpose4x4(const unsigned a[4], unsigned c[4])
 // NT = key/value rows / 32, DT = head dimension / 32. 256 threads = 4 waves = 128 query rows of one head.
 // BIT: rounding kind of the logits (fast_round_kind). FASTP: the probabilities need no clamp and their shift is
 // at most 16, so p = (e * inv) >> shift is read as byte 2 of e * (inv << (16 - shift)).
-template <int NT, int DT, int BIT, bool FASTP>
-__global__ __launch_bounds__(256, 2) void attention_kernel(AttnArgs a) {
+// NW = waves per workgroup. 4: two workgroups share a CU. 8: one workgroup of 256 query rows per CU, which
+// leaves room to store the score table once per LDS bank (entry d for lane c at dword d * 64 + c, byte address
+// (d << 8) | (c << 2) built by one v_perm): with a single copy, lanes that gather different gaps from one bank
+// serialise, and those conflicts were two thirds of this kernel's LDS cycles.
+template <int NT, int DT, int BIT, bool FASTP, int NW = 4>
+__global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(AttnArgs a) {
     constexpr int SK = NT * 32, D = DT * 32, PITCH = SK + 16;
+    constexpr bool BANKED = NW == 8;
+    constexpr int THREADS = NW * 64, ROWS = NW * 32;
     // The score table is a static array: its LDS address is then a compile-time constant that folds into the
     // offset field of the gathers (an array inside the dynamic block costs one address add per gather).
-    __shared__ int table[256];                                     // score of a gap d in [0,255]
+    __shared__ int table[BANKED ? 256 * 64 : 256];                 // score of a gap d in [0,255]
     extern __shared__ __attribute__((aligned(16))) int8_t attn_smem[];
     int8_t* vt = attn_smem;                                        // V^T, k-permuted: [D][PITCH]
     int* colsum = reinterpret_cast<int*>(attn_smem + D * PITCH);   // sum_k V[k][n]
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int m = lane & 31, half = lane >> 5;
-    const int nblk = (a.sq + 127) >> 7;
+    const int nblk = (a.sq + ROWS - 1) / ROWS;
     const int bh = blockIdx.x / nblk, rb = blockIdx.x % nblk;
     const int b = bh / a.heads, h = bh % a.heads;
     const int8_t* Qp = a.Q + b * a.q_sb + h * a.q_sh;
     const int8_t* Kp = a.K + b * a.k_sb + h * a.k_sh;
     const int8_t* Vp = a.V + b * a.v_sb + h * a.v_sh;
     int8_t* Op = a.O + b * a.o_sb + h * a.o_sh;
-    const int row = rb * 128 + wave * 32 + m;
+    const int row = rb * ROWS + wave * 32 + m;
     const bool row_ok = row < a.sq;
     const int rowc = row_ok ? row : a.sq - 1;
 
@@ -77,7 +83,15 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(AttnArgs a) {
         kf[0][ks] = *reinterpret_cast<const v4i*>(Kp + m * a.k_ss + ks * 32 + half * 16);
     }
 
-    table[tid] = table_entry(a.sm, tid);
+    if (BANKED) {
+        // each entry is computed once, parked in the (still unused) V^T area, then copied to its 64 slots
+        int* once = reinterpret_cast<int*>(vt);
+        if (tid < 256) once[tid] = table_entry(a.sm, tid);
+        __syncthreads();
+        for (int i = tid; i < 256 * 64; i += THREADS) table[i] = once[i >> 6];
+    } else {
+        table[tid] = table_entry(a.sm, tid);
+    }
     if (tid < D) colsum[tid] = 0;
     __syncthreads();
 
@@ -85,9 +99,9 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(AttnArgs a) {
     // k = 8*g + 4*half + i: the order in which a lane's probability registers run.
     {
         constexpr int NB = (SK / 4) * (D / 4);
-        const int n0 = (tid % (D / 4)) * 4;  // 256 % (D/4) == 0: a thread keeps its four columns
+        const int n0 = (tid % (D / 4)) * 4;  // THREADS % (D/4) == 0: a thread keeps its four columns
         int part[4] = {0, 0, 0, 0};
-        for (int blk = tid; blk < NB; blk += 256) {
+        for (int blk = tid; blk < NB; blk += THREADS) {
             const int k0 = (blk / (D / 4)) * 4;
             unsigned av[4], cv[4];
 #pragma unroll
@@ -138,6 +152,7 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(AttnArgs a) {
     const unsigned mrep = static_cast<unsigned>((mx ^ 0x80) & 0xFF) * 0x01010101u;
     const char* tbytes = reinterpret_cast<const char*>(table);
     const unsigned two = 2;
+    const unsigned lane4 = static_cast<unsigned>(lane) << 2;  // BANKED: this lane's copy of the table
     unsigned ep[NT][8];  // two 16-bit scores per register
     int sum = 0;
 #pragma unroll
@@ -145,10 +160,18 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(AttnArgs a) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             const unsigned d4 = mrep - (lg[t][g] ^ 0x80808080u);  // per byte, never borrows
-            const int e0 = *reinterpret_cast<const int*>(tbytes + byte_x4<0>(d4, two));
-            const int e1 = *reinterpret_cast<const int*>(tbytes + byte_x4<1>(d4, two));
-            const int e2 = *reinterpret_cast<const int*>(tbytes + byte_x4<2>(d4, two));
-            const int e3 = *reinterpret_cast<const int*>(tbytes + byte_x4<3>(d4, two));
+            int e0, e1, e2, e3;
+            if (BANKED) {
+                e0 = *reinterpret_cast<const int*>(tbytes + __builtin_amdgcn_perm(d4, lane4, 0x0c0c0400u));
+                e1 = *reinterpret_cast<const int*>(tbytes + __builtin_amdgcn_perm(d4, lane4, 0x0c0c0500u));
+                e2 = *reinterpret_cast<const int*>(tbytes + __builtin_amdgcn_perm(d4, lane4, 0x0c0c0600u));
+                e3 = *reinterpret_cast<const int*>(tbytes + __builtin_amdgcn_perm(d4, lane4, 0x0c0c0700u));
+            } else {
+                e0 = *reinterpret_cast<const int*>(tbytes + byte_x4<0>(d4, two));
+                e1 = *reinterpret_cast<const int*>(tbytes + byte_x4<1>(d4, two));
+                e2 = *reinterpret_cast<const int*>(tbytes + byte_x4<2>(d4, two));
+                e3 = *reinterpret_cast<const int*>(tbytes + byte_x4<3>(d4, two));
+            }
             sum += (e0 + e1) + (e2 + e3);
             ep[t][2 * g] = pack2_halves(e0, e1);
             ep[t][2 * g + 1] = pack2_halves(e2, e3);
@@ -220,13 +243,31 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(AttnArgs a) {
     }
 }
 
+template <int NT, int DT, int BIT, bool FASTP>
+static void launch_attention_wide(int grid8, size_t lds, hipStream_t stream, const AttnArgs& a) {
+    auto kern = attention_kernel<NT, DT, BIT, FASTP, 8>;
+    static bool attr_set = false;  // benign race: the attribute is idempotent
+    if (!attr_set) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  static_cast<int>(lds));
+        attr_set = true;
+    }
+    kern<<<grid8, 512, lds, stream>>>(a);
+}
+
+// grid: workgroups of 128 query rows; grid8: workgroups of 256 (0 = do not use the eight-wave form).
 template <int NT, int DT>
-static void launch_attention_nt(int grid, size_t lds, hipStream_t stream, const AttnArgs& a) {
+static void launch_attention_nt(int grid, int grid8, size_t lds, hipStream_t stream, const AttnArgs& a) {
     const bool fastp = a.noclamp && a.sm.out_shift <= 16;
-#define A4G_ATTN(B)                                                              \
-    if (fastp)                                                                   \
-        attention_kernel<NT, DT, B, true><<<grid, 256, lds, stream>>>(a);        \
-    else                                                                         \
+#define A4G_ATTN(B)                                                                  \
+    if (NT >= 8 && grid8 > 0) {                                                      \
+        if constexpr (NT >= 8) {                                                     \
+            if (fastp) launch_attention_wide<NT, DT, B, true>(grid8, lds, stream, a); \
+            else launch_attention_wide<NT, DT, B, false>(grid8, lds, stream, a);      \
+        }                                                                            \
+    } else if (fastp)                                                                \
+        attention_kernel<NT, DT, B, true><<<grid, 256, lds, stream>>>(a);            \
+    else                                                                             \
         attention_kernel<NT, DT, B, false><<<grid, 256, lds, stream>>>(a);
     switch (fast_round_kind(a.lr)) {
     case 0: A4G_ATTN(0) break;
@@ -237,14 +278,14 @@ static void launch_attention_nt(int grid, size_t lds, hipStream_t stream, const 
 }
 
 template <int DT>
-static int launch_attention(int nt, int grid, hipStream_t stream, const AttnArgs& a) {
+static int launch_attention(int nt, int grid, int grid8, hipStream_t stream, const AttnArgs& a) {
     const size_t lds = static_cast<size_t>(DT * 32) * (nt * 32 + 16) + DT * 32 * 4;  // V^T + column sums
     switch (nt) {
-    case 1: launch_attention_nt<1, DT>(grid, lds, stream, a); break;
-    case 2: launch_attention_nt<2, DT>(grid, lds, stream, a); break;
-    case 4: launch_attention_nt<4, DT>(grid, lds, stream, a); break;
-    case 8: launch_attention_nt<8, DT>(grid, lds, stream, a); break;
-    case 16: launch_attention_nt<16, DT>(grid, lds, stream, a); break;
+    case 1: launch_attention_nt<1, DT>(grid, 0, lds, stream, a); break;
+    case 2: launch_attention_nt<2, DT>(grid, 0, lds, stream, a); break;
+    case 4: launch_attention_nt<4, DT>(grid, 0, lds, stream, a); break;
+    case 8: launch_attention_nt<8, DT>(grid, grid8, lds, stream, a); break;
+    case 16: launch_attention_nt<16, DT>(grid, grid8, lds, stream, a); break;
     default: return 1;
     }
     return 0;
@@ -300,7 +341,10 @@ extern "C" int a4g_attention_i8(const int8_t* Q, const int8_t* K, const int8_t* 
     a.orr = make_fast_round(out_round_mode, out_shift);
     a.noclamp = noclamp;
     const int grid = static_cast<int>(batch * heads * ((sq + 127) / 128));
-    if (launch_attention<2>(static_cast<int>(sk / 32), grid, stream, a))
+    // eight waves per workgroup (256 query rows, bank-replicated score table) once every CU gets at least one
+    const int64_t wg8 = batch * heads * ((sq + 255) / 256);
+    const int grid8 = (sq >= 256 && wg8 >= 256) ? static_cast<int>(wg8) : 0;
+    if (launch_attention<2>(static_cast<int>(sk / 32), grid, grid8, stream, a))
         return fail(A4G_ERR_UNSUPPORTED, "%s: no kernel for sk=%lld", who, (long long)sk);
     return check_hip(hipGetLastError(), who);
 }

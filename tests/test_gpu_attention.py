@@ -64,6 +64,20 @@ def test_attention_ragged_query_count(oracle, sq):
     np.testing.assert_array_equal(got, reference(oracle, q, k, v, 6, 'symmetric_inf', sm, 8, 'floor'))
 
 
+@pytest.mark.parametrize('sq,sk', [(512, 512), (300, 256), (256, 512)])
+@pytest.mark.parametrize('mode', ['conv_even', 'symmetric_inf', 'floor'])
+def test_attention_with_256_row_workgroups(oracle, sq, sk, mode):
+    # at least 256 workgroups of 256 query rows and 256 or more keys: the eight-wave form with the score table
+    # stored once per LDS bank; a clamped (non fast-path) probability shift as well
+    nb = 256 // ((sq + 255) // 256) // 16
+    q, k, v = qkv(sq + sk, (nb, 16, sq, 64), (nb, 16, sk, 64), sigma=30.0)
+    B, S, D = HCCS[sk]
+    for sm in ({'kind': 'exp', 'exp_kq': 23}, {'kind': 'hccs', 'B': B, 'S': S, 'Dmax': D},
+               {'kind': 'exp', 'exp_kq': 23, 'inv_shift': 17}):
+        got = ops.attention(dev(q), dev(k), dev(v), 6, mode, sm, 7, mode).cpu().numpy()
+        np.testing.assert_array_equal(got, reference(oracle, q, k, v, 6, mode, sm, 7, mode))
+
+
 def test_attention_zero_shift_and_saturation(oracle):
     # shift 0 on the logits saturates most of them; shift 0 on the output saturates everything
     q, k, v = qkv(3, (2, 64, 64), (2, 64, 64), sigma=60.0)
