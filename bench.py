@@ -140,7 +140,7 @@ def main():
         samples = M
         config = {'workload': 'c2_dense: Dense 8192x4096 -> 4096, int8, bias, per-channel shift 8..12, conv_even, '
                               'sat int8, ReLU'}
-        sample_rows = 256
+        sample_rows = 2048  # about 1 s per pass on 16 host threads, 10 s with the repeats
         cpu_desc = f'oracle Dense on the first {sample_rows} of {M} rows (same W/bias/shifts), scaled per op'
         cpu_fn = lambda: oracle.dense(A[:sample_rows], W, bias, shifts, 'conv_even', relu=True)  # noqa: E731
         cpu_work = 2.0 * sample_rows * N * K
