@@ -163,6 +163,53 @@ __device__ __forceinline__ unsigned pack2_halves(int y0, int y1) {
     return __builtin_amdgcn_perm(static_cast<unsigned>(y1), static_cast<unsigned>(y0), 0x05040100u);
 }
 
+// Requantise four accumulators straight into the four bytes of one dword: the clamp is applied before the shift
+// (to [lo << s, (hi << s) + 2^s - 1], which selects exactly the sums whose shifted value lies in [lo, hi]) and the
+// shift then writes its low byte into byte n of the result (SDWA destination select, other bytes preserved), so
+// no separate packing instructions are needed. Valid for hi << s within int32 (s <= 22 for 8-bit outputs).
+struct ByteRequant {
+    FastRound fr;
+    int lo_s, hi_s;
+};
+static inline ByteRequant make_byte_requant(const FastRound& fr, int lo, int hi) {
+    ByteRequant b;
+    b.fr = fr;
+    b.lo_s = static_cast<int>(static_cast<unsigned>(lo) << fr.s);
+    b.hi_s = static_cast<int>((static_cast<unsigned>(hi) << fr.s) | ((1u << fr.s) - 1u));
+    return b;
+}
+static inline bool byte_requant_ok(const FastRound& fr) { return fr.s >= 0 && fr.s <= 22; }
+
+template <int N>
+__device__ __forceinline__ void shift_into_byte(unsigned& packed, int v, int s) {
+    if (N == 0) asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(packed) : "v"(s), "v"(v));
+    if (N == 1) asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_1 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(packed) : "v"(s), "v"(v));
+    if (N == 2) asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_2 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(packed) : "v"(s), "v"(v));
+    if (N == 3) asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_3 dst_unused:UNUSED_PRESERVE src0_sel:DWORD src1_sel:DWORD" : "+v"(packed) : "v"(s), "v"(v));
+}
+
+// acc[0..3] -> one dword of four requantised bytes (rounding kind BIT as in fast_round_k).
+template <int BIT>
+__device__ __forceinline__ unsigned requant4_bytes(int a0, int a1, int a2, int a3, const ByteRequant& b) {
+    auto pre = [&](int acc) {
+        int bit = 0;
+        if (BIT == 1) bit = static_cast<int>(__builtin_amdgcn_ubfe(static_cast<unsigned>(acc), b.fr.pos, 1));
+        if (BIT == 2) bit = __builtin_amdgcn_sbfe(acc, b.fr.pos, 1);
+        return clamp_med3(acc + b.fr.c0 + bit, b.lo_s, b.hi_s);
+    };
+    unsigned packed;  // byte 0 is written with the other bytes zeroed, bytes 1..3 are then merged in
+    {
+        const int v0 = pre(a0);
+        asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:DWORD"
+            : "=v"(packed)
+            : "v"(b.fr.s), "v"(v0));
+    }
+    shift_into_byte<1>(packed, pre(a1), b.fr.s);
+    shift_into_byte<2>(packed, pre(a2), b.fr.s);
+    shift_into_byte<3>(packed, pre(a3), b.fr.s);
+    return packed;
+}
+
 __device__ __forceinline__ int kind_lo(int kind) {
     return kind == A4G_I8 ? -128 : (kind == A4G_I16 ? -32768 : (kind == A4G_I32 ? INT32_MIN : 0));
 }

@@ -887,6 +887,7 @@ extern "C" int a4g_matmul_i8(const void* A, int a_kind, int64_t lda, int64_t str
         la.lo = out_kind == A4G_I8 ? -128 : 0;
         la.hi = out_kind == A4G_I8 ? 127 : 255;
         la.fr = make_fast_round(round_mode, shift);
+        la.br = make_byte_requant(la.fr, la.lo, la.hi);
         if (trans_b && lean_nt_applicable(la)) return check_hip(launch_lean_nt(la, stream), who);
         if (!trans_b && lean_nn_applicable(la)) return check_hip(launch_lean_nn(la, stream), who);
     }

@@ -49,14 +49,8 @@ __device__ __forceinline__ void lean_nt_compute(const LeanArgs& a, int8_t* Cp, c
 #pragma unroll
             for (int ks = 0; ks < DT; ++ks) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[T][ks], af[rb][ks], acc, 0, 0, 0);
 #pragma unroll
-            for (int gg = 0; gg < 4; ++gg) {
-                int y[4];
-#pragma unroll
-                for (int ii = 0; ii < 4; ++ii)
-                    y[ii] = UOUT ? clamp_i(fast_round_k<BIT>(acc[4 * gg + ii], a.fr), 0, 255)
-                                 : clamp_i(fast_round_k<BIT>(acc[4 * gg + ii], a.fr), -128, 127);
-                o[T][gg] = static_cast<int>(pack4_bytes(y[0], y[1], y[2], y[3]));
-            }
+            for (int gg = 0; gg < 4; ++gg)
+                o[T][gg] = static_cast<int>(requant4_bytes<BIT>(acc[4 * gg], acc[4 * gg + 1], acc[4 * gg + 2], acc[4 * gg + 3], a.br));
         }
         if (TG == 4) {
 #pragma unroll
@@ -228,7 +222,8 @@ static bool lean_common_ok(const LeanArgs& a) {
 }
 
 bool lean_nt_applicable(const LeanArgs& a) {
-    return lean_common_ok(a) && !a.a_unsigned && a.K % 32 == 0 && a.K <= 128 && a.N % 32 == 0 && a.N <= 512 * 65535;
+    return lean_common_ok(a) && !a.a_unsigned && a.K % 32 == 0 && a.K <= 128 && a.N % 32 == 0 && a.N <= 512 * 65535 &&
+           byte_requant_ok(a.fr);
 }
 
 template <int DT, int RB>

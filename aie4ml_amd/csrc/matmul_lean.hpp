@@ -17,6 +17,7 @@ struct LeanArgs {
     int a_unsigned;
     int lo, hi;  // saturation bounds of the output kind
     FastRound fr;
+    ByteRequant br;  // fr with the clamp bounds moved in front of the shift (transposed-B kernel)
 };
 
 // C = srs(A x B^T): B is [N][ldb], K in {32,64,96,128}, N % 32 == 0. Returns false when not applicable.
