@@ -14,7 +14,7 @@ from typing import Iterable
 
 import numpy as np
 
-from ..aie_types import FloatFormat, FloatIntent, is_float_intent
+from ..aie_types import FloatFormat, FloatIntent, QuantIntent, is_float_intent
 from ..ir import TraitInstance, get_backend_context, input_tensor_for_role
 from ..op_impls import get_family_resolver_registry
 from ..op_impls.base import OpImplVariant
@@ -57,6 +57,35 @@ class ForceFloatMode(AIEPass):
             if tv.precision is not None and not is_float_intent(tv.precision):
                 tv.precision = intent
                 changed = True
+        return changed
+
+
+class FoldApplyAlpha(AIEPass):
+    """Fold a per-channel power-of-two output scale (hls4ml's ApplyAlpha after a Dense) into the Dense: the weight
+    intent gains round(-log2(max scale)) fractional bits, the bias is multiplied by the scale, the node goes
+    (src/aie4ml/passes/fold_apply_alpha.py:13-60). Float graphs are left alone, as there."""
+
+    name = 'fold_apply_alpha'
+
+    def transform(self, model_or_ctx) -> bool:
+        graph = get_backend_context(model_or_ctx).ir.logical
+        changed = False
+        for node in list(graph.nodes):
+            if node.op_type != 'applyalpha':
+                continue
+            scale = np.asarray(node.metadata['scale'], dtype=np.float64)
+            p_min = int(np.round(-np.log2(scale.max())))
+            dense = node.inputs[0].producer
+            weight = dense.inputs[1]
+            old = weight.precision
+            if is_float_intent(old):
+                continue
+            weight.precision = QuantIntent(width=old.width, frac=old.frac + p_min, signed=old.signed, rounding=old.rounding,
+                                           saturation=old.saturation)
+            if dense.metadata.get('use_bias') and len(dense.inputs) > 2:
+                dense.inputs[2].data = np.asarray(dense.inputs[2].data, dtype=np.float64) * scale
+            graph.remove_node(node, mode='contract')
+            changed = True
         return changed
 
 
@@ -501,4 +530,4 @@ class PlanGpuFusion(AIEPass):
         return total <= self.MLP_MAX_WEIGHT_BYTES
 
 
-GPU_PIPELINE = (ForceFloatMode, FoldBias, FoldScale, FuseActivationCasts, FoldViewOps, Resolve, PackKernelArtifacts, PlanGpuFusion)
+GPU_PIPELINE = (ForceFloatMode, FoldApplyAlpha, FoldBias, FoldScale, FuseActivationCasts, FoldViewOps, Resolve, PackKernelArtifacts, PlanGpuFusion)

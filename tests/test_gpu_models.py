@@ -360,3 +360,32 @@ def test_predict_with_hip_graph_replay(oracle):
         got = graphed.predict(xi, quantize_in=False, dequantize_out=False)
         assert np.array_equal(got, want), i
     assert len(graphed._captured) == 1
+
+
+# ---- hls4ml model graphs --------------------------------------------------------------------------------------------
+
+def test_hls4ml_mlp_matches_the_quantised_network(oracle):
+    """The network of the reference's hls4ml test (tests/test_hls4ml_dense.py: QDense + quantized_relu layers, 8 bits),
+    presented as hls4ml presents it (stand-in objects), must predict what the quantised network itself computes:
+    exact fixed-point products, round-to-nearest-even and saturation at every activation quantiser."""
+    from aie4ml_amd import from_hls4ml
+    from tests.hls4ml_standin import qkeras_mlp
+
+    dims, batch = [16, 64, 32, 32, 5], 256
+    hls_model, weights = qkeras_mlp(dims, batch)
+    model = from_hls4ml(hls_model)
+    r = np.random.default_rng(11)
+    x = r.uniform(-4, 4, (batch, dims[0]))
+    y = model.predict(x)
+    assert y.shape == (batch, 5) and y.dtype == np.float64
+
+    def quant(v, frac, lo, hi):  # numpy's rint is round-half-even
+        return np.clip(np.rint(v * 2.0 ** frac), lo, hi) / 2.0 ** frac
+
+    h = quant(x, 5, -128, 127)
+    for i, (W, b) in enumerate(weights):
+        z = h @ W + b                                   # exact: every operand is a small dyadic rational
+        h = quant(np.maximum(z, 0), 8, 0, 255) if i < len(weights) - 1 else quant(z, 5, -128, 127)
+    assert np.array_equal(y, h)
+    # and bit for bit against the oracle's graph interpreter
+    _graph_check(model, oracle, {'input_layer': np.rint(quant(x, 5, -128, 127) * 32).astype(np.int8)})

@@ -487,3 +487,67 @@ def test_float_mode_rules():
     v = np.array([1.0, 1.00390625, 1.0078125, -1.00390625, 3.14159], dtype=np.float32)
     assert pack_as_float(v, 'bfloat16').tolist() == [1.0, 1.0, 1.0078125, -1.0, 3.140625]
     assert pack_as_float(v, 'float32').tolist() == v.tolist()
+
+
+# ---- hls4ml model graphs (read by attribute access; stand-in objects, hls4ml is not installed) ----------------
+
+def test_hls4ml_lowering_gives_the_reference_graph():
+    from aie4ml_amd.frontends.hls4ml_lower import lower_hls4ml_model
+    from aie4ml_amd.passes import FoldApplyAlpha
+    from tests.hls4ml_standin import qkeras_mlp
+
+    model, weights = qkeras_mlp([16, 64, 32, 5], batch=8)
+    ctx = lower_hls4ml_model(model)
+    g = ctx.ir.logical
+    assert [n.op_type for n in g.nodes] == ['input', 'dense', 'activation', 'dense', 'activation', 'dense', 'activation']
+    assert g.nodes[0].is_placeholder and g.input_tensor_names == ['input_layer'] and g.output_tensor_names == ['act2_out']
+    d0 = g.nodes[1]
+    assert d0.metadata['n_in'] == 16 and d0.metadata['n_out'] == 64 and d0.metadata['use_bias'] is True
+    assert [d0.roles[t.name] for t in d0.inputs] == ['lhs', 'rhs', 'bias']
+    assert g.tensors['dense0_out'].shape == (8, 64) and g.tensors['input_layer'].shape == (8, 16)
+    w = g.tensors['dense0_weight']
+    assert (w.precision.width, w.precision.frac, w.precision.rounding) == (8, 5, RoundingMode.RND_CONV)
+    assert np.array_equal(w.data, weights[0][0])
+    # through the passes: activations fold away, relu fuses, every dense resolves with the post-activation type
+    run_aie_passes(ctx, [p() for p in (FoldApplyAlpha,) + FRONT])
+    assert [n.op_type for n in g.nodes if not n.is_placeholder] == ['dense', 'dense', 'dense']
+    cfgs = [ctx.ir.execution.get(f'dense{i}_aie').config for i in range(3)]
+    assert [c.flags.use_relu for c in cfgs] == [True, True, False]
+    assert cfgs[0].precision['output'].format == 'uint8' and cfgs[2].precision['output'].format == 'int8'
+    assert cfgs[0].shift == 5 + 5 - 8 and cfgs[1].shift == 8 + 5 - 8 and cfgs[2].shift == 8 + 5 - 5
+    assert cfgs[0].rounding_mode == 'conv_even'
+
+
+def test_hls4ml_apply_alpha_folds_into_the_dense():
+    from aie4ml_amd.frontends.hls4ml_lower import lower_hls4ml_model
+    from aie4ml_amd.passes import FoldApplyAlpha
+    from tests.hls4ml_standin import qkeras_mlp
+
+    model, weights = qkeras_mlp([16, 32, 8], batch=4, alpha=0.25)
+    ctx = lower_hls4ml_model(model)
+    assert 'applyalpha' in [n.op_type for n in ctx.ir.logical.nodes]
+    run_aie_passes(ctx, [p() for p in (FoldApplyAlpha,) + FRONT])
+    assert [n.op_type for n in ctx.ir.logical.nodes if not n.is_placeholder] == ['dense', 'dense']
+    w = ctx.ir.logical.tensors['dense0_weight']
+    assert w.precision.frac == 5 + 2                                     # scale 2^-2 moves the binary point
+    assert np.allclose(ctx.ir.logical.tensors['dense0_bias'].data, weights[0][1] * 0.25)
+    assert ctx.ir.execution.get('dense0_aie').config.shift == 5 + 7 - 8
+
+
+def test_hls4ml_lowering_errors():
+    from aie4ml_amd.frontends.hls4ml_lower import lower_hls4ml_model
+    from tests.hls4ml_standin import Layer, qkeras_mlp
+
+    model, _ = qkeras_mlp([16, 8], batch=4)
+    with pytest.raises(KeyError, match='BatchSize'):
+        lower_hls4ml_model(type(model)(model.get_layers(), model.output_vars, {}))
+    model._layers[1].weights.pop('weight')
+    with pytest.raises(RuntimeError, match='no weight variable'):
+        lower_hls4ml_model(model)
+    conv = Layer('pw', 'Conv1D', ['input'], {'filt_width': 3, 'stride_width': 1, 'pad_left': 0, 'pad_right': 0, 'in_width': 8,
+                                            'out_width': 8})
+    model2, _ = qkeras_mlp([16, 8], batch=4)
+    model2._layers[1] = conv
+    model2.output_vars['pw'] = model2.output_vars['dense0']
+    with pytest.raises(ValueError, match='not true pointwise'):
+        lower_hls4ml_model(model2)
