@@ -389,3 +389,36 @@ def test_hls4ml_mlp_matches_the_quantised_network(oracle):
     assert np.array_equal(y, h)
     # and bit for bit against the oracle's graph interpreter
     _graph_check(model, oracle, {'input_layer': np.rint(quant(x, 5, -128, 127) * 32).astype(np.int8)})
+
+
+@pytest.mark.parametrize('mode', ['io', 'internal'])
+@pytest.mark.parametrize('in_shape', [(384,), (8, 16, 384)])
+def test_fanout_graph_with_two_outputs(oracle, mode, in_shape):
+    """The graphs of the reference's fan-out test (tests/test_hls4ml_fanout.py:28-68): the input ('io') or a shared
+    Dense + ReLU ('internal') feeds two Dense branches, each a graph output; batch 1, five iterations; also with the
+    multi-dimensional input of its nd cases. predict() returns a dict keyed by output tensor name."""
+    r = np.random.default_rng(len(in_shape) + (mode == 'io'))
+    hidden, act, wq, relu6 = 256, qint(8, 5), qint(8, 5), qint(8, 2, signed=False)
+    gb = GraphBuilder({'Iterations': 5})
+    t = gb.input('input_layer', (1,) + in_shape, act)
+
+    def dense(src, name, out_prec, relu):
+        W = r.integers(-128, 128, (int(src.shape[-1]), hidden)) / 32.0
+        b = r.integers(-128, 128, hidden) / 32.0
+        return gb.dense(src, W, wq, out_prec, bias=b, bias_precision=wq, relu=relu, name=name)
+
+    if mode == 'internal':
+        t = dense(t, 'shared_internal_dense', qint(8, 8, signed=False), True)
+    y1 = gb.output(dense(t, 'branch1', relu6, True))
+    y2 = gb.output(dense(t, 'branch2', relu6, True))
+    model = gb.build()
+    x = r.integers(-128, 128, (5, 1) + in_shape).astype(np.int8)
+    got = model.predict(x, quantize_in=False, dequantize_out=False)
+    assert list(got) == [y1.name, y2.name] and got[y1.name].shape == (5,) + in_shape[:-1] + (hidden,)
+    assert not np.array_equal(got[y1.name], got[y2.name])
+    flat = x.reshape((5,) + in_shape)
+    want = run_graph(model, oracle, {'input_layer': flat})
+    for name in (y1.name, y2.name):
+        np.testing.assert_array_equal(got[name].reshape(want[name].shape), want[name].astype(np.int64))
+    deq = model.predict(x.astype(np.float64) / 32.0)
+    np.testing.assert_array_equal(deq[y1.name], got[y1.name] / 4.0)
