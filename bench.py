@@ -46,7 +46,9 @@ def _time_gpu(torch, fn, steps, warmup, use_graph=True):
     """Times exactly `steps` launches between two events on the launch stream, synchronised on both
     sides. The launches are recorded once into a HIP graph and replayed, so that the interval holds
     back-to-back kernels rather than the Python interpreter's per-call cost (which exceeds the run time
-    of the small row kernels); falls back to eager launches if capture is not possible."""
+    of the small row kernels); falls back to eager launches if capture is not possible. Besides the `warmup`
+    eager launches the recorded graph is replayed three times untimed: per-launch times keep falling over the
+    first few hundred launches while the clocks settle."""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -63,7 +65,8 @@ def _time_gpu(torch, fn, steps, warmup, use_graph=True):
             with torch.cuda.graph(graph):
                 for _ in range(steps):
                     fn()
-            graph.replay()  # untimed first replay (uploads the graph)
+            for _ in range(3):  # untimed replays: the first uploads the graph, the others let the clocks settle
+                graph.replay()
             torch.cuda.synchronize()
         except Exception as exc:  # noqa: BLE001
             print(f'bench.py: graph capture failed ({exc}); timing eager launches', file=sys.stderr)
