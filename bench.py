@@ -35,10 +35,10 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
 # WRITE_SIZE, one counter run each, scaled by what the same counter reads for calib_copy).
 # None = not measured.
 MEASURED_TRAFFIC = {
-    'c2_dense': 222949836, 'c1_mlp': 163145, 'c4_add': 48253451, 'c4_layernorm': 32619260,
-    'c4_add_layernorm': 48370373, 'c3_softmax_exp': 260085460, 'c3_softmax_hccs': 260085096,
-    'c3_qk': 181587792, 'c3_pv': 205589019, 'c3_attention_exp': 126645006, 'c3_attention_hccs': 126645224,
-    'calib_copy': 536870912, 'c2_dense_i16': 697020280, 'c2_dense_bf16': 445182204, 'c2_dense_fp8': 223038951,
+    'c2_dense': 227803374, 'c1_mlp': 166940, 'c4_add': 49059234, 'c4_layernorm': 33024803,
+    'c4_add_layernorm': 49179488, 'c3_softmax_exp': 263310672, 'c3_softmax_hccs': 263310853,
+    'c3_qk': 182762264, 'c3_pv': 210430349, 'c3_attention_exp': 128707683, 'c3_attention_hccs': 128709239,
+    'calib_copy': 536870912, 'c2_dense_i16': 713173641, 'c2_dense_bf16': 454954067, 'c2_dense_fp8': 227923232,
 }
 
 
