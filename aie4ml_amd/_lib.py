@@ -71,6 +71,9 @@ SIGNATURES = {
     'a4g_pack_weights_i16': (_i32, [_vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp]),
     'a4g_dense_i16x16': (_i32, [_vp, _i64, _vp, _vp, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _i64, _i64, _i64, _i64,
                                 _vp]),
+    'a4g_matmul_i16_workspace_bytes': (_sz, [_i64, _i64, _i64, _i32]),
+    'a4g_matmul_i16': (_i32, [_vp, _i64, _i64, _vp, _i32, _i64, _i64, _i32, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32,
+                              _i32, _vp, _sz, _vp]),
     'a4g_attention_i8': (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, ctypes.POINTER(ctypes.c_int64), _i32, _i32,
                                 _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp]),
     'a4g_packed_ld_f': (_i64, [_i64, _i32]),

@@ -22,12 +22,24 @@ struct Gemm16Args {
     int64_t lda, ldwt, ldy;  // lda, ldy in elements
     int M, N, K;
     int shift_stride, relu, out_kind, mode;
+    // batched use (dynamic MatMul): element strides between consecutive problems, blockIdx.y = problem
+    int64_t stride_a, stride_w, stride_colsum, stride_y;
+    int shift;  // used when `shifts` is null (MatMul: one host-side shift)
 };
 
 // 128 x 128 output tile, K step 64, 4 waves (2 x 2) of 64 x 64, double-buffered LDS holding the two byte
 // planes of A and the weight tile. Requires K % 8 == 0 and 16-byte aligned rows of A and Wt.
+__device__ __forceinline__ void select_problem(Gemm16Args& g, int b) {
+    const int obytes = (g.out_kind == A4G_I16 || g.out_kind == A4G_U16) ? 2 : 1;
+    g.A += b * g.stride_a;
+    g.Wt += b * g.stride_w;
+    g.colsum += b * g.stride_colsum;
+    g.Y = static_cast<int8_t*>(g.Y) + b * g.stride_y * obytes;
+}
+
 __global__ __launch_bounds__(256) void gemm_i16i8_kernel(Gemm16Args g) {
     constexpr int BM = 128, BN = 128, BK = 64, PITCH = BK + 16;
+    select_problem(g, blockIdx.y);
     constexpr int PLANE = BM * PITCH, STAGE = 2 * PLANE + BN * PITCH;
     __shared__ __attribute__((aligned(16))) int8_t smem[2 * STAGE];
 
@@ -132,7 +144,7 @@ __global__ __launch_bounds__(256) void gemm_i16i8_kernel(Gemm16Args g) {
             for (int t = 0; t < 4; ++t) {
                 const int nn = min(n + t, g.N - 1);
                 add[t] = static_cast<unsigned>(g.bias ? g.bias[nn] : 0) + 128u * static_cast<unsigned>(g.colsum[nn]);
-                const int s = g.shifts[static_cast<int64_t>(nn) * g.shift_stride];
+                const int s = g.shifts ? g.shifts[static_cast<int64_t>(nn) * g.shift_stride] : g.shift;
                 rc[t] = make_round(g.mode, min(max(s, 0), 31));
             }
 #pragma unroll
@@ -156,6 +168,7 @@ __global__ __launch_bounds__(256) void gemm_i16i8_kernel(Gemm16Args g) {
 
 // Any K / alignment: one thread per output element.
 __global__ __launch_bounds__(256) void gemm_i16i8_generic_kernel(Gemm16Args g) {
+    select_problem(g, blockIdx.y);
     const int64_t total = static_cast<int64_t>(g.M) * g.N;
     const int lo_b = g.relu ? max(kind_lo(g.out_kind), 0) : kind_lo(g.out_kind), hi_b = kind_hi(g.out_kind);
     for (int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; idx < total;
@@ -165,7 +178,7 @@ __global__ __launch_bounds__(256) void gemm_i16i8_generic_kernel(Gemm16Args g) {
         const int16_t* ar = g.A + static_cast<int64_t>(m) * g.lda;
         const int8_t* wr = g.Wt + static_cast<int64_t>(n) * g.ldwt;
         for (int k = 0; k < g.K; ++k) acc += static_cast<unsigned>(static_cast<int>(ar[k]) * static_cast<int>(wr[k]));
-        const int s = g.shifts[static_cast<int64_t>(n) * g.shift_stride];
+        const int s = g.shifts ? g.shifts[static_cast<int64_t>(n) * g.shift_stride] : g.shift;
         const int y = clamp_i(apply_round(static_cast<int>(acc), make_round(g.mode, min(max(s, 0), 31))), lo_b, hi_b);
         store_kind(g.Y, static_cast<int64_t>(m) * g.ldy + n, g.out_kind, y);
     }
@@ -191,6 +204,8 @@ struct Gemm16x16Args {
     int64_t lda, ldwt, ldy;
     int M, N, K;
     int shift_stride, relu, out_kind, mode;
+    int64_t stride_a, stride_w, stride_colsum, stride_y;  // batched use, as above
+    int shift;                                            // used when `shifts` is null
 };
 
 __device__ __forceinline__ long long round_shift64(long long v, int s, int mode) {
@@ -216,8 +231,18 @@ __device__ __forceinline__ int requant64(long long v, int s, int mode, int lo, i
 
 // 64 x 128 output tile, K step 64, 4 waves (2 x 2) of 32 x 64, double-buffered LDS with the two byte planes
 // of both operands. Requires K % 16 == 0, 16-byte aligned rows.
+__device__ __forceinline__ void select_problem(Gemm16x16Args& g, int b) {
+    const int obytes = (g.out_kind == A4G_I16 || g.out_kind == A4G_U16) ? 2 : 1;
+    g.A += b * g.stride_a;
+    g.Wh += b * g.stride_w;
+    g.Wl += b * g.stride_w;
+    g.colsum += b * g.stride_colsum;
+    g.Y = static_cast<int8_t*>(g.Y) + b * g.stride_y * obytes;
+}
+
 __global__ __launch_bounds__(256) void gemm_i16i16_kernel(Gemm16x16Args g) {
     constexpr int BM = 64, BN = 128, BK = 64, PITCH = BK + 16;
+    select_problem(g, blockIdx.y);
     constexpr int APLANE = BM * PITCH, WPLANE = BN * PITCH, STAGE = 2 * APLANE + 2 * WPLANE;
     __shared__ __attribute__((aligned(16))) int8_t smem[2 * STAGE];
 
@@ -335,7 +360,7 @@ __global__ __launch_bounds__(256) void gemm_i16i16_kernel(Gemm16x16Args g) {
                 const long long v = (static_cast<long long>(acc_hh[j][q * 4 + t]) << 16) +
                                     ((static_cast<long long>(acc_hl[j][q * 4 + t]) + acc_lh[j][q * 4 + t]) << 8) +
                                     acc_ll[j][q * 4 + t] + row_term + 128ll * g.colsum[nn] + (g.bias ? g.bias[nn] : 0);
-                const int s = min(max(g.shifts[static_cast<int64_t>(nn) * g.shift_stride], 0), 62);
+                const int s = min(max(g.shifts ? g.shifts[static_cast<int64_t>(nn) * g.shift_stride] : g.shift, 0), 62);
                 const int y = requant64(v, s, g.mode, lo_b, hi_b);
                 const int64_t at = static_cast<int64_t>(m) * g.ldy + nn;
                 if (obytes == 1) Yb[at] = static_cast<int8_t>(y);
@@ -347,6 +372,7 @@ __global__ __launch_bounds__(256) void gemm_i16i16_kernel(Gemm16x16Args g) {
 
 // Any K / alignment: one thread per output element, straight from the planes (w = 256 wh + (wl ^ 0x80 as unsigned)).
 __global__ __launch_bounds__(256) void gemm_i16i16_generic_kernel(Gemm16x16Args g) {
+    select_problem(g, blockIdx.y);
     const int64_t total = static_cast<int64_t>(g.M) * g.N;
     const int lo_b = g.relu ? max(kind_lo(g.out_kind), 0) : kind_lo(g.out_kind), hi_b = kind_hi(g.out_kind);
     for (int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; idx < total;
@@ -360,7 +386,7 @@ __global__ __launch_bounds__(256) void gemm_i16i16_generic_kernel(Gemm16x16Args 
             const int w = 256 * static_cast<int>(wh[k]) + static_cast<int>(static_cast<uint8_t>(wl[k]) ^ 0x80u);
             acc += static_cast<long long>(ar[k]) * w;
         }
-        const int s = min(max(g.shifts[static_cast<int64_t>(n) * g.shift_stride], 0), 62);
+        const int s = min(max(g.shifts ? g.shifts[static_cast<int64_t>(n) * g.shift_stride] : g.shift, 0), 62);
         store_kind(g.Y, static_cast<int64_t>(m) * g.ldy + n, g.out_kind, requant64(acc, s, g.mode, lo_b, hi_b));
     }
 }
@@ -383,6 +409,38 @@ __global__ __launch_bounds__(256) void pack_planes_i16_kernel(const int16_t* __r
         Wl[static_cast<int64_t>(n) * ldt + k] = 0;
     }
     colsum[n] = sum;
+}
+
+// Dynamic right operand of a 16-bit MatMul -> what the kernels above read: rows n with k contiguous, plus the column
+// sums. B element (k, n) of problem b sits at B[b * stride_b + (trans_b ? n * ldb + k : k * ldb + n)].
+// WIDE: int16 operand -> the two byte planes and sum_k (b - 128); else int8 -> a transposed copy and sum_k b.
+template <bool WIDE>
+__global__ __launch_bounds__(256) void pack_dynamic_rhs_kernel(const void* __restrict__ B, int64_t ldb, int64_t stride_b, int trans_b,
+                                                               int8_t* __restrict__ hi, int8_t* __restrict__ lo, int64_t ldt,
+                                                               int64_t stride_t, int32_t* __restrict__ colsum, int K, int N) {
+    const int n = blockIdx.x * blockDim.x + threadIdx.x, b = blockIdx.y;
+    if (n >= N) return;
+    int8_t* h = hi + b * stride_t + static_cast<int64_t>(n) * ldt;
+    int8_t* l = WIDE ? lo + b * stride_t + static_cast<int64_t>(n) * ldt : nullptr;
+    int sum = 0;
+    for (int k = 0; k < K; ++k) {
+        const int64_t at = b * stride_b + (trans_b ? static_cast<int64_t>(n) * ldb + k : static_cast<int64_t>(k) * ldb + n);
+        if (WIDE) {
+            const int w = static_cast<const int16_t*>(B)[at];
+            h[k] = static_cast<int8_t>(w >> 8);
+            l[k] = static_cast<int8_t>((w & 0xFF) ^ 0x80);
+            sum += w - 128;
+        } else {
+            const int w = static_cast<const int8_t*>(B)[at];
+            h[k] = static_cast<int8_t>(w);
+            sum += w;
+        }
+    }
+    for (int k = K; k < ldt; ++k) {
+        h[k] = 0;
+        if (WIDE) l[k] = 0;
+    }
+    colsum[static_cast<int64_t>(b) * N + n] = sum;
 }
 
 }  // namespace a4g
@@ -417,7 +475,7 @@ extern "C" int a4g_dense_i16(const int16_t* A, int64_t lda, const int8_t* Wt, in
     if (tiled) {
         const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
         A4G_REQUIRE(tiles <= INT32_MAX, A4G_ERR_UNSUPPORTED, "%s: too many tiles", who);
-        gemm_i16i8_kernel<<<static_cast<unsigned>((tiles + 7) / 8 * 8), 256, 0, stream>>>(g);  // whole ranges for the 8 XCDs
+        gemm_i16i8_kernel<<<dim3(static_cast<unsigned>((tiles + 7) / 8 * 8), 1), 256, 0, stream>>>(g);  // whole ranges for the 8 XCDs
     } else {
         const int grid = static_cast<int>(std::min<int64_t>((M * N + 255) / 256, 256 * 32));
         gemm_i16i8_generic_kernel<<<grid, 256, 0, stream>>>(g);
@@ -466,10 +524,87 @@ extern "C" int a4g_dense_i16x16(const int16_t* A, int64_t lda, const int8_t* Wt_
     if (tiled) {
         const int64_t tiles = ((M + 63) / 64) * ((N + 127) / 128);
         A4G_REQUIRE(tiles <= INT32_MAX, A4G_ERR_UNSUPPORTED, "%s: too many tiles", who);
-        gemm_i16i16_kernel<<<static_cast<unsigned>((tiles + 7) / 8 * 8), 256, 0, stream>>>(g);
+        gemm_i16i16_kernel<<<dim3(static_cast<unsigned>((tiles + 7) / 8 * 8), 1), 256, 0, stream>>>(g);
     } else {
         const int grid = static_cast<int>(std::min<int64_t>((M * N + 255) / 256, 256 * 32));
         gemm_i16i16_generic_kernel<<<grid, 256, 0, stream>>>(g);
+    }
+    return check_hip(hipGetLastError(), who);
+}
+
+extern "C" size_t a4g_matmul_i16_workspace_bytes(int64_t batch, int64_t N, int64_t K, int b_kind) {
+    if (batch <= 0 || N <= 0 || K <= 0) return 0;
+    const int64_t ldt = (K + 15) / 16 * 16;
+    const int64_t planes = b_kind == A4G_I16 ? 2 : 1;
+    return static_cast<size_t>(batch * (planes * N * ldt + N * 4));
+}
+
+extern "C" int a4g_matmul_i16(const int16_t* A, int64_t lda, int64_t stride_a, const void* B, int b_kind, int64_t ldb,
+                              int64_t stride_b, int trans_b, void* C, int64_t ldc, int64_t stride_c, int64_t batch, int64_t M,
+                              int64_t N, int64_t K, int shift, int round_mode, int out_kind, void* workspace,
+                              size_t workspace_bytes, a4g_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const char* who = "a4g_matmul_i16";
+    A4G_REQUIRE(b_kind == A4G_I8 || b_kind == A4G_I16, A4G_ERR_INVALID_ARGUMENT, "%s: matmul RHS must use a signed integer precision", who);
+    A4G_REQUIRE(batch >= 0 && batch <= 65535 && M >= 0 && N >= 1 && K >= 1 && M <= INT32_MAX && N <= (1 << 24) &&
+                    K <= (b_kind == A4G_I16 ? 32768 : (1 << 24)),
+                A4G_ERR_INVALID_ARGUMENT, "%s: bad shape batch=%lld M=%lld N=%lld K=%lld", who, (long long)batch, (long long)M,
+                (long long)N, (long long)K);
+    A4G_REQUIRE(out_kind == A4G_I8 || out_kind == A4G_U8 || out_kind == A4G_I16, A4G_ERR_UNSUPPORTED,
+                "%s: output kind %d is not int8/uint8/int16", who, out_kind);
+    A4G_REQUIRE(valid_round(round_mode), A4G_ERR_INVALID_ARGUMENT, "%s: unknown rounding mode %d", who, round_mode);
+    A4G_REQUIRE(shift >= 0 && shift <= (b_kind == A4G_I16 ? 62 : 31), A4G_ERR_INVALID_ARGUMENT,
+                "%s: matmul accumulator output shift %d out of range", who, shift);
+    A4G_REQUIRE(lda >= K && ldc >= N && ldb >= (trans_b ? K : N), A4G_ERR_INVALID_ARGUMENT, "%s: pitch smaller than the row", who);
+    if (M == 0 || batch == 0) return A4G_OK;
+    A4G_REQUIRE(A && B && C, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+    const size_t need = a4g_matmul_i16_workspace_bytes(batch, N, K, b_kind);
+    A4G_REQUIRE(workspace && workspace_bytes >= need && aligned16(workspace), A4G_ERR_WORKSPACE,
+                "%s: needs a 16-byte aligned workspace of %zu bytes (a4g_matmul_i16_workspace_bytes)", who, need);
+
+    const int64_t ldt = (K + 15) / 16 * 16;
+    const bool wide = b_kind == A4G_I16;
+    int8_t* hi = static_cast<int8_t*>(workspace);
+    int8_t* lo = wide ? hi + batch * N * ldt : nullptr;
+    int32_t* colsum = reinterpret_cast<int32_t*>(hi + (wide ? 2 : 1) * batch * N * ldt);
+    const dim3 pgrid(static_cast<unsigned>((N + 255) / 256), static_cast<unsigned>(batch));
+    if (wide)
+        pack_dynamic_rhs_kernel<true><<<pgrid, 256, 0, stream>>>(B, ldb, stride_b, trans_b, hi, lo, ldt, N * ldt, colsum, (int)K, (int)N);
+    else
+        pack_dynamic_rhs_kernel<false><<<pgrid, 256, 0, stream>>>(B, ldb, stride_b, trans_b, hi, lo, ldt, N * ldt, colsum, (int)K, (int)N);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return check_hip(e, who);
+
+    const bool tiled = K % 16 == 0 && lda % 8 == 0 && stride_a % 8 == 0 && aligned16(A);
+    const unsigned nb = static_cast<unsigned>(batch);
+    if (wide) {
+        Gemm16x16Args g{};
+        g.A = A; g.Wh = hi; g.Wl = lo; g.colsum = colsum; g.bias = nullptr; g.shifts = nullptr; g.Y = C;
+        g.lda = lda; g.ldwt = ldt; g.ldy = ldc;
+        g.M = (int)M; g.N = (int)N; g.K = (int)K;
+        g.out_kind = out_kind; g.mode = round_mode; g.shift = shift;
+        g.stride_a = stride_a; g.stride_w = N * ldt; g.stride_colsum = N; g.stride_y = stride_c;
+        if (tiled) {
+            const int64_t tiles = ((M + 63) / 64) * ((N + 127) / 128);
+            gemm_i16i16_kernel<<<dim3(static_cast<unsigned>((tiles + 7) / 8 * 8), nb), 256, 0, stream>>>(g);
+        } else {
+            const int grid = static_cast<int>(std::min<int64_t>((M * N + 255) / 256, 256 * 32));
+            gemm_i16i16_generic_kernel<<<dim3(grid, nb), 256, 0, stream>>>(g);
+        }
+    } else {
+        Gemm16Args g{};
+        g.A = A; g.Wt = hi; g.colsum = colsum; g.bias = nullptr; g.shifts = nullptr; g.Y = C;
+        g.lda = lda; g.ldwt = ldt; g.ldy = ldc;
+        g.M = (int)M; g.N = (int)N; g.K = (int)K;
+        g.out_kind = out_kind; g.mode = round_mode; g.shift = shift;
+        g.stride_a = stride_a; g.stride_w = N * ldt; g.stride_colsum = N; g.stride_y = stride_c;
+        if (tiled) {
+            const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+            gemm_i16i8_kernel<<<dim3(static_cast<unsigned>((tiles + 7) / 8 * 8), nb), 256, 0, stream>>>(g);
+        } else {
+            const int grid = static_cast<int>(std::min<int64_t>((M * N + 255) / 256, 256 * 32));
+            gemm_i16i8_generic_kernel<<<dim3(grid, nb), 256, 0, stream>>>(g);
+        }
     }
     return check_hip(hipGetLastError(), who);
 }

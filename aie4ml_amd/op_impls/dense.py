@@ -106,7 +106,7 @@ def _resolve_output_scale_shift(node) -> int:
     return shift
 
 
-# (lhs, rhs) storage widths (matmul/common.py:52); the 16-bit ones for Dense only (dynamic MatMul kernels are int8)
+# (lhs, rhs) storage widths (matmul/common.py:52)
 _SUPPORTED_INT_WIDTH_COMBOS = frozenset({(8, 8), (16, 8), (16, 16)})
 
 
@@ -118,7 +118,7 @@ def _bitwidths_supported(node, device) -> bool:
         return False
     lw = resolve_exact_storage_dtype(lhs.precision, namespace='lhs', layer_name=node.name).width
     rw = resolve_exact_storage_dtype(rhs.precision, namespace='rhs', layer_name=node.name).width
-    return (lw, rw) in _SUPPORTED_INT_WIDTH_COMBOS and (node.op_type == 'dense' or lw == 8)
+    return (lw, rw) in _SUPPORTED_INT_WIDTH_COMBOS
 
 
 def _check_out_format(node, fmt: str) -> None:
@@ -288,7 +288,7 @@ class MatmulGpuVariant(OpImplVariant):
         return MatmulConfig(
             precision=precision,
             shift=int(shift),
-            accumulator_tag='acc32',
+            accumulator_tag='acc64' if precision['acc'].format == 'int64' else 'acc32',
             rounding_mode=aie_rounding_token(precision['output']),
             flags=MatmulFlags(transpose_lhs=bool(lp is not None and lp[-1] != len(lp) - 1),
                               transpose_rhs=bool(rp is not None and rp[-1] != len(rp) - 1)),
@@ -304,8 +304,9 @@ class MatmulGpuVariant(OpImplVariant):
             raise ValueError(f'{node.name}: matmul LHS does not support io_view permutation {lp}.')
         if not bool(config.precision['rhs'].signed):
             raise ValueError(f'{node.name}: matmul RHS must use a signed integer precision.')
-        if not 0 <= config.shift <= 31:
-            raise ValueError(f'{node.name}: matmul accumulator output shift must be in [0, 31], got {config.shift}.')
+        top = 62 if config.accumulator_tag == 'acc64' else 31
+        if not 0 <= config.shift <= top:
+            raise ValueError(f'{node.name}: matmul accumulator output shift must be in [0, {top}], got {config.shift}.')
         _check_out_format(node, config.precision['output'].format)
 
     def pack(self, inst) -> Dict[str, Any]:
@@ -318,7 +319,7 @@ class MatmulGpuVariant(OpImplVariant):
         q = to_quant_intent(rhs.precision)
         data = quantize_to_int(rhs.data, q.frac, q.width, signed=q.signed, rounding_mode=q.rounding,
                                saturation_mode=rhs.precision.saturation)
-        return {'rhs_const': torch.from_numpy(np.ascontiguousarray(data.astype(np.int8))).cuda()}
+        return {'rhs_const': torch.from_numpy(np.ascontiguousarray(data.astype(np.int16 if q.width > 8 else np.int8))).cuda()}
 
     def run(self, inst, inputs):
         from .. import ops

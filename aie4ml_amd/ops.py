@@ -155,13 +155,15 @@ def dense(x: torch.Tensor, p: PackedDense, rounding='floor', relu: bool = False,
 
 def matmul(a: torch.Tensor, b: torch.Tensor, shift: int, rounding='floor', trans_b: bool = False, out_kind='int8',
            out: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None):
-    """Batched dynamic MatMul. a: [..., M, K] int8/uint8; b: [..., K, N] int8, or [..., N, K] when
+    """Batched dynamic MatMul. a: [..., M, K] int8/uint8/int16; b: [..., K, N] int8 (int16 with an int16 a), or [..., N, K] when
     ``trans_b`` (the operand is consumed through a last-two-axes transpose view)."""
     _dev(a, 'a'), _dev(b, 'b')
-    if b.dtype != torch.int8:
+    if b.dtype not in (torch.int8, torch.int16):
         raise ValueError('matmul RHS must use a signed integer precision.')
-    if a.dtype not in (torch.int8, torch.uint8):
-        raise NotImplementedError(f'matmul LHS must be int8 or uint8, got {a.dtype}')
+    if a.dtype not in (torch.int8, torch.uint8, torch.int16):
+        raise NotImplementedError(f'matmul LHS must be int8, uint8 or int16, got {a.dtype}')
+    if b.dtype == torch.int16 and a.dtype != torch.int16:
+        raise RuntimeError('unsupported int8 x int16 precision mix for AIE implementations; no implementation variant available.')
     if a.dim() < 2 or b.dim() < 2:
         raise ValueError('matmul operands need rank >= 2')
     a, b = a.contiguous(), b.contiguous()
@@ -180,6 +182,15 @@ def matmul(a: torch.Tensor, b: torch.Tensor, shift: int, rounding='floor', trans
     if out is None:
         out = torch.empty(lead + (M, N), dtype=_KIND_TORCH[ok], device=a.device)
     L = _lib.load()
+    if a.dtype == torch.int16:  # 16-bit left operand: (16, 8) in acc32, (16, 16) in acc64
+        bkind = _TORCH_KIND[b.dtype]
+        need = int(L.a4g_matmul_i16_workspace_bytes(batch, N, K, bkind))
+        if workspace is None or workspace.numel() * workspace.element_size() < need:
+            workspace = torch.empty((need,), dtype=torch.uint8, device=a.device)
+        check(L.a4g_matmul_i16(_ptr(a), K, M * K, _ptr(b), bkind, int(b.shape[-1]), K * N, int(bool(trans_b)), _ptr(out), N, M * N,
+                               batch, M, N, K, int(shift), _mode(rounding), ok, _ptr(workspace),
+                               workspace.numel() * workspace.element_size(), _stream()))
+        return out
     akind = _TORCH_KIND[a.dtype]
     need = int(L.a4g_matmul_i8_workspace_bytes(batch, M, N, K, int(trans_b), akind))
     if need and (workspace is None or workspace.numel() * workspace.element_size() < need):

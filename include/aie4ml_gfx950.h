@@ -66,6 +66,16 @@ enum a4g_kind { A4G_I8 = 0, A4G_U8 = 1, A4G_I16 = 2, A4G_U16 = 3, A4G_I32 = 4 };
 A4G_API int a4g_version(void);
 A4G_API const char* a4g_last_error(void);
 
+/* Dynamic MatMul with an int16 left operand: the (16, 8) and (16, 16) width combinations of the matmul family
+ * (op_impls/families/matmul/common.py:52; docs/support.md: "Dynamic MatMul: Int8/int16"), acc32 and acc64 as for
+ * Dense. B is int8 or int16 (b_kind), [batch][K][ldb] or, with trans_b, [batch][N][ldb]; it is repacked per call
+ * into the workspace (a4g_matmul_i16_workspace_bytes). Other arguments as a4g_matmul_i8. */
+A4G_API size_t a4g_matmul_i16_workspace_bytes(int64_t batch, int64_t N, int64_t K, int b_kind);
+A4G_API int a4g_matmul_i16(const int16_t* A, int64_t lda, int64_t stride_a, const void* B, int b_kind, int64_t ldb,
+                   int64_t stride_b, int trans_b, void* C, int64_t ldc, int64_t stride_c, int64_t batch, int64_t M,
+                   int64_t N, int64_t K, int shift, int round_mode, int out_kind, void* workspace, size_t workspace_bytes,
+                   a4g_stream_t stream);
+
 /* ---- Elementwise Add ---------------------------------------------------------------------------
  * out[i] = srs(a[i] + b[i], shift, round_mode) saturated to `kind` (int8 / uint8 / int16).
  * Replaces elementwise_add_kernel<Cfg>::run, templates/nnet_utils/elementwise_add/

@@ -120,8 +120,17 @@ def dense(A, W, bias, shifts, mode, relu=False, out='int8'):
 
 
 def matmul(A, B, shift, mode, trans_b=False, out='int8'):
-    """Batched: A [..., M, K]; B [..., K, N] (or [..., N, K] when trans_b)."""
+    """Batched: A [..., M, K]; B [..., K, N] (or [..., N, K] when trans_b). An int16 A takes the 16-bit width
+    combinations (B int8: acc32, B int16: acc64): the same accumulation as Dense without bias or ReLU
+    (matmul.cpp:80-115), so each problem of the batch goes through dense()."""
     A = _c(A)
+    if A.dtype == np.int16:
+        B = _c(B)
+        Bm = np.swapaxes(B, -1, -2) if trans_b else B
+        lead = A.shape[:-2]
+        A3, B3 = A.reshape((-1,) + A.shape[-2:]), Bm.reshape((-1,) + Bm.shape[-2:])
+        C = np.stack([dense(A3[i], np.ascontiguousarray(B3[i]), None, int(shift), mode, out=out) for i in range(A3.shape[0])])
+        return C.reshape(lead + C.shape[-2:])
     B = _c(B, np.int8)
     M, K = A.shape[-2:]
     N = B.shape[-2] if trans_b else B.shape[-1]

@@ -236,6 +236,28 @@ def test_int16_weight_mlp_graph(oracle):
     _graph_check(model, oracle, {'x': x})
 
 
+@pytest.mark.parametrize('rhs_bits', [8, 16])
+def test_int16_matmul_graph(oracle, rhs_bits):
+    """Dynamic MatMul with a 16-bit left operand inside a graph: transposed right operand (folded Transpose),
+    then a second MatMul on the result, as the attention score / context pair does."""
+    r = np.random.default_rng(rhs_bits)
+    gb = GraphBuilder()
+    q = gb.input('q', (2, 3, 40, 32), qint(16, 12))
+    k = gb.input('k', (2, 3, 40, 32), qint(rhs_bits, rhs_bits - 2))
+    v = gb.input('v', (2, 3, 40, 32), qint(rhs_bits, rhs_bits - 2))
+    s = gb.matmul(q, gb.transpose(k, (0, 1, 3, 2)), qint(16, 9), name='qk')
+    gb.output(gb.matmul(s, v, qint(16, 8), name='pv'))
+    model = gb.build()
+    model.compile()
+    cfg = model.context.ir.execution.get('qk_aie').config
+    assert cfg.accumulator_tag == ('acc64' if rhs_bits == 16 else 'acc32') and cfg.flags.transpose_rhs
+    lo, hi = -(1 << (rhs_bits - 1)), 1 << (rhs_bits - 1)
+    dt = np.int16 if rhs_bits == 16 else np.int8
+    feeds = {'q': r.integers(-32768, 32768, (2, 3, 40, 32)).astype(np.int16),
+             'k': r.integers(lo, hi, (2, 3, 40, 32)).astype(dt), 'v': r.integers(lo, hi, (2, 3, 40, 32)).astype(dt)}
+    _graph_check(model, oracle, feeds)
+
+
 # ---- float compute path through the graph executor ----------------------------------------------------------------
 
 def _float_net(compute_dtype, batch, n_in=32, n_h=32, n_out=16, seed=0):

@@ -273,6 +273,22 @@ def test_dense_int16_activations_int16_weights(ops, oracle, shape):
         ops.dense(dev(A.astype(np.int8)), p, 'floor')
 
 
+@pytest.mark.parametrize('b_dtype', [np.int8, np.int16])
+@pytest.mark.parametrize('trans_b', [True, False])
+@pytest.mark.parametrize('shape', [((2, 3), 64, 64, 64), ((4,), 130, 96, 48), ((), 70, 17, 24), ((2,), 128, 256, 512)])
+def test_matmul_int16_left_operand(ops, oracle, shape, trans_b, b_dtype):
+    # the 16-bit width combinations of the dynamic MatMul: int16 x int8 (acc32) and int16 x int16 (acc64)
+    lead, M, N, K = shape
+    r = rng(M + N + K + int(trans_b))
+    A = r.integers(-32768, 32768, lead + (M, K)).astype(np.int16)
+    lo, hi = (-128, 128) if b_dtype == np.int8 else (-32768, 32768)
+    B = r.integers(lo, hi, lead + ((N, K) if trans_b else (K, N))).astype(b_dtype)
+    shift = 14 if b_dtype == np.int8 else 22
+    for mode, out in (('conv_even', 'int16'), ('symmetric_inf', 'int8'), ('floor', 'int16')):
+        got = host(ops.matmul(dev(A), dev(B), shift, mode, trans_b=trans_b, out_kind=out))
+        assert np.array_equal(got, oracle.matmul(A, B, shift, mode, trans_b=trans_b, out=out)), (mode, out)
+
+
 @pytest.mark.parametrize('shape', [((2, 3), 200, 96, 32), ((5,), 129, 544, 64), ((2,), 31, 1056, 96), ((), 512, 512, 128),
                                    ((3,), 1, 32, 64)])
 def test_matmul_short_reduction_transposed_rhs(ops, oracle, shape):

@@ -271,11 +271,19 @@ def test_matmul_rules():
     gb.output(gb.dense(a, np.zeros((32, 8)), qint(16, 14), qint(16, 8), name='fc'))
     with pytest.raises((RuntimeError, ValueError)):
         lower(gb)
+    # the dynamic MatMul takes the same width combinations (matmul/common.py:52-66)
+    for rhs_bits, tag in ((8, 'acc32'), (16, 'acc64')):
+        gb = GraphBuilder()
+        a = gb.input('a', (2, 16, 32), qint(16, 8))
+        b = gb.input('b', (2, 32, 16), qint(rhs_bits, 4))
+        gb.output(gb.matmul(a, b, qint(8, 4), name='mm'))
+        cfg = lower(gb).ir.execution.get('mm_aie').config
+        assert cfg.accumulator_tag == tag and cfg.shift == 8 + 4 - 4 and cfg.precision['lhs'].format == 'int16'
     gb = GraphBuilder()
-    a = gb.input('a', (2, 16, 32), qint(16, 8))
-    b = gb.input('b', (2, 32, 16), qint(8, 4))
+    a = gb.input('a', (2, 16, 32), qint(8, 4))
+    b = gb.input('b', (2, 32, 16), qint(16, 4))
     gb.output(gb.matmul(a, b, qint(8, 4)))
-    with pytest.raises(ValueError, match='no matmul variant matches'):
+    with pytest.raises((RuntimeError, ValueError)):
         lower(gb)
 
 
