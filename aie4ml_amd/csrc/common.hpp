@@ -9,6 +9,7 @@
 namespace a4g {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v4f __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef short v2s __attribute__((ext_vector_type(2)));

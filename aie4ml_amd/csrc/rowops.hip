@@ -206,17 +206,46 @@ __device__ __forceinline__ int ln_round(int acc, const LnRound& r) {
     return (acc + r.c0 + bit) >> r.s;
 }
 
+// The normalisation in float arithmetic, exact for the modes whose rounding the float unit has
+// (FR 0: nearest-even, 1: floor of x + h, 2: ceil of x + h) as long as every gamma is within +-511:
+// inv <= 32767 makes |inv * gamma| < 2^24 - 2^14, |x - mu| <= 255 and |fscale| <= 32768 make
+// |vd * fscale + beta + 2^(7+s)| < 2^24 for s <= 15, so each product and sum below is an integer times a
+// power of two that a float holds exactly, and v_rndne / v_floor / v_ceil round the same rational the
+// integer path rounds. The output is produced biased by 128: v_cvt_pk_u8_f32 rounds to nearest even,
+// saturates to 0..255 and inserts the byte, which is the int8 saturation once the bias is removed.
+struct LnFloat {
+    float s1, h1;  // 2^-gamma_shift and the rounding offset of fscale
+    float c, h2;   // 2^-final_shift and 128 + the rounding offset of the output
+};
+static LnFloat make_ln_float(int mode, int gamma_shift, int final_shift, int* fr) {
+    float half = 0.f;
+    int kind = -1;
+    switch (mode) {
+    case A4G_RND_CONV_EVEN: kind = 0; break;
+    case A4G_RND_FLOOR: kind = 1; break;
+    case A4G_RND_POSITIVE_INF: kind = 1; half = 0.5f; break;
+    case A4G_RND_CEIL: kind = 2; break;
+    case A4G_RND_NEGATIVE_INF: kind = 2; half = -0.5f; break;
+    default: break;
+    }
+    *fr = kind;
+    return LnFloat{ldexpf(1.f, -gamma_shift), gamma_shift > 0 ? half : 0.f, ldexpf(1.f, -final_shift),
+                   128.f + (final_shift > 0 ? half : 0.f)};
+}
+constexpr int LN_FLOAT_MAX_GAMMA = 511;
+
 // L lanes per row, 64/L rows per wave at a time; a lane owns the 16-byte chunks l, l+L, ... (NCH of
 // them) of its row. gamma/beta are widened to int32 once per block and kept in LDS, quad-major
 // ([4][nchunks][4] ints) so that the lanes of a group read consecutive 16-byte words. x is read from
 // HBM once: the statistics and the normalisation both work from registers, and the next rows' loads
 // are issued before the current rows are normalised.
-template <int L, int NCH, int BIT, bool FUSE_ADD>
+// FR >= 0 adds the float form of the normalisation, taken by a block whose gamma values allow it.
+template <int L, int NCH, int BIT, bool FUSE_ADD, int FR>
 __global__ __launch_bounds__(256, 2) void layernorm_rows_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ x2,
                                                               const int16_t* __restrict__ gamma,
                                                               const int16_t* __restrict__ beta, int8_t* __restrict__ sum_out,
                                                               int8_t* __restrict__ out, int rows, int cols, int log2c,
-                                                              int eps_q0, LnRound rg, LnRound ro) {
+                                                              int eps_q0, LnRound rg, LnRound ro, LnFloat lf) {
     extern __shared__ int ln_lds[];
     const int nchunks = cols >> 4;
     int* lg = ln_lds;
@@ -253,24 +282,61 @@ __global__ __launch_bounds__(256, 2) void layernorm_rows_kernel(const int8_t* __
         }
     };
 
-    // the first rows are requested before the parameters are staged, so both latencies overlap
+    // The parameter words are requested first and the first rows right behind them: loads return in issue
+    // order, so the parameters (cache hits after the first blocks) are staged while the rows are in flight.
+    const int n_half_chunks = 4 * nchunks;  // 8 int16 parameters each: gamma's, then beta's
+    auto param_word = [&](int hc) {
+        const bool is_beta = hc >= 2 * nchunks;
+        return *reinterpret_cast<const v4i*>((is_beta ? beta : gamma) + (is_beta ? hc - 2 * nchunks : hc) * 8);
+    };
+    v4i first_word = v4i{0, 0, 0, 0};
+    if (static_cast<int>(threadIdx.x) < n_half_chunks) first_word = param_word(threadIdx.x);
     int row0 = wave * G;
     if (row0 < rows) fetch(row0 + grp);
 
-    // 8 int16 parameters per load; half-chunk hc = 8 columns = quads 2*(hc&1), 2*(hc&1)+1 of chunk hc>>1
-    for (int hc = threadIdx.x; hc < 4 * nchunks; hc += blockDim.x) {
-        const bool is_beta = hc >= 2 * nchunks;
-        const int h = is_beta ? hc - 2 * nchunks : hc;
-        const v4i raw = *reinterpret_cast<const v4i*>((is_beta ? beta : gamma) + h * 8);
-        int* dst = is_beta ? lb : lg;
-        const int chunk = h >> 1, q0 = (h & 1) * 2;
-        v4i lo, hi;
-        lo[0] = static_cast<int16_t>(raw[0]); lo[1] = raw[0] >> 16; lo[2] = static_cast<int16_t>(raw[1]); lo[3] = raw[1] >> 16;
-        hi[0] = static_cast<int16_t>(raw[2]); hi[1] = raw[2] >> 16; hi[2] = static_cast<int16_t>(raw[3]); hi[3] = raw[3] >> 16;
-        *reinterpret_cast<v4i*>(dst + ((q0 * nchunks + chunk) << 2)) = lo;
-        *reinterpret_cast<v4i*>(dst + (((q0 + 1) * nchunks + chunk) << 2)) = hi;
+    // half-chunk hc = 8 columns = quads 2*(hc&1), 2*(hc&1)+1 of chunk hc>>1.
+    // as_float: gamma as float, beta scaled to the output's unit, biased and offset (the float form's operands)
+    auto stage_params = [&](bool as_float) {
+        int wide = 0;
+        for (int hc = threadIdx.x; hc < n_half_chunks; hc += blockDim.x) {
+            const bool is_beta = hc >= 2 * nchunks;
+            const int h = is_beta ? hc - 2 * nchunks : hc;
+            const v4i raw = hc == static_cast<int>(threadIdx.x) ? first_word : param_word(hc);
+            int* dst = is_beta ? lb : lg;
+            const int chunk = h >> 1, q0 = (h & 1) * 2;
+            v4i q[2];
+            q[0][0] = static_cast<int16_t>(raw[0]); q[0][1] = raw[0] >> 16; q[0][2] = static_cast<int16_t>(raw[1]); q[0][3] = raw[1] >> 16;
+            q[1][0] = static_cast<int16_t>(raw[2]); q[1][1] = raw[2] >> 16; q[1][2] = static_cast<int16_t>(raw[3]); q[1][3] = raw[3] >> 16;
+#pragma unroll
+            for (int k = 0; k < 2; ++k) {
+                int* at = dst + (((q0 + k) * nchunks + chunk) << 2);
+                if (as_float) {
+                    v4f f;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        if (!is_beta) wide |= abs(q[k][j]) > LN_FLOAT_MAX_GAMMA;
+                        f[j] = is_beta ? fmaf(static_cast<float>(q[k][j]), lf.c, lf.h2) : static_cast<float>(q[k][j]);
+                    }
+                    *reinterpret_cast<v4f*>(at) = f;
+                } else {
+                    *reinterpret_cast<v4i*>(at) = q[k];
+                }
+            }
+        }
+        return wide;
+    };
+    bool in_float = false;
+    if (FR >= 0) {
+        // staged for the float form first; a block that meets a gamma beyond its range stages again as integers
+        in_float = !__syncthreads_or(stage_params(true));
+        if (!in_float) {
+            stage_params(false);
+            __syncthreads();
+        }
+    } else {
+        stage_params(false);
+        __syncthreads();
     }
-    __syncthreads();
 
     for (; row0 < rows; row0 += nwaves * G) {
         const int row = row0 + grp;
@@ -301,6 +367,38 @@ __global__ __launch_bounds__(256, 2) void layernorm_rows_kernel(const int8_t* __
         sq = group_allreduce<L>(sq, OpAdd());
         const RowStats st = row_stats(sx, sq, cols, log2c, eps_q0);
 
+        if (FR >= 0 && in_float) {
+            const float inv_s = static_cast<float>(st.inv) * lf.s1;
+            const float nm = -static_cast<float>(st.mu + 128) * lf.c;
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) {
+                v4i o;
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    const int at = (w * nchunks + chunk_of[i]) << 2;
+                    const v4f g4 = *reinterpret_cast<const v4f*>(lg + at);
+                    const v4f b4 = *reinterpret_cast<const v4f*>(lb + at);
+                    const unsigned word = static_cast<unsigned>(xv[i][w]) ^ 0x80808080u;
+                    unsigned packed = 0;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const float vd = fmaf(static_cast<float>((word >> (8 * j)) & 0xffu), lf.c, nm);
+                        float p;
+                        if (FR == 0) p = rintf(inv_s * g4[j]);
+                        if (FR == 1) p = floorf(fmaf(inv_s, g4[j], lf.h1));
+                        if (FR == 2) p = ceilf(fmaf(inv_s, g4[j], lf.h1));
+                        const float fs = __builtin_amdgcn_fmed3f(p, -32768.f, 32767.f);
+                        float y = fmaf(vd, fs, b4[j]);
+                        if (FR == 1) y = floorf(y);
+                        if (FR == 2) y = ceilf(y);
+                        packed = __builtin_amdgcn_cvt_pk_u8_f32(y, j, packed);
+                    }
+                    o[w] = static_cast<int>(packed ^ 0x80808080u);
+                }
+                if (live && valid[i]) __builtin_nontemporal_store(o, reinterpret_cast<v4i*>(out + base + chunk_of[i] * 16));
+            }
+            continue;
+        }
 #pragma unroll
         for (int i = 0; i < NCH; ++i) {
             v4i o;
@@ -366,20 +464,25 @@ __global__ __launch_bounds__(256) void layernorm_generic_kernel(const int8_t* __
     }
 }
 
+// The rounding modes pair up as (BIT, FR): conv_even (3, 0), floor / positive_inf (0, 1), ceil / negative_inf (0, 2);
+// the symmetric modes and conv_odd have no float form (FR -1).
 template <int L, int NCH>
-static void launch_ln_rows(int bit_kind, bool fuse, int grid, size_t lds, hipStream_t stream, const int8_t* x,
+static void launch_ln_rows(int bit_kind, int fr, bool fuse, int grid, size_t lds, hipStream_t stream, const int8_t* x,
                            const int8_t* x2, const int16_t* gamma, const int16_t* beta, int8_t* sum_out, int8_t* out,
-                           int rows, int cols, int log2c, int eps_q0, const LnRound& rg, const LnRound& ro) {
-#define A4G_LN_CASE(B)                                                                                                   \
-    case B:                                                                                                              \
+                           int rows, int cols, int log2c, int eps_q0, const LnRound& rg, const LnRound& ro,
+                           const LnFloat& lf) {
+#define A4G_LN_CASE(B, F)                                                                                                \
+    if (bit_kind == B && fr == F) {                                                                                      \
         if (fuse)                                                                                                        \
-            layernorm_rows_kernel<L, NCH, B, true><<<grid, 256, lds, stream>>>(x, x2, gamma, beta, sum_out, out, rows,   \
-                                                                               cols, log2c, eps_q0, rg, ro);             \
+            layernorm_rows_kernel<L, NCH, B, true, F><<<grid, 256, lds, stream>>>(x, x2, gamma, beta, sum_out, out,      \
+                                                                                  rows, cols, log2c, eps_q0, rg, ro, lf); \
         else                                                                                                             \
-            layernorm_rows_kernel<L, NCH, B, false><<<grid, 256, lds, stream>>>(x, nullptr, gamma, beta, nullptr, out,   \
-                                                                                rows, cols, log2c, eps_q0, rg, ro);      \
-        break;
-    switch (bit_kind) { A4G_LN_CASE(0) A4G_LN_CASE(1) A4G_LN_CASE(2) A4G_LN_CASE(3) A4G_LN_CASE(4) }
+            layernorm_rows_kernel<L, NCH, B, false, F><<<grid, 256, lds, stream>>>(x, nullptr, gamma, beta, nullptr,     \
+                                                                                   out, rows, cols, log2c, eps_q0, rg,   \
+                                                                                   ro, lf);                              \
+        return;                                                                                                          \
+    }
+    A4G_LN_CASE(3, 0) A4G_LN_CASE(0, 1) A4G_LN_CASE(0, 2) A4G_LN_CASE(1, -1) A4G_LN_CASE(2, -1) A4G_LN_CASE(4, -1)
 #undef A4G_LN_CASE
 }
 
@@ -415,13 +518,16 @@ static int layernorm_dispatch(const int8_t* a, const int8_t* b, int add_shift, i
         int bit_kind = 0, unused = 0;
         const LnRound rg = make_ln_round(mode, gamma_shift, &bit_kind);
         const LnRound ro = make_ln_round(mode, final_shift, &unused);
+        int fr = -1;
+        const LnFloat lf = make_ln_float(mode, gamma_shift, final_shift, &fr);
         const size_t lds = static_cast<size_t>(cols) * 8;
-        // The kernel is bound by its integer arithmetic (about 16 VALU instructions per element), not by
-        // HBM: a grid of 8 blocks per CU keeps every SIMD supplied with ready waves.
-        const int max_grid = 256 * 8;
+        // Four blocks per CU: every wave then normalises at least two groups of rows, so the loads of the
+        // second group and the stores of the first overlap the arithmetic (one group per wave leaves the
+        // three phases of all waves in step with each other).
+        const int max_grid = 256 * 4;
 #define A4G_LN_GO(L, NCH)                                                                                                \
-    launch_ln_rows<L, NCH>(bit_kind, fuse, grid_for(rows, 4 * (64 / L), max_grid), lds, stream, a, b, gamma, beta, sum_out, \
-                           out, (int)rows, (int)cols, log2c, eps_q0, rg, ro)
+    launch_ln_rows<L, NCH>(bit_kind, fr, fuse, grid_for(rows, 4 * (64 / L), max_grid), lds, stream, a, b, gamma, beta,    \
+                           sum_out, out, (int)rows, (int)cols, log2c, eps_q0, rg, ro, lf)
         if (nchunks <= 16) A4G_LN_GO(8, 2);
         else if (nchunks <= 32) A4G_LN_GO(16, 2);
         else if (nchunks <= 48) A4G_LN_GO(16, 3);

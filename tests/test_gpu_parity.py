@@ -375,6 +375,34 @@ def test_layernorm_degenerate_rows(ops, oracle):
     assert np.array_equal(got, oracle.layernorm(x, gamma, beta, 5, 'conv_even'))
 
 
+@pytest.mark.parametrize('mode', MODES)
+@pytest.mark.parametrize('gmax', [511, 512])
+def test_layernorm_gamma_at_the_float_limit(ops, oracle, mode, gmax):
+    """The row kernel normalises in float arithmetic while every |gamma| <= 511 and in integers otherwise; both must
+    be the reference's integers. Rows of tiny variance make inv_std16 as large as it gets (products next to 2^24),
+    beta spans int16, the shifts span their ranges."""
+    cols = 512
+    r = rng(gmax)
+    gamma = r.integers(-gmax, gmax + 1, cols).astype(np.int16)
+    gamma[:4] = (gmax, -gmax, gmax - 1, 1 - gmax)
+    beta = r.integers(-32768, 32768, cols).astype(np.int16)
+    beta[:4] = (32767, -32768, 32767, -32768)
+    x = gauss8(r, 40, (48, cols))
+    x[:8] = 0
+    x[0, 0] = 1                 # variance rounds to 0: inv_std16 = 32767 at eps 1
+    x[1, :3] = (127, -128, 127)
+    x[2] = 5
+    x[3, ::2], x[3, 1::2] = 127, -128
+    x[4, :4] = (-128, -128, 127, 127)
+    for gamma_shift, out_shift, eps in ((7, 5, 1), (0, 15, 1), (15, 0, 2), (3, 8, 1), (7, 0, 1)):
+        got = host(ops.layernorm(dev(x), dev(gamma), dev(beta), out_shift, mode, eps_q0=eps, gamma_shift=gamma_shift))
+        exp = oracle.layernorm(x, gamma, beta, out_shift, mode, eps_q0=eps, gamma_shift=gamma_shift)
+        assert np.array_equal(got, exp), (mode, gmax, gamma_shift, out_shift)
+    a, b = gauss8(r, 70, (48, cols)), gauss8(r, 70, (48, cols))
+    got = host(ops.add_layernorm(dev(a), dev(b), dev(gamma), dev(beta), 6, mode))
+    assert np.array_equal(got, oracle.add_layernorm(a, b, gamma, beta, 6, mode)), (mode, gmax)
+
+
 @pytest.mark.parametrize('cols', [64, 768, 1024, 100])
 def test_add_layernorm_fused(ops, oracle, cols):
     r = rng(cols + 7)
