@@ -28,6 +28,7 @@ struct AttnArgs {
     FastRound lr, orr;  // logits and output requantisation
     SoftmaxParams sm;
     int noclamp;
+    float lscale;  // 2^-logit_shift, for the float form of the logit requantisation
 };
 
 // 4x4 byte transpose: in a[i] byte j  ->  out c[j] byte i.
@@ -43,7 +44,10 @@ __device__ __forceinline__ void transpose4x4(const unsigned a[4], unsigned c[4])
 }
 
 // NT = key/value rows / 32, DT = head dimension / 32. 256 threads = 4 waves = 128 query rows of one head.
-// BIT: rounding kind of the logits (fast_round_kind). FASTP: the probabilities need no clamp and their shift is
+// BIT: rounding kind of the logits (fast_round_kind), or 3: round to nearest even done in float arithmetic -
+// |acc| <= D * 2^14 and the bias 2^(7+shift) stay below 2^24, so (acc + 128 * 2^s) * 2^-s is exact in a float and
+// v_cvt_pk_u8_f32 (nearest even, saturating to 0..255, writing one byte of a dword) is the rounding, the int8
+// saturation (biased by 128) and the packing at once. FASTP: the probabilities need no clamp and their shift is
 // at most 16, so p = (e * inv) >> shift is read as byte 2 of e * (inv << (16 - shift)).
 // NW = waves per workgroup. 4: two workgroups share a CU. 8: one workgroup of 256 query rows per CU, which
 // leaves room to store the score table once per LDS bank (entry d for lane c at dword d * 64 + c, byte address
@@ -120,8 +124,9 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
     }
 
     // ---- pass A: logits = srs(Q K^T), packed int8 in registers; running row maximum -----------------
-    unsigned lg[NT][4];
+    unsigned lg[NT][4];  // biased by 128: byte = logit ^ 0x80
     int mx = -128;
+    float mxf = 0.f;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
         if (t + 1 < NT) {
@@ -136,20 +141,39 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
             acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[t & 1][ks], qf[ks], acc, 0, 0, 0);
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-            int y[4];
+            if (BIT == 3) {
+                float f[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) y[i] = clamp_i(fast_round_k<BIT>(acc[4 * g + i], a.lr), -128, 127);
-            mx = max(max(mx, y[0]), max(y[1], max(y[2], y[3])));
-            lg[t][g] = pack4_bytes(y[0], y[1], y[2], y[3]);
+                for (int i = 0; i < 4; ++i) f[i] = fmaf(static_cast<float>(acc[4 * g + i]), a.lscale, 128.f);
+                mxf = __builtin_fmaxf(__builtin_fmaxf(mxf, __builtin_fmaxf(f[0], f[1])), __builtin_fmaxf(f[2], f[3]));
+                unsigned w = __builtin_amdgcn_cvt_pk_u8_f32(f[0], 0, 0u);
+                w = __builtin_amdgcn_cvt_pk_u8_f32(f[1], 1, w);
+                w = __builtin_amdgcn_cvt_pk_u8_f32(f[2], 2, w);
+                lg[t][g] = __builtin_amdgcn_cvt_pk_u8_f32(f[3], 3, w);
+            } else {
+                int y[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) y[i] = clamp_i(fast_round_k<BIT>(acc[4 * g + i], a.lr), -128, 127);
+                mx = max(max(mx, y[0]), max(y[1], max(y[2], y[3])));
+                lg[t][g] = pack4_bytes(y[0], y[1], y[2], y[3]) ^ 0x80808080u;
+            }
         }
         if (NT >= 16) __builtin_amdgcn_sched_barrier(0);  // one tile of K fragments in flight, not all sixteen
     }
-    mx = max(mx, lane_xor<32>(mx));  // lanes m and m+32 share a row
+    // the row maximum as a biased byte; rounding and saturation are monotone, so they commute with the maximum
+    unsigned mxb;
+    if (BIT == 3) {
+        mxf = __builtin_fmaxf(mxf, __builtin_bit_cast(float, lane_xor<32>(__builtin_bit_cast(int, mxf))));
+        mxb = __builtin_amdgcn_cvt_pk_u8_f32(mxf, 0, 0u);
+    } else {
+        mx = max(mx, lane_xor<32>(mx));  // lanes m and m+32 share a row
+        mxb = static_cast<unsigned>((mx ^ 0x80) & 0xFF);
+    }
 
     __syncthreads();  // V^T, column sums and the score table are complete
 
     // ---- pass B: scores by table lookup on the gap to the maximum; row sum ----------------------------
-    const unsigned mrep = static_cast<unsigned>((mx ^ 0x80) & 0xFF) * 0x01010101u;
+    const unsigned mrep = mxb * 0x01010101u;
     const char* tbytes = reinterpret_cast<const char*>(table);
     const unsigned two = 2;
     const unsigned lane4 = static_cast<unsigned>(lane) << 2;  // BANKED: this lane's copy of the table
@@ -159,7 +183,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
     for (int t = 0; t < NT; ++t) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-            const unsigned d4 = mrep - (lg[t][g] ^ 0x80808080u);  // per byte, never borrows
+            const unsigned d4 = mrep - lg[t][g];  // per byte, never borrows
             int e0, e1, e2, e3;
             if (BANKED) {
                 e0 = *reinterpret_cast<const int*>(tbytes + __builtin_amdgcn_perm(d4, lane4, 0x0c0c0400u));
@@ -269,10 +293,11 @@ static void launch_attention_nt(int grid, int grid8, size_t lds, hipStream_t str
         attention_kernel<NT, DT, B, true><<<grid, 256, lds, stream>>>(a);            \
     else                                                                             \
         attention_kernel<NT, DT, B, false><<<grid, 256, lds, stream>>>(a);
-    switch (fast_round_kind(a.lr)) {
+    switch (a.lscale > 0.f ? 3 : fast_round_kind(a.lr)) {
     case 0: A4G_ATTN(0) break;
     case 1: A4G_ATTN(1) break;
-    default: A4G_ATTN(2) break;
+    case 2: A4G_ATTN(2) break;
+    default: A4G_ATTN(3) break;
     }
 #undef A4G_ATTN
 }
@@ -340,6 +365,9 @@ extern "C" int a4g_attention_i8(const int8_t* Q, const int8_t* K, const int8_t* 
     a.lr = make_fast_round(logit_round_mode, logit_shift);
     a.orr = make_fast_round(out_round_mode, out_shift);
     a.noclamp = noclamp;
+    // nearest-even logits take the float form: d * 2^14 + 2^(7 + shift) < 2^24 for the head dimensions covered
+    a.lscale = (logit_round_mode == A4G_RND_CONV_EVEN && logit_shift >= 1 && logit_shift <= 15 && d <= 512)
+                   ? ldexpf(1.f, -logit_shift) : 0.f;
     const int grid = static_cast<int>(batch * heads * ((sq + 127) / 128));
     // eight waves per workgroup (256 query rows, bank-replicated score table) once every CU gets at least one
     const int64_t wg8 = batch * heads * ((sq + 255) / 256);

@@ -88,6 +88,29 @@ def test_attention_zero_shift_and_saturation(oracle):
     np.testing.assert_array_equal(got, reference(oracle, q, k, v, 10, 'conv_even', sm, 3, 'conv_even'))
 
 
+@pytest.mark.parametrize('sq,sk', [(96, 64), (256, 256)])
+def test_attention_nearest_even_logits_at_every_shift(oracle, sq, sk):
+    """Nearest-even logits are requantised in float arithmetic inside the kernel: every shift it covers, operands
+    at the int8 extremes (accumulators of +-64 * 2^14, saturating both ways) and rows built to land on exact ties."""
+    r = np.random.default_rng(sq + sk)
+    q, k, v = qkv(11, (2, 2, sq, 64), (2, 2, sk, 64), sigma=50.0)
+    q[0, 0, :8] = -128
+    q[0, 0, 8:16] = 127
+    k[0, 0, :8] = -128
+    k[0, 0, 8:16] = 127
+    # ties: q row = one-hot * 1, k rows with odd small values -> acc = odd multiples of 2^(s-1) for several s
+    q[1, 1, :32] = 0
+    q[1, 1, np.arange(32), np.arange(32)] = 1 << (np.arange(32) % 7)
+    k[1, 1] = r.integers(-5, 6, (sk, 64)).astype(np.int8)
+    sm = {'kind': 'exp', 'exp_kq': 23}
+    for shift in range(0, 16):
+        got = ops.attention(dev(q), dev(k), dev(v), shift, 'conv_even', sm, 7, 'conv_even').cpu().numpy()
+        np.testing.assert_array_equal(got, reference(oracle, q, k, v, shift, 'conv_even', sm, 7, 'conv_even'), str(shift))
+    for shift in (16, 20, 24):  # beyond the float form's range: the integer form
+        got = ops.attention(dev(q), dev(k), dev(v), shift, 'conv_even', sm, 7, 'conv_even').cpu().numpy()
+        np.testing.assert_array_equal(got, reference(oracle, q, k, v, shift, 'conv_even', sm, 7, 'conv_even'), str(shift))
+
+
 def test_attention_on_head_slices_of_a_packed_projection(oracle):
     """Q, K, V as strided views of one [batch, seq, 3*hidden] tensor, output written into the head's
     columns of a [batch, seq, hidden] tensor: the layout of an encoder block, no copies."""
