@@ -87,12 +87,31 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
         kf[0][ks] = *reinterpret_cast<const v4i*>(Kp + m * a.k_ss + ks * 32 + half * 16);
     }
 
+    // V is requested before anything else is done with LDS, so that building the score table hides its latency:
+    // a thread owns the 4x4 byte blocks blk = tid, tid + THREADS, ... (rows k0..k0+3, its four columns n0..n0+3)
+    constexpr int NB = (SK / 4) * (D / 4);
+    constexpr int VB = (NB + THREADS - 1) / THREADS;
+    const int n0 = (tid % (D / 4)) * 4;  // THREADS % (D/4) == 0: a thread keeps its four columns
+    unsigned av[VB][4];
+#pragma unroll
+    for (int it = 0; it < VB; ++it) {
+        const int blk = tid + it * THREADS;
+        const int k0 = (blk / (D / 4)) * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            av[it][i] = blk < NB ? *reinterpret_cast<const unsigned*>(Vp + (k0 + i) * a.v_ss + n0) : 0u;
+    }
+
     if (BANKED) {
-        // each entry is computed once, parked in the (still unused) V^T area, then copied to its 64 slots
+        // each entry is computed once, parked in the (still unused) V^T area, then copied to its 64 slots, four
+        // slots per 16-byte store
         int* once = reinterpret_cast<int*>(vt);
         if (tid < 256) once[tid] = table_entry(a.sm, tid);
         __syncthreads();
-        for (int i = tid; i < 256 * 64; i += THREADS) table[i] = once[i >> 6];
+        for (int i = tid * 4; i < 256 * 64; i += THREADS * 4) {
+            const int e = once[i >> 6];
+            *reinterpret_cast<v4i*>(table + i) = v4i{e, e, e, e};
+        }
     } else {
         table[tid] = table_entry(a.sm, tid);
     }
@@ -102,21 +121,21 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
     // V -> LDS, transposed in 4x4 byte blocks. Within each group of 32 k, position 16*half + 4*g + i holds
     // k = 8*g + 4*half + i: the order in which a lane's probability registers run.
     {
-        constexpr int NB = (SK / 4) * (D / 4);
-        const int n0 = (tid % (D / 4)) * 4;  // THREADS % (D/4) == 0: a thread keeps its four columns
         int part[4] = {0, 0, 0, 0};
-        for (int blk = tid; blk < NB; blk += THREADS) {
-            const int k0 = (blk / (D / 4)) * 4;
-            unsigned av[4], cv[4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) av[i] = *reinterpret_cast<const unsigned*>(Vp + (k0 + i) * a.v_ss + n0);
-            transpose4x4(av, cv);
-            const int kk = k0 & 31;
-            const int pos = (k0 & ~31) + ((kk >> 2) & 1) * 16 + (kk >> 3) * 4;
+        for (int it = 0; it < VB; ++it) {
+            const int blk = tid + it * THREADS;
+            if (blk < NB) {
+                const int k0 = (blk / (D / 4)) * 4;
+                unsigned cv[4];
+                transpose4x4(av[it], cv);
+                const int kk = k0 & 31;
+                const int pos = (k0 & ~31) + ((kk >> 2) & 1) * 16 + (kk >> 3) * 4;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                *reinterpret_cast<unsigned*>(vt + (n0 + j) * PITCH + pos) = cv[j];
-                part[j] = __builtin_amdgcn_sdot4(static_cast<int>(cv[j]), 0x01010101, part[j], false);
+                for (int j = 0; j < 4; ++j) {
+                    *reinterpret_cast<unsigned*>(vt + (n0 + j) * PITCH + pos) = cv[j];
+                    part[j] = __builtin_amdgcn_sdot4(static_cast<int>(cv[j]), 0x01010101, part[j], false);
+                }
             }
         }
 #pragma unroll
