@@ -397,6 +397,7 @@ struct I8Policy {
     using acc_t = v16i;
     static constexpr int MMAS = 1;
     static constexpr bool FIX_A = A_UNSIGNED;
+    static constexpr bool SPLIT_A = false;
     static constexpr int MAX_OUT_BYTES = 2;
     template <int BN>
     static constexpr int param_bytes() { return ColParams<BN>::BYTES; }
@@ -420,6 +421,50 @@ struct I8Policy {
                                                     int8_t* smem, int8_t* lds_params, int path, int wm, int wn, int lane,
                                                     int tid) {
         epilogue_store<BM, BN, WTM, WTN, NT>(g, tc, acc, smem, ColParams<BN>(lds_params), path, wm, wn, lane, tid);
+    }
+};
+
+// int16 activations: A is split into its signed high bytes and its low bytes (biased by 128 to be signed too)
+// while it is staged, the two planes being alternate runs of rows of the tile, so the unchanged main loop
+// leaves a wave with the two partial products of every output in the same lane and register of two of its
+// accumulator blocks: acc = 256 * sum(hi * w) + sum((lo - 128) * w) + 128 * sum(w), the last term joining the
+// bias as it does for an unsigned operand. Wrapping 32-bit arithmetic throughout, as acc32 does.
+struct I16Policy : I8Policy<false> {
+    static constexpr bool SPLIT_A = true;
+    __device__ static __forceinline__ void split_a(v4i& x, v4i& y) {
+        v4i hi, lo;
+        hi[0] = static_cast<int>(__builtin_amdgcn_perm(x[1], x[0], 0x07050301u));
+        hi[1] = static_cast<int>(__builtin_amdgcn_perm(x[3], x[2], 0x07050301u));
+        hi[2] = static_cast<int>(__builtin_amdgcn_perm(y[1], y[0], 0x07050301u));
+        hi[3] = static_cast<int>(__builtin_amdgcn_perm(y[3], y[2], 0x07050301u));
+        lo[0] = static_cast<int>(__builtin_amdgcn_perm(x[1], x[0], 0x06040200u) ^ 0x80808080u);
+        lo[1] = static_cast<int>(__builtin_amdgcn_perm(x[3], x[2], 0x06040200u) ^ 0x80808080u);
+        lo[2] = static_cast<int>(__builtin_amdgcn_perm(y[1], y[0], 0x06040200u) ^ 0x80808080u);
+        lo[3] = static_cast<int>(__builtin_amdgcn_perm(y[3], y[2], 0x06040200u) ^ 0x80808080u);
+        x = hi;
+        y = lo;
+    }
+    template <int BN>
+    __device__ static __forceinline__ void fetch_params(const GemmArgs& g, const TileCoord& tc, int tid, ColRegs& r) {
+        fetch_col_params<BN, true>(g, tc, tid, r.add, r.shift);  // + 128 * column sum
+    }
+    template <int BM, int BN, int WTM, int WTN, int NT>
+    __device__ static __forceinline__ void epilogue(const GemmArgs& g, const TileCoord& tc, v16i (&acc)[WTM / 32][WTN / 32],
+                                                    int8_t* smem, int8_t* lds_params, int path, int wm, int wn, int lane,
+                                                    int tid) {
+        constexpr int PB = NT / 256;  // 32-row blocks per run of one plane (rows covered by one load per thread / 32)
+        v16i sum[WTM / 64][WTN / 32];
+#pragma unroll
+        for (int i = 0; i < WTM / 64; ++i) {
+            const int hi_blk = (i / PB) * 2 * PB + i % PB, lo_blk = hi_blk + PB;
+#pragma unroll
+            for (int j = 0; j < WTN / 32; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    sum[i][j][r] = static_cast<int>((static_cast<unsigned>(acc[hi_blk][j][r]) << 8) +
+                                                    static_cast<unsigned>(acc[lo_blk][j][r]));
+        }
+        epilogue_store<BM / 2, BN, WTM / 2, WTN, NT>(g, tc, sum, smem, ColParams<BN>(lds_params), path, wm, wn, lane, tid);
     }
 };
 
@@ -706,6 +751,17 @@ static hipError_t launch_dtl_u(const GemmArgs& g, int batch, hipStream_t stream)
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool A_UNSIGNED, bool EARLY = false>
 static hipError_t launch_rs_u(const GemmArgs& g, int batch, hipStream_t stream) {
     return launch_rs_policy<I8Policy<A_UNSIGNED>, BM, BN, WAVES_M, WAVES_N, EARLY>(g, batch, stream);
+}
+
+bool rs_i16i8_applicable(const GemmArgs& g, int batch) {
+    // whole 128-element K tiles, 16-byte aligned rows, and enough 128 x 256 tiles to give every CU one
+    return g.K % 128 == 0 && g.K >= 256 && g.lda % 16 == 0 && g.stride_a % 16 == 0 && g.ldb % 16 == 0 &&
+           g.stride_b % 16 == 0 && aligned16(g.A) && aligned16(g.Bt) && g.colsum != nullptr &&
+           static_cast<int64_t>((g.M + 127) / 128) * ((g.N + 255) / 256) * batch >= 192;
+}
+
+hipError_t launch_rs_i16i8(const GemmArgs& g, int batch, hipStream_t stream) {
+    return launch_rs_policy<I16Policy, 256, 256, 2, 4, true>(g, batch, stream);
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N>

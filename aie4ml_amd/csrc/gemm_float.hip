@@ -65,6 +65,7 @@ struct FloatPolicy {
     static constexpr int ES = FMT == A4G_F32 ? 4 : (FMT == A4G_FP8 ? 1 : 2);
     static constexpr int MMAS = FMT == A4G_F32 ? 4 : (FMT == A4G_FP8 ? 2 : 1);
     static constexpr bool FIX_A = false;
+    static constexpr bool SPLIT_A = false;
     static constexpr int MAX_OUT_BYTES = ES;
     template <int BN>
     static constexpr int param_bytes() { return 4 * BN; }

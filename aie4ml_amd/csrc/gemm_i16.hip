@@ -471,6 +471,15 @@ extern "C" int a4g_dense_i16(const int16_t* A, int64_t lda, const int8_t* Wt, in
     g.relu = relu != 0;
     g.out_kind = out_kind;
     g.mode = round_mode;
+    {
+        // large problems with whole 128-element K tiles: the software-pipelined kernel with the plane split in its staging
+        GemmArgs r{};
+        r.A = reinterpret_cast<const int8_t*>(A); r.Bt = Wt; r.C = Y; r.bias = bias; r.colsum = colsum; r.shifts = shifts;
+        r.lda = lda * 2; r.ldb = ldwt; r.ldc = ldy;
+        r.M = g.M; r.N = g.N; r.K = g.K;
+        r.shift_stride = g.shift_stride; r.relu = g.relu; r.out_kind = out_kind; r.mode = round_mode;
+        if (rs_i16i8_applicable(r, 1)) return check_hip(launch_rs_i16i8(r, 1, stream), who);
+    }
     const bool tiled = K % 16 == 0 && lda % 8 == 0 && ldwt % 16 == 0 && aligned16(A) && aligned16(Wt);
     if (tiled) {
         const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
@@ -598,6 +607,13 @@ extern "C" int a4g_matmul_i16(const int16_t* A, int64_t lda, int64_t stride_a, c
         g.M = (int)M; g.N = (int)N; g.K = (int)K;
         g.out_kind = out_kind; g.mode = round_mode; g.shift = shift;
         g.stride_a = stride_a; g.stride_w = N * ldt; g.stride_colsum = N; g.stride_y = stride_c;
+        GemmArgs r{};
+        r.A = reinterpret_cast<const int8_t*>(A); r.Bt = hi; r.C = C; r.colsum = colsum;
+        r.lda = lda * 2; r.stride_a = stride_a * 2; r.ldb = ldt; r.stride_b = N * ldt; r.ldc = ldc; r.stride_c = stride_c;
+        r.stride_colsum = N;
+        r.M = g.M; r.N = g.N; r.K = g.K;
+        r.shift = shift; r.out_kind = out_kind; r.mode = round_mode;
+        if (rs_i16i8_applicable(r, nb)) return check_hip(launch_rs_i16i8(r, nb, stream), who);
         if (tiled) {
             const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
             gemm_i16i8_kernel<<<dim3(static_cast<unsigned>((tiles + 7) / 8 * 8), nb), 256, 0, stream>>>(g);

@@ -7,6 +7,8 @@
 //   FIX_A, fix_a(v4i&)           optional fix-up of an A fragment before use
 //   mma(b, a, acc)               acc += the 32 x 32 block product of two fragments
 //   MAX_OUT_BYTES                widest output element (sizes the LDS image of the output tile)
+//   SPLIT_A / split_a(x, y)      A elements are two bytes wide: a thread loads 16 of them as two registers and
+//                                turns them into their 16 high and 16 low bytes, which become two tile rows
 //   param_bytes<BN>()            LDS bytes of the per-column epilogue parameters
 //   ColRegs, fetch_params<BN>, park_params<BN>   issue the loads of a thread's column parameters early,
 //                                store them to LDS later (park_params contains a barrier and returns a
@@ -146,6 +148,14 @@ struct RsCfg {
     static_assert(ROWS_PER_PASS % 16 == 0, "the swizzle term must not depend on the pass");
     static_assert((BM + BN) * BK <= 65536, "ds_write immediate offsets are 16 bits");
     static_assert(LDS_BYTES <= 160 * 1024, "LDS budget");
+    // SPLIT_A: the tile's BM rows are BM/2 rows of two-byte elements seen as byte planes. Load 2j / 2j+1 of a thread
+    // are the two halves of 16 elements of row lrow + j*ROWS_PER_PASS and land, split, in tile rows
+    // lrow + 2j*ROWS_PER_PASS (high bytes) and lrow + (2j+1)*ROWS_PER_PASS (low bytes): runs of ROWS_PER_PASS tile
+    // rows alternate between the high and the low plane of the same ROWS_PER_PASS rows of A, and a wave's
+    // accumulator blocks i and i + ROWS_PER_PASS/32 (within each group of 2*ROWS_PER_PASS/32) belong together.
+    static constexpr int RBM = P::SPLIT_A ? BM / 2 : BM;  // rows of A (and of the output) per tile
+    static_assert(!P::SPLIT_A || (A_LOADS % 2 == 0 && ROWS_PER_PASS % 32 == 0 && WTM % (2 * ROWS_PER_PASS) == 0),
+                  "plane split: a wave's rows must hold whole high/low runs");
 };
 
 template <class P, int BM, int BN, int WAVES_M, int WAVES_N, bool EARLY = false>
@@ -160,7 +170,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 
     A4G_STAMP(0);
-    const TileCoord tc = tile_coord<BM, BN>(g);
+    const TileCoord tc = tile_coord<Cfg::RBM, BN>(g);
     if (!tc.valid) return;
     const int m0 = tc.m0, n0 = tc.n0;
 
@@ -173,8 +183,12 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
     const int8_t* __restrict__ Bbase = g.Bt + tc.batch * g.stride_b + static_cast<int64_t>(n0) * g.ldb;
     int offa[Cfg::A_LOADS], offb[Cfg::B_LOADS];  // 32-bit offsets from the tile's first row
 #pragma unroll
-    for (int i = 0; i < Cfg::A_LOADS; ++i)
-        offa[i] = min(lrow + i * Cfg::ROWS_PER_PASS, g.M - 1 - m0) * static_cast<int>(g.lda) + lchunk * 16;
+    for (int i = 0; i < Cfg::A_LOADS; ++i) {
+        if (P::SPLIT_A)
+            offa[i] = min(lrow + (i >> 1) * Cfg::ROWS_PER_PASS, g.M - 1 - m0) * static_cast<int>(g.lda) + lchunk * 32 + (i & 1) * 16;
+        else
+            offa[i] = min(lrow + i * Cfg::ROWS_PER_PASS, g.M - 1 - m0) * static_cast<int>(g.lda) + lchunk * 16;
+    }
 #pragma unroll
     for (int i = 0; i < Cfg::B_LOADS; ++i)
         offb[i] = min(lrow + i * Cfg::ROWS_PER_PASS, g.N - 1 - n0) * static_cast<int>(g.ldb) + lchunk * 16;
@@ -183,10 +197,13 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
 
     v4i ra[Cfg::A_LOADS], rb[Cfg::B_LOADS];
     auto load_one = [&](int kt, int idx) {
-        if (idx < Cfg::A_LOADS) ra[idx] = *reinterpret_cast<const v4i*>(Abase + offa[idx] + static_cast<int64_t>(kt) * BK);
+        if (idx < Cfg::A_LOADS) ra[idx] = *reinterpret_cast<const v4i*>(Abase + offa[idx] + static_cast<int64_t>(kt) * (P::SPLIT_A ? 2 * BK : BK));
         else rb[idx - Cfg::A_LOADS] = *reinterpret_cast<const v4i*>(Bbase + offb[idx - Cfg::A_LOADS] + static_cast<int64_t>(kt) * BK);
     };
     auto store_one = [&](int8_t* stage, int idx) {
+        if constexpr (P::SPLIT_A) {
+            if (idx < Cfg::A_LOADS && (idx & 1) == 0) P::split_a(ra[idx], ra[idx + 1 < Cfg::A_LOADS ? idx + 1 : idx]);
+        }
         if (idx < Cfg::A_LOADS) *reinterpret_cast<v4i*>(stage + st_off + idx * Cfg::ROWS_PER_PASS * BK) = ra[idx];
         else *reinterpret_cast<v4i*>(stage + BM * BK + st_off + (idx - Cfg::A_LOADS) * Cfg::ROWS_PER_PASS * BK) = rb[idx - Cfg::A_LOADS];
     };
@@ -312,10 +329,16 @@ static hipError_t launch_rs_policy(const GemmArgs& g, int batch, hipStream_t str
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    const int tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
+    const int tiles = ((g.M + Cfg::RBM - 1) / Cfg::RBM) * ((g.N + BN - 1) / BN);
     const int grid_x = (tiles + 7) / 8 * 8;
     hipLaunchKernelGGL(kern, dim3(grid_x, batch), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, g);
     return hipGetLastError();
 }
+
+// int16 activations x int8 weights on the pipelined kernel (defined beside the int8 policy, whose epilogue it
+// shares). g.A points at the int16 matrix, g.lda / g.stride_a are in bytes, g.K counts elements (K % 128 == 0),
+// g.colsum holds the column sums of the weights. False when the shape or the number of tiles does not suit it.
+bool rs_i16i8_applicable(const GemmArgs& g, int batch);
+hipError_t launch_rs_i16i8(const GemmArgs& g, int batch, hipStream_t stream);
 
 }  // namespace a4g

@@ -246,6 +246,33 @@ def test_dense_int16_activations(ops, oracle, shape):
     assert np.array_equal(got, oracle.dense(np.abs(A), np.abs(W), big, 16, 'conv_even', out='int16'))
 
 
+@pytest.mark.parametrize('shape', [(2085, 3000, 256), (4096, 1536, 384)])
+def test_dense_int16_activations_large(ops, oracle, shape):
+    """Problems with whole 128-element K tiles and at least 192 tiles of 128 x 256 take the software-pipelined kernel
+    that splits the activations into byte planes while staging them: ragged M and N, every rounding mode, the three
+    output kinds, rows at the int16 extremes, a bias that makes the 32-bit accumulator wrap."""
+    M, N, K = shape
+    r = rng(M + N + K)
+    A = r.integers(-32768, 32768, (M, K)).astype(np.int16)
+    A[0, :], A[1, :], A[-1, :] = 32767, -32768, -32768
+    A[2, ::2], A[2, 1::2] = 255, -256          # planes at their own extremes: low byte 0xff / 0x00
+    W = gauss8(r, 40, (K, N))
+    W[:, 0], W[:, 1] = 127, -128
+    bias = r.integers(-2**24, 2**24, N).astype(np.int32)
+    shifts = r.integers(10, 16, N).astype(np.int32)
+    p = ops.pack_dense(dev(W), dev(bias), shifts)
+    dA = dev(A)
+    for mode in MODES:
+        got = host(ops.dense(dA, p, mode, out_kind='int16'))
+        assert np.array_equal(got, oracle.dense(A, W, bias, shifts, mode, out='int16')), mode
+    for mode, relu, kind in (('symmetric_inf', True, 'int8'), ('floor', False, 'uint8')):
+        got = host(ops.dense(dA, p, mode, relu=relu, out_kind=kind))
+        assert np.array_equal(got, oracle.dense(A, W, bias, shifts, mode, relu=relu, out=kind)), (mode, kind)
+    big = np.full(N, 2**31 - 77, dtype=np.int32)
+    got = host(ops.dense(dev(np.abs(A)), ops.pack_dense(dev(np.abs(W)), dev(big), 16), 'conv_even', out_kind='int16'))
+    assert np.array_equal(got, oracle.dense(np.abs(A), np.abs(W), big, 16, 'conv_even', out='int16'))
+
+
 MODES8 = ('floor', 'ceil', 'positive_inf', 'negative_inf', 'symmetric_inf', 'symmetric_zero', 'conv_even', 'conv_odd')
 
 
@@ -275,7 +302,8 @@ def test_dense_int16_activations_int16_weights(ops, oracle, shape):
 
 @pytest.mark.parametrize('b_dtype', [np.int8, np.int16])
 @pytest.mark.parametrize('trans_b', [True, False])
-@pytest.mark.parametrize('shape', [((2, 3), 64, 64, 64), ((4,), 130, 96, 48), ((), 70, 17, 24), ((2,), 128, 256, 512)])
+@pytest.mark.parametrize('shape', [((2, 3), 64, 64, 64), ((4,), 130, 96, 48), ((), 70, 17, 24), ((2,), 128, 256, 512),
+                                   ((3,), 1100, 2000, 256)])
 def test_matmul_int16_left_operand(ops, oracle, shape, trans_b, b_dtype):
     # the 16-bit width combinations of the dynamic MatMul: int16 x int8 (acc32) and int16 x int16 (acc64)
     lead, M, N, K = shape
