@@ -397,7 +397,8 @@ struct I8Policy {
     using acc_t = v16i;
     static constexpr int MMAS = 1;
     static constexpr bool FIX_A = A_UNSIGNED;
-    static constexpr bool SPLIT_A = false;
+    static constexpr bool SPLIT_A = false, SPLIT_B = false;
+    struct Extra {};
     static constexpr int MAX_OUT_BYTES = 2;
     template <int BN>
     static constexpr int param_bytes() { return ColParams<BN>::BYTES; }
@@ -419,7 +420,7 @@ struct I8Policy {
     template <int BM, int BN, int WTM, int WTN, int NT>
     __device__ static __forceinline__ void epilogue(const GemmArgs& g, const TileCoord& tc, v16i (&acc)[WTM / 32][WTN / 32],
                                                     int8_t* smem, int8_t* lds_params, int path, int wm, int wn, int lane,
-                                                    int tid) {
+                                                    int tid, Extra&) {
         epilogue_store<BM, BN, WTM, WTN, NT>(g, tc, acc, smem, ColParams<BN>(lds_params), path, wm, wn, lane, tid);
     }
 };
@@ -431,7 +432,7 @@ struct I8Policy {
 // bias as it does for an unsigned operand. Wrapping 32-bit arithmetic throughout, as acc32 does.
 struct I16Policy : I8Policy<false> {
     static constexpr bool SPLIT_A = true;
-    __device__ static __forceinline__ void split_a(v4i& x, v4i& y) {
+    __device__ static __forceinline__ void split_a(v4i& x, v4i& y, Extra&, int, bool) {
         v4i hi, lo;
         hi[0] = static_cast<int>(__builtin_amdgcn_perm(x[1], x[0], 0x07050301u));
         hi[1] = static_cast<int>(__builtin_amdgcn_perm(x[3], x[2], 0x07050301u));
@@ -451,7 +452,7 @@ struct I16Policy : I8Policy<false> {
     template <int BM, int BN, int WTM, int WTN, int NT>
     __device__ static __forceinline__ void epilogue(const GemmArgs& g, const TileCoord& tc, v16i (&acc)[WTM / 32][WTN / 32],
                                                     int8_t* smem, int8_t* lds_params, int path, int wm, int wn, int lane,
-                                                    int tid) {
+                                                    int tid, Extra&) {
         constexpr int PB = NT / 256;  // 32-row blocks per run of one plane (rows covered by one load per thread / 32)
         v16i sum[WTM / 64][WTN / 32];
 #pragma unroll

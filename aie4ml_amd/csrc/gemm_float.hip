@@ -65,7 +65,8 @@ struct FloatPolicy {
     static constexpr int ES = FMT == A4G_F32 ? 4 : (FMT == A4G_FP8 ? 1 : 2);
     static constexpr int MMAS = FMT == A4G_F32 ? 4 : (FMT == A4G_FP8 ? 2 : 1);
     static constexpr bool FIX_A = false;
-    static constexpr bool SPLIT_A = false;
+    static constexpr bool SPLIT_A = false, SPLIT_B = false;
+    struct Extra {};
     static constexpr int MAX_OUT_BYTES = ES;
     template <int BN>
     static constexpr int param_bytes() { return 4 * BN; }
@@ -102,7 +103,8 @@ struct FloatPolicy {
     // acc + bias -> ReLU -> operand format, through an LDS image of the tile, then whole-row stores
     template <int BM, int BN, int WTM, int WTN, int NT>
     __device__ static __forceinline__ void epilogue(const GemmArgs& g, const TileCoord& tc, v16f (&acc)[WTM / 32][WTN / 32],
-                                                    int8_t* smem, int8_t* lds_params, int, int wm, int wn, int lane, int tid) {
+                                                    int8_t* smem, int8_t* lds_params, int, int wm, int wn, int lane, int tid,
+                                                    Extra&) {
         constexpr int TM = WTM / 32, TN = WTN / 32;
         constexpr int cpitch = BN * ES + 16;
         const float* bias = reinterpret_cast<const float*>(lds_params);

@@ -229,6 +229,132 @@ __device__ __forceinline__ int requant64(long long v, int s, int mode, int lo, i
     return static_cast<int>(y < lo ? lo : (y > hi ? hi : y));
 }
 
+// int16 x int16 on the software-pipelined kernel (K % 128 == 0, large problems). Both operands enter the tile as
+// byte planes: the activations are split while they are staged (runs of 64 tile rows alternate between the high
+// and the low plane of the same 64 rows), the weights come packed as two planes that alternate in 32-row blocks.
+// A wave's 128 x 64 accumulator blocks are then, for each of its two 32-row blocks of outputs, the four partial
+// products hh, hl, lh, ll of the same 32 x 32 outputs in the same lanes and registers. With the low planes
+// biased by 128, sum a*w = 65536 hh + 256 (hl + lh) + ll + 128 sum_k a + 128 sum_k (w - 128): the column term
+// comes with the packed weights, the row term is accumulated from the raw activations as they are split.
+struct I16x16Policy {
+    using acc_t = v16i;
+    static constexpr int MMAS = 1;
+    static constexpr bool FIX_A = false, SPLIT_A = true, SPLIT_B = true;
+    static constexpr int MAX_OUT_BYTES = 1;  // the output image holds 128 x 128 two-byte elements in a 256 x 256 one-byte frame
+    static constexpr int MAX_ROWS = 128;
+    struct Extra {
+        int row_sum[2];  // sum over k of the activations of rows lrow and lrow + 64, this thread's 16 columns per K tile
+    };
+    struct ColRegs {
+        int bias, colsum, shift;
+    };
+    struct Params {  // LDS: per output column of the tile, then per output row
+        long long col_term[128];
+        int shift[128];
+        int row_sum[MAX_ROWS];
+    };
+    template <int BN>
+    static constexpr int param_bytes() { return sizeof(Params); }
+    __device__ static __forceinline__ void fix_a(v4i&) {}
+    __device__ static __forceinline__ v16i mma(const v4i& b, const v4i& a, const v16i& c) {
+        return __builtin_amdgcn_mfma_i32_32x32x32_i8(b, a, c, 0, 0, 0);
+    }
+    __device__ static __forceinline__ void split_a(v4i& x, v4i& y, Extra& e, int pair, bool live) {
+        typedef short s2 __attribute__((ext_vector_type(2)));
+        const s2 ones = live ? s2{1, 1} : s2{0, 0};
+        int sum = 0;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int xt = x[t], yt = y[t];  // copies: a bit cast applied to the vector element itself reads element 0
+            sum = __builtin_amdgcn_sdot2(__builtin_bit_cast(s2, xt), ones, sum, false);
+            sum = __builtin_amdgcn_sdot2(__builtin_bit_cast(s2, yt), ones, sum, false);
+        }
+        e.row_sum[pair] += sum;
+        v4i hi, lo;
+        hi[0] = static_cast<int>(__builtin_amdgcn_perm(x[1], x[0], 0x07050301u));
+        hi[1] = static_cast<int>(__builtin_amdgcn_perm(x[3], x[2], 0x07050301u));
+        hi[2] = static_cast<int>(__builtin_amdgcn_perm(y[1], y[0], 0x07050301u));
+        hi[3] = static_cast<int>(__builtin_amdgcn_perm(y[3], y[2], 0x07050301u));
+        lo[0] = static_cast<int>(__builtin_amdgcn_perm(x[1], x[0], 0x06040200u) ^ 0x80808080u);
+        lo[1] = static_cast<int>(__builtin_amdgcn_perm(x[3], x[2], 0x06040200u) ^ 0x80808080u);
+        lo[2] = static_cast<int>(__builtin_amdgcn_perm(y[1], y[0], 0x06040200u) ^ 0x80808080u);
+        lo[3] = static_cast<int>(__builtin_amdgcn_perm(y[3], y[2], 0x06040200u) ^ 0x80808080u);
+        x = hi;
+        y = lo;
+    }
+    template <int BN>
+    __device__ static __forceinline__ void fetch_params(const GemmArgs& g, const TileCoord& tc, int tid, ColRegs& r) {
+        r.bias = r.colsum = r.shift = 0;
+        if (tid < BN / 2) {
+            const int nn = min(tc.n0 + tid, g.N - 1);
+            r.bias = g.bias ? g.bias[nn] : 0;
+            r.colsum = g.colsum[tc.batch * g.stride_colsum + nn];
+            r.shift = g.shifts ? g.shifts[static_cast<int64_t>(nn) * g.shift_stride] : g.shift;
+        }
+    }
+    template <int BN>
+    __device__ static __forceinline__ int park_params(const GemmArgs&, int8_t* lds, int tid, const ColRegs& r) {
+        Params* p = reinterpret_cast<Params*>(lds);
+        if (tid < BN / 2) {
+            p->col_term[tid] = 128ll * r.colsum + r.bias;
+            p->shift[tid] = min(max(r.shift, 0), 62);
+        }
+        return 0;
+    }
+    template <int BM, int BN, int WTM, int WTN, int NT>
+    __device__ static __forceinline__ void epilogue(const GemmArgs& g, const TileCoord& tc, v16i (&acc)[WTM / 32][WTN / 32],
+                                                    int8_t* smem, int8_t* lds_params, int, int wm, int wn, int lane, int tid,
+                                                    Extra& e) {
+        static_assert(BM == 256 && BN == 256 && WTM == 128 && WTN == 64 && NT == 512, "written for the 256 x 256 tile of 8 waves");
+        Params* p = reinterpret_cast<Params*>(lds_params);
+        // the eight threads that staged one row (consecutive lanes) add up their shares of its sum
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            int v = e.row_sum[j];
+            v += __shfl_xor(v, 1);
+            v += __shfl_xor(v, 2);
+            v += __shfl_xor(v, 4);
+            if ((tid & 7) == 0) p->row_sum[(tid >> 3) + 64 * j] = v;
+        }
+        __syncthreads();
+        const int lo_b = g.relu ? max(kind_lo(g.out_kind), 0) : kind_lo(g.out_kind), hi_b = kind_hi(g.out_kind);
+        const int obytes = (g.out_kind == A4G_I16 || g.out_kind == A4G_U16) ? 2 : 1;
+        const int cpitch = 128 * obytes + 16;
+#pragma unroll
+        for (int ri = 0; ri < 2; ++ri) {
+            const int ml = wm * 64 + ri * 32 + (lane & 31);  // output row within the tile
+            const long long row_term = 128ll * p->row_sum[ml];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int nl = wn * 32 + 8 * q + 4 * (lane >> 5);
+                int y[4];
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const int r = 4 * q + t;
+                    const long long v = (static_cast<long long>(acc[ri][0][r]) << 16) +
+                                        ((static_cast<long long>(acc[ri][1][r]) + acc[ri + 2][0][r]) << 8) + acc[ri + 2][1][r] +
+                                        row_term + p->col_term[nl + t];
+                    y[t] = requant64(v, p->shift[nl + t], g.mode, lo_b, hi_b);
+                }
+                if (obytes == 1) {
+                    *reinterpret_cast<unsigned*>(smem + ml * cpitch + nl) = pack4_bytes(y[0], y[1], y[2], y[3]);
+                } else {
+                    v2i o = {static_cast<int>(pack2_halves(y[0], y[1])), static_cast<int>(pack2_halves(y[2], y[3]))};
+                    *reinterpret_cast<v2i*>(smem + ml * cpitch + nl * 2) = o;
+                }
+            }
+        }
+        __syncthreads();
+        store_tile_image<128, 128, NT>(g, tc, smem, obytes, tid);
+    }
+};
+
+static bool rs_i16i16_applicable(const GemmArgs& g, int batch) {
+    return g.K % 128 == 0 && g.K >= 256 && g.K <= 32768 && g.lda % 16 == 0 && g.stride_a % 16 == 0 && g.ldb % 16 == 0 &&
+           g.stride_b % 16 == 0 && aligned16(g.A) && aligned16(g.Bt) && aligned16(g.Bt_lo) &&
+           static_cast<int64_t>((g.M + 127) / 128) * ((g.N + 127) / 128) * batch >= 192;
+}
+
 // 64 x 128 output tile, K step 64, 4 waves (2 x 2) of 32 x 64, double-buffered LDS with the two byte planes
 // of both operands. Requires K % 16 == 0, 16-byte aligned rows.
 __device__ __forceinline__ void select_problem(Gemm16x16Args& g, int b) {
@@ -529,6 +655,16 @@ extern "C" int a4g_dense_i16x16(const int16_t* A, int64_t lda, const int8_t* Wt_
     g.relu = relu != 0;
     g.out_kind = out_kind;
     g.mode = round_mode;
+    {
+        GemmArgs r{};
+        r.A = reinterpret_cast<const int8_t*>(A); r.Bt = Wt_hi; r.Bt_lo = Wt_lo; r.C = Y; r.bias = bias; r.colsum = colsum;
+        r.shifts = shifts;
+        r.lda = lda * 2; r.ldb = ldwt; r.ldc = ldy;
+        r.M = g.M; r.N = g.N; r.K = g.K;
+        r.shift_stride = g.shift_stride; r.relu = g.relu; r.out_kind = out_kind; r.mode = round_mode;
+        if (rs_i16i16_applicable(r, 1))
+            return check_hip(launch_rs_policy<I16x16Policy, 256, 256, 2, 4, true>(r, 1, stream), who);
+    }
     const bool tiled = K % 16 == 0 && lda % 8 == 0 && ldwt % 16 == 0 && aligned16(A) && aligned16(Wt_hi) && aligned16(Wt_lo);
     if (tiled) {
         const int64_t tiles = ((M + 63) / 64) * ((N + 127) / 128);
@@ -593,6 +729,14 @@ extern "C" int a4g_matmul_i16(const int16_t* A, int64_t lda, int64_t stride_a, c
         g.M = (int)M; g.N = (int)N; g.K = (int)K;
         g.out_kind = out_kind; g.mode = round_mode; g.shift = shift;
         g.stride_a = stride_a; g.stride_w = N * ldt; g.stride_colsum = N; g.stride_y = stride_c;
+        GemmArgs r{};
+        r.A = reinterpret_cast<const int8_t*>(A); r.Bt = hi; r.Bt_lo = lo; r.C = C; r.colsum = colsum;
+        r.lda = lda * 2; r.stride_a = stride_a * 2; r.ldb = ldt; r.stride_b = N * ldt; r.ldc = ldc; r.stride_c = stride_c;
+        r.stride_colsum = N;
+        r.M = g.M; r.N = g.N; r.K = g.K;
+        r.shift = shift; r.out_kind = out_kind; r.mode = round_mode;
+        if (rs_i16i16_applicable(r, nb))
+            return check_hip(launch_rs_policy<I16x16Policy, 256, 256, 2, 4, true>(r, nb, stream), who);
         if (tiled) {
             const int64_t tiles = ((M + 63) / 64) * ((N + 127) / 128);
             gemm_i16i16_kernel<<<dim3(static_cast<unsigned>((tiles + 7) / 8 * 8), nb), 256, 0, stream>>>(g);

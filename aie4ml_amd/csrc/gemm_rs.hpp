@@ -7,8 +7,11 @@
 //   FIX_A, fix_a(v4i&)           optional fix-up of an A fragment before use
 //   mma(b, a, acc)               acc += the 32 x 32 block product of two fragments
 //   MAX_OUT_BYTES                widest output element (sizes the LDS image of the output tile)
-//   SPLIT_A / split_a(x, y)      A elements are two bytes wide: a thread loads 16 of them as two registers and
+//   SPLIT_A / split_a(x, y, extra, pair, live)
+//                                A elements are two bytes wide: a thread loads 16 of them as two registers and
 //                                turns them into their 16 high and 16 low bytes, which become two tile rows
+//   SPLIT_B                      B^T comes as two byte planes (Bt, Bt_lo) that alternate in 32-row blocks of the tile
+//   Extra                        per-thread state the policy carries from the staging to the epilogue
 //   param_bytes<BN>()            LDS bytes of the per-column epilogue parameters
 //   ColRegs, fetch_params<BN>, park_params<BN>   issue the loads of a thread's column parameters early,
 //                                store them to LDS later (park_params contains a barrier and returns a
@@ -55,6 +58,7 @@ struct GemmArgs {
     int relu;
     int out_kind;
     int mode;
+    const int8_t* Bt_lo;    // second byte plane of B^T (policies with SPLIT_B), same pitch and strides as Bt
 };
 
 struct TileCoord {
@@ -154,6 +158,8 @@ struct RsCfg {
     // rows alternate between the high and the low plane of the same ROWS_PER_PASS rows of A, and a wave's
     // accumulator blocks i and i + ROWS_PER_PASS/32 (within each group of 2*ROWS_PER_PASS/32) belong together.
     static constexpr int RBM = P::SPLIT_A ? BM / 2 : BM;  // rows of A (and of the output) per tile
+    static constexpr int RBN = P::SPLIT_B ? BN / 2 : BN;  // columns of the output per tile
+    static_assert(!P::SPLIT_B || ROWS_PER_PASS == 64, "B planes alternate in 32-row blocks: 64 tile rows per pass");
     static_assert(!P::SPLIT_A || (A_LOADS % 2 == 0 && ROWS_PER_PASS % 32 == 0 && WTM % (2 * ROWS_PER_PASS) == 0),
                   "plane split: a wave's rows must hold whole high/low runs");
 };
@@ -170,17 +176,19 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
 
     A4G_STAMP(0);
-    const TileCoord tc = tile_coord<Cfg::RBM, BN>(g);
+    const TileCoord tc = tile_coord<Cfg::RBM, Cfg::RBN>(g);
     if (!tc.valid) return;
     const int m0 = tc.m0, n0 = tc.n0;
 
     typename P::ColRegs col_regs;  // this thread's column parameters, in flight until they are parked
+    typename P::Extra extra{};
+    bool split_live = true;  // false while the staging registers hold a repeat of the last K tile
     P::template fetch_params<BN>(g, tc, tid, col_regs);
 
     // ---- global -> register staging: thread t owns chunk t%8 of rows t/8 + pass*ROWS_PER_PASS
     const int lrow = tid / Cfg::CPR, lchunk = tid % Cfg::CPR;
     const int8_t* __restrict__ Abase = g.A + tc.batch * g.stride_a + static_cast<int64_t>(m0) * g.lda;
-    const int8_t* __restrict__ Bbase = g.Bt + tc.batch * g.stride_b + static_cast<int64_t>(n0) * g.ldb;
+    const int8_t* __restrict__ Bbase = ((P::SPLIT_B && (lrow & 32)) ? g.Bt_lo : g.Bt) + tc.batch * g.stride_b + static_cast<int64_t>(n0) * g.ldb;
     int offa[Cfg::A_LOADS], offb[Cfg::B_LOADS];  // 32-bit offsets from the tile's first row
 #pragma unroll
     for (int i = 0; i < Cfg::A_LOADS; ++i) {
@@ -190,8 +198,11 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
             offa[i] = min(lrow + i * Cfg::ROWS_PER_PASS, g.M - 1 - m0) * static_cast<int>(g.lda) + lchunk * 16;
     }
 #pragma unroll
-    for (int i = 0; i < Cfg::B_LOADS; ++i)
-        offb[i] = min(lrow + i * Cfg::ROWS_PER_PASS, g.N - 1 - n0) * static_cast<int>(g.ldb) + lchunk * 16;
+    for (int i = 0; i < Cfg::B_LOADS; ++i) {
+        // SPLIT_B: tile rows [64i, 64i + 32) are the first plane of columns [32i, 32i + 32), the next 32 the second
+        const int brow = P::SPLIT_B ? i * 32 + (lrow & 31) : lrow + i * Cfg::ROWS_PER_PASS;
+        offb[i] = min(brow, g.N - 1 - n0) * static_cast<int>(g.ldb) + lchunk * 16;
+    }
     // LDS slot of that chunk; the swizzle term (row>>1)&7 is the same for every pass
     const int st_off = lrow * BK + ((lchunk ^ ((lrow >> 1) & 7)) * 16);
 
@@ -202,7 +213,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
     };
     auto store_one = [&](int8_t* stage, int idx) {
         if constexpr (P::SPLIT_A) {
-            if (idx < Cfg::A_LOADS && (idx & 1) == 0) P::split_a(ra[idx], ra[idx + 1 < Cfg::A_LOADS ? idx + 1 : idx]);
+            if (idx < Cfg::A_LOADS && (idx & 1) == 0)
+                P::split_a(ra[idx], ra[idx + 1 < Cfg::A_LOADS ? idx + 1 : idx], extra, idx >> 1, split_live);
         }
         if (idx < Cfg::A_LOADS) *reinterpret_cast<v4i*>(stage + st_off + idx * Cfg::ROWS_PER_PASS * BK) = ra[idx];
         else *reinterpret_cast<v4i*>(stage + BM * BK + st_off + (idx - Cfg::A_LOADS) * Cfg::ROWS_PER_PASS * BK) = rb[idx - Cfg::A_LOADS];
@@ -292,6 +304,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
     for (int kt = 0; kt < ktiles; ++kt) {
         int8_t* cur_base = smem + (kt & 1) * Cfg::STAGE_BYTES;
         int8_t* nxt_base = smem + ((kt + 1) & 1) * Cfg::STAGE_BYTES;
+        split_live = kt + 1 < ktiles;
         if (EARLY) {
             step(0, 1, cur_base, 1, Tag3{}, nxt_base, min(kt + 2, ktiles - 1));
             __builtin_amdgcn_sched_barrier(0);
@@ -313,7 +326,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
     __syncthreads();  // every wave is past its last fragment read before the stages become the output image
     A4G_STAMP(3);
 
-    P::template epilogue<BM, BN, Cfg::WTM, Cfg::WTN, Cfg::NT>(g, tc, acc, smem, smem + Cfg::PARAM_OFF, epi_path, wm, wn, lane, tid);
+    P::template epilogue<BM, BN, Cfg::WTM, Cfg::WTN, Cfg::NT>(g, tc, acc, smem, smem + Cfg::PARAM_OFF, epi_path, wm, wn, lane, tid, extra);
     A4G_STAMP(5);
 }
 
@@ -329,7 +342,7 @@ static hipError_t launch_rs_policy(const GemmArgs& g, int batch, hipStream_t str
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    const int tiles = ((g.M + Cfg::RBM - 1) / Cfg::RBM) * ((g.N + BN - 1) / BN);
+    const int tiles = ((g.M + Cfg::RBM - 1) / Cfg::RBM) * ((g.N + Cfg::RBN - 1) / Cfg::RBN);
     const int grid_x = (tiles + 7) / 8 * 8;
     hipLaunchKernelGGL(kern, dim3(grid_x, batch), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, g);
     return hipGetLastError();

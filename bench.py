@@ -6,7 +6,7 @@ Default workload: the single quantized Dense of the baseline configuration
 saturate to int8, fused ReLU). One step = one pass of the operator over the whole synthetic batch,
 inputs already resident in HBM. Prints ONE JSON line.
 
-Other workloads (--workload c2_dense_i16 | c2_dense_bf16 | c2_dense_fp8 | c1_mlp | c3_softmax_exp | c3_softmax_hccs | c3_qk | c3_pv |
+Other workloads (--workload c2_dense_i16 | c2_dense_i16x16 | c2_dense_bf16 | c2_dense_fp8 | c1_mlp | c3_softmax_exp | c3_softmax_hccs | c3_qk | c3_pv |
 c3_attention_exp | c3_attention_hccs | c4_add_layernorm | c4_layernorm | c4_add | c5_encoder) print the same line for that operator or graph;
 --workload calib_copy runs a plain 256 MiB elementwise copy, the known-size kernel the HBM traffic
 counters are scaled against.
@@ -173,7 +173,34 @@ def main():
         cpu_fn = lambda: oracle.dense(A[:sample_rows], W, bias, shifts, 'conv_even', relu=True, out='int16')  # noqa: E731
         cpu_work = 2.0 * sample_rows * N * K
         metric, unit = 'int16x8_dense_tops', 'TOP/s'
-        kernel = 'gemm_i16i8_kernel'
+        kernel = 'gemm_rs_kernel'
+    elif wl == 'c2_dense_i16x16':
+        # the (16, 16) width combination on the C2 shape: int16 activations and weights, 64-bit accumulator, int16 output
+        M, K, N = 8192, 4096, 4096
+        r = np.random.default_rng(29)
+        A = r.integers(-32768, 32768, (M, K)).astype(np.int16)
+        W = r.integers(-32768, 32768, (K, N)).astype(np.int16)
+        bias = r.integers(-2**30, 2**30, N).astype(np.int32)
+        shifts = r.integers(25, 29, N).astype(np.int32)
+        p = ops.pack_dense(dev(W), dev(bias), shifts)
+        dA = dev(A)
+        out = torch.empty((M, N), dtype=torch.int16, device='cuda')
+        fn = lambda: ops.dense(dA, p, 'conv_even', relu=True, out_kind='int16', out=out)  # noqa: E731
+        fn()
+        rows = np.random.default_rng(0).choice(M, 64, replace=False)
+        exp = oracle.dense(A[rows], W, bias, shifts, 'conv_even', relu=True, out='int16')
+        torch.cuda.synchronize()
+        bit_exact = bool(np.array_equal(out[torch.from_numpy(rows).cuda()].cpu().numpy(), exp))
+        work, bound = 2.0 * M * N * K, 'mfma'
+        samples = M
+        config = {'workload': 'c2_dense_i16x16: Dense 8192x4096 -> 4096, int16 activations x int16 weights (acc64), bias, '
+                              'per-channel shift, conv_even, sat int16, ReLU'}
+        sample_rows = 256
+        cpu_desc = f'oracle Dense (int16 x int16) on the first {sample_rows} of {M} rows, scaled per op'
+        cpu_fn = lambda: oracle.dense(A[:sample_rows], W, bias, shifts, 'conv_even', relu=True, out='int16')  # noqa: E731
+        cpu_work = 2.0 * sample_rows * N * K
+        metric, unit = 'int16x16_dense_tops', 'TOP/s'
+        kernel = 'gemm_i16i16_kernel'
     elif wl in ('c2_dense_bf16', 'c2_dense_fp8'):
         # the reference's float compute path on the C2 shape: bfloat16 / fp8 e4m3 operands, float32 accumulation and bias
         M, K, N = 8192, 4096, 4096
@@ -439,7 +466,7 @@ def main():
     line = {
         'metric': metric, 'value': float(f'{value:.6g}'), 'unit': unit, 'n_gpus': 1, 'steps': args.steps,
         'warmup': args.warmup, 'ms_per_step': round(ms, 5), 'higher_is_better': True, 'scaling': 'weak',
-        'vs_baseline': None, 'dtype': {'c2_dense_i16': 'int16', 'c2_dense_bf16': 'bf16', 'c2_dense_fp8': 'fp8'}.get(wl, 'int8'), 'data': 'synthetic', 'config': config,
+        'vs_baseline': None, 'dtype': {'c2_dense_i16': 'int16', 'c2_dense_i16x16': 'int16', 'c2_dense_bf16': 'bf16', 'c2_dense_fp8': 'fp8'}.get(wl, 'int8'), 'data': 'synthetic', 'config': config,
         'samples_per_s': float(f'{samples / (ms * 1e-3):.6g}'), 'bit_exact': bit_exact,
         'roofline': roof, 'cpu_baseline': cpu, 'launch': 'hip_graph' if graphed else 'eager',
     }

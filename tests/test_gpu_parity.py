@@ -300,6 +300,34 @@ def test_dense_int16_activations_int16_weights(ops, oracle, shape):
         ops.dense(dev(A.astype(np.int8)), p, 'floor')
 
 
+@pytest.mark.parametrize('shape', [(2085, 3000, 256), (1024, 3072, 640)])
+def test_dense_int16x16_large(ops, oracle, shape):
+    """int16 x int16 problems with whole 128-element K tiles and at least 192 output tiles of 128 x 128 take the
+    software-pipelined kernel (both operands as byte planes in one tile, row sums gathered while the activations
+    are split): ragged edges, every rounding mode, extreme rows and columns, all three output kinds."""
+    M, N, K = shape
+    r = rng(M + N + K)
+    A = r.integers(-32768, 32768, (M, K)).astype(np.int16)
+    W = r.integers(-32768, 32768, (K, N)).astype(np.int16)
+    A[0, :], A[1, :], A[-1, :] = -32768, 32767, -32768
+    A[2, ::2], A[2, 1::2] = 255, -256
+    W[:, 0], W[:, 1], W[:, -1] = -32768, 32767, -32768
+    W[::2, 2], W[1::2, 2] = 255, -256
+    bias = r.integers(-2**31, 2**31, N).astype(np.int32)
+    shifts = r.integers(14, 32, N).astype(np.int32)
+    p = ops.pack_dense(dev(W), dev(bias), shifts)
+    dA = dev(A)
+    for mode in MODES:
+        got = host(ops.dense(dA, p, mode, out_kind='int16'))
+        assert np.array_equal(got, oracle.dense(A, W, bias, shifts, mode, out='int16')), mode
+    for mode, relu, kind in (('symmetric_inf', True, 'int8'), ('floor', False, 'uint8')):
+        got = host(ops.dense(dA, p, mode, relu=relu, out_kind=kind))
+        assert np.array_equal(got, oracle.dense(A, W, bias, shifts, mode, relu=relu, out=kind)), (mode, kind)
+    p2 = ops.pack_dense(dev(W), None, 40)
+    assert np.array_equal(host(ops.dense(dA, p2, 'conv_even', relu=True, out_kind='int8')),
+                          oracle.dense(A, W, None, 40, 'conv_even', relu=True, out='int8'))
+
+
 @pytest.mark.parametrize('b_dtype', [np.int8, np.int16])
 @pytest.mark.parametrize('trans_b', [True, False])
 @pytest.mark.parametrize('shape', [((2, 3), 64, 64, 64), ((4,), 130, 96, 48), ((), 70, 17, 24), ((2,), 128, 256, 512),
