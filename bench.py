@@ -35,10 +35,11 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
 # WRITE_SIZE, one counter run each, scaled by what the same counter reads for calib_copy).
 # None = not measured.
 MEASURED_TRAFFIC = {
-    'c2_dense': 227803374, 'c1_mlp': 166940, 'c4_add': 49059234, 'c4_layernorm': 33024803,
-    'c4_add_layernorm': 49179488, 'c3_softmax_exp': 263310672, 'c3_softmax_hccs': 263310853,
-    'c3_qk': 182762264, 'c3_pv': 210430349, 'c3_attention_exp': 128707683, 'c3_attention_hccs': 128709239,
-    'calib_copy': 536870912, 'c2_dense_i16': 713173641, 'c2_dense_bf16': 454954067, 'c2_dense_fp8': 227923232,
+    'c2_dense': 227826201, 'c1_mlp': 166940, 'c4_add': 49063352, 'c4_layernorm': 33052160,
+    'c4_add_layernorm': 49190223, 'c3_softmax_exp': 263311379, 'c3_softmax_hccs': 263311577,
+    'c3_qk': 182768882, 'c3_pv': 210431233, 'c3_attention_exp': 118082676, 'c3_attention_hccs': 118082322,
+    'calib_copy': 536870912, 'c2_dense_i16': 454852713, 'c2_dense_i16x16': 842205840, 'c2_dense_bf16': 454925551,
+    'c2_dense_fp8': 227911206,
 }
 
 
