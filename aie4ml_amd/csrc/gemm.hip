@@ -395,7 +395,7 @@ __device__ __forceinline__ void epilogue_store(const GemmArgs& g, const TileCoor
 template <bool A_UNSIGNED>
 struct I8Policy {
     using acc_t = v16i;
-    static constexpr int MMAS = 1;
+    static constexpr int MMAS = 1, KSTEP_BYTES = 32;
     static constexpr bool FIX_A = A_UNSIGNED;
     static constexpr bool SPLIT_A = false, SPLIT_B = false;
     struct Extra {};
@@ -406,8 +406,8 @@ struct I8Policy {
         int add, shift;
     };
     __device__ static __forceinline__ void fix_a(v4i& a) { a ^= static_cast<int>(0x80808080u); }
-    __device__ static __forceinline__ v16i mma(const v4i& b, const v4i& a, const v16i& c) {
-        return __builtin_amdgcn_mfma_i32_32x32x32_i8(b, a, c, 0, 0, 0);
+    __device__ static __forceinline__ v16i mma(const v4i (&b)[1], const v4i (&a)[1], const v16i& c) {
+        return __builtin_amdgcn_mfma_i32_32x32x32_i8(b[0], a[0], c, 0, 0, 0);
     }
     template <int BN>
     __device__ static __forceinline__ void fetch_params(const GemmArgs& g, const TileCoord& tc, int tid, ColRegs& r) {

@@ -63,7 +63,9 @@ template <int FMT>
 struct FloatPolicy {
     using acc_t = v16f;
     static constexpr int ES = FMT == A4G_F32 ? 4 : (FMT == A4G_FP8 ? 1 : 2);
-    static constexpr int MMAS = FMT == A4G_F32 ? 4 : (FMT == A4G_FP8 ? 2 : 1);
+    // fp8 takes the 64-wide instruction (two 16-byte fragments per lane and operand), the others 32 bytes of K per call
+    static constexpr int KSTEP_BYTES = FMT == A4G_FP8 ? 64 : 32;
+    static constexpr int MMAS = FMT == A4G_F32 ? 4 : 1;
     static constexpr bool FIX_A = false;
     static constexpr bool SPLIT_A = false, SPLIT_B = false;
     struct Extra {};
@@ -74,20 +76,22 @@ struct FloatPolicy {
         float bias;
     };
     __device__ static __forceinline__ void fix_a(v4i&) {}
-    __device__ static __forceinline__ v16f mma(const v4i& b, const v4i& a, v16f c) {
-        if (FMT == A4G_F32) {
-            const v4f bf = __builtin_bit_cast(v4f, b), af = __builtin_bit_cast(v4f, a);
+    __device__ static __forceinline__ v16f mma(const v4i (&b)[KSTEP_BYTES / 32], const v4i (&a)[KSTEP_BYTES / 32], v16f c) {
+        if constexpr (FMT == A4G_F32) {
+            const v4f bf = __builtin_bit_cast(v4f, b[0]), af = __builtin_bit_cast(v4f, a[0]);
 #pragma unroll
             for (int t = 0; t < 4; ++t) c = __builtin_amdgcn_mfma_f32_32x32x2f32(bf[t], af[t], c, 0, 0, 0);
             return c;
+        } else if constexpr (FMT == A4G_FP8) {
+            // v_mfma_f32_32x32x64_f8f6f4 with both operands fp8 e4m3 (format codes 0) and no block scaling: a lane
+            // supplies 32 bytes of K per operand; which 32 is immaterial as long as both operands agree
+            typedef int v8i __attribute__((ext_vector_type(8)));
+            const v8i bw = {b[0][0], b[0][1], b[0][2], b[0][3], b[1][0], b[1][1], b[1][2], b[1][3]};
+            const v8i aw = {a[0][0], a[0][1], a[0][2], a[0][3], a[1][0], a[1][1], a[1][2], a[1][3]};
+            return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(bw, aw, c, 0, 0, 0, 0, 0, 0);
+        } else {
+            return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, b[0]), __builtin_bit_cast(v8bf, a[0]), c, 0, 0, 0);
         }
-        if (FMT == A4G_FP8) {
-            typedef long v2l __attribute__((ext_vector_type(2)));
-            const v2l bl = __builtin_bit_cast(v2l, b), al = __builtin_bit_cast(v2l, a);
-            c = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(bl[0], al[0], c, 0, 0, 0);
-            return __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(bl[1], al[1], c, 0, 0, 0);
-        }
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, b), __builtin_bit_cast(v8bf, a), c, 0, 0, 0);
     }
     template <int BN>
     __device__ static __forceinline__ void fetch_params(const GemmArgs& g, const TileCoord& tc, int tid, ColRegs& r) {

@@ -238,7 +238,7 @@ __device__ __forceinline__ int requant64(long long v, int s, int mode, int lo, i
 // comes with the packed weights, the row term is accumulated from the raw activations as they are split.
 struct I16x16Policy {
     using acc_t = v16i;
-    static constexpr int MMAS = 1;
+    static constexpr int MMAS = 1, KSTEP_BYTES = 32;
     static constexpr bool FIX_A = false, SPLIT_A = true, SPLIT_B = true;
     static constexpr int MAX_OUT_BYTES = 1;  // the output image holds 128 x 128 two-byte elements in a 256 x 256 one-byte frame
     static constexpr int MAX_ROWS = 128;
@@ -256,8 +256,8 @@ struct I16x16Policy {
     template <int BN>
     static constexpr int param_bytes() { return sizeof(Params); }
     __device__ static __forceinline__ void fix_a(v4i&) {}
-    __device__ static __forceinline__ v16i mma(const v4i& b, const v4i& a, const v16i& c) {
-        return __builtin_amdgcn_mfma_i32_32x32x32_i8(b, a, c, 0, 0, 0);
+    __device__ static __forceinline__ v16i mma(const v4i (&b)[1], const v4i (&a)[1], const v16i& c) {
+        return __builtin_amdgcn_mfma_i32_32x32x32_i8(b[0], a[0], c, 0, 0, 0);
     }
     __device__ static __forceinline__ void split_a(v4i& x, v4i& y, Extra& e, int pair, bool live) {
         typedef short s2 __attribute__((ext_vector_type(2)));

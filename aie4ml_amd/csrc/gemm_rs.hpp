@@ -6,6 +6,8 @@
 //   MMAS                         MFMA instructions issued per pair of fragments
 //   FIX_A, fix_a(v4i&)           optional fix-up of an A fragment before use
 //   mma(b, a, acc)               acc += the 32 x 32 block product of two fragments
+//   KSTEP_BYTES                  bytes of K one mma() call consumes per operand row: 32 (one 16-byte fragment per lane)
+//                                or 64 (two fragments per lane; the K tile then has two steps instead of four)
 //   MAX_OUT_BYTES                widest output element (sizes the LDS image of the output tile)
 //   SPLIT_A / split_a(x, y, extra, pair, live)
 //                                A elements are two bytes wide: a thread loads 16 of them as two registers and
@@ -133,7 +135,10 @@ __device__ __forceinline__ void wait_lgkmcnt0() { __builtin_amdgcn_s_waitcnt(0xC
 // -----------------------------------------------------------------------------------------------------
 template <class P, int BM, int BN, int WAVES_M, int WAVES_N>
 struct RsCfg {
-    static constexpr int BK = 128, CPR = 8, KSTEPS = 4;
+    static constexpr int BK = 128, CPR = 8;
+    static constexpr int FR = P::KSTEP_BYTES / 32;      // 16-byte fragments per lane, operand row and K step
+    static constexpr int KSTEPS = BK / P::KSTEP_BYTES;  // 4 or 2
+    static_assert(P::KSTEP_BYTES == 32 || P::KSTEP_BYTES == 64, "K step of 32 or 64 bytes");
     static constexpr int NW = WAVES_M * WAVES_N;
     static constexpr int NT = NW * 64;
     static constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
@@ -229,9 +234,12 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
 
     // ---- fragment addressing: row = lane%32 of the block, 16-byte half of the 32-wide K step = lane/32
     const int frow = lane & 31;
-    int koff[KSTEPS];
+    constexpr int FR = Cfg::FR;
+    int koff[KSTEPS][FR];  // lane half h takes the chunks [FR * (2 * kk + h), + FR) of K step kk
 #pragma unroll
-    for (int kk = 0; kk < KSTEPS; ++kk) koff[kk] = ((kk * 2 + (lane >> 5)) ^ ((frow >> 1) & 7)) * 16;
+    for (int kk = 0; kk < KSTEPS; ++kk)
+#pragma unroll
+        for (int f = 0; f < FR; ++f) koff[kk][f] = (((kk * 2 + (lane >> 5)) * FR + f) ^ ((frow >> 1) & 7)) * 16;
     const int a_off = (wm * Cfg::WTM + frow) * BK;
     const int b_off = BM * BK + (wn * Cfg::WTN + frow) * BK;
 
@@ -243,19 +251,22 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
 
-    v4i af[2][Cfg::TM], bf[2][Cfg::TN];
+    v4i af[2][Cfg::TM][FR], bf[2][Cfg::TN][FR];
     constexpr int NR = Cfg::TM + Cfg::TN, NM = Cfg::TM * Cfg::TN;
     auto read_one = [&](int set, const int8_t* base, int kk, int idx) {
         constexpr int TMIN = Cfg::TM < Cfg::TN ? Cfg::TM : Cfg::TN;
-        if (idx < 2 * TMIN) {
-            if (idx & 1) af[set][idx >> 1] = *reinterpret_cast<const v4i*>(base + a_off + (idx >> 1) * 32 * BK + koff[kk]);
-            else bf[set][idx >> 1] = *reinterpret_cast<const v4i*>(base + b_off + (idx >> 1) * 32 * BK + koff[kk]);
-        } else if (Cfg::TM > Cfg::TN) {
-            const int i = idx - TMIN;
-            af[set][i] = *reinterpret_cast<const v4i*>(base + a_off + i * 32 * BK + koff[kk]);
-        } else {
-            const int j = idx - TMIN;
-            bf[set][j] = *reinterpret_cast<const v4i*>(base + b_off + j * 32 * BK + koff[kk]);
+#pragma unroll
+        for (int f = 0; f < FR; ++f) {
+            if (idx < 2 * TMIN) {
+                if (idx & 1) af[set][idx >> 1][f] = *reinterpret_cast<const v4i*>(base + a_off + (idx >> 1) * 32 * BK + koff[kk][f]);
+                else bf[set][idx >> 1][f] = *reinterpret_cast<const v4i*>(base + b_off + (idx >> 1) * 32 * BK + koff[kk][f]);
+            } else if (Cfg::TM > Cfg::TN) {
+                const int i = idx - TMIN;
+                af[set][i][f] = *reinterpret_cast<const v4i*>(base + a_off + i * 32 * BK + koff[kk][f]);
+            } else {
+                const int j = idx - TMIN;
+                bf[set][j][f] = *reinterpret_cast<const v4i*>(base + b_off + j * 32 * BK + koff[kk][f]);
+            }
         }
     };
     // EXTRA: 0 = nothing, 1 = staging writes into `stage_w`, 2 = global loads of tile `kt_load`
@@ -264,7 +275,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
 #pragma unroll
         for (int m = 0; m < NM; ++m) {
             const int i = m / Cfg::TN, j = m % Cfg::TN;
-            if (P::FIX_A && j == 0) P::fix_a(af[cur][i]);
+            if (P::FIX_A && j == 0) {
+#pragma unroll
+                for (int f = 0; f < FR; ++f) P::fix_a(af[cur][i][f]);
+            }
             // operands swapped: the block's first index (registers) runs over n, lanes over m
             acc[i][j] = P::mma(bf[cur][j], af[cur][i], acc[i][j]);
             if (m < NR) read_one(nxt, next_base, next_kk, m);
@@ -276,9 +290,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
         }
 #pragma unroll
         for (int m = 0; m < NM; ++m) {
-            if (P::FIX_A && m % Cfg::TN == 0) __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // operand fix-up
+            if (P::FIX_A && m % Cfg::TN == 0) __builtin_amdgcn_sched_group_barrier(0x002, 4 * FR, 0);  // operand fix-up
             __builtin_amdgcn_sched_group_barrier(0x008, P::MMAS, 0);                              // one fragment pair
-            if (m < NR) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                          // one LDS read
+            if (m < NR) __builtin_amdgcn_sched_group_barrier(0x100, FR, 0);                         // one fragment's LDS reads
 #pragma unroll
             for (int e = m * Cfg::EPM; e < (m + 1) * Cfg::EPM && e < Cfg::LOADS; ++e) {
                 if (EXTRA == 1 || EXTRA == 3) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // one LDS write
@@ -305,6 +319,24 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
         int8_t* cur_base = smem + (kt & 1) * Cfg::STAGE_BYTES;
         int8_t* nxt_base = smem + ((kt + 1) & 1) * Cfg::STAGE_BYTES;
         split_live = kt + 1 < ktiles;
+        if constexpr (KSTEPS == 2) {
+            // two 64-byte steps per K tile: step 0 carries all the memory work, the barrier sits between the two
+            if (EARLY) {
+                step(0, 1, cur_base, 1, Tag3{}, nxt_base, min(kt + 2, ktiles - 1));
+            } else {
+                step(0, 1, cur_base, 1, Tag1{}, nxt_base, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            wait_lgkmcnt0();
+            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_sched_barrier(0);
+            if (EARLY) {
+                step(1, 0, nxt_base, 0, Tag0{}, nullptr, 0);
+            } else {
+                step(1, 0, nxt_base, 0, Tag2{}, nullptr, min(kt + 2, ktiles - 1));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        } else {
         if (EARLY) {
             step(0, 1, cur_base, 1, Tag3{}, nxt_base, min(kt + 2, ktiles - 1));
             __builtin_amdgcn_sched_barrier(0);
@@ -322,6 +354,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
         __builtin_amdgcn_sched_barrier(0);
         step(1, 0, nxt_base, 0, Tag0{}, nullptr, 0);  // after the last tile this reads a stale stage: unused
         __builtin_amdgcn_sched_barrier(0);
+        }
     }
     __syncthreads();  // every wave is past its last fragment read before the stages become the output image
     A4G_STAMP(3);
