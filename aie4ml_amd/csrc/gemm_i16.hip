@@ -7,8 +7,13 @@
 // and lo its unsigned lower byte; lo is fed as the signed byte lo - 128 (lo ^ 0x80). Two accumulator sets
 // per output block then give  a.w = 256 * sum(hi.w) + sum((lo-128).w) + 128 * sum(w),  all in wrapping
 // 32-bit arithmetic, which is exactly the acc32 the reference computes.
+//
+// Large problems with whole 128-element K tiles run on the software-pipelined kernel of gemm_rs.hpp with the
+// planes as rows (and, for int16 weights, columns) of its tile: I16Policy beside the int8 policy whose epilogue
+// it shares, I16x16Policy below. The kernels in this file take every other shape: K a multiple of 16 the
+// double-buffered tiled ones, anything else one thread per output.
 #include "common.hpp"
-#include "gemm_rs.hpp"  // tile_coord: the XCD-aware workgroup -> tile mapping shared with the int8 kernels
+#include "gemm_rs.hpp"  // tile_coord (XCD-aware workgroup -> tile mapping) and the pipelined kernel template
 
 namespace a4g {
 

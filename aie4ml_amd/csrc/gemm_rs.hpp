@@ -1,6 +1,6 @@
 // The register-staged pipelined MFMA kernel, shared by the integer and the floating-point GEMM entry
-// points. Tiles are handled as bytes: a fragment is 16 bytes of one operand row, and one K step is 32 bytes
-// per row, whatever the element type; a policy class supplies what depends on it:
+// points. Tiles are handled as bytes: a fragment is 16 bytes of one operand row, and one K step is 32 (or 64)
+// bytes per row, whatever the element type; a policy class supplies what depends on it:
 //
 //   acc_t                        16 accumulators of one 32 x 32 block (v16i or v16f)
 //   MMAS                         MFMA instructions issued per pair of fragments
