@@ -148,6 +148,28 @@ def test_matmul_batched_and_transposed(oracle):
     assert np.array_equal(oracle.matmul(P, B, 8, 'symmetric_inf').astype(np.int64), exp)
 
 
+def test_matmul_int16_left_operand_against_python_integers(oracle):
+    """The 16-bit MatMul combinations: int16 x int8 wraps to 32 bits before the shift (acc32), int16 x int16 keeps
+    64 bits (acc64); checked against exact integer matrix products and the rational rounding above."""
+    r = _rng(9)
+    A = r.integers(-32768, 32768, (2, 9, 40)).astype(np.int16)
+    A[0, 0] = 32767
+    A[1, 1] = -32768
+    for b_dtype, shift, wrap in ((np.int8, 13, True), (np.int16, 21, False)):
+        lo, hi = (-128, 128) if b_dtype == np.int8 else (-32768, 32768)
+        B = r.integers(lo, hi, (2, 40, 7)).astype(b_dtype)
+        B[0, :, 0] = hi - 1
+        B[1, :, 1] = lo
+        acc = A.astype(np.int64) @ B.astype(np.int64)
+        if wrap:
+            acc = ((acc + 2**31) % 2**32) - 2**31
+        for mode, kind in (('conv_even', 'int16'), ('symmetric_inf', 'int8'), ('floor', 'int16')):
+            exp = np.vectorize(lambda v: exact_srs(int(v), shift, mode, kind))(acc)
+            assert np.array_equal(oracle.matmul(A, B, shift, mode, out=kind).astype(np.int64), exp), (b_dtype, mode)
+            Bt = np.ascontiguousarray(np.swapaxes(B, -1, -2))
+            assert np.array_equal(oracle.matmul(A, Bt, shift, mode, trans_b=True, out=kind).astype(np.int64), exp)
+
+
 def test_add_is_saturating(oracle):
     a = np.arange(-128, 128, dtype=np.int8).repeat(256)
     b = np.tile(np.arange(-128, 128, dtype=np.int8), 256)
