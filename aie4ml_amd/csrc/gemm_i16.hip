@@ -522,56 +522,66 @@ __global__ __launch_bounds__(256) void gemm_i16i16_generic_kernel(Gemm16x16Args 
     }
 }
 
-// W [K][ldw] int16 -> planes [N][ldt] (signed high byte; low byte ^ 0x80), zero padding, and colsum[n] = sum_k (w - 128).
-__global__ __launch_bounds__(256) void pack_planes_i16_kernel(const int16_t* __restrict__ W, int64_t ldw, int8_t* __restrict__ Wh,
-                                                              int8_t* __restrict__ Wl, int64_t ldt, int32_t* __restrict__ colsum,
-                                                              int K, int N) {
-    const int n = blockIdx.x * blockDim.x + threadIdx.x;
-    if (n >= N) return;
-    int sum = 0;
-    for (int k = 0; k < K; ++k) {
-        const int w = W[static_cast<int64_t>(k) * ldw + n];
-        Wh[static_cast<int64_t>(n) * ldt + k] = static_cast<int8_t>(w >> 8);
-        Wl[static_cast<int64_t>(n) * ldt + k] = static_cast<int8_t>((w & 0xFF) ^ 0x80);
-        sum += w - 128;
-    }
-    for (int k = K; k < ldt; ++k) {
-        Wh[static_cast<int64_t>(n) * ldt + k] = 0;
-        Wl[static_cast<int64_t>(n) * ldt + k] = 0;
-    }
-    colsum[n] = sum;
-}
-
-// Dynamic right operand of a 16-bit MatMul -> what the kernels above read: rows n with k contiguous, plus the column
-// sums. B element (k, n) of problem b sits at B[b * stride_b + (trans_b ? n * ldb + k : k * ldb + n)].
-// WIDE: int16 operand -> the two byte planes and sum_k (b - 128); else int8 -> a transposed copy and sum_k b.
+// Right operand of a 16-bit GEMM -> what the kernels above read: rows n with k contiguous (padded with zeros to
+// ldt), plus the column sums. Element (k, n) of problem b sits at B[b * stride_b + (trans_b ? n * ldb + k : k * ldb + n)].
+// WIDE: int16 operand -> the two byte planes (signed high byte; low byte ^ 0x80) and sum_k (w - 128); else
+// int8 -> a transposed copy and sum_k w. Serves the constant weights (a4g_pack_weights_i16) and the dynamic
+// operand of a4g_matmul_i16. One workgroup owns 64 columns and walks K in 64 x 64 tiles through LDS, so that
+// both the reads and the writes are whole rows of a tile; a thread writes four consecutive k of one column as
+// one dword and keeps that column's partial sum, which the 16 threads of a column add up at the end.
 template <bool WIDE>
-__global__ __launch_bounds__(256) void pack_dynamic_rhs_kernel(const void* __restrict__ B, int64_t ldb, int64_t stride_b, int trans_b,
-                                                               int8_t* __restrict__ hi, int8_t* __restrict__ lo, int64_t ldt,
-                                                               int64_t stride_t, int32_t* __restrict__ colsum, int K, int N) {
-    const int n = blockIdx.x * blockDim.x + threadIdx.x, b = blockIdx.y;
-    if (n >= N) return;
-    int8_t* h = hi + b * stride_t + static_cast<int64_t>(n) * ldt;
-    int8_t* l = WIDE ? lo + b * stride_t + static_cast<int64_t>(n) * ldt : nullptr;
-    int sum = 0;
-    for (int k = 0; k < K; ++k) {
-        const int64_t at = b * stride_b + (trans_b ? static_cast<int64_t>(n) * ldb + k : static_cast<int64_t>(k) * ldb + n);
-        if (WIDE) {
-            const int w = static_cast<const int16_t*>(B)[at];
-            h[k] = static_cast<int8_t>(w >> 8);
-            l[k] = static_cast<int8_t>((w & 0xFF) ^ 0x80);
-            sum += w - 128;
-        } else {
-            const int w = static_cast<const int8_t*>(B)[at];
-            h[k] = static_cast<int8_t>(w);
-            sum += w;
+__global__ __launch_bounds__(256) void pack_rhs_kernel(const void* __restrict__ B, int64_t ldb, int64_t stride_b, int trans_b,
+                                                       int8_t* __restrict__ hi, int8_t* __restrict__ lo, int64_t ldt,
+                                                       int64_t stride_t, int32_t* __restrict__ colsum, int K, int N) {
+    __shared__ short tile[64][66];  // [k][n]
+    const int tid = threadIdx.x, b = blockIdx.y, n0 = blockIdx.x * 64;
+    const int kq = tid & 15;
+    // an element past the edge packs to zero bytes and adds nothing to the sum: 128 has high byte 0 and low byte 0x80
+    const short pad = WIDE ? 128 : 0;
+    int col_acc[4] = {0, 0, 0, 0};
+    for (int k0 = 0; k0 < ldt; k0 += 64) {
+        for (int i = tid; i < 64 * 64; i += 256) {
+            const int kk = trans_b ? (i & 63) : (i >> 6), nn = trans_b ? (i >> 6) : (i & 63);
+            const int k = k0 + kk, n = n0 + nn;
+            short v = pad;
+            if (k < K && n < N) {
+                const int64_t at = b * stride_b + (trans_b ? static_cast<int64_t>(n) * ldb + k : static_cast<int64_t>(k) * ldb + n);
+                v = WIDE ? static_cast<const int16_t*>(B)[at] : static_cast<short>(static_cast<const int8_t*>(B)[at]);
+            }
+            tile[kk][nn] = v;
         }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int nn = (tid >> 4) + 16 * j;
+            int w[4];
+#pragma unroll
+            for (int t = 0; t < 4; ++t) w[t] = tile[4 * kq + t][nn];
+            const int64_t at = b * stride_t + static_cast<int64_t>(n0 + nn) * ldt + k0 + 4 * kq;
+            const bool live = n0 + nn < N && k0 + 4 * kq < ldt;
+            if (WIDE) {
+                col_acc[j] += (w[0] - 128) + (w[1] - 128) + (w[2] - 128) + (w[3] - 128);
+                if (live) {
+                    *reinterpret_cast<unsigned*>(hi + at) = pack4_bytes(w[0] >> 8, w[1] >> 8, w[2] >> 8, w[3] >> 8);
+                    *reinterpret_cast<unsigned*>(lo + at) = pack4_bytes(w[0], w[1], w[2], w[3]) ^ 0x80808080u;
+                }
+            } else {
+                col_acc[j] += w[0] + w[1] + w[2] + w[3];
+                if (live) *reinterpret_cast<unsigned*>(hi + at) = pack4_bytes(w[0], w[1], w[2], w[3]);
+            }
+        }
+        __syncthreads();
     }
-    for (int k = K; k < ldt; ++k) {
-        h[k] = 0;
-        if (WIDE) l[k] = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        int v = col_acc[j];
+        v += __shfl_xor(v, 1);
+        v += __shfl_xor(v, 2);
+        v += __shfl_xor(v, 4);
+        v += __shfl_xor(v, 8);
+        const int n = n0 + (tid >> 4) + 16 * j;
+        if (kq == 0 && n < N) colsum[static_cast<int64_t>(b) * N + n] = v;
     }
-    colsum[static_cast<int64_t>(b) * N + n] = sum;
 }
 
 }  // namespace a4g
@@ -631,8 +641,8 @@ extern "C" int a4g_pack_weights_i16(const int16_t* W, int64_t ldw, int64_t K, in
     A4G_REQUIRE(K >= 1 && N >= 1 && K <= 32768 && N <= (1 << 24) && ldw >= N, A4G_ERR_INVALID_ARGUMENT,
                 "%s: bad shape K=%lld (at most 32768) N=%lld ldw=%lld", who, (long long)K, (long long)N, (long long)ldw);
     const int64_t ldt = K <= 0 ? 16 : (K + 15) / 16 * 16;
-    pack_planes_i16_kernel<<<static_cast<unsigned>((N + 255) / 256), 256, 0, stream>>>(W, ldw, Wt_hi, Wt_lo, ldt, colsum,
-                                                                                      static_cast<int>(K), static_cast<int>(N));
+    pack_rhs_kernel<true><<<dim3(static_cast<unsigned>((N + 63) / 64), 1), 256, 0, stream>>>(W, ldw, 0, 0, Wt_hi, Wt_lo, ldt, 0, colsum,
+                                                                                             static_cast<int>(K), static_cast<int>(N));
     return check_hip(hipGetLastError(), who);
 }
 
@@ -717,11 +727,11 @@ extern "C" int a4g_matmul_i16(const int16_t* A, int64_t lda, int64_t stride_a, c
     int8_t* hi = static_cast<int8_t*>(workspace);
     int8_t* lo = wide ? hi + batch * N * ldt : nullptr;
     int32_t* colsum = reinterpret_cast<int32_t*>(hi + (wide ? 2 : 1) * batch * N * ldt);
-    const dim3 pgrid(static_cast<unsigned>((N + 255) / 256), static_cast<unsigned>(batch));
+    const dim3 pgrid(static_cast<unsigned>((N + 63) / 64), static_cast<unsigned>(batch));
     if (wide)
-        pack_dynamic_rhs_kernel<true><<<pgrid, 256, 0, stream>>>(B, ldb, stride_b, trans_b, hi, lo, ldt, N * ldt, colsum, (int)K, (int)N);
+        pack_rhs_kernel<true><<<pgrid, 256, 0, stream>>>(B, ldb, stride_b, trans_b, hi, lo, ldt, N * ldt, colsum, (int)K, (int)N);
     else
-        pack_dynamic_rhs_kernel<false><<<pgrid, 256, 0, stream>>>(B, ldb, stride_b, trans_b, hi, lo, ldt, N * ldt, colsum, (int)K, (int)N);
+        pack_rhs_kernel<false><<<pgrid, 256, 0, stream>>>(B, ldb, stride_b, trans_b, hi, lo, ldt, N * ldt, colsum, (int)K, (int)N);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return check_hip(e, who);
 
