@@ -137,12 +137,14 @@ __global__ __launch_bounds__(256) void gemm_i16i8_kernel(Gemm16Args g) {
     // epilogue: lane owns row lane%32 of each block and, per register quad q, columns 8q + 4*(lane/32) .. +3
     const int lo_b = g.relu ? max(kind_lo(g.out_kind), 0) : kind_lo(g.out_kind), hi_b = kind_hi(g.out_kind);
     const int obytes = (g.out_kind == A4G_I16 || g.out_kind == A4G_U16) ? 2 : 1;
-    int8_t* Yb = static_cast<int8_t*>(g.Y);
+    // the tile leaves through an LDS image (the stages are dead: the loop ended on a barrier), then as whole rows
+    const int cpitch = BN * obytes + 16;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            const int n = n0 + wn * 64 + j * 32 + 8 * q + 4 * (lane >> 5);
+            const int nl = wn * 64 + j * 32 + 8 * q + 4 * (lane >> 5);
+            const int n = n0 + nl;
             unsigned add[4];
             RoundCfg rc[4];
 #pragma unroll
@@ -154,21 +156,32 @@ __global__ __launch_bounds__(256) void gemm_i16i8_kernel(Gemm16Args g) {
             }
 #pragma unroll
             for (int i = 0; i < 2; ++i) {
-                const int m = m0 + wm * 64 + i * 32 + (lane & 31);
-                if (m >= g.M) continue;
+                const int ml = wm * 64 + i * 32 + (lane & 31);
+                int y[4];
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
-                    if (n + t >= g.N) continue;
                     const unsigned a = (static_cast<unsigned>(acc_hi[i][j][q * 4 + t]) << 8) +
                                        static_cast<unsigned>(acc_lo[i][j][q * 4 + t]) + add[t];
-                    const int y = clamp_i(apply_round(static_cast<int>(a), rc[t]), lo_b, hi_b);
-                    const int64_t at = static_cast<int64_t>(m) * g.ldy + n + t;
-                    if (obytes == 1) Yb[at] = static_cast<int8_t>(y);
-                    else reinterpret_cast<int16_t*>(Yb)[at] = static_cast<int16_t>(y);
+                    y[t] = clamp_i(apply_round(static_cast<int>(a), rc[t]), lo_b, hi_b);
+                }
+                if (obytes == 1) {
+                    *reinterpret_cast<unsigned*>(smem + ml * cpitch + nl) = pack4_bytes(y[0], y[1], y[2], y[3]);
+                } else {
+                    v2i o = {static_cast<int>(pack2_halves(y[0], y[1])), static_cast<int>(pack2_halves(y[2], y[3]))};
+                    *reinterpret_cast<v2i*>(smem + ml * cpitch + nl * 2) = o;
                 }
             }
         }
     }
+    __syncthreads();
+    GemmArgs img{};
+    img.C = g.Y;
+    img.ldc = g.ldy;
+    img.M = g.M;
+    img.N = g.N;
+    TileCoord here = tc;
+    here.batch = 0;  // select_problem has already moved the pointers to this problem
+    store_tile_image<BM, BN, 256>(img, here, smem, obytes, tid);
 }
 
 // Any K / alignment: one thread per output element.
@@ -477,28 +490,41 @@ __global__ __launch_bounds__(256) void gemm_i16i16_kernel(Gemm16x16Args g) {
 
     const int lo_b = g.relu ? max(kind_lo(g.out_kind), 0) : kind_lo(g.out_kind), hi_b = kind_hi(g.out_kind);
     const int obytes = (g.out_kind == A4G_I16 || g.out_kind == A4G_U16) ? 2 : 1;
-    int8_t* Yb = static_cast<int8_t*>(g.Y);
-    const int m = m0 + wm * 32 + (lane & 31);
+    // the tile leaves through an LDS image (the stages are dead: the loop ended on a barrier), then as whole rows
+    const int cpitch = BN * obytes + 16;
+    const int ml = wm * 32 + (lane & 31);
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            const int n = n0 + wn * 64 + j * 32 + 8 * q + 4 * (lane >> 5);
+            const int nl = wn * 64 + j * 32 + 8 * q + 4 * (lane >> 5);
+            int y[4];
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
-                if (m >= g.M || n + t >= g.N) continue;
-                const int nn = n + t;
+                const int nn = min(n0 + nl + t, g.N - 1);
                 const long long v = (static_cast<long long>(acc_hh[j][q * 4 + t]) << 16) +
                                     ((static_cast<long long>(acc_hl[j][q * 4 + t]) + acc_lh[j][q * 4 + t]) << 8) +
                                     acc_ll[j][q * 4 + t] + row_term + 128ll * g.colsum[nn] + (g.bias ? g.bias[nn] : 0);
                 const int s = min(max(g.shifts ? g.shifts[static_cast<int64_t>(nn) * g.shift_stride] : g.shift, 0), 62);
-                const int y = requant64(v, s, g.mode, lo_b, hi_b);
-                const int64_t at = static_cast<int64_t>(m) * g.ldy + nn;
-                if (obytes == 1) Yb[at] = static_cast<int8_t>(y);
-                else reinterpret_cast<int16_t*>(Yb)[at] = static_cast<int16_t>(y);
+                y[t] = requant64(v, s, g.mode, lo_b, hi_b);
+            }
+            if (obytes == 1) {
+                *reinterpret_cast<unsigned*>(smem + ml * cpitch + nl) = pack4_bytes(y[0], y[1], y[2], y[3]);
+            } else {
+                v2i o = {static_cast<int>(pack2_halves(y[0], y[1])), static_cast<int>(pack2_halves(y[2], y[3]))};
+                *reinterpret_cast<v2i*>(smem + ml * cpitch + nl * 2) = o;
             }
         }
     }
+    __syncthreads();
+    GemmArgs img{};
+    img.C = g.Y;
+    img.ldc = g.ldy;
+    img.M = g.M;
+    img.N = g.N;
+    TileCoord here = tc;
+    here.batch = 0;  // select_problem has already moved the pointers to this problem
+    store_tile_image<BM, BN, 256>(img, here, smem, obytes, tid);
 }
 
 // Any K / alignment: one thread per output element, straight from the planes (w = 256 wh + (wl ^ 0x80 as unsigned)).
