@@ -697,20 +697,27 @@ __global__ __launch_bounds__(256) void transpose_kn_kernel(const int8_t* __restr
 }
 
 // colsum[b][n] = sum_k rhs[k][n]; trans: rhs stored [N][ld] (sum along the contiguous axis).
+// A workgroup owns 64 columns; its four waves take every fourth k (rows of 64 contiguous bytes when the operand
+// is [K][N]; when it is [N][ld] a thread walks its own row in steps of four) and add up through LDS.
 __global__ __launch_bounds__(256) void colsum_kernel(const int8_t* __restrict__ B, int64_t ld, int64_t stride_b, int trans,
                                                       int32_t* __restrict__ colsum, int64_t stride_c, int K, int N) {
+    __shared__ int part[4][64];
     const int batch = blockIdx.y;
     const int8_t* src = B + batch * stride_b;
-    const int n = blockIdx.x * blockDim.x + threadIdx.x;
-    if (n >= N) return;
+    const int c = threadIdx.x & 63, ks = threadIdx.x >> 6;
+    const int n = blockIdx.x * 64 + c;
     int s = 0;
-    if (trans) {
-        const int8_t* r = src + static_cast<int64_t>(n) * ld;
-        for (int k = 0; k < K; ++k) s += r[k];
-    } else {
-        for (int k = 0; k < K; ++k) s += src[static_cast<int64_t>(k) * ld + n];
+    if (n < N) {
+        if (trans) {
+            const int8_t* r = src + static_cast<int64_t>(n) * ld;
+            for (int k = ks; k < K; k += 4) s += r[k];
+        } else {
+            for (int k = ks; k < K; k += 4) s += src[static_cast<int64_t>(k) * ld + n];
+        }
     }
-    colsum[batch * stride_c + n] = s;
+    part[ks][c] = s;
+    __syncthreads();
+    if (ks == 0 && n < N) colsum[batch * stride_c + n] = part[0][c] + part[1][c] + part[2][c] + part[3][c];
 }
 
 static inline int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
@@ -844,7 +851,7 @@ extern "C" int a4g_pack_weights_i8(const int8_t* W, int64_t ldw, int64_t K, int6
     dim3 grid(static_cast<unsigned>((ldt + 63) / 64), static_cast<unsigned>((N + 63) / 64), 1);
     transpose_kn_kernel<<<grid, 256, 0, stream>>>(W, ldw, 0, Wt, ldt, 0, static_cast<int>(K), static_cast<int>(N));
     if (colsum) {
-        colsum_kernel<<<dim3(static_cast<unsigned>((N + 255) / 256), 1), 256, 0, stream>>>(W, ldw, 0, 0, colsum, 0,
+        colsum_kernel<<<dim3(static_cast<unsigned>((N + 63) / 64), 1), 256, 0, stream>>>(W, ldw, 0, 0, colsum, 0,
                                                                                           static_cast<int>(K),
                                                                                           static_cast<int>(N));
     }
@@ -975,7 +982,7 @@ extern "C" int a4g_matmul_i8(const void* A, int a_kind, int64_t lda, int64_t str
     int32_t* colsum = nullptr;
     if (g.a_unsigned) {
         colsum = reinterpret_cast<int32_t*>(ws + (trans_b ? 0 : round_up(batch * N * ldt, 256)));
-        colsum_kernel<<<dim3(static_cast<unsigned>((N + 255) / 256), static_cast<unsigned>(batch)), 256, 0, stream>>>(
+        colsum_kernel<<<dim3(static_cast<unsigned>((N + 63) / 64), static_cast<unsigned>(batch)), 256, 0, stream>>>(
             B, ldb, stride_b, trans_b, colsum, N, static_cast<int>(K), static_cast<int>(N));
         g.colsum = colsum;
         g.stride_colsum = N;
