@@ -151,23 +151,35 @@ __global__ __launch_bounds__(256, 2) void matmul_lean_nn_kernel(LeanArgs a) {
         const int nb = (a.K >> 2) * (N / 4);
         const int n0 = (tid % (N / 4)) * 4;
         int part[4] = {0, 0, 0, 0};
-        for (int blk = tid; blk < nb; blk += 256) {
-            const int k0 = (blk / (N / 4)) * 4;
-            unsigned av[4], cv[4];
+        // four blocks' loads are issued before the first is transposed: one exposed load latency per four blocks
+        for (int blk0 = tid; blk0 < nb; blk0 += 4 * 256) {
+            unsigned av[4][4];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) av[i] = *reinterpret_cast<const unsigned*>(Bp + static_cast<int64_t>(k0 + i) * a.ldb + n0);
-            const unsigned lo01 = __builtin_amdgcn_perm(av[1], av[0], 0x05010400u);
-            const unsigned hi01 = __builtin_amdgcn_perm(av[1], av[0], 0x07030602u);
-            const unsigned lo23 = __builtin_amdgcn_perm(av[3], av[2], 0x05010400u);
-            const unsigned hi23 = __builtin_amdgcn_perm(av[3], av[2], 0x07030602u);
-            cv[0] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);
-            cv[1] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
-            cv[2] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);
-            cv[3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
+            for (int u = 0; u < 4; ++u) {
+                const int blk = blk0 + u * 256;
+                const int k0 = (min(blk, nb - 1) / (N / 4)) * 4;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                *reinterpret_cast<unsigned*>(bt + (n0 + j) * pitch + k0) = cv[j];
-                part[j] = __builtin_amdgcn_sdot4(static_cast<int>(cv[j]), 0x01010101, part[j], false);
+                for (int i = 0; i < 4; ++i) av[u][i] = *reinterpret_cast<const unsigned*>(Bp + static_cast<int64_t>(k0 + i) * a.ldb + n0);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int blk = blk0 + u * 256;
+                if (blk >= nb) break;
+                const int k0 = (blk / (N / 4)) * 4;
+                unsigned cv[4];
+                const unsigned lo01 = __builtin_amdgcn_perm(av[u][1], av[u][0], 0x05010400u);
+                const unsigned hi01 = __builtin_amdgcn_perm(av[u][1], av[u][0], 0x07030602u);
+                const unsigned lo23 = __builtin_amdgcn_perm(av[u][3], av[u][2], 0x05010400u);
+                const unsigned hi23 = __builtin_amdgcn_perm(av[u][3], av[u][2], 0x07030602u);
+                cv[0] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);
+                cv[1] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
+                cv[2] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);
+                cv[3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    *reinterpret_cast<unsigned*>(bt + (n0 + j) * pitch + k0) = cv[j];
+                    part[j] = __builtin_amdgcn_sdot4(static_cast<int>(cv[j]), 0x01010101, part[j], false);
+                }
             }
         }
         if (a.a_unsigned) {
