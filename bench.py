@@ -35,11 +35,11 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
 # WRITE_SIZE, one counter run each, scaled by what the same counter reads for calib_copy).
 # None = not measured.
 MEASURED_TRAFFIC = {
-    'c2_dense': 227826201, 'c1_mlp': 166940, 'c4_add': 49063352, 'c4_layernorm': 33052160,
-    'c4_add_layernorm': 49190223, 'c3_softmax_exp': 263311379, 'c3_softmax_hccs': 263311577,
-    'c3_qk': 182768882, 'c3_pv': 210431233, 'c3_attention_exp': 118082676, 'c3_attention_hccs': 118082322,
-    'calib_copy': 536870912, 'c2_dense_i16': 454852713, 'c2_dense_i16x16': 842205840, 'c2_dense_bf16': 454925551,
-    'c2_dense_fp8': 244962105,
+    'c2_dense': 227885846, 'c1_mlp': 166941, 'c4_add': 49063677, 'c4_layernorm': 33052188,
+    'c4_add_layernorm': 49190372, 'c3_softmax_exp': 263311713, 'c3_softmax_hccs': 263311775,
+    'c3_qk': 182767058, 'c3_pv': 210446951, 'c3_attention_exp': 118076855, 'c3_attention_hccs': 118071577,
+    'calib_copy': 536870912, 'c2_dense_i16': 454854493, 'c2_dense_i16x16': 842202091, 'c2_dense_bf16': 454969771,
+    'c2_dense_fp8': 244968648,
 }
 
 
