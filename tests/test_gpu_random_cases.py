@@ -1,0 +1,135 @@
+"""Seeded random cases through the C ABI against the CPU oracle: shapes drawn around the tile sizes of every kernel
+family (so that each dispatch branch is met with ragged edges), pitched and misaligned views, every rounding mode,
+operand width and output kind. Bit-exact, like every integer test here."""
+
+import os
+
+import numpy as np
+import pytest
+
+torch = pytest.importorskip('torch')
+
+pytestmark = pytest.mark.gpu
+
+MODES = ['floor', 'ceil', 'positive_inf', 'negative_inf', 'symmetric_inf', 'symmetric_zero', 'conv_even', 'conv_odd']
+M_CHOICES = [1, 7, 31, 64, 127, 128, 129, 255, 300, 513, 1000, 2049]
+N_CHOICES = [1, 17, 32, 64, 96, 128, 192, 200, 256, 384, 768, 1000]
+K_CHOICES = [1, 15, 16, 48, 64, 100, 128, 192, 256, 384, 1000, 1024]
+EXTRA = int(os.environ.get('A4G_RANDOM_EXTRA', '0'))  # more seeds for a longer hunt
+
+
+@pytest.fixture(scope='module')
+def ops():
+    if not torch.cuda.is_available():
+        pytest.skip('no GPU')
+    from aie4ml_amd import ops as _ops
+
+    return _ops
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def draw(r, dtype, shape):
+    info = np.iinfo(dtype)
+    if r.random() < 0.5:   # full range, else a narrow bell (more ties, less saturation)
+        return r.integers(info.min, info.max + 1, shape).astype(dtype)
+    sigma = (info.max - info.min) / 12.0
+    return np.clip(np.rint(r.normal(0, sigma, shape)), info.min, info.max).astype(dtype)
+
+
+def pitched(t, r):
+    """A 2-d tensor as a view into a wider buffer: row pitch and start offset that may break 16-byte alignment."""
+    rows, cols = t.shape
+    pad, off = int(r.choice([0, 0, 16, 3])), int(r.choice([0, 0, 16, 5]))
+    if pad == 0 and off == 0:
+        return t
+    big = torch.zeros((rows, cols + pad + off), dtype=t.dtype, device=t.device)
+    big[:, off:off + cols] = t
+    return big[:, off:off + cols]
+
+
+@pytest.mark.parametrize('seed', range(40 + EXTRA))
+def test_dense_random_case(ops, oracle, seed):
+    r = np.random.default_rng(1000 + seed)
+    a_dtype = [np.int8, np.uint8, np.int16][seed % 3]
+    w_dtype = np.int16 if (a_dtype == np.int16 and r.random() < 0.5) else np.int8
+    M, N, K = int(r.choice(M_CHOICES)), int(r.choice(N_CHOICES)), int(r.choice(K_CHOICES))
+    if seed % 10 == 9:  # large enough for the pipelined kernels of every width
+        M, N, K = int(r.choice([2100, 4096])), int(r.choice([3100, 2048])), int(r.choice([256, 384]))
+    wide = w_dtype == np.int16
+    A, W = draw(r, a_dtype, (M, K)), draw(r, w_dtype, (K, N))
+    bias = None if r.random() < 0.2 else r.integers(-2**31 if wide else -2**24, 2**31 if wide else 2**24, N).astype(np.int32)
+    top = 40 if wide else 20
+    shifts = int(r.integers(0, top)) if r.random() < 0.4 else r.integers(0, top, N).astype(np.int32)
+    mode, relu = str(r.choice(MODES)), bool(r.random() < 0.5)
+    kind = str(r.choice(['int8', 'uint8', 'int16']))
+    p = ops.pack_dense(dev(W), None if bias is None else dev(bias), shifts)
+    x = pitched(dev(A), r)
+    out_full = torch.full((M, N + 16), 77, dtype={'int8': torch.int8, 'uint8': torch.uint8, 'int16': torch.int16}[kind],
+                          device='cuda')
+    out = out_full[:, :N] if r.random() < 0.5 else None
+    got = ops.dense(x, p, mode, relu=relu, out_kind=kind, out=out)
+    exp = oracle.dense(A, W, bias, shifts, mode, relu=relu, out=kind)
+    assert np.array_equal(host(got), exp), (seed, a_dtype, w_dtype, M, N, K, mode, kind)
+    if out is not None:
+        assert bool((out_full[:, N:] == 77).all()), 'wrote beyond the output columns'
+
+
+@pytest.mark.parametrize('seed', range(30 + EXTRA))
+def test_matmul_random_case(ops, oracle, seed):
+    r = np.random.default_rng(2000 + seed)
+    a_dtype = [np.int8, np.uint8, np.int16][seed % 3]
+    b_dtype = np.int16 if (a_dtype == np.int16 and r.random() < 0.5) else np.int8
+    lead = [(), (3,), (2, 2)][int(r.integers(0, 3))]
+    M, N, K = int(r.choice(M_CHOICES[:9])), int(r.choice(N_CHOICES[:10])), int(r.choice(K_CHOICES[:10]))
+    if seed % 10 == 9:
+        lead, M, N, K = (2,), 1500, 2048, 256
+    trans_b = bool(r.random() < 0.5)
+    A = draw(r, a_dtype, lead + (M, K))
+    B = draw(r, b_dtype, lead + ((N, K) if trans_b else (K, N)))
+    shift = int(r.integers(0, 30 if b_dtype == np.int16 else 20))
+    mode, kind = str(r.choice(MODES)), str(r.choice(['int8', 'uint8', 'int16']))
+    got = host(ops.matmul(dev(A), dev(B), shift, mode, trans_b=trans_b, out_kind=kind))
+    exp = oracle.matmul(A, B, shift, mode, trans_b=trans_b, out=kind)
+    assert np.array_equal(got, exp), (seed, a_dtype, b_dtype, lead, M, N, K, trans_b, mode, kind)
+
+
+@pytest.mark.parametrize('seed', range(24 + EXTRA))
+def test_row_operator_random_case(ops, oracle, seed):
+    r = np.random.default_rng(3000 + seed)
+    rows = int(r.choice([1, 5, 63, 64, 100, 257, 1000]))
+    cols = int(r.choice([16, 48, 64, 100, 128, 256, 512, 768, 1024, 2048, 4096, 5000]))
+    x = draw(r, np.int8, (rows, cols))
+    y = draw(r, np.int8, (rows, cols))
+    mode = str(r.choice(MODES))
+    which = seed % 4
+    if which == 0:
+        gmax = int(r.choice([100, 511, 600, 32767]))
+        gamma = r.integers(-gmax, gmax + 1, cols).astype(np.int16)
+        beta = r.integers(-32768, 32768, cols).astype(np.int16)
+        out_shift, gamma_shift, eps = int(r.integers(0, 16)), int(r.integers(0, 16)), int(r.integers(1, 50))
+        got = host(ops.layernorm(dev(x), dev(gamma), dev(beta), out_shift, mode, eps_q0=eps, gamma_shift=gamma_shift))
+        exp = oracle.layernorm(x, gamma, beta, out_shift, mode, eps_q0=eps, gamma_shift=gamma_shift)
+    elif which == 1:
+        gamma = r.integers(-300, 301, cols).astype(np.int16)
+        beta = r.integers(-32768, 32768, cols).astype(np.int16)
+        out_shift = int(r.integers(0, 16))
+        got = host(ops.add_layernorm(dev(x), dev(y), dev(gamma), dev(beta), out_shift, mode))
+        exp = oracle.add_layernorm(x, y, gamma, beta, out_shift, mode)
+    elif which == 2:
+        kq = int(r.integers(1, 129))
+        kind = str(r.choice(['uint8', 'int16']))
+        got = host(ops.softmax_exp(dev(x), kq, out_kind=kind))
+        exp = oracle.softmax_exp(x, kq, out=kind)
+    else:
+        shift = int(r.integers(0, 4))
+        got = host(ops.add(dev(x), dev(y), shift, mode))
+        exp = oracle.add(x, y, shift, mode)
+    assert np.array_equal(got, exp), (seed, which, rows, cols, mode)
