@@ -133,3 +133,36 @@ def test_row_operator_random_case(ops, oracle, seed):
         got = host(ops.add(dev(x), dev(y), shift, mode))
         exp = oracle.add(x, y, shift, mode)
     assert np.array_equal(got, exp), (seed, which, rows, cols, mode)
+
+
+HCCS = {32: (255, 4, 60), 64: (255, 3, 80), 128: (255, 2, 126), 256: (127, 1, 126), 512: (60, 1, 59)}
+
+
+@pytest.mark.parametrize('seed', range(20 + EXTRA // 8))
+def test_attention_random_case(ops, oracle, seed):
+    """The fused attention core against the oracle's three separate operators."""
+    r = np.random.default_rng(4000 + seed)
+    sk = int(r.choice([32, 64, 128, 256, 512]))
+    sq = int(r.choice([1, 33, 128, 200, 256, 512, 700]))
+    lead = [(1, 1), (2, 3), (5, 2)][int(r.integers(0, 3))]
+    if sq >= 256 and r.random() < 0.5:
+        lead = (16, 16)  # enough work for the 256-row workgroups with the bank-replicated score table
+    sigma = float(r.choice([8.0, 24.0, 60.0]))
+    g = lambda s: np.clip(np.rint(r.normal(0, sigma, s)), -128, 127).astype(np.int8)  # noqa: E731
+    q, k, v = g(lead + (sq, 64)), g(lead + (sk, 64)), g(lead + (sk, 64))
+    lshift, oshift = int(r.integers(0, 17)), int(r.integers(0, 12))
+    lmode, omode = str(r.choice(MODES)), str(r.choice(MODES))
+    if r.random() < 0.5:
+        lmode = 'conv_even'
+    if seed % 2 == 0:
+        sm = {'kind': 'exp', 'exp_kq': int(r.integers(1, 129))}
+        logits = oracle.matmul(q, k, lshift, lmode, trans_b=True)
+        p = oracle.softmax_exp(logits, sm['exp_kq'])
+    else:
+        B, S, Dmax = HCCS[sk]
+        sm = {'kind': 'hccs', 'B': B, 'S': S, 'Dmax': Dmax}
+        logits = oracle.matmul(q, k, lshift, lmode, trans_b=True)
+        p = oracle.softmax_hccs(logits, B, S, Dmax, 15, False)
+    exp = oracle.matmul(p, v, oshift, omode)
+    got = host(ops.attention(dev(q), dev(k), dev(v), lshift, lmode, sm, oshift, omode))
+    assert np.array_equal(got, exp), (seed, lead, sq, sk, lshift, lmode, oshift, omode, sm)
