@@ -952,6 +952,8 @@ extern "C" int a4g_matmul_i8(const void* A, int a_kind, int64_t lda, int64_t str
         la.hi = out_kind == A4G_I8 ? 127 : 255;
         la.fr = make_fast_round(round_mode, shift);
         la.br = make_byte_requant(la.fr, la.lo, la.hi);
+        // nearest even over a short reduction: the transposed-B kernel requantises in float (|acc| <= 128 * 2^14)
+        la.fscale = (round_mode == A4G_RND_CONV_EVEN && shift >= 1 && shift <= 15) ? ldexpf(1.f, -shift) : 0.f;
         if (trans_b && lean_nt_applicable(la)) return check_hip(launch_lean_nt(la, stream), who);
         if (!trans_b && lean_nn_applicable(la)) return check_hip(launch_lean_nn(la, stream), who);
     }

@@ -49,8 +49,21 @@ __device__ __forceinline__ void lean_nt_compute(const LeanArgs& a, int8_t* Cp, c
 #pragma unroll
             for (int ks = 0; ks < DT; ++ks) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[T][ks], af[rb][ks], acc, 0, 0, 0);
 #pragma unroll
-            for (int gg = 0; gg < 4; ++gg)
-                o[T][gg] = static_cast<int>(requant4_bytes<BIT>(acc[4 * gg], acc[4 * gg + 1], acc[4 * gg + 2], acc[4 * gg + 3], a.br));
+            for (int gg = 0; gg < 4; ++gg) {
+                if (BIT == 3) {
+                    // |acc| <= K * 2^14 <= 2^21 and the bias 2^(7 + shift) <= 2^22: (acc + 128 * 2^s) * 2^-s is exact
+                    // in a float; v_cvt_pk_u8_f32 rounds to nearest even, saturates to 0..255 and places the byte
+                    const float bias = UOUT ? 0.f : 128.f;
+                    unsigned w = 0;
+                    w = __builtin_amdgcn_cvt_pk_u8_f32(fmaf(static_cast<float>(acc[4 * gg]), a.fscale, bias), 0, w);
+                    w = __builtin_amdgcn_cvt_pk_u8_f32(fmaf(static_cast<float>(acc[4 * gg + 1]), a.fscale, bias), 1, w);
+                    w = __builtin_amdgcn_cvt_pk_u8_f32(fmaf(static_cast<float>(acc[4 * gg + 2]), a.fscale, bias), 2, w);
+                    w = __builtin_amdgcn_cvt_pk_u8_f32(fmaf(static_cast<float>(acc[4 * gg + 3]), a.fscale, bias), 3, w);
+                    o[T][gg] = static_cast<int>(UOUT ? w : w ^ 0x80808080u);
+                } else {
+                    o[T][gg] = static_cast<int>(requant4_bytes<BIT>(acc[4 * gg], acc[4 * gg + 1], acc[4 * gg + 2], acc[4 * gg + 3], a.br));
+                }
+            }
         }
         if (TG == 4) {
 #pragma unroll
@@ -240,14 +253,14 @@ bool lean_nt_applicable(const LeanArgs& a) {
 
 template <int DT, int RB>
 static void launch_lean_nt_cfg(const LeanArgs& a, dim3 grid, hipStream_t stream) {
-    const int bit = fast_round_kind(a.fr);
+    const int bit = a.fscale > 0.f ? 3 : fast_round_kind(a.fr);  // 3: nearest even in float arithmetic
     const bool uo = a.lo == 0;
 #define A4G_NT(B)                                                                          \
     if (uo)                                                                                \
         matmul_lean_nt_kernel<DT, RB, B, true><<<grid, 256, 0, stream>>>(a);               \
     else                                                                                   \
         matmul_lean_nt_kernel<DT, RB, B, false><<<grid, 256, 0, stream>>>(a);
-    if (bit == 0) { A4G_NT(0) } else if (bit == 1) { A4G_NT(1) } else { A4G_NT(2) }
+    if (bit == 0) { A4G_NT(0) } else if (bit == 1) { A4G_NT(1) } else if (bit == 2) { A4G_NT(2) } else { A4G_NT(3) }
 #undef A4G_NT
 }
 

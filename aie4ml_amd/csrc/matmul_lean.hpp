@@ -18,6 +18,7 @@ struct LeanArgs {
     int lo, hi;  // saturation bounds of the output kind
     FastRound fr;
     ByteRequant br;  // fr with the clamp bounds moved in front of the shift (transposed-B kernel)
+    float fscale;    // 2^-shift when the transposed-B kernel may requantise in float (nearest even), else 0
 };
 
 // C = srs(A x B^T): B is [N][ldb], K in {32,64,96,128}, N % 32 == 0. Returns false when not applicable.
