@@ -738,7 +738,8 @@ static int softmax_dispatch(const int8_t* x, void* out, int64_t rows, int64_t co
         while (L < chunks && L < 64) L <<= 1;
         const int nch = (chunks + L - 1) / L;
         const int rpw = 64 / L;
-        const int grid = grid_for((rows + rpw - 1) / rpw, 4, 256 * 8);
+        // 32 blocks per CU measured best on 262144 x 512 (44.5 us; 8 per CU 47 us, 4 per CU 55 us, 128 per CU 46 us)
+        const int grid = grid_for((rows + rpw - 1) / rpw, 4, 256 * 32);
         const int r = static_cast<int>(rows), c = static_cast<int>(cols);
         if (nch > 1) {  // L == 64
             if (nch <= 2) launch_softmax<64, 2>(noclamp, grid, stream, x, out, r, c, p);
