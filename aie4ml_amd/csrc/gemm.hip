@@ -794,7 +794,9 @@ static hipError_t launch_gemm_nt(const GemmArgs& g, int batch, hipStream_t strea
         // else (attention-sized batches, short K, narrow N) measured faster with 128 x 128.
         const int64_t tiles256 = static_cast<int64_t>((g.M + 255) / 256) * ((g.N + 255) / 256) * batch;
         const int64_t rounds256 = (tiles256 + 255) / 256;  // one workgroup per CU at a time
-        const bool fills = tiles256 * 100 >= rounds256 * 256 * 85;
+        // the last round must be 85 % full, or 75 % for deep reductions (8192 x 3072 x 3072, 384 tiles: 94 us against
+        // 103 us with 128 x 128; the same output with K = 768 inside the encoder block: 128 x 128 ahead by 2 %)
+        const bool fills = tiles256 * 100 >= rounds256 * 256 * (g.K >= 2048 ? 75 : 85);
         variant = (g.M >= 256 && g.N >= 256 && g.K >= 512 && fills) ? 1 : 2;
         // Widths that are multiples of 192 but not of 256 (768 = 3 * 256 columns on 256 CUs): 128 x 192
         // tiles that make exactly one round of workgroups measured 5-15 % faster than 128 x 128.
