@@ -12,10 +12,22 @@
 // planes as rows (and, for int16 weights, columns) of its tile: I16Policy beside the int8 policy whose epilogue
 // it shares, I16x16Policy below. The kernels in this file take every other shape: K a multiple of 16 the
 // double-buffered tiled ones, anything else one thread per output.
+#include <cstdlib>
+#include <algorithm>
 #include "common.hpp"
+#include "gemm_epilogue.hpp"
 #include "gemm_rs.hpp"  // tile_coord (XCD-aware workgroup -> tile mapping) and the pipelined kernel template
 
 namespace a4g {
+
+// LDS of the tiled kernels below: one stage of either is 30720 bytes (K step 64, rows padded to 80 bytes), which
+// the output image reuses. A reduction that fits one K tile takes a single stage, so more workgroups share a CU.
+constexpr int TILED16_STAGE_BYTES = 30720;
+static inline size_t tiled16_lds_bytes(int64_t K, int tile_rows) {
+    const size_t stages = static_cast<size_t>(K > 64 ? 2 : 1) * TILED16_STAGE_BYTES;
+    const size_t image = static_cast<size_t>(tile_rows) * (128 * 2 + 16);  // 128 two-byte outputs per row and its padding
+    return stages > image ? stages : image;
+}
 
 struct Gemm16Args {
     const int16_t* A;
@@ -42,11 +54,12 @@ __device__ __forceinline__ void select_problem(Gemm16Args& g, int b) {
     g.Y = static_cast<int8_t*>(g.Y) + b * g.stride_y * obytes;
 }
 
-__global__ __launch_bounds__(256) void gemm_i16i8_kernel(Gemm16Args g) {
+__global__ __launch_bounds__(256, 2) void gemm_i16i8_kernel(Gemm16Args g) {
     constexpr int BM = 128, BN = 128, BK = 64, PITCH = BK + 16;
     select_problem(g, blockIdx.y);
     constexpr int PLANE = BM * PITCH, STAGE = 2 * PLANE + BN * PITCH;
-    __shared__ __attribute__((aligned(16))) int8_t smem[2 * STAGE];
+    static_assert(STAGE == TILED16_STAGE_BYTES, "the launch sizes the LDS");
+    extern __shared__ __attribute__((aligned(16))) int8_t smem[];  // two stages, or one when K fits a single tile
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
@@ -56,6 +69,27 @@ __global__ __launch_bounds__(256) void gemm_i16i8_kernel(Gemm16Args g) {
     const TileCoord tc = tile_coord<BM, BN>(shape);
     if (!tc.valid) return;
     const int m0 = tc.m0, n0 = tc.n0;
+
+    // the epilogue of the int8 kernels, fed with this problem's pointers (select_problem has already moved them)
+    GemmArgs eg{};
+    eg.C = g.Y;
+    eg.ldc = g.ldy;
+    eg.M = g.M;
+    eg.N = g.N;
+    eg.bias = g.bias;
+    eg.colsum = g.colsum;
+    eg.shifts = g.shifts;
+    eg.shift_stride = g.shift_stride;
+    eg.shift = g.shift;
+    eg.mode = g.mode;
+    eg.relu = g.relu;
+    eg.out_kind = g.out_kind;
+    TileCoord here = tc;
+    here.batch = 0;
+    __shared__ __attribute__((aligned(16))) int8_t cp_mem[ColParams<BN>::BYTES];
+    const ColParams<BN> cp(cp_mem);
+    int col_add, col_shift;
+    fetch_col_params<BN, true>(eg, here, tid, col_add, col_shift);
 
     // staging: A tile = 128 rows x 8 chunks of 8 int16 (4 per thread), W tile = 128 rows x 4 chunks of 16 int8 (2 per thread)
     v4i ra[4], rb[2];
@@ -107,6 +141,7 @@ __global__ __launch_bounds__(256) void gemm_i16i8_kernel(Gemm16Args g) {
     const int a_off = (wm * 64 + frow) * PITCH + fk, b_off = 2 * PLANE + (wn * 64 + frow) * PITCH + fk;
     const int ktiles = (g.K + BK - 1) / BK;
     load_tile(0);
+    const int round_path = park_col_params<BN>(eg, cp, tid, col_add, col_shift);  // contains barriers
     store_tile(0);
     __syncthreads();
     for (int kt = 0; kt < ktiles; ++kt) {
@@ -135,53 +170,17 @@ __global__ __launch_bounds__(256) void gemm_i16i8_kernel(Gemm16Args g) {
     }
 
     // epilogue: lane owns row lane%32 of each block and, per register quad q, columns 8q + 4*(lane/32) .. +3
-    const int lo_b = g.relu ? max(kind_lo(g.out_kind), 0) : kind_lo(g.out_kind), hi_b = kind_hi(g.out_kind);
-    const int obytes = (g.out_kind == A4G_I16 || g.out_kind == A4G_U16) ? 2 : 1;
-    // the tile leaves through an LDS image (the stages are dead: the loop ended on a barrier), then as whole rows
-    const int cpitch = BN * obytes + 16;
+    // a.w = 256 * sum(hi.w) + sum((lo - 128).w) + 128 * sum(w): the last term is in the column's addend. The tile
+    // leaves through the epilogue of the int8 kernels (the stages are dead: the loop ended on a barrier).
+    v16i sum[2][2];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int nl = wn * 64 + j * 32 + 8 * q + 4 * (lane >> 5);
-            const int n = n0 + nl;
-            unsigned add[4];
-            RoundCfg rc[4];
+        for (int j = 0; j < 2; ++j)
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                const int nn = min(n + t, g.N - 1);
-                add[t] = static_cast<unsigned>(g.bias ? g.bias[nn] : 0) + 128u * static_cast<unsigned>(g.colsum[nn]);
-                const int s = g.shifts ? g.shifts[static_cast<int64_t>(nn) * g.shift_stride] : g.shift;
-                rc[t] = make_round(g.mode, min(max(s, 0), 31));
-            }
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                const int ml = wm * 64 + i * 32 + (lane & 31);
-                int y[4];
-#pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    const unsigned a = (static_cast<unsigned>(acc_hi[i][j][q * 4 + t]) << 8) +
-                                       static_cast<unsigned>(acc_lo[i][j][q * 4 + t]) + add[t];
-                    y[t] = clamp_i(apply_round(static_cast<int>(a), rc[t]), lo_b, hi_b);
-                }
-                if (obytes == 1) {
-                    *reinterpret_cast<unsigned*>(smem + ml * cpitch + nl) = pack4_bytes(y[0], y[1], y[2], y[3]);
-                } else {
-                    v2i o = {static_cast<int>(pack2_halves(y[0], y[1])), static_cast<int>(pack2_halves(y[2], y[3]))};
-                    *reinterpret_cast<v2i*>(smem + ml * cpitch + nl * 2) = o;
-                }
-            }
-        }
-    }
-    __syncthreads();
-    GemmArgs img{};
-    img.C = g.Y;
-    img.ldc = g.ldy;
-    img.M = g.M;
-    img.N = g.N;
-    TileCoord here = tc;
-    here.batch = 0;  // select_problem has already moved the pointers to this problem
-    store_tile_image<BM, BN, 256>(img, here, smem, obytes, tid);
+            for (int r = 0; r < 16; ++r)
+                sum[i][j][r] = static_cast<int>((static_cast<unsigned>(acc_hi[i][j][r]) << 8) + static_cast<unsigned>(acc_lo[i][j][r]));
+    epilogue_store<BM, BN, 64, 64, 256>(eg, here, sum, smem, cp, round_path, wm, wn, lane, tid);
 }
 
 // Any K / alignment: one thread per output element.
@@ -247,6 +246,59 @@ __device__ __forceinline__ int requant64(long long v, int s, int mode, int lo, i
     return static_cast<int>(y < lo ? lo : (y > hi ? hi : y));
 }
 
+// The same rounding as one add before the shift, for the tiled kernels: v + c0, plus a tie term of -1, 0 or 1
+// that the mode takes from the sign of v or from bit s of v, then the shift and the saturation. c0 and en depend
+// on the column's shift and on the mode only; en is 0 where the shift is 0 (nothing to round) and -1 elsewhere.
+// |v| stays below 2^48 (K <= 32768) and c0 below 2^62, so the sum cannot overflow.
+struct Round64 {
+    long long c0;
+    int s, en;
+};
+
+__device__ __forceinline__ Round64 make_round64(int shift, int mode) {
+    Round64 r;
+    r.s = min(max(shift, 0), 62);
+    r.en = r.s > 0 ? -1 : 0;
+    const long long h = (1ll << r.s) >> 1;
+    switch (mode) {
+    case A4G_RND_FLOOR: r.c0 = 0; break;
+    case A4G_RND_CEIL: r.c0 = (1ll << r.s) - 1; break;
+    case A4G_RND_POSITIVE_INF:
+    case A4G_RND_SYMMETRIC_INF:
+    case A4G_RND_CONV_ODD: r.c0 = h; break;
+    default: r.c0 = h + r.en; break;  // ties go down unless the tie term says otherwise
+    }
+    return r;
+}
+
+template <int MODE>
+__device__ __forceinline__ int requant64_m(long long v, long long c0, int s, int en, int lo, int hi) {
+    long long t = v + c0;
+    if constexpr (MODE == A4G_RND_SYMMETRIC_INF) t += static_cast<int>(v >> 63) & en;   // below zero: h - 1
+    if constexpr (MODE == A4G_RND_SYMMETRIC_ZERO) t -= static_cast<int>(v >> 63) & en;  // below zero: h
+    if constexpr (MODE == A4G_RND_CONV_EVEN) t += static_cast<int>(v >> s) & 1 & en;
+    if constexpr (MODE == A4G_RND_CONV_ODD) t -= static_cast<int>(v >> s) & 1 & en;
+    const long long q = t >> s;
+    const int ql = static_cast<int>(q), qh = static_cast<int>(q >> 32);
+    const int y = qh == (ql >> 31) ? ql : ((qh >> 31) ^ 0x7fffffff);  // beyond 32 bits: the bound on q's side
+    return clamp_med3(y, lo, hi);
+}
+
+// Calls f with the rounding mode as a compile-time constant.
+template <typename F>
+__device__ __forceinline__ void with_round_mode(int mode, F&& f) {
+    switch (mode) {
+    case A4G_RND_FLOOR: f(std::integral_constant<int, A4G_RND_FLOOR>{}); break;
+    case A4G_RND_CEIL: f(std::integral_constant<int, A4G_RND_CEIL>{}); break;
+    case A4G_RND_POSITIVE_INF: f(std::integral_constant<int, A4G_RND_POSITIVE_INF>{}); break;
+    case A4G_RND_NEGATIVE_INF: f(std::integral_constant<int, A4G_RND_NEGATIVE_INF>{}); break;
+    case A4G_RND_SYMMETRIC_INF: f(std::integral_constant<int, A4G_RND_SYMMETRIC_INF>{}); break;
+    case A4G_RND_SYMMETRIC_ZERO: f(std::integral_constant<int, A4G_RND_SYMMETRIC_ZERO>{}); break;
+    case A4G_RND_CONV_EVEN: f(std::integral_constant<int, A4G_RND_CONV_EVEN>{}); break;
+    default: f(std::integral_constant<int, A4G_RND_CONV_ODD>{}); break;
+    }
+}
+
 // int16 x int16 on the software-pipelined kernel (K % 128 == 0, large problems). Both operands enter the tile as
 // byte planes: the activations are split while they are staged (runs of 64 tile rows alternate between the high
 // and the low plane of the same 64 rows), the weights come packed as two planes that alternate in 32-row blocks.
@@ -268,7 +320,9 @@ struct I16x16Policy {
     };
     struct Params {  // LDS: per output column of the tile, then per output row
         long long col_term[128];
+        long long c0[128];  // Round64 of the column's shift
         int shift[128];
+        int en[128];
         int row_sum[MAX_ROWS];
     };
     template <int BN>
@@ -311,11 +365,14 @@ struct I16x16Policy {
         }
     }
     template <int BN>
-    __device__ static __forceinline__ int park_params(const GemmArgs&, int8_t* lds, int tid, const ColRegs& r) {
+    __device__ static __forceinline__ int park_params(const GemmArgs& g, int8_t* lds, int tid, const ColRegs& r) {
         Params* p = reinterpret_cast<Params*>(lds);
         if (tid < BN / 2) {
+            const Round64 rr = make_round64(r.shift, g.mode);
             p->col_term[tid] = 128ll * r.colsum + r.bias;
-            p->shift[tid] = min(max(r.shift, 0), 62);
+            p->c0[tid] = rr.c0;
+            p->shift[tid] = rr.s;
+            p->en[tid] = rr.en;
         }
         return 0;
     }
@@ -338,37 +395,43 @@ struct I16x16Policy {
         const int lo_b = g.relu ? max(kind_lo(g.out_kind), 0) : kind_lo(g.out_kind), hi_b = kind_hi(g.out_kind);
         const int obytes = (g.out_kind == A4G_I16 || g.out_kind == A4G_U16) ? 2 : 1;
         const int cpitch = 128 * obytes + 16;
+        with_round_mode(g.mode, [&](auto mode_tag) {
+            constexpr int MODE = decltype(mode_tag)::value;
 #pragma unroll
-        for (int ri = 0; ri < 2; ++ri) {
-            const int ml = wm * 64 + ri * 32 + (lane & 31);  // output row within the tile
-            const long long row_term = 128ll * p->row_sum[ml];
+            for (int ri = 0; ri < 2; ++ri) {
+                const int ml = wm * 64 + ri * 32 + (lane & 31);  // output row within the tile
+                const long long row_term = 128ll * p->row_sum[ml];
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int nl = wn * 32 + 8 * q + 4 * (lane >> 5);
-                int y[4];
+                for (int q = 0; q < 4; ++q) {
+                    const int nl = wn * 32 + 8 * q + 4 * (lane >> 5);
+                    int y[4];
 #pragma unroll
-                for (int t = 0; t < 4; ++t) {
-                    const int r = 4 * q + t;
-                    const long long v = (static_cast<long long>(acc[ri][0][r]) << 16) +
-                                        ((static_cast<long long>(acc[ri][1][r]) + acc[ri + 2][0][r]) << 8) + acc[ri + 2][1][r] +
-                                        row_term + p->col_term[nl + t];
-                    y[t] = requant64(v, p->shift[nl + t], g.mode, lo_b, hi_b);
-                }
-                if (obytes == 1) {
-                    *reinterpret_cast<unsigned*>(smem + ml * cpitch + nl) = pack4_bytes(y[0], y[1], y[2], y[3]);
-                } else {
-                    v2i o = {static_cast<int>(pack2_halves(y[0], y[1])), static_cast<int>(pack2_halves(y[2], y[3]))};
-                    *reinterpret_cast<v2i*>(smem + ml * cpitch + nl * 2) = o;
+                    for (int t = 0; t < 4; ++t) {
+                        const int r = 4 * q + t;
+                        // hl + lh stays within 32 bits: each is at most K * 2^14 <= 2^29 in magnitude
+                        const long long v = static_cast<long long>(acc[ri][0][r]) * 65536 +
+                                            static_cast<long long>(acc[ri][1][r] + acc[ri + 2][0][r]) * 256 + acc[ri + 2][1][r] +
+                                            row_term + p->col_term[nl + t];
+                        y[t] = requant64_m<MODE>(v, p->c0[nl + t], p->shift[nl + t], p->en[nl + t], lo_b, hi_b);
+                    }
+                    if (obytes == 1) {
+                        *reinterpret_cast<unsigned*>(smem + ml * cpitch + nl) = pack4_bytes(y[0], y[1], y[2], y[3]);
+                    } else {
+                        v2i o = {static_cast<int>(pack2_halves(y[0], y[1])), static_cast<int>(pack2_halves(y[2], y[3]))};
+                        *reinterpret_cast<v2i*>(smem + ml * cpitch + nl * 2) = o;
+                    }
                 }
             }
-        }
+        });
         __syncthreads();
         store_tile_image<128, 128, NT>(g, tc, smem, obytes, tid);
     }
 };
 
 static bool rs_i16i16_applicable(const GemmArgs& g, int batch) {
-    return g.K % 128 == 0 && g.K >= 256 && g.K <= 32768 && g.lda % 16 == 0 && g.stride_a % 16 == 0 && g.ldb % 16 == 0 &&
+    // the pipelined kernel pays from K = 1024 on (3-10 % ahead of the tiled one; a few per cent behind at K <= 512),
+    // and only when the tile's 128 columns are mostly used (N = 64: 299 us against 229 us)
+    return g.K % 128 == 0 && g.K >= 1024 && g.N >= 192 && g.K <= 32768 && g.lda % 16 == 0 && g.stride_a % 16 == 0 && g.ldb % 16 == 0 &&
            g.stride_b % 16 == 0 && aligned16(g.A) && aligned16(g.Bt) && aligned16(g.Bt_lo) &&
            static_cast<int64_t>((g.M + 127) / 128) * ((g.N + 127) / 128) * batch >= 192;
 }
@@ -384,11 +447,12 @@ __device__ __forceinline__ void select_problem(Gemm16x16Args& g, int b) {
     g.Y = static_cast<int8_t*>(g.Y) + b * g.stride_y * obytes;
 }
 
-__global__ __launch_bounds__(256) void gemm_i16i16_kernel(Gemm16x16Args g) {
+__global__ __launch_bounds__(256, 2) void gemm_i16i16_kernel(Gemm16x16Args g) {
     constexpr int BM = 64, BN = 128, BK = 64, PITCH = BK + 16;
     select_problem(g, blockIdx.y);
     constexpr int APLANE = BM * PITCH, WPLANE = BN * PITCH, STAGE = 2 * APLANE + 2 * WPLANE;
-    __shared__ __attribute__((aligned(16))) int8_t smem[2 * STAGE];
+    static_assert(STAGE == TILED16_STAGE_BYTES, "the launch sizes the LDS");
+    extern __shared__ __attribute__((aligned(16))) int8_t smem[];  // two stages, or one when K fits a single tile
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
@@ -398,6 +462,21 @@ __global__ __launch_bounds__(256) void gemm_i16i16_kernel(Gemm16x16Args g) {
     const TileCoord tc = tile_coord<BM, BN>(shape);
     if (!tc.valid) return;
     const int m0 = tc.m0, n0 = tc.n0;
+
+    // per-column terms of the epilogue, parked in LDS while the first tile is on its way (the barriers of the
+    // main loop order the writes before the reads)
+    __shared__ struct {
+        long long col_term[BN], c0[BN];
+        int s[BN], en[BN];
+    } cp;
+    if (tid < BN) {
+        const int nn = min(n0 + tid, g.N - 1);
+        const Round64 rr = make_round64(g.shifts ? g.shifts[static_cast<int64_t>(nn) * g.shift_stride] : g.shift, g.mode);
+        cp.col_term[tid] = 128ll * g.colsum[nn] + (g.bias ? g.bias[nn] : 0);
+        cp.c0[tid] = rr.c0;
+        cp.s[tid] = rr.s;
+        cp.en[tid] = rr.en;
+    }
 
     // staging: A tile = 64 rows x 8 chunks of 8 int16 (2 per thread); each W plane = 128 rows x 4 chunks (2 per thread)
     v4i ra[2], rh[2], rl[2];
@@ -493,29 +572,32 @@ __global__ __launch_bounds__(256) void gemm_i16i16_kernel(Gemm16x16Args g) {
     // the tile leaves through an LDS image (the stages are dead: the loop ended on a barrier), then as whole rows
     const int cpitch = BN * obytes + 16;
     const int ml = wm * 32 + (lane & 31);
+    with_round_mode(g.mode, [&](auto mode_tag) {
+        constexpr int MODE = decltype(mode_tag)::value;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < 2; ++j) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int nl = wn * 64 + j * 32 + 8 * q + 4 * (lane >> 5);
-            int y[4];
+            for (int q = 0; q < 4; ++q) {
+                const int nl = wn * 64 + j * 32 + 8 * q + 4 * (lane >> 5);
+                int y[4];
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                const int nn = min(n0 + nl + t, g.N - 1);
-                const long long v = (static_cast<long long>(acc_hh[j][q * 4 + t]) << 16) +
-                                    ((static_cast<long long>(acc_hl[j][q * 4 + t]) + acc_lh[j][q * 4 + t]) << 8) +
-                                    acc_ll[j][q * 4 + t] + row_term + 128ll * g.colsum[nn] + (g.bias ? g.bias[nn] : 0);
-                const int s = min(max(g.shifts ? g.shifts[static_cast<int64_t>(nn) * g.shift_stride] : g.shift, 0), 62);
-                y[t] = requant64(v, s, g.mode, lo_b, hi_b);
-            }
-            if (obytes == 1) {
-                *reinterpret_cast<unsigned*>(smem + ml * cpitch + nl) = pack4_bytes(y[0], y[1], y[2], y[3]);
-            } else {
-                v2i o = {static_cast<int>(pack2_halves(y[0], y[1])), static_cast<int>(pack2_halves(y[2], y[3]))};
-                *reinterpret_cast<v2i*>(smem + ml * cpitch + nl * 2) = o;
+                for (int t = 0; t < 4; ++t) {
+                    const int r = q * 4 + t;
+                    // hl + lh stays within 32 bits: each is at most K * 2^14 <= 2^29 in magnitude
+                    const long long v = static_cast<long long>(acc_hh[j][r]) * 65536 +
+                                        static_cast<long long>(acc_hl[j][r] + acc_lh[j][r]) * 256 + acc_ll[j][r] + row_term +
+                                        cp.col_term[nl + t];
+                    y[t] = requant64_m<MODE>(v, cp.c0[nl + t], cp.s[nl + t], cp.en[nl + t], lo_b, hi_b);
+                }
+                if (obytes == 1) {
+                    *reinterpret_cast<unsigned*>(smem + ml * cpitch + nl) = pack4_bytes(y[0], y[1], y[2], y[3]);
+                } else {
+                    v2i o = {static_cast<int>(pack2_halves(y[0], y[1])), static_cast<int>(pack2_halves(y[2], y[3]))};
+                    *reinterpret_cast<v2i*>(smem + ml * cpitch + nl * 2) = o;
+                }
             }
         }
-    }
+    });
     __syncthreads();
     GemmArgs img{};
     img.C = g.Y;
@@ -558,14 +640,17 @@ __global__ __launch_bounds__(256) void gemm_i16i16_generic_kernel(Gemm16x16Args 
 template <bool WIDE>
 __global__ __launch_bounds__(256) void pack_rhs_kernel(const void* __restrict__ B, int64_t ldb, int64_t stride_b, int trans_b,
                                                        int8_t* __restrict__ hi, int8_t* __restrict__ lo, int64_t ldt,
-                                                       int64_t stride_t, int32_t* __restrict__ colsum, int K, int N) {
+                                                       int64_t stride_t, int32_t* __restrict__ colsum, int K, int N, int kspan) {
     __shared__ short tile[64][66];  // [k][n]
     const int tid = threadIdx.x, b = blockIdx.y, n0 = blockIdx.x * 64;
+    // blockIdx.z picks a run of kspan (a multiple of 64) values of k; with more than one run the column sums are
+    // added into a zeroed array
+    const int k_begin = blockIdx.z * kspan, k_end = min(static_cast<int>(ldt), k_begin + kspan);
     const int kq = tid & 15;
     // an element past the edge packs to zero bytes and adds nothing to the sum: 128 has high byte 0 and low byte 0x80
     const short pad = WIDE ? 128 : 0;
     int col_acc[4] = {0, 0, 0, 0};
-    for (int k0 = 0; k0 < ldt; k0 += 64) {
+    for (int k0 = k_begin; k0 < k_end; k0 += 64) {
         for (int i = tid; i < 64 * 64; i += 256) {
             const int kk = trans_b ? (i & 63) : (i >> 6), nn = trans_b ? (i >> 6) : (i & 63);
             const int k = k0 + kk, n = n0 + nn;
@@ -606,8 +691,33 @@ __global__ __launch_bounds__(256) void pack_rhs_kernel(const void* __restrict__ 
         v += __shfl_xor(v, 4);
         v += __shfl_xor(v, 8);
         const int n = n0 + (tid >> 4) + 16 * j;
-        if (kq == 0 && n < N) colsum[static_cast<int64_t>(b) * N + n] = v;
+        if (kq == 0 && n < N) {
+            if (gridDim.z == 1) colsum[static_cast<int64_t>(b) * N + n] = v;
+            else atomicAdd(colsum + static_cast<int64_t>(b) * N + n, v);
+        }
     }
+}
+
+__global__ __launch_bounds__(256) void zero_i32_kernel(int32_t* __restrict__ p, int64_t n) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i < n) p[i] = 0;
+}
+
+// Launches the pack with K split into enough runs to give every CU several workgroups.
+static hipError_t launch_pack_rhs(bool wide, const void* B, int64_t ldb, int64_t stride_b, int trans_b, int8_t* hi, int8_t* lo,
+                                  int64_t ldt, int64_t stride_t, int32_t* colsum, int64_t batch, int K, int N, hipStream_t stream) {
+    const int64_t groups = (N + 63) / 64 * batch, ktiles = (ldt + 63) / 64;
+    int64_t runs = std::min<int64_t>(ktiles, std::max<int64_t>(1, 2048 / groups));
+    const int kspan = static_cast<int>((ktiles + runs - 1) / runs) * 64;
+    runs = (ldt + kspan - 1) / kspan;
+    if (runs > 1) {
+        const int64_t n = batch * N;
+        zero_i32_kernel<<<static_cast<unsigned>((n + 255) / 256), 256, 0, stream>>>(colsum, n);
+    }
+    const dim3 grid(static_cast<unsigned>((N + 63) / 64), static_cast<unsigned>(batch), static_cast<unsigned>(runs));
+    if (wide) pack_rhs_kernel<true><<<grid, 256, 0, stream>>>(B, ldb, stride_b, trans_b, hi, lo, ldt, stride_t, colsum, K, N, kspan);
+    else pack_rhs_kernel<false><<<grid, 256, 0, stream>>>(B, ldb, stride_b, trans_b, hi, lo, ldt, stride_t, colsum, K, N, kspan);
+    return hipGetLastError();
 }
 
 }  // namespace a4g
@@ -651,7 +761,7 @@ extern "C" int a4g_dense_i16(const int16_t* A, int64_t lda, const int8_t* Wt, in
     if (tiled) {
         const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
         A4G_REQUIRE(tiles <= INT32_MAX, A4G_ERR_UNSUPPORTED, "%s: too many tiles", who);
-        gemm_i16i8_kernel<<<dim3(static_cast<unsigned>((tiles + 7) / 8 * 8), 1), 256, 0, stream>>>(g);  // whole ranges for the 8 XCDs
+        gemm_i16i8_kernel<<<dim3(static_cast<unsigned>((tiles + 7) / 8 * 8), 1), 256, tiled16_lds_bytes(g.K, 128), stream>>>(g);  // whole ranges for the 8 XCDs
     } else {
         const int grid = static_cast<int>(std::min<int64_t>((M * N + 255) / 256, 256 * 32));
         gemm_i16i8_generic_kernel<<<grid, 256, 0, stream>>>(g);
@@ -667,9 +777,8 @@ extern "C" int a4g_pack_weights_i16(const int16_t* W, int64_t ldw, int64_t K, in
     A4G_REQUIRE(K >= 1 && N >= 1 && K <= 32768 && N <= (1 << 24) && ldw >= N, A4G_ERR_INVALID_ARGUMENT,
                 "%s: bad shape K=%lld (at most 32768) N=%lld ldw=%lld", who, (long long)K, (long long)N, (long long)ldw);
     const int64_t ldt = K <= 0 ? 16 : (K + 15) / 16 * 16;
-    pack_rhs_kernel<true><<<dim3(static_cast<unsigned>((N + 63) / 64), 1), 256, 0, stream>>>(W, ldw, 0, 0, Wt_hi, Wt_lo, ldt, 0, colsum,
-                                                                                             static_cast<int>(K), static_cast<int>(N));
-    return check_hip(hipGetLastError(), who);
+    return check_hip(launch_pack_rhs(true, W, ldw, 0, 0, Wt_hi, Wt_lo, ldt, 0, colsum, 1, static_cast<int>(K), static_cast<int>(N), stream),
+                     who);
 }
 
 extern "C" int a4g_dense_i16x16(const int16_t* A, int64_t lda, const int8_t* Wt_hi, const int8_t* Wt_lo, int64_t ldwt,
@@ -710,7 +819,7 @@ extern "C" int a4g_dense_i16x16(const int16_t* A, int64_t lda, const int8_t* Wt_
     if (tiled) {
         const int64_t tiles = ((M + 63) / 64) * ((N + 127) / 128);
         A4G_REQUIRE(tiles <= INT32_MAX, A4G_ERR_UNSUPPORTED, "%s: too many tiles", who);
-        gemm_i16i16_kernel<<<dim3(static_cast<unsigned>((tiles + 7) / 8 * 8), 1), 256, 0, stream>>>(g);
+        gemm_i16i16_kernel<<<dim3(static_cast<unsigned>((tiles + 7) / 8 * 8), 1), 256, tiled16_lds_bytes(g.K, 64), stream>>>(g);
     } else {
         const int grid = static_cast<int>(std::min<int64_t>((M * N + 255) / 256, 256 * 32));
         gemm_i16i16_generic_kernel<<<grid, 256, 0, stream>>>(g);
@@ -753,12 +862,7 @@ extern "C" int a4g_matmul_i16(const int16_t* A, int64_t lda, int64_t stride_a, c
     int8_t* hi = static_cast<int8_t*>(workspace);
     int8_t* lo = wide ? hi + batch * N * ldt : nullptr;
     int32_t* colsum = reinterpret_cast<int32_t*>(hi + (wide ? 2 : 1) * batch * N * ldt);
-    const dim3 pgrid(static_cast<unsigned>((N + 63) / 64), static_cast<unsigned>(batch));
-    if (wide)
-        pack_rhs_kernel<true><<<pgrid, 256, 0, stream>>>(B, ldb, stride_b, trans_b, hi, lo, ldt, N * ldt, colsum, (int)K, (int)N);
-    else
-        pack_rhs_kernel<false><<<pgrid, 256, 0, stream>>>(B, ldb, stride_b, trans_b, hi, lo, ldt, N * ldt, colsum, (int)K, (int)N);
-    hipError_t e = hipGetLastError();
+    hipError_t e = launch_pack_rhs(wide, B, ldb, stride_b, trans_b, hi, lo, ldt, N * ldt, colsum, batch, (int)K, (int)N, stream);
     if (e != hipSuccess) return check_hip(e, who);
 
     const bool tiled = K % 16 == 0 && lda % 8 == 0 && stride_a % 8 == 0 && aligned16(A);
@@ -780,7 +884,7 @@ extern "C" int a4g_matmul_i16(const int16_t* A, int64_t lda, int64_t stride_a, c
             return check_hip(launch_rs_policy<I16x16Policy, 256, 256, 2, 4, true>(r, nb, stream), who);
         if (tiled) {
             const int64_t tiles = ((M + 63) / 64) * ((N + 127) / 128);
-            gemm_i16i16_kernel<<<dim3(static_cast<unsigned>((tiles + 7) / 8 * 8), nb), 256, 0, stream>>>(g);
+            gemm_i16i16_kernel<<<dim3(static_cast<unsigned>((tiles + 7) / 8 * 8), nb), 256, tiled16_lds_bytes(g.K, 64), stream>>>(g);
         } else {
             const int grid = static_cast<int>(std::min<int64_t>((M * N + 255) / 256, 256 * 32));
             gemm_i16i16_generic_kernel<<<dim3(grid, nb), 256, 0, stream>>>(g);
@@ -801,7 +905,7 @@ extern "C" int a4g_matmul_i16(const int16_t* A, int64_t lda, int64_t stride_a, c
         if (rs_i16i8_applicable(r, nb)) return check_hip(launch_rs_i16i8(r, nb, stream), who);
         if (tiled) {
             const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
-            gemm_i16i8_kernel<<<dim3(static_cast<unsigned>((tiles + 7) / 8 * 8), nb), 256, 0, stream>>>(g);
+            gemm_i16i8_kernel<<<dim3(static_cast<unsigned>((tiles + 7) / 8 * 8), nb), 256, tiled16_lds_bytes(g.K, 128), stream>>>(g);
         } else {
             const int grid = static_cast<int>(std::min<int64_t>((M * N + 255) / 256, 256 * 32));
             gemm_i16i8_generic_kernel<<<dim3(grid, nb), 256, 0, stream>>>(g);

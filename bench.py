@@ -201,7 +201,7 @@ def main():
         cpu_fn = lambda: oracle.dense(A[:sample_rows], W, bias, shifts, 'conv_even', relu=True, out='int16')  # noqa: E731
         cpu_work = 2.0 * sample_rows * N * K
         metric, unit = 'int16x16_dense_tops', 'TOP/s'
-        kernel = 'gemm_i16i16_kernel'
+        kernel = 'gemm_rs_kernel'
     elif wl in ('c2_dense_bf16', 'c2_dense_fp8'):
         # the reference's float compute path on the C2 shape: bfloat16 / fp8 e4m3 operands, float32 accumulation and bias
         M, K, N = 8192, 4096, 4096

@@ -246,11 +246,12 @@ def test_dense_int16_activations(ops, oracle, shape):
     assert np.array_equal(got, oracle.dense(np.abs(A), np.abs(W), big, 16, 'conv_even', out='int16'))
 
 
-@pytest.mark.parametrize('shape', [(2085, 3000, 256), (4096, 1536, 384)])
+@pytest.mark.parametrize('shape', [(2085, 3000, 1024), (4096, 1536, 1152), (2085, 3000, 256)])
 def test_dense_int16_activations_large(ops, oracle, shape):
-    """Problems with whole 128-element K tiles and at least 192 tiles of 128 x 256 take the software-pipelined kernel
-    that splits the activations into byte planes while staging them: ragged M and N, every rounding mode, the three
-    output kinds, rows at the int16 extremes, a bias that makes the 32-bit accumulator wrap."""
+    """Problems with K >= 1024 in whole 128-element tiles and at least 192 tiles of 128 x 256 take the software-pipelined
+    kernel that splits the activations into byte planes while staging them, the last shape the tiled one: ragged M and
+    N, every rounding mode, the three output kinds, rows at the int16 extremes, a bias that makes the 32-bit
+    accumulator wrap."""
     M, N, K = shape
     r = rng(M + N + K)
     A = r.integers(-32768, 32768, (M, K)).astype(np.int16)
@@ -300,11 +301,12 @@ def test_dense_int16_activations_int16_weights(ops, oracle, shape):
         ops.dense(dev(A.astype(np.int8)), p, 'floor')
 
 
-@pytest.mark.parametrize('shape', [(2085, 3000, 256), (1024, 3072, 640)])
+@pytest.mark.parametrize('shape', [(2085, 3000, 1024), (1024, 3072, 1152), (1024, 3072, 640)])
 def test_dense_int16x16_large(ops, oracle, shape):
-    """int16 x int16 problems with whole 128-element K tiles and at least 192 output tiles of 128 x 128 take the
-    software-pipelined kernel (both operands as byte planes in one tile, row sums gathered while the activations
-    are split): ragged edges, every rounding mode, extreme rows and columns, all three output kinds."""
+    """int16 x int16 problems with K >= 1024 in whole 128-element tiles and at least 192 output tiles of 128 x 128 take
+    the software-pipelined kernel (both operands as byte planes in one tile, row sums gathered while the activations
+    are split), the last shape the tiled one: ragged edges, every rounding mode, extreme rows and columns, all three
+    output kinds."""
     M, N, K = shape
     r = rng(M + N + K)
     A = r.integers(-32768, 32768, (M, K)).astype(np.int16)
@@ -331,7 +333,7 @@ def test_dense_int16x16_large(ops, oracle, shape):
 @pytest.mark.parametrize('b_dtype', [np.int8, np.int16])
 @pytest.mark.parametrize('trans_b', [True, False])
 @pytest.mark.parametrize('shape', [((2, 3), 64, 64, 64), ((4,), 130, 96, 48), ((), 70, 17, 24), ((2,), 128, 256, 512),
-                                   ((3,), 1100, 2000, 256)])
+                                   ((3,), 1100, 2000, 256), ((3,), 1100, 2000, 1024), ((1,), 300, 200, 4096)])
 def test_matmul_int16_left_operand(ops, oracle, shape, trans_b, b_dtype):
     # the 16-bit width combinations of the dynamic MatMul: int16 x int8 (acc32) and int16 x int16 (acc64)
     lead, M, N, K = shape
