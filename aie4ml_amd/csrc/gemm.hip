@@ -43,7 +43,7 @@ struct GemmCfg {
     static_assert(WTM % 32 == 0 && WTN % 32 == 0 && BK % 32 == 0, "wave tile must be whole 32x32x32 MFMA blocks");
 };
 
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool RAGGED = false>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_i8_nt_kernel(GemmArgs g) {
     using Cfg = GemmCfg<BM, BN, BK, WAVES_M, WAVES_N>;
     extern __shared__ __attribute__((aligned(16))) int8_t smem[];
@@ -102,12 +102,19 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_i8_nt_kernel(GemmA
     }
 
     auto load_tile = [&](int k0) {
+        if constexpr (RAGGED) {
 #pragma unroll
-        for (int i = 0; i < Cfg::A_PER_T; ++i)
-            ra[i] = (k0 + ka[i] < g.K) ? *reinterpret_cast<const v4i*>(pa[i] + k0) : v4i{0, 0, 0, 0};
+            for (int i = 0; i < Cfg::A_PER_T; ++i) ra[i] = load_chunk_ragged(pa[i] + k0, g.K - (k0 + ka[i]), g.ragged_a);
 #pragma unroll
-        for (int i = 0; i < Cfg::B_PER_T; ++i)
-            rb[i] = (k0 + kb[i] < g.K) ? *reinterpret_cast<const v4i*>(pb[i] + k0) : v4i{0, 0, 0, 0};
+            for (int i = 0; i < Cfg::B_PER_T; ++i) rb[i] = load_chunk_ragged(pb[i] + k0, g.K - (k0 + kb[i]), g.ragged_b);
+        } else {
+#pragma unroll
+            for (int i = 0; i < Cfg::A_PER_T; ++i)
+                ra[i] = (k0 + ka[i] < g.K) ? *reinterpret_cast<const v4i*>(pa[i] + k0) : v4i{0, 0, 0, 0};
+#pragma unroll
+            for (int i = 0; i < Cfg::B_PER_T; ++i)
+                rb[i] = (k0 + kb[i] < g.K) ? *reinterpret_cast<const v4i*>(pb[i] + k0) : v4i{0, 0, 0, 0};
+        }
     };
     auto store_tile = [&](int buf) {
 #pragma unroll
@@ -487,34 +494,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_i8_dtl_kernel(Gemm
 
 
 // -----------------------------------------------------------------------------------------------------
-// Generic kernel: any shape / pitch / alignment; one thread per output element.
-// trans_b == 1: B is [N][ldb]; trans_b == 0: B is [K][ldb].
-// -----------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void gemm_generic_kernel(GemmArgs g, int trans_b) {
-    const int64_t total = static_cast<int64_t>(g.M) * g.N;
-    const int batch = blockIdx.y;
-    const int8_t* Ab = g.A + batch * g.stride_a;
-    const int8_t* Bb = g.Bt + batch * g.stride_b;
-    const int obytes = (g.out_kind == A4G_I16 || g.out_kind == A4G_U16) ? 2 : 1;
-    int8_t* Cb = static_cast<int8_t*>(g.C) + batch * g.stride_c * obytes;
-    const int lo = g.relu ? max(kind_lo(g.out_kind), 0) : kind_lo(g.out_kind), hi = kind_hi(g.out_kind);
-    for (int64_t idx = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; idx < total;
-         idx += static_cast<int64_t>(gridDim.x) * blockDim.x) {
-        const int m = static_cast<int>(idx / g.N), n = static_cast<int>(idx % g.N);
-        unsigned acc = g.bias ? static_cast<unsigned>(g.bias[n]) : 0u;
-        const int8_t* ar = Ab + static_cast<int64_t>(m) * g.lda;
-        for (int k = 0; k < g.K; ++k) {
-            const int a = g.a_unsigned ? static_cast<int>(static_cast<uint8_t>(ar[k])) : static_cast<int>(ar[k]);
-            const int b = trans_b ? Bb[static_cast<int64_t>(n) * g.ldb + k] : Bb[static_cast<int64_t>(k) * g.ldb + n];
-            acc += static_cast<unsigned>(a * b);
-        }
-        const int y = requant(static_cast<int>(acc), make_round(g.mode, column_shift(g, n)), lo, hi);
-        if (obytes == 1) Cb[static_cast<int64_t>(m) * g.ldc + n] = static_cast<int8_t>(y);
-        else reinterpret_cast<int16_t*>(Cb)[static_cast<int64_t>(m) * g.ldc + n] = static_cast<int16_t>(y);
-    }
-}
-
-// -----------------------------------------------------------------------------------------------------
 // Right-hand-side preparation: [K][ldb] -> [N][ldt] (zero padded to ldt) and column sums.
 // -----------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void transpose_kn_kernel(const int8_t* __restrict__ B, int64_t ldb, int64_t stride_b,
@@ -564,10 +543,10 @@ __global__ __launch_bounds__(256) void colsum_kernel(const int8_t* __restrict__ 
 
 static inline int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
 
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N>
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool RAGGED = false>
 static hipError_t launch_tiled(const GemmArgs& g, int batch, hipStream_t stream) {
     using Cfg = GemmCfg<BM, BN, BK, WAVES_M, WAVES_N>;
-    auto kern = gemm_i8_nt_kernel<BM, BN, BK, WAVES_M, WAVES_N>;
+    auto kern = gemm_i8_nt_kernel<BM, BN, BK, WAVES_M, WAVES_N, RAGGED>;
     static bool attr_set = false;  // benign race: the attribute is idempotent
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -678,6 +657,13 @@ static int env_variant() {
     return v;
 }
 
+// Shapes outside the aligned kernels' requirements: same tiles, chunk loads that respect the row ends.
+static hipError_t launch_ragged(GemmArgs g, int batch, hipStream_t stream) {
+    g.ragged_a = ragged_mode(g.A, g.lda, g.stride_a, g.K);
+    g.ragged_b = ragged_mode(g.Bt, g.ldb, g.stride_b, g.K);
+    return launch_tiled<128, 128, 64, 2, 2, true>(g, batch, stream);
+}
+
 static bool out_kind_ok(int k) { return k == A4G_I8 || k == A4G_U8 || k == A4G_I16; }
 
 }  // namespace a4g
@@ -746,10 +732,7 @@ extern "C" int a4g_dense_i8(const void* A, int a_kind, int64_t lda, const int8_t
     if (tiled) {
         e = launch_gemm_nt(g, 1, stream, env_variant());
     } else {
-        const int64_t total = M * N;
-        const int grid = static_cast<int>(std::min<int64_t>((total + 255) / 256, 256 * 32));
-        gemm_generic_kernel<<<dim3(grid, 1), 256, 0, stream>>>(g, 1);
-        e = hipGetLastError();
+        e = launch_ragged(g, 1, stream);
     }
     return check_hip(e, who);
 }
@@ -844,25 +827,16 @@ extern "C" int a4g_matmul_i8(const void* A, int a_kind, int64_t lda, int64_t str
         if (a_ok && ldb % 16 == 0 && stride_b % 16 == 0 && aligned16(B)) {
             e = launch_gemm_nt(g, static_cast<int>(batch), stream, env_variant());
         } else {
-            const int grid = static_cast<int>(std::min<int64_t>((M * N + 255) / 256, 256 * 32));
-            gemm_generic_kernel<<<dim3(grid, static_cast<unsigned>(batch)), 256, 0, stream>>>(g, 1);
-            e = hipGetLastError();
+            e = launch_ragged(g, static_cast<int>(batch), stream);
         }
-    } else if (a_ok) {
+    } else {
         dim3 tg(static_cast<unsigned>((ldt + 63) / 64), static_cast<unsigned>((N + 63) / 64), static_cast<unsigned>(batch));
         transpose_kn_kernel<<<tg, 256, 0, stream>>>(B, ldb, stride_b, ws, ldt, N * ldt, static_cast<int>(K),
                                                     static_cast<int>(N));
         g.Bt = ws;
         g.ldb = ldt;
         g.stride_b = N * ldt;
-        e = launch_gemm_nt(g, static_cast<int>(batch), stream, env_variant());
-    } else {
-        g.Bt = B;
-        g.ldb = ldb;
-        g.stride_b = stride_b;
-        const int grid = static_cast<int>(std::min<int64_t>((M * N + 255) / 256, 256 * 32));
-        gemm_generic_kernel<<<dim3(grid, static_cast<unsigned>(batch)), 256, 0, stream>>>(g, 0);
-        e = hipGetLastError();
+        e = a_ok ? launch_gemm_nt(g, static_cast<int>(batch), stream, env_variant()) : launch_ragged(g, static_cast<int>(batch), stream);
     }
     return check_hip(e, who);
 }

@@ -148,37 +148,6 @@ struct FloatPolicy {
     }
 };
 
-// Any shape / pitch / alignment: one thread per output element, float32 accumulation in k order starting
-// from the bias. lda / ldb / K here are in elements. trans_b == 1: B is [N][ldb]; 0: B is [K][ldb].
-struct FloatGenericArgs {
-    const void *A, *B;
-    void* C;
-    const float* bias;
-    int64_t lda, stride_a, ldb, stride_b, ldc, stride_c;
-    int M, N, K, relu, fmt, trans_b;
-};
-
-__global__ __launch_bounds__(256) void gemm_float_generic_kernel(FloatGenericArgs g) {
-    const int64_t total = static_cast<int64_t>(g.M) * g.N;
-    const int batch = blockIdx.y;
-    const int es = g.fmt == A4G_F32 ? 4 : (g.fmt == A4G_FP8 ? 1 : 2);
-    const char* A = static_cast<const char*>(g.A) + batch * g.stride_a * es;
-    const char* B = static_cast<const char*>(g.B) + batch * g.stride_b * es;
-    char* C = static_cast<char*>(g.C) + batch * g.stride_c * es;
-    for (int64_t idx = blockIdx.x * 256ll + threadIdx.x; idx < total; idx += static_cast<int64_t>(gridDim.x) * 256) {
-        const int m = static_cast<int>(idx / g.N), n = static_cast<int>(idx % g.N);
-        float acc = g.bias ? g.bias[n] : 0.f;
-        for (int k = 0; k < g.K; ++k) {
-            const float a = load_float(A, static_cast<int64_t>(m) * g.lda + k, g.fmt);
-            const float b = g.trans_b ? load_float(B, static_cast<int64_t>(n) * g.ldb + k, g.fmt)
-                                      : load_float(B, static_cast<int64_t>(k) * g.ldb + n, g.fmt);
-            acc = fmaf(a, b, acc);
-        }
-        if (g.relu) acc = fmaxf(acc, 0.f);
-        store_float(C, static_cast<int64_t>(m) * g.ldc + n, g.fmt, acc);
-    }
-}
-
 // [K][ldb] -> [N][ldt] for 2- or 4-byte elements, 32 x 32 tiles through LDS; columns K..ldt-1 are zero filled.
 template <typename T>
 __global__ __launch_bounds__(256) void transpose_elems_kernel(const T* __restrict__ B, int64_t ldb, int64_t stride_b,
@@ -213,13 +182,6 @@ static hipError_t launch_float_nt(const void* A, int64_t lda, int64_t stride_a, 
     const int es = fmt_bytes(fmt);
     const bool tiled = (static_cast<int64_t>(K) * es) % 128 == 0 && (lda * es) % 16 == 0 && (ldb * es) % 16 == 0 &&
                        (stride_a * es) % 16 == 0 && (stride_b * es) % 16 == 0 && aligned16(A) && aligned16(Bt);
-    if (!tiled) {
-        FloatGenericArgs ga{A, Bt, C, bias, lda, stride_a, ldb, stride_b, ldc, stride_c, M, N, K, relu, fmt, 1};
-        const int64_t total = static_cast<int64_t>(M) * N;
-        const int grid = static_cast<int>(std::min<int64_t>((total + 255) / 256, 256 * 32));
-        gemm_float_generic_kernel<<<dim3(grid, batch), 256, 0, stream>>>(ga);
-        return hipGetLastError();
-    }
     GemmArgs g{};
     g.A = static_cast<const int8_t*>(A);
     g.Bt = static_cast<const int8_t*>(Bt);
@@ -235,6 +197,14 @@ static hipError_t launch_float_nt(const void* A, int64_t lda, int64_t stride_a, 
     g.N = N;
     g.K = K * es;
     g.relu = relu != 0;
+    if (!tiled) {
+        // K that does not fill its last 128-byte tile, unaligned rows: the same kernel with loads that respect the row ends
+        g.ragged_a = ragged_mode(g.A, g.lda, g.stride_a, g.K);
+        g.ragged_b = ragged_mode(g.Bt, g.ldb, g.stride_b, g.K);
+        if (fmt == A4G_F32) return launch_rs_policy<FloatPolicy<A4G_F32>, 128, 128, 2, 2, false, true>(g, batch, stream);
+        if (fmt == A4G_FP8) return launch_rs_policy<FloatPolicy<A4G_FP8>, 128, 128, 2, 2, false, true>(g, batch, stream);
+        return launch_rs_policy<FloatPolicy<A4G_BF16>, 128, 128, 2, 2, false, true>(g, batch, stream);
+    }
     if (fmt == A4G_F32) return launch_rs_policy<FloatPolicy<A4G_F32>, 128, 128, 2, 2>(g, batch, stream);
     const int64_t tiles256 = static_cast<int64_t>((M + 255) / 256) * ((N + 255) / 256) * batch;
     const int64_t rounds256 = (tiles256 + 255) / 256;

@@ -61,6 +61,9 @@ struct GemmArgs {
     int out_kind;
     int mode;
     const int8_t* Bt_lo;    // second byte plane of B^T (policies with SPLIT_B), same pitch and strides as Bt
+    // only read by the ragged form of the tiled int8 kernel: how a 16-byte chunk of an operand row may be fetched
+    // (0 = one aligned load inside the row pitch, 1 = dwords, 2 = bytes); bytes at or past K always read as zero
+    int ragged_a, ragged_b;
 };
 
 struct TileCoord {
@@ -169,7 +172,49 @@ struct RsCfg {
                   "plane split: a wave's rows must hold whole high/low runs");
 };
 
-template <class P, int BM, int BN, int WAVES_M, int WAVES_N, bool EARLY = false>
+// One 16-byte chunk of an operand row for shapes the aligned kernels cannot take (K not a multiple of 16, rows that
+// are not 16-byte aligned): `rem` of its bytes belong to the row's K values, the rest read as zero, and no byte
+// past the end of the row's pitch is touched. mode 0: the chunk is aligned and lies inside the pitch; mode 1: rows
+// are 4-byte aligned with a pitch that is a multiple of 4; mode 2: neither.
+__device__ __forceinline__ v4i load_chunk_ragged(const int8_t* p, int rem, int mode) {
+    v4i r = {0, 0, 0, 0};
+    if (rem <= 0) return r;
+    if (mode == 0) {
+        r = *reinterpret_cast<const v4i*>(p);
+    } else if (mode == 1) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (4 * j < rem) r[j] = *reinterpret_cast<const int*>(p + 4 * j);
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            unsigned w = 0;
+#pragma unroll
+            for (int b = 0; b < 4; ++b)
+                if (4 * j + b < rem) w |= static_cast<unsigned>(static_cast<uint8_t>(p[4 * j + b])) << (8 * b);
+            r[j] = static_cast<int>(w);
+        }
+    }
+    if (rem < 16) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int v = rem - 4 * j;  // valid bytes of this dword
+            if (v <= 0) r[j] = 0;
+            else if (v < 4) r[j] &= static_cast<int>((1u << (8 * v)) - 1u);
+        }
+    }
+    return r;
+}
+
+// How the ragged kernels may fetch 16-byte chunks of an operand's rows (see load_chunk_ragged).
+static inline int ragged_mode(const void* p, int64_t ld, int64_t stride, int64_t K) {
+    const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+    if (ld % 16 == 0 && stride % 16 == 0 && a % 16 == 0 && ld >= (K + 15) / 16 * 16) return 0;
+    if (ld % 4 == 0 && stride % 4 == 0 && a % 4 == 0) return 1;
+    return 2;
+}
+
+template <class P, int BM, int BN, int WAVES_M, int WAVES_N, bool EARLY = false, bool RAGGED = false>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs g) {
     using Cfg = RsCfg<P, BM, BN, WAVES_M, WAVES_N>;
     constexpr int BK = Cfg::BK, KSTEPS = Cfg::KSTEPS;
@@ -213,6 +258,14 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
 
     v4i ra[Cfg::A_LOADS], rb[Cfg::B_LOADS];
     auto load_one = [&](int kt, int idx) {
+        if constexpr (RAGGED) {
+            // K (bytes here) need not fill its last tile and rows need not be aligned: bytes past K read as zero
+            static_assert(!RAGGED || (!P::SPLIT_A && !P::SPLIT_B), "the ragged loads serve the unsplit policies");
+            const int rem = g.K - (kt * BK + lchunk * 16);
+            if (idx < Cfg::A_LOADS) ra[idx] = load_chunk_ragged(Abase + offa[idx] + static_cast<int64_t>(kt) * BK, rem, g.ragged_a);
+            else rb[idx - Cfg::A_LOADS] = load_chunk_ragged(Bbase + offb[idx - Cfg::A_LOADS] + static_cast<int64_t>(kt) * BK, rem, g.ragged_b);
+            return;
+        }
         if (idx < Cfg::A_LOADS) ra[idx] = *reinterpret_cast<const v4i*>(Abase + offa[idx] + static_cast<int64_t>(kt) * (P::SPLIT_A ? 2 * BK : BK));
         else rb[idx - Cfg::A_LOADS] = *reinterpret_cast<const v4i*>(Bbase + offb[idx - Cfg::A_LOADS] + static_cast<int64_t>(kt) * BK);
     };
@@ -225,7 +278,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
         else *reinterpret_cast<v4i*>(stage + BM * BK + st_off + (idx - Cfg::A_LOADS) * Cfg::ROWS_PER_PASS * BK) = rb[idx - Cfg::A_LOADS];
     };
 
-    const int ktiles = g.K / BK;
+    const int ktiles = RAGGED ? (g.K + BK - 1) / BK : g.K / BK;
 #pragma unroll
     for (int i = 0; i < Cfg::LOADS; ++i) load_one(0, i);
 
@@ -364,10 +417,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
 }
 
 // Launches one workgroup per tile (padded to whole ranges for the 8 XCDs; surplus workgroups exit at once).
-template <class P, int BM, int BN, int WAVES_M, int WAVES_N, bool EARLY = false>
+template <class P, int BM, int BN, int WAVES_M, int WAVES_N, bool EARLY = false, bool RAGGED = false>
 static hipError_t launch_rs_policy(const GemmArgs& g, int batch, hipStream_t stream) {
     using Cfg = RsCfg<P, BM, BN, WAVES_M, WAVES_N>;
-    auto kern = gemm_rs_kernel<P, BM, BN, WAVES_M, WAVES_N, EARLY>;
+    auto kern = gemm_rs_kernel<P, BM, BN, WAVES_M, WAVES_N, EARLY, RAGGED>;
     static bool attr_set = false;  // benign race: the attribute is idempotent
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
