@@ -42,6 +42,7 @@ struct Gemm16Args {
     // batched use (dynamic MatMul): element strides between consecutive problems, blockIdx.y = problem
     int64_t stride_a, stride_w, stride_colsum, stride_y;
     int shift;  // used when `shifts` is null (MatMul: one host-side shift)
+    int ragged_a;  // RAGGED kernels: how chunks of A's rows may be fetched (load_chunk_ragged)
 };
 
 // 128 x 128 output tile, K step 64, 4 waves (2 x 2) of 64 x 64, double-buffered LDS holding the two byte
@@ -54,6 +55,8 @@ __device__ __forceinline__ void select_problem(Gemm16Args& g, int b) {
     g.Y = static_cast<int8_t*>(g.Y) + b * g.stride_y * obytes;
 }
 
+// RAGGED: K need not be a multiple of 16 nor A's rows 16-byte aligned (the packed weights always are, zero padded).
+template <bool RAGGED>
 __global__ __launch_bounds__(256, 2) void gemm_i16i8_kernel(Gemm16Args g) {
     constexpr int BM = 128, BN = 128, BK = 64, PITCH = BK + 16;
     select_problem(g, blockIdx.y);
@@ -98,8 +101,12 @@ __global__ __launch_bounds__(256, 2) void gemm_i16i8_kernel(Gemm16Args g) {
         for (int i = 0; i < 4; ++i) {
             const int c = tid + i * 256, row = c >> 3, kc = (c & 7) * 8;
             const int gm = min(m0 + row, g.M - 1);
-            ra[i] = (k0 + kc < g.K) ? *reinterpret_cast<const v4i*>(g.A + static_cast<int64_t>(gm) * g.lda + k0 + kc)
-                                    : v4i{0, 0, 0, 0};
+            if constexpr (RAGGED)
+                ra[i] = load_chunk_ragged(reinterpret_cast<const int8_t*>(g.A + static_cast<int64_t>(gm) * g.lda + k0 + kc),
+                                          (g.K - (k0 + kc)) * 2, g.ragged_a);
+            else
+                ra[i] = (k0 + kc < g.K) ? *reinterpret_cast<const v4i*>(g.A + static_cast<int64_t>(gm) * g.lda + k0 + kc)
+                                        : v4i{0, 0, 0, 0};
         }
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
@@ -223,6 +230,7 @@ struct Gemm16x16Args {
     int shift_stride, relu, out_kind, mode;
     int64_t stride_a, stride_w, stride_colsum, stride_y;  // batched use, as above
     int shift;                                            // used when `shifts` is null
+    int ragged_a;                                         // RAGGED kernels: how chunks of A's rows may be fetched
 };
 
 __device__ __forceinline__ long long round_shift64(long long v, int s, int mode) {
@@ -447,6 +455,7 @@ __device__ __forceinline__ void select_problem(Gemm16x16Args& g, int b) {
     g.Y = static_cast<int8_t*>(g.Y) + b * g.stride_y * obytes;
 }
 
+template <bool RAGGED>
 __global__ __launch_bounds__(256, 2) void gemm_i16i16_kernel(Gemm16x16Args g) {
     constexpr int BM = 64, BN = 128, BK = 64, PITCH = BK + 16;
     select_problem(g, blockIdx.y);
@@ -485,8 +494,12 @@ __global__ __launch_bounds__(256, 2) void gemm_i16i16_kernel(Gemm16x16Args g) {
         for (int i = 0; i < 2; ++i) {
             const int c = tid + i * 256, row = c >> 3, kc = (c & 7) * 8;
             const int gm = min(m0 + row, g.M - 1);
-            ra[i] = (k0 + kc < g.K) ? *reinterpret_cast<const v4i*>(g.A + static_cast<int64_t>(gm) * g.lda + k0 + kc)
-                                    : v4i{0, 0, 0, 0};
+            if constexpr (RAGGED)
+                ra[i] = load_chunk_ragged(reinterpret_cast<const int8_t*>(g.A + static_cast<int64_t>(gm) * g.lda + k0 + kc),
+                                          (g.K - (k0 + kc)) * 2, g.ragged_a);
+            else
+                ra[i] = (k0 + kc < g.K) ? *reinterpret_cast<const v4i*>(g.A + static_cast<int64_t>(gm) * g.lda + k0 + kc)
+                                        : v4i{0, 0, 0, 0};
         }
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
@@ -504,11 +517,13 @@ __global__ __launch_bounds__(256, 2) void gemm_i16i16_kernel(Gemm16x16Args g) {
         for (int i = 0; i < 2; ++i) {
             const int c = tid + i * 256, row = c >> 3, kc = (c & 7) * 8;
             const unsigned w0 = ra[i][0], w1 = ra[i][1], w2 = ra[i][2], w3 = ra[i][3];
-            const bool in = k0 + kc < g.K;
-            const unsigned flip = in ? 0x80808080u : 0u;  // beyond K: both planes zero, so the row sums stay exact
+            // beyond K both planes are zero, so the row sums stay exact: the low bytes are biased where k < K only
+            const int live = min(max(g.K - (k0 + kc), 0), 8);  // elements of this chunk below K (0 or 8 unless RAGGED)
+            const unsigned flip0 = live >= 4 ? 0x80808080u : (0x80808080u & ((1u << (8 * live)) - 1u));
+            const unsigned flip1 = live >= 8 ? 0x80808080u : (live > 4 ? (0x80808080u & ((1u << (8 * (live - 4))) - 1u)) : 0u);
             v2i hi = {static_cast<int>(__builtin_amdgcn_perm(w1, w0, 0x07050301u)), static_cast<int>(__builtin_amdgcn_perm(w3, w2, 0x07050301u))};
-            v2i lo = {static_cast<int>(__builtin_amdgcn_perm(w1, w0, 0x06040200u) ^ flip),
-                      static_cast<int>(__builtin_amdgcn_perm(w3, w2, 0x06040200u) ^ flip)};
+            v2i lo = {static_cast<int>(__builtin_amdgcn_perm(w1, w0, 0x06040200u) ^ flip0),
+                      static_cast<int>(__builtin_amdgcn_perm(w3, w2, 0x06040200u) ^ flip1)};
             *reinterpret_cast<v2i*>(st + row * PITCH + kc) = hi;
             *reinterpret_cast<v2i*>(st + APLANE + row * PITCH + kc) = lo;
         }
@@ -757,11 +772,17 @@ extern "C" int a4g_dense_i16(const int16_t* A, int64_t lda, const int8_t* Wt, in
         r.shift_stride = g.shift_stride; r.relu = g.relu; r.out_kind = out_kind; r.mode = round_mode;
         if (rs_i16i8_applicable(r, 1)) return check_hip(launch_rs_i16i8(r, 1, stream), who);
     }
-    const bool tiled = K % 16 == 0 && lda % 8 == 0 && ldwt % 16 == 0 && aligned16(A) && aligned16(Wt);
-    if (tiled) {
+    const bool w_ok = ldwt % 16 == 0 && aligned16(Wt) && ldwt >= (K + 15) / 16 * 16;  // what a4g_pack_weights_i8 writes
+    if (w_ok) {
         const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
         A4G_REQUIRE(tiles <= INT32_MAX, A4G_ERR_UNSUPPORTED, "%s: too many tiles", who);
-        gemm_i16i8_kernel<<<dim3(static_cast<unsigned>((tiles + 7) / 8 * 8), 1), 256, tiled16_lds_bytes(g.K, 128), stream>>>(g);  // whole ranges for the 8 XCDs
+        const dim3 grid(static_cast<unsigned>((tiles + 7) / 8 * 8), 1);  // whole ranges for the 8 XCDs
+        if (K % 16 == 0 && lda % 8 == 0 && aligned16(A)) {
+            gemm_i16i8_kernel<false><<<grid, 256, tiled16_lds_bytes(g.K, 128), stream>>>(g);
+        } else {
+            g.ragged_a = ragged_mode(A, lda * 2, 0, K * 2);
+            gemm_i16i8_kernel<true><<<grid, 256, tiled16_lds_bytes(g.K, 128), stream>>>(g);
+        }
     } else {
         const int grid = static_cast<int>(std::min<int64_t>((M * N + 255) / 256, 256 * 32));
         gemm_i16i8_generic_kernel<<<grid, 256, 0, stream>>>(g);
@@ -815,11 +836,17 @@ extern "C" int a4g_dense_i16x16(const int16_t* A, int64_t lda, const int8_t* Wt_
         if (rs_i16i16_applicable(r, 1))
             return check_hip(launch_rs_policy<I16x16Policy, 256, 256, 2, 4, true>(r, 1, stream), who);
     }
-    const bool tiled = K % 16 == 0 && lda % 8 == 0 && ldwt % 16 == 0 && aligned16(A) && aligned16(Wt_hi) && aligned16(Wt_lo);
-    if (tiled) {
+    const bool w_ok = ldwt % 16 == 0 && aligned16(Wt_hi) && aligned16(Wt_lo) && ldwt >= (K + 15) / 16 * 16;  // a4g_pack_weights_i16
+    if (w_ok) {
         const int64_t tiles = ((M + 63) / 64) * ((N + 127) / 128);
         A4G_REQUIRE(tiles <= INT32_MAX, A4G_ERR_UNSUPPORTED, "%s: too many tiles", who);
-        gemm_i16i16_kernel<<<dim3(static_cast<unsigned>((tiles + 7) / 8 * 8), 1), 256, tiled16_lds_bytes(g.K, 64), stream>>>(g);
+        const dim3 grid(static_cast<unsigned>((tiles + 7) / 8 * 8), 1);
+        if (K % 16 == 0 && lda % 8 == 0 && aligned16(A)) {
+            gemm_i16i16_kernel<false><<<grid, 256, tiled16_lds_bytes(g.K, 64), stream>>>(g);
+        } else {
+            g.ragged_a = ragged_mode(A, lda * 2, 0, K * 2);
+            gemm_i16i16_kernel<true><<<grid, 256, tiled16_lds_bytes(g.K, 64), stream>>>(g);
+        }
     } else {
         const int grid = static_cast<int>(std::min<int64_t>((M * N + 255) / 256, 256 * 32));
         gemm_i16i16_generic_kernel<<<grid, 256, 0, stream>>>(g);
@@ -882,12 +909,13 @@ extern "C" int a4g_matmul_i16(const int16_t* A, int64_t lda, int64_t stride_a, c
         r.shift = shift; r.out_kind = out_kind; r.mode = round_mode;
         if (rs_i16i16_applicable(r, nb))
             return check_hip(launch_rs_policy<I16x16Policy, 256, 256, 2, 4, true>(r, nb, stream), who);
+        const int64_t tiles = ((M + 63) / 64) * ((N + 127) / 128);
+        const dim3 grid(static_cast<unsigned>((tiles + 7) / 8 * 8), nb);
         if (tiled) {
-            const int64_t tiles = ((M + 63) / 64) * ((N + 127) / 128);
-            gemm_i16i16_kernel<<<dim3(static_cast<unsigned>((tiles + 7) / 8 * 8), nb), 256, tiled16_lds_bytes(g.K, 64), stream>>>(g);
-        } else {
-            const int grid = static_cast<int>(std::min<int64_t>((M * N + 255) / 256, 256 * 32));
-            gemm_i16i16_generic_kernel<<<dim3(grid, nb), 256, 0, stream>>>(g);
+            gemm_i16i16_kernel<false><<<grid, 256, tiled16_lds_bytes(g.K, 64), stream>>>(g);
+        } else {  // the packed planes in the workspace are always aligned and zero padded; A is fetched as its rows allow
+            g.ragged_a = ragged_mode(A, lda * 2, stride_a * 2, K * 2);
+            gemm_i16i16_kernel<true><<<grid, 256, tiled16_lds_bytes(g.K, 64), stream>>>(g);
         }
     } else {
         Gemm16Args g{};
@@ -903,12 +931,13 @@ extern "C" int a4g_matmul_i16(const int16_t* A, int64_t lda, int64_t stride_a, c
         r.M = g.M; r.N = g.N; r.K = g.K;
         r.shift = shift; r.out_kind = out_kind; r.mode = round_mode;
         if (rs_i16i8_applicable(r, nb)) return check_hip(launch_rs_i16i8(r, nb, stream), who);
+        const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+        const dim3 grid(static_cast<unsigned>((tiles + 7) / 8 * 8), nb);
         if (tiled) {
-            const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
-            gemm_i16i8_kernel<<<dim3(static_cast<unsigned>((tiles + 7) / 8 * 8), nb), 256, tiled16_lds_bytes(g.K, 128), stream>>>(g);
+            gemm_i16i8_kernel<false><<<grid, 256, tiled16_lds_bytes(g.K, 128), stream>>>(g);
         } else {
-            const int grid = static_cast<int>(std::min<int64_t>((M * N + 255) / 256, 256 * 32));
-            gemm_i16i8_generic_kernel<<<dim3(grid, nb), 256, 0, stream>>>(g);
+            g.ragged_a = ragged_mode(A, lda * 2, stride_a * 2, K * 2);
+            gemm_i16i8_kernel<true><<<grid, 256, tiled16_lds_bytes(g.K, 128), stream>>>(g);
         }
     }
     return check_hip(hipGetLastError(), who);

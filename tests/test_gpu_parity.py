@@ -347,6 +347,53 @@ def test_matmul_int16_left_operand(ops, oracle, shape, trans_b, b_dtype):
         assert np.array_equal(got, oracle.matmul(A, B, shift, mode, trans_b=trans_b, out=out)), (mode, out)
 
 
+RAGGED = [(300, 200, 100, 0, 0), (257, 130, 1000, 0, 0), (129, 70, 37, 3, 1), (64, 33, 7, 5, 3), (500, 256, 1030, 2, 2),
+          (1, 1, 1, 0, 0), (140, 128, 200, 56, 8)]
+
+
+@pytest.mark.parametrize('case', RAGGED)
+@pytest.mark.parametrize('kind', ['int8', 'uint8', 'int16x8', 'int16x16'])
+def test_dense_ragged_reduction_and_unaligned_rows(ops, oracle, kind, case):
+    """K that is not a multiple of 16 and activation rows that start at any byte (a column window of a wider matrix)
+    run on the tiled kernels with loads that stop at the row ends: bytes past K must count as zero whatever lies
+    behind them (here: the rest of the wider matrix, filled with extreme values)."""
+    M, N, K, extra, off = case
+    r = rng(M + N + K + len(kind))
+    adt = {'int8': np.int8, 'uint8': np.uint8}.get(kind, np.int16)
+    info = np.iinfo(adt)
+    wide = np.full((M, off + K + extra), info.max, dtype=adt)
+    wide[:, off + K:] = info.min
+    A = r.integers(info.min, info.max + 1, (M, K)).astype(adt)
+    wide[:, off:off + K] = A
+    W = (r.integers(-32768, 32768, (K, N)).astype(np.int16) if kind == 'int16x16' else gauss8(r, 40, (K, N)))
+    bias = r.integers(-2**15, 2**15, N).astype(np.int32)
+    top = 28 if kind == 'int16x16' else (18 if kind == 'int16x8' else 12)
+    shifts = r.integers(top - 5, top + 1, N).astype(np.int32)
+    p = ops.pack_dense(dev(W), dev(bias), shifts)
+    x = dev(wide)[:, off:off + K]
+    out = 'int16' if kind.startswith('int16') else 'int8'
+    for mode, relu in (('conv_even', False), ('symmetric_inf', True), ('floor', False)):
+        got = host(ops.dense(x, p, mode, relu=relu, out_kind=out))
+        assert np.array_equal(got, oracle.dense(A, W, bias, shifts, mode, relu=relu, out=out)), (mode, relu)
+
+
+@pytest.mark.parametrize('trans_b', [True, False])
+@pytest.mark.parametrize('a_dtype,b_dtype', [(np.int8, np.int8), (np.uint8, np.int8), (np.int16, np.int8), (np.int16, np.int16)])
+@pytest.mark.parametrize('shape', [((2,), 130, 70, 100), ((3,), 64, 129, 37), ((), 257, 200, 1001), ((2, 2), 33, 17, 7)])
+def test_matmul_ragged_reduction(ops, oracle, shape, a_dtype, b_dtype, trans_b):
+    """The dynamic MatMul with K off the 16-element grid (rows of either operand then start at odd addresses)."""
+    lead, M, N, K = shape
+    r = rng(M + N + K + int(trans_b))
+    ia, ib = np.iinfo(a_dtype), np.iinfo(b_dtype)
+    A = r.integers(ia.min, ia.max + 1, lead + (M, K)).astype(a_dtype)
+    B = r.integers(ib.min, ib.max + 1, lead + ((N, K) if trans_b else (K, N))).astype(b_dtype)
+    shift = {1: 9, 2: 16}[np.dtype(a_dtype).itemsize] + (8 if b_dtype == np.int16 else 0)
+    out = 'int16' if a_dtype == np.int16 else 'int8'
+    for mode in ('conv_even', 'symmetric_zero', 'ceil'):
+        got = host(ops.matmul(dev(A), dev(B), shift, mode, trans_b=trans_b, out_kind=out))
+        assert np.array_equal(got, oracle.matmul(A, B, shift, mode, trans_b=trans_b, out=out)), mode
+
+
 @pytest.mark.parametrize('shape', [((2, 3), 200, 96, 32), ((5,), 129, 544, 64), ((2,), 31, 1056, 96), ((), 512, 512, 128),
                                    ((3,), 1, 32, 64)])
 def test_matmul_short_reduction_transposed_rhs(ops, oracle, shape):
