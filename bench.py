@@ -38,7 +38,7 @@ MEASURED_TRAFFIC = {
     'c2_dense': 227885846, 'c1_mlp': 166941, 'c4_add': 49063677, 'c4_layernorm': 33052188,
     'c4_add_layernorm': 49190372, 'c3_softmax_exp': 263311713, 'c3_softmax_hccs': 263311775,
     'c3_qk': 182852908, 'c3_pv': 162043118, 'c3_attention_exp': 118076855, 'c3_attention_hccs': 118071577,
-    'calib_copy': 536870912, 'c2_dense_i16': 454854493, 'c2_dense_i16x16': 842202091, 'c2_dense_bf16': 454969771,
+    'calib_copy': 536870912, 'c2_dense_i16': 454852717, 'c2_dense_i16x16': 842038944, 'c2_dense_bf16': 454969771,
     'c2_dense_fp8': 244968648,
 }
 
