@@ -274,4 +274,59 @@ __device__ __forceinline__ int64_t floordiv64(int64_t a, int64_t b) {
     return (r != 0 && ((r < 0) != (b < 0))) ? q - 1 : q;
 }
 
+// One 16-byte chunk of an operand row for shapes the aligned kernels cannot take (K not a multiple of 16, rows that
+// are not 16-byte aligned): `rem` of its bytes belong to the row's K values, the rest read as zero, and no byte
+// past the end of the row's pitch is touched. mode 0: the chunk is aligned and lies inside the pitch; mode 1: rows
+// are 4-byte aligned with a pitch that is a multiple of 4; mode 2: neither.
+__device__ __forceinline__ v4i load_chunk_ragged(const int8_t* p, int rem, int mode) {
+    v4i r = {0, 0, 0, 0};
+    if (rem <= 0) return r;
+    if (mode == 0) {
+        r = *reinterpret_cast<const v4i*>(p);
+    } else if (mode == 1) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (4 * j < rem) r[j] = *reinterpret_cast<const int*>(p + 4 * j);
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            unsigned w = 0;
+#pragma unroll
+            for (int b = 0; b < 4; ++b)
+                if (4 * j + b < rem) w |= static_cast<unsigned>(static_cast<uint8_t>(p[4 * j + b])) << (8 * b);
+            r[j] = static_cast<int>(w);
+        }
+    }
+    if (rem < 16) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int v = rem - 4 * j;  // valid bytes of this dword
+            if (v <= 0) r[j] = 0;
+            else if (v < 4) r[j] &= static_cast<int>((1u << (8 * v)) - 1u);
+        }
+    }
+    return r;
+}
+
+// The store that goes with it: the first `rem` bytes of a 16-byte chunk, in pieces the row's alignment allows.
+__device__ __forceinline__ void store_chunk_ragged(int8_t* p, const v4i& v, int rem, int mode) {
+    if (rem <= 0) return;
+    if (mode == 0 && rem >= 16) {
+        *reinterpret_cast<v4i*>(p) = v;
+        return;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int n = rem - 4 * j;  // bytes of this dword to write
+        if (n <= 0) break;
+        if (mode <= 1 && n >= 4) {
+            *reinterpret_cast<int*>(p + 4 * j) = v[j];
+        } else {
+#pragma unroll
+            for (int b = 0; b < 4; ++b)
+                if (b < n) p[4 * j + b] = static_cast<int8_t>(static_cast<unsigned>(v[j]) >> (8 * b));
+        }
+    }
+}
+
 }  // namespace a4g

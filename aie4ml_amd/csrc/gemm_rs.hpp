@@ -172,40 +172,6 @@ struct RsCfg {
                   "plane split: a wave's rows must hold whole high/low runs");
 };
 
-// One 16-byte chunk of an operand row for shapes the aligned kernels cannot take (K not a multiple of 16, rows that
-// are not 16-byte aligned): `rem` of its bytes belong to the row's K values, the rest read as zero, and no byte
-// past the end of the row's pitch is touched. mode 0: the chunk is aligned and lies inside the pitch; mode 1: rows
-// are 4-byte aligned with a pitch that is a multiple of 4; mode 2: neither.
-__device__ __forceinline__ v4i load_chunk_ragged(const int8_t* p, int rem, int mode) {
-    v4i r = {0, 0, 0, 0};
-    if (rem <= 0) return r;
-    if (mode == 0) {
-        r = *reinterpret_cast<const v4i*>(p);
-    } else if (mode == 1) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-            if (4 * j < rem) r[j] = *reinterpret_cast<const int*>(p + 4 * j);
-    } else {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            unsigned w = 0;
-#pragma unroll
-            for (int b = 0; b < 4; ++b)
-                if (4 * j + b < rem) w |= static_cast<unsigned>(static_cast<uint8_t>(p[4 * j + b])) << (8 * b);
-            r[j] = static_cast<int>(w);
-        }
-    }
-    if (rem < 16) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int v = rem - 4 * j;  // valid bytes of this dword
-            if (v <= 0) r[j] = 0;
-            else if (v < 4) r[j] &= static_cast<int>((1u << (8 * v)) - 1u);
-        }
-    }
-    return r;
-}
-
 // How the ragged kernels may fetch 16-byte chunks of an operand's rows (see load_chunk_ragged).
 static inline int ragged_mode(const void* p, int64_t ld, int64_t stride, int64_t K) {
     const uintptr_t a = reinterpret_cast<uintptr_t>(p);

@@ -579,9 +579,12 @@ __device__ __forceinline__ int max_i8x4(unsigned w) {
 // l, l+L, ... (NCH of them), 16 int8 each.
 // FASTP: uint8 output that needs no clamp with a shift of at most 16: the probability is read as byte 2 of
 // score * (inv << (16 - shift)), which saves the shift. FULL: cols == L * NCH * 16, no chunk is ever masked.
-template <int L, int NCH, bool FASTP, bool FULL>
+// RAGGED (never with FULL): cols need not be a multiple of 16 nor rows 16-byte aligned; `ragged` says how a row's
+// chunks may be fetched and stored (load_chunk_ragged), the last chunk of a row is cut at cols.
+template <int L, int NCH, bool FASTP, bool FULL, bool RAGGED = false>
 __global__ __launch_bounds__(256) void softmax_lut_kernel(const int8_t* __restrict__ x, void* __restrict__ out, int rows,
-                                                           int cols, SoftmaxParams p) {
+                                                           int cols, SoftmaxParams p, int ragged = 0) {
+    static_assert(!(RAGGED && FULL), "a ragged row never fills its chunks");
     __shared__ int table[256];
     table[threadIdx.x] = table_entry(p, threadIdx.x);
     __syncthreads();
@@ -606,7 +609,20 @@ __global__ __launch_bounds__(256) void softmax_lut_kernel(const int8_t* __restri
             const int col0 = (l + L * i) * 16;
             valid[i] = row_ok && (FULL || col0 < cols);
             xv[i] = v4i{(int)0x80808080, (int)0x80808080, (int)0x80808080, (int)0x80808080};
-            if (valid[i]) xv[i] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(x + base + col0));
+            if constexpr (RAGGED) {
+                if (valid[i]) {
+                    const int rem = cols - col0;
+                    xv[i] = load_chunk_ragged(x + base + col0, rem, ragged);
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) {  // bytes past the row's end: -128, which no maximum notices
+                        const int n = rem - 4 * w;
+                        if (n <= 0) xv[i][w] = static_cast<int>(0x80808080u);
+                        else if (n < 4) xv[i][w] |= static_cast<int>(0x80808080u & ~((1u << (8 * n)) - 1u));
+                    }
+                }
+            } else {
+                if (valid[i]) xv[i] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(x + base + col0));
+            }
 #pragma unroll
             for (int j = 0; j < 4; ++j) m = max(m, max_i8x4(xv[i][j]));
         }
@@ -628,7 +644,8 @@ __global__ __launch_bounds__(256) void softmax_lut_kernel(const int8_t* __restri
                 s4[3] = *reinterpret_cast<const int*>(tbytes + byte_x4<3>(d4, two));
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const int s = (FULL || valid[i]) ? s4[j] : 0;
+                    const bool in = RAGGED ? (l + L * i) * 16 + w * 4 + j < cols : valid[i];
+                    const int s = (FULL || (in && valid[i])) ? s4[j] : 0;
                     e[i][w * 4 + j] = s;
                     sum += s;
                 }
@@ -650,9 +667,17 @@ __global__ __launch_bounds__(256) void softmax_lut_kernel(const int8_t* __restri
                     const int y1 = sat16(__mul24(e[i][2 * k + 1], inv) >> p.out_shift);
                     o[k >> 2][k & 3] = static_cast<int>(pack2_halves(y0, y1));
                 }
-                v4i* dst = reinterpret_cast<v4i*>(static_cast<int16_t*>(out) + base + col0);
-                __builtin_nontemporal_store(o[0], dst);
-                __builtin_nontemporal_store(o[1], dst + 1);
+                if constexpr (RAGGED) {
+                    int8_t* dst = reinterpret_cast<int8_t*>(static_cast<int16_t*>(out) + base + col0);
+                    const int rem = (cols - col0) * 2;  // bytes
+                    const int mode = ragged == 0 ? 1 : ragged;  // two-byte elements: an aligned byte row gives aligned dwords at best
+                    store_chunk_ragged(dst, o[0], rem, (cols % 2 == 0 && mode == 1) ? 1 : 2);
+                    store_chunk_ragged(dst + 16, o[1], rem - 16, (cols % 2 == 0 && mode == 1) ? 1 : 2);
+                } else {
+                    v4i* dst = reinterpret_cast<v4i*>(static_cast<int16_t*>(out) + base + col0);
+                    __builtin_nontemporal_store(o[0], dst);
+                    __builtin_nontemporal_store(o[1], dst + 1);
+                }
             } else {
                 v4i o;
 #pragma unroll
@@ -670,7 +695,10 @@ __global__ __launch_bounds__(256) void softmax_lut_kernel(const int8_t* __restri
                         o[w] = static_cast<int>(pack4_bytes(y4[0], y4[1], y4[2], y4[3]));
                     }
                 }
-                __builtin_nontemporal_store(o, reinterpret_cast<v4i*>(static_cast<uint8_t*>(out) + base + col0));
+                if constexpr (RAGGED)
+                    store_chunk_ragged(static_cast<int8_t*>(out) + base + col0, o, cols - col0, ragged);
+                else
+                    __builtin_nontemporal_store(o, reinterpret_cast<v4i*>(static_cast<uint8_t*>(out) + base + col0));
             }
         }
     }
@@ -713,8 +741,13 @@ __global__ __launch_bounds__(256) void softmax_generic_kernel(const int8_t* __re
 
 template <int L, int NCH>
 static void launch_softmax(bool noclamp, int grid, hipStream_t stream, const int8_t* x, void* out, int rows, int cols,
-                           const SoftmaxParams& p) {
+                           const SoftmaxParams& p, int ragged) {
     const bool fastp = noclamp && !p.out_i16 && p.out_shift <= 16;
+    if (ragged >= 0) {
+        if (fastp) softmax_lut_kernel<L, NCH, true, false, true><<<grid, 256, 0, stream>>>(x, out, rows, cols, p, ragged);
+        else softmax_lut_kernel<L, NCH, false, false, true><<<grid, 256, 0, stream>>>(x, out, rows, cols, p, ragged);
+        return;
+    }
     const bool full = cols == L * NCH * 16;
     if (fastp && full)
         softmax_lut_kernel<L, NCH, true, true><<<grid, 256, 0, stream>>>(x, out, rows, cols, p);
@@ -730,9 +763,16 @@ static int softmax_dispatch(const int8_t* x, void* out, int64_t rows, int64_t co
                             hipStream_t stream, const char* who) {
     if (rows == 0) return A4G_OK;
     A4G_REQUIRE(x && out, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
-    const bool fast = cols % 16 == 0 && cols <= 4096 && aligned16(x) && aligned16(out);
-    if (fast) {
-        const int chunks = static_cast<int>(cols / 16);
+    const bool aligned = cols % 16 == 0 && aligned16(x) && aligned16(out);
+    if (cols <= 4096) {
+        // rows off the 16-byte grid: the same kernel with loads and stores that respect the row ends; the output has
+        // the input's row offsets, so one mode serves both when both bases are equally aligned
+        int ragged = -1;
+        if (!aligned) {
+            const uintptr_t both = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out);
+            ragged = (cols % 4 == 0 && both % 4 == 0) ? 1 : 2;
+        }
+        const int chunks = static_cast<int>((cols + 15) / 16);
         // lanes per row: smallest power of two >= chunks (capped at 64), then chunks per lane
         int L = 1;
         while (L < chunks && L < 64) L <<= 1;
@@ -742,17 +782,17 @@ static int softmax_dispatch(const int8_t* x, void* out, int64_t rows, int64_t co
         const int grid = grid_for((rows + rpw - 1) / rpw, 4, 256 * 32);
         const int r = static_cast<int>(rows), c = static_cast<int>(cols);
         if (nch > 1) {  // L == 64
-            if (nch <= 2) launch_softmax<64, 2>(noclamp, grid, stream, x, out, r, c, p);
-            else launch_softmax<64, 4>(noclamp, grid, stream, x, out, r, c, p);
+            if (nch <= 2) launch_softmax<64, 2>(noclamp, grid, stream, x, out, r, c, p, ragged);
+            else launch_softmax<64, 4>(noclamp, grid, stream, x, out, r, c, p, ragged);
         } else {
             switch (L) {
-            case 1: launch_softmax<1, 1>(noclamp, grid, stream, x, out, r, c, p); break;
-            case 2: launch_softmax<2, 1>(noclamp, grid, stream, x, out, r, c, p); break;
-            case 4: launch_softmax<4, 1>(noclamp, grid, stream, x, out, r, c, p); break;
-            case 8: launch_softmax<8, 1>(noclamp, grid, stream, x, out, r, c, p); break;
-            case 16: launch_softmax<16, 1>(noclamp, grid, stream, x, out, r, c, p); break;
-            case 32: launch_softmax<32, 1>(noclamp, grid, stream, x, out, r, c, p); break;
-            default: launch_softmax<64, 1>(noclamp, grid, stream, x, out, r, c, p); break;
+            case 1: launch_softmax<1, 1>(noclamp, grid, stream, x, out, r, c, p, ragged); break;
+            case 2: launch_softmax<2, 1>(noclamp, grid, stream, x, out, r, c, p, ragged); break;
+            case 4: launch_softmax<4, 1>(noclamp, grid, stream, x, out, r, c, p, ragged); break;
+            case 8: launch_softmax<8, 1>(noclamp, grid, stream, x, out, r, c, p, ragged); break;
+            case 16: launch_softmax<16, 1>(noclamp, grid, stream, x, out, r, c, p, ragged); break;
+            case 32: launch_softmax<32, 1>(noclamp, grid, stream, x, out, r, c, p, ragged); break;
+            default: launch_softmax<64, 1>(noclamp, grid, stream, x, out, r, c, p, ragged); break;
             }
         }
     } else {

@@ -555,6 +555,35 @@ def test_softmax_exp_special_rows(ops, oracle):
     assert not got[0].any()  # uniform row of 512: floor(510/512) = 0 -> all zero
 
 
+@pytest.mark.parametrize('offset', [0, 1, 4, 16])
+@pytest.mark.parametrize('cols', [1, 7, 33, 100, 197, 1000, 1001, 1030, 4090, 4095])
+def test_softmax_ragged_rows(ops, oracle, cols, offset):
+    """Row lengths off the 16-element grid and rows that start at any byte (a window into a larger buffer whose
+    surroundings hold the extreme values): the chunked kernel with row-end-aware loads and stores. Both variants,
+    both output types; the bytes around the output window must stay untouched."""
+    rows = 37
+    r = rng(cols * 7 + offset)
+    x = gauss8(r, 24, (rows, cols))
+    x[0, :] = -128
+    x[1, :] = 127
+    x[2, -1] = 127
+    flat = np.full(offset + rows * cols + 19, 127, dtype=np.int8)
+    flat[offset:offset + rows * cols] = x.ravel()
+    xin = dev(flat)[offset:offset + rows * cols].reshape(rows, cols)
+    for out_kind, tdt in (('uint8', torch.uint8), ('int16', torch.int16)):
+        buf = torch.full((offset + rows * cols + 19,), 77, dtype=tdt, device='cuda')
+        out = buf[offset:offset + rows * cols].reshape(rows, cols)
+        ops.softmax_exp(xin, 23, out_kind=out_kind, out=out)
+        got = host(buf)
+        assert np.array_equal(got[offset:offset + rows * cols].reshape(rows, cols), oracle.softmax_exp(x, 23, out=out_kind))
+        assert (got[:offset] == 77).all() and (got[offset + rows * cols:] == 77).all()
+    B = max(1, min(300, 32767 // cols))
+    S, Dmax = (1, B - 1) if cols * 1 >= 256 else (0, 0)
+    if cols * (B - S * Dmax) >= 256:
+        got = host(ops.softmax_hccs(xin, B, S, Dmax))
+        assert np.array_equal(got, oracle.softmax_hccs(x, B, S, Dmax))
+
+
 @pytest.mark.parametrize('cols,params', [(512, (60, 1, 59)), (512, (63, 2, 31)), (128, (255, 2, 126)),
                                          (64, (400, 3, 100)), (96, (33, 1, 30)), (100, (300, 2, 127))])
 def test_softmax_hccs(ops, oracle, cols, params):
