@@ -35,11 +35,11 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
 # WRITE_SIZE, one counter run each, scaled by what the same counter reads for calib_copy).
 # None = not measured.
 MEASURED_TRAFFIC = {
-    'c2_dense': 227885846, 'c1_mlp': 166941, 'c4_add': 49063677, 'c4_layernorm': 33052188,
-    'c4_add_layernorm': 49190372, 'c3_softmax_exp': 263311713, 'c3_softmax_hccs': 263311775,
-    'c3_qk': 182852908, 'c3_pv': 162043118, 'c3_attention_exp': 118076855, 'c3_attention_hccs': 118071577,
-    'calib_copy': 536870912, 'c2_dense_i16': 454852717, 'c2_dense_i16x16': 842038944, 'c2_dense_bf16': 454969771,
-    'c2_dense_fp8': 244968648,
+    'c2_dense': 227748445, 'c1_mlp': 167079, 'c4_add': 49060185, 'c4_layernorm': 33037970,
+    'c4_add_layernorm': 49194720, 'c3_softmax_exp': 263300558, 'c3_softmax_hccs': 263300829,
+    'c3_qk': 182828639, 'c3_pv': 162044378, 'c3_attention_exp': 118079909, 'c3_attention_hccs': 118083080,
+    'calib_copy': 536870912, 'c2_dense_i16': 454834171, 'c2_dense_i16x16': 842037158, 'c2_dense_bf16': 454970606,
+    'c2_dense_fp8': 244992034,
 }
 
 
