@@ -63,7 +63,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_i8_nt_kernel(GemmA
     const int tiles_n = (g.N + BN - 1) / BN;
     const int tiles = tiles_m * tiles_n;
     const int per_xcd = (tiles + 7) / 8;
-    const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    const int tile = tiles < 8 ? static_cast<int>(blockIdx.x) : (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;  // grid_for_tiles
     if (tile >= tiles) return;
     constexpr int GROUP_M = 8;
     const int band = tile / (GROUP_M * tiles_n);
@@ -555,7 +555,7 @@ static hipError_t launch_tiled(const GemmArgs& g, int batch, hipStream_t stream)
         attr_set = true;
     }
     const int tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
-    const int grid_x = (tiles + 7) / 8 * 8;  // whole ranges for the 8 XCDs; surplus workgroups exit at once
+    const int grid_x = grid_for_tiles(tiles);
     hipLaunchKernelGGL(kern, dim3(grid_x, batch), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, g);
     return hipGetLastError();
 }
@@ -572,7 +572,7 @@ static hipError_t launch_dtl_u(const GemmArgs& g, int batch, hipStream_t stream)
         attr_set = true;
     }
     const int tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
-    const int grid_x = (tiles + 7) / 8 * 8;
+    const int grid_x = grid_for_tiles(tiles);
     hipLaunchKernelGGL(kern, dim3(grid_x, batch), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, g);
     return hipGetLastError();
 }

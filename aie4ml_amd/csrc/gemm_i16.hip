@@ -776,7 +776,7 @@ extern "C" int a4g_dense_i16(const int16_t* A, int64_t lda, const int8_t* Wt, in
     if (w_ok) {
         const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
         A4G_REQUIRE(tiles <= INT32_MAX, A4G_ERR_UNSUPPORTED, "%s: too many tiles", who);
-        const dim3 grid(static_cast<unsigned>((tiles + 7) / 8 * 8), 1);  // whole ranges for the 8 XCDs
+        const dim3 grid(static_cast<unsigned>(grid_for_tiles(tiles)), 1);  // whole ranges for the 8 XCDs
         if (K % 16 == 0 && lda % 8 == 0 && aligned16(A)) {
             gemm_i16i8_kernel<false><<<grid, 256, tiled16_lds_bytes(g.K, 128), stream>>>(g);
         } else {
@@ -840,7 +840,7 @@ extern "C" int a4g_dense_i16x16(const int16_t* A, int64_t lda, const int8_t* Wt_
     if (w_ok) {
         const int64_t tiles = ((M + 63) / 64) * ((N + 127) / 128);
         A4G_REQUIRE(tiles <= INT32_MAX, A4G_ERR_UNSUPPORTED, "%s: too many tiles", who);
-        const dim3 grid(static_cast<unsigned>((tiles + 7) / 8 * 8), 1);
+        const dim3 grid(static_cast<unsigned>(grid_for_tiles(tiles)), 1);
         if (K % 16 == 0 && lda % 8 == 0 && aligned16(A)) {
             gemm_i16i16_kernel<false><<<grid, 256, tiled16_lds_bytes(g.K, 64), stream>>>(g);
         } else {
@@ -910,7 +910,7 @@ extern "C" int a4g_matmul_i16(const int16_t* A, int64_t lda, int64_t stride_a, c
         if (rs_i16i16_applicable(r, nb))
             return check_hip(launch_rs_policy<I16x16Policy, 256, 256, 2, 4, true>(r, nb, stream), who);
         const int64_t tiles = ((M + 63) / 64) * ((N + 127) / 128);
-        const dim3 grid(static_cast<unsigned>((tiles + 7) / 8 * 8), nb);
+        const dim3 grid(static_cast<unsigned>(grid_for_tiles(tiles)), nb);
         if (tiled) {
             gemm_i16i16_kernel<false><<<grid, 256, tiled16_lds_bytes(g.K, 64), stream>>>(g);
         } else {  // the packed planes in the workspace are always aligned and zero padded; A is fetched as its rows allow
@@ -932,7 +932,7 @@ extern "C" int a4g_matmul_i16(const int16_t* A, int64_t lda, int64_t stride_a, c
         r.shift = shift; r.out_kind = out_kind; r.mode = round_mode;
         if (rs_i16i8_applicable(r, nb)) return check_hip(launch_rs_i16i8(r, nb, stream), who);
         const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
-        const dim3 grid(static_cast<unsigned>((tiles + 7) / 8 * 8), nb);
+        const dim3 grid(static_cast<unsigned>(grid_for_tiles(tiles)), nb);
         if (tiled) {
             gemm_i16i8_kernel<false><<<grid, 256, tiled16_lds_bytes(g.K, 128), stream>>>(g);
         } else {

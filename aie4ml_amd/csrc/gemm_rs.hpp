@@ -66,6 +66,11 @@ struct GemmArgs {
     int ragged_a, ragged_b;
 };
 
+// Workgroups per problem for tile_coord: whole ranges for the 8 XCDs (surplus workgroups exit at once), except that a
+// problem of fewer than 8 tiles gets exactly its tiles: padding 768 one-tile problems to 8 workgroups each made the
+// surplus ones queue for LDS they never use (88 us for 768 x 100 x 100 x 64).
+static inline int grid_for_tiles(int64_t tiles) { return static_cast<int>(tiles < 8 ? tiles : (tiles + 7) / 8 * 8); }
+
 struct TileCoord {
     int m0, n0, batch;
     bool valid;
@@ -82,7 +87,8 @@ __device__ __forceinline__ TileCoord tile_coord(const GemmArgs& g) {
     const int tiles_n = (g.N + BN - 1) / BN;
     const int tiles = tiles_m * tiles_n;
     const int per_xcd = (tiles + 7) / 8;
-    const int tile = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+    // fewer than 8 tiles per problem (many small problems): one workgroup per tile, no padding (grid_for_tiles)
+    const int tile = tiles < 8 ? static_cast<int>(blockIdx.x) : (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
     tc.valid = tile < tiles;
     constexpr int GROUP_M = 8;
     const int band = tile / (GROUP_M * tiles_n);
@@ -395,7 +401,7 @@ static hipError_t launch_rs_policy(const GemmArgs& g, int batch, hipStream_t str
         attr_set = true;
     }
     const int tiles = ((g.M + Cfg::RBM - 1) / Cfg::RBM) * ((g.N + Cfg::RBN - 1) / Cfg::RBN);
-    const int grid_x = (tiles + 7) / 8 * 8;
+    const int grid_x = grid_for_tiles(tiles);
     hipLaunchKernelGGL(kern, dim3(grid_x, batch), dim3(Cfg::NT), Cfg::LDS_BYTES, stream, g);
     return hipGetLastError();
 }
