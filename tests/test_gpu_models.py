@@ -54,6 +54,29 @@ def test_mlp_graph_unfused_matches_fused(oracle):
     np.testing.assert_array_equal(fused, unfused)
 
 
+def test_wide_mlp_on_a_large_batch_runs_layer_by_layer(oracle):
+    """A fusable chain whose layers are wide and whose batch is large is planned as a chain but executed as one
+    GEMM per layer (the executor's cost model picks the faster form); the result is the oracle's either way, and
+    a small batch of the same model takes the fused launch."""
+    from aie4ml_amd.model import _mlp_layers_are_faster
+    r = np.random.default_rng(31)
+    dims = [57, 200, 200, 200, 3]
+    for batch in (32768, 64):
+        gb = GraphBuilder()
+        t = gb.input('x', (batch, dims[0]), qint(8, 4))
+        for i in range(4):
+            W = r.integers(-100, 100, (dims[i], dims[i + 1])) / 128.0
+            b = r.integers(-512, 512, dims[i + 1]) / 2048.0
+            t = gb.dense(t, W, qint(8, 7), qint(8, 4), bias=b, bias_precision=qint(32, 11), relu=i < 3, name=f'fc{i}')
+        gb.output(t)
+        model = gb.build()
+        model.compile()
+        assert len(model.context.config['gpu_fusion_plan']['mlp_chains']) == 1
+        assert _mlp_layers_are_faster(batch, list(zip(dims[:-1], dims[1:]))) == (batch == 32768)
+        x = np.clip(np.rint(r.normal(0, 30, (batch, dims[0]))), -128, 127).astype(np.int8)
+        _graph_check(model, oracle, {'x': x})
+
+
 def test_iteration_axis_folds_into_batch(oracle):
     model, x, layers = workloads.c1_mlp_model(batch=64)
     xs = np.stack([x, x[::-1], x])                      # (iterations, batch, features)
