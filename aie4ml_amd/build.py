@@ -39,7 +39,8 @@ def _stale() -> bool:
     if not LIB_PATH.exists():
         return True
     t = LIB_PATH.stat().st_mtime
-    deps = [CSRC / s for s in SOURCES] + [CSRC / 'common.hpp', CSRC / 'softmax_common.hpp', CSRC / 'matmul_lean.hpp', CSRC / 'gemm_rs.hpp', CSRC.parent.parent / 'include' / 'aie4ml_gfx950.h']
+    # every source and header under csrc/ plus the public header: an edited epilogue header must trigger a rebuild
+    deps = [*CSRC.glob('*.hip'), *CSRC.glob('*.hpp'), *(CSRC.parent.parent / 'include').glob('*.h')]
     return any(d.stat().st_mtime > t for d in deps)
 
 

@@ -9,6 +9,7 @@
 // back 128 * colsum[n] (exact in wrapping int32).
 #include <algorithm>
 #include <cstdlib>
+#include <mutex>
 #include <type_traits>
 
 #include "common.hpp"
@@ -761,12 +762,40 @@ extern "C" size_t a4g_matmul_i8_workspace_bytes(int64_t batch, int64_t M, int64_
     return bytes;
 }
 
-extern "C" int a4g_matmul_i8(const void* A, int a_kind, int64_t lda, int64_t stride_a, const int8_t* B, int64_t ldb,
-                             int64_t stride_b, int trans_b, void* C, int64_t ldc, int64_t stride_c, int64_t batch, int64_t M,
-                             int64_t N, int64_t K, int shift, int round_mode, int out_kind, void* workspace,
-                             size_t workspace_bytes, a4g_stream_t stream_) {
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
-    const char* who = "a4g_matmul_i8";
+// ---- a4g_matmul_i8_static: the same MatMul for callers that cannot allocate ---------------------------------
+// The repacked right operand and its column sums go to a fixed array in device memory instead of a caller's
+// workspace. Every GPU the library runs on holds its own copy of the array at its own address; host code never uses
+// the array's name as an address (it is only a handle for hipGetSymbolAddress), it uses the per-device pointer
+// resolved on the first call on that device.
+static __device__ __align__(256) unsigned char scratch[A4G_MATMUL_I8_STATIC_MAX_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex scratch_mutex;
+void* scratch_ptr[kMaxDevices] = {};  // device address of `scratch` on each device, resolved once
+
+int static_scratch(const char* who, void** out) {
+    int dev = -1;
+    if (int st = check_hip(hipGetDevice(&dev), who)) return st;
+    A4G_REQUIRE(dev >= 0 && dev < kMaxDevices, A4G_ERR_UNSUPPORTED, "%s: device ordinal %d beyond %d", who, dev, kMaxDevices);
+    std::lock_guard<std::mutex> lock(scratch_mutex);
+    if (!scratch_ptr[dev]) {
+        void* p = nullptr;
+        if (int st = check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), who)) return st;
+        A4G_REQUIRE(p != nullptr && aligned16(p), A4G_ERR_HIP, "%s: the scratch array resolved to a bad address", who);
+        scratch_ptr[dev] = p;
+    }
+    *out = scratch_ptr[dev];
+    return A4G_OK;
+}
+}  // namespace
+
+// Body of both MatMul entry points. `own_scratch`: the workspace is the library's static scratch array rather than
+// a caller's buffer; it is resolved here, after validation and only when the problem needs it.
+static int matmul_i8_impl(const char* who, bool own_scratch, const void* A, int a_kind, int64_t lda, int64_t stride_a,
+                          const int8_t* B, int64_t ldb, int64_t stride_b, int trans_b, void* C, int64_t ldc, int64_t stride_c,
+                          int64_t batch, int64_t M, int64_t N, int64_t K, int shift, int round_mode, int out_kind,
+                          void* workspace, size_t workspace_bytes, hipStream_t stream) {
     A4G_REQUIRE(batch >= 0 && batch <= 65535 && M >= 0 && N >= 1 && K >= 1 && M <= INT32_MAX && N <= (1 << 24) &&
                     K <= (1 << 24),
                 A4G_ERR_INVALID_ARGUMENT, "%s: bad shape batch=%lld M=%lld N=%lld K=%lld", who, (long long)batch,
@@ -802,6 +831,14 @@ extern "C" int a4g_matmul_i8(const void* A, int a_kind, int64_t lda, int64_t str
     }
 
     const size_t need = a4g_matmul_i8_workspace_bytes(batch, M, N, K, trans_b, a_kind);
+    if (own_scratch && need > 0) {
+        workspace_bytes = static_cast<size_t>(A4G_MATMUL_I8_STATIC_MAX_BYTES);
+        A4G_REQUIRE(need <= workspace_bytes, A4G_ERR_WORKSPACE,
+                    "%s: the repacked right operand needs %zu bytes, the static scratch array holds %zu "
+                    "(A4G_MATMUL_I8_STATIC_MAX_BYTES); use a4g_matmul_i8 with a workspace of that size",
+                    who, need, workspace_bytes);
+        if (int st = static_scratch(who, &workspace)) return st;
+    }
     A4G_REQUIRE(need == 0 || (workspace && workspace_bytes >= need), A4G_ERR_WORKSPACE,
                 "%s: workspace of %zu bytes required, got %zu", who, need, workspace ? workspace_bytes : (size_t)0);
     A4G_REQUIRE(need == 0 || aligned16(workspace), A4G_ERR_WORKSPACE, "%s: workspace must be 16-byte aligned", who);
@@ -854,4 +891,22 @@ extern "C" int a4g_matmul_i8(const void* A, int a_kind, int64_t lda, int64_t str
         e = a_ok ? launch_gemm_nt(g, static_cast<int>(batch), stream, env_variant()) : launch_ragged(g, static_cast<int>(batch), stream);
     }
     return check_hip(e, who);
+}
+
+extern "C" int a4g_matmul_i8(const void* A, int a_kind, int64_t lda, int64_t stride_a, const int8_t* B, int64_t ldb,
+                             int64_t stride_b, int trans_b, void* C, int64_t ldc, int64_t stride_c, int64_t batch, int64_t M,
+                             int64_t N, int64_t K, int shift, int round_mode, int out_kind, void* workspace,
+                             size_t workspace_bytes, a4g_stream_t stream_) {
+    return matmul_i8_impl("a4g_matmul_i8", false, A, a_kind, lda, stride_a, B, ldb, stride_b, trans_b, C, ldc, stride_c, batch, M,
+                          N, K, shift, round_mode, out_kind, workspace, workspace_bytes, static_cast<hipStream_t>(stream_));
+}
+
+extern "C" int a4g_matmul_i8_static(const void* A, int a_kind, int64_t lda, int64_t stride_a, const int8_t* B, int64_t ldb,
+                                    int64_t stride_b, int trans_b, void* C, int64_t ldc, int64_t stride_c, int64_t batch,
+                                    int64_t M, int64_t N, int64_t K, int shift, int round_mode, int out_kind,
+                                    a4g_stream_t stream_) {
+    // Nothing in the array has to start at zero: the repack writes every byte the GEMM reads (rows are zero padded
+    // to the packed pitch) and the column-sum kernel stores, never accumulates.
+    return matmul_i8_impl("a4g_matmul_i8_static", true, A, a_kind, lda, stride_a, B, ldb, stride_b, trans_b, C, ldc, stride_c,
+                          batch, M, N, K, shift, round_mode, out_kind, nullptr, 0, static_cast<hipStream_t>(stream_));
 }

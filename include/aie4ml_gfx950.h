@@ -149,6 +149,20 @@ A4G_API int a4g_matmul_i8(const void* A, int a_kind, int64_t lda, int64_t stride
                   int64_t M, int64_t N, int64_t K, int shift, int round_mode, int out_kind, void* workspace,
                   size_t workspace_bytes, a4g_stream_t stream);
 
+/* The same MatMul for callers that cannot allocate device memory or carry a workspace: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc. It has no counterpart in the reference. Arguments
+ * and results are those of a4g_matmul_i8 without the workspace pair: the repacked right operand and its column sums
+ * go to a fixed array of A4G_MATMUL_I8_STATIC_MAX_BYTES bytes of device memory that every GPU the library is used on
+ * holds until the process ends. The call allocates and frees nothing. A problem whose
+ * a4g_matmul_i8_workspace_bytes() exceeds the array returns A4G_ERR_WORKSPACE (shapes that need no workspace are
+ * never rejected). All calls on one GPU share that GPU's array: calls that may overlap on one GPU (different
+ * streams, different threads) race; the array keeps the last call's contents and nothing in it needs clearing. The
+ * array's address is resolved on the first call on each device, which should be made outside stream capture. */
+#define A4G_MATMUL_I8_STATIC_MAX_BYTES (16u << 20)
+A4G_API int a4g_matmul_i8_static(const void* A, int a_kind, int64_t lda, int64_t stride_a, const int8_t* B, int64_t ldb,
+                         int64_t stride_b, int trans_b, void* C, int64_t ldc, int64_t stride_c, int64_t batch,
+                         int64_t M, int64_t N, int64_t K, int shift, int round_mode, int out_kind, a4g_stream_t stream);
+
 /* ---- Integer LayerNorm, int8 -> int8, over the last axis -------------------------------------------
  * Replaces layernorm_i8<Cfg>::run / layernorm_i8_tiled<Cfg>::run and
  * layernorm_base<Cfg>::row_statistics, templates/nnet_utils/layer_norm/layer_norm.cpp:14-231,

@@ -84,6 +84,10 @@ def test_argument_validation_happens_before_any_launch(libpath):
     assert st == _lib.A4G_ERR_UNSUPPORTED
     with pytest.raises(NotImplementedError):
         _lib.check(st)
+    # the entry point without a workspace validates like a4g_matmul_i8, before it looks at the device
+    st = lib.a4g_matmul_i8_static(None, 0, 16, 0, None, 16, 0, 0, None, 16, 0, 1, 4, 16, 16, 40, 0, 0, None)  # shift 40
+    assert st == _lib.A4G_ERR_INVALID_ARGUMENT and b'a4g_matmul_i8_static' in lib.a4g_last_error()
+    assert lib.a4g_matmul_i8_static(None, 0, 16, 0, None, 16, 0, 0, None, 16, 0, 0, 4, 16, 16, 3, 0, 0, None) == 0  # batch 0
     # empty problems are fine and do nothing
     assert lib.a4g_add(None, None, None, 0, 0, 0, 0, None) == 0
     assert lib.a4g_layernorm_i8(None, None, None, None, 0, 64, 1, 7, 5, 6, None) == 0
