@@ -521,25 +521,39 @@ __global__ __launch_bounds__(256) void transpose_kn_kernel(const int8_t* __restr
 // colsum[b][n] = sum_k rhs[k][n]; trans: rhs stored [N][ld] (sum along the contiguous axis).
 // A workgroup owns 64 columns; its four waves take every fourth k (rows of 64 contiguous bytes when the operand
 // is [K][N]; when it is [N][ld] a thread walks its own row in steps of four) and add up through LDS.
+// k_chunk < K splits the reduction over gridDim.z: every workgroup then adds its partial sums into colsum with
+// integer atomics, and the caller clears colsum first (clear_i32_kernel, not a memset, so that a caller may capture
+// the sequence into a graph).
 __global__ __launch_bounds__(256) void colsum_kernel(const int8_t* __restrict__ B, int64_t ld, int64_t stride_b, int trans,
-                                                      int32_t* __restrict__ colsum, int64_t stride_c, int K, int N) {
+                                                      int32_t* __restrict__ colsum, int64_t stride_c, int K, int N,
+                                                      int k_chunk) {
     __shared__ int part[4][64];
     const int batch = blockIdx.y;
     const int8_t* src = B + batch * stride_b;
     const int c = threadIdx.x & 63, ks = threadIdx.x >> 6;
     const int n = blockIdx.x * 64 + c;
+    const int k0 = blockIdx.z * k_chunk, k1 = min(K, k0 + k_chunk);
     int s = 0;
     if (n < N) {
         if (trans) {
             const int8_t* r = src + static_cast<int64_t>(n) * ld;
-            for (int k = ks; k < K; k += 4) s += r[k];
+            for (int k = k0 + ks; k < k1; k += 4) s += r[k];
         } else {
-            for (int k = ks; k < K; k += 4) s += src[static_cast<int64_t>(k) * ld + n];
+            for (int k = k0 + ks; k < k1; k += 4) s += src[static_cast<int64_t>(k) * ld + n];
         }
     }
     part[ks][c] = s;
     __syncthreads();
-    if (ks == 0 && n < N) colsum[batch * stride_c + n] = part[0][c] + part[1][c] + part[2][c] + part[3][c];
+    if (ks == 0 && n < N) {
+        const int total = part[0][c] + part[1][c] + part[2][c] + part[3][c];
+        if (k_chunk < K) atomicAdd(colsum + batch * stride_c + n, total);
+        else colsum[batch * stride_c + n] = total;
+    }
+}
+
+__global__ __launch_bounds__(256) void clear_i32_kernel(int32_t* __restrict__ p, int64_t n) {
+    const int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (i < n) p[i] = 0;
 }
 
 static inline int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
@@ -659,7 +673,10 @@ static hipError_t launch_gemm_nt(const GemmArgs& g, int batch, hipStream_t strea
     }
 }
 
+// Tuning builds (-DA4G_TUNING) can force a tile shape through the A4G_GEMM_VARIANT environment variable; the shipped
+// library reads no environment and always dispatches automatically.
 static int env_variant() {
+#ifdef A4G_TUNING
     static int v = -1;
     if (v < 0) {
         const char* e = getenv("A4G_GEMM_VARIANT");
@@ -667,6 +684,9 @@ static int env_variant() {
         if (v < 0) v = 0;
     }
     return v;
+#else
+    return 0;
+#endif
 }
 
 // Shapes outside the aligned kernels' requirements: same tiles, chunk loads that respect the row ends.
@@ -698,9 +718,16 @@ extern "C" int a4g_pack_weights_i8(const int8_t* W, int64_t ldw, int64_t K, int6
     dim3 grid(static_cast<unsigned>((ldt + 63) / 64), static_cast<unsigned>((N + 63) / 64), 1);
     transpose_kn_kernel<<<grid, 256, 0, stream>>>(W, ldw, 0, Wt, ldt, 0, static_cast<int>(K), static_cast<int>(N));
     if (colsum) {
-        colsum_kernel<<<dim3(static_cast<unsigned>((N + 63) / 64), 1), 256, 0, stream>>>(W, ldw, 0, 0, colsum, 0,
-                                                                                          static_cast<int>(K),
-                                                                                          static_cast<int>(N));
+        // one workgroup per 64 columns over all of K is 64 workgroups for a 4096 x 4096 matrix: split K so that the
+        // launch has about 2048 workgroups
+        const int64_t col_groups = (N + 63) / 64;
+        int64_t splits = std::min<int64_t>(std::max<int64_t>(1, 2048 / col_groups), (K + 255) / 256);
+        const int k_chunk = static_cast<int>((K + splits - 1) / splits);
+        splits = (K + k_chunk - 1) / k_chunk;
+        if (splits > 1)
+            clear_i32_kernel<<<static_cast<unsigned>((N + 255) / 256), 256, 0, stream>>>(colsum, N);
+        colsum_kernel<<<dim3(static_cast<unsigned>(col_groups), 1, static_cast<unsigned>(splits)), 256, 0, stream>>>(
+            W, ldw, 0, 0, colsum, 0, static_cast<int>(K), static_cast<int>(N), k_chunk);
     }
     return check_hip(hipGetLastError(), "a4g_pack_weights_i8");
 }
@@ -865,7 +892,7 @@ static int matmul_i8_impl(const char* who, bool own_scratch, const void* A, int 
     if (g.a_unsigned) {
         colsum = reinterpret_cast<int32_t*>(ws + (trans_b ? 0 : round_up(batch * N * ldt, 256)));
         colsum_kernel<<<dim3(static_cast<unsigned>((N + 63) / 64), static_cast<unsigned>(batch)), 256, 0, stream>>>(
-            B, ldb, stride_b, trans_b, colsum, N, static_cast<int>(K), static_cast<int>(N));
+            B, ldb, stride_b, trans_b, colsum, N, static_cast<int>(K), static_cast<int>(N), static_cast<int>(K));
         g.colsum = colsum;
         g.stride_colsum = N;
     }

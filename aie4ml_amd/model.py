@@ -281,13 +281,34 @@ class GPUModel:
             q = heads_view(values[grp['q_src']], grp['q_base'])
             k = heads_view(values[grp['k_src']], grp['k_base'])
             v = heads_view(values[grp['v_src']], grp['v_base'])
+            if not _views_are_16_byte_aligned(q, k, v):
+                # slices of slices can start anywhere: the planner sees offsets within the nearest source only
+                self._run_attention_unfused(grp, values, heads_view=(q, k, v))
+                return
             out = torch.empty((q.shape[0], q.shape[2], nh * d), dtype=torch.int8, device=q.device)
             ops.attention(q, k, v, c1.shift, c1.rounding_mode, sm, c3.shift, c3.rounding_mode,
                           out=out.unflatten(-1, (nh, d)).permute(0, 2, 1, 3))
             values[grp['out']] = out
+        elif not _views_are_16_byte_aligned(values[tr0['q']], values[tr0['k']], values[tr0['v']]):
+            self._run_attention_unfused(grp, values)
         else:
             values[grp['out']] = ops.attention(values[tr0['q']], values[tr0['k']], values[tr0['v']], c1.shift, c1.rounding_mode,
                                                sm, c3.shift, c3.rounding_mode)
+
+    def _run_attention_unfused(self, grp, values, heads_view=None) -> None:
+        """The members of a planned attention group one operator at a time: MatMul, Softmax, MatMul per head, then the
+        concat. Taken when the operands turn out not to be 16-byte aligned views at run time."""
+        execution, graph = self.context.ir.execution, self.context.ir.logical
+        for h, tr in enumerate(grp['heads']):
+            if heads_view is not None:  # head h of the [batch, heads, seq, d] views, should its slice node come later
+                for key, view in zip(('q', 'k', 'v'), heads_view):
+                    values.setdefault(tr[key], view[:, h])
+            for key in ('qk', 'softmax', 'pv'):
+                inst = execution.get(tr[key])
+                args = {t.name: values[t.name] for t in inst.node.inputs if not t.is_parameter}
+                values.update(inst.variant.run(inst, args))
+        if grp.get('concat'):
+            self._run_view(next(n for n in graph.nodes if n.name == grp['concat']), values)
 
     def _run_mlp(self, chain: List[str], values, ops) -> None:
         execution = self.context.ir.execution
@@ -306,6 +327,12 @@ class GPUModel:
             return
         y = ops.mlp(x.reshape(-1, x.shape[-1]), specs, insts[0].config.rounding_mode)
         values[insts[-1].node.outputs[0].name] = y.reshape(lead + (y.shape[-1],))
+
+
+def _views_are_16_byte_aligned(*tensors) -> bool:
+    """What the fused attention launch asks of its operands: 16-byte aligned base addresses and row / head / batch
+    pitches (int8 tensors, so elements are bytes)."""
+    return all(t.data_ptr() % 16 == 0 and all(int(st) % 16 == 0 for st in t.stride()[:-1]) for t in tensors)
 
 
 def _mlp_layers_are_faster(rows: int, layers) -> bool:

@@ -408,6 +408,7 @@ class PlanGpuFusion(AIEPass):
     # ---- attention -------------------------------------------------------------------------------------
     ATTN_HEAD_DIM = 64
     ATTN_KEYS = (32, 64, 128, 256, 512)
+    ATTN_MAX_SHIFT = 24
 
     def _plan_attention(self, graph, execution, outputs):
         triples = []
@@ -440,6 +441,8 @@ class PlanGpuFusion(AIEPass):
                 continue
             if int(q.shape[-1]) != self.ATTN_HEAD_DIM or int(k.shape[-2]) not in self.ATTN_KEYS:
                 continue
+            if c1.shift > self.ATTN_MAX_SHIFT or c3.shift > self.ATTN_MAX_SHIFT:
+                continue  # the fused kernel takes shifts up to 24, the MatMul kernels up to 31
             triples.append({'qk': qk.name, 'softmax': sm.name, 'pv': pv.name, 'q': q.name, 'k': k.name, 'v': v.name,
                             'out': pv.outputs[0].name})
         groups, used = [], set()
@@ -490,6 +493,9 @@ class PlanGpuFusion(AIEPass):
                     and c == items[0][3] + h * d
             ref = [self._attn_signature(execution, items[0][4])]
             regular = regular and all(self._attn_signature(execution, it[4]) == ref[0] for it in items)
+            # the fused kernel reads 16-byte chunks: head slices must start on 16-byte boundaries of 16-byte aligned rows
+            srcs = [graph.tensors[t] for t in (qs, ks, vs)]
+            regular = regular and all(b % 16 == 0 for b in items[0][1:4]) and all(int(t.shape[-1]) % 16 == 0 for t in srcs)
             if not regular:
                 continue
             groups.append({'heads': [it[4] for it in items], 'q_src': qs, 'k_src': ks, 'v_src': vs,
@@ -512,6 +518,8 @@ class PlanGpuFusion(AIEPass):
             return False
         if any(execution.get(n.name).config.accumulator_tag != 'acc32' for n in chain):
             return False  # the fused MLP kernel is the int8 one
+        if execution.get(chain[0].name).config.precision['lhs'].format not in ('int8', 'uint8'):
+            return False  # acc32 also covers int16 activations x int8 weights: those layers run one by one
         total, mode = 0, None
         for i, n in enumerate(chain):
             cfg = execution.get(n.name).config

@@ -6,10 +6,14 @@ Default workload: the single quantized Dense of the baseline configuration
 saturate to int8, fused ReLU). One step = one pass of the operator over the whole synthetic batch,
 inputs already resident in HBM. Prints ONE JSON line.
 
+The default run also times, after the headline workload, the matrix-core calibration loop (`roofline.calibrated_peak`,
+`frac_of_calibrated`, the clock under matrix load) and every other baseline configuration with the same method
+(`workloads`: value, ms_per_step, bit_exact, roofline per configuration; no CPU leg). `--only` skips both.
+
 Other workloads (--workload c2_dense_i16 | c2_dense_i16x16 | c2_dense_bf16 | c2_dense_fp8 | c1_mlp | c3_softmax_exp | c3_softmax_hccs | c3_qk | c3_pv |
 c3_attention_exp | c3_attention_hccs | c4_add_layernorm | c4_layernorm | c4_add | c5_encoder) print the same line for that operator or graph;
 --workload calib_copy runs a plain 256 MiB elementwise copy, the known-size kernel the HBM traffic
-counters are scaled against.
+counters are scaled against; --workload calib_mfma runs the register-resident int8 MFMA loop alone.
 """
 
 from __future__ import annotations
@@ -31,16 +35,18 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, TFLOP/s
 PEAK_FP8_TFLOPS = 5000.0   # MI355X dense fp8 MFMA, TFLOP/s
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
 
-# HBM bytes per launch of each workload's dominant kernel, from hardware counters (FETCH_SIZE and
-# WRITE_SIZE, one counter run each, scaled by what the same counter reads for calib_copy).
-# None = not measured.
-MEASURED_TRAFFIC = {
-    'c2_dense': 227748445, 'c1_mlp': 167079, 'c4_add': 49060185, 'c4_layernorm': 33037970,
-    'c4_add_layernorm': 49194720, 'c3_softmax_exp': 263300558, 'c3_softmax_hccs': 263300829,
-    'c3_qk': 182828639, 'c3_pv': 162044378, 'c3_attention_exp': 118079909, 'c3_attention_hccs': 118083080,
-    'calib_copy': 536870912, 'c2_dense_i16': 454834171, 'c2_dense_i16x16': 842037158, 'c2_dense_bf16': 454970606,
-    'c2_dense_fp8': 244992034,
-}
+# HBM bytes per launch of each workload's dominant kernel come from hardware counters (FETCH_SIZE and WRITE_SIZE, one
+# counter run each, scaled by what the same counter reads for calib_copy). The summaries of those runs are the text
+# files under profiles/, named <kernel>__<workload>.txt; the figure is read from their line "traffic = X MB per launch"
+# so that it cannot outlive the profile it came from. None = no profile for this kernel and workload.
+def measured_traffic(kernel, wl):
+    import re
+
+    path = ROOT / 'profiles' / f'{kernel}__{wl}.txt'
+    if not path.exists():
+        return None, None
+    m = re.search(r'^\s*traffic = ([0-9.]+) MB per launch', path.read_text(), flags=re.M)
+    return (int(float(m.group(1)) * 1e6), f'profiles/{path.name}') if m else (None, None)
 
 
 def _time_gpu(torch, fn, steps, warmup, use_graph=True):
@@ -100,31 +106,17 @@ def _time_cpu(fn, budget_s=12.0, min_runs=2):
     return float(np.median(times))
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument('--gpus', type=int, default=1)
-    ap.add_argument('--steps', type=int, default=50)
-    ap.add_argument('--warmup', type=int, default=10)
-    ap.add_argument('--workload', default='c2_dense')
-    ap.add_argument('--no-cpu-baseline', action='store_true')
-    ap.add_argument('--eager', action='store_true', help='time eager launches instead of a replayed HIP graph')
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit('bench.py: this build runs on exactly one GPU (every operator is row-independent, so more GPUs '
-                 'would each take a slice of the batch with the weights replicated). Use --gpus 1.')
-
-    import torch
-
-    if not torch.cuda.is_available():
-        sys.exit('bench.py: no GPU visible')
+def prepare(wl, torch):
+    """Builds one workload on the GPU, runs it once and checks it against the oracle. Returns a dict with the step
+    function `fn`, the algorithmic work per step, the roofline that bounds it and what the CPU leg needs."""
     from aie4ml_amd import ops, workloads
     from oracle import oracle
 
     dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()  # noqa: E731
-    wl = args.workload
     extra = {}
     cpu_fn = None
     cpu_samples = None
+    cpu_work = cpu_desc = None
     peak_mfma, mfma_unit = PEAK_INT8_TOPS, 'TOP/s'
 
     if wl == 'c2_dense':
@@ -315,7 +307,7 @@ def main():
             cpu_work = bytes_ * 4 / (Bt * H)
             cpu_desc = 'oracle MatMul on 4 of 512 (batch, head) slices'
             work = float(bytes_)
-            kernel = 'gemm_i8_dtl_kernel'
+            kernel = 'matmul_lean_nt_kernel'
         elif wl == 'c3_pv':
             ws = torch.empty((ops._lib.load().a4g_matmul_i8_workspace_bytes(Bt * H, S, D, S, 0, 1),), dtype=torch.uint8,
                              device='cuda')
@@ -331,7 +323,7 @@ def main():
             cpu_fn = lambda: oracle.matmul(pl, v[0, :4], prm['pv_shift'], 'conv_even')  # noqa: E731
             cpu_work = bytes_ * 4 / (Bt * H)
             cpu_desc = 'oracle MatMul (uint8 x int8) on 4 of 512 (batch, head) slices'
-            kernel = 'gemm_rs_kernel'
+            kernel = 'matmul_lean_nn_kernel'
         else:
             out = torch.empty(logits.shape, dtype=torch.uint8, device='cuda')
             hc = prm['hccs']
@@ -432,49 +424,151 @@ def main():
     else:
         sys.exit(f'unknown workload {wl}')
 
-    ms_wall, ms_ev, graphed = _time_gpu(torch, fn, args.steps, args.warmup, use_graph=not args.eager)
+
+    return dict(wl=wl, fn=fn, bit_exact=bit_exact, work=work, bound=bound, samples=samples, config=config, metric=metric,
+                unit=unit, kernel=kernel, extra=extra, cpu_fn=cpu_fn, cpu_work=cpu_work, cpu_desc=cpu_desc,
+                cpu_samples=cpu_samples, peak_mfma=peak_mfma, mfma_unit=mfma_unit)
+
+
+KERNEL_FILE = {'whole graph (GEMM kernels dominate)': 'graph_executor'}
+
+
+def measure(torch, w, steps, warmup, eager=False):
+    """Times `steps` launches of a prepared workload; returns (ms per step, value in the workload's unit, roofline)."""
+    ms_wall, ms_ev, graphed = _time_gpu(torch, w['fn'], steps, warmup, use_graph=not eager)
     ms = max(ms_wall, ms_ev)
-    if bound == 'mfma':
+    work, unit = w['work'], w['unit']
+    traffic, source = measured_traffic(KERNEL_FILE.get(w['kernel'], w['kernel']), w['wl'])
+    if w['bound'] == 'mfma':
         achieved = work / (ms_ev * 1e-3) / 1e12
-        roof = {'bound': 'mfma', 'achieved': round(achieved, 3), 'peak': peak_mfma, 'unit': mfma_unit,
-                'frac': round(achieved / peak_mfma, 4), 'traffic': MEASURED_TRAFFIC.get(wl), 'kernel': kernel,
-                'kernel_ms': round(ms_ev, 5)}
+        roof = {'bound': 'mfma', 'achieved': round(achieved, 3), 'peak': w['peak_mfma'], 'unit': w['mfma_unit'],
+                'frac': round(achieved / w['peak_mfma'], 4)}
     else:
         achieved = work / (ms_ev * 1e-3) / 1e9
         roof = {'bound': 'hbm', 'achieved': round(achieved, 2), 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
-                'frac': round(achieved / PEAK_HBM_GBS, 4), 'traffic': MEASURED_TRAFFIC.get(wl), 'kernel': kernel,
-                'kernel_ms': round(ms_ev, 5)}
-
+                'frac': round(achieved / PEAK_HBM_GBS, 4)}
+    roof.update({'traffic': traffic, 'traffic_source': source, 'kernel': w['kernel'], 'kernel_ms': round(ms_ev, 5)})
     if unit in ('TOP/s', 'TFLOP/s'):
         value = work / (ms * 1e-3) / 1e12
     elif unit == 'GB/s':
         value = work / (ms * 1e-3) / 1e9
     else:
-        value = samples / (ms * 1e-3)
+        value = w['samples'] / (ms * 1e-3)
+    return ms, value, roof, graphed
+
+
+def calibrate_mfma(torch, blocks_per_cu=2, iters=4096):
+    """The int8 matrix-core rate this GPU sustains with register-resident operands (no memory traffic), and the clock
+    it holds meanwhile: (TOP/s, GHz)."""
+    from aie4ml_amd import _lib
+
+    L = _lib.load()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    blocks = cus * blocks_per_cu
+    sink = torch.zeros(4, dtype=torch.int32, device='cuda')
+    clocks = torch.zeros(2 * blocks, dtype=torch.int64, device='cuda')
+    fn = lambda: _lib.check(L.a4g_calib_mfma_i8(blocks, iters, sink.data_ptr(), clocks.data_ptr(),  # noqa: E731
+                                                torch.cuda.current_stream().cuda_stream))  # the capture stream, when capturing
+    _, ms_ev, _ = _time_gpu(torch, fn, 20, 5)
+    ops_ = int(L.a4g_calib_mfma_i8_ops(blocks, iters))
+    c = clocks.cpu().numpy().reshape(-1, 2).astype(np.float64)
+    ghz = float(np.median(c[:, 0] / np.maximum(c[:, 1], 1.0)) * 0.1)  # shader ticks per 10 ns tick of the 100 MHz counter
+    return ops_ / (ms_ev * 1e-3) / 1e12, ghz, ms_ev, blocks, iters
+
+
+# the other configurations, timed in the default run after the headline workload (same steps, no CPU leg)
+ALSO = ('c1_mlp', 'c3_qk', 'c3_softmax_exp', 'c3_softmax_hccs', 'c3_pv', 'c3_attention_exp', 'c4_add', 'c4_layernorm',
+        'c4_add_layernorm', 'c5_encoder')
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=50)
+    ap.add_argument('--warmup', type=int, default=10)
+    ap.add_argument('--workload', default='c2_dense')
+    ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--only', action='store_true', help='time the named workload alone (the default run of c2_dense '
+                    'also times the other configurations and the matrix-core calibration loop)')
+    ap.add_argument('--eager', action='store_true', help='time eager launches instead of a replayed HIP graph')
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit('bench.py: this build runs on exactly one GPU (every operator is row-independent, so more GPUs '
+                 'would each take a slice of the batch with the weights replicated). Use --gpus 1.')
+
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.exit('bench.py: no GPU visible')
+    from oracle import oracle
+
+    wl = args.workload
+    if wl == 'calib_mfma':
+        tops, ghz, ms_ev, blocks, iters = calibrate_mfma(torch)
+        print(json.dumps({
+            'metric': 'int8_mfma_calibration_tops', 'value': float(f'{tops:.6g}'), 'unit': 'TOP/s', 'n_gpus': 1, 'steps': 20,
+            'warmup': 5, 'ms_per_step': round(ms_ev, 5), 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
+            'dtype': 'int8', 'data': 'synthetic',
+            'config': {'workload': f'calib_mfma: {blocks} workgroups x 4 waves x {iters} x 16 v_mfma_i32_32x32x32_i8 on '
+                                   'register-resident operands, no memory traffic'},
+            'roofline': {'bound': 'mfma', 'achieved': round(tops, 3), 'peak': PEAK_INT8_TOPS, 'unit': 'TOP/s',
+                         'frac': round(tops / PEAK_INT8_TOPS, 4), 'traffic': None, 'kernel': 'calib_mfma_i8_kernel',
+                         'kernel_ms': round(ms_ev, 5)},
+            'clock_ghz_under_mfma_load': round(ghz, 3), 'cpu_baseline': None}), flush=True)
+        return
+
+    w = prepare(wl, torch)
+    ms, value, roof, graphed = measure(torch, w, args.steps, args.warmup, args.eager)
+    unit, samples, bit_exact = w['unit'], w['samples'], w['bit_exact']
 
     cpu = None
-    if cpu_fn is not None and not args.no_cpu_baseline:
-        t = _time_cpu(cpu_fn)
+    if w['cpu_fn'] is not None and not args.no_cpu_baseline:
+        t = _time_cpu(w['cpu_fn'])
         if unit in ('TOP/s', 'TFLOP/s'):
-            v = cpu_work / t / 1e12
+            v = w['cpu_work'] / t / 1e12
         elif unit == 'GB/s':
-            v = cpu_work / t / 1e9
+            v = w['cpu_work'] / t / 1e9
         else:
-            v = (cpu_samples or samples) / t
+            v = (w['cpu_samples'] or samples) / t
         cpu = {'value': float(f'{v:.6g}'), 'unit': unit, 'cores': oracle.num_threads(), 'kind': 'port',
-               'sample': cpu_desc, 'host_cpus': os.cpu_count()}
+               'sample': w['cpu_desc'], 'host_cpus': os.cpu_count()}
 
     line = {
-        'metric': metric, 'value': float(f'{value:.6g}'), 'unit': unit, 'n_gpus': 1, 'steps': args.steps,
+        'metric': w['metric'], 'value': float(f'{value:.6g}'), 'unit': unit, 'n_gpus': 1, 'steps': args.steps,
         'warmup': args.warmup, 'ms_per_step': round(ms, 5), 'higher_is_better': True, 'scaling': 'weak',
-        'vs_baseline': None, 'dtype': {'c2_dense_i16': 'int16', 'c2_dense_i16x16': 'int16', 'c2_dense_bf16': 'bf16', 'c2_dense_fp8': 'fp8'}.get(wl, 'int8'), 'data': 'synthetic', 'config': config,
+        'vs_baseline': None, 'dtype': {'c2_dense_i16': 'int16', 'c2_dense_i16x16': 'int16', 'c2_dense_bf16': 'bf16', 'c2_dense_fp8': 'fp8'}.get(wl, 'int8'), 'data': 'synthetic', 'config': w['config'],
         'samples_per_s': float(f'{samples / (ms * 1e-3):.6g}'), 'bit_exact': bit_exact,
         'roofline': roof, 'cpu_baseline': cpu, 'launch': 'hip_graph' if graphed else 'eager',
     }
-    line.update(extra)
+    line.update(w['extra'])
+    all_exact = bit_exact
+
+    if wl == 'c2_dense' and not args.only:
+        # what this box's matrix cores sustain with no memory traffic, next to the data-sheet peak
+        tops, ghz, _, _, _ = calibrate_mfma(torch)
+        roof['calibrated_peak'] = round(tops, 1)
+        roof['frac_of_calibrated'] = round(roof['achieved'] / tops, 4)
+        roof['clock_ghz_under_mfma_load'] = round(ghz, 3)
+        # the other configurations: same timing method and step count, no CPU leg
+        del w
+        others = {}
+        for name in ALSO:
+            torch.cuda.empty_cache()
+            try:
+                o = prepare(name, torch)
+                o_ms, o_value, o_roof, _ = measure(torch, o, args.steps, args.warmup, args.eager)
+                others[name] = {'value': float(f'{o_value:.6g}'), 'unit': o['unit'], 'ms_per_step': round(o_ms, 5),
+                                'bit_exact': o['bit_exact'], 'roofline': {k: o_roof[k] for k in ('bound', 'achieved', 'peak', 'unit', 'frac', 'kernel')}}
+                all_exact = all_exact and o['bit_exact']
+                del o
+            except Exception as exc:  # noqa: BLE001
+                others[name] = {'error': f'{type(exc).__name__}: {exc}'}
+                all_exact = False
+        line['workloads'] = others
+
     print(json.dumps(line), flush=True)
-    if not bit_exact:
-        sys.exit('bench.py: GPU result differs from the oracle — throughput above is INVALID')
+    if not all_exact:
+        sys.exit('bench.py: a GPU result differs from the oracle (or a workload failed) — throughput above is INVALID')
 
 
 if __name__ == '__main__':

@@ -30,6 +30,8 @@ def run_graph(model, oracle, inputs):
         if node.op_type == 'dense':
             W, bias = inst.variant.quantize_weight_bias(inst)
             x = vals[input_tensor_for_role(node, 'lhs').name]
+            if cfg.flags.transpose_lhs:  # the operand is consumed through a last-two-axes transpose view
+                x = np.ascontiguousarray(np.swapaxes(x, -1, -2))
             x2 = x.reshape(-1, x.shape[-1])
             shifts = np.array(cfg.shift_per_channel) if cfg.shift_per_channel is not None else cfg.shift
             y = oracle.dense(x2, W, bias, shifts, cfg.rounding_mode, relu=cfg.flags.use_relu,
@@ -37,6 +39,8 @@ def run_graph(model, oracle, inputs):
             vals[out] = y.reshape(x.shape[:-1] + (y.shape[-1],))
         elif node.op_type == 'matmul':
             a = vals[input_tensor_for_role(node, 'lhs').name]
+            if cfg.flags.transpose_lhs:
+                a = np.ascontiguousarray(np.swapaxes(a, -1, -2))
             b = vals[input_tensor_for_role(node, 'rhs').name]
             vals[out] = oracle.matmul(a, b, cfg.shift, cfg.rounding_mode, trans_b=cfg.flags.transpose_rhs,
                                       out=cfg.precision['output'].format)

@@ -467,3 +467,59 @@ def test_fanout_graph_with_two_outputs(oracle, mode, in_shape):
         np.testing.assert_array_equal(got[name].reshape(want[name].shape), want[name].astype(np.int64))
     deq = model.predict(x.astype(np.float64) / 32.0)
     np.testing.assert_array_equal(deq[y1.name], got[y1.name] / 4.0)
+
+
+def test_int16_input_with_8bit_layers_is_not_planned_as_fused_mlp(oracle):
+    """int16 activations x int8 weights accumulate in acc32 like the 8-bit case, but the fused MLP launch only reads
+    8-bit inputs: a chain whose head takes an int16 tensor and whose layers write int8 runs layer by layer."""
+    r = np.random.default_rng(31)
+    gb = GraphBuilder()
+    t = gb.input('x', (48, 40), qint(16, 8))
+    dims = [40, 64, 32, 6]
+    for i in range(3):
+        W = r.integers(-100, 100, (dims[i], dims[i + 1])) / 128.0
+        b = r.integers(-512, 512, dims[i + 1]) / 2.0 ** (15 if i == 0 else 11)
+        t = gb.dense(t, W, qint(8, 7), qint(8, 4), bias=b, bias_precision=qint(32, 15 if i == 0 else 11), relu=i < 2, name=f'fc{i}')
+    gb.output(t)
+    model = gb.build()
+    model.compile()
+    chains = model.context.config['gpu_fusion_plan']['mlp_chains']
+    assert all('fc0_aie' not in c for c in chains)
+    x = r.integers(-3000, 3000, (48, 40)).astype(np.int16)
+    _graph_check(model, oracle, {'x': x})
+
+
+def test_attention_with_unaligned_head_slices_runs_unfused(oracle):
+    """Heads cut from a packed projection at offsets that are not multiples of 16 bytes (an 8-column prefix in front of
+    Q): the fused attention launch needs 16-byte aligned head slices, so the planner must leave these heads to the
+    separate MatMul / Softmax / MatMul launches (decided at run time, on the views' addresses); a logit shift above
+    24 must do the same (decided by the planner)."""
+    r = np.random.default_rng(37)
+    batch, seq, heads, d = 2, 64, 2, 64
+    width = 8 + 3 * heads * d
+    for shift_case in ('unaligned', 'deep_shift'):
+        gb = GraphBuilder()
+        x = gb.input('x', (batch, seq, width), qint(8, 4))
+        if shift_case == 'unaligned':
+            _pad, q, k, v = gb.split(x, -1, [8, heads * d, heads * d, heads * d], name='qkv_split')
+        else:
+            q, k, v, _pad = gb.split(x, -1, [heads * d, heads * d, heads * d, 8], name='qkv_split')
+        qs, ks, vs = (gb.split(t, -1, [d] * heads, name=f'{n}_heads') for t, n in ((q, 'q'), (k, 'k'), (v, 'v')))
+        outs = []
+        for h in range(heads):
+            kt = gb.transpose(ks[h], (0, 2, 1), name=f'kt{h}')
+            # acc frac 8; deep_shift: output frac -17 -> shift 25, beyond what the fused kernel takes
+            lg = gb.matmul(qs[h], kt, qint(8, -3 if shift_case == 'unaligned' else -17), name=f'qk{h}')
+            lg = gb.scale(lg, 2.0 ** (-5 if shift_case == 'unaligned' else -19), name=f'temp{h}')  # EXP_KQ = 92
+            pr = gb.softmax(lg, qint(8, 8, signed=False), name=f'sm{h}')
+            outs.append(gb.matmul(pr, vs[h], qint(8, 4), name=f'pv{h}'))
+        gb.output(gb.concat(outs, -1, name='cat'))
+        model = gb.build()
+        model.compile()
+        plan = model.context.config['gpu_fusion_plan']['attention']
+        if shift_case == 'deep_shift':
+            assert plan == []
+        # 'unaligned': the planner sees head offsets inside the nearest source tensor only (0, 64 of a 128-wide slice);
+        # that the slice itself starts 8 bytes into rows of 392 bytes shows at run time, where the executor falls back
+        xin = np.clip(np.rint(r.normal(0, 24, (batch, seq, width))), -128, 127).astype(np.int8)
+        _graph_check(model, oracle, {'x': xin})
