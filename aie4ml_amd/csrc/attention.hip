@@ -64,6 +64,12 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
     extern __shared__ __attribute__((aligned(16))) int8_t attn_smem[];
     int8_t* vt = attn_smem;                                        // V^T, k-permuted: [D][PITCH]
     int* colsum = reinterpret_cast<int*>(attn_smem + D * PITCH);   // sum_k V[k][n]
+    // The 512-key form holds 64 logit and up to 128 score registers per lane at once; with everything else that is
+    // a handful more than the 256 a lane has, and the compiler's spills went to scratch memory (18 MB of extra HBM
+    // writes per launch). The scores of the last PARK tiles wait in LDS instead: slot s of thread t at dword
+    // s * THREADS + t, so every access is conflict free.
+    constexpr int PARK = (NT >= 16 && BANKED) ? 3 : 0;
+    unsigned* parked = reinterpret_cast<unsigned*>(colsum + D);
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int m = lane & 31, half = lane >> 5;
@@ -216,8 +222,13 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
                 e3 = *reinterpret_cast<const int*>(tbytes + byte_x4<3>(d4, two));
             }
             sum += (e0 + e1) + (e2 + e3);
-            ep[t][2 * g] = pack2_halves(e0, e1);
-            ep[t][2 * g + 1] = pack2_halves(e2, e3);
+            if (t >= NT - PARK) {
+                parked[((t - (NT - PARK)) * 8 + 2 * g) * THREADS + tid] = pack2_halves(e0, e1);
+                parked[((t - (NT - PARK)) * 8 + 2 * g + 1) * THREADS + tid] = pack2_halves(e2, e3);
+            } else {
+                ep[t][2 * g] = pack2_halves(e0, e1);
+                ep[t][2 * g + 1] = pack2_halves(e2, e3);
+            }
         }
         // keep the scheduler from hoisting many tiles' lookups at once (their results would spill)
         if (NT >= 16 && (t & 1)) __builtin_amdgcn_sched_barrier(0);
@@ -233,6 +244,10 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
         v4i pf;
+        if (t >= NT - PARK) {  // own slots only: no barrier needed
+#pragma unroll
+            for (int r = 0; r < 8; ++r) ep[t][r] = parked[((t - (NT - PARK)) * 8 + r) * THREADS + tid];
+        }
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             if (FASTP) {
@@ -323,7 +338,8 @@ static void launch_attention_nt(int grid, int grid8, size_t lds, hipStream_t str
 
 template <int DT>
 static int launch_attention(int nt, int grid, int grid8, hipStream_t stream, const AttnArgs& a) {
-    const size_t lds = static_cast<size_t>(DT * 32) * (nt * 32 + 16) + DT * 32 * 4;  // V^T + column sums
+    size_t lds = static_cast<size_t>(DT * 32) * (nt * 32 + 16) + DT * 32 * 4;  // V^T + column sums
+    if (nt >= 16 && grid8 > 0) lds += 3 * 8 * 512 * sizeof(unsigned);            // + three parked score tiles per thread
     switch (nt) {
     case 1: launch_attention_nt<1, DT>(grid, 0, lds, stream, a); break;
     case 2: launch_attention_nt<2, DT>(grid, 0, lds, stream, a); break;
