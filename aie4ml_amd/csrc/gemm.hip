@@ -44,7 +44,11 @@ struct GemmCfg {
     static_assert(WTM % 32 == 0 && WTN % 32 == 0 && BK % 32 == 0, "wave tile must be whole 32x32x32 MFMA blocks");
 };
 
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool RAGGED = false>
+// TRANS_A: the left operand is stored transposed, [K][lda] with the rows of the product contiguous (TRANSPOSE_A of the
+// reference kernels, matmul.cpp:60-66 / dense_bias_relu.cpp:95-101). Its tile is then fetched as 4 (k) x 4 (m) byte
+// blocks, four dword loads along m, transposed in registers (v_perm) and written to LDS as four dwords along k, so the
+// MFMA side sees the usual [m][k] tile. Rows (m >= M) and reduction positions (k >= K) outside the operand read as zero.
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool RAGGED = false, bool TRANS_A = false>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_i8_nt_kernel(GemmArgs g) {
     using Cfg = GemmCfg<BM, BN, BK, WAVES_M, WAVES_N>;
     extern __shared__ __attribute__((aligned(16))) int8_t smem[];
@@ -102,8 +106,58 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_i8_nt_kernel(GemmA
         offb[i] = row * Cfg::PITCH + kc * 16;
     }
 
+    // TRANS_A: 4 x 4 blocks of the [k][m] tile; block b of a thread covers k = 4 * (b / (BM/4)) .., m = 4 * (b % (BM/4)) ..
+    constexpr int TA_BLOCKS = TRANS_A ? (BM / 4) * (BK / 4) / Cfg::NT : 1;
+    static_assert(!TRANS_A || ((BM / 4) * (BK / 4)) % Cfg::NT == 0, "transposed tile blocks must divide over the threads");
+    unsigned ta[TA_BLOCKS][4];
+    auto load_a_transposed = [&](int k0) {
+#pragma unroll
+        for (int b = 0; b < TA_BLOCKS; ++b) {
+            const int blk = tid + b * Cfg::NT;
+            const int mq = (blk % (BM / 4)) * 4, kq = (blk / (BM / 4)) * 4;
+            const int m = m0 + mq;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int k = k0 + kq + i;
+                unsigned w = 0;
+                if (k < g.K && m < g.M) {
+                    const int8_t* src = Ab + static_cast<int64_t>(k) * g.lda + m;
+                    if (g.ragged_a == 0 && m + 4 <= g.M) {
+                        w = *reinterpret_cast<const unsigned*>(src);
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            if (m + j < g.M) w |= static_cast<unsigned>(static_cast<uint8_t>(src[j])) << (8 * j);
+                    }
+                }
+                ta[b][i] = w;
+            }
+        }
+    };
+    auto store_a_transposed = [&](int buf) {
+#pragma unroll
+        for (int b = 0; b < TA_BLOCKS; ++b) {
+            const int blk = tid + b * Cfg::NT;
+            const int mq = (blk % (BM / 4)) * 4, kq = (blk / (BM / 4)) * 4;
+            // in: ta[b][i] byte j = A^T[k + i][m + j]; out: c[j] byte i = the same element, k-contiguous for row m + j
+            const unsigned lo01 = __builtin_amdgcn_perm(ta[b][1], ta[b][0], 0x05010400u);
+            const unsigned hi01 = __builtin_amdgcn_perm(ta[b][1], ta[b][0], 0x07030602u);
+            const unsigned lo23 = __builtin_amdgcn_perm(ta[b][3], ta[b][2], 0x05010400u);
+            const unsigned hi23 = __builtin_amdgcn_perm(ta[b][3], ta[b][2], 0x07030602u);
+            const unsigned c[4] = {__builtin_amdgcn_perm(lo23, lo01, 0x05040100u), __builtin_amdgcn_perm(lo23, lo01, 0x07060302u),
+                                   __builtin_amdgcn_perm(hi23, hi01, 0x05040100u), __builtin_amdgcn_perm(hi23, hi01, 0x07060302u)};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) *reinterpret_cast<unsigned*>(smem + buf * BUF + (mq + j) * Cfg::PITCH + kq) = c[j];
+        }
+    };
+
     auto load_tile = [&](int k0) {
-        if constexpr (RAGGED) {
+        if constexpr (TRANS_A) {
+            static_assert(!TRANS_A || RAGGED, "the transposed-A form takes B through the ragged loads");
+            load_a_transposed(k0);
+#pragma unroll
+            for (int i = 0; i < Cfg::B_PER_T; ++i) rb[i] = load_chunk_ragged(pb[i] + k0, g.K - (k0 + kb[i]), g.ragged_b);
+        } else if constexpr (RAGGED) {
 #pragma unroll
             for (int i = 0; i < Cfg::A_PER_T; ++i) ra[i] = load_chunk_ragged(pa[i] + k0, g.K - (k0 + ka[i]), g.ragged_a);
 #pragma unroll
@@ -118,8 +172,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_i8_nt_kernel(GemmA
         }
     };
     auto store_tile = [&](int buf) {
+        if constexpr (TRANS_A) store_a_transposed(buf);
 #pragma unroll
-        for (int i = 0; i < Cfg::A_PER_T; ++i) *reinterpret_cast<v4i*>(smem + buf * BUF + offa[i]) = ra[i];
+        for (int i = 0; i < (TRANS_A ? 0 : Cfg::A_PER_T); ++i) *reinterpret_cast<v4i*>(smem + buf * BUF + offa[i]) = ra[i];
 #pragma unroll
         for (int i = 0; i < Cfg::B_PER_T; ++i) *reinterpret_cast<v4i*>(smem + buf * BUF + B_OFF + offb[i]) = rb[i];
     };
@@ -558,10 +613,10 @@ __global__ __launch_bounds__(256) void clear_i32_kernel(int32_t* __restrict__ p,
 
 static inline int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
 
-template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool RAGGED = false>
+template <int BM, int BN, int BK, int WAVES_M, int WAVES_N, bool RAGGED = false, bool TRANS_A = false>
 static hipError_t launch_tiled(const GemmArgs& g, int batch, hipStream_t stream) {
     using Cfg = GemmCfg<BM, BN, BK, WAVES_M, WAVES_N>;
-    auto kern = gemm_i8_nt_kernel<BM, BN, BK, WAVES_M, WAVES_N, RAGGED>;
+    auto kern = gemm_i8_nt_kernel<BM, BN, BK, WAVES_M, WAVES_N, RAGGED, TRANS_A>;
     static bool attr_set = false;  // benign race: the attribute is idempotent
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -700,6 +755,15 @@ static hipError_t launch_ragged(GemmArgs g, int batch, hipStream_t stream) {
     return launch_tiled<128, 128, 64, 2, 2, true>(g, batch, stream);
 }
 
+// Left operand stored transposed ([K][lda]): the tiled kernel with the in-register tile transpose.
+static hipError_t launch_trans_a(GemmArgs g, int batch, hipStream_t stream) {
+    // ragged_a here: 0 = rows of A^T are 4-byte aligned (dword loads along m), else byte loads
+    const uintptr_t a = reinterpret_cast<uintptr_t>(g.A);
+    g.ragged_a = (g.lda % 4 == 0 && g.stride_a % 4 == 0 && a % 4 == 0) ? 0 : 2;
+    g.ragged_b = ragged_mode(g.Bt, g.ldb, g.stride_b, g.K);
+    return launch_tiled<128, 128, 64, 2, 2, true, true>(g, batch, stream);
+}
+
 static bool out_kind_ok(int k) { return k == A4G_I8 || k == A4G_U8 || k == A4G_I16; }
 
 }  // namespace a4g
@@ -732,7 +796,7 @@ extern "C" int a4g_pack_weights_i8(const int8_t* W, int64_t ldw, int64_t K, int6
     return check_hip(hipGetLastError(), "a4g_pack_weights_i8");
 }
 
-extern "C" int a4g_dense_i8(const void* A, int a_kind, int64_t lda, const int8_t* Wt, int64_t ldwt, const int32_t* colsum,
+extern "C" int a4g_dense_i8(const void* A, int a_kind, int trans_a, int64_t lda, const int8_t* Wt, int64_t ldwt, const int32_t* colsum,
                             const int32_t* bias, const int32_t* shifts, int n_shift, int round_mode, int relu, int out_kind,
                             void* Y, int64_t ldy, int64_t M, int64_t N, int64_t K, a4g_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
@@ -745,7 +809,7 @@ extern "C" int a4g_dense_i8(const void* A, int a_kind, int64_t lda, const int8_t
     A4G_REQUIRE(valid_round(round_mode), A4G_ERR_INVALID_ARGUMENT, "%s: unknown rounding mode %d", who, round_mode);
     A4G_REQUIRE(n_shift == 1 || n_shift == N, A4G_ERR_INVALID_ARGUMENT, "%s: n_shift must be 1 or N=%lld, got %d", who,
                 (long long)N, n_shift);
-    A4G_REQUIRE(lda >= K && ldy >= N && ldwt >= K, A4G_ERR_INVALID_ARGUMENT, "%s: pitch smaller than the row", who);
+    A4G_REQUIRE(lda >= (trans_a ? M : K) && ldy >= N && ldwt >= K, A4G_ERR_INVALID_ARGUMENT, "%s: pitch smaller than the row", who);
     if (M == 0) return A4G_OK;
     A4G_REQUIRE(A && Wt && Y && shifts, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
     A4G_REQUIRE(a_kind != A4G_U8 || colsum, A4G_ERR_INVALID_ARGUMENT, "%s: uint8 activations need the packed colsum vector",
@@ -772,7 +836,9 @@ extern "C" int a4g_dense_i8(const void* A, int a_kind, int64_t lda, const int8_t
 
     const bool tiled = K % 16 == 0 && lda % 16 == 0 && ldwt % 16 == 0 && aligned16(A) && aligned16(Wt);
     hipError_t e;
-    if (tiled) {
+    if (trans_a) {
+        e = launch_trans_a(g, 1, stream);
+    } else if (tiled) {
         e = launch_gemm_nt(g, 1, stream, env_variant());
     } else {
         e = launch_ragged(g, 1, stream);
@@ -819,7 +885,7 @@ int static_scratch(const char* who, void** out) {
 
 // Body of both MatMul entry points. `own_scratch`: the workspace is the library's static scratch array rather than
 // a caller's buffer; it is resolved here, after validation and only when the problem needs it.
-static int matmul_i8_impl(const char* who, bool own_scratch, const void* A, int a_kind, int64_t lda, int64_t stride_a,
+static int matmul_i8_impl(const char* who, bool own_scratch, const void* A, int a_kind, int trans_a, int64_t lda, int64_t stride_a,
                           const int8_t* B, int64_t ldb, int64_t stride_b, int trans_b, void* C, int64_t ldc, int64_t stride_c,
                           int64_t batch, int64_t M, int64_t N, int64_t K, int shift, int round_mode, int out_kind,
                           void* workspace, size_t workspace_bytes, hipStream_t stream) {
@@ -833,13 +899,13 @@ static int matmul_i8_impl(const char* who, bool own_scratch, const void* A, int 
     A4G_REQUIRE(valid_round(round_mode), A4G_ERR_INVALID_ARGUMENT, "%s: unknown rounding mode %d", who, round_mode);
     A4G_REQUIRE(shift >= 0 && shift <= 31, A4G_ERR_INVALID_ARGUMENT,
                 "%s: accumulator output shift must be in [0,31], got %d", who, shift);
-    A4G_REQUIRE(lda >= K && ldc >= N && ldb >= (trans_b ? K : N), A4G_ERR_INVALID_ARGUMENT, "%s: pitch smaller than the row",
-                who);
+    A4G_REQUIRE(lda >= (trans_a ? M : K) && ldc >= N && ldb >= (trans_b ? K : N), A4G_ERR_INVALID_ARGUMENT,
+                "%s: pitch smaller than the row", who);
     if (batch == 0 || M == 0) return A4G_OK;
     A4G_REQUIRE(A && B && C, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
 
     // the two attention shapes have kernels of their own that need neither workspace nor K-loop barriers
-    if (out_kind != A4G_I16 && env_variant() == 0) {
+    if (out_kind != A4G_I16 && env_variant() == 0 && !trans_a) {
         LeanArgs la{};
         la.A = static_cast<const int8_t*>(A);
         la.B = B;
@@ -903,7 +969,9 @@ static int matmul_i8_impl(const char* who, bool own_scratch, const void* A, int 
         g.Bt = B;
         g.ldb = ldb;
         g.stride_b = stride_b;
-        if (a_ok && ldb % 16 == 0 && stride_b % 16 == 0 && aligned16(B)) {
+        if (trans_a) {
+            e = launch_trans_a(g, static_cast<int>(batch), stream);
+        } else if (a_ok && ldb % 16 == 0 && stride_b % 16 == 0 && aligned16(B)) {
             e = launch_gemm_nt(g, static_cast<int>(batch), stream, env_variant());
         } else {
             e = launch_ragged(g, static_cast<int>(batch), stream);
@@ -915,25 +983,27 @@ static int matmul_i8_impl(const char* who, bool own_scratch, const void* A, int 
         g.Bt = ws;
         g.ldb = ldt;
         g.stride_b = N * ldt;
-        e = a_ok ? launch_gemm_nt(g, static_cast<int>(batch), stream, env_variant()) : launch_ragged(g, static_cast<int>(batch), stream);
+        e = trans_a ? launch_trans_a(g, static_cast<int>(batch), stream)
+            : a_ok  ? launch_gemm_nt(g, static_cast<int>(batch), stream, env_variant())
+                    : launch_ragged(g, static_cast<int>(batch), stream);
     }
     return check_hip(e, who);
 }
 
-extern "C" int a4g_matmul_i8(const void* A, int a_kind, int64_t lda, int64_t stride_a, const int8_t* B, int64_t ldb,
+extern "C" int a4g_matmul_i8(const void* A, int a_kind, int trans_a, int64_t lda, int64_t stride_a, const int8_t* B, int64_t ldb,
                              int64_t stride_b, int trans_b, void* C, int64_t ldc, int64_t stride_c, int64_t batch, int64_t M,
                              int64_t N, int64_t K, int shift, int round_mode, int out_kind, void* workspace,
                              size_t workspace_bytes, a4g_stream_t stream_) {
-    return matmul_i8_impl("a4g_matmul_i8", false, A, a_kind, lda, stride_a, B, ldb, stride_b, trans_b, C, ldc, stride_c, batch, M,
+    return matmul_i8_impl("a4g_matmul_i8", false, A, a_kind, trans_a, lda, stride_a, B, ldb, stride_b, trans_b, C, ldc, stride_c, batch, M,
                           N, K, shift, round_mode, out_kind, workspace, workspace_bytes, static_cast<hipStream_t>(stream_));
 }
 
-extern "C" int a4g_matmul_i8_static(const void* A, int a_kind, int64_t lda, int64_t stride_a, const int8_t* B, int64_t ldb,
+extern "C" int a4g_matmul_i8_static(const void* A, int a_kind, int trans_a, int64_t lda, int64_t stride_a, const int8_t* B, int64_t ldb,
                                     int64_t stride_b, int trans_b, void* C, int64_t ldc, int64_t stride_c, int64_t batch,
                                     int64_t M, int64_t N, int64_t K, int shift, int round_mode, int out_kind,
                                     a4g_stream_t stream_) {
     // Nothing in the array has to start at zero: the repack writes every byte the GEMM reads (rows are zero padded
     // to the packed pitch) and the column-sum kernel stores, never accumulates.
-    return matmul_i8_impl("a4g_matmul_i8_static", true, A, a_kind, lda, stride_a, B, ldb, stride_b, trans_b, C, ldc, stride_c,
+    return matmul_i8_impl("a4g_matmul_i8_static", true, A, a_kind, trans_a, lda, stride_a, B, ldb, stride_b, trans_b, C, ldc, stride_c,
                           batch, M, N, K, shift, round_mode, out_kind, nullptr, 0, static_cast<hipStream_t>(stream_));
 }

@@ -261,10 +261,9 @@ class DenseGpuVariant(OpImplVariant):
 
         cfg = inst.config
         x = inputs[input_tensor_for_role(inst.node, 'lhs').name]
-        if cfg.flags.transpose_lhs:
-            x = x.transpose(-1, -2).contiguous()
+        # a transposed left operand (io_view perm) is read as stored: the kernel transposes its tiles (dense_bias_relu.cpp:95-101)
         y = ops.dense(x, inst.artifacts['packed_weights'], cfg.rounding_mode, relu=cfg.flags.use_relu,
-                      out_kind=cfg.precision['output'].format)
+                      out_kind=cfg.precision['output'].format, trans_a=cfg.flags.transpose_lhs)
         return {inst.node.outputs[0].name: y}
 
 
@@ -328,11 +327,14 @@ class MatmulGpuVariant(OpImplVariant):
         lhs_t, rhs_t = input_tensor_for_role(node, 'lhs'), input_tensor_for_role(node, 'rhs')
         a = inputs[lhs_t.name]
         b = inst.artifacts['rhs_const'] if rhs_t.is_parameter else inputs[rhs_t.name]
-        if cfg.flags.transpose_lhs:
-            a = a.transpose(-1, -2).contiguous()
-        out_shape = tuple(a.shape[:-1]) + (int(b.shape[-2] if cfg.flags.transpose_rhs else b.shape[-1]),)
+        ta = bool(cfg.flags.transpose_lhs)
+        if ta and b.dim() == 2 and a.dim() > 2:
+            a, ta = a.transpose(-1, -2).contiguous(), False  # shared rank-2 RHS: rows of every leading index are stacked below
+        rows_shape = tuple(a.shape[:-2]) + ((int(a.shape[-1]),) if ta else (int(a.shape[-2]),))
+        out_shape = rows_shape + (int(b.shape[-2] if cfg.flags.transpose_rhs else b.shape[-1]),)
         if b.dim() == 2 and a.dim() > 2:
             a = a.reshape(-1, a.shape[-1])  # rank-2 RHS is shared by every leading index of the LHS
+        # a transposed left operand (io_view perm) is read as stored: the kernel transposes its tiles (matmul.cpp:60-66)
         y = ops.matmul(a, b, cfg.shift, cfg.rounding_mode, trans_b=cfg.flags.transpose_rhs,
-                       out_kind=cfg.precision['output'].format)
+                       out_kind=cfg.precision['output'].format, trans_a=ta)
         return {node.outputs[0].name: y.reshape(out_shape)}

@@ -121,8 +121,29 @@ def pack_dense(weight: torch.Tensor, bias: Optional[torch.Tensor], shifts) -> Pa
 
 
 def dense(x: torch.Tensor, p: PackedDense, rounding='floor', relu: bool = False, out_kind='int8',
-          out: Optional[torch.Tensor] = None):
-    """y = saturate(round((x @ W + bias) >> shift)), optionally ReLU. x: [..., K] int8 / uint8 / int16."""
+          out: Optional[torch.Tensor] = None, trans_a: bool = False):
+    """y = saturate(round((x @ W + bias) >> shift)), optionally ReLU. x: [..., K] int8 / uint8 / int16.
+    ``trans_a``: x is [..., K, M], the operand is consumed through a last-two-axes transpose view; 8-bit operands are
+    transposed inside the kernel, one launch per leading index."""
+    if trans_a:
+        _dev(x, 'x')
+        if x.dim() < 2 or int(x.shape[-2]) != p.K:
+            raise ValueError(f'dense input (transposed) has {tuple(x.shape)}, weights expect {p.K} on the second-to-last axis')
+        if x.dtype not in (torch.int8, torch.uint8) or p.wt_lo is not None:
+            # 16-bit operands: no transposing kernel yet, the view is materialised first
+            return dense(x.transpose(-1, -2).contiguous(), p, rounding, relu, out_kind, out)
+        xs = x.contiguous().reshape(-1, p.K, int(x.shape[-1]))
+        Mt = int(xs.shape[-1])
+        ok = _kind(out_kind)
+        if out is None:
+            out = torch.empty(tuple(x.shape[:-2]) + (Mt, p.N), dtype=_KIND_TORCH[ok], device=x.device)
+        ys = out.reshape(-1, Mt, p.N)
+        L = _lib.load()
+        for i in range(int(xs.shape[0])):
+            check(L.a4g_dense_i8(_ptr(xs[i]), _TORCH_KIND[xs.dtype], 1, Mt, _ptr(p.wt), p.ldwt, _ptr(p.colsum), _ptr(p.bias),
+                                 _ptr(p.shifts), int(p.shifts.numel()), _mode(rounding), int(bool(relu)), ok, _ptr(ys[i]), p.N,
+                                 Mt, p.N, p.K, _stream()))
+        return out
     x2 = _rows2d(x, 'x')
     if x2.dtype not in (torch.int8, torch.uint8, torch.int16):
         raise NotImplementedError(f'dense activations must be int8, uint8 or int16, got {x2.dtype}')
@@ -147,17 +168,20 @@ def dense(x: torch.Tensor, p: PackedDense, rounding='floor', relu: bool = False,
                                         _ptr(p.bias), _ptr(p.shifts), int(p.shifts.numel()), _mode(rounding),
                                         int(bool(relu)), ok, _ptr(y2), y2.stride(0) if M > 0 else p.N, M, p.N, p.K, _stream()))
         return out
-    check(_lib.load().a4g_dense_i8(_ptr(x2), _TORCH_KIND[x2.dtype], x2.stride(0) if M > 0 else p.K, _ptr(p.wt), p.ldwt,
+    check(_lib.load().a4g_dense_i8(_ptr(x2), _TORCH_KIND[x2.dtype], 0, x2.stride(0) if M > 0 else p.K, _ptr(p.wt), p.ldwt,
                                    _ptr(p.colsum), _ptr(p.bias), _ptr(p.shifts), int(p.shifts.numel()), _mode(rounding),
                                    int(bool(relu)), ok, _ptr(y2), y2.stride(0) if M > 0 else p.N, M, p.N, p.K, _stream()))
     return out
 
 
 def matmul(a: torch.Tensor, b: torch.Tensor, shift: int, rounding='floor', trans_b: bool = False, out_kind='int8',
-           out: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None):
+           out: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None, trans_a: bool = False):
     """Batched dynamic MatMul. a: [..., M, K] int8/uint8/int16; b: [..., K, N] int8 (int16 with an int16 a), or [..., N, K] when
-    ``trans_b`` (the operand is consumed through a last-two-axes transpose view)."""
+    ``trans_b`` (the operand is consumed through a last-two-axes transpose view). ``trans_a``: a is [..., K, M]; an
+    8-bit operand is transposed inside the kernel, a 16-bit one is materialised first."""
     _dev(a, 'a'), _dev(b, 'b')
+    if trans_a and a.dtype == torch.int16:
+        a, trans_a = a.transpose(-1, -2).contiguous(), False
     if b.dtype not in (torch.int8, torch.int16):
         raise ValueError('matmul RHS must use a signed integer precision.')
     if a.dtype not in (torch.int8, torch.uint8, torch.int16):
@@ -167,7 +191,7 @@ def matmul(a: torch.Tensor, b: torch.Tensor, shift: int, rounding='floor', trans
     if a.dim() < 2 or b.dim() < 2:
         raise ValueError('matmul operands need rank >= 2')
     a, b = a.contiguous(), b.contiguous()
-    M, K = int(a.shape[-2]), int(a.shape[-1])
+    M, K = (int(a.shape[-1]), int(a.shape[-2])) if trans_a else (int(a.shape[-2]), int(a.shape[-1]))
     N = int(b.shape[-2] if trans_b else b.shape[-1])
     Kb = int(b.shape[-1] if trans_b else b.shape[-2])
     if K != Kb:
@@ -196,7 +220,8 @@ def matmul(a: torch.Tensor, b: torch.Tensor, shift: int, rounding='floor', trans
     if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
         workspace = torch.empty((need,), dtype=torch.uint8, device=a.device)
     ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
-    check(L.a4g_matmul_i8(_ptr(a), akind, K, M * K, _ptr(b), int(b.shape[-1]), K * N, int(bool(trans_b)), _ptr(out), N,
+    check(L.a4g_matmul_i8(_ptr(a), akind, int(bool(trans_a)), M if trans_a else K, M * K, _ptr(b), int(b.shape[-1]), K * N,
+                          int(bool(trans_b)), _ptr(out), N,
                           M * N, batch, M, N, K, int(shift), _mode(rounding), ok, _ptr(workspace), ws_bytes, _stream()))
     return out
 

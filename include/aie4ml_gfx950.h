@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define A4G_VERSION 100 /* major*10000 + minor*100 + patch */
+#define A4G_VERSION 200 /* major*10000 + minor*100 + patch */
 
 #if defined(__GNUC__)
 #define A4G_API __attribute__((visibility("default")))
@@ -99,14 +99,16 @@ A4G_API int a4g_pack_weights_i8(const int8_t* W, int64_t ldw, int64_t K, int64_t
  * Replaces dense_single/first/middle/last<Cfg>::run, templates/nnet_utils/dense_bias_relu/
  * dense_bias_relu.cpp:66-430, configured by _DenseVariantBase.resolve
  * (op_impls/families/matmul/dense.py:94-133) through variants/dense_bias_relu/parameters.h.jinja.
- *   A       [M][lda]  int8 or uint8 (a_kind)
+ *   A       [M][lda]  int8 or uint8 (a_kind); with trans_a != 0 the operand is stored transposed, [K][lda] with
+ *           lda >= M, and is transposed inside the kernel while its tiles are staged (TRANSPOSE_A,
+ *           dense_bias_relu.cpp:95-101, set from an io_view permutation of the input, dense.py:94-133)
  *   Wt      packed weights from a4g_pack_weights_i8, pitch ldwt
  *   colsum  [N] from a4g_pack_weights_i8; required iff a_kind == A4G_U8, else may be NULL
  *   bias    [N] int32 at accumulator scale, or NULL (USE_BIAS = false)
  *   shifts  [n_shift] int32 on the device; n_shift == 1 (the reference's scalar SHIFT) or == N
  *           (per-output-channel extension; identical to the reference when all entries are equal)
  *   Y       [M][ldy]  out_kind in {A4G_I8, A4G_U8, A4G_I16} */
-A4G_API int a4g_dense_i8(const void* A, int a_kind, int64_t lda, const int8_t* Wt, int64_t ldwt,
+A4G_API int a4g_dense_i8(const void* A, int a_kind, int trans_a, int64_t lda, const int8_t* Wt, int64_t ldwt,
                  const int32_t* colsum, const int32_t* bias, const int32_t* shifts, int n_shift,
                  int round_mode, int relu, int out_kind, void* Y, int64_t ldy, int64_t M, int64_t N,
                  int64_t K, a4g_stream_t stream);
@@ -135,7 +137,9 @@ A4G_API int a4g_dense_i16x16(const int16_t* A, int64_t lda, const int8_t* Wt_hi,
  * C[b] = saturate(round((A[b] x B[b]) >> shift)), no bias, no ReLU, for b in [0, batch).
  * Replaces matmul_single/first/middle/last<Cfg>::run, templates/nnet_utils/matmul/matmul.cpp:31-390,
  * configured by _MatmulVariantBase.resolve (op_impls/families/matmul/matmul.py:47-98).
- *   A  [batch][M][lda]  int8 or uint8 (a_kind; uint8 = softmax probabilities)
+ *   A  [batch][M][lda]  int8 or uint8 (a_kind; uint8 = softmax probabilities). trans_a != 0: stored as
+ *      [batch][K][lda], lda >= M — the left operand arrives as the last-two-axes transpose of its producer
+ *      (TRANSPOSE_A, matmul.cpp:60-66; flag from matmul.py:78-81) and is transposed in-kernel, tile by tile.
  *   B  signed int8 (matmul.py:96-98). trans_b == 0: [batch][K][ldb] (logical K x N).
  *      trans_b == 1: [batch][N][ldb] — the operand arrives as the last-two-axes transpose of the
  *      producer tensor (io_view perm, matmul.py:86-95 / TRANSPOSE_B, matmul.cpp:70-76).
@@ -144,7 +148,7 @@ A4G_API int a4g_dense_i16x16(const int16_t* A, int64_t lda, const int8_t* Wt_hi,
  * independent per-slice products. `workspace` must hold a4g_matmul_i8_workspace_bytes(...) bytes
  * (0 for some argument combinations, in which case it may be NULL). */
 A4G_API size_t a4g_matmul_i8_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int trans_b, int a_kind);
-A4G_API int a4g_matmul_i8(const void* A, int a_kind, int64_t lda, int64_t stride_a, const int8_t* B, int64_t ldb,
+A4G_API int a4g_matmul_i8(const void* A, int a_kind, int trans_a, int64_t lda, int64_t stride_a, const int8_t* B, int64_t ldb,
                   int64_t stride_b, int trans_b, void* C, int64_t ldc, int64_t stride_c, int64_t batch,
                   int64_t M, int64_t N, int64_t K, int shift, int round_mode, int out_kind, void* workspace,
                   size_t workspace_bytes, a4g_stream_t stream);
@@ -159,7 +163,7 @@ A4G_API int a4g_matmul_i8(const void* A, int a_kind, int64_t lda, int64_t stride
  * streams, different threads) race; the array keeps the last call's contents and nothing in it needs clearing. The
  * array's address is resolved on the first call on each device, which should be made outside stream capture. */
 #define A4G_MATMUL_I8_STATIC_MAX_BYTES (16u << 20)
-A4G_API int a4g_matmul_i8_static(const void* A, int a_kind, int64_t lda, int64_t stride_a, const int8_t* B, int64_t ldb,
+A4G_API int a4g_matmul_i8_static(const void* A, int a_kind, int trans_a, int64_t lda, int64_t stride_a, const int8_t* B, int64_t ldb,
                          int64_t stride_b, int trans_b, void* C, int64_t ldc, int64_t stride_c, int64_t batch,
                          int64_t M, int64_t N, int64_t K, int shift, int round_mode, int out_kind, a4g_stream_t stream);
 

@@ -169,12 +169,12 @@ def parse(data: bytes):
 
 def _quantize_linear(x, scale, zp):
     info = np.iinfo(zp.dtype)
-    q = np.rint(np.asarray(x, dtype=np.float64) / np.float64(scale)) + np.float64(zp)  # rint: half to even
+    q = np.rint(np.asarray(x, dtype=np.float64) / np.asarray(scale, np.float64)) + np.asarray(zp, np.float64)  # rint: half to even
     return np.clip(q, info.min, info.max).astype(zp.dtype)
 
 
 def _dequantize_linear(x, scale, zp):
-    return (np.asarray(x, dtype=np.float64) - np.float64(zp)) * np.float64(scale)
+    return (np.asarray(x, dtype=np.float64) - np.asarray(zp, np.float64)) * np.asarray(scale, np.float64)
 
 
 def _softmax(x, axis):

@@ -46,7 +46,7 @@ def test_binding_table_matches_header(libpath):
 
     assert sorted(_lib.SIGNATURES) == declared_symbols()
     lib = _lib.load()
-    assert lib.a4g_version() == 100
+    assert lib.a4g_version() == 200
     assert lib.a4g_packed_ld(1) == 16 and lib.a4g_packed_ld(16) == 16 and lib.a4g_packed_ld(17) == 32
     # pure host-side query, no GPU needed: K x N operand transposed into the workspace + colsum
     assert lib.a4g_matmul_i8_workspace_bytes(2, 8, 64, 512, 1, 0) == 0
@@ -80,14 +80,14 @@ def test_argument_validation_happens_before_any_launch(libpath):
     assert st == _lib.A4G_ERR_INVALID_ARGUMENT and b'eps_q0' in lib.a4g_last_error()
     st = lib.a4g_layernorm_i8(None, None, None, None, 4, 64, 1, 7, 16, 6, None)  # out_shift > 15
     assert st == _lib.A4G_ERR_INVALID_ARGUMENT and b'out_shift' in lib.a4g_last_error()
-    st = lib.a4g_dense_i8(None, 2, 16, None, 16, None, None, None, 1, 0, 0, 0, None, 16, 4, 16, 16, None)  # int16 lhs
+    st = lib.a4g_dense_i8(None, 2, 0, 16, None, 16, None, None, None, 1, 0, 0, 0, None, 16, 4, 16, 16, None)  # int16 lhs
     assert st == _lib.A4G_ERR_UNSUPPORTED
     with pytest.raises(NotImplementedError):
         _lib.check(st)
     # the entry point without a workspace validates like a4g_matmul_i8, before it looks at the device
-    st = lib.a4g_matmul_i8_static(None, 0, 16, 0, None, 16, 0, 0, None, 16, 0, 1, 4, 16, 16, 40, 0, 0, None)  # shift 40
+    st = lib.a4g_matmul_i8_static(None, 0, 0, 16, 0, None, 16, 0, 0, None, 16, 0, 1, 4, 16, 16, 40, 0, 0, None)  # shift 40
     assert st == _lib.A4G_ERR_INVALID_ARGUMENT and b'a4g_matmul_i8_static' in lib.a4g_last_error()
-    assert lib.a4g_matmul_i8_static(None, 0, 16, 0, None, 16, 0, 0, None, 16, 0, 0, 4, 16, 16, 3, 0, 0, None) == 0  # batch 0
+    assert lib.a4g_matmul_i8_static(None, 0, 0, 16, 0, None, 16, 0, 0, None, 16, 0, 0, 4, 16, 16, 3, 0, 0, None) == 0  # batch 0
     # empty problems are fine and do nothing
     assert lib.a4g_add(None, None, None, 0, 0, 0, 0, None) == 0
     assert lib.a4g_layernorm_i8(None, None, None, None, 0, 64, 1, 7, 5, 6, None) == 0

@@ -215,6 +215,41 @@ def test_matmul_batched(ops, oracle, shape, trans_b):
         assert np.array_equal(got, oracle.matmul(A, B, 6, mode, trans_b=trans_b))
 
 
+@pytest.mark.parametrize('a_unsigned', [False, True])
+@pytest.mark.parametrize('trans_b', [True, False])
+@pytest.mark.parametrize('shape', [((2, 3), 64, 64, 64), ((4,), 128, 96, 32), ((), 130, 70, 48), ((2,), 50, 17, 24),
+                                   ((3,), 33, 64, 19), ((), 517, 260, 203), ((2,), 256, 128, 320)])
+def test_matmul_transposed_lhs_in_kernel(ops, oracle, shape, trans_b, a_unsigned):
+    """The left operand stored as [..., K, M] (matmul.cpp:60-66, TRANSPOSE_A): the kernel transposes its tiles; the
+    oracle gets the materialised transpose. Row counts off the dword grid take the byte loads."""
+    lead, M, N, K = shape
+    r = rng(M + 2 * N + 3 * K)
+    At = r.integers(0, 256, lead + (K, M)).astype(np.uint8) if a_unsigned else gauss8(r, 40, lead + (K, M))
+    B = gauss8(r, 24, lead + ((N, K) if trans_b else (K, N)))
+    A = np.ascontiguousarray(np.swapaxes(At, -1, -2))
+    for mode, out in (('conv_even', 'int8'), ('floor', 'int16')):
+        got = host(ops.matmul(dev(At), dev(B), 7, mode, trans_b=trans_b, out_kind=out, trans_a=True))
+        assert np.array_equal(got, oracle.matmul(A, B, 7, mode, trans_b=trans_b, out=out))
+
+
+@pytest.mark.parametrize('shape', [((), 64, 64, 64), ((3,), 130, 70, 48), ((2, 2), 33, 19, 100), ((), 1000, 200, 512)])
+def test_dense_transposed_lhs_in_kernel(ops, oracle, shape):
+    """Dense whose input arrives through a last-two-axes transpose view (dense_bias_relu.cpp:95-101), with bias,
+    per-channel shifts and ReLU, signed and unsigned activations."""
+    lead, M, N, K = shape
+    r = rng(7 * M + N + K)
+    W = gauss8(r, 16, (K, N))
+    bias = r.integers(-20000, 20000, N).astype(np.int32)
+    shifts = r.integers(5, 11, N).astype(np.int32)
+    p = ops.pack_dense(dev(W), dev(bias), shifts)
+    for unsigned in (False, True):
+        Xt = r.integers(0, 256, lead + (K, M)).astype(np.uint8) if unsigned else gauss8(r, 32, lead + (K, M))
+        X = np.ascontiguousarray(np.swapaxes(Xt, -1, -2))
+        got = host(ops.dense(dev(Xt), p, 'conv_even', relu=True, trans_a=True))
+        want = oracle.dense(X.reshape(-1, K), W, bias, shifts, 'conv_even', relu=True).reshape(lead + (M, N))
+        assert np.array_equal(got, want)
+
+
 @pytest.mark.parametrize('trans_b', [True, False])
 def test_matmul_unsigned_lhs(ops, oracle, trans_b):
     r = rng(9)

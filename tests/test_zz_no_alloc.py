@@ -18,7 +18,7 @@ def _call(lib_fn, a, b, out, shift, mode, trans_b, out_kind, extra):
     batch, M, K = a.shape
     N = b.shape[1] if trans_b else b.shape[2]
     akind = _lib.KIND['uint8' if a.dtype == torch.uint8 else 'int8']
-    st = lib_fn(a.data_ptr(), akind, K, M * K, b.data_ptr(), b.shape[2], b.shape[1] * b.shape[2], int(trans_b), out.data_ptr(), N,
+    st = lib_fn(a.data_ptr(), akind, 0, K, M * K, b.data_ptr(), b.shape[2], b.shape[1] * b.shape[2], int(trans_b), out.data_ptr(), N,
                 M * N, batch, M, N, K, shift, _lib.ROUNDING[mode], _lib.KIND[out_kind], *extra,
                 torch.cuda.current_stream().cuda_stream)
     _lib.check(st)
@@ -80,7 +80,7 @@ def test_static_matmul_rejects_operands_beyond_the_array():
     a = torch.zeros((batch, M, K), dtype=torch.int8, device='cuda')
     b = torch.zeros((batch, K, N), dtype=torch.int8, device='cuda')
     out = torch.zeros((batch, M, N), dtype=torch.int8, device='cuda')
-    st = L.a4g_matmul_i8_static(a.data_ptr(), 0, K, M * K, b.data_ptr(), N, K * N, 0, out.data_ptr(), N, M * N, batch, M, N, K, 8, 6,
+    st = L.a4g_matmul_i8_static(a.data_ptr(), 0, 0, K, M * K, b.data_ptr(), N, K * N, 0, out.data_ptr(), N, M * N, batch, M, N, K, 8, 6,
                                 0, torch.cuda.current_stream().cuda_stream)
     assert st == _lib.A4G_ERR_WORKSPACE
     assert b'static scratch array holds' in L.a4g_last_error()
