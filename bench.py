@@ -119,9 +119,11 @@ def prepare(wl, torch):
     cpu_work = cpu_desc = None
     peak_mfma, mfma_unit = PEAK_INT8_TOPS, 'TOP/s'
 
-    if wl == 'c2_dense':
+    if wl in ('c2_dense', 'c2_dense_zero'):
         M, K, N = 8192, 4096, 4096
         A, W, bias, shifts = workloads.c2_dense(M, K, N)
+        if wl == 'c2_dense_zero':  # power-limit probe: see main()
+            A, W = np.zeros_like(A), np.zeros_like(W)
         p = ops.pack_dense(dev(W), dev(bias), shifts)
         dA = dev(A)
         out = torch.empty((M, N), dtype=torch.int8, device='cuda')
@@ -134,8 +136,8 @@ def prepare(wl, torch):
         bit_exact = bool(np.array_equal(out[torch.from_numpy(rows).cuda()].cpu().numpy(), exp))
         work, unit_work, bound = 2.0 * M * N * K, 'op', 'mfma'
         samples = M
-        config = {'workload': 'c2_dense: Dense 8192x4096 -> 4096, int8, bias, per-channel shift 8..12, conv_even, '
-                              'sat int8, ReLU'}
+        config = {'workload': f'{wl}: Dense 8192x4096 -> 4096, int8, bias, per-channel shift 8..12, conv_even, '
+                              'sat int8, ReLU' + (' (all-zero operands)' if wl == 'c2_dense_zero' else '')}
         sample_rows = 2048  # about 1 s per pass on 16 host threads, 10 s with the repeats
         cpu_desc = f'oracle Dense on the first {sample_rows} of {M} rows (same W/bias/shifts), scaled per op'
         cpu_fn = lambda: oracle.dense(A[:sample_rows], W, bias, shifts, 'conv_even', relu=True)  # noqa: E731
@@ -549,6 +551,15 @@ def main():
         roof['calibrated_peak'] = round(tops, 1)
         roof['frac_of_calibrated'] = round(roof['achieved'] / tops, 4)
         roof['clock_ghz_under_mfma_load'] = round(ghz, 3)
+        # The same kernel, same shape, all-zero operands: identical instruction stream and memory traffic, but the
+        # multipliers do not toggle. The difference to the headline is what the board's power limit takes for
+        # full-entropy int8 operands (the clock drops under load; the schedule itself sustains the zero-operand rate).
+        z = prepare('c2_dense_zero', torch)
+        _, z_value, z_roof, _ = measure(torch, z, args.steps, args.warmup, args.eager)
+        roof['zero_operand_tops'] = round(z_roof['achieved'], 1)
+        roof['zero_operand_frac'] = z_roof['frac']
+        all_exact = all_exact and z['bit_exact']
+        del z
         # the other configurations: same timing method and step count, no CPU leg
         del w
         others = {}
