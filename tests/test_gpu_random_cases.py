@@ -166,3 +166,32 @@ def test_attention_random_case(ops, oracle, seed):
     exp = oracle.matmul(p, v, oshift, omode)
     got = host(ops.attention(dev(q), dev(k), dev(v), lshift, lmode, sm, oshift, omode))
     assert np.array_equal(got, exp), (seed, lead, sq, sk, lshift, lmode, oshift, omode, sm)
+
+
+@pytest.mark.parametrize('seed', range(24 + EXTRA))
+def test_transposed_lhs_random_case(ops, oracle, seed):
+    """MatMul and Dense whose left operand is stored [K][M] (transposed inside the kernel): shapes around the tile
+    sizes, M off the dword grid (byte loads), every rounding mode, signed and unsigned operands."""
+    r = np.random.default_rng(7000 + seed)
+    M, N, K = int(r.choice(M_CHOICES[:10])), int(r.choice(N_CHOICES)), int(r.choice(K_CHOICES))
+    a_dtype = np.uint8 if seed % 3 == 2 else np.int8
+    mode = str(r.choice(MODES))
+    kind = str(r.choice(['int8', 'uint8', 'int16']))
+    batch = int(r.choice([1, 2, 3]))
+    At = draw(r, a_dtype, (batch, K, M))
+    A = np.ascontiguousarray(np.swapaxes(At, -1, -2))
+    if seed % 2 == 0:
+        trans_b = bool(r.random() < 0.5)
+        B = draw(r, np.int8, (batch, N, K) if trans_b else (batch, K, N))
+        shift = int(r.integers(0, 20))
+        got = ops.matmul(dev(At), dev(B), shift, mode, trans_b=trans_b, out_kind=kind, trans_a=True)
+        exp = oracle.matmul(A, B, shift, mode, trans_b=trans_b, out=kind)
+    else:
+        W = draw(r, np.int8, (K, N))
+        bias = r.integers(-2**24, 2**24, N).astype(np.int32)
+        shifts = r.integers(0, 20, N).astype(np.int32)
+        relu = bool(r.random() < 0.5)
+        p = ops.pack_dense(dev(W), dev(bias), shifts)
+        got = ops.dense(dev(At), p, mode, relu=relu, out_kind=kind, trans_a=True)
+        exp = oracle.dense(A.reshape(-1, K), W, bias, shifts, mode, relu=relu, out=kind).reshape(batch, M, N)
+    assert np.array_equal(host(got), exp), (seed, a_dtype, batch, M, N, K, mode, kind)
