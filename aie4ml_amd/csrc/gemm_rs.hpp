@@ -410,6 +410,11 @@ static hipError_t launch_rs_policy(const GemmArgs& g, int batch, hipStream_t str
 // shares). g.A points at the int16 matrix, g.lda / g.stride_a are in bytes, g.K counts elements (K % 128 == 0),
 // g.colsum holds the column sums of the weights. False when the shape or the number of tiles does not suit it.
 bool rs_i16i8_applicable(const GemmArgs& g, int batch);
+
+// Dense with a short reduction on many rows: weights in registers, activations streamed (gemm_wreg.hip). One problem
+// (no batch), int8 / uint8 activations and outputs.
+bool wreg_applicable(const GemmArgs& g);
+hipError_t launch_wreg(const GemmArgs& g, hipStream_t stream);
 hipError_t launch_rs_i16i8(const GemmArgs& g, int batch, hipStream_t stream);
 
 }  // namespace a4g

@@ -188,6 +188,65 @@ def test_dense_width_multiple_of_192(ops, oracle):
     run_dense(ops, oracle, 7100, 256, 768, 'symmetric_inf', a_dtype=np.uint8, out='int16', seed=42)
 
 
+# Reductions of one to six 128-byte tiles with one-byte outputs take the kernel that keeps the weights in registers:
+# every reduction length, runs of rows that end in a 64-row step or mid-tile, widths that are not whole column blocks,
+# both activation types, and the encoder's projection shapes at full size.
+@pytest.mark.parametrize('case', [
+    (4096, 128, 4096, 'conv_even', np.int8), (4096, 256, 4096, 'symmetric_inf', np.int8), (4096, 384, 4096, 'symmetric_inf', np.uint8),
+    (4096, 512, 4096, 'conv_odd', np.int8), (4096, 640, 4096, 'floor', np.uint8), (4173, 256, 4112, 'conv_even', np.int8),
+    (4173, 384, 4112, 'conv_odd', np.uint8), (8192, 768, 2304, 'conv_even', np.int8), (8192, 768, 3072, 'conv_even', np.uint8),
+    (8192, 768, 768, 'symmetric_zero', np.int8), (1, 256, 128, 'conv_even', np.int8), (63, 768, 16, 'conv_even', np.int8),
+    (65, 640, 144, 'positive_inf', np.uint8), (193, 768, 272, 'negative_inf', np.int8), (2048, 768, 768, 'ceil', np.int8),
+    (320, 512, 3088, 'conv_even', np.uint8)], ids=lambda c: 'x'.join(str(v) for v in c[:3]))
+def test_dense_short_reduction_weights_in_registers(ops, oracle, case):
+    M, K, N, mode, a_dtype = case
+    run_dense(ops, oracle, M, K, N, mode, a_dtype=a_dtype, relu=(M % 2 == 0), out='int8' if a_dtype == np.int8 else 'uint8',
+              seed=M + K + N)
+
+
+@pytest.mark.parametrize('mode', MODES)
+@pytest.mark.parametrize('shift_set', ['1..15', 'with zero', 'beyond 15', 'large bias'])
+def test_dense_short_reduction_requantisation_forms(ops, oracle, mode, shift_set):
+    # the quick form (shifts 1..15, start values below 2^30) and the general one, with accumulators on exact ties and, for
+    # 'large bias', next to both int32 extremes
+    r = rng(57)
+    M, K, N = 200, 384, 272
+    A = gauss8(r, 40, (M, K))
+    W = gauss8(r, 30, (K, N))
+    W[:, ::3] = 0  # those columns give srs(bias) exactly
+    lo, hi = {'1..15': (1, 16), 'with zero': (0, 16), 'beyond 15': (0, 25), 'large bias': (1, 16)}[shift_set]
+    shifts = r.integers(lo, hi, N).astype(np.int32)
+    shifts[:hi - lo] = np.arange(lo, hi)
+    bias = r.integers(-2**20, 2**20, N).astype(np.int64)
+    bias[6::12] = (1 << shifts[6::12].astype(np.int64)) // 2 * r.choice([-3, -1, 1, 3], len(bias[6::12]))
+    if shift_set == 'large bias':
+        bias[0::12] = 2**31 - 1 - r.integers(0, 70000, len(bias[0::12]))
+        bias[3::12] = -2**31 + r.integers(0, 70000, len(bias[3::12]))
+        bias[9::12] = r.choice([2**30 - 1, 2**30, 2**30 + 1, -2**30, -2**30 - 1], len(bias[9::12]))
+    bias = bias.astype(np.int32)
+    p = ops.pack_dense(dev(W), dev(bias), shifts)
+    for out, relu in (('int8', False), ('uint8', False), ('int8', True)):
+        got = host(ops.dense(dev(A), p, mode, relu=relu, out_kind=out))
+        exp = oracle.dense(A, W, bias, shifts, mode, relu=relu, out=out)
+        assert np.array_equal(got, exp), (out, np.argwhere(got != exp)[:5])
+
+
+def test_dense_short_reduction_pitched_views(ops, oracle):
+    # activations and outputs that are column slices of wider tensors: row pitches larger than the rows
+    r = rng(58)
+    M, K, N = 700, 256, 400
+    A_full = gauss8(r, 40, (M, 3 * K))
+    W = gauss8(r, 30, (K, N))
+    b = r.integers(-2**14, 2**14, N).astype(np.int32)
+    p = ops.pack_dense(dev(W), dev(b), 7)
+    y_full = torch.zeros((M, 2 * N), dtype=torch.int8, device='cuda')
+    ops.dense(dev(A_full)[:, K:2 * K], p, 'conv_even', relu=True, out=y_full[:, N:])
+    exp = oracle.dense(np.ascontiguousarray(A_full[:, K:2 * K]), W, b, 7, 'conv_even', relu=True)
+    got = host(y_full)
+    assert np.array_equal(got[:, N:], exp)
+    assert not got[:, :N].any()
+
+
 def test_dense_nd_input_and_empty(ops, oracle):
     r = rng(6)
     A = gauss8(r, 30, (3, 5, 32))

@@ -14,7 +14,7 @@ pytestmark = pytest.mark.gpu
 MODES = ['floor', 'ceil', 'positive_inf', 'negative_inf', 'symmetric_inf', 'symmetric_zero', 'conv_even', 'conv_odd']
 M_CHOICES = [1, 7, 31, 64, 127, 128, 129, 255, 300, 513, 1000, 2049]
 N_CHOICES = [1, 17, 32, 64, 96, 128, 192, 200, 256, 384, 768, 1000]
-K_CHOICES = [1, 15, 16, 48, 64, 100, 128, 192, 256, 384, 1000, 1024]
+K_CHOICES = [1, 15, 16, 48, 64, 100, 128, 192, 256, 384, 1000, 1024, 512, 640, 768]
 EXTRA = int(os.environ.get('A4G_RANDOM_EXTRA', '0'))  # more seeds for a longer hunt
 
 
