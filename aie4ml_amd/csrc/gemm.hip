@@ -840,6 +840,8 @@ extern "C" int a4g_dense_i8(const void* A, int a_kind, int trans_a, int64_t lda,
         e = launch_trans_a(g, 1, stream);
     } else if (tiled && wreg_applicable(g)) {
         e = launch_wreg(g, stream);
+    } else if (tiled && sk_applicable(g) && sk_preferred(g)) {
+        e = launch_sk(g, stream);
     } else if (tiled) {
         e = launch_gemm_nt(g, 1, stream, env_variant());
     } else {

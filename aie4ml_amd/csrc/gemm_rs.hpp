@@ -415,6 +415,12 @@ bool rs_i16i8_applicable(const GemmArgs& g, int batch);
 // (no batch), int8 / uint8 activations and outputs.
 bool wreg_applicable(const GemmArgs& g);
 hipError_t launch_wreg(const GemmArgs& g, hipStream_t stream);
+
+// Dense with a long reduction on 128 x 192 tiles, the reduction split inside an eight-wave workgroup (gemm_sk.hip). One
+// problem (no batch), int8 / uint8 activations and outputs.
+bool sk_applicable(const GemmArgs& g);
+bool sk_preferred(const GemmArgs& g);
+hipError_t launch_sk(const GemmArgs& g, hipStream_t stream);
 hipError_t launch_rs_i16i8(const GemmArgs& g, int batch, hipStream_t stream);
 
 }  // namespace a4g

@@ -17,9 +17,7 @@
 #include <algorithm>
 #include <type_traits>
 
-#include "common.hpp"
-#include "gemm_epilogue.hpp"
-#include "gemm_rs.hpp"
+#include "gemm_direct.hpp"
 
 namespace a4g {
 
@@ -28,68 +26,9 @@ namespace {
 constexpr int WR_BM = 128, WR_BN = 128, WR_BK = 128, WR_NT = 256;
 constexpr int WR_STAGE = WR_BM * WR_BK;  // 16 KiB
 constexpr int WR_NST = 4;                // stages of the ring (power of two); three tiles are in flight
-#ifndef WR_WGS
-#define WR_WGS 512
-#endif
-
-// Per-column requantisation parameters in LDS: the accumulator's start value (bias + 128 * colsum), the constants of
-// RoundCfg, and the output range moved in front of the shift ([lo << s, (hi << s) + 2^s - 1]).
-struct WregParams {
-    int *add, *s, *c0, *cx, *bs, *lo_s, *hi_s;
-    __device__ __forceinline__ explicit WregParams(int8_t* base)
-        : add(reinterpret_cast<int*>(base)), s(add + WR_BN), c0(s + WR_BN), cx(c0 + WR_BN), bs(cx + WR_BN), lo_s(bs + WR_BN), hi_s(lo_s + WR_BN) {}
-    static constexpr int BYTES = 7 * 4 * WR_BN;
-};
+constexpr int WR_WGS = 512;               // two workgroups per CU
+using WregParams = DirectParams<WR_BN>;
 constexpr int WR_LDS = WR_NST * WR_STAGE + WregParams::BYTES;
-
-// Parks the parameters; returns (workgroup-uniform) whether some column needs the general requantisation: a shift
-// outside 1..15 or a start value so large that start + dot product + rounding offset could leave int32. Barrier inside.
-__device__ __forceinline__ bool wreg_park(const GemmArgs& g, const WregParams& wp, int tid, int col_add, int col_shift, int lo, int hi) {
-    int general = 0;
-    if (tid < WR_BN) {
-        const RoundCfg rc = make_round(g.mode, col_shift);
-        wp.add[tid] = col_add;
-        wp.s[tid] = rc.s;
-        wp.c0[tid] = rc.c0;
-        wp.cx[tid] = rc.cx;
-        wp.bs[tid] = rc.bs;
-        const int sc = min(max(rc.s, 0), 15);
-        wp.lo_s[tid] = static_cast<int>(static_cast<unsigned>(lo) << sc);
-        wp.hi_s[tid] = static_cast<int>((static_cast<unsigned>(hi) << sc) | ((1u << sc) - 1u));
-        general = rc.s < 1 || rc.s > 15 || col_add > (1 << 30) || col_add < -(1 << 30);
-    }
-    return __syncthreads_or(general) != 0;
-}
-
-// Four accumulators of four neighbouring columns -> four requantised bytes, for shifts within 1..15 and sums that stay
-// inside int32: rounding offset (BIT 0 none, 1 plus, 2 minus the tie bit, taken at bit s when CONV, else the sign), the
-// clamp in front of the shift, and a shift that writes its low byte straight into byte n of the result.
-template <int BIT, bool CONV>
-__device__ __forceinline__ unsigned wreg_requant4(int a0, int a1, int a2, int a3, const v4i& s4, const v4i& c04, const v4i& lo4,
-                                                  const v4i& hi4) {
-    auto pre = [&](int a, int t) {
-        int bit = 0;
-        if (BIT == 1) bit = static_cast<int>(__builtin_amdgcn_ubfe(static_cast<unsigned>(a), CONV ? s4[t] : 31, 1));
-        if (BIT == 2) bit = __builtin_amdgcn_sbfe(a, CONV ? s4[t] : 31, 1);
-        return clamp_med3(a + c04[t] + bit, lo4[t], hi4[t]);
-    };
-    unsigned packed;
-    {
-        const int v0 = pre(a0, 0);
-        asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:DWORD"
-            : "=v"(packed)
-            : "v"(s4[0]), "v"(v0));
-    }
-    shift_into_byte<1>(packed, pre(a1, 1), s4[1]);
-    shift_into_byte<2>(packed, pre(a2, 2), s4[2]);
-    shift_into_byte<3>(packed, pre(a3, 3), s4[3]);
-    return packed;
-}
-
-// Actual column (within a wave's 32) whose weights the lanes j and j + 32 supply as row j of the MFMA's first operand:
-// accumulator register 4g + i of lane (m, half) is output column 8g + 4half + i of the block, and we want that to be
-// actual column 16half + 4g + i, so that a lane's 16 registers are 16 neighbouring bytes of its output row.
-__device__ __forceinline__ int wreg_col_of_operand_row(int j) { return ((j >> 2) & 1) * 16 + (j >> 3) * 4 + (j & 3); }
 
 // One workgroup: one block of 128 output columns and a run of rows in 64-row halves, [h0, h1) of the `halves_m` halves
 // of the matrix; the `wgs_per_cb` workgroups of a column block share its rows as evenly as halves allow. Rows are
@@ -129,7 +68,7 @@ __global__ __launch_bounds__(WR_NT, 2) void gemm_wreg_kernel(GemmArgs g, int hal
     int koff[4];  // activation fragment of K step kk: row frow (+ 32 i), chunk 2 kk + half
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) koff[kk] = frow * WR_BK + (((kk * 2 + half) ^ ((frow >> 1) & 7)) * 16);
-    const int wrow = wave * 32 + wreg_col_of_operand_row(frow);  // weight fragment: this lane's column of the block
+    const int wrow = wave * 32 + direct_col_of_operand_row(frow);  // weight fragment: this lane's column of the block
 
     const int lo = g.relu ? max(kind_lo(g.out_kind), 0) : kind_lo(g.out_kind), hi = kind_hi(g.out_kind);
 
@@ -169,7 +108,7 @@ __global__ __launch_bounds__(WR_NT, 2) void gemm_wreg_kernel(GemmArgs g, int hal
     fetch_col_params<WR_BN, A_UNSIGNED>(g, tc, tid, col_add, col_shift);
 #pragma unroll
     for (int r = 0; r < 3; ++r) issue_ring(r);
-    const bool general = wreg_park(g, wp, tid, col_add, col_shift, lo, hi);
+    const bool general = direct_park<WR_BN>(g, wp, tid, col_add, col_shift, lo, hi);
 
     // ---- weights of this wave's 32 columns: ring -> registers
     v4i bw[NKS];
@@ -258,7 +197,7 @@ __global__ __launch_bounds__(WR_NT, 2) void gemm_wreg_kernel(GemmArgs g, int hal
                 const v4i hi4 = *reinterpret_cast<const v4i*>(wp.hi_s + nl + 4 * q);
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    acc[i][q] = static_cast<int>(wreg_requant4<BIT, CONV>(acc[i][q * 4], acc[i][q * 4 + 1], acc[i][q * 4 + 2], acc[i][q * 4 + 3], s4, c04, lo4, hi4));
+                    acc[i][q] = static_cast<int>(direct_requant4<BIT, CONV>(acc[i][q * 4], acc[i][q * 4 + 1], acc[i][q * 4 + 2], acc[i][q * 4 + 3], s4, c04, lo4, hi4));
                 __builtin_amdgcn_sched_barrier(0);  // one column group at a time: the weights leave few registers free
             }
         };
@@ -275,19 +214,7 @@ __global__ __launch_bounds__(WR_NT, 2) void gemm_wreg_kernel(GemmArgs g, int hal
                 const v4i bs4 = *reinterpret_cast<const v4i*>(wp.bs + nl + 4 * q);
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    int y[4];
-#pragma unroll
-                    for (int t = 0; t < 4; ++t) {
-                        const int a = static_cast<int>(static_cast<unsigned>(acc[i][q * 4 + t]) + static_cast<unsigned>(add4[t]));
-                        RoundCfg rc;
-                        rc.s = s4[t];
-                        rc.mask = (1u << s4[t]) - 1u;
-                        rc.c0 = c04[t];
-                        rc.cx = cx4[t];
-                        rc.bs = bs4[t];
-                        y[t] = clamp_i(apply_round(a, rc), lo, hi);
-                    }
-                    acc[i][q] = static_cast<int>(pack4_bytes(y[0], y[1], y[2], y[3]));
+                    acc[i][q] = static_cast<int>(direct_requant4_general(acc[i][q * 4], acc[i][q * 4 + 1], acc[i][q * 4 + 2], acc[i][q * 4 + 3], add4, s4, c04, cx4, bs4, lo, hi));
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }

@@ -231,6 +231,43 @@ def test_dense_short_reduction_requantisation_forms(ops, oracle, mode, shift_set
         assert np.array_equal(got, exp), (out, np.argwhere(got != exp)[:5])
 
 
+# Longer reductions on at most 256 tiles of 128 x 192 take the kernel that splits the reduction inside the workgroup.
+@pytest.mark.parametrize('case', [
+    (8192, 3072, 768, 'conv_even', np.int8), (8192, 3072, 768, 'conv_even', np.uint8), (8192, 1024, 768, 'symmetric_inf', np.int8),
+    (4096, 2048, 1536, 'conv_odd', np.uint8), (1000, 1152, 400, 'symmetric_zero', np.uint8), (129, 1024, 208, 'floor', np.int8),
+    (1, 1024, 16, 'conv_even', np.int8), (512, 4096, 1024, 'positive_inf', np.int8), (1024, 8192, 384, 'negative_inf', np.uint8),
+    (8192, 896, 768, 'ceil', np.int8)], ids=lambda c: 'x'.join(str(v) for v in c[:3]))
+def test_dense_long_reduction_split_in_workgroup(ops, oracle, case):
+    M, K, N, mode, a_dtype = case
+    run_dense(ops, oracle, M, K, N, mode, a_dtype=a_dtype, relu=(M % 2 == 0), out='int8' if a_dtype == np.int8 else 'uint8',
+              seed=M + K + N)
+
+
+@pytest.mark.parametrize('mode', MODES)
+@pytest.mark.parametrize('shift_set', ['1..15', 'beyond 15', 'large bias'])
+def test_dense_long_reduction_requantisation_forms(ops, oracle, mode, shift_set):
+    r = rng(59)
+    M, K, N = 200, 1280, 272
+    A = gauss8(r, 40, (M, K))
+    W = gauss8(r, 30, (K, N))
+    W[:, ::3] = 0  # those columns give srs(bias) exactly
+    lo, hi = {'1..15': (1, 16), 'beyond 15': (0, 25), 'large bias': (1, 16)}[shift_set]
+    shifts = r.integers(lo, hi, N).astype(np.int32)
+    shifts[:hi - lo] = np.arange(lo, hi)
+    bias = r.integers(-2**20, 2**20, N).astype(np.int64)
+    bias[6::12] = (1 << shifts[6::12].astype(np.int64)) // 2 * r.choice([-3, -1, 1, 3], len(bias[6::12]))
+    if shift_set == 'large bias':
+        bias[0::12] = 2**31 - 1 - r.integers(0, 70000, len(bias[0::12]))
+        bias[3::12] = -2**31 + r.integers(0, 70000, len(bias[3::12]))
+        bias[9::12] = r.choice([2**30 - 1, 2**30, 2**30 + 1, -2**30, -2**30 - 1], len(bias[9::12]))
+    bias = bias.astype(np.int32)
+    p = ops.pack_dense(dev(W), dev(bias), shifts)
+    for out, relu in (('int8', False), ('uint8', True)):
+        got = host(ops.dense(dev(A), p, mode, relu=relu, out_kind=out))
+        exp = oracle.dense(A, W, bias, shifts, mode, relu=relu, out=out)
+        assert np.array_equal(got, exp), (out, np.argwhere(got != exp)[:5])
+
+
 def test_dense_short_reduction_pitched_views(ops, oracle):
     # activations and outputs that are column slices of wider tensors: row pitches larger than the rows
     r = rng(58)
