@@ -19,8 +19,6 @@
 
 namespace a4g {
 
-namespace {
-
 constexpr int SK_BM = 128, SK_BN = 192, SK_BK = 64, SK_NT = 512;
 constexpr int SK_A = SK_BM * SK_BK, SK_W = SK_BN * SK_BK;  // 8 KiB + 12 KiB per stage
 constexpr int SK_STAGE = SK_A + SK_W;
@@ -267,8 +265,6 @@ hipError_t launch_sk_kernel(const GemmArgs& g, int tiles_m, int tiles_n, int a_b
     kern<<<tiles_m * tiles_n, SK_NT, SK_LDS, stream>>>(g, tiles_n, a_bytes, w_bytes);
     return hipGetLastError();
 }
-
-}  // namespace
 
 // Reductions in whole pairs of 64-byte tiles (one for each group), one-byte outputs, 16-byte aligned rows
 // on both sides, widths in whole 16-column pieces, operands small enough for 32-bit buffer offsets.

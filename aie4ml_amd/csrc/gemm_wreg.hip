@@ -21,8 +21,6 @@
 
 namespace a4g {
 
-namespace {
-
 constexpr int WR_BM = 128, WR_BN = 128, WR_BK = 128, WR_NT = 256;
 constexpr int WR_STAGE = WR_BM * WR_BK;  // 16 KiB
 constexpr int WR_NST = 4;                // stages of the ring (power of two); three tiles are in flight
@@ -257,8 +255,6 @@ hipError_t launch_wreg_nkt(const GemmArgs& g, int halves_m, int wgs_per_cb, int 
     return g.a_unsigned ? launch_wreg_kernel<NKT, true>(g, halves_m, wgs_per_cb, cbs, a_bytes, w_bytes, stream)
                         : launch_wreg_kernel<NKT, false>(g, halves_m, wgs_per_cb, cbs, a_bytes, w_bytes, stream);
 }
-
-}  // namespace
 
 // Reductions of one to six whole 128-byte tiles, one-byte outputs, 16-byte aligned rows on both sides, widths in whole
 // 16-column pieces, and operands small enough for 32-bit buffer offsets. Measured faster than the tiled kernel at every

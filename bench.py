@@ -106,6 +106,16 @@ def _time_cpu(fn, budget_s=12.0, min_runs=2):
     return float(np.median(times))
 
 
+# The four projections of the c5 encoder block as Dense workloads of their own (rows = batch 64 x seq 128): shape,
+# the kernel that runs them, and which projection it is.
+ENCODER_PROJECTIONS = {
+    'c5_proj_qkv': (8192, 768, 2304, 'gemm_wreg_kernel', 'fused Q/K/V projection'),
+    'c5_proj_out': (8192, 768, 768, 'gemm_wreg_kernel', 'attention output projection'),
+    'c5_ffn_up': (8192, 768, 3072, 'gemm_wreg_kernel', 'first feed-forward projection'),
+    'c5_ffn_down': (8192, 3072, 768, 'gemm_sk_kernel', 'second feed-forward projection'),
+}
+
+
 def prepare(wl, torch):
     """Builds one workload on the GPU, runs it once and checks it against the oracle. Returns a dict with the step
     function `fn`, the algorithmic work per step, the roofline that bounds it and what the CPU leg needs."""
@@ -119,8 +129,8 @@ def prepare(wl, torch):
     cpu_work = cpu_desc = None
     peak_mfma, mfma_unit = PEAK_INT8_TOPS, 'TOP/s'
 
-    if wl in ('c2_dense', 'c2_dense_zero'):
-        M, K, N = 8192, 4096, 4096
+    if wl in ('c2_dense', 'c2_dense_zero') or wl in ENCODER_PROJECTIONS:
+        M, K, N = ENCODER_PROJECTIONS[wl][:3] if wl in ENCODER_PROJECTIONS else (8192, 4096, 4096)
         A, W, bias, shifts = workloads.c2_dense(M, K, N)
         if wl == 'c2_dense_zero':  # power-limit probe: see main()
             A, W = np.zeros_like(A), np.zeros_like(W)
@@ -136,14 +146,15 @@ def prepare(wl, torch):
         bit_exact = bool(np.array_equal(out[torch.from_numpy(rows).cuda()].cpu().numpy(), exp))
         work, unit_work, bound = 2.0 * M * N * K, 'op', 'mfma'
         samples = M
-        config = {'workload': f'{wl}: Dense 8192x4096 -> 4096, int8, bias, per-channel shift 8..12, conv_even, '
-                              'sat int8, ReLU' + (' (all-zero operands)' if wl == 'c2_dense_zero' else '')}
+        config = {'workload': f'{wl}: Dense {M}x{K} -> {N}, int8, bias, per-channel shift 8..12, conv_even, '
+                              'sat int8, ReLU' + (' (all-zero operands)' if wl == 'c2_dense_zero' else '') +
+                              (f' (the {ENCODER_PROJECTIONS[wl][4]} of the c5 encoder block, alone)' if wl in ENCODER_PROJECTIONS else '')}
         sample_rows = 2048  # about 1 s per pass on 16 host threads, 10 s with the repeats
         cpu_desc = f'oracle Dense on the first {sample_rows} of {M} rows (same W/bias/shifts), scaled per op'
         cpu_fn = lambda: oracle.dense(A[:sample_rows], W, bias, shifts, 'conv_even', relu=True)  # noqa: E731
         cpu_work = 2.0 * sample_rows * N * K
         metric, unit = 'int8_dense_tops', 'TOP/s'
-        kernel = 'gemm_rs_kernel'
+        kernel = ENCODER_PROJECTIONS[wl][3] if wl in ENCODER_PROJECTIONS else 'gemm_rs_kernel'
     elif wl == 'c2_dense_i16':
         # the (16, 8) width combination on the C2 shape: int16 activations, int8 weights, int16 output
         M, K, N = 8192, 4096, 4096
@@ -480,7 +491,7 @@ def calibrate_mfma(torch, blocks_per_cu=2, iters=4096):
 
 # the other configurations, timed in the default run after the headline workload (same steps, no CPU leg)
 ALSO = ('c1_mlp', 'c3_qk', 'c3_softmax_exp', 'c3_softmax_hccs', 'c3_pv', 'c3_attention_exp', 'c4_add', 'c4_layernorm',
-        'c4_add_layernorm', 'c5_encoder')
+        'c4_add_layernorm', 'c5_encoder', 'c5_proj_qkv', 'c5_proj_out', 'c5_ffn_up', 'c5_ffn_down')
 
 
 def main():
@@ -569,7 +580,7 @@ def main():
                 o = prepare(name, torch)
                 o_ms, o_value, o_roof, _ = measure(torch, o, args.steps, args.warmup, args.eager)
                 others[name] = {'value': float(f'{o_value:.6g}'), 'unit': o['unit'], 'ms_per_step': round(o_ms, 5),
-                                'bit_exact': o['bit_exact'], 'roofline': {k: o_roof[k] for k in ('bound', 'achieved', 'peak', 'unit', 'frac', 'kernel')}}
+                                'bit_exact': o['bit_exact'], 'roofline': {k: o_roof[k] for k in ('bound', 'achieved', 'peak', 'unit', 'frac', 'traffic', 'traffic_source', 'kernel')}}
                 all_exact = all_exact and o['bit_exact']
                 del o
             except Exception as exc:  # noqa: BLE001
