@@ -42,7 +42,13 @@ __global__ __launch_bounds__(WR_NT, 2) void gemm_wreg_kernel(GemmArgs g, int hal
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int frow = lane & 31, half = lane >> 5;
 
-    const int cb = blockIdx.x / wgs_per_cb, part = blockIdx.x - cb * wgs_per_cb;
+    // Workgroups go to the eight XCDs round robin. Renumbered so that an XCD gets consecutive indices, and with the column
+    // block varying fastest, an XCD works on one slice of the rows for all column blocks: its L2 fetches those
+    // activation rows once instead of every XCD fetching all of them.
+    const int nb = gridDim.x, xcd = blockIdx.x & 7, per_xcd = nb >> 3, extra = nb & 7;
+    const int index = xcd * per_xcd + min(xcd, extra) + (blockIdx.x >> 3);
+    const int cbs = nb / wgs_per_cb;
+    const int part = index / cbs, cb = index - part * cbs;
     const int h0 = part * halves_m / wgs_per_cb, h1 = (part + 1) * halves_m / wgs_per_cb;
     const int n0 = cb * WR_BN;
     const int m0 = h0 * 64, m_end = min(g.M, h1 * 64);
