@@ -85,6 +85,7 @@ SIGNATURES = {
     'a4g_matmul_f': (_i32, [_vp, _i32, _i64, _i64, _vp, _i64, _i64, _i32, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _sz,
                             _vp]),
     'a4g_add_f': (_i32, [_vp, _vp, _vp, _i64, _i32, _vp]),
+    'a4g_transpose': (_i32, [_vp, _i32, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
     'a4g_calib_mfma_i8_ops': (_i64, [_i32, _i32]),
     'a4g_calib_mfma_i8': (_i32, [_i32, _i32, _vp, _vp, _vp]),
 }

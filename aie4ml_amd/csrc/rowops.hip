@@ -104,6 +104,54 @@ extern "C" int a4g_add(const void* a, const void* b, void* out, int64_t n, int k
     return check_hip(hipGetLastError(), "a4g_add launch");
 }
 
+// ---- transposes of 1-, 2- and 4-byte elements --------------------------------------------------------------
+// 64 x 64 tiles through LDS (one element of padding per row): both the reads and the writes are rows of a tile.
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_tiles_kernel(const T* __restrict__ src, int64_t ld_src, int64_t stride_src,
+                                                               T* __restrict__ dst, int64_t ld_dst, int64_t stride_dst, int rows,
+                                                               int cols) {
+    __shared__ T tile[64][65];
+    const int r0 = blockIdx.y * 64, c0 = blockIdx.x * 64;
+    const T* s = src + static_cast<int64_t>(blockIdx.z) * stride_src;
+    T* d = dst + static_cast<int64_t>(blockIdx.z) * stride_dst;
+    for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+        const int rr = i >> 6, cc = i & 63;
+        if (r0 + rr < rows && c0 + cc < cols) tile[rr][cc] = s[static_cast<int64_t>(r0 + rr) * ld_src + c0 + cc];
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < 64 * 64; i += 256) {
+        const int cc = i >> 6, rr = i & 63;
+        if (r0 + rr < rows && c0 + cc < cols) d[static_cast<int64_t>(c0 + cc) * ld_dst + r0 + rr] = tile[rr][cc];
+    }
+}
+
+extern "C" int a4g_transpose(const void* src, int elem_bytes, int64_t ld_src, int64_t stride_src, void* dst, int64_t ld_dst,
+                             int64_t stride_dst, int64_t batch, int64_t rows, int64_t cols, a4g_stream_t stream_) {
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const char* who = "a4g_transpose";
+    A4G_REQUIRE(elem_bytes == 1 || elem_bytes == 2 || elem_bytes == 4, A4G_ERR_UNSUPPORTED, "%s: elements of %d bytes", who,
+                elem_bytes);
+    A4G_REQUIRE(batch >= 0 && batch <= 65535 && rows >= 0 && cols >= 0 && rows <= (1 << 30) && cols <= (1 << 30) &&
+                    (rows + 63) / 64 <= 65535,
+                A4G_ERR_INVALID_ARGUMENT, "%s: bad shape batch=%lld rows=%lld cols=%lld", who, (long long)batch, (long long)rows,
+                (long long)cols);
+    A4G_REQUIRE(ld_src >= cols && ld_dst >= rows, A4G_ERR_INVALID_ARGUMENT, "%s: pitch smaller than the row", who);
+    if (batch == 0 || rows == 0 || cols == 0) return A4G_OK;
+    A4G_REQUIRE(src && dst, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+    const dim3 grid(static_cast<unsigned>((cols + 63) / 64), static_cast<unsigned>((rows + 63) / 64), static_cast<unsigned>(batch));
+    const int r = static_cast<int>(rows), c = static_cast<int>(cols);
+    if (elem_bytes == 1)
+        transpose_tiles_kernel<uint8_t><<<grid, 256, 0, stream>>>(static_cast<const uint8_t*>(src), ld_src, stride_src,
+                                                                  static_cast<uint8_t*>(dst), ld_dst, stride_dst, r, c);
+    else if (elem_bytes == 2)
+        transpose_tiles_kernel<uint16_t><<<grid, 256, 0, stream>>>(static_cast<const uint16_t*>(src), ld_src, stride_src,
+                                                                   static_cast<uint16_t*>(dst), ld_dst, stride_dst, r, c);
+    else
+        transpose_tiles_kernel<uint32_t><<<grid, 256, 0, stream>>>(static_cast<const uint32_t*>(src), ld_src, stride_src,
+                                                                   static_cast<uint32_t*>(dst), ld_dst, stride_dst, r, c);
+    return check_hip(hipGetLastError(), who);
+}
+
 namespace a4g {
 
 // =====================================================================================================

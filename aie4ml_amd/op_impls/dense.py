@@ -329,7 +329,7 @@ class MatmulGpuVariant(OpImplVariant):
         b = inst.artifacts['rhs_const'] if rhs_t.is_parameter else inputs[rhs_t.name]
         ta = bool(cfg.flags.transpose_lhs)
         if ta and b.dim() == 2 and a.dim() > 2:
-            a, ta = a.transpose(-1, -2).contiguous(), False  # shared rank-2 RHS: rows of every leading index are stacked below
+            a, ta = ops.transpose_last2(a), False  # shared rank-2 RHS: rows of every leading index are stacked below
         rows_shape = tuple(a.shape[:-2]) + ((int(a.shape[-1]),) if ta else (int(a.shape[-2]),))
         out_shape = rows_shape + (int(b.shape[-2] if cfg.flags.transpose_rhs else b.shape[-1]),)
         if b.dim() == 2 and a.dim() > 2:

@@ -195,7 +195,7 @@ class DenseFloatGpuVariant(OpImplVariant):
         cfg = inst.config
         x = inputs[input_tensor_for_role(inst.node, 'lhs').name]
         if cfg.flags.transpose_lhs:
-            x = x.transpose(-1, -2).contiguous()
+            x = ops.transpose_last2(x)
         return {inst.node.outputs[0].name: ops.dense_float(x, inst.artifacts['packed_weights'], relu=cfg.flags.use_relu)}
 
 
@@ -240,7 +240,7 @@ class MatmulFloatGpuVariant(OpImplVariant):
         a = inputs[lhs_t.name]
         b = inst.artifacts['rhs_const'] if rhs_t.is_parameter else inputs[rhs_t.name]
         if cfg.flags.transpose_lhs:
-            a = a.transpose(-1, -2).contiguous()
+            a = ops.transpose_last2(a)
         out_shape = tuple(a.shape[:-1]) + (int(b.shape[-2] if cfg.flags.transpose_rhs else b.shape[-1]),)
         if b.dim() == 2 and a.dim() > 2:
             a = a.reshape(-1, a.shape[-1])

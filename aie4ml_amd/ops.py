@@ -58,6 +58,24 @@ def _rows2d(t: torch.Tensor, name: str) -> torch.Tensor:
     return t2
 
 
+def transpose_last2(t: torch.Tensor) -> torch.Tensor:
+    """[..., R, C] -> a new contiguous [..., C, R] through the library's transpose kernel (elements of 1, 2 or 4 bytes):
+    how the 16-bit and floating-point operators take a left operand that the graph hands over transposed."""
+    _dev(t, 't')
+    if t.dim() < 2:
+        raise ValueError('transpose needs rank >= 2')
+    t = t.contiguous()
+    R, C = int(t.shape[-2]), int(t.shape[-1])
+    batch = t.numel() // max(R * C, 1)
+    out = torch.empty(tuple(t.shape[:-2]) + (C, R), dtype=t.dtype, device=t.device)
+    if t.numel():
+        src, dst = t.reshape(-1, R, C), out.reshape(-1, C, R)
+        for b0 in range(0, batch, 65535):  # the batch rides on gridDim.z
+            nb = min(65535, batch - b0)
+            check(_lib.load().a4g_transpose(_ptr(src[b0:]), t.element_size(), C, R * C, _ptr(dst[b0:]), R, R * C, nb, R, C, _stream()))
+    return out
+
+
 def add(a: torch.Tensor, b: torch.Tensor, shift: int = 0, rounding='floor', out: Optional[torch.Tensor] = None):
     """Saturating elementwise add of two tensors that share shape and storage type."""
     _dev(a, 'a'), _dev(b, 'b')
@@ -130,8 +148,8 @@ def dense(x: torch.Tensor, p: PackedDense, rounding='floor', relu: bool = False,
         if x.dim() < 2 or int(x.shape[-2]) != p.K:
             raise ValueError(f'dense input (transposed) has {tuple(x.shape)}, weights expect {p.K} on the second-to-last axis')
         if x.dtype not in (torch.int8, torch.uint8) or p.wt_lo is not None:
-            # 16-bit operands: no transposing kernel yet, the view is materialised first
-            return dense(x.transpose(-1, -2).contiguous(), p, rounding, relu, out_kind, out)
+            # 16-bit operands: the GEMM kernels take K-contiguous rows, the operand is transposed on the device first
+            return dense(transpose_last2(x), p, rounding, relu, out_kind, out)
         xs = x.contiguous().reshape(-1, p.K, int(x.shape[-1]))
         Mt = int(xs.shape[-1])
         ok = _kind(out_kind)
@@ -178,10 +196,10 @@ def matmul(a: torch.Tensor, b: torch.Tensor, shift: int, rounding='floor', trans
            out: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None, trans_a: bool = False):
     """Batched dynamic MatMul. a: [..., M, K] int8/uint8/int16; b: [..., K, N] int8 (int16 with an int16 a), or [..., N, K] when
     ``trans_b`` (the operand is consumed through a last-two-axes transpose view). ``trans_a``: a is [..., K, M]; an
-    8-bit operand is transposed inside the kernel, a 16-bit one is materialised first."""
+    8-bit operand is transposed inside the kernel, a 16-bit one by the library's transpose kernel first."""
     _dev(a, 'a'), _dev(b, 'b')
     if trans_a and a.dtype == torch.int16:
-        a, trans_a = a.transpose(-1, -2).contiguous(), False
+        a, trans_a = transpose_last2(a), False
     if b.dtype not in (torch.int8, torch.int16):
         raise ValueError('matmul RHS must use a signed integer precision.')
     if a.dtype not in (torch.int8, torch.uint8, torch.int16):

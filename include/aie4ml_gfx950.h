@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define A4G_VERSION 200 /* major*10000 + minor*100 + patch */
+#define A4G_VERSION 201 /* major*10000 + minor*100 + patch */
 
 #if defined(__GNUC__)
 #define A4G_API __attribute__((visibility("default")))
@@ -273,6 +273,16 @@ A4G_API int a4g_matmul_f(const void* A, int fmt, int64_t lda, int64_t stride_a, 
 /* out[i] = fmt(a[i] + b[i]). Replaces elementwise_add_kernel<Cfg>::run with float types,
  * templates/nnet_utils/elementwise_add/elementwise_add.cpp:12-37. */
 A4G_API int a4g_add_f(const void* a, const void* b, void* out, int64_t n, int fmt, a4g_stream_t stream);
+
+/* ---- Transposed operands of any width ------------------------------------------------------------------
+ * dst[b][c][r] = src[b][r][c] for elements of 1, 2 or 4 bytes; pitches and batch strides in elements.
+ * The kernels of the reference read a transposed operand through a transposing load
+ * (templates/nnet_utils/matmul/matmul.cpp:60-66, dense_bias_relu.cpp:95-101, selected by transpose_lhs / transpose_rhs of
+ * op_impls/families/matmul/matmul.py:78-98). The 8-bit entry points do the same (`trans_a`, `trans_b`); for the 16-bit
+ * and floating-point entry points, which take a K-contiguous left operand, a caller turns a [K][M] operand into
+ * [M][K] with this call, on the device and in memory it owns. */
+A4G_API int a4g_transpose(const void* src, int elem_bytes, int64_t ld_src, int64_t stride_src, void* dst, int64_t ld_dst,
+                  int64_t stride_dst, int64_t batch, int64_t rows, int64_t cols, a4g_stream_t stream);
 
 /* ---- Calibration (measurement aid, no counterpart in the reference) -------------------------------------
  * `blocks` workgroups of four waves issue v_mfma_i32_32x32x32_i8 on register-resident operands, `iters` times 16

@@ -84,6 +84,35 @@ def test_add_unaligned_views(ops, oracle):
     assert np.array_equal(got, oracle.add(a[3:10003], b[5:10005]))
 
 
+# ---- transposes ------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize('dtype', [np.int8, np.int16, np.float32])
+@pytest.mark.parametrize('shape', [(1, 1, 1), (3, 64, 64), (2, 5, 300), (1, 129, 65), (7, 100, 1), (1, 1000, 257)])
+def test_transpose_entry_point(ops, dtype, shape):
+    r = rng(sum(shape))
+    x = (r.standard_normal(shape) * 100).astype(dtype)
+    got = host(ops.transpose_last2(dev(x)))
+    assert got.shape == (shape[0], shape[2], shape[1])
+    assert np.array_equal(got, np.swapaxes(x, -1, -2))
+
+
+def test_transpose_pitched_through_the_c_abi(ops):
+    # source rows and destination rows that are slices of wider buffers, batch stride larger than the matrix
+    import ctypes
+    from aie4ml_amd import _lib
+    L = _lib.load()
+    r = rng(77)
+    src = torch.from_numpy(r.integers(-30000, 30000, (3, 40, 100)).astype(np.int16)).cuda()
+    dst = torch.zeros((3, 70, 64), dtype=torch.int16, device='cuda')
+    R, C = 33, 61
+    rc = L.a4g_transpose(ctypes.c_void_p(src.data_ptr()), 2, 100, 40 * 100, ctypes.c_void_p(dst.data_ptr()), 64, 70 * 64, 3, R, C,
+                         ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    got, s = dst.cpu().numpy(), src.cpu().numpy()
+    assert np.array_equal(got[:, :C, :R], np.swapaxes(s[:, :R, :C], -1, -2))
+    assert not got[:, C:, :].any() and not got[:, :, R:].any()
+
+
 # ---- Dense ----------------------------------------------------------------------------------------------
 
 def run_dense(ops, oracle, M, K, N, mode, a_dtype=np.int8, relu=True, per_channel=True, out='int8', bias=True,
