@@ -968,6 +968,12 @@ static int matmul_i8_impl(const char* who, bool own_scratch, const void* A, int 
     }
 
     const bool a_ok = K % 16 == 0 && lda % 16 == 0 && stride_a % 16 == 0 && aligned16(A);
+    // a single problem is a Dense without bias: the kernels that requantise from registers take it where they apply
+    auto launch_aligned = [&]() {
+        if (batch == 1 && wreg_applicable(g)) return launch_wreg(g, stream);
+        if (batch == 1 && sk_applicable(g) && sk_preferred(g)) return launch_sk(g, stream);
+        return launch_gemm_nt(g, static_cast<int>(batch), stream, env_variant());
+    };
     hipError_t e;
     if (trans_b) {
         g.Bt = B;
@@ -976,7 +982,7 @@ static int matmul_i8_impl(const char* who, bool own_scratch, const void* A, int 
         if (trans_a) {
             e = launch_trans_a(g, static_cast<int>(batch), stream);
         } else if (a_ok && ldb % 16 == 0 && stride_b % 16 == 0 && aligned16(B)) {
-            e = launch_gemm_nt(g, static_cast<int>(batch), stream, env_variant());
+            e = launch_aligned();
         } else {
             e = launch_ragged(g, static_cast<int>(batch), stream);
         }
@@ -988,7 +994,7 @@ static int matmul_i8_impl(const char* who, bool own_scratch, const void* A, int 
         g.ldb = ldt;
         g.stride_b = N * ldt;
         e = trans_a ? launch_trans_a(g, static_cast<int>(batch), stream)
-            : a_ok  ? launch_gemm_nt(g, static_cast<int>(batch), stream, env_variant())
+            : a_ok  ? launch_aligned()
                     : launch_ragged(g, static_cast<int>(batch), stream);
     }
     return check_hip(e, who);

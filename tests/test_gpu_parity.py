@@ -340,6 +340,21 @@ def test_matmul_batched(ops, oracle, shape, trans_b):
         assert np.array_equal(got, oracle.matmul(A, B, 6, mode, trans_b=trans_b))
 
 
+@pytest.mark.parametrize('a_dtype', [np.int8, np.uint8])
+@pytest.mark.parametrize('trans_b', [True, False])
+@pytest.mark.parametrize('shape', [(300, 272, 256), (1000, 128, 768), (129, 400, 1024), (2048, 768, 2048), (65, 16, 128)])
+def test_matmul_single_problem_on_the_dense_kernels(ops, oracle, shape, trans_b, a_dtype):
+    # one problem with K a multiple of 128: the Dense kernels that requantise from registers (weights in registers up to
+    # K = 768, reduction split in the workgroup beyond), here without bias and with a scalar shift
+    M, N, K = shape
+    r = rng(M + N + K + 5)
+    A = r.integers(0, 256, (M, K)).astype(np.uint8) if a_dtype == np.uint8 else gauss8(r, 24, (M, K))
+    B = gauss8(r, 24, (N, K) if trans_b else (K, N))
+    for mode, shift, kind in (('conv_even', 9, 'int8'), ('symmetric_inf', 0, 'int8'), ('floor', 17, 'uint8')):
+        got = host(ops.matmul(dev(A), dev(B), shift, mode, trans_b=trans_b, out_kind=kind))
+        assert np.array_equal(got, oracle.matmul(A, B, shift, mode, trans_b=trans_b, out=kind)), (mode, shift, kind)
+
+
 @pytest.mark.parametrize('a_unsigned', [False, True])
 @pytest.mark.parametrize('trans_b', [True, False])
 @pytest.mark.parametrize('shape', [((2, 3), 64, 64, 64), ((4,), 128, 96, 32), ((), 130, 70, 48), ((2,), 50, 17, 24),
