@@ -10,6 +10,8 @@
 // plus one exchange between the two lanes of a row. The probabilities are then fed to the second MFMA
 // straight from those registers: integer dot products do not care about the order of k, so step t uses the
 // k-set a lane already holds, and V^T is laid out in LDS in the matching order.
+#include <algorithm>
+
 #include "common.hpp"
 #include "softmax_common.hpp"
 
@@ -25,6 +27,7 @@ struct AttnArgs {
     int64_t v_sb, v_sh, v_ss;
     int64_t o_sb, o_sh, o_ss;
     int heads, sq;
+    int items;  // (batch, head, block of query rows) triples in all
     FastRound lr, orr;  // logits and output requantisation
     SoftmaxParams sm;
     int noclamp;
@@ -71,56 +74,86 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
     constexpr int PARK = (NT >= 16 && BANKED) ? 3 : 0;
     unsigned* parked = reinterpret_cast<unsigned*>(colsum + D);
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int m = lane & 31, half = lane >> 5;
     const int nblk = (a.sq + ROWS - 1) / ROWS;
-    const int bh = blockIdx.x / nblk, rb = blockIdx.x % nblk;
-    const int b = bh / a.heads, h = bh % a.heads;
-    const int8_t* Qp = a.Q + b * a.q_sb + h * a.q_sh;
-    const int8_t* Kp = a.K + b * a.k_sb + h * a.k_sh;
-    const int8_t* Vp = a.V + b * a.v_sb + h * a.v_sh;
-    int8_t* Op = a.O + b * a.o_sb + h * a.o_sh;
-    const int row = rb * ROWS + wave * 32 + m;
-    const bool row_ok = row < a.sq;
-    const int rowc = row_ok ? row : a.sq - 1;
+    // The eight-wave form is persistent: one workgroup per CU takes a contiguous run of items (the blocks of query rows
+    // of one head are neighbours, so its K and V are fetched once), builds the 64 KiB replicated score table once
+    // instead of once per item.
+    constexpr bool PERSIST = BANKED;
+    const int item_begin = PERSIST ? static_cast<int>(static_cast<int64_t>(blockIdx.x) * a.items / gridDim.x) : static_cast<int>(blockIdx.x);
+    const int item_end = PERSIST ? static_cast<int>(static_cast<int64_t>(blockIdx.x + 1) * a.items / gridDim.x) : item_begin + 1;
 
     // operand fragments straight from global memory: lane (m, half) holds bytes [16*half, 16*half+16) of
-    // each 32-wide k step of its row
-    v4i qf[DT], kf[2][DT];
-#pragma unroll
-    for (int ks = 0; ks < DT; ++ks) {
-        qf[ks] = *reinterpret_cast<const v4i*>(Qp + rowc * a.q_ss + ks * 32 + half * 16);
-        kf[0][ks] = *reinterpret_cast<const v4i*>(Kp + m * a.k_ss + ks * 32 + half * 16);
-    }
-
-    // V is requested before anything else is done with LDS, so that building the score table hides its latency:
-    // a thread owns the 4x4 byte blocks blk = tid, tid + THREADS, ... (rows k0..k0+3, its four columns n0..n0+3)
+    // each 32-wide k step of its row. V is requested with them: a thread owns the 4x4 byte blocks blk = tid,
+    // tid + THREADS, ... (rows k0..k0+3, its four columns n0..n0+3).
     constexpr int NB = (SK / 4) * (D / 4);
     constexpr int VB = (NB + THREADS - 1) / THREADS;
+    const int wave_uniform = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    for (int item = item_begin; item < item_end; ++item) {
+    // The thread's indices are formed again for every item from an opaque copy of its id: derived from the id itself,
+    // the dozens of per-thread addresses below would be kept in registers across the whole loop, which the 512-key form
+    // has none to spare for.
+    int tid = threadIdx.x;
+    if (PERSIST) {  // wave number from a scalar register, lane number counted afresh: no vector register is carried
+        int lane_now;
+        asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane_now));
+        tid = wave_uniform * 64 + lane_now;
+    }
+    const int lane = tid & 63, wave = tid >> 6;
+    const int m = lane & 31, half = lane >> 5;
     const int n0 = (tid % (D / 4)) * 4;  // THREADS % (D/4) == 0: a thread keeps its four columns
+    const int8_t* Kp;
+    int8_t* Op;
+    int row;
+    bool row_ok;
+    v4i qf[DT], kf[2][DT];
     unsigned av[VB][4];
+    // a block of query rows of the same head as the previous item finds that head's V^T and column sums still in LDS
+    const bool same_head = PERSIST && item != item_begin && item / nblk == (item - 1) / nblk;
+    auto request = [&](int item) {
+        const int bh = item / nblk, rb = item - bh * nblk;
+        const int b = bh / a.heads, h = bh - b * a.heads;
+        const int8_t* Qp = a.Q + b * a.q_sb + h * a.q_sh;
+        const int8_t* Vp = a.V + b * a.v_sb + h * a.v_sh;
+        Kp = a.K + b * a.k_sb + h * a.k_sh;
+        Op = a.O + b * a.o_sb + h * a.o_sh;
+        row = rb * ROWS + wave * 32 + m;
+        row_ok = row < a.sq;
+        const int rowc = row_ok ? row : a.sq - 1;
 #pragma unroll
-    for (int it = 0; it < VB; ++it) {
-        const int blk = tid + it * THREADS;
-        const int k0 = (blk / (D / 4)) * 4;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            av[it][i] = blk < NB ? *reinterpret_cast<const unsigned*>(Vp + (k0 + i) * a.v_ss + n0) : 0u;
-    }
-
-    if (BANKED) {
-        // each entry is computed once, parked in the (still unused) V^T area, then copied to its 64 slots, four
-        // slots per 16-byte store
-        int* once = reinterpret_cast<int*>(vt);
-        if (tid < 256) once[tid] = table_entry(a.sm, tid);
-        __syncthreads();
-        for (int i = tid * 4; i < 256 * 64; i += THREADS * 4) {
-            const int e = once[i >> 6];
-            *reinterpret_cast<v4i*>(table + i) = v4i{e, e, e, e};
+        for (int ks = 0; ks < DT; ++ks) {
+            qf[ks] = *reinterpret_cast<const v4i*>(Qp + rowc * a.q_ss + ks * 32 + half * 16);
+            kf[0][ks] = *reinterpret_cast<const v4i*>(Kp + m * a.k_ss + ks * 32 + half * 16);
         }
-    } else {
-        table[tid] = table_entry(a.sm, tid);
+#pragma unroll
+        for (int it = 0; it < VB; ++it) {
+            const int blk = tid + it * THREADS;
+            const int k0 = (blk / (D / 4)) * 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                av[it][i] = blk < NB ? *reinterpret_cast<const unsigned*>(Vp + (k0 + i) * a.v_ss + n0) : 0u;
+        }
+    };
+    // requested before anything is done with LDS, so that (first item) building the score table hides the latency
+    request(item);
+    if (item == item_begin) {
+        if (BANKED) {
+            // each entry is computed once, parked in the (still unused) V^T area, then copied to its 64 slots, four
+            // slots per 16-byte store
+            int* once = reinterpret_cast<int*>(vt);
+            if (tid < 256) once[tid] = table_entry(a.sm, tid);
+            __syncthreads();
+            for (int i = tid * 4; i < 256 * 64; i += THREADS * 4) {
+                const int e = once[i >> 6];
+                *reinterpret_cast<v4i*>(table + i) = v4i{e, e, e, e};
+            }
+        } else {
+            table[tid] = table_entry(a.sm, tid);
+        }
     }
+    // everybody is done with the previous item's V^T, column sums and parked scores (first item: with the table's
+    // staging area)
+    __syncthreads();
+    if (!same_head) {
     if (tid < D) colsum[tid] = 0;
     __syncthreads();
 
@@ -147,6 +180,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
 #pragma unroll
         for (int j = 0; j < 4; ++j) atomicAdd(&colsum[n0 + j], part[j]);
     }
+    }  // !same_head
 
     // ---- pass A: logits = srs(Q K^T), packed int8 in registers; running row maximum -----------------
     unsigned lg[NT][4];  // biased by 128: byte = logit ^ 0x80
@@ -299,7 +333,10 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
                        static_cast<int>(s13[1])};
         if (row_ok) *reinterpret_cast<v4i*>(Op + row * a.o_ss + 32 * u + 16 * half) = o;
     }
+    }  // items
 }
+
+constexpr int ATTN_CUS = 256;
 
 template <int NT, int DT, int BIT, bool FASTP>
 static void launch_attention_wide(int grid8, size_t lds, hipStream_t stream, const AttnArgs& a) {
@@ -310,7 +347,7 @@ static void launch_attention_wide(int grid8, size_t lds, hipStream_t stream, con
                                   static_cast<int>(lds));
         attr_set = true;
     }
-    kern<<<grid8, 512, lds, stream>>>(a);
+    kern<<<std::min(grid8, ATTN_CUS), 512, lds, stream>>>(a);  // persistent: at most one workgroup per CU
 }
 
 // grid: workgroups of 128 query rows; grid8: workgroups of 256 (0 = do not use the eight-wave form).
@@ -407,6 +444,7 @@ extern "C" int a4g_attention_i8(const int8_t* Q, const int8_t* K, const int8_t* 
     // eight waves per workgroup (256 query rows, bank-replicated score table) once every CU gets at least one
     const int64_t wg8 = batch * heads * ((sq + 255) / 256);
     const int grid8 = (sq >= 256 && wg8 >= 256) ? static_cast<int>(wg8) : 0;
+    a.items = grid8 > 0 ? grid8 : grid;
     if (launch_attention<2>(static_cast<int>(sk / 32), grid, grid8, stream, a))
         return fail(A4G_ERR_UNSUPPORTED, "%s: no kernel for sk=%lld", who, (long long)sk);
     return check_hip(hipGetLastError(), who);
