@@ -204,7 +204,9 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
                 float f[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) f[i] = fmaf(static_cast<float>(acc[4 * g + i]), a.lscale, 128.f);
-                mxf = __builtin_fmaxf(__builtin_fmaxf(mxf, __builtin_fmaxf(f[0], f[1])), __builtin_fmaxf(f[2], f[3]));
+                // two three-operand maxima
+                mxf = __builtin_fmaxf(__builtin_fmaxf(mxf, f[0]), f[1]);
+                mxf = __builtin_fmaxf(__builtin_fmaxf(mxf, f[2]), f[3]);
                 unsigned w = __builtin_amdgcn_cvt_pk_u8_f32(f[0], 0, 0u);
                 w = __builtin_amdgcn_cvt_pk_u8_f32(f[1], 1, w);
                 w = __builtin_amdgcn_cvt_pk_u8_f32(f[2], 2, w);
