@@ -66,6 +66,9 @@ SIGNATURES = {
     'a4g_layernorm_i8': (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, ctypes.c_int32, _i32, _i32, _i32, _vp]),
     'a4g_add_layernorm_i8': (_i32, [_vp, _vp, _i32, _i32, _vp, _vp, _vp, _vp, _i64, _i64, ctypes.c_int32, _i32, _i32,
                                     _i32, _vp]),
+    'a4g_rowpack_weights_i8': (_i32, [_vp, _i64, _i64, _i64, _vp, _vp]),
+    'a4g_dense_add_layernorm_i8': (_i32, [_vp, _i32, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _vp, _i64, _vp, _vp, _vp, _i64,
+                                          _i64, _i64, _i64, ctypes.c_int32, _i32, _i32, _i32, _vp]),
     'a4g_softmax_exp_i8': (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _i32, _vp]),
     'a4g_softmax_hccs_i8': (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _vp]),
     'a4g_mlp_i8': (_i32, [ctypes.POINTER(MlpLayer), _i32, _vp, _i32, _i64, _vp, _i64, _i64, _i32, _vp]),

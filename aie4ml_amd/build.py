@@ -13,7 +13,7 @@ from pathlib import Path
 
 CSRC = Path(__file__).resolve().parent / 'csrc'
 LIB_PATH = Path(__file__).resolve().parent / 'libaie4ml_gfx950.so'
-SOURCES = ('abi.hip', 'rowops.hip', 'gemm.hip', 'mlp.hip', 'attention.hip', 'matmul_lean.hip', 'gemm_i16.hip', 'gemm_float.hip', 'calib.hip', 'gemm_wreg.hip', 'gemm_sk.hip')
+SOURCES = ('abi.hip', 'rowops.hip', 'gemm.hip', 'mlp.hip', 'attention.hip', 'matmul_lean.hip', 'gemm_i16.hip', 'gemm_float.hip', 'calib.hip', 'gemm_wreg.hip', 'gemm_sk.hip', 'gemm_rowln.hip')
 
 HIPCC_FLAGS = [
     '--offload-arch=gfx950',

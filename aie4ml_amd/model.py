@@ -172,9 +172,11 @@ class GPUModel:
         graph, execution = ctx.ir.logical, ctx.ir.execution
         plan = ctx.config.get('gpu_fusion_plan') or {}
         plan = {'add_layernorm': plan.get('add_layernorm', {}), 'mlp_chains': plan.get('mlp_chains', []),
-                'attention': plan.get('attention', [])}
+                'attention': plan.get('attention', []), 'dense_add_layernorm': plan.get('dense_add_layernorm', {})}
         values: Dict[str, Any] = dict(inputs)
         fused_ln = {v['layer_norm'] for v in plan['add_layernorm'].values()}
+        fused_ln |= {v['layer_norm'] for v in plan['dense_add_layernorm'].values()}
+        fused_dense = {v['dense'] for v in plan['dense_add_layernorm'].values()}
         chain_head = {c[0]: c for c in plan['mlp_chains']}
         chain_rest = {n for c in plan['mlp_chains'] for n in c[1:]}
         attn_at, attn_skip = {}, set()
@@ -205,7 +207,7 @@ class GPUModel:
             if node.is_placeholder:
                 self._run_view(node, values)
                 continue
-            if node.name in chain_rest or node.name in fused_ln:
+            if node.name in chain_rest or node.name in fused_ln or node.name in fused_dense:
                 continue  # executed as part of a fused launch
             if node.name in attn_at:
                 grp = attn_at[node.name]
@@ -218,6 +220,11 @@ class GPUModel:
             if node.name in chain_head:
                 chain = chain_head[node.name]
                 launch(node.name, 'mlp', chain, lambda: self._run_mlp(chain, values, ops))
+            elif node.name in plan['dense_add_layernorm']:
+                # launched at the add's position: the residual may be computed after the dense's own input
+                info = plan['dense_add_layernorm'][node.name]
+                launch(info['dense'], 'dense_add_layer_norm', [info['dense'], node.name, info['layer_norm']],
+                       lambda: self._run_dense_add_layernorm(info, values, ops))
             elif node.name in plan['add_layernorm']:
                 # launched at the add's position: everything that reads the sum comes later in the order
                 info = plan['add_layernorm'][node.name]
@@ -257,6 +264,25 @@ class GPUModel:
             values[add_node.outputs[0].name], values[ln_node.outputs[0].name] = res
         else:
             values[ln_node.outputs[0].name] = res
+
+    def _run_dense_add_layernorm(self, info, values, ops) -> None:
+        execution = self.context.ir.execution
+        d_inst, ln_inst = execution.get(info['dense']), execution.get(info['layer_norm'])
+        dcfg, cfg = d_inst.config, ln_inst.config
+        x = values[input_tensor_for_role(d_inst.node, 'lhs').name]
+        packed = d_inst.artifacts['packed_weights']
+        rows = x.numel() // int(x.shape[-1]) if x.numel() else 0
+        if ops.dense_add_layernorm_applicable(x, packed) and ops.dense_add_layernorm_pays(rows, packed):
+            values[ln_inst.node.outputs[0].name] = ops.dense_add_layernorm(
+                x, packed, values[info['residual']], ln_inst.artifacts['packed_gamma'], ln_inst.artifacts['packed_beta'],
+                cfg.out_shift, dense_rounding=dcfg.rounding_mode, relu=dcfg.flags.use_relu, rounding=cfg.rounding_mode,
+                eps_q0=cfg.eps_q0, gamma_shift=cfg.gamma_shift)
+            return
+        # batch sizes at which the one-launch form does not pay: the same integers from two launches
+        y = ops.dense(x, packed, dcfg.rounding_mode, relu=dcfg.flags.use_relu, out_kind='int8')
+        values[ln_inst.node.outputs[0].name] = ops.add_layernorm(
+            y, values[info['residual']], ln_inst.artifacts['packed_gamma'], ln_inst.artifacts['packed_beta'], cfg.out_shift,
+            cfg.rounding_mode, eps_q0=cfg.eps_q0, gamma_shift=cfg.gamma_shift)
 
     def _run_attention(self, grp, values, ops) -> None:
         """One fused launch for a matmul -> softmax -> matmul triple, or for all heads of a merged group

@@ -102,6 +102,8 @@ class PackedDense:
     K: int
     N: int
     wt_lo: Optional[torch.Tensor] = None  # int16 weights only: the low-byte plane (bytes ^ 0x80)
+    shift0: Optional[int] = None          # the shift as a host integer when there is one for every column
+    wf: Optional[torch.Tensor] = None     # int8 weights in fragment order, made on first use by dense_add_layernorm
 
     @property
     def ldwt(self) -> int:
@@ -135,7 +137,8 @@ def pack_dense(weight: torch.Tensor, bias: Optional[torch.Tensor], shifts) -> Pa
     top = 62 if wt_lo is not None else 31
     if int(sh.min()) < 0 or int(sh.max()) > top:
         raise ValueError(f'dense accumulator output shift must be in [0, {top}], got [{int(sh.min())}, {int(sh.max())}].')
-    return PackedDense(wt=wt, colsum=colsum, bias=bias, shifts=sh.to(weight.device), K=K, N=N, wt_lo=wt_lo)
+    return PackedDense(wt=wt, colsum=colsum, bias=bias, shifts=sh.to(weight.device), K=K, N=N, wt_lo=wt_lo,
+                       shift0=int(sh[0]) if sh.numel() == 1 else None)
 
 
 def dense(x: torch.Tensor, p: PackedDense, rounding='floor', relu: bool = False, out_kind='int8',
@@ -288,6 +291,60 @@ def add_layernorm(a: torch.Tensor, b: torch.Tensor, gamma_q7: torch.Tensor, beta
                                            _ptr(s), _ptr(out), int(a2.shape[0]), cols, int(eps_q0), int(gamma_shift),
                                            int(out_shift), _mode(rounding), _stream()))
     return (s, out) if return_sum else out
+
+
+def dense_add_layernorm_applicable(x: torch.Tensor, p: PackedDense) -> bool:
+    """Whether dense_add_layernorm() takes this Dense (the limits of a4g_dense_add_layernorm_i8)."""
+    return (p.wt_lo is None and p.shift0 is not None and p.N % 32 == 0 and p.N <= 768 and p.K % 128 == 0 and p.K <= 4096
+            and x.dtype in (torch.int8, torch.uint8) and x.dim() >= 1 and int(x.shape[-1]) == p.K)
+
+
+def dense_add_layernorm_pays(rows: int, p: PackedDense) -> bool:
+    """Whether the one-launch form is the faster one. Every workgroup of that kernel streams the whole weight matrix,
+    one per 32 rows, and a single round of workgroups has nothing to hide its first loads and its normalisation behind;
+    measured against dense() + add_layernorm() at 768 outputs: 768 inputs 13.0 / 15.0 / 23.8 us against 14.1 / 19.7 /
+    29.2 us at 4096 / 8192 / 16384 rows, but 12.5 against 11.2 us at 2048 rows and 47.2 against 46.1 us at 32768;
+    1536 inputs 20.9 against 25.5 us, 2048 inputs 26.7 against 27.8 us, 3072 inputs 36.0 against 35.0 us (8192 rows);
+    256 outputs (one 32-column block per wave) 9.8 against 9.9 us at 8192 rows, 27.7 against 17.9 us at 32768."""
+    return 4096 <= rows <= 16384 and p.K <= 1536 and p.N >= 384
+
+
+def dense_add_layernorm(x: torch.Tensor, p: PackedDense, residual: Optional[torch.Tensor], gamma_q7: torch.Tensor,
+                        beta_q15: torch.Tensor, out_shift: int, dense_rounding='floor', relu: bool = False,
+                        rounding='floor', eps_q0: int = 1, gamma_shift: int = 7, out: Optional[torch.Tensor] = None):
+    """layernorm(saturate_i8(dense(x) + residual)) in one launch: the same result as dense() (int8 output), add() with
+    shift 0 and layernorm(). ``residual`` may be None. Raises NotImplementedError outside the limits of the fused kernel
+    (dense_add_layernorm_applicable)."""
+    if not dense_add_layernorm_applicable(x, p):
+        raise NotImplementedError('dense_add_layernorm: needs int8 / uint8 rows, one shift, N % 32 == 0, N <= 768, '
+                                  'K % 128 == 0, K <= 4096')
+    x2 = _rows2d(x, 'x')
+    if x2.stride(1) != 1 or x2.stride(0) % 16:
+        x2 = x2.contiguous()
+    M = int(x2.shape[0])
+    r2 = None
+    if residual is not None:
+        if residual.dtype != torch.int8 or tuple(residual.shape) != tuple(x.shape[:-1]) + (p.N,):
+            raise ValueError('dense_add_layernorm: the residual must be an int8 tensor of the output shape')
+        r2 = _rows2d(residual, 'residual').contiguous()
+    g = _dev(gamma_q7, 'gamma').to(torch.int16).contiguous()
+    bt = _dev(beta_q15, 'beta').to(torch.int16).contiguous()
+    if g.numel() != p.N or bt.numel() != p.N:
+        raise ValueError(f'LayerNorm parameter length does not match full_inner={p.N}.')
+    L = _lib.load()
+    if p.wf is None:
+        wf = torch.empty((p.N * p.K,), dtype=torch.int8, device=p.wt.device)
+        check(L.a4g_rowpack_weights_i8(_ptr(p.wt), p.ldwt, p.N, p.K, _ptr(wf), _stream()))
+        p.wf = wf
+    if out is None:
+        out = torch.empty(tuple(x.shape[:-1]) + (p.N,), dtype=torch.int8, device=x.device)
+    elif tuple(out.shape) != tuple(x.shape[:-1]) + (p.N,) or out.dtype != torch.int8 or not out.is_contiguous():
+        raise ValueError('dense_add_layernorm: out must be a contiguous int8 tensor of the output shape')
+    check(L.a4g_dense_add_layernorm_i8(_ptr(x2), _TORCH_KIND[x2.dtype], x2.stride(0) if M > 0 else p.K, _ptr(p.wf),
+                                       _ptr(p.colsum), _ptr(p.bias), int(p.shift0), _mode(dense_rounding), int(bool(relu)),
+                                       _ptr(r2), p.N, _ptr(g), _ptr(bt), _ptr(out), p.N, M, p.N, p.K, int(eps_q0),
+                                       int(gamma_shift), int(out_shift), _mode(rounding), _stream()))
+    return out
 
 
 def softmax_exp(x: torch.Tensor, exp_kq: int, inv_shift: int = 15, out_kind='uint8', out: Optional[torch.Tensor] = None):

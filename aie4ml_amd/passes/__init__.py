@@ -355,6 +355,8 @@ class PlanGpuFusion(AIEPass):
     * add -> layer_norm: the residual add is computed inside the LayerNorm kernel (the sum is written out
       only if something else reads it).
     * a chain of dense nodes whose whole weight set fits LDS: one fused-MLP launch.
+    * dense -> add -> layer_norm where nothing else reads the dense output or the sum: one launch whose workgroups
+      compute whole rows (the dense must fit the limits of that kernel).
     * matmul(Q, K^T) -> softmax -> matmul(P, V) whose logits and probabilities have no other reader: one
       fused-attention launch; triples that read per-head slices of the same three tensors and feed one
       concat are merged into a single launch over all heads that writes the concat's output directly.
@@ -401,9 +403,37 @@ class PlanGpuFusion(AIEPass):
             if len(chain) >= 2 and self._fits(chain, execution):
                 plan['mlp_chains'].append([n.name for n in chain])
                 used.update(n.name for n in chain)
+        # dense -> add -> layer_norm: the dense computes whole rows and normalises them itself
+        plan['dense_add_layernorm'] = {}
+        for add_name, info in plan['add_layernorm'].items():
+            if info['keep_sum']:
+                continue
+            add_node = next(n for n in graph.nodes if n.name == add_name)
+            for t in add_node.inputs:
+                d = t.producer
+                if d is None or d.op_type != 'dense' or d.name in used or execution.get(d.name) is None:
+                    continue
+                if len(t.consumers) != 1 or t.name in outputs or d.traits.get('io_view') or add_node.traits.get('io_view'):
+                    continue
+                if self._rows_complete(execution.get(d.name).config):
+                    other = [u for u in add_node.inputs if u is not t]
+                    if len(other) == 1 and not other[0].is_parameter:
+                        plan['dense_add_layernorm'][add_name] = {'dense': d.name, 'layer_norm': info['layer_norm'],
+                                                                 'residual': other[0].name}
+                        break
         changed = ctx.config.get('gpu_fusion_plan') != plan
         ctx.config['gpu_fusion_plan'] = plan
         return changed
+
+    # Dense layers the row-complete kernel takes (the limits of a4g_dense_add_layernorm_i8) and can win on; whether it
+    # does depends on the number of rows, which the executor knows at launch (ops.dense_add_layernorm_pays).
+    ROWLN_MAX_K = 1536
+
+    def _rows_complete(self, cfg) -> bool:
+        return (cfg.accumulator_tag == 'acc32' and cfg.precision['lhs'].format in ('int8', 'uint8')
+                and cfg.precision['output'].format == 'int8' and cfg.shift_per_channel is None
+                and not cfg.flags.transpose_lhs and cfg.n_out % 32 == 0 and cfg.n_out <= 768 and cfg.n_in % 128 == 0
+                and cfg.n_in <= self.ROWLN_MAX_K and cfg.n_out >= 384)
 
     # ---- attention -------------------------------------------------------------------------------------
     ATTN_HEAD_DIM = 64

@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define A4G_VERSION 201 /* major*10000 + minor*100 + patch */
+#define A4G_VERSION 202 /* major*10000 + minor*100 + patch */
 
 #if defined(__GNUC__)
 #define A4G_API __attribute__((visibility("default")))
@@ -186,6 +186,24 @@ A4G_API int a4g_add_layernorm_i8(const int8_t* a, const int8_t* b, int add_shift
                          const int16_t* gamma, const int16_t* beta, int8_t* sum_out, int8_t* out, int64_t rows,
                          int64_t cols, int32_t eps_q0, int gamma_shift, int out_shift, int round_mode,
                          a4g_stream_t stream);
+
+/* Dense, residual Add and LayerNorm in one launch: out = layernorm(saturate_i8(dense(A) + residual)), the tail of a
+ * transformer sub-block. Equals a4g_dense_i8 (scalar shift, int8 output) followed by a4g_add_layernorm_i8 with
+ * add_shift 0; the reference runs dense_bias_relu.cpp:66-166, elementwise_add.cpp:12-37 and layer_norm.cpp:14-121 as
+ * three kernels with memory tiles between them. A workgroup computes complete output rows, so neither the Dense result
+ * nor the sum is written to memory.
+ *   Wf        the weights in fragment order: a4g_rowpack_weights_i8 applied to the Wt of a4g_pack_weights_i8
+ *             (N * K bytes); colsum, bias as for a4g_dense_i8
+ *   residual  [M][ld_res] int8 or NULL (LayerNorm of the Dense output itself)
+ *   gamma, beta, eps_q0, gamma_shift, out_shift, ln_round_mode as for a4g_layernorm_i8 (cols = N)
+ * Limits: N a multiple of 32 up to 768, K a multiple of 128 up to 4096, pitches multiples of 16, operands 16-byte
+ * aligned; outside them the call returns A4G_ERR_UNSUPPORTED and the caller runs the two calls above. */
+A4G_API int a4g_rowpack_weights_i8(const int8_t* Wt, int64_t ldwt, int64_t N, int64_t K, int8_t* Wf, a4g_stream_t stream);
+A4G_API int a4g_dense_add_layernorm_i8(const void* A, int a_kind, int64_t lda, const int8_t* Wf, const int32_t* colsum,
+                               const int32_t* bias, int shift, int dense_round_mode, int relu, const int8_t* residual,
+                               int64_t ld_res, const int16_t* gamma, const int16_t* beta, int8_t* out, int64_t ld_out,
+                               int64_t M, int64_t N, int64_t K, int32_t eps_q0, int gamma_shift, int out_shift,
+                               int ln_round_mode, a4g_stream_t stream);
 
 /* ---- Integer Softmax over the last axis, int8 -> uint8 (scale 1/256) or int16 -----------------------
  * Accurate form: 2nd-order integer exp. Replaces softmax_exp_i8<Cfg>::run /

@@ -46,7 +46,7 @@ def test_binding_table_matches_header(libpath):
 
     assert sorted(_lib.SIGNATURES) == declared_symbols()
     lib = _lib.load()
-    assert lib.a4g_version() == 201
+    assert lib.a4g_version() == 202
     assert lib.a4g_packed_ld(1) == 16 and lib.a4g_packed_ld(16) == 16 and lib.a4g_packed_ld(17) == 32
     # pure host-side query, no GPU needed: K x N operand transposed into the workspace + colsum
     assert lib.a4g_matmul_i8_workspace_bytes(2, 8, 64, 512, 1, 0) == 0
@@ -78,6 +78,17 @@ def test_argument_validation_happens_before_any_launch(libpath):
     assert st == _lib.A4G_ERR_UNSUPPORTED and b'a4g_transpose' in lib.a4g_last_error()
     assert lib.a4g_transpose(None, 2, 4, 64, None, 8, 64, 1, 8, 8, None) == _lib.A4G_ERR_INVALID_ARGUMENT  # pitch < row
     assert lib.a4g_transpose(None, 2, 8, 64, None, 8, 64, 0, 8, 8, None) == 0  # empty batch
+    # the row-complete Dense + Add + LayerNorm: shapes outside its limits are refused before anything else happens
+    st = lib.a4g_dense_add_layernorm_i8(None, 0, 800, None, None, None, 9, 0, 0, None, 800, None, None, None, 800, 64, 800, 768,
+                                        1, 7, 5, 0, None)  # 800 columns
+    assert st == _lib.A4G_ERR_UNSUPPORTED and b'a4g_dense_add_layernorm_i8' in lib.a4g_last_error()
+    assert lib.a4g_dense_add_layernorm_i8(None, 0, 768, None, None, None, 9, 0, 0, None, 768, None, None, None, 768, 64, 768, 700,
+                                          1, 7, 5, 0, None) == _lib.A4G_ERR_UNSUPPORTED  # K not a multiple of 128
+    assert lib.a4g_dense_add_layernorm_i8(None, 0, 768, None, None, None, 40, 0, 0, None, 768, None, None, None, 768, 64, 768, 768,
+                                          1, 7, 5, 0, None) == _lib.A4G_ERR_INVALID_ARGUMENT  # shift 40
+    assert lib.a4g_dense_add_layernorm_i8(None, 0, 768, None, None, None, 9, 0, 0, None, 768, None, None, None, 768, 0, 768, 768,
+                                          1, 7, 5, 0, None) == 0  # no rows
+    assert lib.a4g_rowpack_weights_i8(None, 768, 100, 768, None, None) == _lib.A4G_ERR_UNSUPPORTED  # 100 columns
     st = lib.a4g_softmax_exp_i8(None, None, 4, 512, 0, 15, 1, None)  # exp_kq out of range
     assert st == _lib.A4G_ERR_INVALID_ARGUMENT and b'EXP_KQ' in lib.a4g_last_error()
     st = lib.a4g_layernorm_i8(None, None, None, None, 4, 64, 0, 7, 5, 6, None)  # eps_q0 < 1

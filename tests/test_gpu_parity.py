@@ -697,6 +697,109 @@ def test_add_layernorm_fused(ops, oracle, cols):
     assert np.array_equal(host(out2), eo)
 
 
+# ---- Dense + Add + LayerNorm in one launch ---------------------------------------------------------------------
+
+def run_dense_add_layernorm(ops, oracle, M, K, N, seed, dmode='conv_even', lmode='conv_even', shift=9, a_dtype=np.int8,
+                            relu=False, residual=True, bias=True, gmax=None, out_shift=5, eps=1, gamma_shift=7, sigma=40):
+    """The row-complete kernel against the oracle's dense -> add -> layernorm, operator by operator."""
+    r = rng(seed)
+    A = r.integers(0, 256, (M, K)).astype(np.uint8) if a_dtype == np.uint8 else gauss8(r, sigma, (M, K))
+    W = gauss8(r, 30, (K, N))
+    b = r.integers(-2**14, 2**14, N).astype(np.int32) if bias else None
+    res = gauss8(r, 50, (M, N)) if residual else None
+    if gmax is None:
+        gamma, beta = ln_params(r, N)
+    else:
+        gamma = r.integers(-gmax, gmax + 1, N).astype(np.int16)
+        beta = r.integers(-32768, 32768, N).astype(np.int16)
+    p = ops.pack_dense(dev(W), dev(b) if bias else None, np.array([shift], np.int32))
+    got = host(ops.dense_add_layernorm(dev(A), p, dev(res) if residual else None, dev(gamma), dev(beta), out_shift, dmode,
+                                       relu, lmode, eps_q0=eps, gamma_shift=gamma_shift))
+    y = oracle.dense(A, W, b, shift, dmode, relu=relu, out='int8')
+    if residual:
+        exp = oracle.add_layernorm(y, res, gamma, beta, out_shift, lmode, eps_q0=eps, gamma_shift=gamma_shift)
+    else:
+        exp = oracle.layernorm(y, gamma, beta, out_shift, lmode, eps_q0=eps, gamma_shift=gamma_shift)
+    assert np.array_equal(got, exp), f'mismatch at {np.argwhere(got != exp)[:5]}'
+
+
+@pytest.mark.parametrize('case', [(1, 128, 32), (31, 128, 768), (33, 256, 256), (100, 768, 768), (64, 384, 512),
+                                  (257, 512, 384), (96, 640, 160), (40, 3072, 768), (700, 1024, 64), (65, 4096, 96)])
+def test_dense_add_layernorm_shapes(ops, oracle, case):
+    M, K, N = case
+    run_dense_add_layernorm(ops, oracle, M, K, N, seed=sum(case))
+    run_dense_add_layernorm(ops, oracle, M, K, N, seed=sum(case) + 1, a_dtype=np.uint8, relu=True, residual=False)
+
+
+@pytest.mark.parametrize('lmode', MODES)
+@pytest.mark.parametrize('dmode', MODES)
+def test_dense_add_layernorm_rounding_modes(ops, oracle, dmode, lmode):
+    """Every pair of rounding modes: the Dense requantisation takes its rounding bit at run time, the LayerNorm has a
+    float form for five of the modes and the integer form for the rest."""
+    run_dense_add_layernorm(ops, oracle, 70, 256, 96, seed=MODES.index(dmode) * 8 + MODES.index(lmode), dmode=dmode, lmode=lmode,
+                            shift=8, sigma=60)
+
+
+@pytest.mark.parametrize('shift', [0, 1, 15, 22, 23, 31])
+def test_dense_add_layernorm_shifts(ops, oracle, shift):
+    """Shifts on both sides of the quick requantisation's limit (22), and none at all."""
+    for dmode in ('conv_even', 'symmetric_inf', 'ceil'):
+        run_dense_add_layernorm(ops, oracle, 45, 128, 64, seed=shift, dmode=dmode, shift=shift, sigma=90 if shift > 15 else 8)
+
+
+def test_dense_add_layernorm_large_start_values(ops, oracle):
+    """A bias next to the int32 limits sends a wave to the general requantisation (the accumulator wraps like the sum)."""
+    r = rng(77)
+    M, K, N = 40, 128, 64
+    A, W = gauss8(r, 40, (M, K)), gauss8(r, 30, (K, N))
+    b = r.integers(-2**14, 2**14, N).astype(np.int32)
+    b[3], b[40] = 2**31 - 5, -2**31 + 9
+    res = gauss8(r, 50, (M, N))
+    gamma, beta = ln_params(r, N)
+    p = ops.pack_dense(dev(W), dev(b), np.array([12], np.int32))
+    got = host(ops.dense_add_layernorm(dev(A), p, dev(res), dev(gamma), dev(beta), 5, 'conv_even', False, 'conv_even'))
+    exp = oracle.add_layernorm(oracle.dense(A, W, b, 12, 'conv_even', out='int8'), res, gamma, beta, 5, 'conv_even')
+    assert np.array_equal(got, exp)
+
+
+@pytest.mark.parametrize('gmax', [511, 512, 32767])
+def test_dense_add_layernorm_gamma_at_the_float_limit(ops, oracle, gmax):
+    for lmode, gs, osft in (('conv_even', 7, 5), ('floor', 0, 15), ('negative_inf', 15, 0), ('symmetric_zero', 3, 8)):
+        run_dense_add_layernorm(ops, oracle, 50, 128, 128, seed=gmax % 97, lmode=lmode, gmax=gmax, gamma_shift=gs, out_shift=osft)
+
+
+def test_dense_add_layernorm_degenerate_rows(ops, oracle):
+    """Constant and extreme rows after the add: zero variance, the int8 limits, maximum variance."""
+    M, K, N = 6, 128, 256
+    A = np.zeros((M, K), np.int8)          # the Dense output is the requantised bias
+    W = np.ones((K, N), np.int8)
+    b = np.zeros(N, np.int32)
+    res = np.zeros((M, N), np.int8)
+    res[0] = 17
+    res[1, :N // 2] = 1
+    res[2] = 127
+    res[3] = -128
+    res[4, ::2], res[4, 1::2] = 127, -128
+    res[5, 0] = 1
+    r = rng(5)
+    gamma = np.full(N, 32767, np.int16)
+    beta = r.integers(-32768, 32768, N).astype(np.int16)
+    p = ops.pack_dense(dev(W), dev(b), np.array([3], np.int32))
+    for lmode in ('conv_even', 'symmetric_inf'):
+        got = host(ops.dense_add_layernorm(dev(A), p, dev(res), dev(gamma), dev(beta), 5, 'floor', False, lmode))
+        exp = oracle.add_layernorm(oracle.dense(A, W, b, 3, 'floor', out='int8'), res, gamma, beta, 5, lmode)
+        assert np.array_equal(got, exp), lmode
+
+
+def test_dense_add_layernorm_refuses_what_it_cannot_take(ops):
+    r = rng(9)
+    W = gauss8(r, 30, (100, 64))  # K not a multiple of 128
+    p = ops.pack_dense(dev(W), None, np.array([7], np.int32))
+    assert not ops.dense_add_layernorm_applicable(dev(gauss8(r, 40, (8, 100))), p)
+    with pytest.raises(NotImplementedError):
+        ops.dense_add_layernorm(dev(gauss8(r, 40, (8, 100))), p, None, dev(np.ones(64, np.int16)), dev(np.zeros(64, np.int16)), 5)
+
+
 # ---- Softmax --------------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize('cols', [16, 32, 64, 128, 512, 1024, 2048, 4096, 48, 96, 100, 8192])

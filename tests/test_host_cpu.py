@@ -371,6 +371,19 @@ def test_encoder_block_graph_lowers():
     assert plan['mlp_chains'] == [['ffn1_aie', 'ffn2_aie']]   # widths 64/128/64 fit the fused-MLP kernel
     assert x.shape == (2, 32, 64) and x.dtype == np.int8
     assert plan['attention'] == []          # head_dim 32 is outside the fused attention kernel's range
+    assert plan['dense_add_layernorm'] == {}  # 64 outputs: too narrow for the projection that normalises its own rows
+
+
+def test_plan_marks_projections_that_can_normalise_their_rows():
+    from aie4ml_amd import workloads
+
+    model, _ = workloads.c5_encoder_block(batch=1, seq=32, hidden=768, heads=12, ffn=3072)
+    ctx = lower(GraphHolder(model), FRONT + (PlanGpuFusion,))
+    plan = ctx.config['gpu_fusion_plan']
+    # the attention output projection (768 -> 768) feeds only the residual add in front of a LayerNorm whose input nobody
+    # else reads; the second feed-forward projection has 3072 inputs, past what that kernel is used for
+    assert plan['dense_add_layernorm'] == {'residual1_aie': {'dense': 'attn_out_aie', 'layer_norm': 'ln1_aie', 'residual': 'x'}}
+    assert set(plan['add_layernorm']) == {'residual1_aie', 'residual2_aie'}
 
 
 def test_attention_plan_merges_heads():
