@@ -155,6 +155,36 @@ def prepare(wl, torch):
         cpu_work = 2.0 * sample_rows * N * K
         metric, unit = 'int8_dense_tops', 'TOP/s'
         kernel = ENCODER_PROJECTIONS[wl][3] if wl in ENCODER_PROJECTIONS else 'gemm_rs_kernel'
+    elif wl == 'c5_proj_out_ln':
+        # the attention output projection of the c5 block together with the residual add and the LayerNorm behind it,
+        # as the graph executor launches them at this batch size: one kernel whose workgroups own whole rows
+        M, K, N = 8192, 768, 768
+        A, W, bias, _ = workloads.c2_dense(M, K, N)
+        r = np.random.default_rng(23)
+        res = np.clip(np.rint(r.normal(0, 30, (M, N))), -128, 127).astype(np.int8)
+        gamma = r.integers(32, 128, N).astype(np.int16)
+        beta = (r.integers(-16, 17, N).astype(np.int32) << 10).astype(np.int16)
+        p = ops.pack_dense(dev(W), dev(bias), np.array([9], np.int32))
+        dA, dres, dg, dbt = dev(A), dev(res), dev(gamma), dev(beta)
+        out = torch.empty((M, N), dtype=torch.int8, device='cuda')
+        fn = lambda: ops.dense_add_layernorm(dA, p, dres, dg, dbt, 5, 'conv_even', False, 'conv_even', out=out)  # noqa: E731
+        fn()
+        rows = np.random.default_rng(0).choice(M, 96, replace=False)
+        ref = lambda sel: oracle.add_layernorm(oracle.dense(A[sel], W, bias, 9, 'conv_even', out='int8'), res[sel], gamma,  # noqa: E731
+                                               beta, 5, 'conv_even')
+        exp = ref(rows)
+        torch.cuda.synchronize()
+        bit_exact = bool(np.array_equal(out[torch.from_numpy(rows).cuda()].cpu().numpy(), exp))
+        work, bound = 2.0 * M * N * K, 'mfma'
+        samples = M
+        config = {'workload': f'c5_proj_out_ln: Dense {M}x{K} -> {N} (int8, bias, shift 9, conv_even) + residual add + LayerNorm '
+                              f'over {N} columns in one launch (the tail of the attention half of the c5 encoder block)'}
+        sample_rows = 2048
+        cpu_desc = f'oracle dense -> add -> layernorm on the first {sample_rows} of {M} rows, scaled per op'
+        cpu_fn = lambda: ref(slice(0, sample_rows))  # noqa: E731
+        cpu_work = 2.0 * sample_rows * N * K
+        metric, unit = 'int8_dense_tops', 'TOP/s'
+        kernel = 'gemm_rowln_kernel'
     elif wl == 'c2_dense_i16':
         # the (16, 8) width combination on the C2 shape: int16 activations, int8 weights, int16 output
         M, K, N = 8192, 4096, 4096
@@ -491,7 +521,7 @@ def calibrate_mfma(torch, blocks_per_cu=2, iters=4096):
 
 # the other configurations, timed in the default run after the headline workload (same steps, no CPU leg)
 ALSO = ('c1_mlp', 'c3_qk', 'c3_softmax_exp', 'c3_softmax_hccs', 'c3_pv', 'c3_attention_exp', 'c4_add', 'c4_layernorm',
-        'c4_add_layernorm', 'c5_encoder', 'c5_proj_qkv', 'c5_proj_out', 'c5_ffn_up', 'c5_ffn_down')
+        'c4_add_layernorm', 'c5_encoder', 'c5_proj_qkv', 'c5_proj_out', 'c5_ffn_up', 'c5_ffn_down', 'c5_proj_out_ln')
 
 
 def main():
