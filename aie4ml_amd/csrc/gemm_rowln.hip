@@ -30,9 +30,9 @@ constexpr int RL_NT = 512, RL_WAVES = 8, RL_BPW = 3;
 constexpr int RL_MAX_N = RL_WAVES * RL_BPW * 32;  // 768
 constexpr int RL_MAX_K = 4096;                    // 128 KiB of activations in LDS at 32 rows
 constexpr int RL_MAX_K2 = 2304;                   // 144 KiB at 64 rows
-// LDS: the activations, then gamma and beta (four bytes each), then the row sums [row][wave]{sum, sum of squares}, then
-// one flag per wave
-constexpr int rl_lds_bytes(int rows, int K, int N) { return rows * K + 8 * N + rows * RL_WAVES * 2 * 4 + RL_WAVES * 4; }
+// LDS: the activations, then gamma, beta and the accumulators' start values (four bytes a column each), then the row
+// sums [row][wave]{sum, sum of squares}, then one flag per wave
+constexpr int rl_lds_bytes(int rows, int K, int N) { return rows * K + 12 * N + rows * RL_WAVES * 2 * 4 + RL_WAVES * 4; }
 
 struct RowLnArgs {
     const int8_t* A;
@@ -78,7 +78,8 @@ __global__ __launch_bounds__(RL_NT, 2) void gemm_rowln_kernel(RowLnArgs g) {
     int8_t* const a_lds = rl_smem;  // K / 128 slabs of BM rows x 128 bytes
     int* const gamma_lds = reinterpret_cast<int*>(rl_smem + BM * g.K);  // floats for the float form, else int32
     int* const beta_lds = gamma_lds + g.N;
-    int* const stat_lds = beta_lds + g.N;
+    int* const start_lds = beta_lds + g.N;
+    int* const stat_lds = start_lds + g.N;
     int* const flag_lds = stat_lds + BM * RL_WAVES * 2;
 
     const int tid = threadIdx.x, lane = tid & 63;
@@ -127,8 +128,6 @@ __global__ __launch_bounds__(RL_NT, 2) void gemm_rowln_kernel(RowLnArgs g) {
         }
         return wide;
     };
-    const int wide_here = FR >= 0 ? stage_params(true) : (stage_params(false), 1);
-
     // ---- this wave's blocks: columns 32 nb .. + 31, nb = wave * bpw + j; a lane ends up with columns 16 half .. + 15
     const auto rsrc_w = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(g.Wf), 0, g.w_bytes, 0x00020000);
     bool live[RL_BPW];
@@ -164,27 +163,18 @@ __global__ __launch_bounds__(RL_NT, 2) void gemm_rowln_kernel(RowLnArgs g) {
             rw[rb][j] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(
                 rsrc_res, live[j] ? (m0 + rb * 32 + frow) * g.ld_res + col0[j] : NOWHERE, 0, 0));
 
-    // ---- accumulators start from bias + 128 * colsum (int32 wraps like the sum it stands for)
-    const auto rsrc_bias = __builtin_amdgcn_make_buffer_rsrc(const_cast<int32_t*>(g.bias), 0, g.bias ? g.N * 4 : 0, 0x00020000);
-    const auto rsrc_cs = __builtin_amdgcn_make_buffer_rsrc(const_cast<int32_t*>(g.colsum), 0, g.a_unsigned ? g.N * 4 : 0, 0x00020000);
-    v16i acc[RB][RL_BPW];
-    bool small = true;
-#pragma unroll
-    for (int j = 0; j < RL_BPW; ++j) {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int at = live[j] ? (col0[j] + 4 * q) * 4 : NOWHERE;
-            const v4i st = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_bias, at, 0, 0)) +
-                           128 * __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_cs, at, 0, 0));
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-#pragma unroll
-                for (int rb = 0; rb < RB; ++rb) acc[rb][j][q * 4 + t] = st[t];
-                small = small && st[t] <= (1 << 30) && st[t] >= -(1 << 30);
-            }
-        }
+    // ---- the accumulators' start values, bias + 128 * colsum (int32 wraps like the sum it stands for), go through LDS:
+    // fetched by every lane for its own columns they would be 24 load instructions per wave, and the vector memory
+    // path takes 16 clocks per instruction however little it fetches
+    if (tid < g.N / 4) {
+        v4i st = {0, 0, 0, 0};
+        if (g.bias) st = *reinterpret_cast<const v4i*>(g.bias + tid * 4);
+        if (g.a_unsigned) st += 128 * *reinterpret_cast<const v4i*>(g.colsum + tid * 4);
+        *reinterpret_cast<v4i*>(start_lds + tid * 4) = st;
     }
-    const bool quick = g.quick && __all(small);
+
+    // the parameter loads come last: their wait, inside the branch that issues them, then covers everything above
+    const int wide_here = FR >= 0 ? stage_params(true) : (stage_params(false), 1);
 
     int koff[4];  // activation fragment of K step kk of a slab: row frow, chunk 2 kk + half
 #pragma unroll
@@ -205,6 +195,22 @@ __global__ __launch_bounds__(RL_NT, 2) void gemm_rowln_kernel(RowLnArgs g) {
     // it believes outstanding on entry to the loop would look younger than everything the loop issues, and every wait
     // inside would become a wait for all loads. The first fragments have arrived with the wait above; passing them
     // through an empty asm makes the compiler wait for them here too, and the loop's waits then count exactly.
+    v16i acc[RB][RL_BPW];
+    bool small = true;
+#pragma unroll
+    for (int j = 0; j < RL_BPW; ++j) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const v4i st = live[j] ? *reinterpret_cast<const v4i*>(start_lds + col0[j] + 4 * q) : v4i{0, 0, 0, 0};
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+#pragma unroll
+                for (int rb = 0; rb < RB; ++rb) acc[rb][j][q * 4 + t] = st[t];
+                small = small && st[t] <= (1 << 30) && st[t] >= -(1 << 30);
+            }
+        }
+    }
+    const bool quick = g.quick && __all(small);
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk)
 #pragma unroll

@@ -302,10 +302,11 @@ def dense_add_layernorm_applicable(x: torch.Tensor, p: PackedDense) -> bool:
 def dense_add_layernorm_pays(rows: int, p: PackedDense) -> bool:
     """Whether the one-launch form is the faster one. Every workgroup of that kernel streams the whole weight matrix,
     one per 32 rows, and a single round of workgroups has nothing to hide its first loads and its normalisation behind;
-    measured against dense() + add_layernorm() at 768 outputs: 768 inputs 13.0 / 15.0 / 23.8 us against 14.1 / 19.7 /
-    29.2 us at 4096 / 8192 / 16384 rows, but 12.5 against 11.2 us at 2048 rows and 47.2 against 46.1 us at 32768;
-    1536 inputs 20.9 against 25.5 us, 2048 inputs 26.7 against 27.8 us, 3072 inputs 36.0 against 35.0 us (8192 rows);
-    256 outputs (one 32-column block per wave) 9.8 against 9.9 us at 8192 rows, 27.7 against 17.9 us at 32768."""
+    measured against dense() + add_layernorm() at 768 outputs: 768 inputs 12.2 / 14.1 / 23.1 us against 14.2 / 19.6 /
+    28.7 us at 4096 / 8192 / 16384 rows, but 11.6 against 11.3 us at 2048 rows and 45.4 against 46.3 us at 32768;
+    1024 inputs 16.1 against 22.1 us, 1536 inputs 20.2 against 25.2 us, 2048 inputs 26.1 against 27.9 us, 3072 inputs
+    35.2 against 34.2 us (8192 rows); 512 -> 512: 11.0 against 13.7 us; 256 outputs (one 32-column block per wave) 8.8
+    against 10.0 us at 8192 rows, 26.5 against 17.7 us at 32768."""
     return 4096 <= rows <= 16384 and p.K <= 1536 and p.N >= 384
 
 
