@@ -9,6 +9,8 @@
 
 namespace a4g {
 
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+
 __device__ __forceinline__ int lean_col(int j) { return ((j >> 2) & 1) * 16 + (j >> 3) * 4 + (j & 3); }
 
 // ---- A x B^T, short K ----------------------------------------------------------------------------------
@@ -17,14 +19,15 @@ __device__ __forceinline__ int lean_col(int j) { return ((j >> 2) & 1) * 16 + (j
 // j = 8*g + 4*h' + i of tile T loads actual column (16*TG)*h' + 16*T + 4*g + i, so that lane (m, half) ends
 // the group with 16*TG contiguous output bytes of row m (a whole 128-byte line per row for TG = 4).
 template <int DT, int TG>
-__device__ __forceinline__ void lean_nt_load(const LeanArgs& a, const int8_t* Bp, v4i (&bf)[TG][DT], int col0, int m, int half) {
+__device__ __forceinline__ void lean_nt_load(const LeanArgs& a, __amdgpu_buffer_rsrc_t rsrc_b, v4i (&bf)[TG][DT], int col0, int m, int half) {
     const int g = m >> 3, hp = (m >> 2) & 1, i = m & 3;
 #pragma unroll
     for (int T = 0; T < TG; ++T) {
         const int col = col0 + 16 * TG * hp + 16 * T + 4 * g + i;
+        // a column past the matrix lies past the descriptor and reads as zero: no branch around the load
 #pragma unroll
         for (int ks = 0; ks < DT; ++ks)
-            bf[T][ks] = *reinterpret_cast<const v4i*>(Bp + static_cast<int64_t>(col) * a.ldb + ks * 32 + half * 16);
+            bf[T][ks] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, col * static_cast<int>(a.ldb) + ks * 32 + half * 16, 0, 0));
     }
 }
 
@@ -36,7 +39,7 @@ constexpr int LEAN_PATCH_PITCH = 144;
 constexpr int LEAN_PATCH_BYTES = 32 * LEAN_PATCH_PITCH;
 
 template <int DT, int TG, int RB, int BIT, bool UOUT>
-__device__ __forceinline__ void lean_nt_compute(const LeanArgs& a, int8_t* Cp, const v4i (&af)[RB][DT], const v4i (&bf)[TG][DT],
+__device__ __forceinline__ void lean_nt_compute(const LeanArgs& a, __amdgpu_buffer_rsrc_t rsrc_c, const v4i (&af)[RB][DT], const v4i (&bf)[TG][DT],
                                                 int col0, int lane, const int (&row)[RB], const bool (&row_ok)[RB],
                                                 int8_t* patch, int row_base) {
     const int m = lane & 31, half = lane >> 5;
@@ -74,13 +77,14 @@ __device__ __forceinline__ void lean_nt_compute(const LeanArgs& a, int8_t* Cp, c
             for (int s4 = 0; s4 < 4; ++s4) {
                 const int r = 8 * s4 + (lane >> 3), c = lane & 7;
                 const v4i v = *reinterpret_cast<const v4i*>(patch + r * LEAN_PATCH_PITCH + 16 * c);
-                if (r0 + r < a.M) *reinterpret_cast<v4i*>(Cp + static_cast<int64_t>(r0 + r) * a.ldc + col0 + 16 * c) = v;
+                // a row past the matrix lies past the descriptor: the store is dropped, again without a branch
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), rsrc_c, (r0 + r) * static_cast<int>(a.ldc) + col0 + 16 * c, 0, 0);
             }
         } else {
 #pragma unroll
             for (int T = 0; T < TG; ++T)
-                if (row_ok[rb])
-                    *reinterpret_cast<v4i*>(Cp + static_cast<int64_t>(row[rb]) * a.ldc + col0 + 16 * TG * half + 16 * T) = o[T];
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, o[T]), rsrc_c,
+                                                       row[rb] * static_cast<int>(a.ldc) + col0 + 16 * TG * half + 16 * T, 0, 0);
         }
     }
 }
@@ -94,8 +98,14 @@ __global__ __launch_bounds__(256, 2) void matmul_lean_nt_kernel(LeanArgs a) {
     int8_t* patch = patches + wave * LEAN_PATCH_BYTES;
     const int row_base = blockIdx.x * (128 * RB) + wave * RB * 32;
     const int8_t* Ap = a.A + blockIdx.z * a.stride_a;
-    const int8_t* Bp = a.B + blockIdx.z * a.stride_b;
-    int8_t* Cp = a.C + blockIdx.z * a.stride_c;
+    // B and C of this problem behind descriptors that end with the matrices. The compiler counts outstanding memory
+    // operations from the youngest back, and a load or store inside a branch makes every later wait a wait for
+    // everything: with them the prefetch of the next column group was waited for at once, before the arithmetic it was
+    // meant to overlap.
+    const auto rsrc_b = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.B + blockIdx.z * a.stride_b), 0,
+                                                          (a.N - 1) * static_cast<int>(a.ldb) + a.K, 0x00020000);
+    const auto rsrc_c = __builtin_amdgcn_make_buffer_rsrc(a.C + blockIdx.z * a.stride_c, 0, (a.M - 1) * static_cast<int>(a.ldc) + a.N,
+                                                          0x00020000);
     const int c0 = blockIdx.y * 512, c1 = min(c0 + 512, a.N);
 
     int row[RB];
@@ -112,23 +122,20 @@ __global__ __launch_bounds__(256, 2) void matmul_lean_nt_kernel(LeanArgs a) {
     int col = c0;
     if (col + 128 <= c1) {
         v4i bf[4][DT], nbf[4][DT];
-        lean_nt_load<DT, 4>(a, Bp, bf, col, m, half);
+        lean_nt_load<DT, 4>(a, rsrc_b, bf, col, m, half);
         for (; col + 128 <= c1; col += 128) {
-            const bool more = col + 256 <= c1;
-            if (more) lean_nt_load<DT, 4>(a, Bp, nbf, col + 128, m, half);  // in flight during the arithmetic below
-            lean_nt_compute<DT, 4, RB, BIT, UOUT>(a, Cp, af, bf, col, lane, row, row_ok, patch, row_base);
-            if (more) {
+            lean_nt_load<DT, 4>(a, rsrc_b, nbf, col + 128, m, half);  // in flight during the arithmetic below (zeros past the end)
+            lean_nt_compute<DT, 4, RB, BIT, UOUT>(a, rsrc_c, af, bf, col, lane, row, row_ok, patch, row_base);
 #pragma unroll
-                for (int T = 0; T < 4; ++T)
+            for (int T = 0; T < 4; ++T)
 #pragma unroll
-                    for (int ks = 0; ks < DT; ++ks) bf[T][ks] = nbf[T][ks];
-            }
+                for (int ks = 0; ks < DT; ++ks) bf[T][ks] = nbf[T][ks];
         }
     }
     for (; col < c1; col += 32) {
         v4i bf[1][DT];
-        lean_nt_load<DT, 1>(a, Bp, bf, col, m, half);
-        lean_nt_compute<DT, 1, RB, BIT, UOUT>(a, Cp, af, bf, col, lane, row, row_ok, patch, row_base);
+        lean_nt_load<DT, 1>(a, rsrc_b, bf, col, m, half);
+        lean_nt_compute<DT, 1, RB, BIT, UOUT>(a, rsrc_c, af, bf, col, lane, row, row_ok, patch, row_base);
     }
 }
 
@@ -151,12 +158,20 @@ __global__ __launch_bounds__(256, 2) void matmul_lean_nn_kernel(LeanArgs a, int 
     int8_t* Cp = a.C + blockIdx.y * a.stride_c;
     // a workgroup transposes B once and then takes `row_blocks` consecutive blocks of 128 rows
     int row = blockIdx.x * row_blocks * 128 + wave * 32 + m;
-    bool row_ok = row < a.M;
-    const int8_t* arow = Ap + static_cast<int64_t>(row_ok ? row : a.M - 1) * a.lda + half * 64;
+    // A and C of this problem behind descriptors that end with the matrices: a row past the end reads as zero and its
+    // store is dropped, so that neither the prefetch of the next group nor a store sits inside a branch (the compiler
+    // would otherwise wait for the prefetch at once, see matmul_lean_nt_kernel)
+    constexpr unsigned NOWHERE = 0x80000000u;
+    const int lda = static_cast<int>(a.lda), ldc = static_cast<int>(a.ldc);
+    const auto rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(Ap), 0, (a.M - 1) * lda + a.K, 0x00020000);
+    const auto rsrc_c = __builtin_amdgcn_make_buffer_rsrc(Cp, 0, (a.M - 1) * ldc + N, 0x00020000);
+    unsigned aoff = row < a.M ? static_cast<unsigned>(row * lda + half * 64) : NOWHERE;
+    auto load_a = [&](unsigned off) { return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, off, 0, 0)); };
 
+    const int groups = a.K >> 7;
     v4i af[4], af_next[4];  // the group being multiplied and the one in flight
 #pragma unroll
-    for (int s = 0; s < 4; ++s) af[s] = *reinterpret_cast<const v4i*>(arow + s * 16);
+    for (int s = 0; s < 4; ++s) af[s] = load_a(aoff + s * 16);
 
     if (tid < N) colsum[tid] = 0;
     __syncthreads();
@@ -205,26 +220,14 @@ __global__ __launch_bounds__(256, 2) void matmul_lean_nn_kernel(LeanArgs a, int 
 
     const int xm = a.a_unsigned ? static_cast<int>(0x80808080u) : 0;
     const int8_t* brow = bt + lean_col(m) * pitch + half * 64;
-    const int groups = a.K >> 7;
     for (int rbk = 0; rbk < row_blocks; ++rbk) {
     v16i acc[NTL];
 #pragma unroll
     for (int u = 0; u < NTL; ++u) acc[u] = v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-    // the next block's first group is requested while this block's last group is multiplied
-    const int next_row = row + 128;
-    const bool more = rbk + 1 < row_blocks && (blockIdx.x * row_blocks + rbk + 1) * 128 < a.M;
-    const int8_t* next_arow = Ap + static_cast<int64_t>(next_row < a.M ? next_row : a.M - 1) * a.lda + half * 64;
-    for (int G = 0; G < groups; ++G) {
-        if (G + 1 < groups) {
-#pragma unroll
-            for (int s = 0; s < 4; ++s) af_next[s] = *reinterpret_cast<const v4i*>(arow + (G + 1) * 128 + s * 16);
-        } else if (more) {
-#pragma unroll
-            for (int s = 0; s < 4; ++s) af_next[s] = *reinterpret_cast<const v4i*>(next_arow + s * 16);
-        }
+    auto multiply = [&](const v4i (&grp)[4], int G) {
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-            v4i av = af[s];
+            v4i av = grp[s];
             av[0] ^= xm; av[1] ^= xm; av[2] ^= xm; av[3] ^= xm;
 #pragma unroll
             for (int u = 0; u < NTL; ++u) {
@@ -232,6 +235,19 @@ __global__ __launch_bounds__(256, 2) void matmul_lean_nn_kernel(LeanArgs a, int 
                 acc[u] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bv, av, acc[u], 0, 0, 0);
             }
         }
+    };
+    // the next block's first group is requested while this block's last group is multiplied
+    const int next_row = row + 128;
+    const bool more = rbk + 1 < row_blocks && (blockIdx.x * row_blocks + rbk + 1) * 128 < a.M;
+    const unsigned next_aoff = more && next_row < a.M ? static_cast<unsigned>(next_row * lda + half * 64) : NOWHERE;
+    for (int G = 0; G < groups; ++G) {
+        // One group ahead; three groups ahead through a ring of four register sets measured the same (C3 P x V: 29.0 us
+        // either way, the rate of a plain copy on that box).
+        const unsigned pre = G + 1 < groups ? aoff + (G + 1) * 128 : next_aoff;
+#pragma unroll
+        for (int s = 0; s < 4; ++s) af_next[s] = load_a(pre + s * 16);
+        __builtin_amdgcn_sched_barrier(0);  // the requests stay in front of the arithmetic they are meant to overlap
+        multiply(af, G);
 #pragma unroll
         for (int s = 0; s < 4; ++s) af[s] = af_next[s];
     }
@@ -247,12 +263,12 @@ __global__ __launch_bounds__(256, 2) void matmul_lean_nn_kernel(LeanArgs a, int 
             for (int i = 0; i < 4; ++i) y[i] = clamp_i(fast_round(acc[u][4 * g + i] + 128 * cs[i], a.fr), a.lo, a.hi);
             o[g] = static_cast<int>(pack4_bytes(y[0], y[1], y[2], y[3]));
         }
-        if (row_ok) *reinterpret_cast<v4i*>(Cp + static_cast<int64_t>(row) * a.ldc + 32 * u + 16 * half) = o;
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, o), rsrc_c,
+                                               row < a.M ? static_cast<unsigned>(row * ldc + 32 * u + 16 * half) : NOWHERE, 0, 0);
     }
     if (!more) break;
     row = next_row;
-    row_ok = row < a.M;
-    arow = next_arow;
+    aoff = next_aoff;
     }  // row blocks
 }
 
@@ -263,7 +279,8 @@ static bool lean_common_ok(const LeanArgs& a) {
 
 bool lean_nt_applicable(const LeanArgs& a) {
     return lean_common_ok(a) && !a.a_unsigned && a.K % 32 == 0 && a.K <= 128 && a.N % 32 == 0 && a.N <= 512 * 65535 &&
-           byte_requant_ok(a.fr);
+           byte_requant_ok(a.fr) && (static_cast<int64_t>(a.N) + 128) * a.ldb < (int64_t{1} << 31) &&
+           (static_cast<int64_t>(a.M) + 512) * a.ldc < (int64_t{1} << 31);  // 32-bit offsets inside one problem
 }
 
 template <int DT, int RB>
@@ -301,7 +318,9 @@ hipError_t launch_lean_nt(const LeanArgs& a, hipStream_t stream) {
 
 bool lean_nn_applicable(const LeanArgs& a) {
     return lean_common_ok(a) && (a.N == 32 || a.N == 64 || a.N == 128) && a.K % 128 == 0 &&
-           static_cast<int64_t>(a.N) * (a.K + 16) + a.N * 4 <= 60 * 1024;
+           static_cast<int64_t>(a.N) * (a.K + 16) + a.N * 4 <= 60 * 1024 &&
+           (static_cast<int64_t>(a.M) + 128) * a.lda < (int64_t{1} << 31) &&
+           (static_cast<int64_t>(a.M) + 128) * a.ldc < (int64_t{1} << 31);  // 32-bit offsets inside one problem
 }
 
 hipError_t launch_lean_nn(const LeanArgs& a, hipStream_t stream) {

@@ -4,6 +4,9 @@
 // Layout: plain row-major int8 rows. Fast paths stream each row exactly once as 16-byte chunks per
 // lane (fully coalesced: 64 lanes x 16 B = 1 KiB per wave-load), keep the row in registers between
 // the reduction and the normalisation, and reduce across lanes with DPP / ds_swizzle butterflies.
+#include <algorithm>
+#include <type_traits>
+
 #include "common.hpp"
 #include "layernorm_common.hpp"
 #include "softmax_common.hpp"
@@ -180,20 +183,32 @@ __global__ __launch_bounds__(256, 2) void layernorm_rows_kernel(const int8_t* __
         chunk_of[i] = valid[i] ? chunk : 0;
     }
 
+    // Rows travel through buffer descriptors that end where the tensors end: a chunk that does not exist (a row past the
+    // end, a lane past the row's last chunk, a null sum_out) is an offset beyond the descriptor, reads as zero and is
+    // dropped on a store, so that no load or store sits inside a branch. The compiler counts outstanding memory
+    // operations from the youngest back; one conditional operation between a load and its use would turn every wait for
+    // that load into a wait for everything, stores included.
+    typedef unsigned v4u __attribute__((ext_vector_type(4)));
+    constexpr unsigned NOWHERE = 0xfffffff0u;
+    const int tensor_bytes = rows * cols;  // < 2^31: the host splits larger tensors over several launches
+    const auto rsrc_x = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(x), 0, tensor_bytes, 0x00020000);
+    const auto rsrc_x2 = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(x2), 0, FUSE_ADD ? tensor_bytes : 0, 0x00020000);
+    const auto rsrc_sum = __builtin_amdgcn_make_buffer_rsrc(sum_out, 0, sum_out ? tensor_bytes : 0, 0x00020000);
+    const auto rsrc_out = __builtin_amdgcn_make_buffer_rsrc(out, 0, tensor_bytes, 0x00020000);
+    constexpr int NT = 2;  // non-temporal
+    auto offset_of = [&](int row, int i) {
+        return row < rows && valid[i] ? static_cast<unsigned>(row) * static_cast<unsigned>(cols) + chunk_of[i] * 16 : NOWHERE;
+    };
     v4i nx[NCH], nx2[NCH];
     auto fetch = [&](int row) {
-        const bool live = row < rows;
-        const int64_t base = static_cast<int64_t>(row) * cols;
 #pragma unroll
         for (int i = 0; i < NCH; ++i) {
-            nx[i] = v4i{0, 0, 0, 0};
-            if (FUSE_ADD) nx2[i] = v4i{0, 0, 0, 0};
-            if (live && valid[i]) {
-                nx[i] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(x + base + chunk_of[i] * 16));
-                if (FUSE_ADD)
-                    nx2[i] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(x2 + base + chunk_of[i] * 16));
-            }
+            nx[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, offset_of(row, i), 0, NT));
+            if (FUSE_ADD) nx2[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_x2, offset_of(row, i), 0, NT));
         }
+    };
+    auto put = [&](__amdgpu_buffer_rsrc_t rsrc, const v4i& v, int row, int i) {
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v), rsrc, offset_of(row, i), 0, NT);
     };
 
     // The parameter words are requested first and the first rows right behind them: loads return in issue
@@ -204,18 +219,17 @@ __global__ __launch_bounds__(256, 2) void layernorm_rows_kernel(const int8_t* __
         return *reinterpret_cast<const v4i*>((is_beta ? beta : gamma) + (is_beta ? hc - 2 * nchunks : hc) * 8);
     };
     v4i first_word = v4i{0, 0, 0, 0};
-    if (static_cast<int>(threadIdx.x) < n_half_chunks) first_word = param_word(threadIdx.x);
+    first_word = param_word(min(static_cast<int>(threadIdx.x), n_half_chunks - 1));  // unconditional: see the rows' loads
     int row0 = wave * G;
-    if (row0 < rows) fetch(row0 + grp);
+    fetch(row0 + grp);
 
     // half-chunk hc = 8 columns = quads 2*(hc&1), 2*(hc&1)+1 of chunk hc>>1.
     // as_float: gamma as float, beta scaled to the output's unit, biased and offset (the float form's operands)
-    auto stage_params = [&](bool as_float) {
+    auto stage_word = [&](int hc, const v4i& raw, bool as_float) {
         int wide = 0;
-        for (int hc = threadIdx.x; hc < n_half_chunks; hc += blockDim.x) {
+        {
             const bool is_beta = hc >= 2 * nchunks;
             const int h = is_beta ? hc - 2 * nchunks : hc;
-            const v4i raw = hc == static_cast<int>(threadIdx.x) ? first_word : param_word(hc);
             int* dst = is_beta ? lb : lg;
             const int chunk = h >> 1, q0 = (h & 1) * 2;
             v4i q[2];
@@ -239,6 +253,14 @@ __global__ __launch_bounds__(256, 2) void layernorm_rows_kernel(const int8_t* __
         }
         return wide;
     };
+    // the word requested ahead is staged outside the loop over the others, so that no load stands between its request
+    // and its use on any path
+    auto stage_params = [&](bool as_float) {
+        int wide = 0;
+        if (static_cast<int>(threadIdx.x) < n_half_chunks) wide |= stage_word(threadIdx.x, first_word, as_float);
+        for (int hc = threadIdx.x + blockDim.x; hc < n_half_chunks; hc += blockDim.x) wide |= stage_word(hc, param_word(hc), as_float);
+        return wide;
+    };
     bool in_float = false;
     if (FR >= 0) {
         // staged for the float form first; a block that meets a gamma beyond its range stages again as integers
@@ -252,36 +274,39 @@ __global__ __launch_bounds__(256, 2) void layernorm_rows_kernel(const int8_t* __
         __syncthreads();
     }
 
-    for (; row0 < rows; row0 += nwaves * G) {
-        const int row = row0 + grp;
-        const bool live = row < rows;
-        const int64_t base = static_cast<int64_t>(row) * cols;
-        v4i xv[NCH];
-        int sx = 0, sq = 0;
+    // One loop per form of the normalisation (the choice is the block's, made above): a loop with a single path lets the
+    // compiler count the loads and stores in flight exactly.
+    auto row_loop = [&](auto float_tag) {
+        constexpr bool AS_FLOAT = decltype(float_tag)::value;
+        for (; row0 < rows; row0 += nwaves * G) {
+            const int row = row0 + grp;
+            v4i xv[NCH];
+            int sx = 0, sq = 0;
 #pragma unroll
-        for (int i = 0; i < NCH; ++i) {
-            xv[i] = nx[i];
+            for (int i = 0; i < NCH; ++i) {
+                xv[i] = nx[i];
+                if (FUSE_ADD) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) xv[i][j] = static_cast<int>(sat_add_i8x4(xv[i][j], nx2[i][j]));
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);  // every register of this group is taken over before the next loads may land
+            fetch(row + nwaves * G);            // past the last row: zeros, never used
             if (FUSE_ADD) {
 #pragma unroll
-                for (int j = 0; j < 4; ++j) xv[i][j] = static_cast<int>(sat_add_i8x4(xv[i][j], nx2[i][j]));
-                if (sum_out && live && valid[i])
-                    __builtin_nontemporal_store(xv[i], reinterpret_cast<v4i*>(sum_out + base + chunk_of[i] * 16));
+                for (int i = 0; i < NCH; ++i) put(rsrc_sum, xv[i], row, i);
             }
-        }
-        if (row0 + nwaves * G < rows) fetch(row + nwaves * G);
 #pragma unroll
-        for (int i = 0; i < NCH; ++i) {
+            for (int i = 0; i < NCH; ++i) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                sx = __builtin_amdgcn_sdot4(xv[i][j], 0x01010101, sx, false);
-                sq = __builtin_amdgcn_sdot4(xv[i][j], xv[i][j], sq, false);
+                for (int j = 0; j < 4; ++j) {
+                    sx = __builtin_amdgcn_sdot4(xv[i][j], 0x01010101, sx, false);
+                    sq = __builtin_amdgcn_sdot4(xv[i][j], xv[i][j], sq, false);
+                }
             }
-        }
-        sx = group_allreduce<L>(sx, OpAdd());
-        sq = group_allreduce<L>(sq, OpAdd());
-        const RowStats st = row_stats(sx, sq, cols, log2c, eps_q0);
-
-        if (FR >= 0 && in_float) {
+            sx = group_allreduce<L>(sx, OpAdd());
+            sq = group_allreduce<L>(sq, OpAdd());
+            const RowStats st = row_stats(sx, sq, cols, log2c, eps_q0);
             const float inv_s = static_cast<float>(st.inv) * lf.s1;
             const float nm = -static_cast<float>(st.mu + 128) * lf.c;
 #pragma unroll
@@ -290,49 +315,44 @@ __global__ __launch_bounds__(256, 2) void layernorm_rows_kernel(const int8_t* __
 #pragma unroll
                 for (int w = 0; w < 4; ++w) {
                     const int at = (w * nchunks + chunk_of[i]) << 2;
-                    const v4f g4 = *reinterpret_cast<const v4f*>(lg + at);
-                    const v4f b4 = *reinterpret_cast<const v4f*>(lb + at);
-                    const unsigned word = static_cast<unsigned>(xv[i][w]) ^ 0x80808080u;
-                    unsigned packed = 0;
+                    if (AS_FLOAT) {
+                        const v4f g4 = *reinterpret_cast<const v4f*>(lg + at);
+                        const v4f b4 = *reinterpret_cast<const v4f*>(lb + at);
+                        const unsigned word = static_cast<unsigned>(xv[i][w]) ^ 0x80808080u;
+                        unsigned packed = 0;
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const float vd = fmaf(static_cast<float>((word >> (8 * j)) & 0xffu), lf.c, nm);
-                        float p;
-                        if (FR == 0) p = rintf(inv_s * g4[j]);
-                        if (FR == 1) p = floorf(fmaf(inv_s, g4[j], lf.h1));
-                        if (FR == 2) p = ceilf(fmaf(inv_s, g4[j], lf.h1));
-                        const float fs = __builtin_amdgcn_fmed3f(p, -32768.f, 32767.f);
-                        float y = fmaf(vd, fs, b4[j]);
-                        if (FR == 1) y = floorf(y);
-                        if (FR == 2) y = ceilf(y);
-                        packed = __builtin_amdgcn_cvt_pk_u8_f32(y, j, packed);
+                        for (int j = 0; j < 4; ++j) {
+                            const float vd = fmaf(static_cast<float>((word >> (8 * j)) & 0xffu), lf.c, nm);
+                            float p = 0.f;
+                            if (FR == 0) p = rintf(inv_s * g4[j]);
+                            if (FR == 1) p = floorf(fmaf(inv_s, g4[j], lf.h1));
+                            if (FR == 2) p = ceilf(fmaf(inv_s, g4[j], lf.h1));
+                            const float fs = __builtin_amdgcn_fmed3f(p, -32768.f, 32767.f);
+                            float y = fmaf(vd, fs, b4[j]);
+                            if (FR == 1) y = floorf(y);
+                            if (FR == 2) y = ceilf(y);
+                            packed = __builtin_amdgcn_cvt_pk_u8_f32(y, j, packed);
+                        }
+                        o[w] = static_cast<int>(packed ^ 0x80808080u);
+                    } else {
+                        const v4i g4 = *reinterpret_cast<const v4i*>(lg + at);
+                        const v4i b4 = *reinterpret_cast<const v4i*>(lb + at);
+                        int y4[4];
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const int vd = sext8(xv[i][w], j) - st.mu;
+                            const int fs = clamp_i(ln_round<BIT>(__mul24(st.inv, g4[j]), rg), -32768, 32767);
+                            y4[j] = clamp_i(ln_round<BIT>(__mul24(vd, fs) + b4[j], ro), -128, 127);
+                        }
+                        o[w] = static_cast<int>(pack4_bytes(y4[0], y4[1], y4[2], y4[3]));
                     }
-                    o[w] = static_cast<int>(packed ^ 0x80808080u);
                 }
-                if (live && valid[i]) __builtin_nontemporal_store(o, reinterpret_cast<v4i*>(out + base + chunk_of[i] * 16));
+                put(rsrc_out, o, row, i);
             }
-            continue;
         }
-#pragma unroll
-        for (int i = 0; i < NCH; ++i) {
-            v4i o;
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                const int at = (w * nchunks + chunk_of[i]) << 2;
-                const v4i g4 = *reinterpret_cast<const v4i*>(lg + at);
-                const v4i b4 = *reinterpret_cast<const v4i*>(lb + at);
-                int y4[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int vd = sext8(xv[i][w], j) - st.mu;
-                    const int fs = clamp_i(ln_round<BIT>(__mul24(st.inv, g4[j]), rg), -32768, 32767);
-                    y4[j] = clamp_i(ln_round<BIT>(__mul24(vd, fs) + b4[j], ro), -128, 127);
-                }
-                o[w] = static_cast<int>(pack4_bytes(y4[0], y4[1], y4[2], y4[3]));
-            }
-            if (live && valid[i]) __builtin_nontemporal_store(o, reinterpret_cast<v4i*>(out + base + chunk_of[i] * 16));
-        }
-    }
+    };
+    if (FR >= 0 && in_float) row_loop(std::true_type{});
+    else row_loop(std::false_type{});
 }
 
 // Any column count / alignment / add shift: one 256-thread block per row, three passes over global
@@ -440,16 +460,26 @@ static int layernorm_dispatch(const int8_t* a, const int8_t* b, int add_shift, i
         // phases of all waves in step with each other). Measured on 16384 x 1024: 8.9 us against 9.5 us with four
         // blocks per CU and 10.2 us with 2.5.
         const int max_grid = 256 * 3;
+        // the kernel addresses its tensors with 32-bit offsets: launches of less than 2 GiB each
+        const int64_t rows_per_launch = std::max<int64_t>(1, ((int64_t{1} << 31) - 1) / cols);
+        for (int64_t r0 = 0; r0 < rows; r0 += rows_per_launch) {
+            const int nrows = static_cast<int>(std::min(rows_per_launch, rows - r0));
+            const int64_t skip = r0 * cols;
+            const int8_t* ac = a + skip;
+            const int8_t* bc = b ? b + skip : nullptr;
+            int8_t* sc = sum_out ? sum_out + skip : nullptr;
+            int8_t* oc = out + skip;
 #define A4G_LN_GO(L, NCH)                                                                                                \
-    launch_ln_rows<L, NCH>(bit_kind, fr, fuse, grid_for(rows, 4 * (64 / L), max_grid), lds, stream, a, b, gamma, beta,    \
-                           sum_out, out, (int)rows, (int)cols, log2c, eps_q0, rg, ro, lf)
-        if (nchunks <= 16) A4G_LN_GO(8, 2);
-        else if (nchunks <= 32) A4G_LN_GO(16, 2);
-        else if (nchunks <= 48) A4G_LN_GO(16, 3);
-        else if (nchunks <= 64) A4G_LN_GO(32, 2);
-        else if (nchunks <= 128) A4G_LN_GO(64, 2);
-        else A4G_LN_GO(64, 4);
+    launch_ln_rows<L, NCH>(bit_kind, fr, fuse, grid_for(nrows, 4 * (64 / L), max_grid), lds, stream, ac, bc, gamma, beta, \
+                           sc, oc, nrows, (int)cols, log2c, eps_q0, rg, ro, lf)
+            if (nchunks <= 16) A4G_LN_GO(8, 2);
+            else if (nchunks <= 32) A4G_LN_GO(16, 2);
+            else if (nchunks <= 48) A4G_LN_GO(16, 3);
+            else if (nchunks <= 64) A4G_LN_GO(32, 2);
+            else if (nchunks <= 128) A4G_LN_GO(64, 2);
+            else A4G_LN_GO(64, 4);
 #undef A4G_LN_GO
+        }
     } else {
         const int grid = grid_for(rows, 1, 256 * 8);
         layernorm_generic_kernel<<<grid, 256, 0, stream>>>(a, b, add_shift, add_mode, gamma, beta, sum_out, out, (int)rows,

@@ -683,6 +683,25 @@ def test_layernorm_gamma_at_the_float_limit(ops, oracle, mode, gmax):
     assert np.array_equal(got, oracle.add_layernorm(a, b, gamma, beta, 6, mode)), (mode, gmax)
 
 
+def test_layernorm_tensor_beyond_two_gib(ops, oracle):
+    """The row kernel addresses its tensors with 32-bit offsets; the host splits a larger tensor over several launches.
+    Rows on both sides of the split and at the very end are checked."""
+    import torch
+
+    cols = 4096
+    per_launch = (2**31 - 1) // cols
+    rows = per_launch + 5
+    r = rng(99)
+    gamma, beta = ln_params(r, cols)
+    x = torch.randint(-128, 128, (rows, cols), dtype=torch.int8, device='cuda')
+    y = ops.layernorm(x, dev(gamma), dev(beta), 5, 'conv_even')
+    pick = torch.tensor([0, 1, per_launch - 1, per_launch, per_launch + 1, rows - 1], device='cuda')
+    exp = oracle.layernorm(host(x[pick]), gamma, beta, 5, 'conv_even')
+    assert np.array_equal(host(y[pick]), exp)
+    del x, y
+    torch.cuda.empty_cache()
+
+
 @pytest.mark.parametrize('cols', [64, 768, 1024, 100])
 def test_add_layernorm_fused(ops, oracle, cols):
     r = rng(cols + 7)
