@@ -810,6 +810,38 @@ def test_dense_add_layernorm_degenerate_rows(ops, oracle):
         assert np.array_equal(got, exp), lmode
 
 
+def test_dense_add_layernorm_pitched_through_the_c_abi(ops, oracle):
+    """Activations, residual and result as column windows of wider buffers (row pitches larger than the rows), 64 rows
+    per workgroup not taken; what lies outside the result window must stay untouched."""
+    import ctypes
+    from aie4ml_amd import _lib
+    L = _lib.load()
+    r = rng(123)
+    M, K, N = 77, 256, 96
+    lda, ldr, ldo = 320, 128, 160
+    abuf = gauss8(r, 40, (M, lda))
+    rbuf = gauss8(r, 50, (M, ldr))
+    W = gauss8(r, 30, (K, N))
+    b = r.integers(-2**14, 2**14, N).astype(np.int32)
+    gamma, beta = ln_params(r, N)
+    p = ops.pack_dense(dev(W), dev(b), np.array([8], np.int32))
+    wf = torch.empty(N * K, dtype=torch.int8, device='cuda')
+    vp = lambda t: ctypes.c_void_p(t.data_ptr())  # noqa: E731
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    assert L.a4g_rowpack_weights_i8(vp(p.wt), p.ldwt, N, K, vp(wf), stream) == 0
+    da, dr, dg, dbt = dev(abuf), dev(rbuf), dev(gamma), dev(beta)
+    out = torch.full((M, ldo), 99, dtype=torch.int8, device='cuda')
+    a_win, r_win, o_win = da[:, 64:], dr[:, 32:], out[:, 16:]   # 16-byte aligned windows
+    rc = L.a4g_dense_add_layernorm_i8(vp(a_win), 0, lda, vp(wf), None, vp(p.bias), 8, 6, 0, vp(r_win), ldr, vp(dg), vp(dbt),
+                                      vp(o_win), ldo, M, N, K, 1, 7, 5, 6, stream)
+    assert rc == 0, L.a4g_last_error()
+    got = host(out)
+    y = oracle.dense(abuf[:, 64:64 + K], W, b, 8, 'conv_even', out='int8')
+    exp = oracle.add_layernorm(y, rbuf[:, 32:32 + N], gamma, beta, 5, 'conv_even')
+    assert np.array_equal(got[:, 16:16 + N], exp)
+    assert (got[:, :16] == 99).all() and (got[:, 16 + N:] == 99).all()
+
+
 def test_dense_add_layernorm_refuses_what_it_cannot_take(ops):
     r = rng(9)
     W = gauss8(r, 30, (100, 64))  # K not a multiple of 128
