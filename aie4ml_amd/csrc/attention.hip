@@ -27,6 +27,7 @@ struct AttnArgs {
     int64_t v_sb, v_sh, v_ss;
     int64_t o_sb, o_sh, o_ss;
     int heads, sq;
+    int sk;     // key / value rows that exist (the ragged form; the kernel's tiles cover the next power of two of 32s)
     int items;  // (batch, head, block of query rows) triples in all
     FastRound lr, orr;  // logits and output requantisation
     SoftmaxParams sm;
@@ -52,11 +53,14 @@ __device__ __forceinline__ void transpose4x4(const unsigned a[4], unsigned c[4])
 // v_cvt_pk_u8_f32 (nearest even, saturating to 0..255, writing one byte of a dword) is the rounding, the int8
 // saturation (biased by 128) and the packing at once. FASTP: the probabilities need no clamp and their shift is
 // at most 16, so p = (e * inv) >> shift is read as byte 2 of e * (inv << (16 - shift)).
+// RAGGED: fewer keys exist than the NT tiles cover (any count >= 1). K rows past the end alias the last row, V rows
+// past the end load as zero; their logits are forced to the minimum (they cannot raise the row maximum), their scores
+// to zero (they add nothing to the row sum, and a zero probability times a zero V row nothing to the output).
 // NW = waves per workgroup. 4: two workgroups share a CU. 8: one workgroup of 256 query rows per CU, which
 // leaves room to store the score table once per LDS bank (entry d for lane c at dword d * 64 + c, byte address
 // (d << 8) | (c << 2) built by one v_perm): with a single copy, lanes that gather different gaps from one bank
 // serialise, and those conflicts were two thirds of this kernel's LDS cycles.
-template <int NT, int DT, int BIT, bool FASTP, int NW = 4>
+template <int NT, int DT, int BIT, bool FASTP, int NW = 4, bool RAGGED = false>
 __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(AttnArgs a) {
     constexpr int SK = NT * 32, D = DT * 32, PITCH = SK + 16;
     constexpr bool BANKED = NW == 8;
@@ -122,7 +126,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
 #pragma unroll
         for (int ks = 0; ks < DT; ++ks) {
             qf[ks] = *reinterpret_cast<const v4i*>(Qp + rowc * a.q_ss + ks * 32 + half * 16);
-            kf[0][ks] = *reinterpret_cast<const v4i*>(Kp + m * a.k_ss + ks * 32 + half * 16);
+            kf[0][ks] = *reinterpret_cast<const v4i*>(Kp + (RAGGED ? min(m, a.sk - 1) : m) * a.k_ss + ks * 32 + half * 16);
         }
 #pragma unroll
         for (int it = 0; it < VB; ++it) {
@@ -130,7 +134,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
             const int k0 = (blk / (D / 4)) * 4;
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                av[it][i] = blk < NB ? *reinterpret_cast<const unsigned*>(Vp + (k0 + i) * a.v_ss + n0) : 0u;
+                av[it][i] = blk < NB && (!RAGGED || k0 + i < a.sk) ? *reinterpret_cast<const unsigned*>(Vp + (k0 + i) * a.v_ss + n0) : 0u;
         }
     };
     // requested before anything is done with LDS, so that (first item) building the score table hides the latency
@@ -191,8 +195,8 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
         if (t + 1 < NT) {
 #pragma unroll
             for (int ks = 0; ks < DT; ++ks)
-                kf[(t + 1) & 1][ks] =
-                    *reinterpret_cast<const v4i*>(Kp + ((t + 1) * 32 + m) * a.k_ss + ks * 32 + half * 16);
+                kf[(t + 1) & 1][ks] = *reinterpret_cast<const v4i*>(
+                    Kp + (RAGGED ? min((t + 1) * 32 + m, a.sk - 1) : (t + 1) * 32 + m) * a.k_ss + ks * 32 + half * 16);
         }
         v16i acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
@@ -200,10 +204,15 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
             acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[t & 1][ks], qf[ks], acc, 0, 0, 0);
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
+            // accumulator 4 g + i belongs to key 32 t + 8 g + 4 half + i: `left` of this group's four keys exist
+            const int left = RAGGED ? a.sk - (t * 32 + 8 * g + 4 * half) : 4;
             if (BIT == 3) {
                 float f[4];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) f[i] = fmaf(static_cast<float>(acc[4 * g + i]), a.lscale, 128.f);
+                for (int i = 0; i < 4; ++i) {
+                    f[i] = fmaf(static_cast<float>(acc[4 * g + i]), a.lscale, 128.f);
+                    if (RAGGED) f[i] = i < left ? f[i] : 0.f;
+                }
                 // two three-operand maxima
                 mxf = __builtin_fmaxf(__builtin_fmaxf(mxf, f[0]), f[1]);
                 mxf = __builtin_fmaxf(__builtin_fmaxf(mxf, f[2]), f[3]);
@@ -214,7 +223,10 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
             } else {
                 int y[4];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) y[i] = clamp_i(fast_round_k<BIT>(acc[4 * g + i], a.lr), -128, 127);
+                for (int i = 0; i < 4; ++i) {
+                    y[i] = clamp_i(fast_round_k<BIT>(acc[4 * g + i], a.lr), -128, 127);
+                    if (RAGGED) y[i] = i < left ? y[i] : -128;
+                }
                 mx = max(max(mx, y[0]), max(y[1], max(y[2], y[3])));
                 lg[t][g] = pack4_bytes(y[0], y[1], y[2], y[3]) ^ 0x80808080u;
             }
@@ -256,6 +268,13 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
                 e1 = *reinterpret_cast<const int*>(tbytes + byte_x4<1>(d4, two));
                 e2 = *reinterpret_cast<const int*>(tbytes + byte_x4<2>(d4, two));
                 e3 = *reinterpret_cast<const int*>(tbytes + byte_x4<3>(d4, two));
+            }
+            if (RAGGED) {
+                const int left = a.sk - (t * 32 + 8 * g + 4 * half);
+                e0 = left > 0 ? e0 : 0;
+                e1 = left > 1 ? e1 : 0;
+                e2 = left > 2 ? e2 : 0;
+                e3 = left > 3 ? e3 : 0;
             }
             sum += (e0 + e1) + (e2 + e3);
             if (t >= NT - PARK) {
@@ -356,8 +375,12 @@ static void launch_attention_wide(int grid8, size_t lds, hipStream_t stream, con
 template <int NT, int DT>
 static void launch_attention_nt(int grid, int grid8, size_t lds, hipStream_t stream, const AttnArgs& a) {
     const bool fastp = a.noclamp && a.sm.out_shift <= 16;
+    const bool ragged = a.sk != NT * 32;  // always in workgroups of four waves (grid8 == 0)
 #define A4G_ATTN(B)                                                                  \
-    if (NT >= 8 && grid8 > 0) {                                                      \
+    if (ragged) {                                                                    \
+        if (fastp) attention_kernel<NT, DT, B, true, 4, true><<<grid, 256, lds, stream>>>(a);   \
+        else attention_kernel<NT, DT, B, false, 4, true><<<grid, 256, lds, stream>>>(a);        \
+    } else if (NT >= 8 && grid8 > 0) {                                                      \
         if constexpr (NT >= 8) {                                                     \
             if (fastp) launch_attention_wide<NT, DT, B, true>(grid8, lds, stream, a); \
             else launch_attention_wide<NT, DT, B, false>(grid8, lds, stream, a);      \
@@ -417,10 +440,11 @@ extern "C" int a4g_attention_i8(const int8_t* Q, const int8_t* K, const int8_t* 
         if (int rc = make_hccs_params(who, sk, hccs_B, hccs_S, hccs_Dmax, inv_shift, use_clb, A4G_U8, &a.sm, &noclamp))
             return rc;
     }
-    const bool pow2_tiles = sk % 32 == 0 && sk <= 512 && ((sk / 32) & (sk / 32 - 1)) == 0;
-    A4G_REQUIRE(d == 64 && pow2_tiles, A4G_ERR_UNSUPPORTED,
-                "%s: fused path covers head_dim 64 and 32/64/128/256/512 keys, got d=%lld sk=%lld", who, (long long)d,
-                (long long)sk);
+    A4G_REQUIRE(d == 64 && sk <= 512, A4G_ERR_UNSUPPORTED,
+                "%s: fused path covers head_dim 64 and up to 512 keys, got d=%lld sk=%lld", who, (long long)d, (long long)sk);
+    int nt = 1;  // tiles of 32 keys the kernel is instantiated for: the next power of two
+    while (nt * 32 < sk) nt *= 2;
+    const bool ragged = nt * 32 != sk;
     A4G_REQUIRE(batch * heads * ((sq + 127) / 128) <= INT32_MAX && sq <= (1 << 24), A4G_ERR_UNSUPPORTED, "%s: too many rows", who);
     if (batch == 0) return A4G_OK;
     A4G_REQUIRE(Q && K && V && O && strides, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
@@ -436,6 +460,7 @@ extern "C" int a4g_attention_i8(const int8_t* Q, const int8_t* K, const int8_t* 
     a.o_sb = strides[9]; a.o_sh = strides[10]; a.o_ss = strides[11];
     a.heads = static_cast<int>(heads);
     a.sq = static_cast<int>(sq);
+    a.sk = static_cast<int>(sk);
     a.lr = make_fast_round(logit_round_mode, logit_shift);
     a.orr = make_fast_round(out_round_mode, out_shift);
     a.noclamp = noclamp;
@@ -445,9 +470,9 @@ extern "C" int a4g_attention_i8(const int8_t* Q, const int8_t* K, const int8_t* 
     const int grid = static_cast<int>(batch * heads * ((sq + 127) / 128));
     // eight waves per workgroup (256 query rows, bank-replicated score table) once every CU gets at least one
     const int64_t wg8 = batch * heads * ((sq + 255) / 256);
-    const int grid8 = (sq >= 256 && wg8 >= 256) ? static_cast<int>(wg8) : 0;
+    const int grid8 = (!ragged && sq >= 256 && wg8 >= 256) ? static_cast<int>(wg8) : 0;
     a.items = grid8 > 0 ? grid8 : grid;
-    if (launch_attention<2>(static_cast<int>(sk / 32), grid, grid8, stream, a))
+    if (launch_attention<2>(nt, grid, grid8, stream, a))
         return fail(A4G_ERR_UNSUPPORTED, "%s: no kernel for sk=%lld", who, (long long)sk);
     return check_hip(hipGetLastError(), who);
 }

@@ -437,7 +437,7 @@ class PlanGpuFusion(AIEPass):
 
     # ---- attention -------------------------------------------------------------------------------------
     ATTN_HEAD_DIM = 64
-    ATTN_KEYS = (32, 64, 128, 256, 512)
+    ATTN_MAX_KEYS = 512
     ATTN_MAX_SHIFT = 24
 
     def _plan_attention(self, graph, execution, outputs):
@@ -469,7 +469,7 @@ class PlanGpuFusion(AIEPass):
             if len(q.shape) != len(k.shape) or len(k.shape) != len(v.shape) or tuple(k.shape) != tuple(v.shape) \
                     or tuple(q.shape[:-2]) != tuple(k.shape[:-2]) or len(q.shape) not in (2, 3, 4):
                 continue
-            if int(q.shape[-1]) != self.ATTN_HEAD_DIM or int(k.shape[-2]) not in self.ATTN_KEYS:
+            if int(q.shape[-1]) != self.ATTN_HEAD_DIM or not 1 <= int(k.shape[-2]) <= self.ATTN_MAX_KEYS:
                 continue
             if c1.shift > self.ATTN_MAX_SHIFT or c3.shift > self.ATTN_MAX_SHIFT:
                 continue  # the fused kernel takes shifts up to 24, the MatMul kernels up to 31

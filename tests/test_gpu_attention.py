@@ -64,6 +64,42 @@ def test_attention_ragged_query_count(oracle, sq):
     np.testing.assert_array_equal(got, reference(oracle, q, k, v, 6, 'symmetric_inf', sm, 8, 'floor'))
 
 
+@pytest.mark.parametrize('sk', [1, 5, 31, 33, 96, 100, 197, 250, 300, 511])
+@pytest.mark.parametrize('kind', ['exp', 'hccs'])
+def test_attention_key_count_off_the_tile_grid(oracle, sk, kind):
+    """Any number of keys up to 512: the kernel of the next power of two runs with the missing keys masked (they
+    must neither raise a row's maximum, nor add to its sum, nor to the output). Self-attention shapes (sq == sk, as
+    a 197-token ViT block has them), plus a query count of its own; both forms of the logit requantisation."""
+    for sq in (sk, 70):
+        q, k, v = qkv(1000 + sk + sq, (2, 3, sq, 64), (2, 3, sk, 64), sigma=30.0)
+        if kind == 'exp':
+            sm = {'kind': 'exp', 'exp_kq': 23}
+        else:
+            if sk == 1:
+                return  # the parameter rules of HCCS (cols * (B - S * Dmax) >= 256, B <= 255) leave nothing for one key
+            B = min(255, 32767 // sk)
+            sm = {'kind': 'hccs', 'B': B, 'S': 1, 'Dmax': min(126, B - (256 + sk - 1) // sk)}
+        lmode = 'conv_even' if sk % 2 else 'symmetric_inf'
+        got = ops.attention(dev(q), dev(k), dev(v), 6, lmode, sm, 7, 'conv_even').cpu().numpy()
+        np.testing.assert_array_equal(got, reference(oracle, q, k, v, 6, lmode, sm, 7, 'conv_even'))
+
+
+def test_attention_masked_keys_do_not_leak(oracle):
+    """The rows behind the last key are other tensors' memory: whatever they hold, the result is that of the keys that
+    exist (K rows past the end alias the last row inside the kernel, V rows past the end are not read)."""
+    sk = 100
+    r = np.random.default_rng(5)
+    big_k = np.full((2, 128, 64), 127, np.int8)
+    big_v = np.full((2, 128, 64), -128, np.int8)
+    big_k[:, :sk] = np.clip(np.rint(r.normal(0, 30, (2, sk, 64))), -128, 127)
+    big_v[:, :sk] = np.clip(np.rint(r.normal(0, 30, (2, sk, 64))), -128, 127)
+    q = np.clip(np.rint(r.normal(0, 30, (2, sk, 64))), -128, 127).astype(np.int8)
+    sm = {'kind': 'exp', 'exp_kq': 23}
+    got = ops.attention(dev(q), dev(big_k)[:, :sk], dev(big_v)[:, :sk], 6, 'conv_even', sm, 7, 'floor').cpu().numpy()
+    want = reference(oracle, q, big_k[:, :sk].copy(), big_v[:, :sk].copy(), 6, 'conv_even', sm, 7, 'floor')
+    np.testing.assert_array_equal(got, want)
+
+
 @pytest.mark.parametrize('sq,sk', [(512, 512), (300, 256), (256, 512)])
 @pytest.mark.parametrize('mode', ['conv_even', 'symmetric_inf', 'floor'])
 def test_attention_with_256_row_workgroups(oracle, sq, sk, mode):
@@ -144,7 +180,7 @@ def test_attention_uncovered_shapes_and_bad_parameters():
     q = torch.zeros((2, 64, 32), dtype=torch.int8, device='cuda')
     with pytest.raises(NotImplementedError, match='fused path covers head_dim 64'):
         ops.attention(q, q, q, 6, 'floor', {'kind': 'exp', 'exp_kq': 23}, 7, 'floor')
-    q = torch.zeros((2, 96, 64), dtype=torch.int8, device='cuda')
+    q = torch.zeros((2, 544, 64), dtype=torch.int8, device='cuda')
     with pytest.raises(NotImplementedError, match='fused path covers'):
         ops.attention(q, q, q, 6, 'floor', {'kind': 'exp', 'exp_kq': 23}, 7, 'floor')
     q = torch.zeros((2, 64, 64), dtype=torch.int8, device='cuda')

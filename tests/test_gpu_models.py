@@ -166,6 +166,26 @@ def test_encoder_block_small(oracle, softmax):
     assert len(np.unique(out)) > 32        # a live signal, not a saturated or constant tensor
 
 
+@pytest.mark.parametrize('seq', [100, 197])
+def test_encoder_block_with_a_sequence_off_the_tile_grid(oracle, seq):
+    """A vision transformer's token counts (196 patches + 1, or 100): the heads still go to the fused attention
+    launch, which masks the keys that its tiles of 32 have too many."""
+    model, x = workloads.c5_encoder_block(batch=2, seq=seq, hidden=128, heads=2, ffn=256, softmax='exp')
+    model.compile()
+    (grp,) = model.context.config['gpu_fusion_plan']['attention']
+    assert len(grp['heads']) == 2 and grp['concat']
+    import torch
+
+    trace = []
+    dx = {'x': torch.from_numpy(x).cuda()}
+    model.execute(dx, trace=trace)
+    assert [t['kind'] for t in trace].count('attention') == 1 and not any(t['kind'] in ('matmul', 'softmax') for t in trace)
+    got = _graph_check(model, oracle, {'x': x})
+    model.context.config['gpu_fusion_plan'] = {}        # and the same graph operator by operator
+    _graph_check(model, oracle, {'x': x})
+    assert len(np.unique(next(iter(got.values())))) > 32
+
+
 def test_encoder_block_c5_shape(oracle):
     """BERT-base geometry (hidden 768, 12 heads of 64, FFN 3072, seq 128) on a batch the oracle finishes
     in seconds; the full batch of 64 differs only in the number of independent sequences."""
