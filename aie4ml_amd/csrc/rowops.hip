@@ -221,7 +221,10 @@ __global__ __launch_bounds__(256, 2) void layernorm_rows_kernel(const int8_t* __
     v4i first_word = v4i{0, 0, 0, 0};
     first_word = param_word(min(static_cast<int>(threadIdx.x), n_half_chunks - 1));  // unconditional: see the rows' loads
     int row0 = wave * G;
-    fetch(row0 + grp);
+    // Rows of thousands of columns fill the registers by themselves (16 per 256 columns and operand): those forms fetch
+    // a row when its turn comes instead of one turn ahead, and leave the overlap to the other waves of the CU.
+    constexpr bool AHEAD = NCH <= 4 || (NCH <= 8 && !FUSE_ADD);
+    if (AHEAD) fetch(row0 + grp);
 
     // half-chunk hc = 8 columns = quads 2*(hc&1), 2*(hc&1)+1 of chunk hc>>1.
     // as_float: gamma as float, beta scaled to the output's unit, biased and offset (the float form's operands)
@@ -282,6 +285,7 @@ __global__ __launch_bounds__(256, 2) void layernorm_rows_kernel(const int8_t* __
             const int row = row0 + grp;
             v4i xv[NCH];
             int sx = 0, sq = 0;
+            if (!AHEAD) fetch(row);
 #pragma unroll
             for (int i = 0; i < NCH; ++i) {
                 xv[i] = nx[i];
@@ -291,7 +295,7 @@ __global__ __launch_bounds__(256, 2) void layernorm_rows_kernel(const int8_t* __
                 }
             }
             __builtin_amdgcn_sched_barrier(0);  // every register of this group is taken over before the next loads may land
-            fetch(row + nwaves * G);            // past the last row: zeros, never used
+            if (AHEAD) fetch(row + nwaves * G);  // past the last row: zeros, never used
             if (FUSE_ADD) {
 #pragma unroll
                 for (int i = 0; i < NCH; ++i) put(rsrc_sum, xv[i], row, i);
@@ -401,23 +405,43 @@ __global__ __launch_bounds__(256) void layernorm_generic_kernel(const int8_t* __
 // The rounding modes pair up as (BIT, FR): conv_even (3, 0), floor / positive_inf (0, 1), ceil / negative_inf (0, 2);
 // the symmetric modes and conv_odd have no float form (FR -1).
 template <int L, int NCH>
-static void launch_ln_rows(int bit_kind, int fr, bool fuse, int grid, size_t lds, hipStream_t stream, const int8_t* x,
+static hipError_t launch_ln_rows(int bit_kind, int fr, bool fuse, int grid, size_t lds, hipStream_t stream, const int8_t* x,
                            const int8_t* x2, const int16_t* gamma, const int16_t* beta, int8_t* sum_out, int8_t* out,
                            int rows, int cols, int log2c, int eps_q0, const LnRound& rg, const LnRound& ro,
                            const LnFloat& lf) {
+    // rows of more than 4096 columns stage more than 32 KiB of parameters: the kernels that take them are allowed the
+    // 128 KiB that 16384 columns need (not the whole LDS: the kernel has a few static bytes of its own; the attribute
+    // is idempotent, the race on the flag benign)
+#define A4G_LN_LDS(KERN)                                                                                                 \
+    if (NCH > 4) {                                                                                                       \
+        static bool attr_set = false;                                                                                    \
+        if (!attr_set) {                                                                                                 \
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(KERN),                                \
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);            \
+            if (e != hipSuccess) return e;                                                                               \
+            attr_set = true;                                                                                             \
+        }                                                                                                                \
+    }
 #define A4G_LN_CASE(B, F)                                                                                                \
     if (bit_kind == B && fr == F) {                                                                                      \
-        if (fuse)                                                                                                        \
-            layernorm_rows_kernel<L, NCH, B, true, F><<<grid, 256, lds, stream>>>(x, x2, gamma, beta, sum_out, out,      \
-                                                                                  rows, cols, log2c, eps_q0, rg, ro, lf); \
-        else                                                                                                             \
-            layernorm_rows_kernel<L, NCH, B, false, F><<<grid, 256, lds, stream>>>(x, nullptr, gamma, beta, nullptr,     \
-                                                                                   out, rows, cols, log2c, eps_q0, rg,   \
-                                                                                   ro, lf);                              \
-        return;                                                                                                          \
+        if (fuse) {                                                                                                      \
+            if constexpr (NCH <= 8) { /* the sixteen-chunk form with a second operand has no registers left */           \
+                auto kern = layernorm_rows_kernel<L, NCH, B, true, F>;                                                   \
+                A4G_LN_LDS(kern)                                                                                         \
+                kern<<<grid, 256, lds, stream>>>(x, x2, gamma, beta, sum_out, out, rows, cols, log2c, eps_q0, rg, ro, lf); \
+            }                                                                                                            \
+        } else {                                                                                                         \
+            auto kern = layernorm_rows_kernel<L, NCH, B, false, F>;                                                      \
+            A4G_LN_LDS(kern)                                                                                             \
+            kern<<<grid, 256, lds, stream>>>(x, nullptr, gamma, beta, nullptr, out, rows, cols, log2c, eps_q0, rg, ro,   \
+                                             lf);                                                                        \
+        }                                                                                                                \
+        return hipSuccess;                                                                                               \
     }
     A4G_LN_CASE(3, 0) A4G_LN_CASE(0, 1) A4G_LN_CASE(0, 2) A4G_LN_CASE(1, -1) A4G_LN_CASE(2, -1) A4G_LN_CASE(4, -1)
 #undef A4G_LN_CASE
+#undef A4G_LN_LDS
+    return hipErrorInvalidValue;  // no such pair of rounding forms
 }
 
 static int layernorm_dispatch(const int8_t* a, const int8_t* b, int add_shift, int add_mode, const int16_t* gamma,
@@ -445,7 +469,7 @@ static int layernorm_dispatch(const int8_t* a, const int8_t* b, int add_shift, i
     }
     const int final_shift = 15 - out_shift;
     const bool fuse = b != nullptr;
-    const bool fast = cols % 16 == 0 && cols <= 4096 && aligned16(a) && aligned16(out) && (!fuse || aligned16(b)) &&
+    const bool fast = cols % 16 == 0 && cols <= (fuse ? 8192 : 16384) && aligned16(a) && aligned16(out) && (!fuse || aligned16(b)) &&
                       (!sum_out || aligned16(sum_out)) && aligned16(gamma) && aligned16(beta) && (!fuse || add_shift == 0);
     if (fast) {
         const int nchunks = static_cast<int>(cols / 16);
@@ -459,7 +483,8 @@ static int layernorm_dispatch(const int8_t* a, const int8_t* b, int add_shift, i
         // group and the stores of the previous one overlap the arithmetic (one group per wave leaves the three
         // phases of all waves in step with each other). Measured on 16384 x 1024: 8.9 us against 9.5 us with four
         // blocks per CU and 10.2 us with 2.5.
-        const int max_grid = 256 * 3;
+        // (fewer where the staged parameters, 8 bytes a column, leave room for fewer)
+        const int max_grid = 256 * static_cast<int>(std::min<size_t>(3, (160 * 1024) / lds));
         // the kernel addresses its tensors with 32-bit offsets: launches of less than 2 GiB each
         const int64_t rows_per_launch = std::max<int64_t>(1, ((int64_t{1} << 31) - 1) / cols);
         for (int64_t r0 = 0; r0 < rows; r0 += rows_per_launch) {
@@ -470,15 +495,22 @@ static int layernorm_dispatch(const int8_t* a, const int8_t* b, int add_shift, i
             int8_t* sc = sum_out ? sum_out + skip : nullptr;
             int8_t* oc = out + skip;
 #define A4G_LN_GO(L, NCH)                                                                                                \
-    launch_ln_rows<L, NCH>(bit_kind, fr, fuse, grid_for(nrows, 4 * (64 / L), max_grid), lds, stream, ac, bc, gamma, beta, \
-                           sc, oc, nrows, (int)cols, log2c, eps_q0, rg, ro, lf)
+    launched = launch_ln_rows<L, NCH>(bit_kind, fr, fuse, grid_for(nrows, 4 * (64 / L), max_grid), lds, stream, ac, bc,  \
+                                      gamma, beta, sc, oc, nrows, (int)cols, log2c, eps_q0, rg, ro, lf)
+            hipError_t launched = hipSuccess;
             if (nchunks <= 16) A4G_LN_GO(8, 2);
             else if (nchunks <= 32) A4G_LN_GO(16, 2);
             else if (nchunks <= 48) A4G_LN_GO(16, 3);
             else if (nchunks <= 64) A4G_LN_GO(32, 2);
             else if (nchunks <= 128) A4G_LN_GO(64, 2);
-            else A4G_LN_GO(64, 4);
+            else if (nchunks <= 256) A4G_LN_GO(64, 4);
+            else if (nchunks <= 320) A4G_LN_GO(64, 5);
+            else if (nchunks <= 384) A4G_LN_GO(64, 6);
+            else if (nchunks <= 448) A4G_LN_GO(64, 7);
+            else if (nchunks <= 512) A4G_LN_GO(64, 8);
+            else A4G_LN_GO(64, 16);
 #undef A4G_LN_GO
+            if (launched != hipSuccess) return check_hip(launched, who);
         }
     } else {
         const int grid = grid_for(rows, 1, 256 * 8);
@@ -574,24 +606,33 @@ __global__ __launch_bounds__(256) void softmax_lut_kernel(const int8_t* __restri
 
         // gaps d = m - x per byte: with both biased to unsigned the word subtraction never borrows
         const unsigned mrep = static_cast<unsigned>((m ^ 0x80) & 0xFF) * 0x01010101u;
-        int e[NCH][16];
+        // Rows of up to 4096 columns keep their scores (16 registers a chunk) between the sum and the products; longer
+        // rows have no room for that and look every score up a second time.
+        constexpr bool KEEP = NCH <= 4;
+        int e[KEEP ? NCH : 1][16];
         int sum = 0;
+        auto scores_of = [&](int i, int w, int (&s4)[4]) {
+            const unsigned d4 = mrep - (static_cast<unsigned>(xv[i][w]) ^ 0x80808080u);
+            s4[0] = *reinterpret_cast<const int*>(tbytes + byte_x4<0>(d4, two));
+            s4[1] = *reinterpret_cast<const int*>(tbytes + byte_x4<1>(d4, two));
+            s4[2] = *reinterpret_cast<const int*>(tbytes + byte_x4<2>(d4, two));
+            s4[3] = *reinterpret_cast<const int*>(tbytes + byte_x4<3>(d4, two));
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const bool in = RAGGED ? (l + L * i) * 16 + w * 4 + j < cols : valid[i];
+                s4[j] = (FULL || (in && valid[i])) ? s4[j] : 0;
+            }
+        };
 #pragma unroll
         for (int i = 0; i < NCH; ++i) {
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
-                const unsigned d4 = mrep - (static_cast<unsigned>(xv[i][w]) ^ 0x80808080u);
                 int s4[4];
-                s4[0] = *reinterpret_cast<const int*>(tbytes + byte_x4<0>(d4, two));
-                s4[1] = *reinterpret_cast<const int*>(tbytes + byte_x4<1>(d4, two));
-                s4[2] = *reinterpret_cast<const int*>(tbytes + byte_x4<2>(d4, two));
-                s4[3] = *reinterpret_cast<const int*>(tbytes + byte_x4<3>(d4, two));
+                scores_of(i, w, s4);
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const bool in = RAGGED ? (l + L * i) * 16 + w * 4 + j < cols : valid[i];
-                    const int s = (FULL || (in && valid[i])) ? s4[j] : 0;
-                    e[i][w * 4 + j] = s;
-                    sum += s;
+                    if (KEEP) e[i][w * 4 + j] = s4[j];
+                    sum += s4[j];
                 }
             }
         }
@@ -603,12 +644,20 @@ __global__ __launch_bounds__(256) void softmax_lut_kernel(const int8_t* __restri
         for (int i = 0; i < NCH; ++i) {
             if (!valid[i]) continue;
             const int col0 = (l + L * i) * 16;
+            int ei[16];
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                int s4[4];
+                if (!KEEP) scores_of(i, w, s4);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) ei[w * 4 + j] = KEEP ? e[i][w * 4 + j] : s4[j];
+            }
             if (p.out_i16) {
                 v4i o[2];
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
-                    const int y0 = sat16(__mul24(e[i][2 * k], inv) >> p.out_shift);
-                    const int y1 = sat16(__mul24(e[i][2 * k + 1], inv) >> p.out_shift);
+                    const int y0 = sat16(__mul24(ei[2 * k], inv) >> p.out_shift);
+                    const int y1 = sat16(__mul24(ei[2 * k + 1], inv) >> p.out_shift);
                     o[k >> 2][k & 3] = static_cast<int>(pack2_halves(y0, y1));
                 }
                 if constexpr (RAGGED) {
@@ -629,13 +678,13 @@ __global__ __launch_bounds__(256) void softmax_lut_kernel(const int8_t* __restri
                     if (FASTP) {
                         unsigned q[4];
 #pragma unroll
-                        for (int j = 0; j < 4; ++j) q[j] = __umul24(static_cast<unsigned>(e[i][w * 4 + j]), inv16);
+                        for (int j = 0; j < 4; ++j) q[j] = __umul24(static_cast<unsigned>(ei[w * 4 + j]), inv16);
                         o[w] = static_cast<int>(__builtin_amdgcn_perm(q[1], q[0], 0x0c0c0602u) |
                                                 __builtin_amdgcn_perm(q[3], q[2], 0x06020c0cu));
                     } else {
                         int y4[4];
 #pragma unroll
-                        for (int j = 0; j < 4; ++j) y4[j] = clamp_i(__mul24(e[i][w * 4 + j], inv) >> p.out_shift, 0, 255);
+                        for (int j = 0; j < 4; ++j) y4[j] = clamp_i(__mul24(ei[w * 4 + j], inv) >> p.out_shift, 0, 255);
                         o[w] = static_cast<int>(pack4_bytes(y4[0], y4[1], y4[2], y4[3]));
                     }
                 }
@@ -688,8 +737,10 @@ static void launch_softmax(bool noclamp, int grid, hipStream_t stream, const int
                            const SoftmaxParams& p, int ragged) {
     const bool fastp = noclamp && !p.out_i16 && p.out_shift <= 16;
     if (ragged >= 0) {
-        if (fastp) softmax_lut_kernel<L, NCH, true, false, true><<<grid, 256, 0, stream>>>(x, out, rows, cols, p, ragged);
-        else softmax_lut_kernel<L, NCH, false, false, true><<<grid, 256, 0, stream>>>(x, out, rows, cols, p, ragged);
+        if constexpr (NCH <= 4) {  // the ragged form stops at 4096 columns
+            if (fastp) softmax_lut_kernel<L, NCH, true, false, true><<<grid, 256, 0, stream>>>(x, out, rows, cols, p, ragged);
+            else softmax_lut_kernel<L, NCH, false, false, true><<<grid, 256, 0, stream>>>(x, out, rows, cols, p, ragged);
+        }
         return;
     }
     const bool full = cols == L * NCH * 16;
@@ -708,7 +759,7 @@ static int softmax_dispatch(const int8_t* x, void* out, int64_t rows, int64_t co
     if (rows == 0) return A4G_OK;
     A4G_REQUIRE(x && out, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
     const bool aligned = cols % 16 == 0 && aligned16(x) && aligned16(out);
-    if (cols <= 4096) {
+    if (cols <= 4096 || (aligned && cols <= 16384)) {
         // rows off the 16-byte grid: the same kernel with loads and stores that respect the row ends; the output has
         // the input's row offsets, so one mode serves both when both bases are equally aligned
         int ragged = -1;
@@ -727,7 +778,9 @@ static int softmax_dispatch(const int8_t* x, void* out, int64_t rows, int64_t co
         const int r = static_cast<int>(rows), c = static_cast<int>(cols);
         if (nch > 1) {  // L == 64
             if (nch <= 2) launch_softmax<64, 2>(noclamp, grid, stream, x, out, r, c, p, ragged);
-            else launch_softmax<64, 4>(noclamp, grid, stream, x, out, r, c, p, ragged);
+            else if (nch <= 4) launch_softmax<64, 4>(noclamp, grid, stream, x, out, r, c, p, ragged);
+            else if (nch <= 8) launch_softmax<64, 8>(noclamp, grid, stream, x, out, r, c, p, ragged);
+            else launch_softmax<64, 16>(noclamp, grid, stream, x, out, r, c, p, ragged);
         } else {
             switch (L) {
             case 1: launch_softmax<1, 1>(noclamp, grid, stream, x, out, r, c, p, ragged); break;

@@ -702,6 +702,33 @@ def test_layernorm_tensor_beyond_two_gib(ops, oracle):
     torch.cuda.empty_cache()
 
 
+@pytest.mark.parametrize('cols', [4112, 5120, 6144, 7168, 8192, 8208, 12288, 16384, 16400])
+@pytest.mark.parametrize('mode', ['conv_even', 'floor', 'symmetric_zero', 'conv_odd'])
+def test_layernorm_long_rows(ops, oracle, cols, mode):
+    """Rows of thousands of columns (the hidden sizes of large transformers): five to sixteen 16-byte chunks per lane,
+    the staged parameters up to 128 KiB of LDS; 16400 is past the row kernel and takes the general one. Both forms of
+    the normalisation (float where the mode has one), more rows than one round of waves, a ragged last round."""
+    r = rng(cols + 3)
+    rows = 301
+    x = gauss8(r, 25, (rows, cols)) + np.int8(-5)
+    gamma, beta = ln_params(r, cols)
+    got = host(ops.layernorm(dev(x), dev(gamma), dev(beta), 6, mode, eps_q0=2))
+    assert np.array_equal(got, oracle.layernorm(x, gamma, beta, 6, mode, eps_q0=2)), (cols, mode)
+
+
+@pytest.mark.parametrize('cols', [4112, 5120, 6144, 7168, 8192, 8208])
+@pytest.mark.parametrize('mode', ['conv_even', 'ceil', 'symmetric_inf'])
+def test_add_layernorm_long_rows(ops, oracle, cols, mode):
+    r = rng(cols + 11)
+    a = gauss8(r, 60, (150, cols))
+    b = gauss8(r, 60, (150, cols))
+    gamma, beta = ln_params(r, cols)
+    s, out = ops.add_layernorm(dev(a), dev(b), dev(gamma), dev(beta), 5, mode, return_sum=True)
+    es, eo = oracle.add_layernorm(a, b, gamma, beta, 5, mode, return_sum=True)
+    assert np.array_equal(host(s), es) and np.array_equal(host(out), eo), (cols, mode)
+    assert np.array_equal(host(ops.add_layernorm(dev(a), dev(b), dev(gamma), dev(beta), 5, mode)), eo)
+
+
 @pytest.mark.parametrize('cols', [64, 768, 1024, 100])
 def test_add_layernorm_fused(ops, oracle, cols):
     r = rng(cols + 7)
@@ -862,6 +889,25 @@ def test_softmax_exp_columns(ops, oracle, cols):
         assert np.array_equal(got, oracle.softmax_exp(x, kq)), (cols, kq)
     got16 = host(ops.softmax_exp(dev(x), 23, out_kind='int16'))
     assert np.array_equal(got16, oracle.softmax_exp(x, 23, out='int16'))
+
+
+@pytest.mark.parametrize('cols', [4112, 5120, 8192, 8208, 12288, 16384, 16400])
+def test_softmax_long_rows(ops, oracle, cols):
+    """Rows beyond 4096 columns: eight or sixteen chunks per lane, scores looked up once for the sum and once more for
+    the products; 16400 is past the row kernel. Both score forms, both output types, a clamping and a plain shift."""
+    r = rng(cols + 19)
+    x = gauss8(r, 30, (131, cols))
+    x[5] = -128
+    x[6, ::7] = 127
+    for kq, inv_shift in ((23, 15), (128, 15), (1, 12)):
+        got = host(ops.softmax_exp(dev(x), kq, inv_shift))
+        assert np.array_equal(got, oracle.softmax_exp(x, kq, inv_shift)), (cols, kq, inv_shift)
+    got16 = host(ops.softmax_exp(dev(x), 23, out_kind='int16'))
+    assert np.array_equal(got16, oracle.softmax_exp(x, 23, out='int16'))
+    B = 32767 // cols
+    if B >= 2:
+        got = host(ops.softmax_hccs(dev(x), B, 1, B - 1))
+        assert np.array_equal(got, oracle.softmax_hccs(x, B, 1, B - 1)), cols
 
 
 def test_softmax_exp_every_gap_and_kq(ops, oracle):
