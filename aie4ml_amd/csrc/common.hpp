@@ -211,6 +211,25 @@ __device__ __forceinline__ unsigned requant4_bytes(int a0, int a1, int a2, int a
     return packed;
 }
 
+// The same with the rounding bit's position, width and sign given at run time (|acc| + 2^s < 2^31, s <= 22).
+__device__ __forceinline__ unsigned requant4_bytes_rt(int a0, int a1, int a2, int a3, const ByteRequant& b) {
+    auto pre = [&](int acc) {
+        const int bit = static_cast<int>(__builtin_amdgcn_ubfe(static_cast<unsigned>(acc), b.fr.pos, b.fr.w));
+        return clamp_med3(acc + b.fr.c0 + __mul24(bit, b.fr.cx), b.lo_s, b.hi_s);
+    };
+    unsigned packed = 0;
+    shift_into_byte<0>(packed, pre(a0), b.fr.s);
+    shift_into_byte<1>(packed, pre(a1), b.fr.s);
+    shift_into_byte<2>(packed, pre(a2), b.fr.s);
+    shift_into_byte<3>(packed, pre(a3), b.fr.s);
+    return packed;
+}
+
+// Actual column (within a block of 32) whose weights the lanes j and j + 32 supply as row j of the MFMA's first operand:
+// accumulator register 4g + i of lane (m, half) is output column 8g + 4half + i of the block, and we want that to be
+// actual column 16half + 4g + i, so that a lane's 16 registers are 16 neighbouring bytes of its output row.
+__device__ __forceinline__ int direct_col_of_operand_row(int j) { return ((j >> 2) & 1) * 16 + (j >> 3) * 4 + (j & 3); }
+
 __device__ __forceinline__ int kind_lo(int kind) {
     return kind == A4G_I8 ? -128 : (kind == A4G_I16 ? -32768 : (kind == A4G_I32 ? INT32_MIN : 0));
 }

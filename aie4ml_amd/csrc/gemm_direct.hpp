@@ -66,11 +66,6 @@ __device__ __forceinline__ unsigned direct_requant4(int a0, int a1, int a2, int 
     return packed;
 }
 
-// Actual column (within a wave's 32) whose weights the lanes j and j + 32 supply as row j of the MFMA's first operand:
-// accumulator register 4g + i of lane (m, half) is output column 8g + 4half + i of the block, and we want that to be
-// actual column 16half + 4g + i, so that a lane's 16 registers are 16 neighbouring bytes of its output row.
-__device__ __forceinline__ int direct_col_of_operand_row(int j) { return ((j >> 2) & 1) * 16 + (j >> 3) * 4 + (j & 3); }
-
 // The general requantisation of the same four values: any shift, any start value (`add4` is added here, the accumulators
 // started from zero).
 __device__ __forceinline__ unsigned direct_requant4_general(int a0, int a1, int a2, int a3, const v4i& add4, const v4i& s4, const v4i& c04,

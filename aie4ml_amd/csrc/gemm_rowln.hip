@@ -55,21 +55,6 @@ struct RowLnArgs {
     LnFloat lf;
 };
 
-// Four accumulators -> four requantised bytes with the rounding bit's position, width and sign given at run time
-// (|acc| + 2^s < 2^31, s <= 22).
-__device__ __forceinline__ unsigned rowln_requant4(int a0, int a1, int a2, int a3, const ByteRequant& b) {
-    auto pre = [&](int acc) {
-        const int bit = static_cast<int>(__builtin_amdgcn_ubfe(static_cast<unsigned>(acc), b.fr.pos, b.fr.w));
-        return clamp_med3(acc + b.fr.c0 + __mul24(bit, b.fr.cx), b.lo_s, b.hi_s);
-    };
-    unsigned packed = 0;
-    shift_into_byte<0>(packed, pre(a0), b.fr.s);
-    shift_into_byte<1>(packed, pre(a1), b.fr.s);
-    shift_into_byte<2>(packed, pre(a2), b.fr.s);
-    shift_into_byte<3>(packed, pre(a3), b.fr.s);
-    return packed;
-}
-
 // FR: the float form of the normalisation (0 nearest even, 1 floor family, 2 ceil family), -1: integer form only.
 template <int RB, int FR>
 __global__ __launch_bounds__(RL_NT, 2) void gemm_rowln_kernel(RowLnArgs g) {
@@ -255,7 +240,7 @@ __global__ __launch_bounds__(RL_NT, 2) void gemm_rowln_kernel(RowLnArgs g) {
             for (int q = 0; q < 4; ++q) {
                 unsigned y;
                 if (quick) {
-                    y = rowln_requant4(acc[rb][j][q * 4], acc[rb][j][q * 4 + 1], acc[rb][j][q * 4 + 2], acc[rb][j][q * 4 + 3], g.dq);
+                    y = requant4_bytes_rt(acc[rb][j][q * 4], acc[rb][j][q * 4 + 1], acc[rb][j][q * 4 + 2], acc[rb][j][q * 4 + 3], g.dq);
                 } else {
                     int v[4];
 #pragma unroll

@@ -172,6 +172,228 @@ __global__ __launch_bounds__(256) void mlp_fused_kernel(MlpArgs a) {
     }
 }
 
+
+// =====================================================================================================
+// The same chain on the matrix units, for batches large enough to be bound by arithmetic.
+// =====================================================================================================
+// A wave owns 32 samples at a time. Layer l computes, per block of 32 neurons, one 32x32x32 MFMA per 32 inputs with the
+// weights as the first operand and the activations as the second: lane (m, half) supplies bytes [16 half, 16 half + 16)
+// of sample m's 32 inputs, and receives 16 accumulators of sample m. The weight rows are handed over in the order
+// direct_col_of_operand_row, which makes those 16 accumulators the neurons 32 nb + 16 half + 0..15 - requantised and
+// packed they are exactly the lane's operand bytes for K step nb of the next layer, so the activations of a sample never
+// leave the lane's registers between the first load and the last store. Weight fragments (1 KiB per 32 neurons x 32
+// inputs, zero padded) and the accumulators' start values (bias + 128 * column sum for uint8 inputs) are staged in LDS
+// once per workgroup.
+struct MlpMfmaLayer {
+    const int8_t* wt;
+    const int32_t* colsum;
+    const int32_t* bias;
+    int ldwt, K, N;
+    int Kb, Nb;   // blocks of 32 inputs / neurons
+    int frag0;    // first fragment of the layer in LDS
+    int start0;   // first start value of the layer (int32 index)
+    int in_unsigned, out_kind;
+    int quick;    // the shift allows the requantisation that clamps in front of the shift
+    int fold;     // its rounding constant, added to the start values once instead of to every accumulator
+    int lo, hi;
+    ByteRequant dq;
+    RoundCfg drc;
+};
+
+struct MlpMfmaArgs {
+    MlpMfmaLayer layer[MLP_MAX_LAYERS];
+    int n_layers;
+    const int8_t* X;
+    void* Y;
+    int ldx, ldy;
+    int batch;
+    int x_bytes;      // bytes of X the launch may read
+    int nfrag, nstart;
+    int y_vec;        // rows of Y can be stored as 16-byte pieces
+};
+
+constexpr int64_t MLP_MFMA_MIN_BATCH = 4096;
+
+// MAXB: blocks of 32 that the widest layer has (2, 4 or 8: the loops over blocks are unrolled that far and guarded).
+// BIT: what the rounding mode adds besides its constant (fast_round_kind: 0 nothing, 1 a bit of the accumulator,
+// 2 minus that bit).
+template <int MAXB, int BIT>
+__global__ __launch_bounds__(1024) void mlp_mfma_kernel(MlpMfmaArgs a) {
+    constexpr int MLP_MFMA_BLOCKS = MAXB;
+    extern __shared__ __attribute__((aligned(16))) int8_t smem[];
+    int8_t* const frag = smem;
+    int* const start = reinterpret_cast<int*>(smem + a.nfrag * 1024);
+    int* const big = start + a.nstart;  // per layer: a start value too large for the quick requantisation
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int m = lane & 31, half = lane >> 5;
+    const int nthreads = blockDim.x;  // four to sixteen waves: as many as it takes to have sixteen on the CU
+    int8_t* const zero_frag = frag + (a.nfrag - 1) * 1024;  // the last fragment is all zeros
+
+    if (tid < MLP_MAX_LAYERS) big[tid] = 0;
+    if (tid < 64) *reinterpret_cast<v4i*>(zero_frag + tid * 16) = v4i{0, 0, 0, 0};
+    __syncthreads();
+    for (int l = 0; l < a.n_layers; ++l) {
+        const MlpMfmaLayer& L = a.layer[l];
+        const int pieces = L.Nb * L.Kb * 64;
+        for (int p = tid; p < pieces; p += nthreads) {
+            const int f = p >> 6, ln = p & 63;
+            const int nb = f / L.Kb, ks = f - nb * L.Kb;
+            const int col = nb * 32 + direct_col_of_operand_row(ln & 31);
+            const int k0 = ks * 32 + (ln >> 5) * 16;
+            v4i w = {0, 0, 0, 0};
+            if (col < L.N && k0 < L.K) {
+                w = *reinterpret_cast<const v4i*>(L.wt + static_cast<int64_t>(col) * L.ldwt + k0);  // ldwt % 16 == 0
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {  // inputs past K count nothing, whatever the packed rows hold there
+                    const int left = L.K - (k0 + 4 * q);
+                    if (left <= 0) w[q] = 0;
+                    else if (left < 4) w[q] &= static_cast<int>((1u << (8 * left)) - 1u);
+                }
+            }
+            *reinterpret_cast<v4i*>(frag + (L.frag0 + f) * 1024 + ln * 16) = w;
+        }
+        for (int c = tid; c < L.Nb * 32; c += nthreads) {
+            unsigned sv = 0;  // wraps like the int32 sum it stands for
+            if (c < L.N) {
+                if (L.bias) sv = static_cast<unsigned>(L.bias[c]);
+                if (L.in_unsigned) sv += 128u * static_cast<unsigned>(L.colsum[c]);
+            }
+            const int sval = static_cast<int>(sv);
+            start[L.start0 + c] = static_cast<int>(sv + static_cast<unsigned>(L.fold));
+            if (sval > (1 << 30) || sval < -(1 << 30)) big[l] = 1;  // every writer writes the same value
+        }
+    }
+    __syncthreads();
+
+    const auto rsrc_x = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.X), 0, a.x_bytes, 0x00020000);
+    const int units = (a.batch + 31) >> 5;
+    const int wpb = nthreads >> 6;
+    const int nwaves = gridDim.x * wpb;
+    const int Kb0 = a.layer[0].Kb;
+    const int xm0 = a.layer[0].in_unsigned ? static_cast<int>(0x80808080u) : 0;
+    for (int u = blockIdx.x * wpb + __builtin_amdgcn_readfirstlane(tid >> 6); u < units; u += nwaves) {
+        const int row = u * 32 + m;
+        const bool row_ok = row < a.batch;
+        v4i act[MLP_MFMA_BLOCKS];
+#pragma unroll
+        for (int ks = 0; ks < MLP_MFMA_BLOCKS; ++ks) {
+            act[ks] = v4i{0, 0, 0, 0};
+            // bytes past the row's end meet zero weights; a piece past the end of X reads as zero
+            if (ks < Kb0)
+                act[ks] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(
+                                                      rsrc_x, row_ok ? row * a.ldx + ks * 32 + half * 16 : 0x7ffffff0, 0, 0)) ^ xm0;
+        }
+        for (int l = 0; l < a.n_layers; ++l) {
+            const MlpMfmaLayer& L = a.layer[l];
+            const bool last = l + 1 == a.n_layers;
+            // The layer's constants live in the kernel's argument block, indexed by l: each is fetched once per layer and
+            // pinned to a scalar register here (an empty asm that claims to modify it), or the compiler fetches it again
+            // in every branch that uses it, with a wait each time.
+            int Kb = L.Kb, Nb = L.Nb, frag0 = L.frag0, start0 = L.start0, width = L.N, okind = L.out_kind;
+            int q_s = L.dq.fr.s, q_c0 = L.dq.fr.c0, q_pos = L.dq.fr.pos, q_lo = L.dq.lo_s, q_hi = L.dq.hi_s;
+            int quick_l = L.quick;
+            asm volatile("" : "+s"(Kb), "+s"(Nb), "+s"(frag0), "+s"(start0), "+s"(width), "+s"(okind), "+s"(quick_l));
+            asm volatile("" : "+s"(q_s), "+s"(q_c0), "+s"(q_pos), "+s"(q_lo), "+s"(q_hi));
+            ByteRequant dq;
+            dq.fr = FastRound{q_s, q_c0, q_pos, 1, 0};
+            dq.lo_s = q_lo;
+            dq.hi_s = q_hi;
+            const bool quick = quick_l != 0 && __builtin_amdgcn_readfirstlane(big[l]) == 0;
+            v4i out[MLP_MFMA_BLOCKS];
+#pragma unroll
+            for (int nb = 0; nb < MLP_MFMA_BLOCKS; ++nb) {
+                out[nb] = v4i{0, 0, 0, 0};
+                if (nb >= Nb) continue;
+                v16i acc;
+                {
+                    const int* sp = start + start0 + nb * 32 + 16 * half;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const v4i s4 = *reinterpret_cast<const v4i*>(sp + 4 * q);
+#pragma unroll
+                        for (int t = 0; t < 4; ++t) acc[4 * q + t] = s4[t];
+                    }
+                }
+                // All MAXB fragments are requested before the first product, an absent one as the fragment of zeros (no
+                // branch between the loads: the compiler keeps them all in flight), and the products go to two
+                // accumulators in turn, which halves the chain of dependent MFMAs.
+                const int8_t* fp = frag + (frag0 + nb * Kb) * 1024 + lane * 16;
+                v4i wf[MLP_MFMA_BLOCKS];
+#pragma unroll
+                for (int ks = 0; ks < MLP_MFMA_BLOCKS; ++ks)
+                    wf[ks] = *reinterpret_cast<const v4i*>(ks < Kb ? fp + ks * 1024 : zero_frag + lane * 16);
+                v16i acc1 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+                for (int ks = 0; ks < MLP_MFMA_BLOCKS; ++ks) {
+                    if (ks & 1) acc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[ks], act[ks], acc1, 0, 0, 0);
+                    else acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[ks], act[ks], acc, 0, 0, 0);
+                }
+                if (MLP_MFMA_BLOCKS > 1) acc += acc1;
+                const int col0 = nb * 32 + 16 * half;
+                if (last && okind == A4G_I16) {
+                    int16_t* y = static_cast<int16_t*>(a.Y) + static_cast<int64_t>(row) * a.ldy;
+#pragma unroll
+                    for (int t = 0; t < 16; ++t)
+                        if (row_ok && col0 + t < width) y[col0 + t] = static_cast<int16_t>(clamp_i(apply_round(acc[t] - L.fold, L.drc), L.lo, L.hi));
+                    continue;
+                }
+                v4i o;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    if (quick) {
+                        if (BIT == 0) {  // the rounding constant is in the start value already: clamp, shift into place
+                            unsigned packed = 0;
+                            shift_into_byte<0>(packed, clamp_med3(acc[4 * q], dq.lo_s, dq.hi_s), dq.fr.s);
+                            shift_into_byte<1>(packed, clamp_med3(acc[4 * q + 1], dq.lo_s, dq.hi_s), dq.fr.s);
+                            shift_into_byte<2>(packed, clamp_med3(acc[4 * q + 2], dq.lo_s, dq.hi_s), dq.fr.s);
+                            shift_into_byte<3>(packed, clamp_med3(acc[4 * q + 3], dq.lo_s, dq.hi_s), dq.fr.s);
+                            o[q] = static_cast<int>(packed);
+                        } else {
+                            o[q] = static_cast<int>(requant4_bytes<BIT>(acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3], dq));
+                        }
+                    } else {
+                        int v[4];
+#pragma unroll
+                        for (int t = 0; t < 4; ++t)  // the folded constant is taken out again (wrapping, like the sum itself)
+                            v[t] = clamp_i(apply_round(static_cast<int>(static_cast<unsigned>(acc[4 * q + t]) - static_cast<unsigned>(L.fold)), L.drc), L.lo, L.hi);
+                        o[q] = static_cast<int>(pack4_bytes(v[0], v[1], v[2], v[3]));
+                    }
+                }
+                if (!last) {
+                    // neurons past N have zero weights and a zero start value: they requantise to zero, and meet zero
+                    // weights in the next layer; a uint8 result is biased to int8 for the next MFMA
+                    out[nb] = okind == A4G_U8 ? o ^ static_cast<int>(0x80808080u) : o;
+                } else if (row_ok) {
+                    int8_t* y = static_cast<int8_t*>(a.Y) + static_cast<int64_t>(row) * a.ldy;
+                    if (a.y_vec) {
+                        if (col0 < width) *reinterpret_cast<v4i*>(y + col0) = o;  // N % 16 == 0
+                    } else {
+#pragma unroll
+                        for (int t = 0; t < 16; ++t)
+                            if (col0 + t < width) y[col0 + t] = static_cast<int8_t>(static_cast<unsigned>(o[t >> 2]) >> (8 * (t & 3)));
+                    }
+                }
+            }
+#pragma unroll
+            for (int nb = 0; nb < MLP_MFMA_BLOCKS; ++nb) act[nb] = out[nb];
+        }
+    }
+}
+
+template <int MAXB, int BIT>
+static hipError_t launch_mlp_mfma(int grid, int threads, size_t lds, hipStream_t stream, const MlpMfmaArgs& f) {
+    auto kern = mlp_mfma_kernel<MAXB, BIT>;
+    static bool attr_set = false;  // benign race: the attribute is idempotent
+    if (!attr_set) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                 128 * 1024);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    kern<<<grid, threads, lds, stream>>>(f);
+    return hipGetLastError();
+}
+
 }  // namespace a4g
 
 using namespace a4g;
@@ -243,6 +465,83 @@ extern "C" int a4g_mlp_i8(const a4g_mlp_layer* layers, int n_layers, const void*
     a.weight_bytes = (off + 15) / 16 * 16;
 
     a.total_chunks = weights_only / 16;
+
+    // Large batches: the chain on the matrix units, if its fragments fit the LDS and the rows can be fetched in 16-byte
+    // pieces. (Small batches are a chain of latencies either way, and the kernel below spreads 16 samples per workgroup.)
+    {
+        MlpMfmaArgs f{};
+        int nfrag = 0, nstart = 0, in_u = x_kind == A4G_U8;
+        bool ok = batch >= MLP_MFMA_MIN_BATCH && ldx % 16 == 0 && aligned16(X) && ldx <= INT32_MAX && ldy <= INT32_MAX &&
+                  (batch - 1) * ldx + layers[0].K < (int64_t{1} << 31) - 64;
+        const FastRound fr1 = make_fast_round(round_mode, 1);  // the kind of bit is the same for every shift >= 1
+        for (int l = 0; l < n_layers && ok; ++l) {
+            const a4g_mlp_layer& s = layers[l];
+            MlpMfmaLayer& d = f.layer[l];
+            d.wt = s.wt;
+            d.colsum = s.colsum;
+            d.bias = s.bias;
+            d.ldwt = static_cast<int>(s.ldwt);
+            d.K = s.K;
+            d.N = s.N;
+            d.Kb = (s.K + 31) / 32;
+            d.Nb = (s.N + 31) / 32;
+            d.frag0 = nfrag;
+            d.start0 = nstart;
+            d.in_unsigned = in_u;
+            d.out_kind = s.out_kind;
+            const int klo = s.out_kind == A4G_I8 ? -128 : (s.out_kind == A4G_I16 ? -32768 : 0);
+            d.lo = s.relu ? std::max(klo, 0) : klo;
+            d.hi = s.out_kind == A4G_I8 ? 127 : (s.out_kind == A4G_I16 ? 32767 : 255);
+            const FastRound fr = make_fast_round(round_mode, s.shift);
+            // |sum| <= 256 * 2^14: no overflow below 2^30 + 2^23; a shift of 0 rounds nothing, which the kernels that add
+            // a bit of the accumulator do not know
+            d.quick = byte_requant_ok(fr) && s.out_kind != A4G_I16 && (s.shift >= 1 || fast_round_kind(fr1) == 0);
+            // modes that add a bit of the accumulator (its sign, or the parity of the quotient) need the accumulator as it
+            // is: only the others fold their constant into the start values
+            d.fold = d.quick && fast_round_kind(fr1) == 0 ? fr.c0 : 0;
+            d.dq = make_byte_requant(fr, d.lo, d.hi);
+            d.drc = make_round(round_mode, s.shift);
+            nfrag += d.Nb * d.Kb;
+            nstart += d.Nb * 32;
+            in_u = s.out_kind == A4G_U8;
+        }
+        nfrag += 1;  // the fragment of zeros that absent K steps read
+        const size_t lds_f = static_cast<size_t>(nfrag) * 1024 + static_cast<size_t>(nstart) * 4 + MLP_MAX_LAYERS * 4;
+        if (ok && lds_f <= 128 * 1024) {
+            const a4g_mlp_layer& lastl = layers[n_layers - 1];
+            f.n_layers = n_layers;
+            f.X = static_cast<const int8_t*>(X);
+            f.Y = Y;
+            f.ldx = static_cast<int>(ldx);
+            f.ldy = static_cast<int>(ldy);
+            f.batch = static_cast<int>(batch);
+            f.x_bytes = static_cast<int>((batch - 1) * ldx + layers[0].K);
+            f.nfrag = nfrag;
+            f.nstart = nstart;
+            f.y_vec = lastl.out_kind != A4G_I16 && lastl.N % 16 == 0 && ldy % 16 == 0 && aligned16(Y);
+            int widest = 0;
+            for (int l = 0; l < n_layers; ++l) widest = std::max(widest, std::max(f.layer[l].Kb, f.layer[l].Nb));
+            const int bit_kind = fast_round_kind(fr1);
+            // sixteen waves per CU (32 samples per wave and turn): four workgroups of four waves where the LDS holds four
+            // copies of the fragments, fewer and larger workgroups otherwise
+            const int per_cu = static_cast<int>(std::max<size_t>(1, std::min<size_t>(4, (160 * 1024) / lds_f)));
+            const int threads = per_cu >= 4 ? 256 : (per_cu >= 2 ? 512 : 1024);
+            const int64_t wanted = (batch + (threads / 2) - 1) / (threads / 2);
+            const int grid_f = static_cast<int>(std::min<int64_t>(wanted, 256 * per_cu));
+            hipError_t e = hipErrorInvalidValue;
+#define A4G_MLP_GO(MAXB, BIT) e = launch_mlp_mfma<MAXB, BIT>(grid_f, threads, lds_f, stream, f)
+#define A4G_MLP_BITS(MAXB)                                                  \
+    if (bit_kind == 0) A4G_MLP_GO(MAXB, 0);                                  \
+    else if (bit_kind == 1) A4G_MLP_GO(MAXB, 1);                             \
+    else A4G_MLP_GO(MAXB, 2)
+            if (widest <= 2) { A4G_MLP_BITS(2); }
+            else if (widest <= 4) { A4G_MLP_BITS(4); }
+            else { A4G_MLP_BITS(8); }
+#undef A4G_MLP_BITS
+#undef A4G_MLP_GO
+            return check_hip(e, who);
+        }
+    }
 
     static bool attr_set = false;
     if (!attr_set) {

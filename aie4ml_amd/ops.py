@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import ctypes
 from dataclasses import dataclass
-from typing import List, Optional, Sequence
+from typing import Tuple, List, Optional, Sequence
 
 import torch
 
@@ -383,9 +383,21 @@ class MlpLayerSpec:
     out_kind: str = 'int8'
 
 
+def mlp_runs_on_matrix_units(rows: int, x_pitch: int, layers: Sequence[Tuple[int, int]]) -> bool:
+    """Whether a4g_mlp_i8 takes its large-batch form for this chain (``layers``: (K, N) per layer; ``x_pitch``: bytes
+    between input rows): from 4096 rows, rows fetched in 16-byte pieces, weight fragments of 1 KiB per 32 x 32 block
+    plus 128 bytes of start values per 32 neurons within 128 KiB of LDS."""
+    blocks = sum(((k + 31) // 32) * ((n + 31) // 32) for k, n in layers) + 1
+    start = sum((n + 31) // 32 * 32 for _k, n in layers)
+    return rows >= 4096 and x_pitch % 16 == 0 and blocks * 1024 + start * 4 + 32 <= 128 * 1024
+
+
 def mlp(x: torch.Tensor, layers: Sequence[MlpLayerSpec], rounding='floor', out: Optional[torch.Tensor] = None):
-    """Whole MLP in one launch (weights resident in LDS). x: [batch, K0] int8/uint8."""
-    x2 = _rows2d(x, 'x').contiguous()
+    """Whole MLP in one launch (weights resident in LDS). x: [batch, K0] int8/uint8; rows of a wider matrix are taken
+    where they lie."""
+    x2 = _rows2d(x, 'x')
+    if x2.stride(1) != 1 or (x2.shape[0] > 1 and x2.stride(0) < x2.shape[1]):
+        x2 = x2.contiguous()
     n = len(layers)
     arr = (MlpLayer * max(n, 1))()
     keep: List[torch.Tensor] = []

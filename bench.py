@@ -10,7 +10,7 @@ The default run also times, after the headline workload, the matrix-core calibra
 `frac_of_calibrated`, the clock under matrix load) and every other baseline configuration with the same method
 (`workloads`: value, ms_per_step, bit_exact, roofline per configuration; no CPU leg). `--only` skips both.
 
-Other workloads (--workload c2_dense_i16 | c2_dense_i16x16 | c2_dense_bf16 | c2_dense_fp8 | c1_mlp | c3_softmax_exp | c3_softmax_hccs | c3_qk | c3_pv |
+Other workloads (--workload c2_dense_i16 | c2_dense_i16x16 | c2_dense_bf16 | c2_dense_fp8 | c1_mlp | c1_mlp_stream | c3_softmax_exp | c3_softmax_hccs | c3_qk | c3_pv |
 c3_attention_exp | c3_attention_hccs | c4_add_layernorm | c4_layernorm | c4_add | c5_encoder) print the same line for that operator or graph;
 --workload calib_copy runs a plain 256 MiB elementwise copy, the known-size kernel the HBM traffic
 counters are scaled against; --workload calib_mfma runs the register-resident int8 MFMA loop alone.
@@ -294,6 +294,30 @@ def prepare(wl, torch):
         cpu_work = work
         metric, unit = 'int8_mlp_samples_per_s', 'samples/s'
         kernel = 'mlp_fused_kernel'
+    elif wl == 'c1_mlp_stream':
+        # the same network on a stream of samples: what a trigger or a tagging farm asks of it (throughput, not latency)
+        nb = 1 << 20
+        x, layers = workloads.c1_mlp(nb)
+        specs = [ops.MlpLayerSpec(ops.pack_dense(dev(Wl), dev(b), s), s, relu, o) for (Wl, b, s, relu, o) in layers]
+        dx = dev(x)
+        out = torch.empty((nb, 5), dtype=torch.int8, device='cuda')
+        fn = lambda: ops.mlp(dx, specs, 'positive_inf', out=out)  # noqa: E731
+        fn()
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+        sl = slice(0, 65536)
+        bit_exact = bool(np.array_equal(got[sl], oracle.mlp(x[sl], layers, 'positive_inf'))
+                         and np.array_equal(got[-4099:], oracle.mlp(x[-4099:], layers, 'positive_inf')))
+        work, bound = 21.0 * nb, 'hbm'  # 16 bytes in, 5 out per sample
+        samples = nb
+        config = {'workload': 'c1_mlp_stream: int8 MLP 16-64-32-32-5, batch 1048576, shift 7, round half up, fused single '
+                              'launch on the matrix units'}
+        cpu_desc = 'oracle MLP (layer by layer) on 65536 samples'
+        cpu_fn = lambda: oracle.mlp(x[sl], layers, 'positive_inf')  # noqa: E731
+        cpu_work = 21.0 * 65536
+        cpu_samples = 65536
+        metric, unit = 'int8_mlp_samples_per_s', 'samples/s'
+        kernel = 'mlp_mfma_kernel'
     elif wl in ('c4_add_layernorm', 'c4_layernorm', 'c4_add'):
         rows, cols = 16384, 1024
         a, b, gamma, beta, prm = workloads.c4_add_layernorm(rows, cols)
@@ -520,7 +544,7 @@ def calibrate_mfma(torch, blocks_per_cu=2, iters=4096):
 
 
 # the other configurations, timed in the default run after the headline workload (same steps, no CPU leg)
-ALSO = ('c1_mlp', 'c3_qk', 'c3_softmax_exp', 'c3_softmax_hccs', 'c3_pv', 'c3_attention_exp', 'c4_add', 'c4_layernorm',
+ALSO = ('c1_mlp', 'c1_mlp_stream', 'c3_qk', 'c3_softmax_exp', 'c3_softmax_hccs', 'c3_pv', 'c3_attention_exp', 'c4_add', 'c4_layernorm',
         'c4_add_layernorm', 'c5_encoder', 'c5_proj_qkv', 'c5_proj_out', 'c5_ffn_up', 'c5_ffn_down', 'c5_proj_out_ln')
 
 

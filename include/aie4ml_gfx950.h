@@ -228,7 +228,11 @@ A4G_API int a4g_softmax_hccs_i8(const int8_t* x, void* out, int64_t rows, int64_
  * dense_bias_relu_graph instances the reference wires for an hls4ml MLP
  * (templates/nnet_utils/dense_bias_relu/dense_bias_relu_graph.h:12-134).
  * `layers` is a HOST array. Limits: n_layers <= 8, every K and N <= 256, packed weights <= 96 KiB in
- * total; beyond them the call returns A4G_ERR_UNSUPPORTED and the caller runs layer by layer. */
+ * total; beyond them the call returns A4G_ERR_UNSUPPORTED and the caller runs layer by layer.
+ * Two forms behind the one call, the same integers from both: batches below 4096 samples (a chain of
+ * latencies) take dot-product instructions on 16 or 64 samples per workgroup; from 4096 samples, with ldx
+ * and X multiples of 16 bytes, the chain runs on the matrix units, 32 samples per wave, the activations in
+ * registers from the first layer to the last. */
 typedef struct a4g_mlp_layer {
     const int8_t* wt;      /* packed weights (a4g_pack_weights_i8), pitch ldwt */
     int64_t ldwt;

@@ -77,6 +77,30 @@ def test_wide_mlp_on_a_large_batch_runs_layer_by_layer(oracle):
         _graph_check(model, oracle, {'x': x})
 
 
+def test_wide_mlp_with_aligned_rows_on_a_large_batch_stays_fused(oracle):
+    """The same widths behind 64 inputs (rows that can be fetched in 16-byte pieces): from 4096 samples the fused launch
+    runs on the matrix units and the executor keeps it, whatever the per-layer model says."""
+    import torch
+
+    r = np.random.default_rng(33)
+    dims = [64, 200, 200, 200, 3]
+    batch = 8192 + 40
+    gb = GraphBuilder()
+    t = gb.input('x', (batch, dims[0]), qint(8, 4))
+    for i in range(4):
+        W = r.integers(-100, 100, (dims[i], dims[i + 1])) / 128.0
+        b = r.integers(-512, 512, dims[i + 1]) / 2048.0
+        t = gb.dense(t, W, qint(8, 7), qint(8, 4), bias=b, bias_precision=qint(32, 11), relu=i < 3, name=f'fc{i}')
+    gb.output(t)
+    model = gb.build()
+    model.compile()
+    x = np.clip(np.rint(r.normal(0, 30, (batch, dims[0]))), -128, 127).astype(np.int8)
+    trace = []
+    model.execute({'x': torch.from_numpy(x).cuda()}, trace=trace)
+    assert [t['kind'] for t in trace] == ['mlp']
+    _graph_check(model, oracle, {'x': x})
+
+
 def test_iteration_axis_folds_into_batch(oracle):
     model, x, layers = workloads.c1_mlp_model(batch=64)
     xs = np.stack([x, x[::-1], x])                      # (iterations, batch, features)

@@ -1031,6 +1031,66 @@ def test_mlp_unsigned_hidden_activations_and_odd_widths(ops, oracle):
     assert np.array_equal(got, oracle.mlp(x, layers_np, 'conv_even'))
 
 
+def make_mlp_general(ops, r, widths, shifts, relus, outs, bias_span=4096, wmax=64):
+    layers_np, specs = [], []
+    for (k, n), sh, relu, out in zip(zip(widths[:-1], widths[1:]), shifts, relus, outs):
+        W = r.integers(-wmax, wmax, (k, n)).astype(np.int8)
+        b = r.integers(-bias_span, bias_span + 1, n).astype(np.int32)
+        layers_np.append((W, b, sh, relu, out))
+        specs.append(ops.MlpLayerSpec(ops.pack_dense(dev(W), dev(b), sh), sh, relu, out))
+    return layers_np, specs
+
+
+@pytest.mark.parametrize('mode', MODES)
+def test_mlp_large_batch_every_rounding_mode(ops, oracle, mode):
+    """Batches from 4096 samples run the chain on the matrix units (activations stay in registers from layer to layer):
+    the C1 widths, a batch that is not a multiple of 32, every rounding mode."""
+    r = rng(31)
+    x = r.integers(-128, 128, (4096 + 77, 16)).astype(np.int8)
+    layers_np, specs = make_mlp(ops, r, [16, 64, 32, 32, 5])
+    assert np.array_equal(host(ops.mlp(dev(x), specs, mode)), oracle.mlp(x, layers_np, mode)), mode
+
+
+@pytest.mark.parametrize('case', [
+    dict(widths=[16, 64, 32, 32, 5], shifts=[7, 0, 15, 3], relus=[1, 1, 0, 0], outs=['int8', 'uint8', 'int8', 'int8']),
+    dict(widths=[32, 256, 256, 16], shifts=[9, 10, 8], relus=[1, 1, 0], outs=['uint8', 'uint8', 'int8']),
+    dict(widths=[48, 50, 7, 200, 3], shifts=[6, 5, 4, 7], relus=[1, 0, 1, 0], outs=['uint8', 'int8', 'uint8', 'int8']),
+    dict(widths=[64, 33, 5], shifts=[8, 20], relus=[0, 0], outs=['int8', 'int16']),
+    dict(widths=[16, 32], shifts=[24], relus=[1], outs=['uint8']),
+    dict(widths=[128, 96, 64], shifts=[12, 31], relus=[1, 0], outs=['int8', 'int8']),
+])
+@pytest.mark.parametrize('x_kind', ['int8', 'uint8'])
+def test_mlp_large_batch_shapes(ops, oracle, case, x_kind):
+    """Widths off the 32-grid (zero-padded fragments), uint8 inputs and hidden activations (biased to int8, corrected by
+    the column sums), a 16-bit last layer, shifts from 0 to 31 (the quick requantisation up to 22, the general one
+    above), outputs stored as 16-byte pieces (16 columns) and byte by byte (5, 3)."""
+    r = rng(len(case['widths']) * 100 + case['widths'][0])
+    k0 = case['widths'][0]
+    x = (r.integers(0, 256, (5000, k0)).astype(np.uint8) if x_kind == 'uint8' else r.integers(-128, 128, (5000, k0)).astype(np.int8))
+    layers_np, specs = make_mlp_general(ops, r, case['widths'], case['shifts'], case['relus'], case['outs'])
+    for mode in ('conv_even', 'symmetric_zero'):
+        assert np.array_equal(host(ops.mlp(dev(x), specs, mode)), oracle.mlp(x, layers_np, mode)), (case, mode)
+
+
+def test_mlp_large_batch_large_bias(ops, oracle):
+    """Biases next to the int32 limits: the quick requantisation (which adds its rounding constant to the accumulator)
+    would overflow, so the kernel notices them while staging and takes the general form."""
+    r = rng(41)
+    x = r.integers(-128, 128, (4500, 32)).astype(np.int8)
+    layers_np, specs = make_mlp_general(ops, r, [32, 64, 16], [9, 9], [1, 0], ['int8', 'int8'], bias_span=2**31 - 2**22)
+    assert np.array_equal(host(ops.mlp(dev(x), specs, 'conv_even')), oracle.mlp(x, layers_np, 'conv_even'))
+
+
+def test_mlp_large_batch_pitched_rows(ops, oracle):
+    """Rows of a wider matrix as input (pitch 64, 16 used) and a column window as output."""
+    r = rng(43)
+    wide = r.integers(-128, 128, (6000, 64)).astype(np.int8)
+    layers_np, specs = make_mlp(ops, r, [16, 64, 32, 32, 5])
+    dx = dev(wide)[:, :16]
+    got = ops.mlp(dx, specs, 'positive_inf')
+    assert np.array_equal(host(got), oracle.mlp(np.ascontiguousarray(wide[:, :16]), layers_np, 'positive_inf'))
+
+
 def test_mlp_limits(ops):
     r = rng(19)
     _, specs = make_mlp(ops, r, [16, 300, 4])
