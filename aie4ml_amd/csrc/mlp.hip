@@ -6,6 +6,8 @@
 // and four output neurons at a time; weights are read from LDS as (mostly) wave-uniform dwords,
 // activations as per-lane dwords from a padded LDS row, and four MACs retire per v_dot4_i32_i8.
 // uint8 activations are biased to int8 with x ^ 0x80 and corrected by 128 * colsum.
+#include <type_traits>
+
 #include "common.hpp"
 
 namespace a4g {
@@ -208,8 +210,10 @@ struct MlpMfmaArgs {
     int ldx, ldy;
     int batch;
     int x_bytes;      // bytes of X the launch may read
+    int y_bytes;      // bytes of Y it may write
     int nfrag, nstart;
     int y_vec;        // rows of Y can be stored as 16-byte pieces
+    int y_packed;     // at most 32 outputs in rows without gaps, Y 4-byte aligned: the tile store
 };
 
 constexpr int64_t MLP_MFMA_MIN_BATCH = 4096;
@@ -217,7 +221,8 @@ constexpr int64_t MLP_MFMA_MIN_BATCH = 4096;
 // MAXB: blocks of 32 that the widest layer has (2, 4 or 8: the loops over blocks are unrolled that far and guarded).
 // BIT: what the rounding mode adds besides its constant (fast_round_kind: 0 nothing, 1 a bit of the accumulator,
 // 2 minus that bit).
-template <int MAXB, int BIT>
+// YVEC: the result's rows can be stored as 16-byte pieces.
+template <int MAXB, int BIT, bool YVEC>
 __global__ __launch_bounds__(1024) void mlp_mfma_kernel(MlpMfmaArgs a) {
     constexpr int MLP_MFMA_BLOCKS = MAXB;
     extern __shared__ __attribute__((aligned(16))) int8_t smem[];
@@ -271,17 +276,55 @@ __global__ __launch_bounds__(1024) void mlp_mfma_kernel(MlpMfmaArgs a) {
     const int nwaves = gridDim.x * wpb;
     const int Kb0 = a.layer[0].Kb;
     const int xm0 = a.layer[0].in_unsigned ? static_cast<int>(0x80808080u) : 0;
-    for (int u = blockIdx.x * wpb + __builtin_amdgcn_readfirstlane(tid >> 6); u < units; u += nwaves) {
+    // A sample's input bytes, one 16-byte piece per 32 inputs and lane; a piece the first layer does not have, and a
+    // sample past the end of the batch, lie beyond the descriptor and read as zero, so that no load sits in a branch
+    // and all of a unit's pieces are in flight together. Bytes past the row's end meet zero weights.
+    const auto rsrc_y = __builtin_amdgcn_make_buffer_rsrc(static_cast<int8_t*>(a.Y), 0, a.y_bytes, 0x00020000);
+    const int last_n = a.layer[a.n_layers - 1].N;
+    // the packed store's tile, and where in it the four bytes of the lane's dwords come from (row * 32 + column of byte
+    // j = 4 * dword + b of the unit's 32 N bytes; three 10-bit addresses in one register, the fourth in another)
+    uint8_t* const tile = reinterpret_cast<uint8_t*>(big + MLP_MAX_LAYERS) + (tid >> 6) * 1024;
+    unsigned tsrc[4] = {0, 0, 0, 0}, tsrc2[4] = {0, 0, 0, 0};
+    if (!YVEC && a.y_packed) {
+#pragma unroll
+        for (int sl = 0; sl < 4; ++sl) {
+            unsigned at[4];
+#pragma unroll
+            for (int b = 0; b < 4; ++b) {
+                const int j = min((sl * 64 + lane) * 4 + b, 32 * last_n - 1);
+                const int r = j / last_n;
+                at[b] = static_cast<unsigned>(r * 32 + (j - r * last_n));
+            }
+            tsrc[sl] = at[0] | (at[1] << 10) | (at[2] << 20);
+            tsrc2[sl] = at[3];
+        }
+    }
+    // Narrow chains request the next unit's input before this unit's layers (and stores); the wide ones have no
+    // registers to spare for that (it cost them 10 %).
+    constexpr bool AHEAD = MAXB <= 2;
+    v4i nact[AHEAD ? MLP_MFMA_BLOCKS : 1];
+    auto fetch = [&](int unit, v4i* dst) {
+        const int r = unit * 32 + m;
+#pragma unroll
+        for (int ks = 0; ks < MLP_MFMA_BLOCKS; ++ks)
+            dst[ks] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(
+                                                  rsrc_x, (ks < Kb0 && r < a.batch) ? r * a.ldx + ks * 32 + half * 16 : 0x7ffffff0, 0, 0));
+    };
+    const int u0 = blockIdx.x * wpb + __builtin_amdgcn_readfirstlane(tid >> 6);
+    if (AHEAD) fetch(u0, nact);
+    for (int u = u0; u < units; u += nwaves) {
         const int row = u * 32 + m;
         const bool row_ok = row < a.batch;
         v4i act[MLP_MFMA_BLOCKS];
+        if (AHEAD) {
 #pragma unroll
-        for (int ks = 0; ks < MLP_MFMA_BLOCKS; ++ks) {
-            act[ks] = v4i{0, 0, 0, 0};
-            // bytes past the row's end meet zero weights; a piece past the end of X reads as zero
-            if (ks < Kb0)
-                act[ks] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(
-                                                      rsrc_x, row_ok ? row * a.ldx + ks * 32 + half * 16 : 0x7ffffff0, 0, 0)) ^ xm0;
+            for (int ks = 0; ks < MLP_MFMA_BLOCKS; ++ks) act[ks] = nact[ks] ^ xm0;
+            __builtin_amdgcn_sched_barrier(0);
+            fetch(u + nwaves, nact);  // past the end: zeros, unused
+        } else {
+            fetch(u, act);
+#pragma unroll
+            for (int ks = 0; ks < MLP_MFMA_BLOCKS; ++ks) act[ks] ^= xm0;
         }
         for (int l = 0; l < a.n_layers; ++l) {
             const MlpMfmaLayer& L = a.layer[l];
@@ -300,93 +343,136 @@ __global__ __launch_bounds__(1024) void mlp_mfma_kernel(MlpMfmaArgs a) {
             dq.hi_s = q_hi;
             const bool quick = quick_l != 0 && __builtin_amdgcn_readfirstlane(big[l]) == 0;
             v4i out[MLP_MFMA_BLOCKS];
+            // one copy of the layer per form of the requantisation: the choice is made once, not per group of four values
+            auto run_layer = [&](auto quick_tag) __attribute__((always_inline)) {
+                constexpr bool QUICK = decltype(quick_tag)::value;
 #pragma unroll
-            for (int nb = 0; nb < MLP_MFMA_BLOCKS; ++nb) {
-                out[nb] = v4i{0, 0, 0, 0};
-                if (nb >= Nb) continue;
-                v16i acc;
-                {
-                    const int* sp = start + start0 + nb * 32 + 16 * half;
+                for (int nb = 0; nb < MLP_MFMA_BLOCKS; ++nb) {
+                    out[nb] = v4i{0, 0, 0, 0};
+                    if (nb >= Nb) continue;
+                    v16i acc;
+                    {
+                        const int* sp = start + start0 + nb * 32 + 16 * half;
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) {
+                            const v4i s4 = *reinterpret_cast<const v4i*>(sp + 4 * q);
+#pragma unroll
+                            for (int t = 0; t < 4; ++t) acc[4 * q + t] = s4[t];
+                        }
+                    }
+                    // All MAXB fragments are requested before the first product, an absent one as the fragment of zeros (no
+                    // branch between the loads: the compiler keeps them all in flight), and from four K steps on the products
+                    // go to two accumulators in turn, which halves the chain of dependent MFMAs.
+                    const int8_t* fp = frag + (frag0 + nb * Kb) * 1024 + lane * 16;
+                    v4i wf[MLP_MFMA_BLOCKS];
+#pragma unroll
+                    for (int ks = 0; ks < MLP_MFMA_BLOCKS; ++ks)
+                        wf[ks] = *reinterpret_cast<const v4i*>(ks < Kb ? fp + ks * 1024 : zero_frag + lane * 16);
+                    if (MLP_MFMA_BLOCKS >= 4) {
+                        v16i acc1 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+                        for (int ks = 0; ks < MLP_MFMA_BLOCKS; ++ks) {
+                            if (ks & 1) acc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[ks], act[ks], acc1, 0, 0, 0);
+                            else acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[ks], act[ks], acc, 0, 0, 0);
+                        }
+                        acc += acc1;
+                    } else {
+#pragma unroll
+                        for (int ks = 0; ks < MLP_MFMA_BLOCKS; ++ks) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[ks], act[ks], acc, 0, 0, 0);
+                    }
+                    const int col0 = nb * 32 + 16 * half;
+                    if (QUICK && BIT == 0) {
+                        // This form's first readers of the accumulators are inline asm (v_med3), which the compiler's
+                        // hazard recogniser does not look into: it would insert no wait states between the MFMA and them.
+                        // One ordinary vector instruction reads the accumulator first (an identity DPP move, which gets
+                        // the wait states), and nothing is scheduled across the barrier behind it.
+                        acc[15] = __builtin_amdgcn_update_dpp(0, acc[15], 0xE4, 0xF, 0xF, false);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                    v4i o;
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
-                        const v4i s4 = *reinterpret_cast<const v4i*>(sp + 4 * q);
-#pragma unroll
-                        for (int t = 0; t < 4; ++t) acc[4 * q + t] = s4[t];
-                    }
-                }
-                // All MAXB fragments are requested before the first product, an absent one as the fragment of zeros (no
-                // branch between the loads: the compiler keeps them all in flight), and the products go to two
-                // accumulators in turn, which halves the chain of dependent MFMAs.
-                const int8_t* fp = frag + (frag0 + nb * Kb) * 1024 + lane * 16;
-                v4i wf[MLP_MFMA_BLOCKS];
-#pragma unroll
-                for (int ks = 0; ks < MLP_MFMA_BLOCKS; ++ks)
-                    wf[ks] = *reinterpret_cast<const v4i*>(ks < Kb ? fp + ks * 1024 : zero_frag + lane * 16);
-                v16i acc1 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-                for (int ks = 0; ks < MLP_MFMA_BLOCKS; ++ks) {
-                    if (ks & 1) acc1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[ks], act[ks], acc1, 0, 0, 0);
-                    else acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[ks], act[ks], acc, 0, 0, 0);
-                }
-                if (MLP_MFMA_BLOCKS > 1) acc += acc1;
-                const int col0 = nb * 32 + 16 * half;
-                if (last && okind == A4G_I16) {
-                    int16_t* y = static_cast<int16_t*>(a.Y) + static_cast<int64_t>(row) * a.ldy;
-#pragma unroll
-                    for (int t = 0; t < 16; ++t)
-                        if (row_ok && col0 + t < width) y[col0 + t] = static_cast<int16_t>(clamp_i(apply_round(acc[t] - L.fold, L.drc), L.lo, L.hi));
-                    continue;
-                }
-                v4i o;
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    if (quick) {
-                        if (BIT == 0) {  // the rounding constant is in the start value already: clamp, shift into place
-                            unsigned packed = 0;
-                            shift_into_byte<0>(packed, clamp_med3(acc[4 * q], dq.lo_s, dq.hi_s), dq.fr.s);
-                            shift_into_byte<1>(packed, clamp_med3(acc[4 * q + 1], dq.lo_s, dq.hi_s), dq.fr.s);
-                            shift_into_byte<2>(packed, clamp_med3(acc[4 * q + 2], dq.lo_s, dq.hi_s), dq.fr.s);
-                            shift_into_byte<3>(packed, clamp_med3(acc[4 * q + 3], dq.lo_s, dq.hi_s), dq.fr.s);
-                            o[q] = static_cast<int>(packed);
+                        if (QUICK) {
+                            if (BIT == 0) {  // the rounding constant is in the start value already: clamp, shift into place
+                                unsigned packed;  // byte 0 is written with the other bytes zeroed, bytes 1..3 are merged in
+                                {
+                                    const int v0 = clamp_med3(acc[4 * q], dq.lo_s, dq.hi_s);
+                                    asm("v_ashrrev_i32_sdwa %0, %1, %2 dst_sel:BYTE_0 dst_unused:UNUSED_PAD src0_sel:DWORD src1_sel:DWORD"
+                                        : "=v"(packed)
+                                        : "v"(dq.fr.s), "v"(v0));
+                                }
+                                shift_into_byte<1>(packed, clamp_med3(acc[4 * q + 1], dq.lo_s, dq.hi_s), dq.fr.s);
+                                shift_into_byte<2>(packed, clamp_med3(acc[4 * q + 2], dq.lo_s, dq.hi_s), dq.fr.s);
+                                shift_into_byte<3>(packed, clamp_med3(acc[4 * q + 3], dq.lo_s, dq.hi_s), dq.fr.s);
+                                o[q] = static_cast<int>(packed);
+                            } else {
+                                o[q] = static_cast<int>(requant4_bytes<BIT>(acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3], dq));
+                            }
                         } else {
-                            o[q] = static_cast<int>(requant4_bytes<BIT>(acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3], dq));
+                            int v[4];
+#pragma unroll
+                            for (int t = 0; t < 4; ++t)  // the folded constant is taken out again (wrapping, like the sum itself)
+                                v[t] = clamp_i(apply_round(static_cast<int>(static_cast<unsigned>(acc[4 * q + t]) - static_cast<unsigned>(L.fold)), L.drc), L.lo, L.hi);
+                            o[q] = static_cast<int>(pack4_bytes(v[0], v[1], v[2], v[3]));
                         }
-                    } else {
-                        int v[4];
-#pragma unroll
-                        for (int t = 0; t < 4; ++t)  // the folded constant is taken out again (wrapping, like the sum itself)
-                            v[t] = clamp_i(apply_round(static_cast<int>(static_cast<unsigned>(acc[4 * q + t]) - static_cast<unsigned>(L.fold)), L.drc), L.lo, L.hi);
-                        o[q] = static_cast<int>(pack4_bytes(v[0], v[1], v[2], v[3]));
                     }
+                    // neurons past N have zero weights and a zero start value: they requantise to zero, and meet zero weights
+                    // in the next layer; a uint8 result is biased to int8 for the next MFMA (the last layer's is kept as it is)
+                    out[nb] = (!last && okind == A4G_U8) ? o ^ static_cast<int>(0x80808080u) : o;
                 }
-                if (!last) {
-                    // neurons past N have zero weights and a zero start value: they requantise to zero, and meet zero
-                    // weights in the next layer; a uint8 result is biased to int8 for the next MFMA
-                    out[nb] = okind == A4G_U8 ? o ^ static_cast<int>(0x80808080u) : o;
-                } else if (row_ok) {
-                    int8_t* y = static_cast<int8_t*>(a.Y) + static_cast<int64_t>(row) * a.ldy;
-                    if (a.y_vec) {
-                        if (col0 < width) *reinterpret_cast<v4i*>(y + col0) = o;  // N % 16 == 0
-                    } else {
-#pragma unroll
-                        for (int t = 0; t < 16; ++t)
-                            if (col0 + t < width) y[col0 + t] = static_cast<int8_t>(static_cast<unsigned>(o[t >> 2]) >> (8 * (t & 3)));
-                    }
-                }
-            }
+            };
+            if (quick) run_layer(std::true_type{});
+            else run_layer(std::false_type{});
 #pragma unroll
             for (int nb = 0; nb < MLP_MFMA_BLOCKS; ++nb) act[nb] = out[nb];
+        }
+        // The last layer's bytes, stored outside the loop over the layers and without a branch: a byte (or 16-byte piece)
+        // that does not exist gets an offset past the descriptor and is dropped. The compiler then knows how many stores
+        // are in flight, and the wait for the next unit's input, requested before them, does not include their
+        // acknowledgement.
+        if (!YVEC && a.y_packed && u * 32 + 32 <= a.batch) {
+            // At most 32 neurons in rows that follow each other without a gap (a classifier's few outputs): the unit's
+            // 32 rows are 32 N consecutive bytes. They go through a 1 KiB tile of the wave's own (no barrier: a wave's
+            // LDS operations complete in order) and leave as whole dwords, instead of N byte stores per lane.
+            *reinterpret_cast<v4i*>(tile + m * 32 + 16 * half) = act[0];
+            const unsigned ubase = static_cast<unsigned>(u) * 32u * static_cast<unsigned>(last_n);
+#pragma unroll
+            for (int sl = 0; sl < 4; ++sl) {
+                if (sl * 256 < 32 * last_n) {
+                    const unsigned word = static_cast<unsigned>(tile[tsrc[sl] & 0x3ff]) | (static_cast<unsigned>(tile[(tsrc[sl] >> 10) & 0x3ff]) << 8) |
+                                          (static_cast<unsigned>(tile[(tsrc[sl] >> 20) & 0x3ff]) << 16) |
+                                          (static_cast<unsigned>(tile[tsrc2[sl]]) << 24);
+                    __builtin_amdgcn_raw_buffer_store_b32(word, rsrc_y, (sl * 64 + lane) * 4 < 32 * last_n ? ubase + (sl * 64 + lane) * 4 : 0x7ffffff0u, 0, 0);
+                }
+            }
+        } else {
+            typedef unsigned v4u __attribute__((ext_vector_type(4)));
+#pragma unroll
+            for (int nb = 0; nb < MLP_MFMA_BLOCKS; ++nb) {
+                const int col0 = nb * 32 + 16 * half;
+                if (nb * 32 >= last_n) continue;  // (uniform)
+                const unsigned y0 = static_cast<unsigned>(row) * static_cast<unsigned>(a.ldy) + col0;
+                if (YVEC) {  // N % 16 == 0, rows 16-byte aligned
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, act[nb]), rsrc_y,
+                                                           (row_ok && col0 < last_n) ? y0 : 0x7ffffff0u, 0, 0);
+                } else {
+#pragma unroll
+                    for (int t = 0; t < 16; ++t)
+                        __builtin_amdgcn_raw_buffer_store_b8(static_cast<unsigned char>(static_cast<unsigned>(act[nb][t >> 2]) >> (8 * (t & 3))),
+                                                             rsrc_y, (row_ok && col0 + t < last_n) ? y0 + t : 0x7ffffff0u, 0, 0);
+                }
+            }
         }
     }
 }
 
-template <int MAXB, int BIT>
+template <int MAXB, int BIT, bool YVEC>
 static hipError_t launch_mlp_mfma(int grid, int threads, size_t lds, hipStream_t stream, const MlpMfmaArgs& f) {
-    auto kern = mlp_mfma_kernel<MAXB, BIT>;
+    auto kern = mlp_mfma_kernel<MAXB, BIT, YVEC>;
     static bool attr_set = false;  // benign race: the attribute is idempotent
     if (!attr_set) {
         const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                 128 * 1024);
+                                                 144 * 1024);
         if (e != hipSuccess) return e;
         attr_set = true;
     }
@@ -471,8 +557,9 @@ extern "C" int a4g_mlp_i8(const a4g_mlp_layer* layers, int n_layers, const void*
     {
         MlpMfmaArgs f{};
         int nfrag = 0, nstart = 0, in_u = x_kind == A4G_U8;
-        bool ok = batch >= MLP_MFMA_MIN_BATCH && ldx % 16 == 0 && aligned16(X) && ldx <= INT32_MAX && ldy <= INT32_MAX &&
-                  (batch - 1) * ldx + layers[0].K < (int64_t{1} << 31) - 64;
+        bool ok = batch >= MLP_MFMA_MIN_BATCH && layers[n_layers - 1].out_kind != A4G_I16 && ldx % 16 == 0 && aligned16(X) && ldx <= INT32_MAX && ldy <= INT32_MAX &&
+                  (batch - 1) * ldx + layers[0].K < (int64_t{1} << 31) - 64 &&
+                  ((batch - 1) * ldy + layers[n_layers - 1].N) * 2 < (int64_t{1} << 31) - 64;
         const FastRound fr1 = make_fast_round(round_mode, 1);  // the kind of bit is the same for every shift >= 1
         for (int l = 0; l < n_layers && ok; ++l) {
             const a4g_mlp_layer& s = layers[l];
@@ -506,8 +593,9 @@ extern "C" int a4g_mlp_i8(const a4g_mlp_layer* layers, int n_layers, const void*
             in_u = s.out_kind == A4G_U8;
         }
         nfrag += 1;  // the fragment of zeros that absent K steps read
-        const size_t lds_f = static_cast<size_t>(nfrag) * 1024 + static_cast<size_t>(nstart) * 4 + MLP_MAX_LAYERS * 4;
-        if (ok && lds_f <= 128 * 1024) {
+        // fragments, start values, one flag per layer (and, below, a 1 KiB tile per wave for the packed store)
+        const size_t lds_core = static_cast<size_t>(nfrag) * 1024 + static_cast<size_t>(nstart) * 4 + MLP_MAX_LAYERS * 4;
+        if (ok && lds_core <= 128 * 1024) {
             const a4g_mlp_layer& lastl = layers[n_layers - 1];
             f.n_layers = n_layers;
             f.X = static_cast<const int8_t*>(X);
@@ -516,20 +604,26 @@ extern "C" int a4g_mlp_i8(const a4g_mlp_layer* layers, int n_layers, const void*
             f.ldy = static_cast<int>(ldy);
             f.batch = static_cast<int>(batch);
             f.x_bytes = static_cast<int>((batch - 1) * ldx + layers[0].K);
+            f.y_bytes = static_cast<int>(((batch - 1) * ldy + lastl.N) * (lastl.out_kind == A4G_I16 ? 2 : 1));
             f.nfrag = nfrag;
             f.nstart = nstart;
             f.y_vec = lastl.out_kind != A4G_I16 && lastl.N % 16 == 0 && ldy % 16 == 0 && aligned16(Y);
+            f.y_packed = !f.y_vec && lastl.N <= 32 && ldy == lastl.N && reinterpret_cast<uintptr_t>(Y) % 4 == 0;
             int widest = 0;
             for (int l = 0; l < n_layers; ++l) widest = std::max(widest, std::max(f.layer[l].Kb, f.layer[l].Nb));
             const int bit_kind = fast_round_kind(fr1);
             // sixteen waves per CU (32 samples per wave and turn): four workgroups of four waves where the LDS holds four
             // copies of the fragments, fewer and larger workgroups otherwise
-            const int per_cu = static_cast<int>(std::max<size_t>(1, std::min<size_t>(4, (160 * 1024) / lds_f)));
+            const size_t tile_bytes = f.y_packed ? 16 * 1024 : 0;  // per CU, however its sixteen waves are grouped
+            const int per_cu = static_cast<int>(std::max<size_t>(1, std::min<size_t>(4, (160 * 1024 - tile_bytes) / lds_core)));
             const int threads = per_cu >= 4 ? 256 : (per_cu >= 2 ? 512 : 1024);
+            const size_t lds_f = lds_core + (f.y_packed ? static_cast<size_t>(threads / 64) * 1024 : 0);
             const int64_t wanted = (batch + (threads / 2) - 1) / (threads / 2);
             const int grid_f = static_cast<int>(std::min<int64_t>(wanted, 256 * per_cu));
             hipError_t e = hipErrorInvalidValue;
-#define A4G_MLP_GO(MAXB, BIT) e = launch_mlp_mfma<MAXB, BIT>(grid_f, threads, lds_f, stream, f)
+#define A4G_MLP_GO(MAXB, BIT)                                                                    \
+    e = f.y_vec ? launch_mlp_mfma<MAXB, BIT, true>(grid_f, threads, lds_f, stream, f)             \
+                : launch_mlp_mfma<MAXB, BIT, false>(grid_f, threads, lds_f, stream, f)
 #define A4G_MLP_BITS(MAXB)                                                  \
     if (bit_kind == 0) A4G_MLP_GO(MAXB, 0);                                  \
     else if (bit_kind == 1) A4G_MLP_GO(MAXB, 1);                             \
