@@ -145,6 +145,9 @@ __device__ __forceinline__ int clamp_i(int v, int lo, int hi) { return min(max(v
 
 // clamp_i as one instruction for bounds that are only known at run time (callers guarantee lo <= hi,
 // which the compiler would have to prove before it forms the median by itself).
+// Not to be the first reader of an MFMA result: the compiler's hazard recogniser does not look into inline asm, so it
+// inserts no wait states between the MFMA and this instruction. Every caller either applies it to a sum formed by an
+// ordinary instruction, or reads the accumulator through one first (mlp_mfma_kernel).
 __device__ __forceinline__ int clamp_med3(int v, int lo, int hi) {
     int y;
     asm("v_med3_i32 %0, %1, %2, %3" : "=v"(y) : "v"(v), "v"(lo), "v"(hi));
