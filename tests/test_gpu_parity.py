@@ -142,6 +142,21 @@ def test_dense_shapes_mfma_path(ops, oracle, shape):
     run_dense(ops, oracle, M, K, N, 'conv_even', seed=M + K + N)
 
 
+@pytest.mark.parametrize('shape', [(5000, 16, 64), (4096, 64, 32), (4100, 32, 5), (6000, 48, 200), (4500, 192, 256),
+                                   (4097, 80, 33), (5000, 20, 64), (5000, 16, 300)])
+@pytest.mark.parametrize('mode', ['conv_even', 'positive_inf', 'symmetric_zero'])
+def test_dense_narrow_layer_on_a_long_batch(ops, oracle, shape, mode):
+    """Narrow layers with one shift on 4096 rows or more go to the kernel that walks a chain of layers (a chain of one):
+    signed and unsigned rows and results, with and without ReLU and bias; the last two shapes (rows of 20 bytes, 300
+    outputs) and per-channel shifts are outside it and take the GEMM kernels, with the same integers."""
+    M, K, N = shape
+    run_dense(ops, oracle, M, K, N, mode, per_channel=False, seed=M + K + N)
+    run_dense(ops, oracle, M, K, N, mode, a_dtype=np.uint8, relu=False, per_channel=False, out='uint8', seed=M + K + N + 1)
+    run_dense(ops, oracle, M, K, N, mode, relu=False, per_channel=False, bias=False, seed=M + K + N + 2)
+    run_dense(ops, oracle, M, K, N, mode, per_channel=True, seed=M + K + N + 3)
+    run_dense(ops, oracle, M, K, N, mode, per_channel=False, out='int16', seed=M + K + N + 4)
+
+
 @pytest.mark.parametrize('shape', [(5, 3, 2), (64, 17, 33), (9, 100, 12), (128, 250, 64)])
 def test_dense_ragged_k_generic_path(ops, oracle, shape):
     M, K, N = shape
