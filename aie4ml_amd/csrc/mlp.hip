@@ -209,7 +209,9 @@ struct MlpMfmaArgs {
     void* Y;
     int ldx, ldy;
     int batch;
-    int x_bytes;      // bytes of X the launch may read
+    int x_bytes;      // bytes the launch may read from X on
+    int x_aligned;    // rows start at multiples of 16 bytes
+    int x_delta;      // else: X points to the dword below the first row, which starts this many bytes in
     int y_bytes;      // bytes of Y it may write
     int nfrag, nstart;
     int y_vec;        // rows of Y can be stored as 16-byte pieces
@@ -305,10 +307,27 @@ __global__ __launch_bounds__(1024) void mlp_mfma_kernel(MlpMfmaArgs a) {
     v4i nact[AHEAD ? MLP_MFMA_BLOCKS : 1];
     auto fetch = [&](int unit, v4i* dst) {
         const int r = unit * 32 + m;
+        if (a.x_aligned) {
 #pragma unroll
-        for (int ks = 0; ks < MLP_MFMA_BLOCKS; ++ks)
-            dst[ks] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(
-                                                  rsrc_x, (ks < Kb0 && r < a.batch) ? r * a.ldx + ks * 32 + half * 16 : 0x7ffffff0, 0, 0));
+            for (int ks = 0; ks < MLP_MFMA_BLOCKS; ++ks)
+                dst[ks] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(
+                                                      rsrc_x, (ks < Kb0 && r < a.batch) ? r * a.ldx + ks * 32 + half * 16 : 0x7ffffff0, 0, 0));
+        } else {
+            // Rows at any address (57 inputs, a window of a wider matrix): the piece is cut out of the five dwords that
+            // cover it. The descriptor starts at the dword below X (x_delta bytes), so every load is dword-aligned.
+#pragma unroll
+            for (int ks = 0; ks < MLP_MFMA_BLOCKS; ++ks) {
+                const unsigned at = static_cast<unsigned>(r * a.ldx + ks * 32 + half * 16 + a.x_delta);
+                const bool there = ks < Kb0 && r < a.batch;
+                const unsigned sh = at & 3u;
+                const v4i w = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, there ? (at & ~3u) : 0x7ffffff0u, 0, 0));
+                const int w4 = static_cast<int>(__builtin_amdgcn_raw_buffer_load_b32(rsrc_x, there ? (at & ~3u) + 16u : 0x7ffffff0u, 0, 0));
+                dst[ks][0] = static_cast<int>(__builtin_amdgcn_alignbyte(w[1], w[0], sh));
+                dst[ks][1] = static_cast<int>(__builtin_amdgcn_alignbyte(w[2], w[1], sh));
+                dst[ks][2] = static_cast<int>(__builtin_amdgcn_alignbyte(w[3], w[2], sh));
+                dst[ks][3] = static_cast<int>(__builtin_amdgcn_alignbyte(w4, w[3], sh));
+            }
+        }
     };
     const int u0 = blockIdx.x * wpb + __builtin_amdgcn_readfirstlane(tid >> 6);
     if (AHEAD) fetch(u0, nact);
@@ -557,7 +576,7 @@ extern "C" int a4g_mlp_i8(const a4g_mlp_layer* layers, int n_layers, const void*
     {
         MlpMfmaArgs f{};
         int nfrag = 0, nstart = 0, in_u = x_kind == A4G_U8;
-        bool ok = batch >= MLP_MFMA_MIN_BATCH && layers[n_layers - 1].out_kind != A4G_I16 && ldx % 16 == 0 && aligned16(X) && ldx <= INT32_MAX && ldy <= INT32_MAX &&
+        bool ok = batch >= MLP_MFMA_MIN_BATCH && layers[n_layers - 1].out_kind != A4G_I16 && ldx <= INT32_MAX && ldy <= INT32_MAX &&
                   (batch - 1) * ldx + layers[0].K < (int64_t{1} << 31) - 64 &&
                   ((batch - 1) * ldy + layers[n_layers - 1].N) * 2 < (int64_t{1} << 31) - 64;
         const FastRound fr1 = make_fast_round(round_mode, 1);  // the kind of bit is the same for every shift >= 1
@@ -598,12 +617,16 @@ extern "C" int a4g_mlp_i8(const a4g_mlp_layer* layers, int n_layers, const void*
         if (ok && lds_core <= 128 * 1024) {
             const a4g_mlp_layer& lastl = layers[n_layers - 1];
             f.n_layers = n_layers;
-            f.X = static_cast<const int8_t*>(X);
+            f.x_aligned = ldx % 16 == 0 && aligned16(X);
+            f.x_delta = f.x_aligned ? 0 : static_cast<int>(reinterpret_cast<uintptr_t>(X) & 3);
+            f.X = static_cast<const int8_t*>(X) - f.x_delta;
             f.Y = Y;
             f.ldx = static_cast<int>(ldx);
             f.ldy = static_cast<int>(ldy);
             f.batch = static_cast<int>(batch);
-            f.x_bytes = static_cast<int>((batch - 1) * ldx + layers[0].K);
+            // up to the end of the dword that holds the last byte: the range check is per dword, and a dword that
+            // straddles the end of the descriptor would read as zero
+            f.x_bytes = (static_cast<int>((batch - 1) * ldx + layers[0].K) + f.x_delta + 3) & ~3;
             f.y_bytes = static_cast<int>(((batch - 1) * ldy + lastl.N) * (lastl.out_kind == A4G_I16 ? 2 : 1));
             f.nfrag = nfrag;
             f.nstart = nstart;

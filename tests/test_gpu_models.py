@@ -54,14 +54,15 @@ def test_mlp_graph_unfused_matches_fused(oracle):
     np.testing.assert_array_equal(fused, unfused)
 
 
-def test_wide_mlp_on_a_large_batch_runs_layer_by_layer(oracle):
-    """A fusable chain whose layers are wide and whose batch is large is planned as a chain but executed as one
-    GEMM per layer (the executor's cost model picks the faster form); the result is the oracle's either way, and
-    a small batch of the same model takes the fused launch."""
+def test_wide_mlp_picks_its_form_by_batch(oracle):
+    """A fusable chain of wide layers (57-200-200-200-3, rows of 57 bytes): planned as one chain; on 32 768 samples the
+    fused launch runs on the matrix units and is taken, on 3000 samples the executor's cost model prefers one GEMM per
+    layer to the small-batch form of the fused launch, on 64 samples it takes that form. The oracle's integers in all."""
+    import torch
     from aie4ml_amd.model import _mlp_layers_are_faster
     r = np.random.default_rng(31)
     dims = [57, 200, 200, 200, 3]
-    for batch in (32768, 64):
+    for batch, kinds in ((32768, ['mlp']), (64, ['mlp'])):
         gb = GraphBuilder()
         t = gb.input('x', (batch, dims[0]), qint(8, 4))
         for i in range(4):
@@ -72,9 +73,13 @@ def test_wide_mlp_on_a_large_batch_runs_layer_by_layer(oracle):
         model = gb.build()
         model.compile()
         assert len(model.context.config['gpu_fusion_plan']['mlp_chains']) == 1
-        assert _mlp_layers_are_faster(batch, list(zip(dims[:-1], dims[1:]))) == (batch == 32768)
         x = np.clip(np.rint(r.normal(0, 30, (batch, dims[0]))), -128, 127).astype(np.int8)
+        trace = []
+        model.execute({'x': torch.from_numpy(x).cuda()}, trace=trace)
+        assert [t['kind'] for t in trace] == kinds
         _graph_check(model, oracle, {'x': x})
+    shapes = list(zip(dims[:-1], dims[1:]))
+    assert _mlp_layers_are_faster(32768, shapes) and not _mlp_layers_are_faster(64, shapes)
 
 
 def test_wide_mlp_with_aligned_rows_on_a_large_batch_stays_fused(oracle):

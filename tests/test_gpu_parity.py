@@ -147,8 +147,9 @@ def test_dense_shapes_mfma_path(ops, oracle, shape):
 @pytest.mark.parametrize('mode', ['conv_even', 'positive_inf', 'symmetric_zero'])
 def test_dense_narrow_layer_on_a_long_batch(ops, oracle, shape, mode):
     """Narrow layers with one shift on 4096 rows or more go to the kernel that walks a chain of layers (a chain of one):
-    signed and unsigned rows and results, with and without ReLU and bias; the last two shapes (rows of 20 bytes, 300
-    outputs) and per-channel shifts are outside it and take the GEMM kernels, with the same integers."""
+    signed and unsigned rows and results, with and without ReLU and bias, rows of 20 bytes (cut out of the dwords that
+    cover them); 300 outputs, per-channel shifts and 16-bit results are outside it and take the GEMM kernels, with the
+    same integers."""
     M, K, N = shape
     run_dense(ops, oracle, M, K, N, mode, per_channel=False, seed=M + K + N)
     run_dense(ops, oracle, M, K, N, mode, a_dtype=np.uint8, relu=False, per_channel=False, out='uint8', seed=M + K + N + 1)
@@ -1104,6 +1105,27 @@ def test_mlp_large_batch_pitched_rows(ops, oracle):
     dx = dev(wide)[:, :16]
     got = ops.mlp(dx, specs, 'positive_inf')
     assert np.array_equal(host(got), oracle.mlp(np.ascontiguousarray(wide[:, :16]), layers_np, 'positive_inf'))
+
+
+@pytest.mark.parametrize('widths', [[57, 200, 200, 200, 3], [23, 50, 7, 256, 3], [17, 33, 5], [1, 8, 1], [5, 16]])
+def test_mlp_large_batch_rows_at_any_address(ops, oracle, widths):
+    """Input rows whose pitch is not a multiple of 16 bytes (57 features), at byte offsets 0, 1 and 3 from an aligned
+    address: the kernel cuts each 16-byte piece out of the dwords that cover it; the last row ends inside the last dword
+    the kernel may read."""
+    r = rng(sum(widths))
+    batch = 4096 + widths[0]
+    layers_np, specs = make_mlp(ops, r, widths)
+    x = r.integers(-128, 128, (batch, widths[0])).astype(np.int8)
+    want = oracle.mlp(x, layers_np, 'conv_even')
+    for off in (0, 1, 3):
+        buf = torch.zeros(batch * widths[0] + 16, dtype=torch.int8, device='cuda')
+        xv = buf[off:off + batch * widths[0]].view(batch, widths[0])
+        xv.copy_(torch.from_numpy(x))
+        assert np.array_equal(host(ops.mlp(xv, specs, 'conv_even')), want), (widths, off)
+    # rows of a wider matrix whose pitch is a multiple of 16 while the row length is not a multiple of 4
+    wide = torch.zeros((batch, 64), dtype=torch.int8, device='cuda')
+    wide[:, :widths[0]] = torch.from_numpy(x)
+    assert np.array_equal(host(ops.mlp(wide[:, :widths[0]], specs, 'conv_even')), want), widths
 
 
 def test_mlp_limits(ops):
