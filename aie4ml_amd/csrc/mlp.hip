@@ -236,42 +236,6 @@ __global__ __launch_bounds__(1024) void mlp_mfma_kernel(MlpMfmaArgs a) {
     const int nthreads = blockDim.x;  // four to sixteen waves: as many as it takes to have sixteen on the CU
     int8_t* const zero_frag = frag + (a.nfrag - 1) * 1024;  // the last fragment is all zeros
 
-    if (tid < MLP_MAX_LAYERS) big[tid] = 0;
-    if (tid < 64) *reinterpret_cast<v4i*>(zero_frag + tid * 16) = v4i{0, 0, 0, 0};
-    __syncthreads();
-    for (int l = 0; l < a.n_layers; ++l) {
-        const MlpMfmaLayer& L = a.layer[l];
-        const int pieces = L.Nb * L.Kb * 64;
-        for (int p = tid; p < pieces; p += nthreads) {
-            const int f = p >> 6, ln = p & 63;
-            const int nb = f / L.Kb, ks = f - nb * L.Kb;
-            const int col = nb * 32 + direct_col_of_operand_row(ln & 31);
-            const int k0 = ks * 32 + (ln >> 5) * 16;
-            v4i w = {0, 0, 0, 0};
-            if (col < L.N && k0 < L.K) {
-                w = *reinterpret_cast<const v4i*>(L.wt + static_cast<int64_t>(col) * L.ldwt + k0);  // ldwt % 16 == 0
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {  // inputs past K count nothing, whatever the packed rows hold there
-                    const int left = L.K - (k0 + 4 * q);
-                    if (left <= 0) w[q] = 0;
-                    else if (left < 4) w[q] &= static_cast<int>((1u << (8 * left)) - 1u);
-                }
-            }
-            *reinterpret_cast<v4i*>(frag + (L.frag0 + f) * 1024 + ln * 16) = w;
-        }
-        for (int c = tid; c < L.Nb * 32; c += nthreads) {
-            unsigned sv = 0;  // wraps like the int32 sum it stands for
-            if (c < L.N) {
-                if (L.bias) sv = static_cast<unsigned>(L.bias[c]);
-                if (L.in_unsigned) sv += 128u * static_cast<unsigned>(L.colsum[c]);
-            }
-            const int sval = static_cast<int>(sv);
-            start[L.start0 + c] = static_cast<int>(sv + static_cast<unsigned>(L.fold));
-            if (sval > (1 << 30) || sval < -(1 << 30)) big[l] = 1;  // every writer writes the same value
-        }
-    }
-    __syncthreads();
-
     const auto rsrc_x = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.X), 0, a.x_bytes, 0x00020000);
     const int units = (a.batch + 31) >> 5;
     const int wpb = nthreads >> 6;
@@ -330,7 +294,44 @@ __global__ __launch_bounds__(1024) void mlp_mfma_kernel(MlpMfmaArgs a) {
         }
     };
     const int u0 = blockIdx.x * wpb + __builtin_amdgcn_readfirstlane(tid >> 6);
-    if (AHEAD) fetch(u0, nact);
+    if (AHEAD) fetch(u0, nact);  // the first unit's input travels while the fragments are staged
+
+    if (tid < MLP_MAX_LAYERS) big[tid] = 0;
+    if (tid < 64) *reinterpret_cast<v4i*>(zero_frag + tid * 16) = v4i{0, 0, 0, 0};
+    __syncthreads();
+    for (int l = 0; l < a.n_layers; ++l) {
+        const MlpMfmaLayer& L = a.layer[l];
+        const int pieces = L.Nb * L.Kb * 64;
+        for (int p = tid; p < pieces; p += nthreads) {
+            const int f = p >> 6, ln = p & 63;
+            const int nb = f / L.Kb, ks = f - nb * L.Kb;
+            const int col = nb * 32 + direct_col_of_operand_row(ln & 31);
+            const int k0 = ks * 32 + (ln >> 5) * 16;
+            v4i w = {0, 0, 0, 0};
+            if (col < L.N && k0 < L.K) {
+                w = *reinterpret_cast<const v4i*>(L.wt + static_cast<int64_t>(col) * L.ldwt + k0);  // ldwt % 16 == 0
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {  // inputs past K count nothing, whatever the packed rows hold there
+                    const int left = L.K - (k0 + 4 * q);
+                    if (left <= 0) w[q] = 0;
+                    else if (left < 4) w[q] &= static_cast<int>((1u << (8 * left)) - 1u);
+                }
+            }
+            *reinterpret_cast<v4i*>(frag + (L.frag0 + f) * 1024 + ln * 16) = w;
+        }
+        for (int c = tid; c < L.Nb * 32; c += nthreads) {
+            unsigned sv = 0;  // wraps like the int32 sum it stands for
+            if (c < L.N) {
+                if (L.bias) sv = static_cast<unsigned>(L.bias[c]);
+                if (L.in_unsigned) sv += 128u * static_cast<unsigned>(L.colsum[c]);
+            }
+            const int sval = static_cast<int>(sv);
+            start[L.start0 + c] = static_cast<int>(sv + static_cast<unsigned>(L.fold));
+            if (sval > (1 << 30) || sval < -(1 << 30)) big[l] = 1;  // every writer writes the same value
+        }
+    }
+    __syncthreads();
+
     for (int u = u0; u < units; u += nwaves) {
         const int row = u * 32 + m;
         const bool row_ok = row < a.batch;
