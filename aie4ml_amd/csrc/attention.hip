@@ -380,8 +380,8 @@ static void launch_attention_nt(int grid, int grid8, size_t lds, hipStream_t str
     if (ragged) {                                                                    \
         if (fastp) attention_kernel<NT, DT, B, true, 4, true><<<grid, 256, lds, stream>>>(a);   \
         else attention_kernel<NT, DT, B, false, 4, true><<<grid, 256, lds, stream>>>(a);        \
-    } else if (NT >= 8 && grid8 > 0) {                                                      \
-        if constexpr (NT >= 8) {                                                     \
+    } else if (NT >= 8 && DT == 2 && grid8 > 0) {                                           \
+        if constexpr (NT >= 8 && DT == 2) {                                                     \
             if (fastp) launch_attention_wide<NT, DT, B, true>(grid8, lds, stream, a); \
             else launch_attention_wide<NT, DT, B, false>(grid8, lds, stream, a);      \
         }                                                                            \
@@ -407,7 +407,10 @@ static int launch_attention(int nt, int grid, int grid8, hipStream_t stream, con
     case 2: launch_attention_nt<2, DT>(grid, 0, lds, stream, a); break;
     case 4: launch_attention_nt<4, DT>(grid, 0, lds, stream, a); break;
     case 8: launch_attention_nt<8, DT>(grid, grid8, lds, stream, a); break;
-    case 16: launch_attention_nt<16, DT>(grid, grid8, lds, stream, a); break;
+    case 16:
+        if constexpr (DT <= 2) launch_attention_nt<16, DT>(grid, grid8, lds, stream, a);
+        else return 1;
+        break;
     default: return 1;
     }
     return 0;
@@ -440,8 +443,9 @@ extern "C" int a4g_attention_i8(const int8_t* Q, const int8_t* K, const int8_t* 
         if (int rc = make_hccs_params(who, sk, hccs_B, hccs_S, hccs_Dmax, inv_shift, use_clb, A4G_U8, &a.sm, &noclamp))
             return rc;
     }
-    A4G_REQUIRE(d == 64 && sk <= 512, A4G_ERR_UNSUPPORTED,
-                "%s: fused path covers head_dim 64 and up to 512 keys, got d=%lld sk=%lld", who, (long long)d, (long long)sk);
+    A4G_REQUIRE((d == 64 && sk <= 512) || (d == 32 && sk <= 512) || (d == 128 && sk <= 256), A4G_ERR_UNSUPPORTED,
+                "%s: fused path covers head_dim 64 and 32 with up to 512 keys and head_dim 128 with up to 256, got d=%lld sk=%lld",
+                who, (long long)d, (long long)sk);
     int nt = 1;  // tiles of 32 keys the kernel is instantiated for: the next power of two
     while (nt * 32 < sk) nt *= 2;
     const bool ragged = nt * 32 != sk;
@@ -470,9 +474,10 @@ extern "C" int a4g_attention_i8(const int8_t* Q, const int8_t* K, const int8_t* 
     const int grid = static_cast<int>(batch * heads * ((sq + 127) / 128));
     // eight waves per workgroup (256 query rows, bank-replicated score table) once every CU gets at least one
     const int64_t wg8 = batch * heads * ((sq + 255) / 256);
-    const int grid8 = (!ragged && sq >= 256 && wg8 >= 256) ? static_cast<int>(wg8) : 0;
+    const int grid8 = (!ragged && d == 64 && sq >= 256 && wg8 >= 256) ? static_cast<int>(wg8) : 0;
     a.items = grid8 > 0 ? grid8 : grid;
-    if (launch_attention<2>(nt, grid, grid8, stream, a))
-        return fail(A4G_ERR_UNSUPPORTED, "%s: no kernel for sk=%lld", who, (long long)sk);
+    const int no_kernel = d == 64 ? launch_attention<2>(nt, grid, grid8, stream, a)
+                          : (d == 32 ? launch_attention<1>(nt, grid, 0, stream, a) : launch_attention<4>(nt, grid, 0, stream, a));
+    if (no_kernel) return fail(A4G_ERR_UNSUPPORTED, "%s: no kernel for sk=%lld", who, (long long)sk);
     return check_hip(hipGetLastError(), who);
 }

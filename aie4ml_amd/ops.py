@@ -445,7 +445,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, logit_shift: in
     contiguous last axis (head slices of a packed projection are fine). `softmax` is
     {'kind': 'exp', 'exp_kq': .., 'inv_shift': 15} or {'kind': 'hccs', 'B': .., 'S': .., 'Dmax': .., 'inv_shift': 15,
     'use_clb': False}. Bit-identical to matmul(trans_b) -> softmax_* -> matmul. Raises NotImplementedError for
-    shapes the fused kernel does not cover (head_dim != 64, more than 512 keys, unaligned views).
+    shapes the fused kernel does not cover (head_dim other than 32, 64 or 128, more than 512 keys - 256 at head_dim 128 -,
+    unaligned views).
     """
     for name, t in (('q', q), ('k', k), ('v', v)):
         _dev(t, name)

@@ -436,8 +436,7 @@ class PlanGpuFusion(AIEPass):
                 and cfg.n_in <= self.ROWLN_MAX_K and cfg.n_out >= 384)
 
     # ---- attention -------------------------------------------------------------------------------------
-    ATTN_HEAD_DIM = 64
-    ATTN_MAX_KEYS = 512
+    ATTN_MAX_KEYS = {32: 512, 64: 512, 128: 256}  # head dimension -> keys the fused kernel takes
     ATTN_MAX_SHIFT = 24
 
     def _plan_attention(self, graph, execution, outputs):
@@ -469,7 +468,7 @@ class PlanGpuFusion(AIEPass):
             if len(q.shape) != len(k.shape) or len(k.shape) != len(v.shape) or tuple(k.shape) != tuple(v.shape) \
                     or tuple(q.shape[:-2]) != tuple(k.shape[:-2]) or len(q.shape) not in (2, 3, 4):
                 continue
-            if int(q.shape[-1]) != self.ATTN_HEAD_DIM or not 1 <= int(k.shape[-2]) <= self.ATTN_MAX_KEYS:
+            if not 1 <= int(k.shape[-2]) <= self.ATTN_MAX_KEYS.get(int(q.shape[-1]), 0):
                 continue
             if c1.shift > self.ATTN_MAX_SHIFT or c3.shift > self.ATTN_MAX_SHIFT:
                 continue  # the fused kernel takes shifts up to 24, the MatMul kernels up to 31
@@ -515,7 +514,7 @@ class PlanGpuFusion(AIEPass):
             cand.setdefault(key, []).append((o_start, sq[1], sk_[1], sv_[1], tr))
         for (qs, ks, vs, cat_name), items in cand.items():
             items.sort(key=lambda x: x[0])
-            d = self.ATTN_HEAD_DIM
+            d = int(graph.tensors[items[0][4]['q']].shape[-1])  # head dimension
             cat = by_name[cat_name]
             regular = len(items) == len(cat.traits['concat_view'].data['slices']) and len(items) >= 2
             for h, (o, a, b, c, tr) in enumerate(items):

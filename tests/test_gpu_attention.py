@@ -84,6 +84,24 @@ def test_attention_key_count_off_the_tile_grid(oracle, sk, kind):
         np.testing.assert_array_equal(got, reference(oracle, q, k, v, 6, lmode, sm, 7, 'conv_even'))
 
 
+@pytest.mark.parametrize('d,sk', [(32, 32), (32, 128), (32, 512), (32, 197), (128, 64), (128, 256), (128, 100)])
+@pytest.mark.parametrize('kind', ['exp', 'hccs'])
+def test_attention_head_dimensions_32_and_128(oracle, d, sk, kind):
+    """One and four MFMA K steps per key tile instead of two; sequence lengths on and off the tile grid; a query count
+    of its own; both logit requantisations."""
+    for sq in (sk, 45):
+        q, k, v = qkv(7000 + d + sk + sq, (2, 3, sq, d), (2, 3, sk, d), sigma=24.0 if d <= 64 else 16.0)
+        if kind == 'exp':
+            sm = {'kind': 'exp', 'exp_kq': 23}
+        else:
+            B = min(255, 32767 // sk)
+            sm = {'kind': 'hccs', 'B': B, 'S': 1, 'Dmax': min(126, B - (256 + sk - 1) // sk)}
+        lmode = 'conv_even' if sq == sk else 'floor'
+        lshift = 6 if d <= 64 else 7
+        got = ops.attention(dev(q), dev(k), dev(v), lshift, lmode, sm, 7, 'conv_even').cpu().numpy()
+        np.testing.assert_array_equal(got, reference(oracle, q, k, v, lshift, lmode, sm, 7, 'conv_even'))
+
+
 def test_attention_masked_keys_do_not_leak(oracle):
     """The rows behind the last key are other tensors' memory: whatever they hold, the result is that of the keys that
     exist (K rows past the end alias the last row inside the kernel, V rows past the end are not read)."""
@@ -177,7 +195,7 @@ def test_attention_on_head_slices_of_a_packed_projection(oracle):
 
 
 def test_attention_uncovered_shapes_and_bad_parameters():
-    q = torch.zeros((2, 64, 32), dtype=torch.int8, device='cuda')
+    q = torch.zeros((2, 64, 96), dtype=torch.int8, device='cuda')
     with pytest.raises(NotImplementedError, match='fused path covers head_dim 64'):
         ops.attention(q, q, q, 6, 'floor', {'kind': 'exp', 'exp_kq': 23}, 7, 'floor')
     q = torch.zeros((2, 544, 64), dtype=torch.int8, device='cuda')

@@ -370,7 +370,8 @@ def test_encoder_block_graph_lowers():
     assert plan['add_layernorm']['residual1_aie'] == {'layer_norm': 'ln1_aie', 'keep_sum': False}
     assert plan['mlp_chains'] == [['ffn1_aie', 'ffn2_aie']]   # widths 64/128/64 fit the fused-MLP kernel
     assert x.shape == (2, 32, 64) and x.dtype == np.int8
-    assert plan['attention'] == []          # head_dim 32 is outside the fused attention kernel's range
+    (grp,) = plan['attention']              # head_dim 32: both heads in one fused launch, Q / K / V slices 32 apart
+    assert len(grp['heads']) == 2 and grp['concat'] == 'heads_concat_aie'
     assert plan['dense_add_layernorm'] == {}  # 64 outputs: too narrow for the projection that normalises its own rows
 
 
@@ -397,7 +398,15 @@ def test_attention_plan_merges_heads():
     # a lone triple (its probabilities are also a graph output in the second graph: not fusable)
     gb = attention_graph(scale=None)
     ctx = lower(gb, FRONT + (PlanGpuFusion,))
-    assert ctx.config['gpu_fusion_plan']['attention'] == []     # head_dim 32
+    (grp,) = ctx.config['gpu_fusion_plan']['attention']         # head_dim 32 has a fused kernel of its own
+    assert grp['concat'] is None
+    gb = GraphBuilder()                                         # head_dim 48 has none
+    q = gb.input('q', (2, 64, 48), qint(8, 4))
+    k = gb.input('k', (2, 64, 48), qint(8, 4))
+    v = gb.input('v', (2, 64, 48), qint(8, 4))
+    p = gb.softmax(gb.matmul(q, gb.transpose(k, (0, 2, 1)), qint(8, 4), name='qk'), qint(8, 8, signed=False), name='sm')
+    gb.output(gb.matmul(p, v, qint(8, 4), name='pv'))
+    assert lower(gb, FRONT + (PlanGpuFusion,)).config['gpu_fusion_plan']['attention'] == []
     gb = GraphBuilder()
     q = gb.input('q', (2, 64, 64), qint(8, 4))
     k = gb.input('k', (2, 64, 64), qint(8, 4))
