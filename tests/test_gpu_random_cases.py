@@ -168,6 +168,104 @@ def test_attention_random_case(ops, oracle, seed):
     assert np.array_equal(got, exp), (seed, lead, sq, sk, lshift, lmode, oshift, omode, sm)
 
 
+@pytest.mark.parametrize('seed', range(24 + EXTRA // 4))
+def test_attention_any_key_count_and_head_dimension_random_case(ops, oracle, seed):
+    """Head dimensions 32, 64 and 128, any number of keys the fused kernel takes for them, any number of queries."""
+    r = np.random.default_rng(4500 + seed)
+    d = int(r.choice([32, 64, 128]))
+    sk = int(r.integers(1, (256 if d == 128 else 512) + 1))
+    if r.random() < 0.3:
+        sk = int(r.choice([31, 33, 64, 100, 197, 255, 256]))
+    sq = int(r.choice([1, 33, 100, sk, 197, 300]))
+    lead = [(1, 1), (2, 3), (5, 2), (3,)][int(r.integers(0, 4))]
+    sigma = float(r.choice([8.0, 24.0, 60.0])) * (0.6 if d == 128 else 1.0)
+    g = lambda s: np.clip(np.rint(r.normal(0, sigma, s)), -128, 127).astype(np.int8)  # noqa: E731
+    q, k, v = g(lead + (sq, d)), g(lead + (sk, d)), g(lead + (sk, d))
+    lshift, oshift = int(r.integers(0, 17)), int(r.integers(0, 12))
+    lmode, omode = str(r.choice(MODES)), str(r.choice(MODES))
+    if r.random() < 0.5:
+        lmode = 'conv_even'
+    logits = oracle.matmul(q, k, lshift, lmode, trans_b=True)
+    B = min(255, 32767 // sk)
+    dmax = min(126, B - (256 + sk - 1) // sk)
+    if seed % 2 == 0 or dmax < 1:
+        sm = {'kind': 'exp', 'exp_kq': int(r.integers(1, 129))}
+        p = oracle.softmax_exp(logits, sm['exp_kq'])
+    else:
+        sm = {'kind': 'hccs', 'B': B, 'S': 1, 'Dmax': dmax}
+        p = oracle.softmax_hccs(logits, B, 1, dmax, 15, False)
+    exp = oracle.matmul(p, v, oshift, omode)
+    got = host(ops.attention(dev(q), dev(k), dev(v), lshift, lmode, sm, oshift, omode))
+    assert np.array_equal(got, exp), (seed, lead, sq, sk, d, lshift, lmode, oshift, omode, sm)
+
+
+@pytest.mark.parametrize('seed', range(24 + EXTRA // 4))
+def test_mlp_chain_on_a_long_batch_random_case(ops, oracle, seed):
+    """Chains of one to five layers of random widths up to 256 on 4096 samples or more (the matrix-unit form where the
+    fragments fit the LDS, the dot-product form otherwise): random shifts, ReLU, signed and unsigned activations, rows at
+    random byte offsets, biases that sometimes reach the int32 limits."""
+    r = np.random.default_rng(4700 + seed)
+    n_layers = int(r.integers(1, 6))
+    widths = [int(r.choice([1, 5, 16, 17, 32, 48, 57, 64, 100, 128, 200, 256])) for _ in range(n_layers + 1)]
+    batch = 4096 + int(r.integers(0, 200))
+    mode = str(r.choice(MODES))
+    x_unsigned = bool(r.random() < 0.3)
+    x = r.integers(0, 256, (batch, widths[0])).astype(np.uint8) if x_unsigned else r.integers(-128, 128, (batch, widths[0])).astype(np.int8)
+    big_bias = r.random() < 0.15
+    layers_np, specs = [], []
+    for i, (k, n) in enumerate(zip(widths[:-1], widths[1:])):
+        W = r.integers(-64, 64, (k, n)).astype(np.int8)
+        span = 2**31 - 2**23 if big_bias else 2**13
+        b = r.integers(-span, span + 1, n).astype(np.int32) if r.random() < 0.9 else None
+        sh = int(r.integers(0, 13)) if r.random() < 0.85 else int(r.integers(13, 32))
+        relu = bool(r.random() < 0.6)
+        last = i == n_layers - 1
+        out = str(r.choice(['int8', 'uint8', 'int16'])) if last else str(r.choice(['int8', 'uint8']))
+        layers_np.append((W, b, sh, relu, out))
+        specs.append(ops.MlpLayerSpec(ops.pack_dense(dev(W), dev(b) if b is not None else None, sh), sh, relu, out))
+    off = int(r.choice([0, 0, 1, 2, 3, 16]))
+    buf = torch.zeros(batch * widths[0] + 32, dtype=torch.uint8 if x_unsigned else torch.int8, device='cuda')
+    xv = buf[off:off + batch * widths[0]].view(batch, widths[0])
+    xv.copy_(torch.from_numpy(x))
+    try:
+        got = host(ops.mlp(xv, specs, mode))
+    except NotImplementedError:
+        return  # more weights than the fused kernels hold
+    assert np.array_equal(got, oracle.mlp(x, layers_np, mode)), (seed, widths, batch, mode, off, [(l[2], l[3], l[4]) for l in layers_np])
+
+
+@pytest.mark.parametrize('seed', range(16 + EXTRA // 4))
+def test_long_row_operator_random_case(ops, oracle, seed):
+    """LayerNorm, fused Add + LayerNorm and both Softmax forms on rows of 4112 to 20 000 columns."""
+    r = np.random.default_rng(4900 + seed)
+    cols = int(r.choice([4112, 4608, 5120, 6144, 7168, 8192, 8208, 10240, 12288, 16384, 16400, 20000]))
+    rows = int(r.integers(1, 80))
+    mode = str(r.choice(MODES))
+    x = np.clip(np.rint(r.normal(float(r.integers(-20, 20)), float(r.choice([5.0, 25.0, 70.0])), (rows, cols))), -128, 127).astype(np.int8)
+    gamma = r.integers(-600, 600, cols).astype(np.int16)
+    beta = r.integers(-20000, 20000, cols).astype(np.int16)
+    oshift, eps = int(r.integers(0, 9)), int(r.integers(1, 50))
+    which = seed % 4
+    if which == 0:
+        got = host(ops.layernorm(dev(x), dev(gamma), dev(beta), oshift, mode, eps_q0=eps))
+        assert np.array_equal(got, oracle.layernorm(x, gamma, beta, oshift, mode, eps_q0=eps)), (seed, cols, rows, mode)
+    elif which == 1:
+        x2 = np.clip(np.rint(r.normal(0, 40, (rows, cols))), -128, 127).astype(np.int8)
+        s_, o_ = ops.add_layernorm(dev(x), dev(x2), dev(gamma), dev(beta), oshift, mode, eps_q0=eps, return_sum=True)
+        es, eo = oracle.add_layernorm(x, x2, gamma, beta, oshift, mode, eps_q0=eps, return_sum=True)
+        assert np.array_equal(host(s_), es) and np.array_equal(host(o_), eo), (seed, cols, rows, mode)
+    elif which == 2:
+        kq, out = int(r.integers(1, 129)), str(r.choice(['uint8', 'int16']))
+        got = host(ops.softmax_exp(dev(x), kq, out_kind=out))
+        assert np.array_equal(got, oracle.softmax_exp(x, kq, out=out)), (seed, cols, rows, kq, out)
+    else:
+        B = max(2, 32767 // cols)
+        if cols * B > 32767:
+            return
+        got = host(ops.softmax_hccs(dev(x), B, 1, B - 1))
+        assert np.array_equal(got, oracle.softmax_hccs(x, B, 1, B - 1)), (seed, cols, rows)
+
+
 @pytest.mark.parametrize('seed', range(24 + EXTRA))
 def test_transposed_lhs_random_case(ops, oracle, seed):
     """MatMul and Dense whose left operand is stored [K][M] (transposed inside the kernel): shapes around the tile
