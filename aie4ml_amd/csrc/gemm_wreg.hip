@@ -66,6 +66,11 @@ __global__ __launch_bounds__(WR_NT, 2) void gemm_wreg_kernel(GemmArgs g, int hal
     // offsets (j = 0, 1) cover all four instructions; j = 2, 3 add 16 rows, a scalar
     const int row0 = wave * 32 + lrow8, sw0 = (slot ^ (lrow8 >> 1)) * 16;
     const int va0 = row0 * lda + sw0, va1 = (row0 + 8) * lda + (sw0 ^ 64);
+    // A reduction that ends inside its last 128-byte tile (K a multiple of 16 only): the lanes whose chunk of that tile
+    // lies past K fetch nothing (an offset of the buffer's size: zeros), and zero activations make whatever the weight
+    // tile holds there (the next weight row's first bytes) count for nothing.
+    const int k_last = g.K - (NKT - 1) * WR_BK;  // bytes of the last tile that exist, 16 .. 128
+    const int va0_last = sw0 < k_last ? va0 : a_bytes, va1_last = (sw0 ^ 64) < k_last ? va1 : a_bytes;
     const auto rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(g.A), 0, a_bytes, 0x00020000);
     const auto rsrc_w = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(g.Bt), 0, w_bytes, 0x00020000);
 
@@ -89,7 +94,8 @@ __global__ __launch_bounds__(WR_NT, 2) void gemm_wreg_kernel(GemmArgs g, int hal
     // activation tile (step, kt) of the run; nothing is fetched past its end (the lower 64 rows of a short last step)
     auto issue_a = [&](int step, int kt, int st) {
         const bool live = step < steps && !(short_last && step == steps - 1 && wave >= 2);
-        issue(rsrc_a, va0, va1, lda, live ? (m0 + step * WR_BM) * lda + kt * WR_BK : a_bytes, st);
+        const bool last_kt = kt == NKT - 1;
+        issue(rsrc_a, last_kt ? va0_last : va0, last_kt ? va1_last : va1, lda, live ? (m0 + step * WR_BM) * lda + kt * WR_BK : a_bytes, st);
     };
     // ring position r: the NKT weight tiles of the column block, then the activation tiles
     auto issue_ring = [&](int r) {
@@ -266,7 +272,9 @@ hipError_t launch_wreg_nkt(const GemmArgs& g, int halves_m, int wgs_per_cb, int 
 // 16-column pieces, and operands small enough for 32-bit buffer offsets. Measured faster than the tiled kernel at every
 // size tried, from one row to 8192 x 3072.
 bool wreg_applicable(const GemmArgs& g) {
-    return g.M > 0 && g.K % 128 == 0 && g.K >= 128 && g.K <= 768 && g.N % 16 == 0 && g.N >= 16 &&
+    // K a multiple of 128, or of 16 with signed activations (a uint8 operand is biased by 128 in the registers, which
+    // would turn the zeros of a partial last tile into -128)
+    return g.M > 0 && (g.K % 128 == 0 || (g.K % 16 == 0 && !g.a_unsigned)) && g.K >= 16 && g.K <= 768 && g.N % 16 == 0 && g.N >= 16 &&
            (g.out_kind == A4G_I8 || g.out_kind == A4G_U8) && g.lda % 16 == 0 && g.ldb % 16 == 0 && g.ldc % 16 == 0 && aligned16(g.A) &&
            aligned16(g.Bt) && aligned16(g.C) && (static_cast<int64_t>(g.M) + 2 * WR_BM) * g.lda < (int64_t{1} << 31) &&
            (static_cast<int64_t>(g.N) + WR_BN) * g.ldb < (int64_t{1} << 31) && (g.N + WR_BN - 1) / WR_BN <= 65536;
@@ -281,7 +289,7 @@ hipError_t launch_wreg(const GemmArgs& g, hipStream_t stream) {
     const int wgs_per_cb = (halves_m + longest - 1) / longest;
     const int a_bytes = static_cast<int>(static_cast<int64_t>(g.M - 1) * g.lda + g.K);
     const int w_bytes = static_cast<int>(static_cast<int64_t>(g.N - 1) * g.ldb + g.K);
-    switch (g.K / 128) {
+    switch ((g.K + 127) / 128) {
     case 1: return launch_wreg_nkt<1>(g, halves_m, wgs_per_cb, cbs, a_bytes, w_bytes, stream);
     case 2: return launch_wreg_nkt<2>(g, halves_m, wgs_per_cb, cbs, a_bytes, w_bytes, stream);
     case 3: return launch_wreg_nkt<3>(g, halves_m, wgs_per_cb, cbs, a_bytes, w_bytes, stream);

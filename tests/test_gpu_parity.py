@@ -158,6 +158,20 @@ def test_dense_narrow_layer_on_a_long_batch(ops, oracle, shape, mode):
     run_dense(ops, oracle, M, K, N, mode, per_channel=False, out='int16', seed=M + K + N + 4)
 
 
+@pytest.mark.parametrize('shape', [(5000, 192, 576), (700, 80, 384), (130, 16, 1024), (64, 656, 768), (333, 208, 512),
+                                   (1, 48, 16), (129, 752, 272)])
+@pytest.mark.parametrize('mode', ['conv_even', 'symmetric_inf'])
+def test_dense_reduction_that_ends_inside_a_tile(ops, oracle, shape, mode):
+    """K a multiple of 16 but not of 128 (192 inputs of a small vision transformer): the weights-in-registers kernel
+    takes it with signed activations, fetching nothing for the part of the last 128-byte tile past K; unsigned
+    activations (biased in registers) keep the tiled kernel. Per-channel and single shifts, every output kind it has."""
+    M, K, N = shape
+    run_dense(ops, oracle, M, K, N, mode, seed=M + K + N)
+    run_dense(ops, oracle, M, K, N, mode, per_channel=False, relu=False, out='uint8', seed=M + K + N + 1)
+    run_dense(ops, oracle, M, K, N, mode, a_dtype=np.uint8, seed=M + K + N + 2)
+    run_dense(ops, oracle, M, K, N, mode, bias=False, out='int16', seed=M + K + N + 3)
+
+
 @pytest.mark.parametrize('shape', [(5, 3, 2), (64, 17, 33), (9, 100, 12), (128, 250, 64)])
 def test_dense_ragged_k_generic_path(ops, oracle, shape):
     M, K, N = shape
