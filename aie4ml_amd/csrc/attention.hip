@@ -151,7 +151,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
                 *reinterpret_cast<v4i*>(table + i) = v4i{e, e, e, e};
             }
         } else {
-            table[tid] = table_entry(a.sm, tid);
+            for (int i = tid; i < 256; i += THREADS) table[i] = table_entry(a.sm, i);
         }
     }
     // everybody is done with the previous item's V^T, column sums and parked scores (first item: with the table's
@@ -398,6 +398,22 @@ static void launch_attention_nt(int grid, int grid8, size_t lds, hipStream_t str
 #undef A4G_ATTN
 }
 
+// Seven key tiles, seven waves (224 x 224 covers a head of 193 .. 224 tokens), always in the ragged form.
+static void launch_attention_seven(int grid, hipStream_t stream, const AttnArgs& a) {
+    const size_t lds = static_cast<size_t>(64) * (7 * 32 + 16) + 64 * 4;
+    const bool fastp = a.noclamp && a.sm.out_shift <= 16;
+#define A4G_ATTN7(B)                                                                       \
+    if (fastp) attention_kernel<7, 2, B, true, 7, true><<<grid, 448, lds, stream>>>(a);    \
+    else attention_kernel<7, 2, B, false, 7, true><<<grid, 448, lds, stream>>>(a);
+    switch (a.lscale > 0.f ? 3 : fast_round_kind(a.lr)) {
+    case 0: A4G_ATTN7(0) break;
+    case 1: A4G_ATTN7(1) break;
+    case 2: A4G_ATTN7(2) break;
+    default: A4G_ATTN7(3) break;
+    }
+#undef A4G_ATTN7
+}
+
 template <int DT>
 static int launch_attention(int nt, int grid, int grid8, hipStream_t stream, const AttnArgs& a) {
     size_t lds = static_cast<size_t>(DT * 32) * (nt * 32 + 16) + DT * 32 * 4;  // V^T + column sums
@@ -476,6 +492,13 @@ extern "C" int a4g_attention_i8(const int8_t* Q, const int8_t* K, const int8_t* 
     const int64_t wg8 = batch * heads * ((sq + 255) / 256);
     const int grid8 = (!ragged && d == 64 && sq >= 256 && wg8 >= 256) ? static_cast<int>(wg8) : 0;
     a.items = grid8 > 0 ? grid8 : grid;
+    if (d == 64 && sq > 192 && sq <= 224 && sk > 192 && sk <= 224) {
+        // 193 .. 224 queries and keys (the 197 tokens of a vision transformer): seven key tiles instead of eight, and one
+        // workgroup of seven waves per head instead of two of four, so that a head's V^T and score table are built once
+        a.items = static_cast<int>(batch * heads);
+        launch_attention_seven(a.items, stream, a);
+        return check_hip(hipGetLastError(), who);
+    }
     const int no_kernel = d == 64 ? launch_attention<2>(nt, grid, grid8, stream, a)
                           : (d == 32 ? launch_attention<1>(nt, grid, 0, stream, a) : launch_attention<4>(nt, grid, 0, stream, a));
     if (no_kernel) return fail(A4G_ERR_UNSUPPORTED, "%s: no kernel for sk=%lld", who, (long long)sk);
