@@ -498,7 +498,10 @@ static int layernorm_dispatch(const int8_t* a, const int8_t* b, int add_shift, i
     launched = launch_ln_rows<L, NCH>(bit_kind, fr, fuse, grid_for(nrows, 4 * (64 / L), max_grid), lds, stream, ac, bc,  \
                                       gamma, beta, sc, oc, nrows, (int)cols, log2c, eps_q0, rg, ro, lf)
             hipError_t launched = hipSuccess;
-            if (nchunks <= 16) A4G_LN_GO(8, 2);
+            if (nchunks <= 8) A4G_LN_GO(4, 2);
+            else if (nchunks <= 12) A4G_LN_GO(4, 3);
+            else if (nchunks <= 16) A4G_LN_GO(8, 2);
+            else if (nchunks <= 24) A4G_LN_GO(8, 3);
             else if (nchunks <= 32) A4G_LN_GO(16, 2);
             else if (nchunks <= 48) A4G_LN_GO(16, 3);
             else if (nchunks <= 64) A4G_LN_GO(32, 2);

@@ -647,7 +647,7 @@ def ln_params(r, cols):
     return gamma, beta
 
 
-@pytest.mark.parametrize('cols', [16, 32, 128, 768, 1024, 2048, 4096, 48, 100, 8192])
+@pytest.mark.parametrize('cols', [16, 32, 64, 128, 192, 256, 384, 512, 768, 1024, 2048, 4096, 48, 100, 8192])
 def test_layernorm_columns(ops, oracle, cols):
     r = rng(cols)
     rows = 37
@@ -759,7 +759,7 @@ def test_add_layernorm_long_rows(ops, oracle, cols, mode):
     assert np.array_equal(host(ops.add_layernorm(dev(a), dev(b), dev(gamma), dev(beta), 5, mode)), eo)
 
 
-@pytest.mark.parametrize('cols', [64, 768, 1024, 100])
+@pytest.mark.parametrize('cols', [64, 128, 192, 384, 768, 1024, 100])
 def test_add_layernorm_fused(ops, oracle, cols):
     r = rng(cols + 7)
     a = gauss8(r, 60, (41, cols))
