@@ -301,24 +301,39 @@ __global__ __launch_bounds__(1024) void mlp_mfma_kernel(MlpMfmaArgs a) {
     __syncthreads();
     for (int l = 0; l < a.n_layers; ++l) {
         const MlpMfmaLayer& L = a.layer[l];
+        // Fragments, one 16-byte piece at a time per thread; where a layer has four rounds of pieces or more, four are
+        // fetched together (a few round trips to L2 instead of one per piece). A piece that does not exist lies past the descriptor and reads as zero.
         const int pieces = L.Nb * L.Kb * 64;
-        for (int p = tid; p < pieces; p += nthreads) {
+        const int Kb_l = L.Kb, N_l = L.N, K_l = L.K, ldwt_l = L.ldwt, frag0_l = L.frag0;
+        const auto rsrc_w = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(L.wt), 0, N_l * ldwt_l, 0x00020000);
+        auto piece_from = [&](int p) -> int {  // byte offset of piece p in the packed weights, or nowhere
             const int f = p >> 6, ln = p & 63;
-            const int nb = f / L.Kb, ks = f - nb * L.Kb;
+            const int nb = f / Kb_l, ks = f - nb * Kb_l;
             const int col = nb * 32 + direct_col_of_operand_row(ln & 31);
             const int k0 = ks * 32 + (ln >> 5) * 16;
-            v4i w = {0, 0, 0, 0};
-            if (col < L.N && k0 < L.K) {
-                w = *reinterpret_cast<const v4i*>(L.wt + static_cast<int64_t>(col) * L.ldwt + k0);  // ldwt % 16 == 0
+            return (p < pieces && col < N_l && k0 < K_l) ? col * ldwt_l + k0 : 0x7ffffff0;
+        };
+        auto piece_store = [&](int p, v4i w) {
+            const int f = p >> 6, ln = p & 63;
+            const int k0 = (f - (f / Kb_l) * Kb_l) * 32 + (ln >> 5) * 16;
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {  // inputs past K count nothing, whatever the packed rows hold there
-                    const int left = L.K - (k0 + 4 * q);
-                    if (left <= 0) w[q] = 0;
-                    else if (left < 4) w[q] &= static_cast<int>((1u << (8 * left)) - 1u);
-                }
+            for (int q = 0; q < 4; ++q) {  // inputs past K count nothing, whatever the packed rows hold there
+                const int left = K_l - (k0 + 4 * q);
+                if (left <= 0) w[q] = 0;
+                else if (left < 4) w[q] &= static_cast<int>((1u << (8 * left)) - 1u);
             }
-            *reinterpret_cast<v4i*>(frag + (L.frag0 + f) * 1024 + ln * 16) = w;
+            if (p < pieces) *reinterpret_cast<v4i*>(frag + (frag0_l + f) * 1024 + ln * 16) = w;
+        };
+        int p = tid;
+        for (; p - tid + 4 * nthreads <= pieces; p += 4 * nthreads) {  // (uniform: four whole rounds are left)
+            v4i w[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) w[j] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, piece_from(p + j * nthreads), 0, 0));
+#pragma unroll
+            for (int j = 0; j < 4; ++j) piece_store(p + j * nthreads, w[j]);
         }
+        for (; p < pieces; p += nthreads)
+            piece_store(p, __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, piece_from(p), 0, 0)));
         for (int c = tid; c < L.Nb * 32; c += nthreads) {
             unsigned sv = 0;  // wraps like the int32 sum it stands for
             if (c < L.N) {

@@ -348,7 +348,7 @@ class GPUModel:
             rows *= int(d)
         shapes = [(s.params.K, s.params.N) for s in specs]
         x_pitch = int(x.shape[-1]) if x.is_contiguous() else 0
-        if not ops.mlp_runs_on_matrix_units(rows, x_pitch, shapes) and _mlp_layers_are_faster(rows, shapes):
+        if _mlp_layers_are_faster(rows, shapes, ops.mlp_runs_on_matrix_units(rows, x_pitch, shapes)):
             for inst in insts:  # wide layers on a large batch: one GEMM per layer beats the launch that keeps weights in LDS
                 values.update(inst.variant.run(inst, {input_tensor_for_role(inst.node, 'lhs').name:
                                                       values[input_tensor_for_role(inst.node, 'lhs').name]}))
@@ -363,7 +363,7 @@ def _views_are_16_byte_aligned(*tensors) -> bool:
     return all(t.data_ptr() % 16 == 0 and all(int(st) % 16 == 0 for st in t.stride()[:-1]) for t in tensors)
 
 
-def _mlp_layers_are_faster(rows: int, layers) -> bool:
+def _mlp_layers_are_faster(rows: int, layers, on_matrix_units: bool = False) -> bool:
     """Whether a chain of Dense layers should run as one GEMM per layer instead of the fused launch, where that launch
     takes its small-batch form (its large-batch form, on the matrix units, is ahead of the per-layer GEMMs wherever it
     applies: 16-64-32-32-5 on 1 048 576 rows 44 us against 479 us, 64-200-200-200-3 on 65 536 rows 33 against 114 us).
@@ -373,6 +373,12 @@ def _mlp_layers_are_faster(rows: int, layers) -> bool:
     about 200 TOP/s on its tiles, which are 128 wide in N and 64 deep in K at least (256 for wide layers).
     Measured: 57-200-200-200-3 on 65 536 rows 299 us fused / 139 us per layer; on 8192 rows 65 / 70 us;
     16-64-32-32-5 on 1 000 000 rows 190 / 478 us. The per-layer form must be ahead by a quarter to be chosen."""
+    if on_matrix_units:
+        # ahead of the per-layer GEMMs except for layers that suit the weights-in-registers GEMM (reductions in whole
+        # 128-byte tiles, 128 outputs or more) on a batch that gives a CU only a few units of 32 samples:
+        # 128-256-128, fused / per layer: 13.4 / 9.3 us on 4096 rows, 14.0 / 10.8 on 16 384, 15.8 / 17.8 on 65 536
+        return rows < 32768 and all(k % 128 == 0 and n >= 128 for k, n in layers)
+
     def up(v, m):
         return (v + m - 1) // m * m
     macs = sum(k * n for k, n in layers)
