@@ -218,7 +218,7 @@ struct MlpMfmaArgs {
     int y_packed;     // at most 32 outputs in rows without gaps, Y 4-byte aligned: the tile store
 };
 
-constexpr int64_t MLP_MFMA_MIN_BATCH = 4096;
+constexpr int64_t MLP_MFMA_MIN_BATCH = 512;
 
 // MAXB: blocks of 32 that the widest layer has (2, 4 or 8: the loops over blocks are unrolled that far and guarded).
 // BIT: what the rounding mode adds besides its constant (fast_round_kind: 0 nothing, 1 a bit of the accumulator,

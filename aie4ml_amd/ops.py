@@ -406,11 +406,11 @@ class MlpLayerSpec:
 
 def mlp_runs_on_matrix_units(rows: int, x_pitch: int, layers: Sequence[Tuple[int, int]]) -> bool:
     """Whether a4g_mlp_i8 takes its large-batch form for this chain (``layers``: (K, N) per layer; ``x_pitch``: bytes
-    between input rows, 0 if unknown): from 4096 rows, weight fragments of 1 KiB per 32 x 32 block plus 128 bytes of
+    between input rows, 0 if unknown): from 512 rows, weight fragments of 1 KiB per 32 x 32 block plus 128 bytes of
     start values per 32 neurons within 128 KiB of LDS."""
     blocks = sum(((k + 31) // 32) * ((n + 31) // 32) for k, n in layers) + 1
     start = sum((n + 31) // 32 * 32 for _k, n in layers)
-    return rows >= 4096 and x_pitch >= 1 and blocks * 1024 + start * 4 + 32 <= 128 * 1024
+    return rows >= 512 and x_pitch >= 1 and blocks * 1024 + start * 4 + 32 <= 128 * 1024
 
 
 def mlp(x: torch.Tensor, layers: Sequence[MlpLayerSpec], rounding='floor', out: Optional[torch.Tensor] = None):

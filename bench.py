@@ -293,7 +293,7 @@ def prepare(wl, torch):
         cpu_fn = lambda: oracle.mlp(x, layers, 'positive_inf')  # noqa: E731
         cpu_work = work
         metric, unit = 'int8_mlp_samples_per_s', 'samples/s'
-        kernel = 'mlp_fused_kernel'
+        kernel = 'mlp_mfma_kernel'
     elif wl == 'c1_mlp_stream':
         # the same network on a stream of samples: what a trigger or a tagging farm asks of it (throughput, not latency)
         nb = 1 << 20

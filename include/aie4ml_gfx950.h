@@ -229,8 +229,8 @@ A4G_API int a4g_softmax_hccs_i8(const int8_t* x, void* out, int64_t rows, int64_
  * (templates/nnet_utils/dense_bias_relu/dense_bias_relu_graph.h:12-134).
  * `layers` is a HOST array. Limits: n_layers <= 8, every K and N <= 256, packed weights <= 96 KiB in
  * total; beyond them the call returns A4G_ERR_UNSUPPORTED and the caller runs layer by layer.
- * Two forms behind the one call, the same integers from both: batches below 4096 samples (a chain of
- * latencies) take dot-product instructions on 16 or 64 samples per workgroup; from 4096 samples the chain
+ * Two forms behind the one call, the same integers from both: batches below 512 samples (a chain of
+ * latencies) take dot-product instructions on 16 or 64 samples per workgroup; from 512 samples the chain
  * runs on the matrix units, 32 samples per wave, the activations in registers from the first layer to the
  * last (rows at any address and pitch; fastest with ldx and X multiples of 16 bytes). A single narrow layer on a long batch (n_layers == 1, say
  * a million rows of 16 -> 64) is served by that form at the speed of its rows' traffic, 1.5 to 2 times
