@@ -162,7 +162,12 @@ __global__ __launch_bounds__(WR_NT, 2) void gemm_wreg_kernel(GemmArgs g, int hal
                 for (int i = 0; i < 4; ++i) {
                     if (i < NRB) {
                         v4i a_op = af[kk % AFS][i];
-                        if (A_UNSIGNED) a_op ^= static_cast<int>(0x80808080u);  // uint8 -> int8; 128 * colsum is in the start value
+                        // uint8 -> int8; 128 * colsum is in the start value. The chunks of the last tile that lie past K were
+                        // fetched as zeros and stay zeros (biased they would count as -128 against whatever the weight tile
+                        // holds there).
+                        // (Not in the six-tile form, which has no register left for the mask: there K is 768.)
+                        if (A_UNSIGNED)
+                            a_op ^= (NKT == 6 || kt < NKT - 1 || kk * 32 + half * 16 < k_last) ? static_cast<int>(0x80808080u) : 0;
                         acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bw[kt * 4 + kk], a_op, acc[i], 0, 0, 0);
                     }
                     // the fragment of the next K step follows the MFMA that read this one: steps 1..3 from this tile, step
@@ -272,9 +277,8 @@ hipError_t launch_wreg_nkt(const GemmArgs& g, int halves_m, int wgs_per_cb, int 
 // 16-column pieces, and operands small enough for 32-bit buffer offsets. Measured faster than the tiled kernel at every
 // size tried, from one row to 8192 x 3072.
 bool wreg_applicable(const GemmArgs& g) {
-    // K a multiple of 128, or of 16 with signed activations (a uint8 operand is biased by 128 in the registers, which
-    // would turn the zeros of a partial last tile into -128)
-    return g.M > 0 && (g.K % 128 == 0 || (g.K % 16 == 0 && !g.a_unsigned)) && g.K >= 16 && g.K <= 768 && g.N % 16 == 0 && g.N >= 16 &&
+    // K in whole 128-byte tiles, or ending inside the last one on a multiple of 16 (unsigned activations: up to 640)
+    return g.M > 0 && g.K % 16 == 0 && g.K >= 16 && g.K <= 768 && (g.K % 128 == 0 || !g.a_unsigned || g.K <= 640) && g.N % 16 == 0 && g.N >= 16 &&
            (g.out_kind == A4G_I8 || g.out_kind == A4G_U8) && g.lda % 16 == 0 && g.ldb % 16 == 0 && g.ldc % 16 == 0 && aligned16(g.A) &&
            aligned16(g.Bt) && aligned16(g.C) && (static_cast<int64_t>(g.M) + 2 * WR_BM) * g.lda < (int64_t{1} << 31) &&
            (static_cast<int64_t>(g.N) + WR_BN) * g.ldb < (int64_t{1} << 31) && (g.N + WR_BN - 1) / WR_BN <= 65536;

@@ -163,8 +163,9 @@ def test_dense_narrow_layer_on_a_long_batch(ops, oracle, shape, mode):
 @pytest.mark.parametrize('mode', ['conv_even', 'symmetric_inf'])
 def test_dense_reduction_that_ends_inside_a_tile(ops, oracle, shape, mode):
     """K a multiple of 16 but not of 128 (192 inputs of a small vision transformer): the weights-in-registers kernel
-    takes it with signed activations, fetching nothing for the part of the last 128-byte tile past K; unsigned
-    activations (biased in registers) keep the tiled kernel. Per-channel and single shifts, every output kind it has."""
+    takes it, fetching nothing for the part of the last 128-byte tile past K (unsigned activations are biased in
+    registers: the chunks past K are left out of that, up to K = 640; 752 keeps the tiled kernel). Per-channel and single
+    shifts, every output kind it has."""
     M, K, N = shape
     run_dense(ops, oracle, M, K, N, mode, seed=M + K + N)
     run_dense(ops, oracle, M, K, N, mode, per_channel=False, relu=False, out='uint8', seed=M + K + N + 1)
