@@ -216,6 +216,7 @@ struct MlpMfmaArgs {
     int nfrag, nstart;
     int y_vec;        // rows of Y can be stored as 16-byte pieces
     int y_packed;     // at most 32 outputs in rows without gaps, Y 4-byte aligned: the tile store
+    int y_magic;      // ceil(65536 / N): (j * y_magic) >> 16 == j / N for every j < 32 N
 };
 
 constexpr int64_t MLP_MFMA_MIN_BATCH = 512;
@@ -258,7 +259,7 @@ __global__ __launch_bounds__(1024) void mlp_mfma_kernel(MlpMfmaArgs a) {
 #pragma unroll
             for (int b = 0; b < 4; ++b) {
                 const int j = min((sl * 64 + lane) * 4 + b, 32 * last_n - 1);
-                const int r = j / last_n;
+                const int r = (j * a.y_magic) >> 16;  // j / last_n for j < 1024 (checked on the host for this N)
                 at[b] = static_cast<unsigned>(r * 32 + (j - r * last_n));
             }
             tsrc[sl] = at[0] | (at[1] << 10) | (at[2] << 20);
@@ -648,6 +649,9 @@ extern "C" int a4g_mlp_i8(const a4g_mlp_layer* layers, int n_layers, const void*
             f.nstart = nstart;
             f.y_vec = lastl.out_kind != A4G_I16 && lastl.N % 16 == 0 && ldy % 16 == 0 && aligned16(Y);
             f.y_packed = !f.y_vec && lastl.N <= 32 && ldy == lastl.N && reinterpret_cast<uintptr_t>(Y) % 4 == 0;
+            f.y_magic = (65536 + lastl.N - 1) / lastl.N;
+            for (int j = 0; f.y_packed && j < 32 * lastl.N; ++j)
+                if (((j * f.y_magic) >> 16) != j / lastl.N) f.y_packed = 0;  // (never, for N <= 32)
             int widest = 0;
             for (int l = 0; l < n_layers; ++l) widest = std::max(widest, std::max(f.layer[l].Kb, f.layer[l].Nb));
             const int bit_kind = fast_round_kind(fr1);
