@@ -31,7 +31,8 @@ constexpr int WR_LDS = WR_NST * WR_STAGE + WregParams::BYTES;
 // One workgroup: one block of 128 output columns and a run of rows in 64-row halves, [h0, h1) of the `halves_m` halves
 // of the matrix; the `wgs_per_cb` workgroups of a column block share its rows as evenly as halves allow. Rows are
 // processed 128 at a time; a run of an odd number of halves ends with a step of 64 rows.
-template <int NKT, bool A_UNSIGNED>
+// PARTIAL: the reduction ends inside its last 128-byte tile (K a multiple of 16 only).
+template <int NKT, bool A_UNSIGNED, bool PARTIAL = false>
 __global__ __launch_bounds__(WR_NT, 2) void gemm_wreg_kernel(GemmArgs g, int halves_m, int wgs_per_cb, int a_bytes, int w_bytes) {
     constexpr int NKS = NKT * 4;  // K steps of 32 bytes
     extern __shared__ __attribute__((aligned(16))) int8_t wr_smem[];
@@ -70,7 +71,7 @@ __global__ __launch_bounds__(WR_NT, 2) void gemm_wreg_kernel(GemmArgs g, int hal
     // lies past K fetch nothing (an offset of the buffer's size: zeros), and zero activations make whatever the weight
     // tile holds there (the next weight row's first bytes) count for nothing.
     const int k_last = g.K - (NKT - 1) * WR_BK;  // bytes of the last tile that exist, 16 .. 128
-    const int va0_last = sw0 < k_last ? va0 : a_bytes, va1_last = (sw0 ^ 64) < k_last ? va1 : a_bytes;
+    const int va0_last = (!PARTIAL || sw0 < k_last) ? va0 : a_bytes, va1_last = (!PARTIAL || (sw0 ^ 64) < k_last) ? va1 : a_bytes;
     const auto rsrc_a = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(g.A), 0, a_bytes, 0x00020000);
     const auto rsrc_w = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(g.Bt), 0, w_bytes, 0x00020000);
 
@@ -94,7 +95,7 @@ __global__ __launch_bounds__(WR_NT, 2) void gemm_wreg_kernel(GemmArgs g, int hal
     // activation tile (step, kt) of the run; nothing is fetched past its end (the lower 64 rows of a short last step)
     auto issue_a = [&](int step, int kt, int st) {
         const bool live = step < steps && !(short_last && step == steps - 1 && wave >= 2);
-        const bool last_kt = kt == NKT - 1;
+        const bool last_kt = PARTIAL && kt == NKT - 1;
         issue(rsrc_a, last_kt ? va0_last : va0, last_kt ? va1_last : va1, lda, live ? (m0 + step * WR_BM) * lda + kt * WR_BK : a_bytes, st);
     };
     // ring position r: the NKT weight tiles of the column block, then the activation tiles
@@ -167,7 +168,7 @@ __global__ __launch_bounds__(WR_NT, 2) void gemm_wreg_kernel(GemmArgs g, int hal
                         // holds there).
                         // (Not in the six-tile form, which has no register left for the mask: there K is 768.)
                         if (A_UNSIGNED)
-                            a_op ^= (NKT == 6 || kt < NKT - 1 || kk * 32 + half * 16 < k_last) ? static_cast<int>(0x80808080u) : 0;
+                            a_op ^= (!PARTIAL || NKT == 6 || kt < NKT - 1 || kk * 32 + half * 16 < k_last) ? static_cast<int>(0x80808080u) : 0;
                         acc[i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bw[kt * 4 + kk], a_op, acc[i], 0, 0, 0);
                     }
                     // the fragment of the next K step follows the MFMA that read this one: steps 1..3 from this tile, step
@@ -255,9 +256,9 @@ __global__ __launch_bounds__(WR_NT, 2) void gemm_wreg_kernel(GemmArgs g, int hal
     A4G_STAMP(5);
 }
 
-template <int NKT, bool A_UNSIGNED>
+template <int NKT, bool A_UNSIGNED, bool PARTIAL>
 hipError_t launch_wreg_kernel(const GemmArgs& g, int halves_m, int wgs_per_cb, int cbs, int a_bytes, int w_bytes, hipStream_t stream) {
-    auto kern = gemm_wreg_kernel<NKT, A_UNSIGNED>;
+    auto kern = gemm_wreg_kernel<NKT, A_UNSIGNED, PARTIAL>;
     static bool attr_set = false;  // benign race: the attribute is idempotent
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, WR_LDS);
@@ -269,8 +270,13 @@ hipError_t launch_wreg_kernel(const GemmArgs& g, int halves_m, int wgs_per_cb, i
 }
 template <int NKT>
 hipError_t launch_wreg_nkt(const GemmArgs& g, int halves_m, int wgs_per_cb, int cbs, int a_bytes, int w_bytes, hipStream_t stream) {
-    return g.a_unsigned ? launch_wreg_kernel<NKT, true>(g, halves_m, wgs_per_cb, cbs, a_bytes, w_bytes, stream)
-                        : launch_wreg_kernel<NKT, false>(g, halves_m, wgs_per_cb, cbs, a_bytes, w_bytes, stream);
+    if (g.K % 128 == 0)
+        return g.a_unsigned ? launch_wreg_kernel<NKT, true, false>(g, halves_m, wgs_per_cb, cbs, a_bytes, w_bytes, stream)
+                            : launch_wreg_kernel<NKT, false, false>(g, halves_m, wgs_per_cb, cbs, a_bytes, w_bytes, stream);
+    if constexpr (NKT < 6) {
+        if (g.a_unsigned) return launch_wreg_kernel<NKT, true, true>(g, halves_m, wgs_per_cb, cbs, a_bytes, w_bytes, stream);
+    }
+    return launch_wreg_kernel<NKT, false, true>(g, halves_m, wgs_per_cb, cbs, a_bytes, w_bytes, stream);
 }
 
 // Reductions of one to six whole 128-byte tiles, one-byte outputs, 16-byte aligned rows on both sides, widths in whole
