@@ -202,18 +202,20 @@ def dense(x: torch.Tensor, p: PackedDense, rounding='floor', relu: bool = False,
 
 def _narrow_dense_as_chain(x2: torch.Tensor, p: PackedDense, out_kind: int, rows: int) -> bool:
     """Dense layers that a4g_mlp_i8 with one layer runs faster than a4g_dense_i8: up to 256 wide both ways, one shift,
-    8-bit result, a batch on which a4g_mlp_i8 uses the matrix units, and either at most 64 outputs or a shape the
-    weights-in-registers GEMM does not take (that one wants K and N in multiples of 16, signed activations when K is not
-    a multiple of 128, and 16-byte aligned rows). Measured, chain / GEMM in us: 1 Mi x 16 -> 64 23.8 / 38.1 (151 on the
-    tiled kernel), 1 Mi x 64 -> 32 19.4 / 36.2, 1 Mi x 16 -> 16 15.4 / 35.3, 65 536 x 64 -> 64 5.3 / 6.6; but 50 432 x
-    192 -> 192 14.0 / 10.7, 262 144 x 48 -> 256 32.9 / 24.6, 32 768 x 240 -> 240 13.8 / 8.3."""
-    if not (p.shift0 is not None and p.wt_lo is None and p.K <= 256 and p.N <= 256 and p.K % 128 != 0 and out_kind in (0, 1)
+    8-bit result, a batch on which a4g_mlp_i8 uses the matrix units, and either a shape the weights-in-registers GEMM
+    does not take (that one wants K and N in multiples of 16 and 16-byte aligned rows: a classifier's 10 outputs are not),
+    or at most 64 outputs behind a reduction that ends inside a 128-byte tile. Measured, chain / GEMM in us:
+    1 Mi x 16 -> 64 23.8 / 38.1 (151 on the tiled kernel), 1 Mi x 64 -> 32 19.4 / 36.2, 1 Mi x 16 -> 16 15.4 / 35.3,
+    65 536 x 64 -> 64 5.3 / 6.6, 65 536 x 128 -> 10 6.3 / 10.6, 262 144 x 128 -> 8 11.3 / 31.4; but 50 432 x 192 -> 192
+    14.0 / 10.7, 262 144 x 48 -> 256 32.9 / 24.6, 32 768 x 240 -> 240 13.8 / 8.3, and level at 128 or 256 inputs with 16 to
+    64 outputs."""
+    if not (p.shift0 is not None and p.wt_lo is None and p.K <= 256 and p.N <= 256 and out_kind in (0, 1)
             and x2.dtype in (torch.int8, torch.uint8) and x2.stride(1) == 1
             and mlp_runs_on_matrix_units(rows, int(x2.stride(0)), [(p.K, p.N)])):
         return False
-    gemm_takes_it = (p.K % 16 == 0 and p.N % 16 == 0 and x2.dtype == torch.int8 and int(x2.stride(0)) % 16 == 0
-                     and x2.data_ptr() % 16 == 0)
-    return p.N <= 64 or not gemm_takes_it
+    gemm_takes_it = (p.K % 16 == 0 and p.N % 16 == 0 and int(x2.stride(0)) % 16 == 0 and x2.data_ptr() % 16 == 0
+                     and (p.K % 128 == 0 or x2.dtype == torch.int8 or p.K <= 640))
+    return not gemm_takes_it or (p.N <= 64 and p.K % 128 != 0)
 
 
 def matmul(a: torch.Tensor, b: torch.Tensor, shift: int, rounding='floor', trans_b: bool = False, out_kind='int8',

@@ -143,7 +143,7 @@ def test_dense_shapes_mfma_path(ops, oracle, shape):
 
 
 @pytest.mark.parametrize('shape', [(5000, 16, 64), (4096, 64, 32), (4100, 32, 5), (6000, 48, 200), (4500, 192, 256),
-                                   (4097, 80, 33), (5000, 20, 64), (5000, 16, 300)])
+                                   (4097, 80, 33), (5000, 20, 64), (5000, 16, 300), (5000, 128, 10), (600, 256, 3)])
 @pytest.mark.parametrize('mode', ['conv_even', 'positive_inf', 'symmetric_zero'])
 def test_dense_narrow_layer_on_a_long_batch(ops, oracle, shape, mode):
     """Narrow layers with one shift on 4096 rows or more go to the kernel that walks a chain of layers (a chain of one):
