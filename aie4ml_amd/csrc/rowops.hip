@@ -44,6 +44,39 @@ __global__ __launch_bounds__(256) void add_sat8_kernel(const v4i* __restrict__ a
     }
 }
 
+// Any shift, 8- and 16-bit kinds: 16 bytes per lane and turn, each element widened, added, rounded (the sum of two
+// operands and the rounding constant stay far below 2^31, so the short form of the rounding applies), clamped and packed
+// again. KIND: A4G_I8, A4G_U8 or A4G_I16.
+template <int KIND>
+__global__ __launch_bounds__(256) void add_vec_kernel(const v4i* __restrict__ a, const v4i* __restrict__ b, v4i* __restrict__ out,
+                                                       int64_t nvec, FastRound fr, int lo, int hi) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec; i += stride) {
+        const v4i va = __builtin_nontemporal_load(a + i);
+        const v4i vb = __builtin_nontemporal_load(b + i);
+        v4i r;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const unsigned wa = static_cast<unsigned>(va[j]), wb = static_cast<unsigned>(vb[j]);
+            if (KIND == A4G_I16) {
+                const int s0 = static_cast<int16_t>(wa) + static_cast<int16_t>(wb);
+                const int s1 = (va[j] >> 16) + (vb[j] >> 16);
+                r[j] = static_cast<int>(pack2_halves(clamp_i(fast_round(s0, fr), lo, hi), clamp_i(fast_round(s1, fr), lo, hi)));
+            } else {
+                int y[4];
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const int ea = KIND == A4G_I8 ? sext8(wa, t) : static_cast<int>((wa >> (8 * t)) & 0xffu);
+                    const int eb = KIND == A4G_I8 ? sext8(wb, t) : static_cast<int>((wb >> (8 * t)) & 0xffu);
+                    y[t] = clamp_i(fast_round(ea + eb, fr), lo, hi);
+                }
+                r[j] = static_cast<int>(pack4_bytes(y[0], y[1], y[2], y[3]));
+            }
+        }
+        __builtin_nontemporal_store(r, out + i);
+    }
+}
+
 __global__ __launch_bounds__(256) void add_generic_kernel(const void* __restrict__ a, const void* __restrict__ b,
                                                            void* __restrict__ out, int64_t first, int64_t n, int kind,
                                                            int shift, int mode) {
@@ -88,6 +121,19 @@ extern "C" int a4g_add(const void* a, const void* b, void* out, int64_t n, int k
             add_sat8_kernel<false><<<grid, 256, 0, stream>>>(static_cast<const v4i*>(a), static_cast<const v4i*>(b),
                                                              static_cast<v4i*>(out), nvec);
         done = nvec * 16;
+    } else if (aligned16(a) && aligned16(b) && aligned16(out) && n * (kind == A4G_I16 ? 2 : 1) >= 16) {
+        const int per_vec = kind == A4G_I16 ? 8 : 16;
+        const int64_t nvec = n / per_vec;
+        const int grid = grid_for(nvec, 256, 256 * 16);
+        const FastRound fr = make_fast_round(round_mode, shift);
+        const int lo = kind == A4G_I8 ? -128 : (kind == A4G_I16 ? -32768 : 0), hi = kind == A4G_I8 ? 127 : (kind == A4G_I16 ? 32767 : 255);
+        const v4i* va = static_cast<const v4i*>(a);
+        const v4i* vb = static_cast<const v4i*>(b);
+        v4i* vo = static_cast<v4i*>(out);
+        if (kind == A4G_I8) add_vec_kernel<A4G_I8><<<grid, 256, 0, stream>>>(va, vb, vo, nvec, fr, lo, hi);
+        else if (kind == A4G_U8) add_vec_kernel<A4G_U8><<<grid, 256, 0, stream>>>(va, vb, vo, nvec, fr, lo, hi);
+        else add_vec_kernel<A4G_I16><<<grid, 256, 0, stream>>>(va, vb, vo, nvec, fr, lo, hi);
+        done = nvec * per_vec;
     }
     if (done < n) {
         const int grid = grid_for(n - done, 256, 256 * 8);

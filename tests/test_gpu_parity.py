@@ -75,6 +75,24 @@ def test_add_shift_and_modes(ops, oracle, mode):
     assert np.array_equal(host(ops.add(dev(a16), dev(b16), 0, mode)), oracle.add(a16, b16, 0, mode))
 
 
+@pytest.mark.parametrize('mode', MODES)
+def test_add_every_pair_at_every_shift(ops, oracle, mode):
+    """All 65 536 pairs of 8-bit operands, signed and unsigned, at shifts 0 to 9 (the 16-byte-per-lane kernel), and 16-bit
+    operands at the ends of their range at shifts 0 to 15."""
+    a = np.arange(-128, 128, dtype=np.int8).repeat(256)
+    b = np.tile(np.arange(-128, 128, dtype=np.int8), 256)
+    au, bu = a.view(np.uint8), b.view(np.uint8)
+    for shift in range(0, 10):
+        assert np.array_equal(host(ops.add(dev(a), dev(b), shift, mode)), oracle.add(a, b, shift, mode)), (mode, shift)
+        assert np.array_equal(host(ops.add(dev(au), dev(bu), shift, mode)), oracle.add(au, bu, shift, mode)), (mode, shift)
+    r = rng(5)
+    edge = np.array([-32768, -32767, -16385, -16384, -3, -2, -1, 0, 1, 2, 3, 16383, 16384, 32766, 32767], dtype=np.int16)
+    a16 = np.concatenate([edge.repeat(len(edge)), r.integers(-32768, 32768, 4001).astype(np.int16)])
+    b16 = np.concatenate([np.tile(edge, len(edge)), r.integers(-32768, 32768, 4001).astype(np.int16)])
+    for shift in range(0, 16):
+        assert np.array_equal(host(ops.add(dev(a16), dev(b16), shift, mode)), oracle.add(a16, b16, shift, mode)), (mode, shift)
+
+
 def test_add_unaligned_views(ops, oracle):
     r = rng(4)
     a = r.integers(-128, 128, 10007).astype(np.int8)
