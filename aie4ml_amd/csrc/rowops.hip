@@ -544,7 +544,10 @@ static int layernorm_dispatch(const int8_t* a, const int8_t* b, int add_shift, i
     launched = launch_ln_rows<L, NCH>(bit_kind, fr, fuse, grid_for(nrows, 4 * (64 / L), max_grid), lds, stream, ac, bc,  \
                                       gamma, beta, sc, oc, nrows, (int)cols, log2c, eps_q0, rg, ro, lf)
             hipError_t launched = hipSuccess;
-            if (nchunks <= 8) A4G_LN_GO(4, 2);
+            if (nchunks <= 1) A4G_LN_GO(1, 1);
+            else if (nchunks <= 2) A4G_LN_GO(2, 1);
+            else if (nchunks <= 4) A4G_LN_GO(4, 1);
+            else if (nchunks <= 8) A4G_LN_GO(4, 2);
             else if (nchunks <= 12) A4G_LN_GO(4, 3);
             else if (nchunks <= 16) A4G_LN_GO(8, 2);
             else if (nchunks <= 24) A4G_LN_GO(8, 3);
