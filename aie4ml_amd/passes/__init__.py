@@ -436,7 +436,8 @@ class PlanGpuFusion(AIEPass):
                 and cfg.n_in <= self.ROWLN_MAX_K and cfg.n_out >= 384)
 
     # ---- attention -------------------------------------------------------------------------------------
-    ATTN_MAX_KEYS = {32: 512, 64: 512, 128: 256}  # head dimension -> keys the fused kernel takes
+    # head dimension -> keys the fused kernel takes (16, 48, 80, 96, 112 run padded to 32, 64, 128)
+    ATTN_MAX_KEYS = {16: 512, 32: 512, 48: 512, 64: 512, 80: 256, 96: 256, 112: 256, 128: 256}
     ATTN_MAX_SHIFT = 24
 
     def _plan_attention(self, graph, execution, outputs):

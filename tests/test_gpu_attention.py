@@ -102,6 +102,20 @@ def test_attention_head_dimensions_32_and_128(oracle, d, sk, kind):
         np.testing.assert_array_equal(got, reference(oracle, q, k, v, lshift, lmode, sm, 7, 'conv_even'))
 
 
+@pytest.mark.parametrize('d,sk', [(16, 64), (16, 100), (48, 128), (80, 96), (96, 256), (112, 33)])
+def test_attention_head_dimensions_between_the_kernels(oracle, d, sk):
+    """Head dimensions 16, 48, 80, 96, 112 run padded with zero columns to the next dimension that has a kernel; also into
+    a strided output (the heads of a concatenated result)."""
+    q, k, v = qkv(9000 + d + sk, (2, 3, sk, d), (2, 3, sk, d), sigma=24.0)
+    sm = {'kind': 'exp', 'exp_kq': 23}
+    want = reference(oracle, q, k, v, 6, 'conv_even', sm, 7, 'symmetric_inf')
+    got = ops.attention(dev(q), dev(k), dev(v), 6, 'conv_even', sm, 7, 'symmetric_inf').cpu().numpy()
+    np.testing.assert_array_equal(got, want)
+    out = torch.zeros((2, sk, 3 * d), dtype=torch.int8, device='cuda')
+    ops.attention(dev(q), dev(k), dev(v), 6, 'conv_even', sm, 7, 'symmetric_inf', out=out.unflatten(-1, (3, d)).permute(0, 2, 1, 3))
+    np.testing.assert_array_equal(out.cpu().numpy().reshape(2, sk, 3, d).transpose(0, 2, 1, 3), want)
+
+
 def test_attention_masked_keys_do_not_leak(oracle):
     """The rows behind the last key are other tensors' memory: whatever they hold, the result is that of the keys that
     exist (K rows past the end alias the last row inside the kernel, V rows past the end are not read)."""
@@ -195,7 +209,7 @@ def test_attention_on_head_slices_of_a_packed_projection(oracle):
 
 
 def test_attention_uncovered_shapes_and_bad_parameters():
-    q = torch.zeros((2, 64, 96), dtype=torch.int8, device='cuda')
+    q = torch.zeros((2, 64, 40), dtype=torch.int8, device='cuda')
     with pytest.raises(NotImplementedError, match='fused path covers head_dim 64'):
         ops.attention(q, q, q, 6, 'floor', {'kind': 'exp', 'exp_kq': 23}, 7, 'floor')
     q = torch.zeros((2, 544, 64), dtype=torch.int8, device='cuda')
