@@ -27,6 +27,7 @@ struct AttnArgs {
     int64_t v_sb, v_sh, v_ss;
     int64_t o_sb, o_sh, o_ss;
     int heads, sq;
+    int d16;    // head dimension 16 on the 32-wide kernel: the upper halves of its fragments do not exist
     int sk;     // key / value rows that exist (the ragged form; the kernel's tiles cover the next power of two of 32s)
     int items;  // (batch, head, block of query rows) triples in all
     FastRound lr, orr;  // logits and output requantisation
@@ -104,6 +105,10 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
     }
     const int lane = tid & 63, wave = tid >> 6;
     const int m = lane & 31, half = lane >> 5;
+    // Head dimension 16 on the 32-wide kernel (DT == 1 only): the lanes of the upper half fetch the lower half again (no
+    // access leaves the row), multiply with zero queries, see zero V columns and store nothing.
+    const bool upper_missing = DT == 1 && a.d16 && half == 1;
+    const int hoff = upper_missing ? 0 : half * 16;
     const int n0 = (tid % (D / 4)) * 4;  // THREADS % (D/4) == 0: a thread keeps its four columns
     const int8_t* Kp;
     int8_t* Op;
@@ -125,8 +130,9 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
         const int rowc = row_ok ? row : a.sq - 1;
 #pragma unroll
         for (int ks = 0; ks < DT; ++ks) {
-            qf[ks] = *reinterpret_cast<const v4i*>(Qp + rowc * a.q_ss + ks * 32 + half * 16);
-            kf[0][ks] = *reinterpret_cast<const v4i*>(Kp + (RAGGED ? min(m, a.sk - 1) : m) * a.k_ss + ks * 32 + half * 16);
+            qf[ks] = *reinterpret_cast<const v4i*>(Qp + rowc * a.q_ss + ks * 32 + hoff);
+            kf[0][ks] = *reinterpret_cast<const v4i*>(Kp + (RAGGED ? min(m, a.sk - 1) : m) * a.k_ss + ks * 32 + hoff);
+            if (DT == 1 && upper_missing) qf[ks] = v4i{0, 0, 0, 0};  // zero queries there: whatever K holds counts nothing
         }
 #pragma unroll
         for (int it = 0; it < VB; ++it) {
@@ -134,7 +140,8 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
             const int k0 = (blk / (D / 4)) * 4;
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                av[it][i] = blk < NB && (!RAGGED || k0 + i < a.sk) ? *reinterpret_cast<const unsigned*>(Vp + (k0 + i) * a.v_ss + n0) : 0u;
+                av[it][i] = blk < NB && (!RAGGED || k0 + i < a.sk) && !(DT == 1 && a.d16 && n0 >= 16)
+                                ? *reinterpret_cast<const unsigned*>(Vp + (k0 + i) * a.v_ss + n0) : 0u;
         }
     };
     // requested before anything is done with LDS, so that (first item) building the score table hides the latency
@@ -196,7 +203,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
 #pragma unroll
             for (int ks = 0; ks < DT; ++ks)
                 kf[(t + 1) & 1][ks] = *reinterpret_cast<const v4i*>(
-                    Kp + (RAGGED ? min((t + 1) * 32 + m, a.sk - 1) : (t + 1) * 32 + m) * a.k_ss + ks * 32 + half * 16);
+                    Kp + (RAGGED ? min((t + 1) * 32 + m, a.sk - 1) : (t + 1) * 32 + m) * a.k_ss + ks * 32 + hoff);
         }
         v16i acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
@@ -352,7 +359,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
         const auto s13 = __builtin_amdgcn_permlane32_swap(ow[1], ow[3], false, false);
         const v4i o = {static_cast<int>(s02[0]), static_cast<int>(s02[1]), static_cast<int>(s13[0]),
                        static_cast<int>(s13[1])};
-        if (row_ok) *reinterpret_cast<v4i*>(Op + row * a.o_ss + 32 * u + 16 * half) = o;
+        if (row_ok && !(DT == 1 && upper_missing)) *reinterpret_cast<v4i*>(Op + row * a.o_ss + 32 * u + 16 * half) = o;
     }
     }  // items
 }
@@ -459,8 +466,8 @@ extern "C" int a4g_attention_i8(const int8_t* Q, const int8_t* K, const int8_t* 
         if (int rc = make_hccs_params(who, sk, hccs_B, hccs_S, hccs_Dmax, inv_shift, use_clb, A4G_U8, &a.sm, &noclamp))
             return rc;
     }
-    A4G_REQUIRE((d == 64 && sk <= 512) || (d == 32 && sk <= 512) || (d == 128 && sk <= 256), A4G_ERR_UNSUPPORTED,
-                "%s: fused path covers head_dim 64 and 32 with up to 512 keys and head_dim 128 with up to 256, got d=%lld sk=%lld",
+    A4G_REQUIRE(((d == 64 || d == 32 || d == 16) && sk <= 512) || (d == 128 && sk <= 256), A4G_ERR_UNSUPPORTED,
+                "%s: fused path covers head_dim 64, 32 and 16 with up to 512 keys and head_dim 128 with up to 256, got d=%lld sk=%lld",
                 who, (long long)d, (long long)sk);
     int nt = 1;  // tiles of 32 keys the kernel is instantiated for: the next power of two
     while (nt * 32 < sk) nt *= 2;
@@ -481,6 +488,7 @@ extern "C" int a4g_attention_i8(const int8_t* Q, const int8_t* K, const int8_t* 
     a.heads = static_cast<int>(heads);
     a.sq = static_cast<int>(sq);
     a.sk = static_cast<int>(sk);
+    a.d16 = d == 16;
     a.lr = make_fast_round(logit_round_mode, logit_shift);
     a.orr = make_fast_round(out_round_mode, out_shift);
     a.noclamp = noclamp;
@@ -500,7 +508,7 @@ extern "C" int a4g_attention_i8(const int8_t* Q, const int8_t* K, const int8_t* 
         return check_hip(hipGetLastError(), who);
     }
     const int no_kernel = d == 64 ? launch_attention<2>(nt, grid, grid8, stream, a)
-                          : (d == 32 ? launch_attention<1>(nt, grid, 0, stream, a) : launch_attention<4>(nt, grid, 0, stream, a));
+                          : (d <= 32 ? launch_attention<1>(nt, grid, 0, stream, a) : launch_attention<4>(nt, grid, 0, stream, a));
     if (no_kernel) return fail(A4G_ERR_UNSUPPORTED, "%s: no kernel for sk=%lld", who, (long long)sk);
     return check_hip(hipGetLastError(), who);
 }

@@ -454,7 +454,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, logit_shift: in
     {'kind': 'exp', 'exp_kq': .., 'inv_shift': 15} or {'kind': 'hccs', 'B': .., 'S': .., 'Dmax': .., 'inv_shift': 15,
     'use_clb': False}. Bit-identical to matmul(trans_b) -> softmax_* -> matmul. Raises NotImplementedError for
     shapes the fused kernel does not cover (head_dim not a multiple of 16 or above 128, more than 512 keys - 256 from
-    head_dim 80 on -, unaligned views). Head dimensions 16, 48, 80, 96 and 112 are padded with zero columns to 32, 64 and 128.
+    head_dim 80 on -, unaligned views). Head dimension 16 runs on the 32-wide kernel; 48, 80, 96 and 112 are padded with zero columns to 64
+    and 128.
     """
     for name, t in (('q', q), ('k', k), ('v', v)):
         _dev(t, name)
@@ -464,11 +465,10 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, logit_shift: in
         raise ValueError(f'attention: incompatible shapes {tuple(q.shape)}, {tuple(k.shape)}, {tuple(v.shape)}')
     lead = tuple(q.shape[:-2])
     sq, d, sk = int(q.shape[-2]), int(q.shape[-1]), int(k.shape[-2])
-    if d not in (32, 64, 128) and d % 16 == 0 and d < 128:
-        # head dimensions 16, 48, 80, 96, 112: zero columns up to the next dimension the kernel has change neither Q K^T nor
-        # the columns of P V that exist (three small copies and one back, against three launches through HBM:
-        # 4096 heads of 64 x 64 x 16 50 us against 143 us)
-        pad = (32 if d < 32 else (64 if d < 64 else 128)) - d
+    if d not in (16, 32, 64, 128) and d % 16 == 0 and d < 128:
+        # head dimensions 48, 80, 96, 112: zero columns up to the next dimension the kernel has change neither Q K^T nor
+        # the columns of P V that exist (three small copies and one back, against three launches through HBM)
+        pad = (64 if d < 64 else 128) - d
         padded = attention(torch.nn.functional.pad(q, (0, pad)), torch.nn.functional.pad(k, (0, pad)),
                            torch.nn.functional.pad(v, (0, pad)), logit_shift, logit_rounding, softmax, out_shift, out_rounding)
         if out is None:

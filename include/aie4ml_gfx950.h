@@ -261,7 +261,7 @@ A4G_API int a4g_mlp_i8(const a4g_mlp_layer* layers, int n_layers, const void* X,
  *   slices of a packed QKV projection and a concatenated output need no copies.
  *   softmax_kind 0: accurate exp (exp_kq, inv_shift); 1: HCCS (hccs_B, hccs_S, hccs_Dmax, inv_shift,
  *   use_clb), same parameter rules as the stand-alone entries; probabilities are uint8.
- * Covered shapes: d == 64 or 32 with 1 <= sk <= 512, d == 128 with 1 <= sk <= 256 (any count: key counts off
+ * Covered shapes: d == 64, 32 or 16 with 1 <= sk <= 512, d == 128 with 1 <= sk <= 256 (any count: key counts off
  * the 32-grid, e.g. 197 tokens, run the kernel of the next power of two with the missing keys masked out), any
  * sq, pointers and strides multiples of 16 bytes; anything else returns A4G_ERR_UNSUPPORTED and the caller runs the three operators separately. */
 A4G_API int a4g_attention_i8(const int8_t* Q, const int8_t* K, const int8_t* V, int8_t* O, int64_t batch, int64_t heads,

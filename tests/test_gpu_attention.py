@@ -84,10 +84,11 @@ def test_attention_key_count_off_the_tile_grid(oracle, sk, kind):
         np.testing.assert_array_equal(got, reference(oracle, q, k, v, 6, lmode, sm, 7, 'conv_even'))
 
 
-@pytest.mark.parametrize('d,sk', [(32, 32), (32, 128), (32, 512), (32, 197), (128, 64), (128, 256), (128, 100)])
+@pytest.mark.parametrize('d,sk', [(32, 32), (32, 128), (32, 512), (32, 197), (128, 64), (128, 256), (128, 100), (16, 32),
+                                  (16, 128), (16, 512), (16, 77)])
 @pytest.mark.parametrize('kind', ['exp', 'hccs'])
-def test_attention_head_dimensions_32_and_128(oracle, d, sk, kind):
-    """One and four MFMA K steps per key tile instead of two; sequence lengths on and off the tile grid; a query count
+def test_attention_head_dimensions_16_32_and_128(oracle, d, sk, kind):
+    """One and four MFMA K steps per key tile instead of two (16: one, its upper half masked); sequence lengths on and off the tile grid; a query count
     of its own; both logit requantisations."""
     for sq in (sk, 45):
         q, k, v = qkv(7000 + d + sk + sq, (2, 3, sq, d), (2, 3, sk, d), sigma=24.0 if d <= 64 else 16.0)

@@ -170,9 +170,9 @@ def test_attention_random_case(ops, oracle, seed):
 
 @pytest.mark.parametrize('seed', range(24 + EXTRA // 4))
 def test_attention_any_key_count_and_head_dimension_random_case(ops, oracle, seed):
-    """Head dimensions 32, 64 and 128, any number of keys the fused kernel takes for them, any number of queries."""
+    """Head dimensions 16, 32, 64 and 128, any number of keys the fused kernel takes for them, any number of queries."""
     r = np.random.default_rng(4500 + seed)
-    d = int(r.choice([32, 64, 128]))
+    d = int(r.choice([16, 32, 64, 128]))
     sk = int(r.integers(1, (256 if d == 128 else 512) + 1))
     if r.random() < 0.3:
         sk = int(r.choice([31, 33, 64, 100, 197, 255, 256]))
