@@ -72,6 +72,8 @@ SIGNATURES = {
     'a4g_softmax_exp_i8': (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _i32, _vp]),
     'a4g_softmax_hccs_i8': (_i32, [_vp, _vp, _i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _vp]),
     'a4g_mlp_i8': (_i32, [ctypes.POINTER(MlpLayer), _i32, _vp, _i32, _i64, _vp, _i64, _i64, _i32, _vp]),
+    'a4g_mlp_add_layernorm_i8': (_i32, [ctypes.POINTER(MlpLayer), _i32, _vp, _i32, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _i32,
+                                        _i32, _i32, _i32, _i32, _vp]),
     'a4g_dense_i16': (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _i64, _i64, _i64, _i64, _vp]),
     'a4g_pack_weights_i16': (_i32, [_vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp]),
     'a4g_dense_i16x16': (_i32, [_vp, _i64, _vp, _vp, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _i64, _i64, _i64, _i64,

@@ -9,6 +9,7 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "layernorm_common.hpp"
 
 namespace a4g {
 
@@ -217,6 +218,13 @@ struct MlpMfmaArgs {
     int y_vec;        // rows of Y can be stored as 16-byte pieces
     int y_packed;     // at most 32 outputs in rows without gaps, Y 4-byte aligned: the tile store
     int y_magic;      // ceil(65536 / N): (j * y_magic) >> 16 == j / N for every j < 32 N
+    // the form that adds a residual to the last layer's int8 result and normalises the row (LN kernels only)
+    const int8_t* res;    // [batch][ld_res] int8, or null
+    const int16_t* gamma; // [N] Q7
+    const int16_t* beta;  // [N] Q15
+    int ld_res, res_bytes;
+    int ln_off;           // byte offset in LDS of gamma then beta widened to int32 (2 x 4 N bytes)
+    int log2c, eps_q0, ln_mode, gamma_shift, final_shift;
 };
 
 constexpr int64_t MLP_MFMA_MIN_BATCH = 512;
@@ -225,7 +233,9 @@ constexpr int64_t MLP_MFMA_MIN_BATCH = 512;
 // BIT: what the rounding mode adds besides its constant (fast_round_kind: 0 nothing, 1 a bit of the accumulator,
 // 2 minus that bit).
 // YVEC: the result's rows can be stored as 16-byte pieces.
-template <int MAXB, int BIT, bool YVEC>
+// LN: out = LayerNorm(saturate_i8(last layer + residual)) instead of the last layer's bytes (int8 result, N a multiple of
+// 16, YVEC): a sample's row lies in the two lanes m and m + 32, so its sums are an in-lane sum and one exchange.
+template <int MAXB, int BIT, bool YVEC, bool LN = false>
 __global__ __launch_bounds__(1024) void mlp_mfma_kernel(MlpMfmaArgs a) {
     constexpr int MLP_MFMA_BLOCKS = MAXB;
     extern __shared__ __attribute__((aligned(16))) int8_t smem[];
@@ -297,6 +307,15 @@ __global__ __launch_bounds__(1024) void mlp_mfma_kernel(MlpMfmaArgs a) {
     const int u0 = blockIdx.x * wpb + __builtin_amdgcn_readfirstlane(tid >> 6);
     if (AHEAD) fetch(u0, nact);  // the first unit's input travels while the fragments are staged
 
+    int* const gamma_lds = reinterpret_cast<int*>(smem + a.ln_off);
+    int* const beta_lds = gamma_lds + (LN ? a.layer[a.n_layers - 1].N : 0);
+    if (LN) {
+        const int n_ln = a.layer[a.n_layers - 1].N;
+        for (int c = tid; c < n_ln; c += nthreads) {
+            gamma_lds[c] = a.gamma[c];
+            beta_lds[c] = a.beta[c];
+        }
+    }
     if (tid < MLP_MAX_LAYERS) big[tid] = 0;
     if (tid < 64) *reinterpret_cast<v4i*>(zero_frag + tid * 16) = v4i{0, 0, 0, 0};
     __syncthreads();
@@ -466,6 +485,50 @@ __global__ __launch_bounds__(1024) void mlp_mfma_kernel(MlpMfmaArgs a) {
         // that does not exist gets an offset past the descriptor and is dropped. The compiler then knows how many stores
         // are in flight, and the wait for the next unit's input, requested before them, does not include their
         // acknowledgement.
+        if (LN) {
+            const auto rsrc_res = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.res), 0, a.res ? a.res_bytes : 0, 0x00020000);
+            int sx = 0, sq = 0;
+#pragma unroll
+            for (int nb = 0; nb < MLP_MFMA_BLOCKS; ++nb) {
+                const int col0 = nb * 32 + 16 * half;
+                const bool there = col0 < last_n;  // N % 16 == 0: a piece of 16 columns exists as a whole or not at all
+                const v4i rw = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(
+                                                          rsrc_res, (row_ok && there) ? row * a.ld_res + col0 : 0x7ffffff0, 0, 0));
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    unsigned y = static_cast<unsigned>(act[nb][q]);
+                    if (a.res) y = sat_add_i8x4(y, static_cast<unsigned>(rw[q]));
+                    if (!there) y = 0;
+                    act[nb][q] = static_cast<int>(y);
+                    sx = __builtin_amdgcn_sdot4(static_cast<int>(y), 0x01010101, sx, false);
+                    sq = __builtin_amdgcn_sdot4(static_cast<int>(y), static_cast<int>(y), sq, false);
+                }
+            }
+            sx += __shfl_xor(sx, 32);
+            sq += __shfl_xor(sq, 32);
+            const RowStats st = row_stats(sx, sq, last_n, a.log2c, a.eps_q0);
+#pragma unroll
+            for (int nb = 0; nb < MLP_MFMA_BLOCKS; ++nb) {
+                const int col0 = nb * 32 + 16 * half;
+                if (nb * 32 >= last_n) continue;  // (uniform)
+                const int cj = col0 < last_n ? col0 : 0;
+                v4i o;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const v4i g4 = *reinterpret_cast<const v4i*>(gamma_lds + cj + 4 * q);
+                    const v4i b4 = *reinterpret_cast<const v4i*>(beta_lds + cj + 4 * q);
+                    int y4[4];
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const int vd = sext8(static_cast<unsigned>(act[nb][q]), t) - st.mu;
+                        const int fs = clamp_i(round_shift_rt(st.inv * g4[t], a.gamma_shift, a.ln_mode), -32768, 32767);
+                        y4[t] = clamp_i(round_shift_rt(vd * fs + b4[t], a.final_shift, a.ln_mode), -128, 127);
+                    }
+                    o[q] = static_cast<int>(pack4_bytes(y4[0], y4[1], y4[2], y4[3]));
+                }
+                act[nb] = o;
+            }
+        }
         if (!YVEC && a.y_packed && u * 32 + 32 <= a.batch) {
             // At most 32 neurons in rows that follow each other without a gap (a classifier's few outputs): the unit's
             // 32 rows are 32 N consecutive bytes. They go through a 1 KiB tile of the wave's own (no barrier: a wave's
@@ -502,9 +565,9 @@ __global__ __launch_bounds__(1024) void mlp_mfma_kernel(MlpMfmaArgs a) {
     }
 }
 
-template <int MAXB, int BIT, bool YVEC>
+template <int MAXB, int BIT, bool YVEC, bool LN>
 static hipError_t launch_mlp_mfma(int grid, int threads, size_t lds, hipStream_t stream, const MlpMfmaArgs& f) {
-    auto kern = mlp_mfma_kernel<MAXB, BIT, YVEC>;
+    auto kern = mlp_mfma_kernel<MAXB, BIT, YVEC, LN>;
     static bool attr_set = false;  // benign race: the attribute is idempotent
     if (!attr_set) {
         const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -520,10 +583,19 @@ static hipError_t launch_mlp_mfma(int grid, int threads, size_t lds, hipStream_t
 
 using namespace a4g;
 
-extern "C" int a4g_mlp_i8(const a4g_mlp_layer* layers, int n_layers, const void* X, int x_kind, int64_t ldx, void* Y,
-                          int64_t ldy, int64_t batch, int round_mode, a4g_stream_t stream_) {
+namespace {
+struct MlpLnExtra {  // what a4g_mlp_add_layernorm_i8 has beyond a4g_mlp_i8
+    const int8_t* res;
+    int64_t ld_res;
+    const int16_t* gamma;
+    const int16_t* beta;
+    int eps_q0, gamma_shift, out_shift, ln_mode;
+};
+}  // namespace
+
+static int mlp_entry(const a4g_mlp_layer* layers, int n_layers, const void* X, int x_kind, int64_t ldx, void* Y, int64_t ldy,
+                     int64_t batch, int round_mode, const MlpLnExtra* ln, a4g_stream_t stream_, const char* who) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    const char* who = "a4g_mlp_i8";
     A4G_REQUIRE(layers && n_layers >= 1, A4G_ERR_INVALID_ARGUMENT, "%s: no layers", who);
     A4G_REQUIRE(n_layers <= MLP_MAX_LAYERS, A4G_ERR_UNSUPPORTED, "%s: %d layers exceed the fused limit of %d", who, n_layers,
                 MLP_MAX_LAYERS);
@@ -593,7 +665,7 @@ extern "C" int a4g_mlp_i8(const a4g_mlp_layer* layers, int n_layers, const void*
     {
         MlpMfmaArgs f{};
         int nfrag = 0, nstart = 0, in_u = x_kind == A4G_U8;
-        bool ok = batch >= MLP_MFMA_MIN_BATCH && layers[n_layers - 1].out_kind != A4G_I16 && ldx <= INT32_MAX && ldy <= INT32_MAX &&
+        bool ok = (ln || batch >= MLP_MFMA_MIN_BATCH) && layers[n_layers - 1].out_kind != A4G_I16 && ldx <= INT32_MAX && ldy <= INT32_MAX &&
                   (batch - 1) * ldx + layers[0].K < (int64_t{1} << 31) - 64 &&
                   ((batch - 1) * ldy + layers[n_layers - 1].N) * 2 < (int64_t{1} << 31) - 64;
         const FastRound fr1 = make_fast_round(round_mode, 1);  // the kind of bit is the same for every shift >= 1
@@ -631,7 +703,13 @@ extern "C" int a4g_mlp_i8(const a4g_mlp_layer* layers, int n_layers, const void*
         nfrag += 1;  // the fragment of zeros that absent K steps read
         // fragments, start values, one flag per layer (and, below, a 1 KiB tile per wave for the packed store)
         const size_t lds_core = static_cast<size_t>(nfrag) * 1024 + static_cast<size_t>(nstart) * 4 + MLP_MAX_LAYERS * 4;
-        if (ok && lds_core <= 128 * 1024) {
+        if (ok && ln) {  // the normalising form: int8 rows in whole 16-column pieces, 16-byte aligned on every side
+            const a4g_mlp_layer& l_ = layers[n_layers - 1];
+            ok = l_.out_kind == A4G_I8 && l_.N % 16 == 0 && ldy % 16 == 0 && aligned16(Y) &&
+                 (!ln->res || (aligned16(ln->res) && ln->ld_res % 16 == 0 && ln->ld_res >= l_.N &&
+                               (batch - 1) * ln->ld_res + l_.N < (int64_t{1} << 31) - 64));
+        }
+        if (ok && lds_core + (ln ? 8 * layers[n_layers - 1].N + 16 : 0) <= 128 * 1024) {
             const a4g_mlp_layer& lastl = layers[n_layers - 1];
             f.n_layers = n_layers;
             f.x_aligned = ldx % 16 == 0 && aligned16(X);
@@ -660,13 +738,32 @@ extern "C" int a4g_mlp_i8(const a4g_mlp_layer* layers, int n_layers, const void*
             const size_t tile_bytes = f.y_packed ? 16 * 1024 : 0;  // per CU, however its sixteen waves are grouped
             const int per_cu = static_cast<int>(std::max<size_t>(1, std::min<size_t>(4, (160 * 1024 - tile_bytes) / lds_core)));
             const int threads = per_cu >= 4 ? 256 : (per_cu >= 2 ? 512 : 1024);
-            const size_t lds_f = lds_core + (f.y_packed ? static_cast<size_t>(threads / 64) * 1024 : 0);
+            size_t lds_f = lds_core + (f.y_packed ? static_cast<size_t>(threads / 64) * 1024 : 0);
+            if (ln) {
+                f.res = ln->res;
+                f.gamma = ln->gamma;
+                f.beta = ln->beta;
+                f.ld_res = static_cast<int>(ln->ld_res);
+                f.res_bytes = ln->res ? static_cast<int>((batch - 1) * ln->ld_res + lastl.N) : 0;
+                f.log2c = -1;
+                if ((lastl.N & (lastl.N - 1)) == 0) {
+                    f.log2c = 0;
+                    while ((1 << f.log2c) < lastl.N) ++f.log2c;
+                }
+                f.eps_q0 = ln->eps_q0;
+                f.ln_mode = ln->ln_mode;
+                f.gamma_shift = ln->gamma_shift;
+                f.final_shift = 15 - ln->out_shift;
+                f.ln_off = static_cast<int>((lds_f + 15) / 16 * 16);
+                lds_f = static_cast<size_t>(f.ln_off) + 8 * static_cast<size_t>(lastl.N);
+            }
             const int64_t wanted = (batch + (threads / 2) - 1) / (threads / 2);
             const int grid_f = static_cast<int>(std::min<int64_t>(wanted, 256 * per_cu));
             hipError_t e = hipErrorInvalidValue;
 #define A4G_MLP_GO(MAXB, BIT)                                                                    \
-    e = f.y_vec ? launch_mlp_mfma<MAXB, BIT, true>(grid_f, threads, lds_f, stream, f)             \
-                : launch_mlp_mfma<MAXB, BIT, false>(grid_f, threads, lds_f, stream, f)
+    e = ln ? launch_mlp_mfma<MAXB, BIT, true, true>(grid_f, threads, lds_f, stream, f)            \
+           : (f.y_vec ? launch_mlp_mfma<MAXB, BIT, true, false>(grid_f, threads, lds_f, stream, f) \
+                      : launch_mlp_mfma<MAXB, BIT, false, false>(grid_f, threads, lds_f, stream, f))
 #define A4G_MLP_BITS(MAXB)                                                  \
     if (bit_kind == 0) A4G_MLP_GO(MAXB, 0);                                  \
     else if (bit_kind == 1) A4G_MLP_GO(MAXB, 1);                             \
@@ -679,6 +776,10 @@ extern "C" int a4g_mlp_i8(const a4g_mlp_layer* layers, int n_layers, const void*
             return check_hip(e, who);
         }
     }
+    if (ln)
+        return fail(A4G_ERR_UNSUPPORTED,
+                    "%s: needs an int8 last layer of N %% 16 == 0 columns, 16-byte aligned rows of the result and the residual, "
+                    "and weight fragments within 128 KiB of LDS", who);
 
     static bool attr_set = false;
     if (!attr_set) {
@@ -700,4 +801,25 @@ extern "C" int a4g_mlp_i8(const a4g_mlp_layer* layers, int n_layers, const void*
     else
         hipLaunchKernelGGL(mlp_fused_kernel<16>, dim3(grid), dim3(256), lds, stream, a);
     return check_hip(hipGetLastError(), who);
+}
+
+extern "C" int a4g_mlp_i8(const a4g_mlp_layer* layers, int n_layers, const void* X, int x_kind, int64_t ldx, void* Y,
+                          int64_t ldy, int64_t batch, int round_mode, a4g_stream_t stream) {
+    return mlp_entry(layers, n_layers, X, x_kind, ldx, Y, ldy, batch, round_mode, nullptr, stream, "a4g_mlp_i8");
+}
+
+extern "C" int a4g_mlp_add_layernorm_i8(const a4g_mlp_layer* layers, int n_layers, const void* X, int x_kind, int64_t ldx,
+                                        const int8_t* residual, int64_t ld_res, const int16_t* gamma, const int16_t* beta,
+                                        int8_t* Y, int64_t ldy, int64_t batch, int round_mode, int32_t eps_q0, int gamma_shift,
+                                        int out_shift, int ln_round_mode, a4g_stream_t stream) {
+    const char* who = "a4g_mlp_add_layernorm_i8";
+    A4G_REQUIRE(eps_q0 >= 1 && eps_q0 <= (1 << 30), A4G_ERR_INVALID_ARGUMENT,
+                "%s: eps_q0 must be positive (integer LayerNorm requires a positive variance floor), got %d", who, eps_q0);
+    A4G_REQUIRE(out_shift >= 0 && out_shift <= 15, A4G_ERR_INVALID_ARGUMENT, "%s: out_shift=%d must be in [0, 15]", who, out_shift);
+    A4G_REQUIRE(gamma_shift >= 0 && gamma_shift <= 15, A4G_ERR_INVALID_ARGUMENT, "%s: gamma_shift=%d must be in [0, 15]", who,
+                gamma_shift);
+    A4G_REQUIRE(valid_round(ln_round_mode), A4G_ERR_INVALID_ARGUMENT, "%s: unknown rounding mode", who);
+    A4G_REQUIRE(batch == 0 || (gamma && beta), A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+    const MlpLnExtra ln{residual, ld_res, gamma, beta, eps_q0, gamma_shift, out_shift, ln_round_mode};
+    return mlp_entry(layers, n_layers, X, x_kind, ldx, Y, ldy, batch, round_mode, &ln, stream, who);
 }

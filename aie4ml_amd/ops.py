@@ -445,6 +445,69 @@ def mlp(x: torch.Tensor, layers: Sequence[MlpLayerSpec], rounding='floor', out: 
     return out
 
 
+def _mlp_layer_array(layers: Sequence[MlpLayerSpec]):
+    arr = (MlpLayer * max(len(layers), 1))()
+    for i, spec in enumerate(layers):
+        p = spec.params
+        arr[i].wt = p.wt.data_ptr()
+        arr[i].ldwt = p.ldwt
+        arr[i].colsum = p.colsum.data_ptr()
+        arr[i].bias = p.bias.data_ptr() if p.bias is not None else None
+        arr[i].K, arr[i].N = p.K, p.N
+        arr[i].shift = int(spec.shift)
+        arr[i].relu = int(bool(spec.relu))
+        arr[i].out_kind = _kind(spec.out_kind)
+    return arr
+
+
+def mlp_add_layernorm_applicable(x: torch.Tensor, layers: Sequence[MlpLayerSpec]) -> bool:
+    """Whether mlp_add_layernorm() takes this chain (the limits of a4g_mlp_add_layernorm_i8)."""
+    if not layers or len(layers) > 8 or x.dtype not in (torch.int8, torch.uint8) or x.dim() < 1:
+        return False
+    shapes = [(s.params.K, s.params.N) for s in layers]
+    last = layers[-1]
+    blocks = sum(((k + 31) // 32) * ((n + 31) // 32) for k, n in shapes) + 1
+    start = sum((n + 31) // 32 * 32 for _k, n in shapes)
+    return (all(s.params.wt_lo is None and s.params.K <= 256 and s.params.N <= 256 for s in layers)
+            and all(a[1] == b[0] for a, b in zip(shapes[:-1], shapes[1:])) and int(x.shape[-1]) == shapes[0][0]
+            and all(_kind(s.out_kind) in (0, 1) for s in layers) and _kind(last.out_kind) == 0 and last.params.N % 16 == 0
+            and sum(s.params.N * s.params.ldwt for s in layers) <= 96 * 1024
+            and blocks * 1024 + start * 4 + 32 + 8 * last.params.N + 16 <= 128 * 1024)
+
+
+def mlp_add_layernorm(x: torch.Tensor, layers: Sequence[MlpLayerSpec], residual: Optional[torch.Tensor], gamma_q7: torch.Tensor,
+                      beta_q15: torch.Tensor, out_shift: int, rounding='floor', ln_rounding='floor', eps_q0: int = 1,
+                      gamma_shift: int = 7, out: Optional[torch.Tensor] = None):
+    """layernorm(saturate_i8(mlp(x) + residual)) in one launch: the same result as mlp() (int8 last layer), add() with
+    shift 0 and layernorm(). ``residual`` may be None. Raises NotImplementedError outside the limits of the fused kernel
+    (mlp_add_layernorm_applicable)."""
+    if not mlp_add_layernorm_applicable(x, layers):
+        raise NotImplementedError('mlp_add_layernorm: needs int8 / uint8 rows, up to 8 layers up to 256 wide whose fragments fit '
+                                  '128 KiB of LDS, and an int8 last layer of N % 16 == 0 columns')
+    x2 = _rows2d(x, 'x')
+    if x2.stride(1) != 1 or (x2.shape[0] > 1 and x2.stride(0) < x2.shape[1]):
+        x2 = x2.contiguous()
+    M, N = int(x2.shape[0]), layers[-1].params.N
+    r2 = None
+    if residual is not None:
+        if residual.dtype != torch.int8 or tuple(residual.shape) != tuple(x.shape[:-1]) + (N,):
+            raise ValueError('mlp_add_layernorm: the residual must be an int8 tensor of the output shape')
+        r2 = _rows2d(residual, 'residual').contiguous()
+    g = _dev(gamma_q7, 'gamma').to(torch.int16).contiguous()
+    bt = _dev(beta_q15, 'beta').to(torch.int16).contiguous()
+    if g.numel() != N or bt.numel() != N:
+        raise ValueError(f'LayerNorm parameter length does not match full_inner={N}.')
+    if out is None:
+        out = torch.empty(tuple(x.shape[:-1]) + (N,), dtype=torch.int8, device=x.device)
+    elif tuple(out.shape) != tuple(x.shape[:-1]) + (N,) or out.dtype != torch.int8 or not out.is_contiguous():
+        raise ValueError('mlp_add_layernorm: out must be a contiguous int8 tensor of the output shape')
+    arr = _mlp_layer_array(layers)
+    check(_lib.load().a4g_mlp_add_layernorm_i8(
+        arr, len(layers), _ptr(x2), _TORCH_KIND[x2.dtype], x2.stride(0) if M > 0 else layers[0].params.K, _ptr(r2), N, _ptr(g),
+        _ptr(bt), _ptr(out), N, M, _mode(rounding), int(eps_q0), int(gamma_shift), int(out_shift), _mode(ln_rounding), _stream()))
+    return out
+
+
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, logit_shift: int, logit_rounding, softmax: dict,
               out_shift: int, out_rounding, out: Optional[torch.Tensor] = None):
     """Fused attention core: srs(softmax(srs(q k^T)) v) per (batch, head), one launch.

@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define A4G_VERSION 202 /* major*10000 + minor*100 + patch */
+#define A4G_VERSION 203 /* major*10000 + minor*100 + patch */
 
 #if defined(__GNUC__)
 #define A4G_API __attribute__((visibility("default")))
@@ -248,6 +248,22 @@ typedef struct a4g_mlp_layer {
 
 A4G_API int a4g_mlp_i8(const a4g_mlp_layer* layers, int n_layers, const void* X, int x_kind, int64_t ldx, void* Y,
                int64_t ldy, int64_t batch, int round_mode, a4g_stream_t stream);
+
+/* The same chain with the block's tail in the same launch:
+ *   Y = LayerNorm(saturate_i8(chain(X) + residual))
+ * i.e. a4g_mlp_i8 (int8 last layer) -> a4g_add (shift 0) -> a4g_layernorm_i8, the integers of those three calls. It is
+ * what a small transformer block ends its two halves with: the attention output projection, or the pair of
+ * feed-forward layers, then the residual Add (elementwise_add.cpp:12-37) and the LayerNorm (layer_norm.cpp:14-121) -
+ * three kernels connected through memtile buffers in the reference's graph. A sample's row lies in two lanes of
+ * the chain kernel, so the row sums cost one exchange. residual may be NULL; gamma int16 Q7, beta int16 Q15 as in
+ * a4g_layernorm_i8, ln_round_mode its rounding, round_mode the layers'.
+ * Limits: those of the chain's matrix-unit form (weight fragments within 128 KiB of LDS, any batch), an int8
+ * last layer of N % 16 == 0 columns (N <= 256), Y and residual 16-byte aligned with pitches that are multiples
+ * of 16; otherwise A4G_ERR_UNSUPPORTED, and the caller issues the three calls. */
+A4G_API int a4g_mlp_add_layernorm_i8(const a4g_mlp_layer* layers, int n_layers, const void* X, int x_kind, int64_t ldx,
+                             const int8_t* residual, int64_t ld_res, const int16_t* gamma, const int16_t* beta,
+                             int8_t* Y, int64_t ldy, int64_t batch, int round_mode, int32_t eps_q0, int gamma_shift,
+                             int out_shift, int ln_round_mode, a4g_stream_t stream);
 
 /* ---- Fused attention core -----------------------------------------------------------------------------
  * O[b,h] = srs( softmax( srs(Q[b,h] x K[b,h]^T, logit_shift) ) x V[b,h], out_shift ) in one launch: the

@@ -1161,6 +1161,55 @@ def test_mlp_large_batch_rows_at_any_address(ops, oracle, widths):
     assert np.array_equal(host(ops.mlp(wide[:, :widths[0]], specs, 'conv_even')), want), widths
 
 
+@pytest.mark.parametrize('case', [
+    dict(widths=[64, 128, 64], batch=3000, residual=True),
+    dict(widths=[64, 64], batch=100, residual=True),
+    dict(widths=[128, 256, 128], batch=5000, residual=True),
+    dict(widths=[32, 64, 16], batch=33, residual=False),
+    dict(widths=[57, 200, 96, 48], batch=700, residual=True),
+    dict(widths=[256, 256], batch=1, residual=True),
+])
+@pytest.mark.parametrize('modes', [('conv_even', 'conv_even'), ('positive_inf', 'floor'), ('symmetric_inf', 'symmetric_zero'),
+                                   ('floor', 'conv_odd')])
+def test_mlp_add_layernorm(ops, oracle, case, modes):
+    """A chain of layers, the residual Add and the LayerNorm in one launch against the oracle's three operators: the two
+    halves of a small transformer block (one projection, or the feed-forward pair), widths on and off the 32-grid, uint8
+    hidden activations, batches from one sample to thousands, with and without a residual, gamma beyond 511."""
+    widths, batch = case['widths'], case['batch']
+    r = rng(sum(widths) + batch)
+    n_l = len(widths) - 1
+    outs = ['uint8' if i % 2 == 0 else 'int8' for i in range(n_l - 1)] + ['int8']
+    layers_np, specs = make_mlp_general(ops, r, widths, [int(r.integers(5, 10)) for _ in range(n_l)],
+                                        [i < n_l - 1 for i in range(n_l)], outs)
+    x = gauss8(r, 40, (batch, widths[0]))
+    N = widths[-1]
+    res = gauss8(r, 50, (batch, N)) if case['residual'] else None
+    gamma = r.integers(-700, 700, N).astype(np.int16)
+    beta = r.integers(-30000, 30000, N).astype(np.int16)
+    mode, lmode = modes
+    got = host(ops.mlp_add_layernorm(dev(x), specs, dev(res) if res is not None else None, dev(gamma), dev(beta), 6, mode,
+                                     lmode, eps_q0=3, gamma_shift=8))
+    y = oracle.mlp(x, layers_np, mode)
+    if res is not None:
+        want = oracle.add_layernorm(y, res, gamma, beta, 6, lmode, eps_q0=3, gamma_shift=8)
+    else:
+        want = oracle.layernorm(y, gamma, beta, 6, lmode, eps_q0=3, gamma_shift=8)
+    assert np.array_equal(got, want), (case, modes)
+
+
+def test_mlp_add_layernorm_refuses_what_it_cannot_take(ops):
+    r = rng(77)
+    _, specs = make_mlp_general(ops, r, [64, 40], [7], [False], ['int8'])       # 40 columns: not in 16-column pieces
+    x = torch.zeros((8, 64), dtype=torch.int8, device='cuda')
+    g = torch.ones(40, dtype=torch.int16, device='cuda')
+    with pytest.raises(NotImplementedError):
+        ops.mlp_add_layernorm(x, specs, None, g, g, 5)
+    _, specs = make_mlp_general(ops, r, [64, 32], [7], [False], ['uint8'])      # the sum is defined on int8
+    g = torch.ones(32, dtype=torch.int16, device='cuda')
+    with pytest.raises(NotImplementedError):
+        ops.mlp_add_layernorm(x, specs, None, g, g, 5)
+
+
 def test_mlp_limits(ops):
     r = rng(19)
     _, specs = make_mlp(ops, r, [16, 300, 4])
