@@ -224,7 +224,8 @@ struct MlpMfmaArgs {
     const int16_t* beta;  // [N] Q15
     int ld_res, res_bytes;
     int ln_off;           // byte offset in LDS of gamma then beta widened to int32 (2 x 4 N bytes)
-    int log2c, eps_q0, ln_mode, gamma_shift, final_shift;
+    int log2c, eps_q0;
+    FastRound ln_rg, ln_ro;  // the two requantisations of the normalisation (gamma scale, output)
 };
 
 constexpr int64_t MLP_MFMA_MIN_BATCH = 512;
@@ -381,6 +382,20 @@ __global__ __launch_bounds__(1024) void mlp_mfma_kernel(MlpMfmaArgs a) {
 #pragma unroll
             for (int ks = 0; ks < MLP_MFMA_BLOCKS; ++ks) act[ks] ^= xm0;
         }
+        // The residual's pieces are requested here, a whole chain ahead of their use, where the registers allow it: a unit
+        // is one wave's work from end to end, and a load that starts after the last layer is waited for in full.
+        constexpr bool RES_AHEAD = LN && MAXB <= 4;
+        const auto rsrc_res = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.res), 0, (LN && a.res) ? a.res_bytes : 0, 0x00020000);
+        auto residual_piece = [&](int nb) __attribute__((always_inline)) {
+            const int col0 = nb * 32 + 16 * half;
+            return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(
+                                               rsrc_res, (row_ok && col0 < last_n) ? row * a.ld_res + col0 : 0x7ffffff0, 0, 0));
+        };
+        v4i rw_ahead[RES_AHEAD ? MLP_MFMA_BLOCKS : 1];
+        if (RES_AHEAD) {
+#pragma unroll
+            for (int nb = 0; nb < MLP_MFMA_BLOCKS; ++nb) rw_ahead[nb] = residual_piece(nb);
+        }
         for (int l = 0; l < a.n_layers; ++l) {
             const MlpMfmaLayer& L = a.layer[l];
             const bool last = l + 1 == a.n_layers;
@@ -486,14 +501,12 @@ __global__ __launch_bounds__(1024) void mlp_mfma_kernel(MlpMfmaArgs a) {
         // are in flight, and the wait for the next unit's input, requested before them, does not include their
         // acknowledgement.
         if (LN) {
-            const auto rsrc_res = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.res), 0, a.res ? a.res_bytes : 0, 0x00020000);
             int sx = 0, sq = 0;
 #pragma unroll
             for (int nb = 0; nb < MLP_MFMA_BLOCKS; ++nb) {
                 const int col0 = nb * 32 + 16 * half;
                 const bool there = col0 < last_n;  // N % 16 == 0: a piece of 16 columns exists as a whole or not at all
-                const v4i rw = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(
-                                                          rsrc_res, (row_ok && there) ? row * a.ld_res + col0 : 0x7ffffff0, 0, 0));
+                const v4i rw = RES_AHEAD ? rw_ahead[RES_AHEAD ? nb : 0] : residual_piece(nb);
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                     unsigned y = static_cast<unsigned>(act[nb][q]);
@@ -521,8 +534,9 @@ __global__ __launch_bounds__(1024) void mlp_mfma_kernel(MlpMfmaArgs a) {
 #pragma unroll
                     for (int t = 0; t < 4; ++t) {
                         const int vd = sext8(static_cast<unsigned>(act[nb][q]), t) - st.mu;
-                        const int fs = clamp_i(round_shift_rt(st.inv * g4[t], a.gamma_shift, a.ln_mode), -32768, 32767);
-                        y4[t] = clamp_i(round_shift_rt(vd * fs + b4[t], a.final_shift, a.ln_mode), -128, 127);
+                        // (both within fast_round's range: |inv * gamma| < 2^30, |vd * fs| < 2^23)
+                        const int fs = clamp_i(fast_round(__mul24(st.inv, g4[t]), a.ln_rg), -32768, 32767);
+                        y4[t] = clamp_i(fast_round(__mul24(vd, fs) + b4[t], a.ln_ro), -128, 127);
                     }
                     o[q] = static_cast<int>(pack4_bytes(y4[0], y4[1], y4[2], y4[3]));
                 }
@@ -751,9 +765,8 @@ static int mlp_entry(const a4g_mlp_layer* layers, int n_layers, const void* X, i
                     while ((1 << f.log2c) < lastl.N) ++f.log2c;
                 }
                 f.eps_q0 = ln->eps_q0;
-                f.ln_mode = ln->ln_mode;
-                f.gamma_shift = ln->gamma_shift;
-                f.final_shift = 15 - ln->out_shift;
+                f.ln_rg = make_fast_round(ln->ln_mode, ln->gamma_shift);
+                f.ln_ro = make_fast_round(ln->ln_mode, 15 - ln->out_shift);
                 f.ln_off = static_cast<int>((lds_f + 15) / 16 * 16);
                 lds_f = static_cast<size_t>(f.ln_off) + 8 * static_cast<size_t>(lastl.N);
             }

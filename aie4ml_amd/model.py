@@ -172,11 +172,14 @@ class GPUModel:
         graph, execution = ctx.ir.logical, ctx.ir.execution
         plan = ctx.config.get('gpu_fusion_plan') or {}
         plan = {'add_layernorm': plan.get('add_layernorm', {}), 'mlp_chains': plan.get('mlp_chains', []),
-                'attention': plan.get('attention', []), 'dense_add_layernorm': plan.get('dense_add_layernorm', {})}
+                'attention': plan.get('attention', []), 'dense_add_layernorm': plan.get('dense_add_layernorm', {}),
+                'mlp_add_layernorm': plan.get('mlp_add_layernorm', {})}
         values: Dict[str, Any] = dict(inputs)
         fused_ln = {v['layer_norm'] for v in plan['add_layernorm'].values()}
         fused_ln |= {v['layer_norm'] for v in plan['dense_add_layernorm'].values()}
+        fused_ln |= {v['layer_norm'] for v in plan['mlp_add_layernorm'].values()}
         fused_dense = {v['dense'] for v in plan['dense_add_layernorm'].values()}
+        fused_dense |= {n for v in plan['mlp_add_layernorm'].values() for n in v['chain']}  # run at the add's position
         chain_head = {c[0]: c for c in plan['mlp_chains']}
         chain_rest = {n for c in plan['mlp_chains'] for n in c[1:]}
         attn_at, attn_skip = {}, set()
@@ -207,7 +210,7 @@ class GPUModel:
             if node.is_placeholder:
                 self._run_view(node, values)
                 continue
-            if node.name in chain_rest or node.name in fused_ln or node.name in fused_dense:
+            if node.name in fused_ln or node.name in fused_dense or node.name in chain_rest:
                 continue  # executed as part of a fused launch
             if node.name in attn_at:
                 grp = attn_at[node.name]
@@ -220,6 +223,10 @@ class GPUModel:
             if node.name in chain_head:
                 chain = chain_head[node.name]
                 launch(node.name, 'mlp', chain, lambda: self._run_mlp(chain, values, ops))
+            elif node.name in plan['mlp_add_layernorm']:
+                info = plan['mlp_add_layernorm'][node.name]
+                launch(info['chain'][0], 'mlp_add_layer_norm', [*info['chain'], node.name, info['layer_norm']],
+                       lambda: self._run_mlp_add_layernorm(info, values, ops))
             elif node.name in plan['dense_add_layernorm']:
                 # launched at the add's position: the residual may be computed after the dense's own input
                 info = plan['dense_add_layernorm'][node.name]
@@ -280,6 +287,34 @@ class GPUModel:
             return
         # batch sizes at which the one-launch form does not pay: the same integers from two launches
         y = ops.dense(x, packed, dcfg.rounding_mode, relu=dcfg.flags.use_relu, out_kind='int8')
+        values[ln_inst.node.outputs[0].name] = ops.add_layernorm(
+            y, values[info['residual']], ln_inst.artifacts['packed_gamma'], ln_inst.artifacts['packed_beta'], cfg.out_shift,
+            cfg.rounding_mode, eps_q0=cfg.eps_q0, gamma_shift=cfg.gamma_shift)
+
+    def _run_mlp_add_layernorm(self, info, values, ops) -> None:
+        execution = self.context.ir.execution
+        insts = [execution.get(n) for n in info['chain']]
+        ln_inst = execution.get(info['layer_norm'])
+        cfg = ln_inst.config
+        specs = [ops.MlpLayerSpec(i.artifacts['packed_weights'], i.config.shift, i.config.flags.use_relu,
+                                  i.config.precision['output'].format) for i in insts]
+        x = values[input_tensor_for_role(insts[0].node, 'lhs').name]
+        same_mode = all(i.config.rounding_mode == insts[0].config.rounding_mode for i in insts)
+        rows = x.numel() // max(1, int(x.shape[-1]))
+        shapes = [(s.params.K, s.params.N) for s in specs]
+        if same_mode and ops.mlp_add_layernorm_applicable(x, specs) and ops.mlp_add_layernorm_pays(rows, shapes):
+            values[ln_inst.node.outputs[0].name] = ops.mlp_add_layernorm(
+                x, specs, values[info['residual']], ln_inst.artifacts['packed_gamma'], ln_inst.artifacts['packed_beta'],
+                cfg.out_shift, rounding=insts[0].config.rounding_mode, ln_rounding=cfg.rounding_mode, eps_q0=cfg.eps_q0,
+                gamma_shift=cfg.gamma_shift)
+            return
+        # outside the fused launch's limits: the chain (or the single layer) as planned without it, then Add + LayerNorm
+        if len(insts) > 1:
+            self._run_mlp(info['chain'], values, ops)
+        else:
+            name = input_tensor_for_role(insts[0].node, 'lhs').name
+            values.update(insts[0].variant.run(insts[0], {name: values[name]}))
+        y = values[insts[-1].node.outputs[0].name]
         values[ln_inst.node.outputs[0].name] = ops.add_layernorm(
             y, values[info['residual']], ln_inst.artifacts['packed_gamma'], ln_inst.artifacts['packed_beta'], cfg.out_shift,
             cfg.rounding_mode, eps_q0=cfg.eps_q0, gamma_shift=cfg.gamma_shift)

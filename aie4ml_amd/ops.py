@@ -475,6 +475,16 @@ def mlp_add_layernorm_applicable(x: torch.Tensor, layers: Sequence[MlpLayerSpec]
             and blocks * 1024 + start * 4 + 32 + 8 * last.params.N + 16 <= 128 * 1024)
 
 
+def mlp_add_layernorm_pays(rows: int, shapes: Sequence[Tuple[int, int]]) -> bool:
+    """Whether the one-launch form is the faster one (``shapes``: (K, N) per layer). Its normalisation is serial work of
+    the two lanes that hold a row, where the row kernel spreads a row over as many lanes as it has 16-byte pieces: the
+    launch it saves pays up to 128 columns. Measured against mlp() + add_layernorm() at 2048 / 32768 / 131072 rows:
+    64 -> 64: 9.6 / 10.3 / 14.9 us against 11.6 / 12.3 / 17.2; 64 -> 128 -> 64: 13.2 / 13.9 / 21.5 against 14.5 / 15.6 /
+    22.6; 128 -> 128: 13.1 / 13.9 / 25.9 against 13.8 / 16.0 / 29.2; but 64 -> 256 -> 64: 17.8 / 19.2 / 32.8 against
+    17.5 / 19.0 / 31.0 and 256 -> 256: 25.2 / 28.0 / 44.7 against 20.3 / 25.1 / 48.3."""
+    return rows >= 1 and all(k <= 128 and n <= 128 for k, n in shapes)
+
+
 def mlp_add_layernorm(x: torch.Tensor, layers: Sequence[MlpLayerSpec], residual: Optional[torch.Tensor], gamma_q7: torch.Tensor,
                       beta_q15: torch.Tensor, out_shift: int, rounding='floor', ln_rounding='floor', eps_q0: int = 1,
                       gamma_shift: int = 7, out: Optional[torch.Tensor] = None):

@@ -421,6 +421,29 @@ class PlanGpuFusion(AIEPass):
                         plan['dense_add_layernorm'][add_name] = {'dense': d.name, 'layer_norm': info['layer_norm'],
                                                                  'residual': other[0].name}
                         break
+        # (chain of) narrow dense -> add -> layer_norm: the chain kernel normalises the rows itself
+        plan['mlp_add_layernorm'] = {}
+        by_name = {n.name: n for n in graph.nodes}
+        chain_of_tail = {c[-1]: c for c in plan['mlp_chains']}
+        for add_name, info in plan['add_layernorm'].items():
+            add_node = by_name[add_name]
+            if info['keep_sum'] or add_node.traits.get('io_view') or add_name in plan['dense_add_layernorm']:
+                continue
+            for t in add_node.inputs:
+                d = t.producer
+                if d is None or d.op_type != 'dense' or execution.get(d.name) is None or len(t.consumers) != 1 or t.name in outputs:
+                    continue
+                chain = chain_of_tail.get(d.name)
+                if chain is None:
+                    if d.name in used or not self._fits([d], execution):
+                        continue
+                    chain = [d.name]
+                cfg = execution.get(chain[-1]).config
+                other = [u for u in add_node.inputs if u is not t]
+                if cfg.precision['output'].format == 'int8' and cfg.n_out % 16 == 0 and len(other) == 1 and not other[0].is_parameter:
+                    plan['mlp_add_layernorm'][add_name] = {'chain': list(chain), 'layer_norm': info['layer_norm'],
+                                                           'residual': other[0].name}
+                    break
         changed = ctx.config.get('gpu_fusion_plan') != plan
         ctx.config['gpu_fusion_plan'] = plan
         return changed

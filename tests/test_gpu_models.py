@@ -215,6 +215,30 @@ def test_encoder_block_with_a_sequence_off_the_tile_grid(oracle, seq):
     assert len(np.unique(next(iter(got.values())))) > 32
 
 
+@pytest.mark.parametrize('batch,taken', [(16, True), (2, True), (16, False)])
+def test_narrow_encoder_block_runs_in_four_launches(oracle, batch, taken, monkeypatch):
+    """64 features, 4 heads of 16, feed-forward width 256: the Q/K/V projection, the attention, the output projection
+    with its Add and LayerNorm, and the feed-forward pair with theirs. Where the chain kernel refuses at launch, the last
+    two run as their parts."""
+    import torch
+
+    from aie4ml_amd import ops
+
+    model, x = workloads.c5_encoder_block(batch=batch, seq=64, hidden=64, heads=4, ffn=256, softmax='exp')
+    model.compile()
+    plan = model.context.config['gpu_fusion_plan']
+    assert [len(v['chain']) for v in plan['mlp_add_layernorm'].values()] == [1, 2]
+    if not taken:
+        monkeypatch.setattr(ops, 'mlp_add_layernorm_applicable', lambda x, layers: False)
+    trace = []
+    model.execute({'x': torch.from_numpy(x).cuda()}, trace=trace)
+    assert [t['kind'] for t in trace] == ['dense', 'attention', 'mlp_add_layer_norm', 'mlp_add_layer_norm']
+    got = _graph_check(model, oracle, {'x': x})
+    model.context.config['gpu_fusion_plan'] = {}        # and the same graph operator by operator
+    _graph_check(model, oracle, {'x': x})
+    assert len(np.unique(next(iter(got.values())))) > 32
+
+
 def test_encoder_block_c5_shape(oracle):
     """BERT-base geometry (hidden 768, 12 heads of 64, FFN 3072, seq 128) on a batch the oracle finishes
     in seconds; the full batch of 64 differs only in the number of independent sequences."""
@@ -432,9 +456,9 @@ def test_report_times_every_launch(oracle):
     enc = from_onnx(onnx_bytes, config)
     rep = enc.report(repeats=3)
     kinds = [k['kind'] for k in rep['kernels']]
-    # QKV and output projections, all heads in one attention launch, both residual adds inside their LayerNorm,
-    # and an FFN this small runs as one fused-MLP launch
-    assert kinds == ['dense', 'attention', 'dense', 'add_layer_norm', 'mlp', 'add_layer_norm']
+    # the QKV projection, all heads in one attention launch, and layers this narrow carry the residual add and the
+    # LayerNorm behind them: the output projection in one launch, the FFN pair in another
+    assert kinds == ['dense', 'attention', 'mlp_add_layer_norm', 'mlp_add_layer_norm']
     assert abs(sum(k['pct'] for k in rep['kernels']) - 100.0) < 1.0
     assert all(k['time_us'] > 0 for k in rep['kernels'])
 

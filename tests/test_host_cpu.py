@@ -375,6 +375,21 @@ def test_encoder_block_graph_lowers():
     assert plan['dense_add_layernorm'] == {}  # 64 outputs: too narrow for the projection that normalises its own rows
 
 
+def test_plan_joins_narrow_layers_with_the_add_and_layernorm_behind_them():
+    from aie4ml_amd import workloads
+
+    model, _ = workloads.c5_encoder_block(batch=2, seq=32, hidden=64, heads=2, ffn=128)
+    plan = lower(GraphHolder(model), FRONT + (PlanGpuFusion,)).config['gpu_fusion_plan']
+    # the attention output projection (64 -> 64) is a chain of one; the feed-forward pair is a chain of two
+    assert plan['mlp_add_layernorm'] == {
+        'residual1_aie': {'chain': ['attn_out_aie'], 'layer_norm': 'ln1_aie', 'residual': 'x'},
+        'residual2_aie': {'chain': ['ffn1_aie', 'ffn2_aie'], 'layer_norm': 'ln2_aie', 'residual': 'ln1_out'}}
+    assert plan['dense_add_layernorm'] == {}
+    # layers wider than the chain kernel's 256 columns stay out of it
+    model, _ = workloads.c5_encoder_block(batch=1, seq=32, hidden=768, heads=12, ffn=3072)
+    assert lower(GraphHolder(model), FRONT + (PlanGpuFusion,)).config['gpu_fusion_plan']['mlp_add_layernorm'] == {}
+
+
 def test_plan_marks_projections_that_can_normalise_their_rows():
     from aie4ml_amd import workloads
 
