@@ -89,6 +89,15 @@ def test_argument_validation_happens_before_any_launch(libpath):
     assert lib.a4g_dense_add_layernorm_i8(None, 0, 768, None, None, None, 9, 0, 0, None, 768, None, None, None, 768, 0, 768, 768,
                                           1, 7, 5, 0, None) == 0  # no rows
     assert lib.a4g_rowpack_weights_i8(None, 768, 100, 768, None, None) == _lib.A4G_ERR_UNSUPPORTED  # 100 columns
+    # the chain that ends in Add + LayerNorm checks the normalisation's constants before it looks at the chain
+    st = lib.a4g_mlp_add_layernorm_i8(None, 1, None, 0, 64, None, 64, None, None, None, 64, 32, 0, 0, 7, 5, 0, None)  # eps_q0 < 1
+    assert st == _lib.A4G_ERR_INVALID_ARGUMENT and b'a4g_mlp_add_layernorm_i8: eps_q0' in lib.a4g_last_error()
+    assert lib.a4g_mlp_add_layernorm_i8(None, 1, None, 0, 64, None, 64, None, None, None, 64, 32, 0, 1, 7, 16, 0,
+                                        None) == _lib.A4G_ERR_INVALID_ARGUMENT  # out_shift 16
+    assert lib.a4g_mlp_add_layernorm_i8(None, 1, None, 0, 64, None, 64, None, None, None, 64, 32, 0, 1, 16, 5, 0,
+                                        None) == _lib.A4G_ERR_INVALID_ARGUMENT  # gamma_shift 16
+    assert lib.a4g_mlp_add_layernorm_i8(None, 1, None, 0, 64, None, 64, None, None, None, 64, 32, 0, 1, 7, 5, 9,
+                                        None) == _lib.A4G_ERR_INVALID_ARGUMENT  # rounding mode 9
     st = lib.a4g_softmax_exp_i8(None, None, 4, 512, 0, 15, 1, None)  # exp_kq out of range
     assert st == _lib.A4G_ERR_INVALID_ARGUMENT and b'EXP_KQ' in lib.a4g_last_error()
     st = lib.a4g_layernorm_i8(None, None, None, None, 4, 64, 0, 7, 5, 6, None)  # eps_q0 < 1
