@@ -234,6 +234,53 @@ def test_mlp_chain_on_a_long_batch_random_case(ops, oracle, seed):
     assert np.array_equal(got, oracle.mlp(x, layers_np, mode)), (seed, widths, batch, mode, off, [(l[2], l[3], l[4]) for l in layers_np])
 
 
+@pytest.mark.parametrize('seed', range(24 + EXTRA // 4))
+def test_mlp_chain_with_add_and_layernorm_random_case(ops, oracle, seed):
+    """Chains of one to four layers that end in 16 to 256 int8 columns, then the residual Add and the LayerNorm, in one
+    launch: random widths, shifts, ReLU, hidden activation signs, batches from one sample to thousands, both rounding
+    modes, the LayerNorm's two shifts and its variance floor; the residual is sometimes absent and sometimes a window of
+    a wider matrix (16-byte aligned, as the entry point asks)."""
+    r = np.random.default_rng(9100 + seed)
+    n_layers = int(r.integers(1, 5))
+    widths = [int(r.choice([5, 16, 17, 32, 48, 57, 64, 100, 128, 200, 256])) for _ in range(n_layers)]
+    widths.append(int(r.choice([16, 32, 48, 64, 80, 128, 144, 256])))
+    batch = int(r.choice([1, 31, 32, 33, 500, 1000, 4096 + int(r.integers(0, 100))]))
+    mode, lmode = str(r.choice(MODES)), str(r.choice(MODES))
+    x = draw(r, np.int8, (batch, widths[0]))
+    layers_np, specs = [], []
+    for i, (k, n) in enumerate(zip(widths[:-1], widths[1:])):
+        W = r.integers(-64, 64, (k, n)).astype(np.int8)
+        b = r.integers(-2**13, 2**13 + 1, n).astype(np.int32) if r.random() < 0.9 else None
+        sh = int(r.integers(4, 12))
+        last = i == n_layers - 1
+        relu = bool(r.random() < 0.6) and not last
+        out = 'int8' if last else str(r.choice(['int8', 'uint8']))
+        layers_np.append((W, b, sh, relu, out))
+        specs.append(ops.MlpLayerSpec(ops.pack_dense(dev(W), dev(b) if b is not None else None, sh), sh, relu, out))
+    N = widths[-1]
+    res = draw(r, np.int8, (batch, N)) if r.random() < 0.8 else None
+    dres = None
+    if res is not None:
+        pad = int(r.choice([0, 16, 48]))
+        wide = torch.zeros((batch, N + pad), dtype=torch.int8, device='cuda')
+        dres = wide[:, pad:]
+        dres.copy_(torch.from_numpy(res))
+    gamma = r.integers(-700, 700, N).astype(np.int16) if r.random() < 0.5 else r.integers(-32768, 32768, N).astype(np.int16)
+    beta = r.integers(-32768, 32768, N).astype(np.int16)
+    out_shift, gamma_shift, eps = int(r.integers(0, 16)), int(r.integers(0, 16)), int(r.choice([1, 3, 100, 1 << 20]))
+    try:
+        got = host(ops.mlp_add_layernorm(dev(x), specs, dres, dev(gamma), dev(beta), out_shift, mode, lmode, eps_q0=eps,
+                                         gamma_shift=gamma_shift))
+    except NotImplementedError:
+        return  # more weights than the kernel holds
+    y = oracle.mlp(x, layers_np, mode)
+    if res is not None:
+        want = oracle.add_layernorm(y, res, gamma, beta, out_shift, lmode, eps_q0=eps, gamma_shift=gamma_shift)
+    else:
+        want = oracle.layernorm(y, gamma, beta, out_shift, lmode, eps_q0=eps, gamma_shift=gamma_shift)
+    assert np.array_equal(got, want), (seed, widths, batch, mode, lmode, out_shift, gamma_shift, eps, res is not None)
+
+
 @pytest.mark.parametrize('seed', range(16 + EXTRA // 4))
 def test_long_row_operator_random_case(ops, oracle, seed):
     """LayerNorm, fused Add + LayerNorm and both Softmax forms on rows of 4112 to 20 000 columns."""
