@@ -58,6 +58,8 @@ SIGNATURES = {
     'a4g_pack_weights_i8': (_i32, [_vp, _i64, _i64, _i64, _vp, _vp, _vp]),
     'a4g_dense_i8': (_i32, [_vp, _i32, _i32, _i64, _vp, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _i64, _i64, _i64,
                             _i64, _vp]),
+    'a4g_dense_i8_wf': (_i32, [_vp, _i32, _i32, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _i64, _i64, _i64,
+                               _i64, _vp]),
     'a4g_matmul_i8_workspace_bytes': (_sz, [_i64, _i64, _i64, _i64, _i32, _i32]),
     'a4g_matmul_i8': (_i32, [_vp, _i32, _i32, _i64, _i64, _vp, _i64, _i64, _i32, _vp, _i64, _i64, _i64, _i64, _i64, _i64,
                              _i32, _i32, _i32, _vp, _sz, _vp]),
@@ -66,6 +68,7 @@ SIGNATURES = {
     'a4g_layernorm_i8': (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, ctypes.c_int32, _i32, _i32, _i32, _vp]),
     'a4g_add_layernorm_i8': (_i32, [_vp, _vp, _i32, _i32, _vp, _vp, _vp, _vp, _i64, _i64, ctypes.c_int32, _i32, _i32,
                                     _i32, _vp]),
+    'a4g_rowpacked_bytes': (_i64, [_i64, _i64]),
     'a4g_rowpack_weights_i8': (_i32, [_vp, _i64, _i64, _i64, _vp, _vp]),
     'a4g_dense_add_layernorm_i8': (_i32, [_vp, _i32, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _vp, _i64, _vp, _vp, _vp, _i64,
                                           _i64, _i64, _i64, ctypes.c_int32, _i32, _i32, _i32, _vp]),

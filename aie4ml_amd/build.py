@@ -13,7 +13,7 @@ from pathlib import Path
 
 CSRC = Path(__file__).resolve().parent / 'csrc'
 LIB_PATH = Path(__file__).resolve().parent / 'libaie4ml_gfx950.so'
-SOURCES = ('abi.hip', 'rowops.hip', 'gemm.hip', 'mlp.hip', 'attention.hip', 'matmul_lean.hip', 'gemm_i16.hip', 'gemm_float.hip', 'calib.hip', 'gemm_wreg.hip', 'gemm_sk.hip', 'gemm_rowln.hip')
+SOURCES = ('abi.hip', 'rowops.hip', 'gemm.hip', 'mlp.hip', 'attention.hip', 'matmul_lean.hip', 'gemm_i16.hip', 'gemm_float.hip', 'calib.hip', 'gemm_wreg.hip', 'gemm_wrow.hip', 'gemm_wrow_plain.hip', 'gemm_wrow_sym_inf.hip', 'gemm_wrow_conv_even.hip', 'gemm_sk.hip', 'gemm_rowln.hip')
 
 HIPCC_FLAGS = [
     '--offload-arch=gfx950',
@@ -64,7 +64,7 @@ def build(force: bool = False, verbose: bool = False) -> Path:
             print(errs, file=sys.stderr)
         return obj
 
-    with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as pool:
+    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
         objs = list(pool.map(compile_one, SOURCES))
     cmd = [hipcc, '--offload-arch=gfx950', '-shared', '-fPIC', '-o', str(LIB_PATH), *map(str, objs)]
     res = subprocess.run(cmd, capture_output=True, text=True)

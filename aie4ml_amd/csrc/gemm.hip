@@ -796,11 +796,10 @@ extern "C" int a4g_pack_weights_i8(const int8_t* W, int64_t ldw, int64_t K, int6
     return check_hip(hipGetLastError(), "a4g_pack_weights_i8");
 }
 
-extern "C" int a4g_dense_i8(const void* A, int a_kind, int trans_a, int64_t lda, const int8_t* Wt, int64_t ldwt, const int32_t* colsum,
-                            const int32_t* bias, const int32_t* shifts, int n_shift, int round_mode, int relu, int out_kind,
-                            void* Y, int64_t ldy, int64_t M, int64_t N, int64_t K, a4g_stream_t stream_) {
+static int dense_i8(const char* who, const void* A, int a_kind, int trans_a, int64_t lda, const int8_t* Wt, int64_t ldwt, const int8_t* Wf,
+                    const int32_t* colsum, const int32_t* bias, const int32_t* shifts, int n_shift, int round_mode, int relu,
+                    int out_kind, void* Y, int64_t ldy, int64_t M, int64_t N, int64_t K, a4g_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
-    const char* who = "a4g_dense_i8";
     A4G_REQUIRE(M >= 0 && N >= 1 && K >= 1 && M <= INT32_MAX && N <= (1 << 24) && K <= (1 << 24), A4G_ERR_INVALID_ARGUMENT,
                 "%s: bad shape M=%lld N=%lld K=%lld", who, (long long)M, (long long)N, (long long)K);
     A4G_REQUIRE(a_kind == A4G_I8 || a_kind == A4G_U8, A4G_ERR_UNSUPPORTED, "%s: activations must be int8 or uint8 (kind %d)",
@@ -833,6 +832,7 @@ extern "C" int a4g_dense_i8(const void* A, int a_kind, int trans_a, int64_t lda,
     g.relu = relu != 0;
     g.out_kind = out_kind;
     g.mode = round_mode;
+    g.Wf = Wf;
 
     const bool tiled = K % 16 == 0 && lda % 16 == 0 && ldwt % 16 == 0 && aligned16(A) && aligned16(Wt);
     hipError_t e;
@@ -848,6 +848,20 @@ extern "C" int a4g_dense_i8(const void* A, int a_kind, int trans_a, int64_t lda,
         e = launch_ragged(g, 1, stream);
     }
     return check_hip(e, who);
+}
+
+extern "C" int a4g_dense_i8(const void* A, int a_kind, int trans_a, int64_t lda, const int8_t* Wt, int64_t ldwt, const int32_t* colsum,
+                            const int32_t* bias, const int32_t* shifts, int n_shift, int round_mode, int relu, int out_kind,
+                            void* Y, int64_t ldy, int64_t M, int64_t N, int64_t K, a4g_stream_t stream_) {
+    return dense_i8("a4g_dense_i8", A, a_kind, trans_a, lda, Wt, ldwt, nullptr, colsum, bias, shifts, n_shift, round_mode, relu, out_kind, Y,
+                    ldy, M, N, K, stream_);
+}
+
+extern "C" int a4g_dense_i8_wf(const void* A, int a_kind, int trans_a, int64_t lda, const int8_t* Wt, int64_t ldwt, const int8_t* Wf,
+                               const int32_t* colsum, const int32_t* bias, const int32_t* shifts, int n_shift, int round_mode, int relu,
+                               int out_kind, void* Y, int64_t ldy, int64_t M, int64_t N, int64_t K, a4g_stream_t stream_) {
+    return dense_i8("a4g_dense_i8_wf", A, a_kind, trans_a, lda, Wt, ldwt, Wf, colsum, bias, shifts, n_shift, round_mode, relu, out_kind, Y,
+                    ldy, M, N, K, stream_);
 }
 
 extern "C" size_t a4g_matmul_i8_workspace_bytes(int64_t batch, int64_t M, int64_t N, int64_t K, int trans_b, int a_kind) {

@@ -326,16 +326,19 @@ __global__ __launch_bounds__(RL_NT, 2) void gemm_rowln_kernel(RowLnArgs g) {
 }
 
 // Wt [N][ldwt] (a4g_pack_weights_i8) -> fragments: the 16 bytes of lane l of fragment (nb, ks) are K chunk
-// 32 ks + 16 (l / 32) of the weight row of column 32 nb + direct_col_of_operand_row(l % 32).
+// 32 ks + 16 (l / 32) of the weight row of column 32 nb + direct_col_of_operand_row(l % 32); columns past N and
+// chunks past K are zero (whole 32-column groups, whole 128-byte K tiles: rowpacked_bytes).
 __global__ __launch_bounds__(256) void rowpack_kernel(const int8_t* __restrict__ wt, int64_t ldwt, int N, int K, v4i* __restrict__ wf) {
-    const int64_t chunks = static_cast<int64_t>(N) * K / 16;
-    const int ksteps = K >> 5;
+    const int ksteps = (K + 127) / 128 * 4;
+    const int64_t chunks = static_cast<int64_t>((N + 31) / 32) * ksteps * 64;
     for (int64_t c = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; c < chunks; c += static_cast<int64_t>(gridDim.x) * blockDim.x) {
         const int l = static_cast<int>(c & 63);
         const int64_t frag = c >> 6;
         const int ks = static_cast<int>(frag % ksteps), nb = static_cast<int>(frag / ksteps);
-        const int n = nb * 32 + direct_col_of_operand_row(l & 31);
-        wf[c] = *reinterpret_cast<const v4i*>(wt + static_cast<int64_t>(n) * ldwt + ks * 32 + 16 * (l >> 5));
+        const int n = nb * 32 + direct_col_of_operand_row(l & 31), k0 = ks * 32 + 16 * (l >> 5);
+        v4i v = {0, 0, 0, 0};
+        if (n < N && k0 < K) v = *reinterpret_cast<const v4i*>(wt + static_cast<int64_t>(n) * ldwt + k0);
+        wf[c] = v;
     }
 }
 
@@ -366,16 +369,18 @@ static hipError_t launch_rowln_rb(const RowLnArgs& g, int fr, hipStream_t stream
 
 using namespace a4g;
 
+extern "C" int64_t a4g_rowpacked_bytes(int64_t N, int64_t K) { return N <= 0 || K <= 0 ? 0 : rowpacked_bytes(N, K); }
+
 extern "C" int a4g_rowpack_weights_i8(const int8_t* Wt, int64_t ldwt, int64_t N, int64_t K, int8_t* Wf, a4g_stream_t stream_) {
     const char* who = "a4g_rowpack_weights_i8";
     A4G_REQUIRE(N >= 0 && K >= 0 && ldwt >= K, A4G_ERR_INVALID_ARGUMENT, "%s: bad shape N=%lld K=%lld ldwt=%lld", who, (long long)N,
                 (long long)K, (long long)ldwt);
-    A4G_REQUIRE(N % 32 == 0 && K % 128 == 0 && N <= RL_MAX_N && K <= RL_MAX_K && ldwt % 16 == 0, A4G_ERR_UNSUPPORTED,
-                "%s: needs N %% 32 == 0, N <= %d, K %% 128 == 0, K <= %d, ldwt %% 16 == 0 (N=%lld K=%lld ldwt=%lld)", who, RL_MAX_N,
-                RL_MAX_K, (long long)N, (long long)K, (long long)ldwt);
+    A4G_REQUIRE(K % 16 == 0 && ldwt % 16 == 0 && N <= (1 << 24) && K <= (1 << 24) && rowpacked_bytes(N, K) < (int64_t{1} << 31),
+                A4G_ERR_UNSUPPORTED, "%s: needs K %% 16 == 0, ldwt %% 16 == 0 and a result below 2 GiB (N=%lld K=%lld ldwt=%lld)", who,
+                (long long)N, (long long)K, (long long)ldwt);
     if (N == 0 || K == 0) return A4G_OK;
     A4G_REQUIRE(Wt && Wf && aligned16(Wt) && aligned16(Wf), A4G_ERR_INVALID_ARGUMENT, "%s: null or misaligned pointer", who);
-    const int64_t chunks = N * K / 16;
+    const int64_t chunks = rowpacked_bytes(N, K) / 16;
     const int grid = static_cast<int>(std::min<int64_t>((chunks + 255) / 256, 2048));
     rowpack_kernel<<<grid, 256, 0, static_cast<hipStream_t>(stream_)>>>(Wt, ldwt, static_cast<int>(N), static_cast<int>(K),
                                                                         reinterpret_cast<v4i*>(Wf));

@@ -64,7 +64,13 @@ struct GemmArgs {
     // only read by the ragged form of the tiled int8 kernel: how a 16-byte chunk of an operand row may be fetched
     // (0 = one aligned load inside the row pitch, 1 = dwords, 2 = bytes); bytes at or past K always read as zero
     int ragged_a, ragged_b;
+    // the same weights in fragment order (a4g_rowpack_weights_i8) or null; only Dense kernels that keep weights in
+    // registers read it
+    const int8_t* Wf;
 };
+
+// Bytes of the fragment-order copy of an [N][K] int8 weight matrix: whole 32-column groups, whole 128-byte K tiles.
+static inline int64_t rowpacked_bytes(int64_t N, int64_t K) { return (N + 31) / 32 * 32 * ((K + 127) / 128 * 128); }
 
 // Workgroups per problem for tile_coord: whole ranges for the 8 XCDs (surplus workgroups exit at once), except that a
 // problem of fewer than 8 tiles gets exactly its tiles: padding 768 one-tile problems to 8 workgroups each made the
@@ -415,6 +421,9 @@ bool rs_i16i8_applicable(const GemmArgs& g, int batch);
 // (no batch), int8 / uint8 activations and outputs.
 bool wreg_applicable(const GemmArgs& g);
 hipError_t launch_wreg(const GemmArgs& g, hipStream_t stream);
+// The same shapes with the weights in fragment order as well (gemm_wrow.hip): 64-row pieces, requantisation overlapped.
+bool wrow_applicable(const GemmArgs& g);
+hipError_t launch_wrow(const GemmArgs& g, hipStream_t stream);
 
 // Dense with a long reduction on 128 x 192 tiles, the reduction split inside an eight-wave workgroup (gemm_sk.hip). One
 // problem (no batch), int8 / uint8 activations and outputs.

@@ -291,6 +291,7 @@ bool wreg_applicable(const GemmArgs& g) {
 }
 
 hipError_t launch_wreg(const GemmArgs& g, hipStream_t stream) {
+    if (wrow_applicable(g)) return launch_wrow(g, stream);
     const int halves_m = (g.M + 63) / 64, cbs = (g.N + WR_BN - 1) / WR_BN;
     // 512 workgroups fill the chip (two per CU) and the column blocks get an equal share of them each; of the counts
     // that give the longest run the same number of halves, the smallest loads the weights least often

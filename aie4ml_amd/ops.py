@@ -103,7 +103,8 @@ class PackedDense:
     N: int
     wt_lo: Optional[torch.Tensor] = None  # int16 weights only: the low-byte plane (bytes ^ 0x80)
     shift0: Optional[int] = None          # the shift as a host integer when there is one for every column
-    wf: Optional[torch.Tensor] = None     # int8 weights in fragment order, made on first use by dense_add_layernorm
+    wf: Optional[torch.Tensor] = None     # int8 weights in fragment order (short reductions: at pack time; else on
+                                          # first use by dense_add_layernorm)
 
     @property
     def ldwt(self) -> int:
@@ -137,8 +138,21 @@ def pack_dense(weight: torch.Tensor, bias: Optional[torch.Tensor], shifts) -> Pa
     top = 62 if wt_lo is not None else 31
     if int(sh.min()) < 0 or int(sh.max()) > top:
         raise ValueError(f'dense accumulator output shift must be in [0, {top}], got [{int(sh.min())}, {int(sh.max())}].')
-    return PackedDense(wt=wt, colsum=colsum, bias=bias, shifts=sh.to(weight.device), K=K, N=N, wt_lo=wt_lo,
-                       shift0=int(sh[0]) if sh.numel() == 1 else None)
+    p = PackedDense(wt=wt, colsum=colsum, bias=bias, shifts=sh.to(weight.device), K=K, N=N, wt_lo=wt_lo,
+                    shift0=int(sh[0]) if sh.numel() == 1 else None)
+    if wt_lo is None and K <= 768 and K % 16 == 0:
+        _rowpack(p)  # the Dense kernel for short reductions fetches its weights in this order
+    return p
+
+
+def _rowpack(p: PackedDense) -> torch.Tensor:
+    """The fragment-order copy of p's int8 weights (made once, kept in p.wf)."""
+    if p.wf is None:
+        L = _lib.load()
+        wf = torch.empty((int(L.a4g_rowpacked_bytes(p.N, p.K)),), dtype=torch.int8, device=p.wt.device)
+        check(L.a4g_rowpack_weights_i8(_ptr(p.wt), p.ldwt, p.N, p.K, _ptr(wf), _stream()))
+        p.wf = wf
+    return p.wf
 
 
 def dense(x: torch.Tensor, p: PackedDense, rounding='floor', relu: bool = False, out_kind='int8',
@@ -194,9 +208,10 @@ def dense(x: torch.Tensor, p: PackedDense, rounding='floor', relu: bool = False,
         # of layers over 32 samples per wave does a chain of one at 3-5 TB/s (1 Mi x 16 -> 64: 23 us against 151 us)
         mlp(x2, [MlpLayerSpec(p, int(p.shift0), bool(relu), 'uint8' if ok == 1 else 'int8')], rounding, out=y2)
         return out
-    check(_lib.load().a4g_dense_i8(_ptr(x2), _TORCH_KIND[x2.dtype], 0, x2.stride(0) if M > 0 else p.K, _ptr(p.wt), p.ldwt,
-                                   _ptr(p.colsum), _ptr(p.bias), _ptr(p.shifts), int(p.shifts.numel()), _mode(rounding),
-                                   int(bool(relu)), ok, _ptr(y2), y2.stride(0) if M > 0 else p.N, M, p.N, p.K, _stream()))
+    check(_lib.load().a4g_dense_i8_wf(_ptr(x2), _TORCH_KIND[x2.dtype], 0, x2.stride(0) if M > 0 else p.K, _ptr(p.wt), p.ldwt,
+                                      _ptr(p.wf), _ptr(p.colsum), _ptr(p.bias), _ptr(p.shifts), int(p.shifts.numel()),
+                                      _mode(rounding), int(bool(relu)), ok, _ptr(y2), y2.stride(0) if M > 0 else p.N, M, p.N,
+                                      p.K, _stream()))
     return out
 
 
@@ -356,10 +371,7 @@ def dense_add_layernorm(x: torch.Tensor, p: PackedDense, residual: Optional[torc
     if g.numel() != p.N or bt.numel() != p.N:
         raise ValueError(f'LayerNorm parameter length does not match full_inner={p.N}.')
     L = _lib.load()
-    if p.wf is None:
-        wf = torch.empty((p.N * p.K,), dtype=torch.int8, device=p.wt.device)
-        check(L.a4g_rowpack_weights_i8(_ptr(p.wt), p.ldwt, p.N, p.K, _ptr(wf), _stream()))
-        p.wf = wf
+    _rowpack(p)
     if out is None:
         out = torch.empty(tuple(x.shape[:-1]) + (p.N,), dtype=torch.int8, device=x.device)
     elif tuple(out.shape) != tuple(x.shape[:-1]) + (p.N,) or out.dtype != torch.int8 or not out.is_contiguous():

@@ -109,9 +109,9 @@ def _time_cpu(fn, budget_s=12.0, min_runs=2):
 # The four projections of the c5 encoder block as Dense workloads of their own (rows = batch 64 x seq 128): shape,
 # the kernel that runs them, and which projection it is.
 ENCODER_PROJECTIONS = {
-    'c5_proj_qkv': (8192, 768, 2304, 'gemm_wreg_kernel', 'fused Q/K/V projection'),
-    'c5_proj_out': (8192, 768, 768, 'gemm_wreg_kernel', 'attention output projection'),
-    'c5_ffn_up': (8192, 768, 3072, 'gemm_wreg_kernel', 'first feed-forward projection'),
+    'c5_proj_qkv': (8192, 768, 2304, 'gemm_wrow_kernel', 'fused Q/K/V projection'),
+    'c5_proj_out': (8192, 768, 768, 'gemm_wrow_kernel', 'attention output projection'),
+    'c5_ffn_up': (8192, 768, 3072, 'gemm_wrow_kernel', 'first feed-forward projection'),
     'c5_ffn_down': (8192, 3072, 768, 'gemm_sk_kernel', 'second feed-forward projection'),
 }
 

@@ -113,6 +113,18 @@ A4G_API int a4g_dense_i8(const void* A, int a_kind, int trans_a, int64_t lda, co
                  int round_mode, int relu, int out_kind, void* Y, int64_t ldy, int64_t M, int64_t N,
                  int64_t K, a4g_stream_t stream);
 
+/* The same Dense for a caller that also holds the weights in fragment order (the layout a matrix-core operand has
+ * in registers; the counterpart of the microtile order pack_mmul_rhs_matrix gives the AIE kernels,
+ * op_impls/families/matmul/common.py:307-358). Same arguments and results as a4g_dense_i8, plus
+ *   Wf      a4g_rowpack_weights_i8 applied to Wt (a4g_rowpacked_bytes(N, K) bytes, 16-byte aligned), or NULL
+ * With Wf, reductions of up to 768 with 16-byte aligned rows on both sides take a kernel that keeps a column block's
+ * weights in registers and fetches them with whole-line loads (csrc/gemm_wrow.hip); every other shape, and a NULL Wf,
+ * runs exactly as a4g_dense_i8. */
+A4G_API int a4g_dense_i8_wf(const void* A, int a_kind, int trans_a, int64_t lda, const int8_t* Wt, int64_t ldwt,
+                    const int8_t* Wf, const int32_t* colsum, const int32_t* bias, const int32_t* shifts, int n_shift,
+                    int round_mode, int relu, int out_kind, void* Y, int64_t ldy, int64_t M, int64_t N,
+                    int64_t K, a4g_stream_t stream);
+
 /* Dense with int16 activations and int8 weights: the reference's (16, 8) width combination
  * (op_impls/families/matmul/common.py:52), accumulated in acc32 like the 8-bit case
  * (op_impls/utils/precision.py:120-121). Same arguments as a4g_dense_i8 with A [M][lda] int16 (lda in
@@ -193,11 +205,15 @@ A4G_API int a4g_add_layernorm_i8(const int8_t* a, const int8_t* b, int add_shift
  * three kernels with memory tiles between them. A workgroup computes complete output rows, so neither the Dense result
  * nor the sum is written to memory.
  *   Wf        the weights in fragment order: a4g_rowpack_weights_i8 applied to the Wt of a4g_pack_weights_i8
- *             (N * K bytes); colsum, bias as for a4g_dense_i8
+ *             (a4g_rowpacked_bytes(N, K) bytes, = N * K within this call's limits); colsum, bias as for a4g_dense_i8
  *   residual  [M][ld_res] int8 or NULL (LayerNorm of the Dense output itself)
  *   gamma, beta, eps_q0, gamma_shift, out_shift, ln_round_mode as for a4g_layernorm_i8 (cols = N)
  * Limits: N a multiple of 32 up to 768, K a multiple of 128 up to 4096, pitches multiples of 16, operands 16-byte
  * aligned; outside them the call returns A4G_ERR_UNSUPPORTED and the caller runs the two calls above. */
+/* Fragment order: N is taken in groups of 32 columns and K in 128-byte tiles (both zero padded); the 1 KiB fragment
+ * of (column group nb, K step ks of 32 bytes) lies at ((nb * (tiles * 4)) + ks) * 1024, 16 bytes per wavefront lane.
+ * K a multiple of 16. Device-side, like a4g_pack_weights_i8. */
+A4G_API int64_t a4g_rowpacked_bytes(int64_t N, int64_t K);
 A4G_API int a4g_rowpack_weights_i8(const int8_t* Wt, int64_t ldwt, int64_t N, int64_t K, int8_t* Wf, a4g_stream_t stream);
 A4G_API int a4g_dense_add_layernorm_i8(const void* A, int a_kind, int64_t lda, const int8_t* Wf, const int32_t* colsum,
                                const int32_t* bias, int shift, int dense_round_mode, int relu, const int8_t* residual,

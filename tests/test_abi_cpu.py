@@ -88,7 +88,9 @@ def test_argument_validation_happens_before_any_launch(libpath):
                                           1, 7, 5, 0, None) == _lib.A4G_ERR_INVALID_ARGUMENT  # shift 40
     assert lib.a4g_dense_add_layernorm_i8(None, 0, 768, None, None, None, 9, 0, 0, None, 768, None, None, None, 768, 0, 768, 768,
                                           1, 7, 5, 0, None) == 0  # no rows
-    assert lib.a4g_rowpack_weights_i8(None, 768, 100, 768, None, None) == _lib.A4G_ERR_UNSUPPORTED  # 100 columns
+    assert lib.a4g_rowpack_weights_i8(None, 768, 100, 760, None, None) == _lib.A4G_ERR_UNSUPPORTED  # K off the 16-byte grid
+    assert lib.a4g_rowpack_weights_i8(None, 768, 100, 768, None, None) == _lib.A4G_ERR_INVALID_ARGUMENT  # null pointers
+    assert lib.a4g_rowpacked_bytes(100, 200) == 128 * 256 and lib.a4g_rowpacked_bytes(0, 64) == 0
     # the chain that ends in Add + LayerNorm checks the normalisation's constants before it looks at the chain
     st = lib.a4g_mlp_add_layernorm_i8(None, 1, None, 0, 64, None, 64, None, None, None, 64, 32, 0, 0, 7, 5, 0, None)  # eps_q0 < 1
     assert st == _lib.A4G_ERR_INVALID_ARGUMENT and b'a4g_mlp_add_layernorm_i8: eps_q0' in lib.a4g_last_error()

@@ -309,6 +309,35 @@ def test_dense_short_reduction_requantisation_forms(ops, oracle, mode, shift_set
         assert np.array_equal(got, exp), (out, np.argwhere(got != exp)[:5])
 
 
+def test_dense_short_reduction_with_and_without_fragment_order_weights(ops, oracle):
+    """a4g_dense_i8_wf with the fragment-order copy (64-row pieces, weights fetched with whole-line loads) and with NULL
+    in its place (the kernel that takes them from the row-major weights) give the oracle's integers. Of the four
+    256-column blocks only the third needs the general requantisation (a zero shift, a shift of 20 and biases next to
+    the int32 limits), so the runs of pieces go from the quick form into the general one and back; 2000 rows end inside a
+    piece, 1000 columns inside a column block."""
+    import dataclasses
+    r = rng(61)
+    for (M, K, N, a_dtype, mode) in [(2000, 768, 1000 // 16 * 16, np.int8, 'conv_even'), (4100, 320, 1024, np.uint8, 'symmetric_inf'),
+                                     (8192, 768, 2304, np.int8, 'positive_inf'), (70, 128, 1024, np.int8, 'conv_even')]:
+        A = r.integers(0, 256, (M, K)).astype(np.uint8) if a_dtype == np.uint8 else gauss8(r, 40, (M, K))
+        W = gauss8(r, 30, (K, N))
+        shifts = r.integers(1, 16, N).astype(np.int32)
+        bias = r.integers(-2**20, 2**20, N).astype(np.int64)
+        if N > 600:
+            shifts[520] = 0
+            shifts[530] = 20
+            bias[540], bias[541] = 2**31 - 5, -2**31 + 7
+        bias = bias.astype(np.int32)
+        p = ops.pack_dense(dev(W), dev(bias), shifts)
+        assert p.wf is not None
+        exp = oracle.dense(A, W, bias, shifts, mode, relu=False, out='int8')
+        got = host(ops.dense(dev(A), p, mode, relu=False, out_kind='int8'))
+        assert np.array_equal(got, exp), (M, K, N, np.argwhere(got != exp)[:5])
+        plain = dataclasses.replace(p, wf=None)
+        got = host(ops.dense(dev(A), plain, mode, relu=False, out_kind='int8'))
+        assert np.array_equal(got, exp), ('row-major weights', M, K, N, np.argwhere(got != exp)[:5])
+
+
 # Longer reductions on at most 256 tiles of 128 x 192 take the kernel that splits the reduction inside the workgroup.
 @pytest.mark.parametrize('case', [
     (8192, 3072, 768, 'conv_even', np.int8), (8192, 3072, 768, 'conv_even', np.uint8), (8192, 1024, 768, 'symmetric_inf', np.int8),
