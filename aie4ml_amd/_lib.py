@@ -49,6 +49,10 @@ class MlpLayer(ctypes.Structure):
     ]
 
 
+# The interface revision (A4G_VERSION of include/aie4ml_gfx950.h) the signatures below were written for. load() refuses
+# a library of any other revision: a stale build would misread every argument behind a changed one without an error.
+EXPECTED_VERSION = 300
+
 # name -> (restype, argtypes); must list every symbol the public header declares
 SIGNATURES = {
     'a4g_version': (_i32, []),
@@ -77,20 +81,20 @@ SIGNATURES = {
     'a4g_mlp_i8': (_i32, [ctypes.POINTER(MlpLayer), _i32, _vp, _i32, _i64, _vp, _i64, _i64, _i32, _vp]),
     'a4g_mlp_add_layernorm_i8': (_i32, [ctypes.POINTER(MlpLayer), _i32, _vp, _i32, _i64, _vp, _i64, _vp, _vp, _vp, _i64, _i64, _i32,
                                         _i32, _i32, _i32, _i32, _vp]),
-    'a4g_dense_i16': (_i32, [_vp, _i64, _vp, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _i64, _i64, _i64, _i64, _vp]),
+    'a4g_dense_i16': (_i32, [_vp, _i32, _i64, _vp, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _i64, _i64, _i64, _i64, _vp]),
     'a4g_pack_weights_i16': (_i32, [_vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp]),
-    'a4g_dense_i16x16': (_i32, [_vp, _i64, _vp, _vp, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _i64, _i64, _i64, _i64,
+    'a4g_dense_i16x16': (_i32, [_vp, _i32, _i64, _vp, _vp, _i64, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp, _i64, _i64, _i64, _i64,
                                 _vp]),
     'a4g_matmul_i16_workspace_bytes': (_sz, [_i64, _i64, _i64, _i32]),
-    'a4g_matmul_i16': (_i32, [_vp, _i64, _i64, _vp, _i32, _i64, _i64, _i32, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32,
+    'a4g_matmul_i16': (_i32, [_vp, _i32, _i64, _i64, _vp, _i32, _i64, _i64, _i32, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _i32, _i32,
                               _i32, _vp, _sz, _vp]),
     'a4g_attention_i8': (_i32, [_vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, ctypes.POINTER(ctypes.c_int64), _i32, _i32,
                                 _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp]),
     'a4g_packed_ld_f': (_i64, [_i64, _i32]),
     'a4g_pack_weights_f': (_i32, [_vp, _i32, _i64, _i64, _i64, _vp, _vp]),
-    'a4g_dense_f': (_i32, [_vp, _i32, _i64, _vp, _i64, _vp, _i32, _vp, _i64, _i64, _i64, _i64, _vp]),
+    'a4g_dense_f': (_i32, [_vp, _i32, _i32, _i64, _vp, _i64, _vp, _i32, _vp, _i64, _i64, _i64, _i64, _vp]),
     'a4g_matmul_f_workspace_bytes': (_sz, [_i64, _i64, _i64, _i32, _i32]),
-    'a4g_matmul_f': (_i32, [_vp, _i32, _i64, _i64, _vp, _i64, _i64, _i32, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _sz,
+    'a4g_matmul_f': (_i32, [_vp, _i32, _i32, _i64, _i64, _vp, _i64, _i64, _i32, _vp, _i64, _i64, _i64, _i64, _i64, _i64, _vp, _sz,
                             _vp]),
     'a4g_add_f': (_i32, [_vp, _vp, _vp, _i64, _i32, _vp]),
     'a4g_transpose': (_i32, [_vp, _i32, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
@@ -120,6 +124,10 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)  # AttributeError if the symbol is not exported
         fn.restype = restype
         fn.argtypes = argtypes
+    have = int(lib.a4g_version())
+    if have != EXPECTED_VERSION:
+        raise RuntimeError(f'{LIB_PATH} is interface revision {have}, these bindings are written for {EXPECTED_VERSION}: '
+                           'rebuild it with `python -m aie4ml_amd.build --force`')
     _lib = lib
     return lib
 

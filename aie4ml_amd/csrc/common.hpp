@@ -330,6 +330,28 @@ __device__ __forceinline__ v4i load_chunk_ragged(const int8_t* p, int rem, int m
     return r;
 }
 
+// One 16-byte chunk of a row of A when A is stored transposed ([K][ld], TRANSPOSE_A of matmul.cpp:60-66 and
+// dense_bias_relu.cpp:95-101): element e of the chunk is the `es`-byte element (1, 2 or 4 bytes) at
+// col + (k0 + e) * ld_bytes, `col` pointing at the row's element of k = 0; elements at or past K read as zero.
+__device__ __forceinline__ v4i load_chunk_transposed(const int8_t* col, int64_t ld_bytes, int k0, int K, int es) {
+    v4i r = {0, 0, 0, 0};
+    const int8_t* p = col + static_cast<int64_t>(k0) * ld_bytes;
+    if (es == 4) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            if (k0 + e < K) r[e] = *reinterpret_cast<const int*>(p + e * ld_bytes);
+    } else if (es == 2) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            if (k0 + e < K) r[e >> 1] |= static_cast<int>(static_cast<unsigned>(*reinterpret_cast<const uint16_t*>(p + e * ld_bytes)) << (16 * (e & 1)));
+    } else {
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+            if (k0 + e < K) r[e >> 2] |= static_cast<int>(static_cast<unsigned>(static_cast<uint8_t>(p[e * ld_bytes])) << (8 * (e & 3)));
+    }
+    return r;
+}
+
 // The store that goes with it: the first `rem` bytes of a 16-byte chunk, in pieces the row's alignment allows.
 __device__ __forceinline__ void store_chunk_ragged(int8_t* p, const v4i& v, int rem, int mode) {
     if (rem <= 0) return;

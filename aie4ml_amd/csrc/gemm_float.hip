@@ -176,11 +176,11 @@ __global__ __launch_bounds__(256) void add_float_kernel(const void* a, const voi
 static inline int64_t round_up64(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
 
 // A is [batch][M][lda], Bt is [batch][N][ldb], both K-contiguous, element counts; C [batch][M][ldc].
-static hipError_t launch_float_nt(const void* A, int64_t lda, int64_t stride_a, const void* Bt, int64_t ldb, int64_t stride_b,
+static hipError_t launch_float_nt(const void* A, int trans_a, int64_t lda, int64_t stride_a, const void* Bt, int64_t ldb, int64_t stride_b,
                                   const float* bias, int relu, void* C, int64_t ldc, int64_t stride_c, int batch, int M, int N,
                                   int K, int fmt, hipStream_t stream) {
     const int es = fmt_bytes(fmt);
-    const bool tiled = (static_cast<int64_t>(K) * es) % 128 == 0 && (lda * es) % 16 == 0 && (ldb * es) % 16 == 0 &&
+    const bool tiled = !trans_a && (static_cast<int64_t>(K) * es) % 128 == 0 && (lda * es) % 16 == 0 && (ldb * es) % 16 == 0 &&
                        (stride_a * es) % 16 == 0 && (stride_b * es) % 16 == 0 && aligned16(A) && aligned16(Bt);
     GemmArgs g{};
     g.A = static_cast<const int8_t*>(A);
@@ -201,6 +201,7 @@ static hipError_t launch_float_nt(const void* A, int64_t lda, int64_t stride_a, 
         // K that does not fill its last 128-byte tile, unaligned rows: the same kernel with loads that respect the row ends
         g.ragged_a = ragged_mode(g.A, g.lda, g.stride_a, g.K);
         g.ragged_b = ragged_mode(g.Bt, g.ldb, g.stride_b, g.K);
+        g.trans_a_es = trans_a ? es : 0;  // A stored transposed: its chunks are gathered element by element
         if (fmt == A4G_F32) return launch_rs_policy<FloatPolicy<A4G_F32>, 128, 128, 2, 2, false, true>(g, batch, stream);
         if (fmt == A4G_FP8) return launch_rs_policy<FloatPolicy<A4G_FP8>, 128, 128, 2, 2, false, true>(g, batch, stream);
         return launch_rs_policy<FloatPolicy<A4G_BF16>, 128, 128, 2, 2, false, true>(g, batch, stream);
@@ -253,17 +254,17 @@ extern "C" int a4g_pack_weights_f(const void* W, int fmt, int64_t ldw, int64_t K
     return check_hip(launch_transpose_fmt(fmt, W, ldw, 0, Wt, ldt, 0, 1, (int)K, (int)N, stream), who);
 }
 
-extern "C" int a4g_dense_f(const void* A, int fmt, int64_t lda, const void* Wt, int64_t ldwt, const float* bias, int relu, void* Y,
+extern "C" int a4g_dense_f(const void* A, int fmt, int trans_a, int64_t lda, const void* Wt, int64_t ldwt, const float* bias, int relu, void* Y,
                            int64_t ldy, int64_t M, int64_t N, int64_t K, a4g_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const char* who = "a4g_dense_f";
     A4G_REQUIRE(fmt_ok(fmt), A4G_ERR_UNSUPPORTED, "%s: format %d is not bfloat16 / float32 / fp8 e4m3", who, fmt);
     A4G_REQUIRE(M >= 0 && N >= 1 && K >= 1 && M <= INT32_MAX && N <= (1 << 24) && K <= (1 << 24), A4G_ERR_INVALID_ARGUMENT,
                 "%s: bad shape M=%lld N=%lld K=%lld", who, (long long)M, (long long)N, (long long)K);
-    A4G_REQUIRE(lda >= K && ldy >= N && ldwt >= K, A4G_ERR_INVALID_ARGUMENT, "%s: pitch smaller than the row", who);
+    A4G_REQUIRE(lda >= (trans_a ? M : K) && ldy >= N && ldwt >= K, A4G_ERR_INVALID_ARGUMENT, "%s: pitch smaller than the row", who);
     if (M == 0) return A4G_OK;
     A4G_REQUIRE(A && Wt && Y, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
-    return check_hip(launch_float_nt(A, lda, 0, Wt, ldwt, 0, bias, relu, Y, ldy, 0, 1, (int)M, (int)N, (int)K, fmt, stream), who);
+    return check_hip(launch_float_nt(A, trans_a, lda, 0, Wt, ldwt, 0, bias, relu, Y, ldy, 0, 1, (int)M, (int)N, (int)K, fmt, stream), who);
 }
 
 extern "C" size_t a4g_matmul_f_workspace_bytes(int64_t batch, int64_t N, int64_t K, int trans_b, int fmt) {
@@ -271,7 +272,7 @@ extern "C" size_t a4g_matmul_f_workspace_bytes(int64_t batch, int64_t N, int64_t
     return static_cast<size_t>(batch) * N * a4g_packed_ld_f(K, fmt) * fmt_bytes(fmt);
 }
 
-extern "C" int a4g_matmul_f(const void* A, int fmt, int64_t lda, int64_t stride_a, const void* B, int64_t ldb, int64_t stride_b,
+extern "C" int a4g_matmul_f(const void* A, int fmt, int trans_a, int64_t lda, int64_t stride_a, const void* B, int64_t ldb, int64_t stride_b,
                             int trans_b, void* C, int64_t ldc, int64_t stride_c, int64_t batch, int64_t M, int64_t N, int64_t K,
                             void* workspace, size_t workspace_bytes, a4g_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
@@ -280,11 +281,12 @@ extern "C" int a4g_matmul_f(const void* A, int fmt, int64_t lda, int64_t stride_
     A4G_REQUIRE(batch >= 0 && batch <= 65535 && M >= 0 && N >= 1 && K >= 1 && M <= INT32_MAX && N <= (1 << 24) && K <= (1 << 24),
                 A4G_ERR_INVALID_ARGUMENT, "%s: bad shape batch=%lld M=%lld N=%lld K=%lld", who, (long long)batch, (long long)M,
                 (long long)N, (long long)K);
-    A4G_REQUIRE(lda >= K && ldc >= N && ldb >= (trans_b ? K : N), A4G_ERR_INVALID_ARGUMENT, "%s: pitch smaller than the row", who);
+    A4G_REQUIRE(lda >= (trans_a ? M : K) && ldc >= N && ldb >= (trans_b ? K : N), A4G_ERR_INVALID_ARGUMENT, "%s: pitch smaller than the row",
+                who);
     if (M == 0 || batch == 0) return A4G_OK;
     A4G_REQUIRE(A && B && C, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
     if (trans_b)
-        return check_hip(launch_float_nt(A, lda, stride_a, B, ldb, stride_b, nullptr, 0, C, ldc, stride_c, (int)batch, (int)M, (int)N,
+        return check_hip(launch_float_nt(A, trans_a, lda, stride_a, B, ldb, stride_b, nullptr, 0, C, ldc, stride_c, (int)batch, (int)M, (int)N,
                                          (int)K, fmt, stream), who);
     const size_t need = a4g_matmul_f_workspace_bytes(batch, N, K, 0, fmt);
     A4G_REQUIRE(workspace && workspace_bytes >= need && aligned16(workspace), A4G_ERR_WORKSPACE,
@@ -292,7 +294,7 @@ extern "C" int a4g_matmul_f(const void* A, int fmt, int64_t lda, int64_t stride_
     const int64_t ldt = a4g_packed_ld_f(K, fmt);
     hipError_t e = launch_transpose_fmt(fmt, B, ldb, stride_b, workspace, ldt, N * ldt, (int)batch, (int)K, (int)N, stream);
     if (e != hipSuccess) return check_hip(e, who);
-    return check_hip(launch_float_nt(A, lda, stride_a, workspace, ldt, N * ldt, nullptr, 0, C, ldc, stride_c, (int)batch, (int)M, (int)N,
+    return check_hip(launch_float_nt(A, trans_a, lda, stride_a, workspace, ldt, N * ldt, nullptr, 0, C, ldc, stride_c, (int)batch, (int)M, (int)N,
                                      (int)K, fmt, stream), who);
 }
 

@@ -43,6 +43,7 @@ struct Gemm16Args {
     int64_t stride_a, stride_w, stride_colsum, stride_y;
     int shift;  // used when `shifts` is null (MatMul: one host-side shift)
     int ragged_a;  // RAGGED kernels: how chunks of A's rows may be fetched (load_chunk_ragged)
+    int trans_a;   // RAGGED kernels: A is stored transposed, [K][lda]
 };
 
 // 128 x 128 output tile, K step 64, 4 waves (2 x 2) of 64 x 64, double-buffered LDS holding the two byte
@@ -102,8 +103,9 @@ __global__ __launch_bounds__(256, 2) void gemm_i16i8_kernel(Gemm16Args g) {
             const int c = tid + i * 256, row = c >> 3, kc = (c & 7) * 8;
             const int gm = min(m0 + row, g.M - 1);
             if constexpr (RAGGED)
-                ra[i] = load_chunk_ragged(reinterpret_cast<const int8_t*>(g.A + static_cast<int64_t>(gm) * g.lda + k0 + kc),
-                                          (g.K - (k0 + kc)) * 2, g.ragged_a);
+                ra[i] = g.trans_a ? load_chunk_transposed(reinterpret_cast<const int8_t*>(g.A + gm), g.lda * 2, k0 + kc, g.K, 2)
+                                  : load_chunk_ragged(reinterpret_cast<const int8_t*>(g.A + static_cast<int64_t>(gm) * g.lda + k0 + kc),
+                                                      (g.K - (k0 + kc)) * 2, g.ragged_a);
             else
                 ra[i] = (k0 + kc < g.K) ? *reinterpret_cast<const v4i*>(g.A + static_cast<int64_t>(gm) * g.lda + k0 + kc)
                                         : v4i{0, 0, 0, 0};
@@ -230,6 +232,7 @@ struct Gemm16x16Args {
     int shift_stride, relu, out_kind, mode;
     int64_t stride_a, stride_w, stride_colsum, stride_y;  // batched use, as above
     int shift;                                            // used when `shifts` is null
+    int trans_a;                                          // RAGGED kernels: A is stored transposed, [K][lda]
     int ragged_a;                                         // RAGGED kernels: how chunks of A's rows may be fetched
 };
 
@@ -495,8 +498,9 @@ __global__ __launch_bounds__(256, 2) void gemm_i16i16_kernel(Gemm16x16Args g) {
             const int c = tid + i * 256, row = c >> 3, kc = (c & 7) * 8;
             const int gm = min(m0 + row, g.M - 1);
             if constexpr (RAGGED)
-                ra[i] = load_chunk_ragged(reinterpret_cast<const int8_t*>(g.A + static_cast<int64_t>(gm) * g.lda + k0 + kc),
-                                          (g.K - (k0 + kc)) * 2, g.ragged_a);
+                ra[i] = g.trans_a ? load_chunk_transposed(reinterpret_cast<const int8_t*>(g.A + gm), g.lda * 2, k0 + kc, g.K, 2)
+                                  : load_chunk_ragged(reinterpret_cast<const int8_t*>(g.A + static_cast<int64_t>(gm) * g.lda + k0 + kc),
+                                                      (g.K - (k0 + kc)) * 2, g.ragged_a);
             else
                 ra[i] = (k0 + kc < g.K) ? *reinterpret_cast<const v4i*>(g.A + static_cast<int64_t>(gm) * g.lda + k0 + kc)
                                         : v4i{0, 0, 0, 0};
@@ -739,7 +743,7 @@ static hipError_t launch_pack_rhs(bool wide, const void* B, int64_t ldb, int64_t
 
 using namespace a4g;
 
-extern "C" int a4g_dense_i16(const int16_t* A, int64_t lda, const int8_t* Wt, int64_t ldwt, const int32_t* colsum,
+extern "C" int a4g_dense_i16(const int16_t* A, int trans_a, int64_t lda, const int8_t* Wt, int64_t ldwt, const int32_t* colsum,
                              const int32_t* bias, const int32_t* shifts, int n_shift, int round_mode, int relu, int out_kind,
                              void* Y, int64_t ldy, int64_t M, int64_t N, int64_t K, a4g_stream_t stream_) {
     hipStream_t stream = static_cast<hipStream_t>(stream_);
@@ -751,7 +755,7 @@ extern "C" int a4g_dense_i16(const int16_t* A, int64_t lda, const int8_t* Wt, in
     A4G_REQUIRE(valid_round(round_mode), A4G_ERR_INVALID_ARGUMENT, "%s: unknown rounding mode %d", who, round_mode);
     A4G_REQUIRE(n_shift == 1 || n_shift == N, A4G_ERR_INVALID_ARGUMENT, "%s: n_shift must be 1 or N=%lld, got %d", who,
                 (long long)N, n_shift);
-    A4G_REQUIRE(lda >= K && ldy >= N && ldwt >= K, A4G_ERR_INVALID_ARGUMENT, "%s: pitch smaller than the row", who);
+    A4G_REQUIRE(lda >= (trans_a ? M : K) && ldy >= N && ldwt >= K, A4G_ERR_INVALID_ARGUMENT, "%s: pitch smaller than the row", who);
     if (M == 0) return A4G_OK;
     A4G_REQUIRE(A && Wt && Y && shifts && colsum, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer (the packed colsum vector is required)",
                 who);
@@ -770,14 +774,16 @@ extern "C" int a4g_dense_i16(const int16_t* A, int64_t lda, const int8_t* Wt, in
         r.lda = lda * 2; r.ldb = ldwt; r.ldc = ldy;
         r.M = g.M; r.N = g.N; r.K = g.K;
         r.shift_stride = g.shift_stride; r.relu = g.relu; r.out_kind = out_kind; r.mode = round_mode;
-        if (rs_i16i8_applicable(r, 1)) return check_hip(launch_rs_i16i8(r, 1, stream), who);
+        if (!trans_a && rs_i16i8_applicable(r, 1)) return check_hip(launch_rs_i16i8(r, 1, stream), who);
     }
     const bool w_ok = ldwt % 16 == 0 && aligned16(Wt) && ldwt >= (K + 15) / 16 * 16;  // what a4g_pack_weights_i8 writes
+    A4G_REQUIRE(!trans_a || w_ok, A4G_ERR_UNSUPPORTED, "%s: a transposed left operand needs weights as a4g_pack_weights_i8 writes them", who);
+    g.trans_a = trans_a != 0;
     if (w_ok) {
         const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
         A4G_REQUIRE(tiles <= INT32_MAX, A4G_ERR_UNSUPPORTED, "%s: too many tiles", who);
         const dim3 grid(static_cast<unsigned>(grid_for_tiles(tiles)), 1);  // whole ranges for the 8 XCDs
-        if (K % 16 == 0 && lda % 8 == 0 && aligned16(A)) {
+        if (!trans_a && K % 16 == 0 && lda % 8 == 0 && aligned16(A)) {
             gemm_i16i8_kernel<false><<<grid, 256, tiled16_lds_bytes(g.K, 128), stream>>>(g);
         } else {
             g.ragged_a = ragged_mode(A, lda * 2, 0, K * 2);
@@ -802,7 +808,7 @@ extern "C" int a4g_pack_weights_i16(const int16_t* W, int64_t ldw, int64_t K, in
                      who);
 }
 
-extern "C" int a4g_dense_i16x16(const int16_t* A, int64_t lda, const int8_t* Wt_hi, const int8_t* Wt_lo, int64_t ldwt,
+extern "C" int a4g_dense_i16x16(const int16_t* A, int trans_a, int64_t lda, const int8_t* Wt_hi, const int8_t* Wt_lo, int64_t ldwt,
                                 const int32_t* colsum, const int32_t* bias, const int32_t* shifts, int n_shift, int round_mode,
                                 int relu, int out_kind, void* Y, int64_t ldy, int64_t M, int64_t N, int64_t K,
                                 a4g_stream_t stream_) {
@@ -815,7 +821,7 @@ extern "C" int a4g_dense_i16x16(const int16_t* A, int64_t lda, const int8_t* Wt_
     A4G_REQUIRE(valid_round(round_mode), A4G_ERR_INVALID_ARGUMENT, "%s: unknown rounding mode %d", who, round_mode);
     A4G_REQUIRE(n_shift == 1 || n_shift == N, A4G_ERR_INVALID_ARGUMENT, "%s: n_shift must be 1 or N=%lld, got %d", who,
                 (long long)N, n_shift);
-    A4G_REQUIRE(lda >= K && ldy >= N && ldwt >= K, A4G_ERR_INVALID_ARGUMENT, "%s: pitch smaller than the row", who);
+    A4G_REQUIRE(lda >= (trans_a ? M : K) && ldy >= N && ldwt >= K, A4G_ERR_INVALID_ARGUMENT, "%s: pitch smaller than the row", who);
     if (M == 0) return A4G_OK;
     A4G_REQUIRE(A && Wt_hi && Wt_lo && Y && shifts && colsum, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
     Gemm16x16Args g{};
@@ -833,15 +839,17 @@ extern "C" int a4g_dense_i16x16(const int16_t* A, int64_t lda, const int8_t* Wt_
         r.lda = lda * 2; r.ldb = ldwt; r.ldc = ldy;
         r.M = g.M; r.N = g.N; r.K = g.K;
         r.shift_stride = g.shift_stride; r.relu = g.relu; r.out_kind = out_kind; r.mode = round_mode;
-        if (rs_i16i16_applicable(r, 1))
+        if (!trans_a && rs_i16i16_applicable(r, 1))
             return check_hip(launch_rs_policy<I16x16Policy, 256, 256, 2, 4, true>(r, 1, stream), who);
     }
     const bool w_ok = ldwt % 16 == 0 && aligned16(Wt_hi) && aligned16(Wt_lo) && ldwt >= (K + 15) / 16 * 16;  // a4g_pack_weights_i16
+    A4G_REQUIRE(!trans_a || w_ok, A4G_ERR_UNSUPPORTED, "%s: a transposed left operand needs weights as a4g_pack_weights_i16 writes them", who);
+    g.trans_a = trans_a != 0;
     if (w_ok) {
         const int64_t tiles = ((M + 63) / 64) * ((N + 127) / 128);
         A4G_REQUIRE(tiles <= INT32_MAX, A4G_ERR_UNSUPPORTED, "%s: too many tiles", who);
         const dim3 grid(static_cast<unsigned>(grid_for_tiles(tiles)), 1);
-        if (K % 16 == 0 && lda % 8 == 0 && aligned16(A)) {
+        if (!trans_a && K % 16 == 0 && lda % 8 == 0 && aligned16(A)) {
             gemm_i16i16_kernel<false><<<grid, 256, tiled16_lds_bytes(g.K, 64), stream>>>(g);
         } else {
             g.ragged_a = ragged_mode(A, lda * 2, 0, K * 2);
@@ -861,7 +869,7 @@ extern "C" size_t a4g_matmul_i16_workspace_bytes(int64_t batch, int64_t N, int64
     return static_cast<size_t>(batch * (planes * N * ldt + N * 4));
 }
 
-extern "C" int a4g_matmul_i16(const int16_t* A, int64_t lda, int64_t stride_a, const void* B, int b_kind, int64_t ldb,
+extern "C" int a4g_matmul_i16(const int16_t* A, int trans_a, int64_t lda, int64_t stride_a, const void* B, int b_kind, int64_t ldb,
                               int64_t stride_b, int trans_b, void* C, int64_t ldc, int64_t stride_c, int64_t batch, int64_t M,
                               int64_t N, int64_t K, int shift, int round_mode, int out_kind, void* workspace,
                               size_t workspace_bytes, a4g_stream_t stream_) {
@@ -877,7 +885,8 @@ extern "C" int a4g_matmul_i16(const int16_t* A, int64_t lda, int64_t stride_a, c
     A4G_REQUIRE(valid_round(round_mode), A4G_ERR_INVALID_ARGUMENT, "%s: unknown rounding mode %d", who, round_mode);
     A4G_REQUIRE(shift >= 0 && shift <= (b_kind == A4G_I16 ? 62 : 31), A4G_ERR_INVALID_ARGUMENT,
                 "%s: matmul accumulator output shift %d out of range", who, shift);
-    A4G_REQUIRE(lda >= K && ldc >= N && ldb >= (trans_b ? K : N), A4G_ERR_INVALID_ARGUMENT, "%s: pitch smaller than the row", who);
+    A4G_REQUIRE(lda >= (trans_a ? M : K) && ldc >= N && ldb >= (trans_b ? K : N), A4G_ERR_INVALID_ARGUMENT, "%s: pitch smaller than the row",
+                who);
     if (M == 0 || batch == 0) return A4G_OK;
     A4G_REQUIRE(A && B && C, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
     const size_t need = a4g_matmul_i16_workspace_bytes(batch, N, K, b_kind);
@@ -892,7 +901,7 @@ extern "C" int a4g_matmul_i16(const int16_t* A, int64_t lda, int64_t stride_a, c
     hipError_t e = launch_pack_rhs(wide, B, ldb, stride_b, trans_b, hi, lo, ldt, N * ldt, colsum, batch, (int)K, (int)N, stream);
     if (e != hipSuccess) return check_hip(e, who);
 
-    const bool tiled = K % 16 == 0 && lda % 8 == 0 && stride_a % 8 == 0 && aligned16(A);
+    const bool tiled = !trans_a && K % 16 == 0 && lda % 8 == 0 && stride_a % 8 == 0 && aligned16(A);
     const unsigned nb = static_cast<unsigned>(batch);
     if (wide) {
         Gemm16x16Args g{};
@@ -907,8 +916,9 @@ extern "C" int a4g_matmul_i16(const int16_t* A, int64_t lda, int64_t stride_a, c
         r.stride_colsum = N;
         r.M = g.M; r.N = g.N; r.K = g.K;
         r.shift = shift; r.out_kind = out_kind; r.mode = round_mode;
-        if (rs_i16i16_applicable(r, nb))
+        if (!trans_a && rs_i16i16_applicable(r, nb))
             return check_hip(launch_rs_policy<I16x16Policy, 256, 256, 2, 4, true>(r, nb, stream), who);
+        g.trans_a = trans_a != 0;
         const int64_t tiles = ((M + 63) / 64) * ((N + 127) / 128);
         const dim3 grid(static_cast<unsigned>(grid_for_tiles(tiles)), nb);
         if (tiled) {
@@ -930,7 +940,8 @@ extern "C" int a4g_matmul_i16(const int16_t* A, int64_t lda, int64_t stride_a, c
         r.stride_colsum = N;
         r.M = g.M; r.N = g.N; r.K = g.K;
         r.shift = shift; r.out_kind = out_kind; r.mode = round_mode;
-        if (rs_i16i8_applicable(r, nb)) return check_hip(launch_rs_i16i8(r, nb, stream), who);
+        if (!trans_a && rs_i16i8_applicable(r, nb)) return check_hip(launch_rs_i16i8(r, nb, stream), who);
+        g.trans_a = trans_a != 0;
         const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
         const dim3 grid(static_cast<unsigned>(grid_for_tiles(tiles)), nb);
         if (tiled) {

@@ -64,6 +64,9 @@ struct GemmArgs {
     // only read by the ragged form of the tiled int8 kernel: how a 16-byte chunk of an operand row may be fetched
     // (0 = one aligned load inside the row pitch, 1 = dwords, 2 = bytes); bytes at or past K always read as zero
     int ragged_a, ragged_b;
+    // only read by the ragged forms of gemm_rs_kernel: 0, or the element size in bytes of an A that is stored transposed
+    // ([K][lda]: lda, stride_a and K stay in bytes, K in bytes of a row of the untransposed operand)
+    int trans_a_es;
     // the same weights in fragment order (a4g_rowpack_weights_i8) or null; only Dense kernels that keep weights in
     // registers read it
     const int8_t* Wf;
@@ -240,6 +243,12 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
             // K (bytes here) need not fill its last tile and rows need not be aligned: bytes past K read as zero
             static_assert(!RAGGED || (!P::SPLIT_A && !P::SPLIT_B), "the ragged loads serve the unsplit policies");
             const int rem = g.K - (kt * BK + lchunk * 16);
+            if (idx < Cfg::A_LOADS && g.trans_a_es) {
+                // A stored transposed: the chunk's elements lie a row pitch apart, starting at column m of row k
+                const int es = g.trans_a_es, m = m0 + min(lrow + idx * Cfg::ROWS_PER_PASS, g.M - 1 - m0);
+                ra[idx] = load_chunk_transposed(g.A + tc.batch * g.stride_a + static_cast<int64_t>(m) * es, g.lda, (kt * BK + lchunk * 16) / es, g.K / es, es);
+                return;
+            }
             if (idx < Cfg::A_LOADS) ra[idx] = load_chunk_ragged(Abase + offa[idx] + static_cast<int64_t>(kt) * BK, rem, g.ragged_a);
             else rb[idx - Cfg::A_LOADS] = load_chunk_ragged(Bbase + offb[idx - Cfg::A_LOADS] + static_cast<int64_t>(kt) * BK, rem, g.ragged_b);
             return;

@@ -328,8 +328,15 @@ class MatmulGpuVariant(OpImplVariant):
         a = inputs[lhs_t.name]
         b = inst.artifacts['rhs_const'] if rhs_t.is_parameter else inputs[rhs_t.name]
         ta = bool(cfg.flags.transpose_lhs)
-        if ta and b.dim() == 2 and a.dim() > 2:
-            a, ta = ops.transpose_last2(a), False  # shared rank-2 RHS: rows of every leading index are stacked below
+        if ta and b.dim() == 2 and a.dim() > 2:  # shared rank-2 RHS: one product per leading index, each read as stored
+            import torch
+
+            lead = tuple(a.shape[:-2])
+            a3 = a.reshape((-1,) + tuple(a.shape[-2:]))
+            ys = [ops.matmul(a3[i], b, cfg.shift, cfg.rounding_mode, trans_b=cfg.flags.transpose_rhs,
+                             out_kind=cfg.precision['output'].format, trans_a=True) for i in range(int(a3.shape[0]))]
+            y = torch.stack(ys) if len(ys) != 1 else ys[0][None]
+            return {node.outputs[0].name: y.reshape(lead + tuple(y.shape[-2:]))}
         rows_shape = tuple(a.shape[:-2]) + ((int(a.shape[-1]),) if ta else (int(a.shape[-2]),))
         out_shape = rows_shape + (int(b.shape[-2] if cfg.flags.transpose_rhs else b.shape[-1]),)
         if b.dim() == 2 and a.dim() > 2:

@@ -10,6 +10,8 @@ LayerNorm and Softmax have no float variant there (layer_norm.py:84-85, softmax.
 
 from __future__ import annotations
 
+import torch
+
 from dataclasses import dataclass
 from typing import Any, Dict
 
@@ -194,9 +196,9 @@ class DenseFloatGpuVariant(OpImplVariant):
 
         cfg = inst.config
         x = inputs[input_tensor_for_role(inst.node, 'lhs').name]
-        if cfg.flags.transpose_lhs:
-            x = ops.transpose_last2(x)
-        return {inst.node.outputs[0].name: ops.dense_float(x, inst.artifacts['packed_weights'], relu=cfg.flags.use_relu)}
+        # a transposed input (io_view perm) is read as stored: the kernel transposes its tiles (dense_bias_relu.cpp:95-101)
+        return {inst.node.outputs[0].name: ops.dense_float(x, inst.artifacts['packed_weights'], relu=cfg.flags.use_relu,
+                                                           trans_a=bool(cfg.flags.transpose_lhs))}
 
 
 @register_variant
@@ -239,12 +241,20 @@ class MatmulFloatGpuVariant(OpImplVariant):
         lhs_t, rhs_t = input_tensor_for_role(node, 'lhs'), input_tensor_for_role(node, 'rhs')
         a = inputs[lhs_t.name]
         b = inst.artifacts['rhs_const'] if rhs_t.is_parameter else inputs[rhs_t.name]
-        if cfg.flags.transpose_lhs:
-            a = ops.transpose_last2(a)
-        out_shape = tuple(a.shape[:-1]) + (int(b.shape[-2] if cfg.flags.transpose_rhs else b.shape[-1]),)
+        ta = bool(cfg.flags.transpose_lhs)
+        n_out = int(b.shape[-2] if cfg.flags.transpose_rhs else b.shape[-1])
+        # a transposed left operand (io_view perm) is read as stored: the kernel transposes its tiles (matmul.cpp:60-66)
+        if ta and b.dim() == 2 and a.dim() > 2:  # shared rank-2 RHS: one product per leading index
+            lead = tuple(a.shape[:-2])
+            a3 = a.reshape((-1,) + tuple(a.shape[-2:]))
+            y = torch.empty((a3.shape[0], int(a.shape[-1]), n_out), dtype=a.dtype, device=a.device)
+            for i in range(int(a3.shape[0])):
+                ops.matmul_float(a3[i], b, trans_b=cfg.flags.transpose_rhs, trans_a=True, out=y[i])
+            return {node.outputs[0].name: y.reshape(lead + tuple(y.shape[-2:]))}
+        out_shape = tuple(a.shape[:-2]) + (int(a.shape[-1] if ta else a.shape[-2]), n_out)
         if b.dim() == 2 and a.dim() > 2:
             a = a.reshape(-1, a.shape[-1])
-        y = ops.matmul_float(a, b, trans_b=cfg.flags.transpose_rhs)
+        y = ops.matmul_float(a, b, trans_b=cfg.flags.transpose_rhs, trans_a=ta)
         return {node.outputs[0].name: y.reshape(out_shape)}
 
 

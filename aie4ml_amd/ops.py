@@ -158,15 +158,17 @@ def _rowpack(p: PackedDense) -> torch.Tensor:
 def dense(x: torch.Tensor, p: PackedDense, rounding='floor', relu: bool = False, out_kind='int8',
           out: Optional[torch.Tensor] = None, trans_a: bool = False):
     """y = saturate(round((x @ W + bias) >> shift)), optionally ReLU. x: [..., K] int8 / uint8 / int16.
-    ``trans_a``: x is [..., K, M], the operand is consumed through a last-two-axes transpose view; 8-bit operands are
-    transposed inside the kernel, one launch per leading index."""
+    ``trans_a``: x is [..., K, M], the operand is consumed through a last-two-axes transpose view and transposed inside
+    the kernel, one launch per leading index."""
     if trans_a:
         _dev(x, 'x')
         if x.dim() < 2 or int(x.shape[-2]) != p.K:
             raise ValueError(f'dense input (transposed) has {tuple(x.shape)}, weights expect {p.K} on the second-to-last axis')
-        if x.dtype not in (torch.int8, torch.uint8) or p.wt_lo is not None:
-            # 16-bit operands: the GEMM kernels take K-contiguous rows, the operand is transposed on the device first
-            return dense(transpose_last2(x), p, rounding, relu, out_kind, out)
+        if x.dtype not in (torch.int8, torch.uint8, torch.int16):
+            raise NotImplementedError(f'dense activations must be int8, uint8 or int16, got {x.dtype}')
+        if p.wt_lo is not None and x.dtype != torch.int16:
+            raise RuntimeError('unsupported int8 x int16 precision mix for AIE implementations; no implementation variant '
+                               'available.')
         xs = x.contiguous().reshape(-1, p.K, int(x.shape[-1]))
         Mt = int(xs.shape[-1])
         ok = _kind(out_kind)
@@ -174,10 +176,16 @@ def dense(x: torch.Tensor, p: PackedDense, rounding='floor', relu: bool = False,
             out = torch.empty(tuple(x.shape[:-2]) + (Mt, p.N), dtype=_KIND_TORCH[ok], device=x.device)
         ys = out.reshape(-1, Mt, p.N)
         L = _lib.load()
-        for i in range(int(xs.shape[0])):
-            check(L.a4g_dense_i8(_ptr(xs[i]), _TORCH_KIND[xs.dtype], 1, Mt, _ptr(p.wt), p.ldwt, _ptr(p.colsum), _ptr(p.bias),
-                                 _ptr(p.shifts), int(p.shifts.numel()), _mode(rounding), int(bool(relu)), ok, _ptr(ys[i]), p.N,
-                                 Mt, p.N, p.K, _stream()))
+        tail = (_ptr(p.colsum), _ptr(p.bias), _ptr(p.shifts), int(p.shifts.numel()), _mode(rounding), int(bool(relu)), ok)
+        for i in range(int(xs.shape[0])):  # the operand is transposed inside the kernel, one launch per leading index
+            if p.wt_lo is not None:
+                check(L.a4g_dense_i16x16(_ptr(xs[i]), 1, Mt, _ptr(p.wt), _ptr(p.wt_lo), p.ldwt, *tail, _ptr(ys[i]), p.N, Mt, p.N, p.K,
+                                         _stream()))
+            elif xs.dtype == torch.int16:
+                check(L.a4g_dense_i16(_ptr(xs[i]), 1, Mt, _ptr(p.wt), p.ldwt, *tail, _ptr(ys[i]), p.N, Mt, p.N, p.K, _stream()))
+            else:
+                check(L.a4g_dense_i8(_ptr(xs[i]), _TORCH_KIND[xs.dtype], 1, Mt, _ptr(p.wt), p.ldwt, *tail, _ptr(ys[i]), p.N, Mt, p.N,
+                                     p.K, _stream()))
         return out
     x2 = _rows2d(x, 'x')
     if x2.dtype not in (torch.int8, torch.uint8, torch.int16):
@@ -193,13 +201,13 @@ def dense(x: torch.Tensor, p: PackedDense, rounding='floor', relu: bool = False,
         if x2.dtype != torch.int16:
             raise RuntimeError('unsupported int8 x int16 precision mix for AIE implementations; no implementation variant '
                                'available.')
-        check(_lib.load().a4g_dense_i16x16(_ptr(x2), x2.stride(0) if M > 0 else p.K, _ptr(p.wt), _ptr(p.wt_lo), p.ldwt,
+        check(_lib.load().a4g_dense_i16x16(_ptr(x2), 0, x2.stride(0) if M > 0 else p.K, _ptr(p.wt), _ptr(p.wt_lo), p.ldwt,
                                            _ptr(p.colsum), _ptr(p.bias), _ptr(p.shifts), int(p.shifts.numel()), _mode(rounding),
                                            int(bool(relu)), ok, _ptr(y2), y2.stride(0) if M > 0 else p.N, M, p.N, p.K,
                                            _stream()))
         return out
     if x2.dtype == torch.int16:
-        check(_lib.load().a4g_dense_i16(_ptr(x2), x2.stride(0) if M > 0 else p.K, _ptr(p.wt), p.ldwt, _ptr(p.colsum),
+        check(_lib.load().a4g_dense_i16(_ptr(x2), 0, x2.stride(0) if M > 0 else p.K, _ptr(p.wt), p.ldwt, _ptr(p.colsum),
                                         _ptr(p.bias), _ptr(p.shifts), int(p.shifts.numel()), _mode(rounding),
                                         int(bool(relu)), ok, _ptr(y2), y2.stride(0) if M > 0 else p.N, M, p.N, p.K, _stream()))
         return out
@@ -236,11 +244,9 @@ def _narrow_dense_as_chain(x2: torch.Tensor, p: PackedDense, out_kind: int, rows
 def matmul(a: torch.Tensor, b: torch.Tensor, shift: int, rounding='floor', trans_b: bool = False, out_kind='int8',
            out: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None, trans_a: bool = False):
     """Batched dynamic MatMul. a: [..., M, K] int8/uint8/int16; b: [..., K, N] int8 (int16 with an int16 a), or [..., N, K] when
-    ``trans_b`` (the operand is consumed through a last-two-axes transpose view). ``trans_a``: a is [..., K, M]; an
-    8-bit operand is transposed inside the kernel, a 16-bit one by the library's transpose kernel first."""
+    ``trans_b`` (the operand is consumed through a last-two-axes transpose view). ``trans_a``: a is [..., K, M] and is
+    transposed inside the kernel."""
     _dev(a, 'a'), _dev(b, 'b')
-    if trans_a and a.dtype == torch.int16:
-        a, trans_a = transpose_last2(a), False
     if b.dtype not in (torch.int8, torch.int16):
         raise ValueError('matmul RHS must use a signed integer precision.')
     if a.dtype not in (torch.int8, torch.uint8, torch.int16):
@@ -270,7 +276,7 @@ def matmul(a: torch.Tensor, b: torch.Tensor, shift: int, rounding='floor', trans
         need = int(L.a4g_matmul_i16_workspace_bytes(batch, N, K, bkind))
         if workspace is None or workspace.numel() * workspace.element_size() < need:
             workspace = torch.empty((need,), dtype=torch.uint8, device=a.device)
-        check(L.a4g_matmul_i16(_ptr(a), K, M * K, _ptr(b), bkind, int(b.shape[-1]), K * N, int(bool(trans_b)), _ptr(out), N, M * N,
+        check(L.a4g_matmul_i16(_ptr(a), int(bool(trans_a)), M if trans_a else K, M * K, _ptr(b), bkind, int(b.shape[-1]), K * N, int(bool(trans_b)), _ptr(out), N, M * N,
                                batch, M, N, K, int(shift), _mode(rounding), ok, _ptr(workspace),
                                workspace.numel() * workspace.element_size(), _stream()))
         return out
@@ -633,8 +639,26 @@ def pack_dense_float(weight: torch.Tensor, bias: Optional[torch.Tensor]) -> Pack
     return PackedDenseFloat(wt=wt, bias=bias, K=K, N=N)
 
 
-def dense_float(x: torch.Tensor, p: PackedDenseFloat, relu: bool = False, out: Optional[torch.Tensor] = None):
-    """y = fmt(relu?(bias + x @ W)) with float32 accumulation; x: [..., K] in the weights' format."""
+def dense_float(x: torch.Tensor, p: PackedDenseFloat, relu: bool = False, out: Optional[torch.Tensor] = None,
+                trans_a: bool = False):
+    """y = fmt(relu?(bias + x @ W)) with float32 accumulation; x: [..., K] in the weights' format. ``trans_a``: x is
+    [..., K, M] and is transposed inside the kernel, one launch per leading index."""
+    if trans_a:
+        _dev(x, 'x')
+        fmt = _float_format(x, 'x')
+        if x.dtype != p.wt.dtype:
+            raise ValueError(f'float dense requires lhs/rhs/output to share float precision, got {x.dtype} and {p.wt.dtype}.')
+        if x.dim() < 2 or int(x.shape[-2]) != p.K:
+            raise ValueError(f'dense input (transposed) has {tuple(x.shape)}, weights expect {p.K} on the second-to-last axis')
+        xs = x.contiguous().reshape(-1, p.K, int(x.shape[-1]))
+        Mt = int(xs.shape[-1])
+        if out is None:
+            out = torch.empty(tuple(x.shape[:-2]) + (Mt, p.N), dtype=x.dtype, device=x.device)
+        ys = out.reshape(-1, Mt, p.N)
+        for i in range(int(xs.shape[0])):
+            check(_lib.load().a4g_dense_f(_ptr(xs[i]), fmt, 1, Mt, _ptr(p.wt), p.ldwt, _ptr(p.bias), int(bool(relu)), _ptr(ys[i]), p.N,
+                                          Mt, p.N, p.K, _stream()))
+        return out
     x2 = _rows2d(x, 'x')
     fmt = _float_format(x2, 'x')
     if x2.dtype != p.wt.dtype:
@@ -645,14 +669,15 @@ def dense_float(x: torch.Tensor, p: PackedDenseFloat, relu: bool = False, out: O
     if out is None:
         out = torch.empty(tuple(x.shape[:-1]) + (p.N,), dtype=x.dtype, device=x.device)
     y2 = out.reshape(-1, p.N)
-    check(_lib.load().a4g_dense_f(_ptr(x2), fmt, x2.stride(0) if M > 0 else p.K, _ptr(p.wt), p.ldwt, _ptr(p.bias),
+    check(_lib.load().a4g_dense_f(_ptr(x2), fmt, 0, x2.stride(0) if M > 0 else p.K, _ptr(p.wt), p.ldwt, _ptr(p.bias),
                                   int(bool(relu)), _ptr(y2), y2.stride(0) if M > 0 else p.N, M, p.N, p.K, _stream()))
     return out
 
 
 def matmul_float(a: torch.Tensor, b: torch.Tensor, trans_b: bool = False, out: Optional[torch.Tensor] = None,
-                 workspace: Optional[torch.Tensor] = None):
-    """Batched float MatMul. a: [..., M, K]; b: [..., K, N], or [..., N, K] when ``trans_b``."""
+                 workspace: Optional[torch.Tensor] = None, trans_a: bool = False):
+    """Batched float MatMul. a: [..., M, K] (``trans_a``: [..., K, M], transposed inside the kernel); b: [..., K, N], or
+    [..., N, K] when ``trans_b``."""
     _dev(a, 'a'), _dev(b, 'b')
     fmt = _float_format(a, 'a')
     if a.dtype != b.dtype:
@@ -660,7 +685,7 @@ def matmul_float(a: torch.Tensor, b: torch.Tensor, trans_b: bool = False, out: O
     if a.dim() < 2 or b.dim() < 2:
         raise ValueError('matmul operands need rank >= 2')
     a, b = a.contiguous(), b.contiguous()
-    M, K = int(a.shape[-2]), int(a.shape[-1])
+    M, K = (int(a.shape[-1]), int(a.shape[-2])) if trans_a else (int(a.shape[-2]), int(a.shape[-1]))
     N = int(b.shape[-2] if trans_b else b.shape[-1])
     Kb = int(b.shape[-1] if trans_b else b.shape[-2])
     if K != Kb:
@@ -678,7 +703,7 @@ def matmul_float(a: torch.Tensor, b: torch.Tensor, trans_b: bool = False, out: O
     if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
         workspace = torch.empty((need,), dtype=torch.uint8, device=a.device)
     ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
-    check(L.a4g_matmul_f(_ptr(a), fmt, K, M * K, _ptr(b), int(b.shape[-1]), K * N, int(bool(trans_b)), _ptr(out), N, M * N,
+    check(L.a4g_matmul_f(_ptr(a), fmt, int(bool(trans_a)), M if trans_a else K, M * K, _ptr(b), int(b.shape[-1]), K * N, int(bool(trans_b)), _ptr(out), N, M * N,
                          batch, M, N, K, _ptr(workspace), ws_bytes, _stream()))
     return out
 

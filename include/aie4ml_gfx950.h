@@ -28,7 +28,10 @@
 extern "C" {
 #endif
 
-#define A4G_VERSION 203 /* major*10000 + minor*100 + patch */
+/* Interface revision. Revisions 2xx and 3xx changed signatures that existed before (2xx: `trans_a` in a4g_dense_i8 and
+ * a4g_matmul_i8; 3xx: `trans_a` in the 16-bit and floating-point Dense and MatMul), so a caller compiled against an
+ * older header must not bind a newer library: compare a4g_version() with the header's value at load time. */
+#define A4G_VERSION 300
 
 #if defined(__GNUC__)
 #define A4G_API __attribute__((visibility("default")))
@@ -69,9 +72,10 @@ A4G_API const char* a4g_last_error(void);
 /* Dynamic MatMul with an int16 left operand: the (16, 8) and (16, 16) width combinations of the matmul family
  * (op_impls/families/matmul/common.py:52; docs/support.md: "Dynamic MatMul: Int8/int16"), acc32 and acc64 as for
  * Dense. B is int8 or int16 (b_kind), [batch][K][ldb] or, with trans_b, [batch][N][ldb]; it is repacked per call
- * into the workspace (a4g_matmul_i16_workspace_bytes). Other arguments as a4g_matmul_i8. */
+ * into the workspace (a4g_matmul_i16_workspace_bytes). Other arguments as a4g_matmul_i8, `trans_a` included: the left
+ * operand stored as [batch][K][lda], lda >= M (TRANSPOSE_A, matmul.cpp:60-66), gathered while its tiles are staged. */
 A4G_API size_t a4g_matmul_i16_workspace_bytes(int64_t batch, int64_t N, int64_t K, int b_kind);
-A4G_API int a4g_matmul_i16(const int16_t* A, int64_t lda, int64_t stride_a, const void* B, int b_kind, int64_t ldb,
+A4G_API int a4g_matmul_i16(const int16_t* A, int trans_a, int64_t lda, int64_t stride_a, const void* B, int b_kind, int64_t ldb,
                    int64_t stride_b, int trans_b, void* C, int64_t ldc, int64_t stride_c, int64_t batch, int64_t M,
                    int64_t N, int64_t K, int shift, int round_mode, int out_kind, void* workspace, size_t workspace_bytes,
                    a4g_stream_t stream);
@@ -129,8 +133,9 @@ A4G_API int a4g_dense_i8_wf(const void* A, int a_kind, int trans_a, int64_t lda,
  * (op_impls/families/matmul/common.py:52), accumulated in acc32 like the 8-bit case
  * (op_impls/utils/precision.py:120-121). Same arguments as a4g_dense_i8 with A [M][lda] int16 (lda in
  * elements); colsum (from a4g_pack_weights_i8) is always required: the low bytes of A are fed to the
- * matrix cores biased by 128. */
-A4G_API int a4g_dense_i16(const int16_t* A, int64_t lda, const int8_t* Wt, int64_t ldwt, const int32_t* colsum,
+ * matrix cores biased by 128. trans_a != 0: A is stored transposed, [K][lda] with lda >= M, and gathered while its
+ * tiles are staged (TRANSPOSE_A, dense_bias_relu.cpp:95-101); the weights must then be a4g_pack_weights_i8's. */
+A4G_API int a4g_dense_i16(const int16_t* A, int trans_a, int64_t lda, const int8_t* Wt, int64_t ldwt, const int32_t* colsum,
                   const int32_t* bias, const int32_t* shifts, int n_shift, int round_mode, int relu, int out_kind,
                   void* Y, int64_t ldy, int64_t M, int64_t N, int64_t K, a4g_stream_t stream);
 
@@ -138,10 +143,10 @@ A4G_API int a4g_dense_i16(const int16_t* A, int64_t lda, const int8_t* Wt, int64
  * (op_impls/families/matmul/common.py:52, op_impls/utils/precision.py:122-123), bias int32 at the accumulator
  * scale. a4g_pack_weights_i16 turns W [K][ldw] int16 into two byte planes [N][ld] (ld = K rounded up to 16:
  * signed high bytes; low bytes ^ 0x80) and colsum[n] = sum_k (W[k][n] - 128); K <= 32768 keeps every partial
- * sum exact. Shifts up to 62. Other arguments as a4g_dense_i8. */
+ * sum exact. Shifts up to 62. Other arguments as a4g_dense_i16. */
 A4G_API int a4g_pack_weights_i16(const int16_t* W, int64_t ldw, int64_t K, int64_t N, int8_t* Wt_hi, int8_t* Wt_lo,
                          int32_t* colsum, a4g_stream_t stream);
-A4G_API int a4g_dense_i16x16(const int16_t* A, int64_t lda, const int8_t* Wt_hi, const int8_t* Wt_lo, int64_t ldwt,
+A4G_API int a4g_dense_i16x16(const int16_t* A, int trans_a, int64_t lda, const int8_t* Wt_hi, const int8_t* Wt_lo, int64_t ldwt,
                      const int32_t* colsum, const int32_t* bias, const int32_t* shifts, int n_shift, int round_mode,
                      int relu, int out_kind, void* Y, int64_t ldy, int64_t M, int64_t N, int64_t K, a4g_stream_t stream);
 
@@ -316,15 +321,16 @@ A4G_API int64_t a4g_packed_ld_f(int64_t K, int fmt);
 A4G_API int a4g_pack_weights_f(const void* W, int fmt, int64_t ldw, int64_t K, int64_t N, void* Wt, a4g_stream_t stream);
 /* Y = fmt(relu?(bias + A x W)). Replaces dense_single<Cfg>::run with float types,
  * templates/nnet_utils/dense_bias_relu/dense_bias_relu.cpp:66-166 (the bias is the accumulator's start
- * value, :112-124). A [M][lda], Wt packed, bias float32 [N] or null, Y [M][ldy]. */
-A4G_API int a4g_dense_f(const void* A, int fmt, int64_t lda, const void* Wt, int64_t ldwt, const float* bias, int relu, void* Y,
+ * value, :112-124). A [M][lda] (trans_a != 0: stored transposed, [K][lda] with lda >= M, TRANSPOSE_A of
+ * dense_bias_relu.cpp:95-101, gathered while its tiles are staged), Wt packed, bias float32 [N] or null, Y [M][ldy]. */
+A4G_API int a4g_dense_f(const void* A, int fmt, int trans_a, int64_t lda, const void* Wt, int64_t ldwt, const float* bias, int relu, void* Y,
                 int64_t ldy, int64_t M, int64_t N, int64_t K, a4g_stream_t stream);
 /* C[b] = fmt(A[b] x B[b]). Replaces matmul_single<Cfg>::run with float types,
  * templates/nnet_utils/matmul/matmul.cpp:31-118. trans_b != 0: B is [batch][N][ldb] (the io_view swap of
  * matmul.py:84-98); otherwise B is [batch][K][ldb] and a workspace of a4g_matmul_f_workspace_bytes()
- * holds its transpose. */
+ * holds its transpose. trans_a != 0: A is [batch][K][lda], lda >= M (TRANSPOSE_A, matmul.cpp:60-66). */
 A4G_API size_t a4g_matmul_f_workspace_bytes(int64_t batch, int64_t N, int64_t K, int trans_b, int fmt);
-A4G_API int a4g_matmul_f(const void* A, int fmt, int64_t lda, int64_t stride_a, const void* B, int64_t ldb, int64_t stride_b,
+A4G_API int a4g_matmul_f(const void* A, int fmt, int trans_a, int64_t lda, int64_t stride_a, const void* B, int64_t ldb, int64_t stride_b,
                  int trans_b, void* C, int64_t ldc, int64_t stride_c, int64_t batch, int64_t M, int64_t N, int64_t K,
                  void* workspace, size_t workspace_bytes, a4g_stream_t stream);
 /* out[i] = fmt(a[i] + b[i]). Replaces elementwise_add_kernel<Cfg>::run with float types,
@@ -335,9 +341,8 @@ A4G_API int a4g_add_f(const void* a, const void* b, void* out, int64_t n, int fm
  * dst[b][c][r] = src[b][r][c] for elements of 1, 2 or 4 bytes; pitches and batch strides in elements.
  * The kernels of the reference read a transposed operand through a transposing load
  * (templates/nnet_utils/matmul/matmul.cpp:60-66, dense_bias_relu.cpp:95-101, selected by transpose_lhs / transpose_rhs of
- * op_impls/families/matmul/matmul.py:78-98). The 8-bit entry points do the same (`trans_a`, `trans_b`); for the 16-bit
- * and floating-point entry points, which take a K-contiguous left operand, a caller turns a [K][M] operand into
- * [M][K] with this call, on the device and in memory it owns. */
+ * op_impls/families/matmul/matmul.py:78-98), and so does every Dense and MatMul entry point here (`trans_a`, `trans_b`).
+ * This call is for a caller that wants the transposed copy itself, on the device and in memory it owns. */
 A4G_API int a4g_transpose(const void* src, int elem_bytes, int64_t ld_src, int64_t stride_src, void* dst, int64_t ld_dst,
                   int64_t stride_dst, int64_t batch, int64_t rows, int64_t cols, a4g_stream_t stream);
 

@@ -46,7 +46,7 @@ def test_binding_table_matches_header(libpath):
 
     assert sorted(_lib.SIGNATURES) == declared_symbols()
     lib = _lib.load()
-    assert lib.a4g_version() == 203
+    assert lib.a4g_version() == _lib.EXPECTED_VERSION == 300
     assert lib.a4g_packed_ld(1) == 16 and lib.a4g_packed_ld(16) == 16 and lib.a4g_packed_ld(17) == 32
     # pure host-side query, no GPU needed: K x N operand transposed into the workspace + colsum
     assert lib.a4g_matmul_i8_workspace_bytes(2, 8, 64, 512, 1, 0) == 0

@@ -113,6 +113,31 @@ def test_matmul_float(ops, oracle, fmt, trans_b, shape):
 
 
 @pytest.mark.parametrize('fmt', FORMATS)
+@pytest.mark.parametrize('shape', [((), 64, 64, 64), ((3,), 130, 70, 48), ((2,), 50, 17, 24), ((), 300, 256, 128)])
+def test_transposed_lhs_in_kernel_float(ops, oracle, fmt, shape):
+    """Float Dense and MatMul read a left operand stored as [..., K, M] themselves (TRANSPOSE_A, matmul.cpp:60-66,
+    dense_bias_relu.cpp:95-101); same tolerances as the untransposed operand, against the oracle on the materialised
+    transpose."""
+    lead, M, K, N = shape
+    r = np.random.default_rng(M * 5 + K + N)
+    At = operand(r, lead + (K, M), fmt, oracle)
+    A = np.ascontiguousarray(np.swapaxes(At, -1, -2))
+    W = operand(r, (K, N), fmt, oracle, 0.1)
+    b = r.normal(0, 0.05, N).astype(np.float32)
+    p = ops.pack_dense_float(dev(W, fmt), torch.from_numpy(b).cuda())
+    got = host(ops.dense_float(dev(At, fmt), p, relu=True, trans_a=True))
+    absprod = np.abs(A).astype(np.float64) @ np.abs(W).astype(np.float64) + np.abs(b)
+    want = oracle.dense_float(A.reshape(-1, K), W, b, relu=True, fmt=fmt).reshape(lead + (M, N))
+    check(got, want, fmt, K, absprod)
+    for trans_b in (True, False):
+        B = operand(r, lead + ((N, K) if trans_b else (K, N)), fmt, oracle)
+        got = host(ops.matmul_float(dev(At, fmt), dev(B, fmt), trans_b=trans_b, trans_a=True))
+        Bm = np.swapaxes(B, -1, -2) if trans_b else B
+        absprod = np.abs(A).astype(np.float64) @ np.abs(Bm).astype(np.float64)
+        check(got, oracle.matmul_float(A, B, trans_b=trans_b, fmt=fmt), fmt, K, absprod)
+
+
+@pytest.mark.parametrize('fmt', FORMATS)
 def test_add_float(ops, oracle, fmt):
     r = np.random.default_rng(9)
     a = operand(r, (5, 1001), fmt, oracle, 3.0)

@@ -468,6 +468,32 @@ def test_dense_transposed_lhs_in_kernel(ops, oracle, shape):
         assert np.array_equal(got, want)
 
 
+@pytest.mark.parametrize('wide', [False, True])
+@pytest.mark.parametrize('shape', [((), 64, 64, 64), ((3,), 130, 70, 48), ((2,), 33, 19, 100), ((), 1000, 200, 512), ((), 517, 260, 203)])
+def test_transposed_lhs_in_kernel_16_bit(ops, oracle, shape, wide):
+    """The 16-bit Dense and MatMul entry points read a left operand stored as [..., K, M] themselves (TRANSPOSE_A,
+    matmul.cpp:60-66, dense_bias_relu.cpp:95-101): (16, 8) and (16, 16), every leading index, reductions off the tile grid,
+    checked against the oracle on the materialised transpose."""
+    lead, M, N, K = shape
+    r = rng(11 * M + N + K + wide)
+    At = r.integers(-32768, 32768, lead + (K, M)).astype(np.int16)
+    A = np.ascontiguousarray(np.swapaxes(At, -1, -2))
+    W = r.integers(-32768, 32768, (K, N)).astype(np.int16) if wide else gauss8(r, 16, (K, N))
+    bias = r.integers(-20000, 20000, N).astype(np.int32)
+    shifts = r.integers(17, 23, N).astype(np.int32) if wide else r.integers(9, 15, N).astype(np.int32)
+    p = ops.pack_dense(dev(W), dev(bias), shifts)
+    for mode, kind, relu in (('conv_even', 'int16', False), ('symmetric_inf', 'int8', True)):
+        got = host(ops.dense(dev(At), p, mode, relu=relu, out_kind=kind, trans_a=True))
+        want = oracle.dense(A.reshape(-1, K), W, bias, shifts, mode, relu=relu, out=kind).reshape(lead + (M, N))
+        assert np.array_equal(got, want), ('dense', mode, kind)
+    for trans_b in (True, False):
+        B = (r.integers(-32768, 32768, lead + ((N, K) if trans_b else (K, N))).astype(np.int16) if wide
+             else gauss8(r, 24, lead + ((N, K) if trans_b else (K, N))))
+        sh = 22 if wide else 14
+        got = host(ops.matmul(dev(At), dev(B), sh, 'conv_even', trans_b=trans_b, out_kind='int16', trans_a=True))
+        assert np.array_equal(got, oracle.matmul(A, B, sh, 'conv_even', trans_b=trans_b, out='int16')), ('matmul', trans_b)
+
+
 @pytest.mark.parametrize('trans_b', [True, False])
 def test_matmul_unsigned_lhs(ops, oracle, trans_b):
     r = rng(9)
