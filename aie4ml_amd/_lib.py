@@ -98,8 +98,6 @@ SIGNATURES = {
                             _vp]),
     'a4g_add_f': (_i32, [_vp, _vp, _vp, _i64, _i32, _vp]),
     'a4g_transpose': (_i32, [_vp, _i32, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
-    'a4g_calib_mfma_i8_ops': (_i64, [_i32, _i32]),
-    'a4g_calib_mfma_i8': (_i32, [_i32, _i32, _vp, _vp, _vp]),
 }
 
 _lib = None

@@ -283,13 +283,16 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
                 e2 = left > 2 ? e2 : 0;
                 e3 = left > 3 ? e3 : 0;
             }
-            sum += (e0 + e1) + (e2 + e3);
+            // scores are at most 32767: both halves of a pair are summed by one dot product with (1, 1)
+            const unsigned p01 = pack2_halves(e0, e1), p23 = pack2_halves(e2, e3);
+            sum = static_cast<int>(__builtin_amdgcn_udot2(__builtin_bit_cast(v2us, p01), __builtin_bit_cast(v2us, 0x00010001u), static_cast<unsigned>(sum), false));
+            sum = static_cast<int>(__builtin_amdgcn_udot2(__builtin_bit_cast(v2us, p23), __builtin_bit_cast(v2us, 0x00010001u), static_cast<unsigned>(sum), false));
             if (t >= NT - PARK) {
-                parked[((t - (NT - PARK)) * 8 + 2 * g) * THREADS + tid] = pack2_halves(e0, e1);
-                parked[((t - (NT - PARK)) * 8 + 2 * g + 1) * THREADS + tid] = pack2_halves(e2, e3);
+                parked[((t - (NT - PARK)) * 8 + 2 * g) * THREADS + tid] = p01;
+                parked[((t - (NT - PARK)) * 8 + 2 * g + 1) * THREADS + tid] = p23;
             } else {
-                ep[t][2 * g] = pack2_halves(e0, e1);
-                ep[t][2 * g + 1] = pack2_halves(e2, e3);
+                ep[t][2 * g] = p01;
+                ep[t][2 * g + 1] = p23;
             }
         }
         // keep the scheduler from hoisting many tiles' lookups at once (their results would spill)
@@ -316,8 +319,11 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
                 unsigned q[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
+                    // score (one half of its register, picked by the instruction) times inv16, which is below 2^16 whenever
+                    // no clamp is needed (255 * 65536 / the smallest possible row sum): p in bits 16..23, nothing above
                     const unsigned pair = ep[t][2 * g + (i >> 1)];
-                    q[i] = __umul24((i & 1) ? (pair >> 16) : (pair & 0xFFFFu), inv16);  // p in bits 16..23, nothing above
+                    if (i & 1) asm("v_mad_u32_u16 %0, %1, %2, 0 op_sel:[1,0,0,0]" : "=v"(q[i]) : "v"(pair), "v"(inv16));
+                    else asm("v_mad_u32_u16 %0, %1, %2, 0" : "=v"(q[i]) : "v"(pair), "v"(inv16));
                 }
                 const unsigned lo = __builtin_amdgcn_perm(q[1], q[0], 0x0c0c0602u);
                 const unsigned hi = __builtin_amdgcn_perm(q[3], q[2], 0x06020c0cu);

@@ -1,6 +1,7 @@
 // Calibration kernels: what the int8 matrix cores of this GPU sustain with no memory traffic at all, and the clock
 // they run at while doing so. bench.py times them beside the GEMM so that "fraction of the 5.0 POP/s data-sheet peak"
-// can be read next to "fraction of what this box sustains".
+// can be read next to "fraction of what this box sustains". A measurement aid with no counterpart in the reference:
+// it is built into a library of its own (libaie4ml_bench_gfx950.so), not into the one an integrator ships.
 #include "common.hpp"
 
 namespace a4g {
@@ -9,20 +10,22 @@ namespace a4g {
 // v_mfma_i32_32x32x32_i8 back to back on operands that never leave registers. Two operand sets alternate so that the
 // multiplier inputs toggle the way streamed operands do. clocks[2*block] = shader-clock ticks, [2*block+1] = ticks of
 // the 100 MHz constant counter over the same interval (wave 0 of each workgroup).
-__global__ __launch_bounds__(256) void calib_mfma_i8_kernel(int iters, int* __restrict__ sink,
+// `zero`: all-zero operands instead (the same instruction stream with nothing toggling in the multipliers: what the
+// power limit leaves when the data costs nothing).
+__global__ __launch_bounds__(256) void calib_mfma_i8_kernel(int iters, int zero, int* __restrict__ sink,
                                                             unsigned long long* __restrict__ clocks) {
-    const unsigned seed = (blockIdx.x * 256u + threadIdx.x) * 2654435761u;
+    const unsigned seed = zero ? 0u : (blockIdx.x * 256u + threadIdx.x) * 2654435761u;
     v4i a[2][4], b[2][2];
 #pragma unroll
     for (int s = 0; s < 2; ++s) {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) a[s][i][r] = static_cast<int>((seed ^ (0x9E3779B9u * (s * 16 + i * 4 + r + 1))) * 0x85EBCA6Bu);
+            for (int r = 0; r < 4; ++r) a[s][i][r] = zero ? 0 : static_cast<int>((seed ^ (0x9E3779B9u * (s * 16 + i * 4 + r + 1))) * 0x85EBCA6Bu);
 #pragma unroll
         for (int j = 0; j < 2; ++j)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) b[s][j][r] = static_cast<int>((seed ^ (0xC2B2AE35u * (s * 8 + j * 4 + r + 1))) * 0x27D4EB2Fu);
+            for (int r = 0; r < 4; ++r) b[s][j][r] = zero ? 0 : static_cast<int>((seed ^ (0xC2B2AE35u * (s * 8 + j * 4 + r + 1))) * 0x27D4EB2Fu);
     }
     v16i acc[4][2];
 #pragma unroll
@@ -62,15 +65,16 @@ __global__ __launch_bounds__(256) void calib_mfma_i8_kernel(int iters, int* __re
 
 using namespace a4g;
 
-extern "C" int64_t a4g_calib_mfma_i8_ops(int blocks, int iters) {
-    // per wave and iteration: 2 operand sets x 8 MFMAs x 2 * 32 * 32 * 32 operations; 4 waves per workgroup
-    return static_cast<int64_t>(blocks) * 4 * iters * 16 * 65536;
-}
+#define A4G_BENCH_API extern "C" __attribute__((visibility("default")))
 
-extern "C" int a4g_calib_mfma_i8(int blocks, int iters, int* sink, unsigned long long* clocks, a4g_stream_t stream_) {
-    A4G_REQUIRE(blocks >= 1 && blocks <= (1 << 20) && iters >= 1 && iters <= (1 << 24), A4G_ERR_INVALID_ARGUMENT,
-                "a4g_calib_mfma_i8: blocks %d / iters %d out of range", blocks, iters);
-    A4G_REQUIRE(sink != nullptr, A4G_ERR_INVALID_ARGUMENT, "a4g_calib_mfma_i8: null sink");
-    calib_mfma_i8_kernel<<<blocks, 256, 0, static_cast<hipStream_t>(stream_)>>>(iters, sink, clocks);
-    return check_hip(hipGetLastError(), "a4g_calib_mfma_i8");
+// operations of one launch: per wave and iteration 2 operand sets x 8 MFMAs x 2 * 32 * 32 * 32; 4 waves per workgroup
+A4G_BENCH_API int64_t a4g_calib_mfma_i8_ops(int blocks, int iters) { return static_cast<int64_t>(blocks) * 4 * iters * 16 * 65536; }
+
+// 0, or -1 for arguments out of range, or a HIP error code. clocks (nullable, 2 * blocks entries) receives per workgroup
+// the shader-clock ticks and the 100 MHz counter ticks over the loop; sink: one int of device memory (never written in
+// practice).
+A4G_BENCH_API int a4g_calib_mfma_i8(int blocks, int iters, int zero, int* sink, unsigned long long* clocks, void* stream) {
+    if (blocks < 1 || blocks > (1 << 20) || iters < 1 || iters > (1 << 24) || sink == nullptr) return -1;
+    calib_mfma_i8_kernel<<<blocks, 256, 0, static_cast<hipStream_t>(stream)>>>(iters, zero, sink, clocks);
+    return static_cast<int>(hipGetLastError());
 }

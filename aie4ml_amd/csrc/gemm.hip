@@ -885,12 +885,18 @@ constexpr int kMaxDevices = 64;
 std::mutex scratch_mutex;
 void* scratch_ptr[kMaxDevices] = {};  // device address of `scratch` on each device, resolved once
 
-int static_scratch(const char* who, void** out) {
+int static_scratch(const char* who, hipStream_t stream, void** out) {
     int dev = -1;
     if (int st = check_hip(hipGetDevice(&dev), who)) return st;
     A4G_REQUIRE(dev >= 0 && dev < kMaxDevices, A4G_ERR_UNSUPPORTED, "%s: device ordinal %d beyond %d", who, dev, kMaxDevices);
     std::lock_guard<std::mutex> lock(scratch_mutex);
     if (!scratch_ptr[dev]) {
+        // Resolving the symbol is not a call a stream capture survives: the first call on a device has to come before any
+        // capture, and says so instead of breaking the capture with an error nobody can place.
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (int st = check_hip(hipStreamIsCapturing(stream, &cap), who)) return st;
+        A4G_REQUIRE(cap == hipStreamCaptureStatusNone, A4G_ERR_UNSUPPORTED,
+                    "%s: the first call on a device must be made outside stream capture (it resolves the scratch array's address)", who);
         void* p = nullptr;
         if (int st = check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), who)) return st;
         A4G_REQUIRE(p != nullptr && aligned16(p), A4G_ERR_HIP, "%s: the scratch array resolved to a bad address", who);
@@ -948,7 +954,7 @@ static int matmul_i8_impl(const char* who, bool own_scratch, const void* A, int 
                     "%s: the repacked right operand needs %zu bytes, the static scratch array holds %zu "
                     "(A4G_MATMUL_I8_STATIC_MAX_BYTES); use a4g_matmul_i8 with a workspace of that size",
                     who, need, workspace_bytes);
-        if (int st = static_scratch(who, &workspace)) return st;
+        if (int st = static_scratch(who, stream, &workspace)) return st;
     }
     A4G_REQUIRE(need == 0 || (workspace && workspace_bytes >= need), A4G_ERR_WORKSPACE,
                 "%s: workspace of %zu bytes required, got %zu", who, need, workspace ? workspace_bytes : (size_t)0);

@@ -383,7 +383,7 @@ class GPUModel:
             rows *= int(d)
         shapes = [(s.params.K, s.params.N) for s in specs]
         x_pitch = int(x.shape[-1]) if x.is_contiguous() else 0
-        if _mlp_layers_are_faster(rows, shapes, ops.mlp_runs_on_matrix_units(rows, x_pitch, shapes)):
+        if _mlp_layers_are_faster(rows, shapes, ops.mlp_runs_on_matrix_units(rows, x_pitch, shapes, specs[-1].out_kind)):
             for inst in insts:  # wide layers on a large batch: one GEMM per layer beats the launch that keeps weights in LDS
                 values.update(inst.variant.run(inst, {input_tensor_for_role(inst.node, 'lhs').name:
                                                       values[input_tensor_for_role(inst.node, 'lhs').name]}))

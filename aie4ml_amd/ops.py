@@ -43,6 +43,21 @@ def _ptr(t: Optional[torch.Tensor]):
     return ctypes.c_void_p(t.data_ptr()) if t is not None else None
 
 
+def _pitched_rows(t: torch.Tensor, name: str) -> torch.Tensor:
+    """t as a 2-D [rows, cols] view whose rows the kernels can read in place: a contiguous last axis, a row pitch that is
+    a multiple of 16 bytes and a 16-byte aligned start (a column window of a wider tensor qualifies); anything else is
+    copied to a dense buffer."""
+    t2 = _rows2d(t, name)
+    if t2.dim() == 2 and t2.stride(1) == 1 and (t2.shape[0] <= 1 or (t2.stride(0) * t2.element_size()) % 16 == 0) \
+            and t2.data_ptr() % 16 == 0 and (t2.shape[0] <= 1 or t2.stride(0) >= t2.shape[1]):
+        return t2
+    return t2.contiguous()
+
+
+def _pitch(t2: torch.Tensor) -> int:
+    return int(t2.stride(0)) if t2.shape[0] > 1 else int(t2.shape[1])
+
+
 def _stream() -> ctypes.c_void_p:
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
@@ -371,7 +386,7 @@ def dense_add_layernorm(x: torch.Tensor, p: PackedDense, residual: Optional[torc
     if residual is not None:
         if residual.dtype != torch.int8 or tuple(residual.shape) != tuple(x.shape[:-1]) + (p.N,):
             raise ValueError('dense_add_layernorm: the residual must be an int8 tensor of the output shape')
-        r2 = _rows2d(residual, 'residual').contiguous()
+        r2 = _pitched_rows(residual, 'residual')  # a window of a wider tensor is read where it lies
     g = _dev(gamma_q7, 'gamma').to(torch.int16).contiguous()
     bt = _dev(beta_q15, 'beta').to(torch.int16).contiguous()
     if g.numel() != p.N or bt.numel() != p.N:
@@ -380,11 +395,15 @@ def dense_add_layernorm(x: torch.Tensor, p: PackedDense, residual: Optional[torc
     _rowpack(p)
     if out is None:
         out = torch.empty(tuple(x.shape[:-1]) + (p.N,), dtype=torch.int8, device=x.device)
-    elif tuple(out.shape) != tuple(x.shape[:-1]) + (p.N,) or out.dtype != torch.int8 or not out.is_contiguous():
-        raise ValueError('dense_add_layernorm: out must be a contiguous int8 tensor of the output shape')
+    elif tuple(out.shape) != tuple(x.shape[:-1]) + (p.N,) or out.dtype != torch.int8:
+        raise ValueError('dense_add_layernorm: out must be an int8 tensor of the output shape')
+    o2 = _pitched_rows(out, 'out')
+    if o2.data_ptr() != out.data_ptr():
+        raise ValueError('dense_add_layernorm: out needs a contiguous last axis, a row pitch in whole 16 bytes and a 16-byte aligned start')
     check(L.a4g_dense_add_layernorm_i8(_ptr(x2), _TORCH_KIND[x2.dtype], x2.stride(0) if M > 0 else p.K, _ptr(p.wf),
                                        _ptr(p.colsum), _ptr(p.bias), int(p.shift0), _mode(dense_rounding), int(bool(relu)),
-                                       _ptr(r2), p.N, _ptr(g), _ptr(bt), _ptr(out), p.N, M, p.N, p.K, int(eps_q0),
+                                       _ptr(r2), _pitch(r2) if r2 is not None else p.N, _ptr(g), _ptr(bt), _ptr(o2),
+                                       _pitch(o2) if M > 0 else p.N, M, p.N, p.K, int(eps_q0),
                                        int(gamma_shift), int(out_shift), _mode(rounding), _stream()))
     return out
 
@@ -424,13 +443,18 @@ class MlpLayerSpec:
     out_kind: str = 'int8'
 
 
-def mlp_runs_on_matrix_units(rows: int, x_pitch: int, layers: Sequence[Tuple[int, int]]) -> bool:
+def mlp_runs_on_matrix_units(rows: int, x_pitch: int, layers: Sequence[Tuple[int, int]], last_out_kind='int8',
+                             y_pitch: Optional[int] = None) -> bool:
     """Whether a4g_mlp_i8 takes its large-batch form for this chain (``layers``: (K, N) per layer; ``x_pitch``: bytes
-    between input rows, 0 if unknown): from 512 rows, weight fragments of 1 KiB per 32 x 32 block plus 128 bytes of
-    start values per 32 neurons within 128 KiB of LDS."""
+    between input rows, 0 if unknown; ``y_pitch``: elements between result rows, the last width if not given): from 512
+    rows, an 8-bit last layer, weight fragments of 1 KiB per 32 x 32 block plus 128 bytes of start values per 32
+    neurons within 128 KiB of LDS, and both ends addressable with 32-bit offsets (the conditions of csrc/mlp.hip)."""
     blocks = sum(((k + 31) // 32) * ((n + 31) // 32) for k, n in layers) + 1
     start = sum((n + 31) // 32 * 32 for _k, n in layers)
-    return rows >= 512 and x_pitch >= 1 and blocks * 1024 + start * 4 + 32 <= 128 * 1024
+    ldy = int(y_pitch) if y_pitch else layers[-1][1]
+    limit = (1 << 31) - 64
+    return (rows >= 512 and x_pitch >= 1 and _kind(last_out_kind) in (0, 1) and blocks * 1024 + start * 4 + 32 <= 128 * 1024
+            and (rows - 1) * x_pitch + layers[0][0] < limit and ((rows - 1) * ldy + layers[-1][1]) * 2 < limit)
 
 
 def mlp(x: torch.Tensor, layers: Sequence[MlpLayerSpec], rounding='floor', out: Optional[torch.Tensor] = None):
@@ -520,19 +544,22 @@ def mlp_add_layernorm(x: torch.Tensor, layers: Sequence[MlpLayerSpec], residual:
     if residual is not None:
         if residual.dtype != torch.int8 or tuple(residual.shape) != tuple(x.shape[:-1]) + (N,):
             raise ValueError('mlp_add_layernorm: the residual must be an int8 tensor of the output shape')
-        r2 = _rows2d(residual, 'residual').contiguous()
+        r2 = _pitched_rows(residual, 'residual')  # a window of a wider tensor is read where it lies
     g = _dev(gamma_q7, 'gamma').to(torch.int16).contiguous()
     bt = _dev(beta_q15, 'beta').to(torch.int16).contiguous()
     if g.numel() != N or bt.numel() != N:
         raise ValueError(f'LayerNorm parameter length does not match full_inner={N}.')
     if out is None:
         out = torch.empty(tuple(x.shape[:-1]) + (N,), dtype=torch.int8, device=x.device)
-    elif tuple(out.shape) != tuple(x.shape[:-1]) + (N,) or out.dtype != torch.int8 or not out.is_contiguous():
-        raise ValueError('mlp_add_layernorm: out must be a contiguous int8 tensor of the output shape')
+    elif tuple(out.shape) != tuple(x.shape[:-1]) + (N,) or out.dtype != torch.int8:
+        raise ValueError('mlp_add_layernorm: out must be an int8 tensor of the output shape')
+    o2 = _pitched_rows(out, 'out')
+    if o2.data_ptr() != out.data_ptr():
+        raise ValueError('mlp_add_layernorm: out needs a contiguous last axis, a row pitch in whole 16 bytes and a 16-byte aligned start')
     arr = _mlp_layer_array(layers)
     check(_lib.load().a4g_mlp_add_layernorm_i8(
-        arr, len(layers), _ptr(x2), _TORCH_KIND[x2.dtype], x2.stride(0) if M > 0 else layers[0].params.K, _ptr(r2), N, _ptr(g),
-        _ptr(bt), _ptr(out), N, M, _mode(rounding), int(eps_q0), int(gamma_shift), int(out_shift), _mode(ln_rounding), _stream()))
+        arr, len(layers), _ptr(x2), _TORCH_KIND[x2.dtype], x2.stride(0) if M > 0 else layers[0].params.K, _ptr(r2),
+        _pitch(r2) if r2 is not None else N, _ptr(g), _ptr(bt), _ptr(o2), _pitch(o2) if M > 0 else N, M, _mode(rounding), int(eps_q0), int(gamma_shift), int(out_shift), _mode(ln_rounding), _stream()))
     return out
 
 

@@ -524,18 +524,43 @@ def measure(torch, w, steps, warmup, eager=False):
     return ms, value, roof, graphed
 
 
-def calibrate_mfma(torch, blocks_per_cu=2, iters=4096):
-    """The int8 matrix-core rate this GPU sustains with register-resident operands (no memory traffic), and the clock
-    it holds meanwhile: (TOP/s, GHz)."""
-    from aie4ml_amd import _lib
+_BENCH_LIB = None
 
-    L = _lib.load()
+
+def _bench_lib():
+    """The measurement-aid library (the matrix-core calibration loop), built beside the product library."""
+    global _BENCH_LIB
+    if _BENCH_LIB is None:
+        import ctypes
+
+        from aie4ml_amd import _lib
+        from aie4ml_amd.build import BENCH_LIB_PATH
+
+        _lib.load()  # the HIP runtime torch owns is in the process before this library binds to it
+        L = ctypes.CDLL(str(BENCH_LIB_PATH))
+        L.a4g_calib_mfma_i8_ops.restype = ctypes.c_int64
+        L.a4g_calib_mfma_i8_ops.argtypes = [ctypes.c_int, ctypes.c_int]
+        L.a4g_calib_mfma_i8.restype = ctypes.c_int
+        L.a4g_calib_mfma_i8.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+        _BENCH_LIB = L
+    return _BENCH_LIB
+
+
+def calibrate_mfma(torch, blocks_per_cu=2, iters=4096, zero=False):
+    """The int8 matrix-core rate this GPU sustains with register-resident operands (no memory traffic), and the clock
+    it holds meanwhile: (TOP/s, GHz). ``zero``: all-zero operands, i.e. the same instruction stream at the power the
+    multipliers draw when nothing toggles."""
+    L = _bench_lib()
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     blocks = cus * blocks_per_cu
     sink = torch.zeros(4, dtype=torch.int32, device='cuda')
     clocks = torch.zeros(2 * blocks, dtype=torch.int64, device='cuda')
-    fn = lambda: _lib.check(L.a4g_calib_mfma_i8(blocks, iters, sink.data_ptr(), clocks.data_ptr(),  # noqa: E731
-                                                torch.cuda.current_stream().cuda_stream))  # the capture stream, when capturing
+    def fn():
+        rc = L.a4g_calib_mfma_i8(blocks, iters, int(zero), sink.data_ptr(), clocks.data_ptr(),
+                                 torch.cuda.current_stream().cuda_stream)  # the capture stream, when capturing
+        if rc != 0:
+            raise RuntimeError(f'a4g_calib_mfma_i8 failed with {rc}')
+
     _, ms_ev, _ = _time_gpu(torch, fn, 20, 5)
     ops_ = int(L.a4g_calib_mfma_i8_ops(blocks, iters))
     c = clocks.cpu().numpy().reshape(-1, 2).astype(np.float64)
@@ -570,14 +595,14 @@ def main():
     from oracle import oracle
 
     wl = args.workload
-    if wl == 'calib_mfma':
-        tops, ghz, ms_ev, blocks, iters = calibrate_mfma(torch)
+    if wl in ('calib_mfma', 'calib_mfma_zero'):
+        tops, ghz, ms_ev, blocks, iters = calibrate_mfma(torch, zero=wl == 'calib_mfma_zero')
         print(json.dumps({
             'metric': 'int8_mfma_calibration_tops', 'value': float(f'{tops:.6g}'), 'unit': 'TOP/s', 'n_gpus': 1, 'steps': 20,
             'warmup': 5, 'ms_per_step': round(ms_ev, 5), 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
             'dtype': 'int8', 'data': 'synthetic',
-            'config': {'workload': f'calib_mfma: {blocks} workgroups x 4 waves x {iters} x 16 v_mfma_i32_32x32x32_i8 on '
-                                   'register-resident operands, no memory traffic'},
+            'config': {'workload': f'{wl}: {blocks} workgroups x 4 waves x {iters} x 16 v_mfma_i32_32x32x32_i8 on '
+                                   f'register-resident {"all-zero" if wl == "calib_mfma_zero" else "pseudo-random"} operands, no memory traffic'},
             'roofline': {'bound': 'mfma', 'achieved': round(tops, 3), 'peak': PEAK_INT8_TOPS, 'unit': 'TOP/s',
                          'frac': round(tops / PEAK_INT8_TOPS, 4), 'traffic': None, 'kernel': 'calib_mfma_i8_kernel',
                          'kernel_ms': round(ms_ev, 5)},
@@ -616,6 +641,10 @@ def main():
         roof['calibrated_peak'] = round(tops, 1)
         roof['frac_of_calibrated'] = round(roof['achieved'] / tops, 4)
         roof['clock_ghz_under_mfma_load'] = round(ghz, 3)
+        # the control: the same register-only loop on all-zero operands (nothing toggles in the multipliers)
+        ztops, zghz, _, _, _ = calibrate_mfma(torch, zero=True)
+        roof['calibrated_peak_zero_operands'] = round(ztops, 1)
+        roof['clock_ghz_zero_operands'] = round(zghz, 3)
         # The same kernel, same shape, all-zero operands: identical instruction stream and memory traffic, but the
         # multipliers do not toggle. The difference to the headline is what the board's power limit takes for
         # full-entropy int8 operands (the clock drops under load; the schedule itself sustains the zero-operand rate).

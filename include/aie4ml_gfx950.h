@@ -346,15 +346,6 @@ A4G_API int a4g_add_f(const void* a, const void* b, void* out, int64_t n, int fm
 A4G_API int a4g_transpose(const void* src, int elem_bytes, int64_t ld_src, int64_t stride_src, void* dst, int64_t ld_dst,
                   int64_t stride_dst, int64_t batch, int64_t rows, int64_t cols, a4g_stream_t stream);
 
-/* ---- Calibration (measurement aid, no counterpart in the reference) -------------------------------------
- * `blocks` workgroups of four waves issue v_mfma_i32_32x32x32_i8 on register-resident operands, `iters` times 16
- * instructions per wave, with no memory traffic: a4g_calib_mfma_i8_ops(blocks, iters) operations in all. Timed by the
- * caller, it gives the int8 rate this GPU sustains, the ceiling a GEMM can be held against. clocks (nullable,
- * 2 * blocks entries) receives per workgroup the shader-clock ticks and the 100 MHz counter ticks over the loop, from
- * which the clock under matrix load follows. sink: one int of device memory (never written in practice). */
-A4G_API int64_t a4g_calib_mfma_i8_ops(int blocks, int iters);
-A4G_API int a4g_calib_mfma_i8(int blocks, int iters, int* sink, unsigned long long* clocks, a4g_stream_t stream);
-
 #ifdef __cplusplus
 }
 #endif

@@ -973,6 +973,62 @@ def test_dense_add_layernorm_pitched_through_the_c_abi(ops, oracle):
     assert (got[:, :16] == 99).all() and (got[:, 16 + N:] == 99).all()
 
 
+@pytest.mark.parametrize('with_residual', [True, False])
+def test_mlp_add_layernorm_pitched_through_the_c_abi(ops, oracle, with_residual):
+    """a4g_mlp_add_layernorm_i8 with a residual and a result that are column windows of wider buffers (ld_res > N,
+    ldy > N), and with no residual at all: the same bytes as a4g_mlp_i8 -> a4g_add -> a4g_layernorm_i8 through their own
+    entry points, and as the oracle; nothing outside the result window is written."""
+    import ctypes
+    from aie4ml_amd import _lib
+    L = _lib.load()
+    r = rng(63 + with_residual)
+    M, widths = 5000, [48, 128, 64]
+    x = gauss8(r, 40, (M, widths[0]))
+    specs, layers_np = [], []
+    for i in range(len(widths) - 1):
+        W = gauss8(r, 30, (widths[i], widths[i + 1]))
+        b = r.integers(-2**12, 2**12, widths[i + 1]).astype(np.int32)
+        last = i == len(widths) - 2
+        specs.append(ops.MlpLayerSpec(ops.pack_dense(dev(W), dev(b), 7), 7, not last, 'int8'))
+        layers_np.append((W, b, 7, not last, 'int8'))
+    N = widths[-1]
+    ldr, ldy = N + 48, N + 32
+    rbuf = gauss8(r, 40, (M, ldr))
+    gamma = r.integers(32, 128, N).astype(np.int16)
+    beta = (r.integers(-16, 17, N).astype(np.int32) << 10).astype(np.int16)
+    vp = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None  # noqa: E731
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    arr = ops._mlp_layer_array(specs)
+    dx, dr, dg, dbt = dev(x), dev(rbuf), dev(gamma), dev(beta)
+    r_win = dr[:, 32:] if with_residual else None
+    out = torch.full((M, ldy), 99, dtype=torch.int8, device='cuda')
+    rc = L.a4g_mlp_add_layernorm_i8(arr, len(specs), vp(dx), 0, widths[0], vp(r_win), ldr, vp(dg), vp(dbt), vp(out[:, 16:]), ldy, M,
+                                    6, 1, 7, 5, 6, stream)
+    assert rc == 0, L.a4g_last_error()
+    got = host(out)
+    # the three entry points it replaces
+    y = torch.empty((M, N), dtype=torch.int8, device='cuda')
+    assert L.a4g_mlp_i8(arr, len(specs), vp(dx), 0, widths[0], vp(y), N, M, 6, stream) == 0
+    ref = torch.empty((M, N), dtype=torch.int8, device='cuda')
+    if with_residual:
+        res = dr[:, 32:32 + N].contiguous()
+        ssum = torch.empty((M, N), dtype=torch.int8, device='cuda')
+        assert L.a4g_add(vp(y), vp(res), vp(ssum), M * N, 0, 0, 6, stream) == 0
+        y = ssum
+    assert L.a4g_layernorm_i8(vp(y), vp(dg), vp(dbt), vp(ref), M, N, 1, 7, 5, 6, stream) == 0
+    assert np.array_equal(got[:, 16:16 + N], host(ref))
+    yo = oracle.mlp(x, layers_np, 'conv_even')
+    want = (oracle.add_layernorm(yo, rbuf[:, 32:32 + N], gamma, beta, 5, 'conv_even') if with_residual
+            else oracle.layernorm(yo, gamma, beta, 5, 'conv_even'))
+    assert np.array_equal(got[:, 16:16 + N], want)
+    assert (got[:, :16] == 99).all() and (got[:, 16 + N:] == 99).all()
+    # and through the wrapper, which hands the windows over as they lie
+    out2 = torch.full((M, ldy), 77, dtype=torch.int8, device='cuda')
+    ops.mlp_add_layernorm(dx, specs, r_win[:, :N] if with_residual else None, dg, dbt, 5, 'conv_even', 'conv_even', out=out2[:, 16:16 + N])
+    got2 = host(out2)
+    assert np.array_equal(got2[:, 16:16 + N], want) and (got2[:, :16] == 77).all() and (got2[:, 16 + N:] == 77).all()
+
+
 def test_dense_add_layernorm_refuses_what_it_cannot_take(ops):
     r = rng(9)
     W = gauss8(r, 30, (100, 64))  # K not a multiple of 128
