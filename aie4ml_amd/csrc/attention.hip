@@ -93,8 +93,13 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
     constexpr int NB = (SK / 4) * (D / 4);
     constexpr int VB = (NB + THREADS - 1) / THREADS;
     const int wave_uniform = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    for (int item = item_begin; item < item_end; ++item) {
-    // The thread's indices are formed again for every item from an opaque copy of its id: derived from the id itself,
+    // The items of a workgroup are taken head by head. A head's V^T and column sums are laid down once, between two
+    // barriers; the blocks of query rows that follow touch nothing in LDS that another wave writes (the parked scores are
+    // a thread's own), so their waves do not meet again until the next head and may drift a block apart meanwhile.
+    for (int head_item = item_begin; head_item < item_end;) {
+    const int bh = head_item / nblk;
+    const int run_end = PERSIST ? min(item_end, (bh + 1) * nblk) : head_item + 1;
+    // The thread's indices are formed again for every head from an opaque copy of its id: derived from the id itself,
     // the dozens of per-thread addresses below would be kept in registers across the whole loop, which the 512-key form
     // has none to spare for.
     int tid = threadIdx.x;
@@ -110,43 +115,53 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
     const bool upper_missing = DT == 1 && a.d16 && half == 1;
     const int hoff = upper_missing ? 0 : half * 16;
     const int n0 = (tid % (D / 4)) * 4;  // THREADS % (D/4) == 0: a thread keeps its four columns
-    const int8_t* Kp;
-    int8_t* Op;
-    int row;
-    bool row_ok;
-    v4i qf[DT], kf[2][DT];
-    unsigned av[VB][4];
-    // a block of query rows of the same head as the previous item finds that head's V^T and column sums still in LDS
-    const bool same_head = PERSIST && item != item_begin && item / nblk == (item - 1) / nblk;
-    auto request = [&](int item) {
-        const int bh = item / nblk, rb = item - bh * nblk;
-        const int b = bh / a.heads, h = bh - b * a.heads;
+    const int b = bh / a.heads, h = bh - b * a.heads;
+    // K fragments run KD - 1 tiles ahead of the matrix unit (a slot is fetched again as soon as its tile has been
+    // multiplied): a tile's worth of work is a quarter of what a fetch from the L2 takes, and with one tile in flight the
+    // first pass spent most of its time waiting for it
+    constexpr int KD = NT < 4 ? NT : 4;
+    v4i qf[DT], kf[KD][DT];
+    const int k_ss = static_cast<int>(a.k_ss);  // the host has checked that a head's keys span less than 2 GiB
+    // K through a buffer descriptor of this head: the lane's offset is formed once, a tile adds a scalar and a
+    // constant, and rows past the last key read as zero
+    const __amdgpu_buffer_rsrc_t rsrc_k =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.K + b * a.k_sb + h * a.k_sh), 0, (a.sk - 1) * k_ss + D, 0x00020000);
+    const int kvoff = m * k_ss + hoff;
+    auto load_k = [&](int t, int ks) __attribute__((always_inline)) {
+        return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_k, kvoff + ks * 32, t * 32 * k_ss, 0));
+    };
+    // the query rows of a block and the first K tiles
+    auto request = [&](int item) __attribute__((always_inline)) {
         const int8_t* Qp = a.Q + b * a.q_sb + h * a.q_sh;
-        const int8_t* Vp = a.V + b * a.v_sb + h * a.v_sh;
-        Kp = a.K + b * a.k_sb + h * a.k_sh;
-        Op = a.O + b * a.o_sb + h * a.o_sh;
-        row = rb * ROWS + wave * 32 + m;
-        row_ok = row < a.sq;
-        const int rowc = row_ok ? row : a.sq - 1;
+        const int row = (item - bh * nblk) * ROWS + wave * 32 + m;
+        const int rowc = row < a.sq ? row : a.sq - 1;
 #pragma unroll
         for (int ks = 0; ks < DT; ++ks) {
             qf[ks] = *reinterpret_cast<const v4i*>(Qp + rowc * a.q_ss + ks * 32 + hoff);
-            kf[0][ks] = *reinterpret_cast<const v4i*>(Kp + (RAGGED ? min(m, a.sk - 1) : m) * a.k_ss + ks * 32 + hoff);
             if (DT == 1 && upper_missing) qf[ks] = v4i{0, 0, 0, 0};  // zero queries there: whatever K holds counts nothing
         }
 #pragma unroll
-        for (int it = 0; it < VB; ++it) {
-            const int blk = tid + it * THREADS;
-            const int k0 = (blk / (D / 4)) * 4;
+        for (int t = 0; t < KD; ++t) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                av[it][i] = blk < NB && (!RAGGED || k0 + i < a.sk) && !(DT == 1 && a.d16 && n0 >= 16)
-                                ? *reinterpret_cast<const unsigned*>(Vp + (k0 + i) * a.v_ss + n0) : 0u;
+            for (int ks = 0; ks < DT; ++ks) kf[t][ks] = load_k(t, ks);
         }
     };
-    // requested before anything is done with LDS, so that (first item) building the score table hides the latency
-    request(item);
-    if (item == item_begin) {
+    {
+    // V is requested before anything is done with LDS, so that (first head) building the score table hides the latency;
+    // the first block's operands follow it
+    unsigned av[VB][4];
+    const int8_t* Vp = a.V + b * a.v_sb + h * a.v_sh;
+#pragma unroll
+    for (int it = 0; it < VB; ++it) {
+        const int blk = tid + it * THREADS;
+        const int k0 = (blk / (D / 4)) * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            av[it][i] = blk < NB && (!RAGGED || k0 + i < a.sk) && !(DT == 1 && a.d16 && n0 >= 16)
+                            ? *reinterpret_cast<const unsigned*>(Vp + (k0 + i) * a.v_ss + n0) : 0u;
+    }
+    request(head_item);
+    if (head_item == item_begin) {
         if (BANKED) {
             // each entry is computed once, parked in the (still unused) V^T area, then copied to its 64 slots, four
             // slots per 16-byte store
@@ -161,10 +176,8 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
             for (int i = tid; i < 256; i += THREADS) table[i] = table_entry(a.sm, i);
         }
     }
-    // everybody is done with the previous item's V^T, column sums and parked scores (first item: with the table's
-    // staging area)
+    // everybody is done with the previous head's V^T and column sums (first head: with the table's staging area)
     __syncthreads();
-    if (!same_head) {
     if (tid < D) colsum[tid] = 0;
     __syncthreads();
 
@@ -191,24 +204,41 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
 #pragma unroll
         for (int j = 0; j < 4; ++j) atomicAdd(&colsum[n0 + j], part[j]);
     }
-    }  // !same_head
+    }
+    // A persistent workgroup meets here, once per head; one with a single item does after its first pass, which then
+    // hides the wait.
+    if (PERSIST) __syncthreads();  // V^T, column sums and the score table are complete
 
+    for (int item = head_item; item < run_end; ++item) {
     // ---- pass A: logits = srs(Q K^T), packed int8 in registers; running row maximum -----------------
     unsigned lg[NT][4];  // biased by 128: byte = logit ^ 0x80
     int mx = -128;
     float mxf = 0.f;
+    // (1.5 * 2^23 + x) * 2^-s + (128 - 1.5 * 2^23 * 2^-s) = x * 2^-s + 128, exactly: every term is a multiple of 2^-s
+    // below 2^24, and a fused multiply-add rounds once
+    const float lbias = 128.f - 12582912.f * a.lscale;
+    constexpr int START = 0x4B400000;
+    const v16i start16 = {START, START, START, START, START, START, START, START, START, START, START, START, START, START, START, START};
+    // BIT == 3: the sums start from the bit pattern of the float 1.5 * 2^23. Floats of that binade are one apart, so
+    // adding an integer x (|x| <= D * 2^14 < 2^22) to the pattern gives the pattern of the float 1.5 * 2^23 + x: the
+    // accumulators come out of the matrix unit already converted.
+    auto logits_of_tile = [&](int t) __attribute__((always_inline)) {
+        v16i sums = BIT == 3 ? start16 : v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int ks = 0; ks < DT; ++ks) sums = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[t % KD][ks], qf[ks], sums, 0, 0, 0);
+        return sums;
+    };
+    // The matrix unit works a tile ahead of the requantisation: its products of tile t + 1 are under way while the
+    // vector unit packs tile t.
+    v16i acc_next = logits_of_tile(0);
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-        if (t + 1 < NT) {
+        const v16i acc = acc_next;
+        if (t + 1 < NT) acc_next = logits_of_tile(t + 1);
+        if (KD > 1 && t + KD < NT) {
 #pragma unroll
-            for (int ks = 0; ks < DT; ++ks)
-                kf[(t + 1) & 1][ks] = *reinterpret_cast<const v4i*>(
-                    Kp + (RAGGED ? min((t + 1) * 32 + m, a.sk - 1) : (t + 1) * 32 + m) * a.k_ss + ks * 32 + hoff);
+            for (int ks = 0; ks < DT; ++ks) kf[(t + KD) % KD][ks] = load_k(t + KD, ks);
         }
-        v16i acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-        for (int ks = 0; ks < DT; ++ks)
-            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(kf[t & 1][ks], qf[ks], acc, 0, 0, 0);
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             // accumulator 4 g + i belongs to key 32 t + 8 g + 4 half + i: `left` of this group's four keys exist
@@ -217,7 +247,8 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
                 float f[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    f[i] = fmaf(static_cast<float>(acc[4 * g + i]), a.lscale, 128.f);
+                    const int sum_bits = acc[4 * g + i];
+                    f[i] = fmaf(__builtin_bit_cast(float, sum_bits), a.lscale, lbias);
                     if (RAGGED) f[i] = i < left ? f[i] : 0.f;
                 }
                 // two three-operand maxima
@@ -238,7 +269,11 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
                 lg[t][g] = pack4_bytes(y[0], y[1], y[2], y[3]) ^ 0x80808080u;
             }
         }
-        if (NT >= 16) __builtin_amdgcn_sched_barrier(0);  // one tile of K fragments in flight, not all sixteen
+        // The packed logits are pinned here: left to itself, the compiler moves the packing down to where the second
+        // pass reads them and keeps four floats alive per register it would have packed.
+#pragma unroll
+        for (int g = 0; g < 4; ++g) asm volatile("" : "+v"(lg[t][g]));
+        if (NT >= 16) __builtin_amdgcn_sched_barrier(0);  // KD - 1 tiles of K fragments in flight, not all sixteen
     }
     // the row maximum as a biased byte; rounding and saturation are monotone, so they commute with the maximum
     unsigned mxb;
@@ -250,7 +285,9 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
         mxb = static_cast<unsigned>((mx ^ 0x80) & 0xFF);
     }
 
-    __syncthreads();  // V^T, column sums and the score table are complete
+    // the operands of the head's next block of rows travel while this block goes through its second and third pass
+    if (PERSIST && item + 1 < run_end) request(item + 1);
+    if (!PERSIST) __syncthreads();  // V^T, column sums and the score table are complete
 
     // ---- pass B: scores by table lookup on the gap to the maximum; row sum ----------------------------
     const unsigned mrep = mxb * 0x01010101u;
@@ -258,46 +295,53 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
     const unsigned two = 2;
     const unsigned lane4 = static_cast<unsigned>(lane) << 2;  // BANKED: this lane's copy of the table
     unsigned ep[NT][8];  // two 16-bit scores per register
-    int sum = 0;
+    unsigned sum_even = 0, sum_odd = 0;
+    auto sum_and_keep = [&](int t, const unsigned (&pr)[8]) __attribute__((always_inline)) {
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const unsigned d4 = mrep - lg[t][g];  // per byte, never borrows
-            int e0, e1, e2, e3;
-            if (BANKED) {
-                e0 = *reinterpret_cast<const int*>(tbytes + __builtin_amdgcn_perm(d4, lane4, 0x0c0c0400u));
-                e1 = *reinterpret_cast<const int*>(tbytes + __builtin_amdgcn_perm(d4, lane4, 0x0c0c0500u));
-                e2 = *reinterpret_cast<const int*>(tbytes + __builtin_amdgcn_perm(d4, lane4, 0x0c0c0600u));
-                e3 = *reinterpret_cast<const int*>(tbytes + __builtin_amdgcn_perm(d4, lane4, 0x0c0c0700u));
-            } else {
-                e0 = *reinterpret_cast<const int*>(tbytes + byte_x4<0>(d4, two));
-                e1 = *reinterpret_cast<const int*>(tbytes + byte_x4<1>(d4, two));
-                e2 = *reinterpret_cast<const int*>(tbytes + byte_x4<2>(d4, two));
-                e3 = *reinterpret_cast<const int*>(tbytes + byte_x4<3>(d4, two));
-            }
-            if (RAGGED) {
-                const int left = a.sk - (t * 32 + 8 * g + 4 * half);
-                e0 = left > 0 ? e0 : 0;
-                e1 = left > 1 ? e1 : 0;
-                e2 = left > 2 ? e2 : 0;
-                e3 = left > 3 ? e3 : 0;
-            }
+        for (int r = 0; r < 8; ++r) {
             // scores are at most 32767: both halves of a pair are summed by one dot product with (1, 1)
-            const unsigned p01 = pack2_halves(e0, e1), p23 = pack2_halves(e2, e3);
-            sum = static_cast<int>(__builtin_amdgcn_udot2(__builtin_bit_cast(v2us, p01), __builtin_bit_cast(v2us, 0x00010001u), static_cast<unsigned>(sum), false));
-            sum = static_cast<int>(__builtin_amdgcn_udot2(__builtin_bit_cast(v2us, p23), __builtin_bit_cast(v2us, 0x00010001u), static_cast<unsigned>(sum), false));
-            if (t >= NT - PARK) {
-                parked[((t - (NT - PARK)) * 8 + 2 * g) * THREADS + tid] = p01;
-                parked[((t - (NT - PARK)) * 8 + 2 * g + 1) * THREADS + tid] = p23;
-            } else {
-                ep[t][2 * g] = p01;
-                ep[t][2 * g + 1] = p23;
-            }
+            // (into two sums in turn: a dot product that waits for the one before it costs an idle slot)
+            unsigned& part = (r & 1) ? sum_odd : sum_even;
+            part = __builtin_amdgcn_udot2(__builtin_bit_cast(v2us, pr[r]), __builtin_bit_cast(v2us, 0x00010001u), part, false);
+            if (t >= NT - PARK) parked[((t - (NT - PARK)) * 8 + r) * THREADS + tid] = pr[r];
+            else ep[t][r] = pr[r];
         }
-        // keep the scheduler from hoisting many tiles' lookups at once (their results would spill)
-        if (NT >= 16 && (t & 1)) __builtin_amdgcn_sched_barrier(0);
+    };
+    {
+#pragma unroll
+        for (int t = 0; t < NT; ++t) {
+            unsigned pr[8];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const unsigned d4 = mrep - lg[t][g];  // per byte, never borrows
+                int e0, e1, e2, e3;
+                if (BANKED) {
+                    e0 = *reinterpret_cast<const int*>(tbytes + __builtin_amdgcn_perm(d4, lane4, 0x0c0c0400u));
+                    e1 = *reinterpret_cast<const int*>(tbytes + __builtin_amdgcn_perm(d4, lane4, 0x0c0c0500u));
+                    e2 = *reinterpret_cast<const int*>(tbytes + __builtin_amdgcn_perm(d4, lane4, 0x0c0c0600u));
+                    e3 = *reinterpret_cast<const int*>(tbytes + __builtin_amdgcn_perm(d4, lane4, 0x0c0c0700u));
+                } else {
+                    e0 = *reinterpret_cast<const int*>(tbytes + byte_x4<0>(d4, two));
+                    e1 = *reinterpret_cast<const int*>(tbytes + byte_x4<1>(d4, two));
+                    e2 = *reinterpret_cast<const int*>(tbytes + byte_x4<2>(d4, two));
+                    e3 = *reinterpret_cast<const int*>(tbytes + byte_x4<3>(d4, two));
+                }
+                if (RAGGED) {
+                    const int left = a.sk - (t * 32 + 8 * g + 4 * half);
+                    e0 = left > 0 ? e0 : 0;
+                    e1 = left > 1 ? e1 : 0;
+                    e2 = left > 2 ? e2 : 0;
+                    e3 = left > 3 ? e3 : 0;
+                }
+                pr[2 * g] = pack2_halves(e0, e1);
+                pr[2 * g + 1] = pack2_halves(e2, e3);
+            }
+            sum_and_keep(t, pr);
+            // keep the scheduler from hoisting many tiles' lookups at once (their results would spill)
+            if (NT >= 16 && (t & 1)) __builtin_amdgcn_sched_barrier(0);
+        }
     }
+    int sum = static_cast<int>(sum_even + sum_odd);
     sum += lane_xor<32>(sum);
     const int inv = row_inverse(a.sm, sum);
 
@@ -348,6 +392,9 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
     }
 
     // ---- epilogue: + 128 * colsum (undoes the ^0x80), requantise, 16 contiguous bytes per lane ---------
+    int8_t* Op = a.O + b * a.o_sb + h * a.o_sh;
+    const int row = (item - bh * nblk) * ROWS + wave * 32 + m;
+    const bool row_ok = row < a.sq;
 #pragma unroll
     for (int u = 0; u < DT; ++u) {
         unsigned ow[4];
@@ -367,7 +414,9 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
                        static_cast<int>(s13[1])};
         if (row_ok && !(DT == 1 && upper_missing)) *reinterpret_cast<v4i*>(Op + row * a.o_ss + 32 * u + 16 * half) = o;
     }
-    }  // items
+    }  // blocks of query rows
+    head_item = run_end;
+    }  // heads
 }
 
 constexpr int ATTN_CUS = 256;
@@ -486,6 +535,8 @@ extern "C" int a4g_attention_i8(const int8_t* Q, const int8_t* K, const int8_t* 
     A4G_REQUIRE(ok, A4G_ERR_UNSUPPORTED, "%s: pointers and strides must be multiples of 16 bytes", who);
     A4G_REQUIRE(strides[2] >= d && strides[5] >= d && strides[8] >= d && strides[11] >= d, A4G_ERR_INVALID_ARGUMENT,
                 "%s: row stride smaller than the head dimension", who);
+    A4G_REQUIRE((sk + 32) * strides[5] < (int64_t{1} << 31), A4G_ERR_UNSUPPORTED,
+                "%s: the keys of one head must span less than 2 GiB (row stride %lld bytes)", who, (long long)strides[5]);
     a.Q = Q; a.K = K; a.V = V; a.O = O;
     a.q_sb = strides[0]; a.q_sh = strides[1]; a.q_ss = strides[2];
     a.k_sb = strides[3]; a.k_sh = strides[4]; a.k_ss = strides[5];
