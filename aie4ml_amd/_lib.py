@@ -98,6 +98,7 @@ SIGNATURES = {
                             _vp]),
     'a4g_add_f': (_i32, [_vp, _vp, _vp, _i64, _i32, _vp]),
     'a4g_transpose': (_i32, [_vp, _i32, _i64, _i64, _vp, _i64, _i64, _i64, _i64, _i64, _vp]),
+    'a4g_copy_2d': (_i32, [_vp, _i64, _vp, _i64, _i64, _i64, _vp]),
 }
 
 _lib = None

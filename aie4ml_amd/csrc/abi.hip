@@ -33,3 +33,17 @@ int check_hip(hipError_t e, const char* what) {
 extern "C" int a4g_version(void) { return A4G_VERSION; }
 
 extern "C" const char* a4g_last_error(void) { return a4g::g_error; }
+
+// A window of rows copied on the device with the runtime's own 2-D copy (a memcpy node under stream capture).
+extern "C" int a4g_copy_2d(const void* src, int64_t ld_src, void* dst, int64_t ld_dst, int64_t rows, int64_t row_bytes,
+                           a4g_stream_t stream) {
+    using namespace a4g;
+    const char* who = "a4g_copy_2d";
+    A4G_REQUIRE(rows >= 0 && row_bytes >= 0 && ld_src >= row_bytes && ld_dst >= row_bytes, A4G_ERR_INVALID_ARGUMENT,
+                "%s: bad window rows=%lld row_bytes=%lld ld_src=%lld ld_dst=%lld", who, (long long)rows, (long long)row_bytes,
+                (long long)ld_src, (long long)ld_dst);
+    if (rows == 0 || row_bytes == 0) return A4G_OK;
+    A4G_REQUIRE(src && dst, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+    return check_hip(hipMemcpy2DAsync(dst, static_cast<size_t>(ld_dst), src, static_cast<size_t>(ld_src), static_cast<size_t>(row_bytes),
+                                      static_cast<size_t>(rows), hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream)), who);
+}

@@ -27,7 +27,7 @@ struct AttnArgs {
     int64_t v_sb, v_sh, v_ss;
     int64_t o_sb, o_sh, o_ss;
     int heads, sq;
-    int d16;    // head dimension 16 on the 32-wide kernel: the upper halves of its fragments do not exist
+    int d;      // head dimension that exists, a multiple of 16 up to the kernel's width: the 16-byte pieces of a row past it do not
     int sk;     // key / value rows that exist (the ragged form; the kernel's tiles cover the next power of two of 32s)
     int items;  // (batch, head, block of query rows) triples in all
     FastRound lr, orr;  // logits and output requantisation
@@ -54,8 +54,8 @@ __device__ __forceinline__ void transpose4x4(const unsigned a[4], unsigned c[4])
 // v_cvt_pk_u8_f32 (nearest even, saturating to 0..255, writing one byte of a dword) is the rounding, the int8
 // saturation (biased by 128) and the packing at once. FASTP: the probabilities need no clamp and their shift is
 // at most 16, so p = (e * inv) >> shift is read as byte 2 of e * (inv << (16 - shift)).
-// RAGGED: fewer keys exist than the NT tiles cover (any count >= 1). K rows past the end alias the last row, V rows
-// past the end load as zero; their logits are forced to the minimum (they cannot raise the row maximum), their scores
+// RAGGED: fewer keys exist than the NT tiles cover (any count >= 1). K and V rows past the end load as zero; their
+// logits are forced to the minimum (they cannot raise the row maximum), their scores
 // to zero (they add nothing to the row sum, and a zero probability times a zero V row nothing to the output).
 // NW = waves per workgroup. 4: two workgroups share a CU. 8: one workgroup of 256 query rows per CU, which
 // leaves room to store the score table once per LDS bank (entry d for lane c at dword d * 64 + c, byte address
@@ -110,10 +110,12 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
     }
     const int lane = tid & 63, wave = tid >> 6;
     const int m = lane & 31, half = lane >> 5;
-    // Head dimension 16 on the 32-wide kernel (DT == 1 only): the lanes of the upper half fetch the lower half again (no
-    // access leaves the row), multiply with zero queries, see zero V columns and store nothing.
-    const bool upper_missing = DT == 1 && a.d16 && half == 1;
-    const int hoff = upper_missing ? 0 : half * 16;
+    // A head dimension below the kernel's width (16 on the 32-wide kernel, 48 on the 64-wide, 80 .. 112 on the 128-wide):
+    // the lanes whose 16-byte piece of a row does not exist fetch the row's first piece for Q (no access leaves the row)
+    // and put zeros in its place, so that whatever the K fragment holds there counts nothing; K is read through a
+    // descriptor that ends with the last row that exists; V columns past the dimension load as zero and output pieces
+    // past it are not stored.
+    const int hoff = half * 16;
     const int n0 = (tid % (D / 4)) * 4;  // THREADS % (D/4) == 0: a thread keeps its four columns
     const int b = bh / a.heads, h = bh - b * a.heads;
     // K fragments run KD - 1 tiles ahead of the matrix unit (a slot is fetched again as soon as its tile has been
@@ -125,7 +127,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
     // K through a buffer descriptor of this head: the lane's offset is formed once, a tile adds a scalar and a
     // constant, and rows past the last key read as zero
     const __amdgpu_buffer_rsrc_t rsrc_k =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.K + b * a.k_sb + h * a.k_sh), 0, (a.sk - 1) * k_ss + D, 0x00020000);
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.K + b * a.k_sb + h * a.k_sh), 0, (a.sk - 1) * k_ss + a.d, 0x00020000);
     const int kvoff = m * k_ss + hoff;
     auto load_k = [&](int t, int ks) __attribute__((always_inline)) {
         return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_k, kvoff + ks * 32, t * 32 * k_ss, 0));
@@ -137,8 +139,9 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
         const int rowc = row < a.sq ? row : a.sq - 1;
 #pragma unroll
         for (int ks = 0; ks < DT; ++ks) {
-            qf[ks] = *reinterpret_cast<const v4i*>(Qp + rowc * a.q_ss + ks * 32 + hoff);
-            if (DT == 1 && upper_missing) qf[ks] = v4i{0, 0, 0, 0};  // zero queries there: whatever K holds counts nothing
+            const bool missing = a.d < D && ks * 32 + hoff >= a.d;
+            qf[ks] = *reinterpret_cast<const v4i*>(Qp + rowc * a.q_ss + (missing ? 0 : ks * 32 + hoff));
+            if (missing) qf[ks] = v4i{0, 0, 0, 0};
         }
 #pragma unroll
         for (int t = 0; t < KD; ++t) {
@@ -157,7 +160,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
         const int k0 = (blk / (D / 4)) * 4;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-            av[it][i] = blk < NB && (!RAGGED || k0 + i < a.sk) && !(DT == 1 && a.d16 && n0 >= 16)
+            av[it][i] = blk < NB && (!RAGGED || k0 + i < a.sk) && n0 < a.d
                             ? *reinterpret_cast<const unsigned*>(Vp + (k0 + i) * a.v_ss + n0) : 0u;
     }
     request(head_item);
@@ -412,7 +415,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
         const auto s13 = __builtin_amdgcn_permlane32_swap(ow[1], ow[3], false, false);
         const v4i o = {static_cast<int>(s02[0]), static_cast<int>(s02[1]), static_cast<int>(s13[0]),
                        static_cast<int>(s13[1])};
-        if (row_ok && !(DT == 1 && upper_missing)) *reinterpret_cast<v4i*>(Op + row * a.o_ss + 32 * u + 16 * half) = o;
+        if (row_ok && 32 * u + 16 * half < a.d) *reinterpret_cast<v4i*>(Op + row * a.o_ss + 32 * u + 16 * half) = o;
     }
     }  // blocks of query rows
     head_item = run_end;
@@ -521,9 +524,10 @@ extern "C" int a4g_attention_i8(const int8_t* Q, const int8_t* K, const int8_t* 
         if (int rc = make_hccs_params(who, sk, hccs_B, hccs_S, hccs_Dmax, inv_shift, use_clb, A4G_U8, &a.sm, &noclamp))
             return rc;
     }
-    A4G_REQUIRE(((d == 64 || d == 32 || d == 16) && sk <= 512) || (d == 128 && sk <= 256), A4G_ERR_UNSUPPORTED,
-                "%s: fused path covers head_dim 64, 32 and 16 with up to 512 keys and head_dim 128 with up to 256, got d=%lld sk=%lld",
-                who, (long long)d, (long long)sk);
+    A4G_REQUIRE(d % 16 == 0 && d <= 128 && sk <= (d > 64 ? 256 : 512), A4G_ERR_UNSUPPORTED,
+                "%s: fused path covers head dimensions that are multiples of 16, up to 64 with up to 512 keys and up to 128 with up "
+                "to 256, got d=%lld sk=%lld", who, (long long)d, (long long)sk);
+    const int width = d <= 32 ? 32 : (d <= 64 ? 64 : 128);  // of the kernel: narrower heads run with their missing pieces masked
     int nt = 1;  // tiles of 32 keys the kernel is instantiated for: the next power of two
     while (nt * 32 < sk) nt *= 2;
     const bool ragged = nt * 32 != sk;
@@ -545,7 +549,7 @@ extern "C" int a4g_attention_i8(const int8_t* Q, const int8_t* K, const int8_t* 
     a.heads = static_cast<int>(heads);
     a.sq = static_cast<int>(sq);
     a.sk = static_cast<int>(sk);
-    a.d16 = d == 16;
+    a.d = static_cast<int>(d);
     a.lr = make_fast_round(logit_round_mode, logit_shift);
     a.orr = make_fast_round(out_round_mode, out_shift);
     a.noclamp = noclamp;
@@ -564,8 +568,8 @@ extern "C" int a4g_attention_i8(const int8_t* Q, const int8_t* K, const int8_t* 
         launch_attention_seven(a.items, stream, a);
         return check_hip(hipGetLastError(), who);
     }
-    const int no_kernel = d == 64 ? launch_attention<2>(nt, grid, grid8, stream, a)
-                          : (d <= 32 ? launch_attention<1>(nt, grid, 0, stream, a) : launch_attention<4>(nt, grid, 0, stream, a));
+    const int no_kernel = width == 64 ? launch_attention<2>(nt, grid, grid8, stream, a)
+                          : (width == 32 ? launch_attention<1>(nt, grid, 0, stream, a) : launch_attention<4>(nt, grid, 0, stream, a));
     if (no_kernel) return fail(A4G_ERR_UNSUPPORTED, "%s: no kernel for sk=%lld", who, (long long)sk);
     return check_hip(hipGetLastError(), who);
 }

@@ -243,7 +243,7 @@ class GPUModel:
         return {name: values[name] for name in graph.output_tensor_names}
 
     def _run_view(self, node, values) -> None:
-        import torch
+        from . import ops
 
         sv, cv = node.traits.get('slice_view'), node.traits.get('concat_view')
         if sv is not None:
@@ -251,7 +251,7 @@ class GPUModel:
             for item in sv.data['slices']:
                 values[item['output']] = src.narrow(int(sv.data['axis']), int(item['start']), int(item['extent']))
         elif cv is not None:
-            values[cv.data['output']] = torch.cat([values[i['input']] for i in cv.data['slices']], dim=int(cv.data['axis']))
+            values[cv.data['output']] = ops.concat([values[i['input']] for i in cv.data['slices']], int(cv.data['axis']))
         elif node.op_type == 'input':
             pass  # hls4ml-style input placeholder
         else:

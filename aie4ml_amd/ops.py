@@ -91,6 +91,37 @@ def transpose_last2(t: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def concat(parts: Sequence[torch.Tensor], axis: int) -> torch.Tensor:
+    """The parts side by side along `axis` in one new tensor, each placed with the library's 2-D device copy (the
+    reference's Concat is a view: its producers write their slices of one buffer, docs/support.md:13-15)."""
+    if not parts:
+        raise ValueError('concat needs at least one tensor')
+    first = parts[0]
+    axis = axis % first.dim()
+    for t in parts:
+        _dev(t, 'part')
+        if t.dtype != first.dtype or t.dim() != first.dim() or any(
+                t.shape[i] != first.shape[i] for i in range(first.dim()) if i != axis):
+            raise ValueError('concat: parts must share dtype and every extent but the one along the axis')
+    shape = list(first.shape)
+    shape[axis] = sum(int(t.shape[axis]) for t in parts)
+    out = torch.empty(shape, dtype=first.dtype, device=first.device)
+    rows = 1
+    for e in shape[:axis]:
+        rows *= int(e)
+    inner = first.element_size()
+    for e in shape[axis + 1:]:
+        inner *= int(e)
+    ld_dst, at = shape[axis] * inner, 0
+    for t in parts:
+        t = t.contiguous()
+        row_bytes = int(t.shape[axis]) * inner
+        if rows and row_bytes:
+            check(_lib.load().a4g_copy_2d(_ptr(t), row_bytes, out.data_ptr() + at, ld_dst, rows, row_bytes, _stream()))
+        at += row_bytes
+    return out
+
+
 def add(a: torch.Tensor, b: torch.Tensor, shift: int = 0, rounding='floor', out: Optional[torch.Tensor] = None):
     """Saturating elementwise add of two tensors that share shape and storage type."""
     _dev(a, 'a'), _dev(b, 'b')
@@ -572,8 +603,8 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, logit_shift: in
     {'kind': 'exp', 'exp_kq': .., 'inv_shift': 15} or {'kind': 'hccs', 'B': .., 'S': .., 'Dmax': .., 'inv_shift': 15,
     'use_clb': False}. Bit-identical to matmul(trans_b) -> softmax_* -> matmul. Raises NotImplementedError for
     shapes the fused kernel does not cover (head_dim not a multiple of 16 or above 128, more than 512 keys - 256 from
-    head_dim 80 on -, unaligned views). Head dimension 16 runs on the 32-wide kernel; 48, 80, 96 and 112 are padded with zero columns to 64
-    and 128.
+    head_dim 80 on -, unaligned views). Head dimensions 16, 48, 80, 96 and 112 run on the next wider kernel (32, 64, 128) with the pieces of a
+    row that do not exist masked inside it.
     """
     for name, t in (('q', q), ('k', k), ('v', v)):
         _dev(t, name)
@@ -583,18 +614,6 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, logit_shift: in
         raise ValueError(f'attention: incompatible shapes {tuple(q.shape)}, {tuple(k.shape)}, {tuple(v.shape)}')
     lead = tuple(q.shape[:-2])
     sq, d, sk = int(q.shape[-2]), int(q.shape[-1]), int(k.shape[-2])
-    if d not in (16, 32, 64, 128) and d % 16 == 0 and d < 128:
-        # head dimensions 48, 80, 96, 112: zero columns up to the next dimension the kernel has change neither Q K^T nor
-        # the columns of P V that exist (three small copies and one back, against three launches through HBM)
-        pad = (64 if d < 64 else 128) - d
-        padded = attention(torch.nn.functional.pad(q, (0, pad)), torch.nn.functional.pad(k, (0, pad)),
-                           torch.nn.functional.pad(v, (0, pad)), logit_shift, logit_rounding, softmax, out_shift, out_rounding)
-        if out is None:
-            return padded[..., :d].contiguous()
-        if out.shape != lead + (sq, d) or out.dtype != torch.int8:
-            raise ValueError('attention: out must be int8 of shape [..., sq, d]')
-        out.copy_(padded[..., :d])
-        return out
     if out is None:
         out = torch.empty(lead + (sq, d), dtype=torch.int8, device=q.device)
     elif out.shape != lead + (sq, d) or out.dtype != torch.int8 or out.stride(-1) != 1:

@@ -298,9 +298,11 @@ A4G_API int a4g_mlp_add_layernorm_i8(const a4g_mlp_layer* layers, int n_layers, 
  *   slices of a packed QKV projection and a concatenated output need no copies.
  *   softmax_kind 0: accurate exp (exp_kq, inv_shift); 1: HCCS (hccs_B, hccs_S, hccs_Dmax, inv_shift,
  *   use_clb), same parameter rules as the stand-alone entries; probabilities are uint8.
- * Covered shapes: d == 64, 32 or 16 with 1 <= sk <= 512, d == 128 with 1 <= sk <= 256 (any count: key counts off
- * the 32-grid, e.g. 197 tokens, run the kernel of the next power of two with the missing keys masked out), any
- * sq, pointers and strides multiples of 16 bytes; anything else returns A4G_ERR_UNSUPPORTED and the caller runs the three operators separately. */
+ * Covered shapes: d a multiple of 16, up to 64 with 1 <= sk <= 512 and up to 128 with 1 <= sk <= 256 (head
+ * dimensions 16, 48, 80, 96 and 112 run the 32-, 64- and 128-wide kernels with the missing 16-byte pieces of a row
+ * masked; any key count: counts off the 32-grid, e.g. 197 tokens, run the kernel of the next power of two with the
+ * missing keys masked out), any sq, pointers and strides multiples of 16 bytes, the keys of one head within
+ * 2 GiB; anything else returns A4G_ERR_UNSUPPORTED and the caller runs the three operators separately. */
 A4G_API int a4g_attention_i8(const int8_t* Q, const int8_t* K, const int8_t* V, int8_t* O, int64_t batch, int64_t heads,
                      int64_t sq, int64_t sk, int64_t d, const int64_t* strides, int logit_shift,
                      int logit_round_mode, int softmax_kind, int exp_kq, int hccs_B, int hccs_S, int hccs_Dmax,
@@ -345,6 +347,14 @@ A4G_API int a4g_add_f(const void* a, const void* b, void* out, int64_t n, int fm
  * This call is for a caller that wants the transposed copy itself, on the device and in memory it owns. */
 A4G_API int a4g_transpose(const void* src, int elem_bytes, int64_t ld_src, int64_t stride_src, void* dst, int64_t ld_dst,
                   int64_t stride_dst, int64_t batch, int64_t rows, int64_t cols, a4g_stream_t stream);
+
+/* ---- Concatenated results --------------------------------------------------------------------------------
+ * rows windows of row_bytes bytes, pitches ld_src and ld_dst in bytes, copied device to device (the runtime's 2-D
+ * copy; a memcpy node under stream capture). The reference never copies for Concat: its producers write their slices
+ * of one memtile buffer (docs/support.md:13-15, passes/fold_views.py). A graph executor whose producers return tensors
+ * of their own places each one in its slice of the concatenated tensor with this call. */
+A4G_API int a4g_copy_2d(const void* src, int64_t ld_src, void* dst, int64_t ld_dst, int64_t rows, int64_t row_bytes,
+                a4g_stream_t stream);
 
 #ifdef __cplusplus
 }

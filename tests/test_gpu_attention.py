@@ -105,8 +105,9 @@ def test_attention_head_dimensions_16_32_and_128(oracle, d, sk, kind):
 
 @pytest.mark.parametrize('d,sk', [(16, 64), (16, 100), (48, 128), (80, 96), (96, 256), (112, 33)])
 def test_attention_head_dimensions_between_the_kernels(oracle, d, sk):
-    """Head dimensions 16, 48, 80, 96, 112 run padded with zero columns to the next dimension that has a kernel; also into
-    a strided output (the heads of a concatenated result)."""
+    """Head dimensions 16, 48, 80, 96, 112 run on the next wider kernel with the missing pieces of a row masked; also into
+    a strided output (the heads of a concatenated result) and from head slices of packed projections, where the bytes
+    behind a head's row are the next head's."""
     q, k, v = qkv(9000 + d + sk, (2, 3, sk, d), (2, 3, sk, d), sigma=24.0)
     sm = {'kind': 'exp', 'exp_kq': 23}
     want = reference(oracle, q, k, v, 6, 'conv_even', sm, 7, 'symmetric_inf')
@@ -115,11 +116,15 @@ def test_attention_head_dimensions_between_the_kernels(oracle, d, sk):
     out = torch.zeros((2, sk, 3 * d), dtype=torch.int8, device='cuda')
     ops.attention(dev(q), dev(k), dev(v), 6, 'conv_even', sm, 7, 'symmetric_inf', out=out.unflatten(-1, (3, d)).permute(0, 2, 1, 3))
     np.testing.assert_array_equal(out.cpu().numpy().reshape(2, sk, 3, d).transpose(0, 2, 1, 3), want)
+    packed = [dev(np.ascontiguousarray(t.transpose(0, 2, 1, 3))).permute(0, 2, 1, 3) for t in (q, k, v)]  # [2, sk, 3, d] in memory
+    got = ops.attention(packed[0], packed[1], packed[2], 6, 'conv_even', sm, 7, 'symmetric_inf').cpu().numpy()
+    np.testing.assert_array_equal(got, want)
 
 
 def test_attention_masked_keys_do_not_leak(oracle):
     """The rows behind the last key are other tensors' memory: whatever they hold, the result is that of the keys that
-    exist (K rows past the end alias the last row inside the kernel, V rows past the end are not read)."""
+    exist (K rows past the end read as zero inside the kernel and their logits are forced to the minimum, V rows past the
+    end are not read)."""
     sk = 100
     r = np.random.default_rng(5)
     big_k = np.full((2, 128, 64), 127, np.int8)
@@ -211,7 +216,7 @@ def test_attention_on_head_slices_of_a_packed_projection(oracle):
 
 def test_attention_uncovered_shapes_and_bad_parameters():
     q = torch.zeros((2, 64, 40), dtype=torch.int8, device='cuda')
-    with pytest.raises(NotImplementedError, match='fused path covers head_dim 64'):
+    with pytest.raises(NotImplementedError, match='fused path covers head dimensions that are multiples of 16'):
         ops.attention(q, q, q, 6, 'floor', {'kind': 'exp', 'exp_kq': 23}, 7, 'floor')
     q = torch.zeros((2, 544, 64), dtype=torch.int8, device='cuda')
     with pytest.raises(NotImplementedError, match='fused path covers'):

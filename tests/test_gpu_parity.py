@@ -1326,3 +1326,20 @@ def test_mlp_limits(ops):
     _, specs = make_mlp(ops, r, [16, 300, 4])
     with pytest.raises(NotImplementedError):
         ops.mlp(torch.zeros((4, 16), dtype=torch.int8, device='cuda'), specs, 'floor')
+
+
+@pytest.mark.parametrize('axis', [-1, 1, 0])
+@pytest.mark.parametrize('dtype', [torch.int8, torch.int16])
+def test_concat_places_parts_with_the_device_copy(ops, axis, dtype):
+    """Concat of producer outputs: every part lands in its slice of one new tensor (last, middle and first axis; parts of
+    different extents along it, a non-contiguous part, an empty part)."""
+    r = np.random.default_rng(77)
+    shapes = {-1: [(3, 5, 7), (3, 5, 1), (3, 5, 0), (3, 5, 16)], 1: [(3, 2, 7), (3, 9, 7)], 0: [(1, 5, 7), (4, 5, 7)]}[axis]
+    info = np.iinfo(np.int8 if dtype == torch.int8 else np.int16)
+    parts = [r.integers(info.min, info.max + 1, s).astype(info.dtype) for s in shapes]
+    dev_parts = [torch.from_numpy(p).cuda() for p in parts]
+    dev_parts[0] = torch.from_numpy(np.ascontiguousarray(parts[0].swapaxes(0, 1))).cuda().transpose(0, 1)  # same values, strided
+    got = ops.concat(dev_parts, axis)
+    np.testing.assert_array_equal(got.cpu().numpy(), np.concatenate(parts, axis=axis))
+    with pytest.raises(ValueError, match='share dtype'):
+        ops.concat([dev_parts[0], dev_parts[0][:, :1, :1]], axis)
