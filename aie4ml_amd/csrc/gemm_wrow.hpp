@@ -129,9 +129,6 @@ __global__ __launch_bounds__(WS_NT, 1) void gemm_wrow_kernel(GemmArgs g, int pie
     int sl = 0;                          // ... and the ring slot it goes to
     // Tile kt of the piece the issue cursor points at: two instructions per wave. `advance` moves the cursor on.
     auto issue_tile = [&](int kt, int j2) WS_INLINE {
-#ifdef WS_KO_LOADS
-        if (itl > it0) return;
-#endif
         const int base = itl < it1 ? hl * WS_ROWS * lda : a_bytes;  // past the run: every lane out of range
         int8_t* dst = stages + (sl * NKT + kt) * WS_STAGE + wave * 2048 + j2 * 1024;
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (__attribute__((address_space(3))) void*)dst, 16, (j2 ? va1 : va0) + base + kt * WS_BK, 0, 0, 0);
@@ -309,19 +306,15 @@ __global__ __launch_bounds__(WS_NT, 1) void gemm_wrow_kernel(GemmArgs g, int pie
                 issue_tile(Z / 16, (Z / 8) & 1);
                 __builtin_amdgcn_sched_barrier(0);
             }
-#ifndef WS_KO_READS
             if constexpr (c == 1 && F + AFS < 2 * NKS) {
                 read_fragment(F + AFS);
                 __builtin_amdgcn_sched_barrier(0);
             }
-#endif
             if constexpr (!GEN) {
-#ifndef WS_KO_EPI
                 constexpr int LEAD = NM > 2 ? 2 : NM - 1;
                 static_for<0, 32>([&](auto v_tag) WS_INLINE {
                     if constexpr (LEAD + (decltype(v_tag)::value * (NM - LEAD)) / 32 == z) epi_value(i ^ 1, v_tag);
                 });
-#endif
                 __builtin_amdgcn_sched_barrier(0);
             }
             if constexpr (z == NM - 1) {  // row block i is complete: these are its rows
