@@ -84,7 +84,11 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
     // of one head are neighbours, so its K and V are fetched once), builds the 64 KiB replicated score table once
     // instead of once per item.
     constexpr bool PERSIST = BANKED;
-    const int item_begin = PERSIST ? static_cast<int>(static_cast<int64_t>(blockIdx.x) * a.items / gridDim.x) : static_cast<int>(blockIdx.x);
+    // One item per workgroup: workgroups go to the eight XCDs round robin, so the items are renumbered to give an XCD
+    // consecutive ones. Neighbouring heads of a packed projection share cache lines (a head's row is 64 bytes of a 128-byte
+    // line); on one XCD, launched one after the other, the second finds in L2 what the first fetched.
+    const int spread = (gridDim.x & 7) == 0 ? static_cast<int>((blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3)) : static_cast<int>(blockIdx.x);
+    const int item_begin = PERSIST ? static_cast<int>(static_cast<int64_t>(blockIdx.x) * a.items / gridDim.x) : spread;
     const int item_end = PERSIST ? static_cast<int>(static_cast<int64_t>(blockIdx.x + 1) * a.items / gridDim.x) : item_begin + 1;
 
     // operand fragments straight from global memory: lane (m, half) holds bytes [16*half, 16*half+16) of
