@@ -7,16 +7,17 @@
 
 namespace a4g {
 
-// Saturating add of four packed int8 lanes. Even bytes are moved to the high byte of each 16-bit
-// half so that the 16-bit saturating add clamps exactly where the int8 add would.
+// Saturating add of four packed int8 lanes. Even and odd bytes are moved to the high byte of each 16-bit half (one
+// v_perm each for the even ones, one mask for the odd ones) so that the packed 16-bit saturating add clamps exactly
+// where the int8 add would; a last v_perm gathers the four high bytes.
 __device__ __forceinline__ unsigned sat_add_i8x4(unsigned a, unsigned b) {
-    const v2s ae = __builtin_bit_cast(v2s, (a << 8) & 0xFF00FF00u);
-    const v2s be = __builtin_bit_cast(v2s, (b << 8) & 0xFF00FF00u);
-    const v2s ao = __builtin_bit_cast(v2s, a & 0xFF00FF00u);
+    const v2s ae = __builtin_bit_cast(v2s, __builtin_amdgcn_perm(a, 0u, 0x060c040cu));  // [0, a0, 0, a2]
+    const v2s be = __builtin_bit_cast(v2s, __builtin_amdgcn_perm(b, 0u, 0x060c040cu));
+    const v2s ao = __builtin_bit_cast(v2s, a & 0xFF00FF00u);                            // [0, a1, 0, a3]
     const v2s bo = __builtin_bit_cast(v2s, b & 0xFF00FF00u);
     const unsigned se = __builtin_bit_cast(unsigned, __builtin_elementwise_add_sat(ae, be));
     const unsigned so = __builtin_bit_cast(unsigned, __builtin_elementwise_add_sat(ao, bo));
-    return (so & 0xFF00FF00u) | ((se >> 8) & 0x00FF00FFu);
+    return __builtin_amdgcn_perm(so, se, 0x07030501u);  // bytes: se.1, so.1, se.3, so.3
 }
 
 // Nearest Q15 of 1/sqrt(v), v >= 1, clamped to 32767: the answer is the largest q with
