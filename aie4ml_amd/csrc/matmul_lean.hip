@@ -48,20 +48,29 @@ __device__ __forceinline__ void lean_nt_compute(const LeanArgs& a, __amdgpu_buff
         v4i o[TG];
 #pragma unroll
         for (int T = 0; T < TG; ++T) {
-            v16i acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            // BIT == 3: the sums start from the bit pattern of the float 1.5 * 2^23. Floats of that binade are one apart,
+            // so adding an integer x (|x| <= K * 2^14 <= 2^21 here) to the pattern gives the pattern of 1.5 * 2^23 + x:
+            // the accumulators leave the matrix unit already converted, and one fused multiply-add with the constant
+            // bias - 1.5 * 2^23 * 2^-s yields x * 2^-s + bias exactly (every term a multiple of 2^-s below 2^24).
+            constexpr int START = BIT == 3 ? 0x4B400000 : 0;
+            v16i acc = {START, START, START, START, START, START, START, START, START, START, START, START, START, START, START, START};
 #pragma unroll
             for (int ks = 0; ks < DT; ++ks) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[T][ks], af[rb][ks], acc, 0, 0, 0);
 #pragma unroll
             for (int gg = 0; gg < 4; ++gg) {
                 if (BIT == 3) {
-                    // |acc| <= K * 2^14 <= 2^21 and the bias 2^(7 + shift) <= 2^22: (acc + 128 * 2^s) * 2^-s is exact
-                    // in a float; v_cvt_pk_u8_f32 rounds to nearest even, saturates to 0..255 and places the byte
-                    const float bias = UOUT ? 0.f : 128.f;
+                    // v_cvt_pk_u8_f32 rounds to nearest even, saturates to 0..255 and places the byte
+                    const float bias = (UOUT ? 0.f : 128.f) - 12582912.f * a.fscale;
                     unsigned w = 0;
-                    w = __builtin_amdgcn_cvt_pk_u8_f32(fmaf(static_cast<float>(acc[4 * gg]), a.fscale, bias), 0, w);
-                    w = __builtin_amdgcn_cvt_pk_u8_f32(fmaf(static_cast<float>(acc[4 * gg + 1]), a.fscale, bias), 1, w);
-                    w = __builtin_amdgcn_cvt_pk_u8_f32(fmaf(static_cast<float>(acc[4 * gg + 2]), a.fscale, bias), 2, w);
-                    w = __builtin_amdgcn_cvt_pk_u8_f32(fmaf(static_cast<float>(acc[4 * gg + 3]), a.fscale, bias), 3, w);
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        const int sum_bits = acc[4 * gg + t];  // (a bit cast applied to the vector's element reads element 0)
+                        const float v = fmaf(__builtin_bit_cast(float, sum_bits), a.fscale, bias);
+                        if (t == 0) w = __builtin_amdgcn_cvt_pk_u8_f32(v, 0, w);
+                        if (t == 1) w = __builtin_amdgcn_cvt_pk_u8_f32(v, 1, w);
+                        if (t == 2) w = __builtin_amdgcn_cvt_pk_u8_f32(v, 2, w);
+                        if (t == 3) w = __builtin_amdgcn_cvt_pk_u8_f32(v, 3, w);
+                    }
                     o[T][gg] = static_cast<int>(UOUT ? w : w ^ 0x80808080u);
                 } else {
                     o[T][gg] = static_cast<int>(requant4_bytes<BIT>(acc[4 * gg], acc[4 * gg + 1], acc[4 * gg + 2], acc[4 * gg + 3], a.br));
