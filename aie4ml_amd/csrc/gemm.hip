@@ -13,6 +13,7 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "gemm_direct.hpp"
 #include "gemm_epilogue.hpp"
 #include "gemm_rs.hpp"
 #include "matmul_lean.hpp"
@@ -303,6 +304,7 @@ struct I8Policy {
     static constexpr int MMAS = 1, KSTEP_BYTES = 32;
     static constexpr bool FIX_A = A_UNSIGNED;
     static constexpr bool SPLIT_A = false, SPLIT_B = false;
+    static constexpr bool PERM_B = false;
     struct Extra {};
     static constexpr int MAX_OUT_BYTES = 2;
     template <int BN>
@@ -327,6 +329,91 @@ struct I8Policy {
                                                     int8_t* smem, int8_t* lds_params, int path, int wm, int wn, int lane,
                                                     int tid, Extra&) {
         epilogue_store<BM, BN, WTM, WTN, NT>(g, tc, acc, smem, ColParams<BN>(lds_params), path, wm, wn, lane, tid);
+    }
+};
+
+// The int8 policy with the epilogue of the register-requantising kernels (gemm_direct.hpp): weight rows in the order that
+// makes a lane's 16 accumulators of a block 16 neighbouring columns, accumulators started from bias + 128 * colsum, four
+// vector instructions per value in the quick form (shifts within 1..15, sums inside int32), 16-byte stores straight from
+// registers: no LDS image of the output tile. For one-byte outputs in whole 16-column pieces on 16-byte aligned rows;
+// column blocks that need the general requantisation leave through the LDS image as before (same bits either way:
+// int32 addition wraps, so where the bias joins the sum does not matter).
+template <bool A_UNSIGNED>
+struct I8DirectPolicy : I8Policy<A_UNSIGNED> {
+    static constexpr bool PERM_B = true;
+    using Extra = typename I8Policy<A_UNSIGNED>::Extra;
+    using ColRegs = typename I8Policy<A_UNSIGNED>::ColRegs;
+    template <int BN>
+    static constexpr int param_bytes() { return DirectParams<BN>::BYTES; }
+    template <int BN>
+    __device__ static __forceinline__ int park_params(const GemmArgs& g, int8_t* lds, int tid, const ColRegs& r) {
+        const int lo = g.relu ? max(kind_lo(g.out_kind), 0) : kind_lo(g.out_kind), hi = kind_hi(g.out_kind);
+        return direct_park<BN>(g, DirectParams<BN>(lds), tid, r.add, r.shift, lo, hi) ? 2 : 0;
+    }
+    template <int BN, int WTN, int TM, int TN>
+    __device__ static __forceinline__ void start_acc(v16i (&acc)[TM][TN], int8_t* lds_params, int wn, int lane) {
+        const DirectParams<BN> wp(lds_params);
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const v4i add4 = *reinterpret_cast<const v4i*>(wp.add + wn * WTN + j * 32 + 16 * (lane >> 5) + 4 * q);
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) acc[i][j][q * 4 + t] = add4[t];
+            }
+    }
+    template <int BM, int BN, int WTM, int WTN, int NT>
+    __device__ static __forceinline__ void epilogue(const GemmArgs& g, const TileCoord& tc, v16i (&acc)[WTM / 32][WTN / 32],
+                                                    int8_t* smem, int8_t* lds_params, int path, int wm, int wn, int lane,
+                                                    int tid, Extra&) {
+        if (path != 0) {  // some column of the tile needs the general form
+            epilogue_store<BM, BN, WTM, WTN, NT, true, true>(g, tc, acc, smem, ColParams<BN>(lds_params), 2, wm, wn, lane, tid);
+            return;
+        }
+        constexpr int TM = WTM / 32, TN = WTN / 32;
+        const DirectParams<BN> wp(lds_params);
+        const int half = lane >> 5, frow = lane & 31;
+        auto quick = [&](auto bit_tag, auto conv_tag) {
+            constexpr int BIT = decltype(bit_tag)::value;
+            constexpr bool CONV = decltype(conv_tag)::value;
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int nl = wn * WTN + j * 32 + 16 * half + 4 * q;
+                    const v4i s4 = *reinterpret_cast<const v4i*>(wp.s + nl);
+                    const v4i c04 = *reinterpret_cast<const v4i*>(wp.c0 + nl);
+                    const v4i lo4 = *reinterpret_cast<const v4i*>(wp.lo_s + nl);
+                    const v4i hi4 = *reinterpret_cast<const v4i*>(wp.hi_s + nl);
+#pragma unroll
+                    for (int i = 0; i < TM; ++i)
+                        acc[i][j][q] = static_cast<int>(direct_requant4<BIT, CONV>(acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2],
+                                                                                     acc[i][j][q * 4 + 3], s4, c04, lo4, hi4));
+                }
+        };
+        using B0 = std::integral_constant<int, 0>;
+        using B1 = std::integral_constant<int, 1>;
+        using B2 = std::integral_constant<int, 2>;
+        if (g.mode <= A4G_RND_NEGATIVE_INF) quick(B0{}, std::false_type{});
+        else if (g.mode == A4G_RND_SYMMETRIC_INF) quick(B2{}, std::false_type{});
+        else if (g.mode == A4G_RND_SYMMETRIC_ZERO) quick(B1{}, std::false_type{});
+        else if (g.mode == A4G_RND_CONV_EVEN) quick(B1{}, std::true_type{});
+        else quick(B2{}, std::true_type{});
+        int8_t* Cb = static_cast<int8_t*>(g.C) + tc.batch * g.stride_c;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+            const int m = tc.m0 + wm * WTM + i * 32 + frow;
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int n = tc.n0 + wn * WTN + j * 32 + 16 * half;
+                if (m < g.M && n + 16 <= g.N) {
+                    const v4i o = {acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]};
+                    *reinterpret_cast<v4i*>(Cb + static_cast<int64_t>(m) * g.ldc + n) = o;
+                }
+            }
+        }
     }
 };
 
@@ -698,6 +785,10 @@ static hipError_t launch_gemm_nt(const GemmArgs& g, int batch, hipStream_t strea
     const bool k128 = g.K % 128 == 0, k64 = g.K % 64 == 0;
     switch (variant) {
     case 1:  // 256 x 256
+        if (k128 && (g.out_kind == A4G_I8 || g.out_kind == A4G_U8) && g.N % 16 == 0 && g.ldc % 16 == 0 && g.stride_c % 16 == 0 &&
+            aligned16(g.C))  // the epilogue that requantises and stores from registers
+            return g.a_unsigned ? launch_rs_policy<I8DirectPolicy<true>, 256, 256, 2, 4, true>(g, batch, stream)
+                                : launch_rs_policy<I8DirectPolicy<false>, 256, 256, 2, 4, true>(g, batch, stream);
         if (k128) return g.a_unsigned ? launch_rs_u<256, 256, 2, 4, true, true>(g, batch, stream)
                                       : launch_rs_u<256, 256, 2, 4, false, true>(g, batch, stream);
         if (k64) return launch_dtl<256, 256, 64, 2, 4, 4>(g, batch, stream);

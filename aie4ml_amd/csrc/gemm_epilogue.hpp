@@ -67,7 +67,9 @@ __device__ __forceinline__ int park_col_params(const GemmArgs& g, const ColParam
 // offset is added with a saturating add: a sum that would overflow lies far above any output range
 // either way, so the clamp gives the same value. Larger shifts take the overflow-free form.
 // The caller has made sure that no tile load is in flight and that all waves are past the main loop.
-template <int BM, int BN, int WTM, int WTN, int NT>
+// PERM: the weight rows were taken in the order of direct_col_of_operand_row, so accumulator 4 q + t of a lane is column
+// 16 * (lane / 32) + 4 q + t of its block (not 8 q + 4 * (lane / 32) + t); ADDED: the accumulators started from `add`.
+template <int BM, int BN, int WTM, int WTN, int NT, bool PERM = false, bool ADDED = false>
 __device__ __forceinline__ void epilogue_store(const GemmArgs& g, const TileCoord& tc, v16i (&acc)[WTM / 32][WTN / 32],
                                                int8_t* smem, const ColParams<BN>& cp, int round_path, int wm, int wn, int lane,
                                                int tid) {
@@ -90,8 +92,8 @@ __device__ __forceinline__ void epilogue_store(const GemmArgs& g, const TileCoor
         for (int j = 0; j < TN; ++j) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const int nl = wn * WTN + j * 32 + 8 * q + 4 * (lane >> 5);  // column inside the tile
-                const v4i add4 = *reinterpret_cast<const v4i*>(cp.add + nl);
+                const int nl = wn * WTN + j * 32 + (PERM ? 16 * (lane >> 5) + 4 * q : 8 * q + 4 * (lane >> 5));  // column inside the tile
+                const v4i add4 = ADDED ? v4i{0, 0, 0, 0} : *reinterpret_cast<const v4i*>(cp.add + nl);
                 const v4i s4 = *reinterpret_cast<const v4i*>(cp.s + nl);
                 const v4i c04 = *reinterpret_cast<const v4i*>(cp.c0 + nl);
                 const v4i cx4 = *reinterpret_cast<const v4i*>(cp.cx + nl);
@@ -132,8 +134,8 @@ __device__ __forceinline__ void epilogue_store(const GemmArgs& g, const TileCoor
         for (int j = 0; j < TN; ++j) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                const int nl = wn * WTN + j * 32 + 8 * q + 4 * (lane >> 5);
-                const v4i add4 = *reinterpret_cast<const v4i*>(cp.add + nl);
+                const int nl = wn * WTN + j * 32 + (PERM ? 16 * (lane >> 5) + 4 * q : 8 * q + 4 * (lane >> 5));
+                const v4i add4 = ADDED ? v4i{0, 0, 0, 0} : *reinterpret_cast<const v4i*>(cp.add + nl);
                 const v4i s4 = *reinterpret_cast<const v4i*>(cp.s + nl);
                 const v4i c04 = *reinterpret_cast<const v4i*>(cp.c0 + nl);
 #pragma unroll

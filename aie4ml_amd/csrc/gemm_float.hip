@@ -68,6 +68,7 @@ struct FloatPolicy {
     static constexpr int MMAS = FMT == A4G_F32 ? 4 : 1;
     static constexpr bool FIX_A = false;
     static constexpr bool SPLIT_A = false, SPLIT_B = false;
+    static constexpr bool PERM_B = false;
     struct Extra {};
     static constexpr int MAX_OUT_BYTES = ES;
     template <int BN>

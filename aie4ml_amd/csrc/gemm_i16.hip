@@ -321,6 +321,7 @@ struct I16x16Policy {
     using acc_t = v16i;
     static constexpr int MMAS = 1, KSTEP_BYTES = 32;
     static constexpr bool FIX_A = false, SPLIT_A = true, SPLIT_B = true;
+    static constexpr bool PERM_B = false;
     static constexpr int MAX_OUT_BYTES = 1;  // the output image holds 128 x 128 two-byte elements in a 256 x 256 one-byte frame
     static constexpr int MAX_ROWS = 128;
     struct Extra {

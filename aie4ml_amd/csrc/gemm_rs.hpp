@@ -281,7 +281,16 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
 #pragma unroll
         for (int f = 0; f < FR; ++f) koff[kk][f] = (((kk * 2 + (lane >> 5)) * FR + f) ^ ((frow >> 1) & 7)) * 16;
     const int a_off = (wm * Cfg::WTM + frow) * BK;
-    const int b_off = BM * BK + (wn * Cfg::WTN + frow) * BK;
+    // PERM_B: the lane supplies the weight row of another column of its 32-column block (direct_col_of_operand_row), so that
+    // a lane's 16 accumulators of a block are 16 neighbouring columns, which the policy's epilogue requantises and
+    // stores straight from registers
+    const int brow = P::PERM_B ? direct_col_of_operand_row(frow) : frow;
+    const int b_off = BM * BK + (wn * Cfg::WTN + brow) * BK;
+    int koffb[KSTEPS][FR];
+#pragma unroll
+    for (int kk = 0; kk < KSTEPS; ++kk)
+#pragma unroll
+        for (int f = 0; f < FR; ++f) koffb[kk][f] = P::PERM_B ? (((kk * 2 + (lane >> 5)) * FR + f) ^ ((brow >> 1) & 7)) * 16 : koff[kk][f];
 
     typename P::acc_t acc[Cfg::TM][Cfg::TN];
 #pragma unroll
@@ -290,6 +299,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
         for (int j = 0; j < Cfg::TN; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+    if constexpr (P::PERM_B) P::template start_acc<BN, Cfg::WTN>(acc, smem + Cfg::PARAM_OFF, wn, lane);
 
     v4i af[2][Cfg::TM][FR], bf[2][Cfg::TN][FR];
     constexpr int NR = Cfg::TM + Cfg::TN, NM = Cfg::TM * Cfg::TN;
@@ -299,13 +309,13 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
         for (int f = 0; f < FR; ++f) {
             if (idx < 2 * TMIN) {
                 if (idx & 1) af[set][idx >> 1][f] = *reinterpret_cast<const v4i*>(base + a_off + (idx >> 1) * 32 * BK + koff[kk][f]);
-                else bf[set][idx >> 1][f] = *reinterpret_cast<const v4i*>(base + b_off + (idx >> 1) * 32 * BK + koff[kk][f]);
+                else bf[set][idx >> 1][f] = *reinterpret_cast<const v4i*>(base + b_off + (idx >> 1) * 32 * BK + koffb[kk][f]);
             } else if (Cfg::TM > Cfg::TN) {
                 const int i = idx - TMIN;
                 af[set][i][f] = *reinterpret_cast<const v4i*>(base + a_off + i * 32 * BK + koff[kk][f]);
             } else {
                 const int j = idx - TMIN;
-                bf[set][j][f] = *reinterpret_cast<const v4i*>(base + b_off + j * 32 * BK + koff[kk][f]);
+                bf[set][j][f] = *reinterpret_cast<const v4i*>(base + b_off + j * 32 * BK + koffb[kk][f]);
             }
         }
     };
