@@ -734,8 +734,15 @@ static hipError_t launch_dtl_u(const GemmArgs& g, int batch, hipStream_t stream)
     return hipGetLastError();
 }
 
+// One-byte outputs in whole 16-column pieces on 16-byte aligned rows take the epilogue that requantises and stores from
+// registers (I8DirectPolicy); everything else the LDS image.
+static bool direct_epilogue_ok(const GemmArgs& g) {
+    return (g.out_kind == A4G_I8 || g.out_kind == A4G_U8) && g.N % 16 == 0 && g.ldc % 16 == 0 && g.stride_c % 16 == 0 && aligned16(g.C);
+}
+
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool A_UNSIGNED, bool EARLY = false>
 static hipError_t launch_rs_u(const GemmArgs& g, int batch, hipStream_t stream) {
+    if (direct_epilogue_ok(g)) return launch_rs_policy<I8DirectPolicy<A_UNSIGNED>, BM, BN, WAVES_M, WAVES_N, EARLY>(g, batch, stream);
     return launch_rs_policy<I8Policy<A_UNSIGNED>, BM, BN, WAVES_M, WAVES_N, EARLY>(g, batch, stream);
 }
 
@@ -785,10 +792,6 @@ static hipError_t launch_gemm_nt(const GemmArgs& g, int batch, hipStream_t strea
     const bool k128 = g.K % 128 == 0, k64 = g.K % 64 == 0;
     switch (variant) {
     case 1:  // 256 x 256
-        if (k128 && (g.out_kind == A4G_I8 || g.out_kind == A4G_U8) && g.N % 16 == 0 && g.ldc % 16 == 0 && g.stride_c % 16 == 0 &&
-            aligned16(g.C))  // the epilogue that requantises and stores from registers
-            return g.a_unsigned ? launch_rs_policy<I8DirectPolicy<true>, 256, 256, 2, 4, true>(g, batch, stream)
-                                : launch_rs_policy<I8DirectPolicy<false>, 256, 256, 2, 4, true>(g, batch, stream);
         if (k128) return g.a_unsigned ? launch_rs_u<256, 256, 2, 4, true, true>(g, batch, stream)
                                       : launch_rs_u<256, 256, 2, 4, false, true>(g, batch, stream);
         if (k64) return launch_dtl<256, 256, 64, 2, 4, 4>(g, batch, stream);
