@@ -28,7 +28,7 @@ struct AttnArgs {
     int64_t o_sb, o_sh, o_ss;
     int heads, sq;
     int d;      // head dimension that exists, a multiple of 16 up to the kernel's width: the 16-byte pieces of a row past it do not
-    int sk;     // key / value rows that exist (the ragged form; the kernel's tiles cover the next power of two of 32s)
+    int sk;     // key / value rows that exist (the ragged form; the kernel's tiles cover the next tile count that has an instance)
     int items;  // (batch, head, block of query rows) triples in all
     FastRound lr, orr;  // logits and output requantisation
     SoftmaxParams sm;
@@ -492,6 +492,24 @@ static int launch_attention(int nt, int grid, int grid8, hipStream_t stream, con
     case 2: launch_attention_nt<2, DT>(grid, 0, lds, stream, a); break;
     case 4: launch_attention_nt<4, DT>(grid, 0, lds, stream, a); break;
     case 8: launch_attention_nt<8, DT>(grid, grid8, lds, stream, a); break;
+    // tile counts between the powers of two, for the 64-wide heads only (96, 160, 192 and 384 keys: a kernel of the next
+    // power of two would spend a quarter to three eighths of its three passes on keys that do not exist)
+    case 3:
+        if constexpr (DT == 2) launch_attention_nt<3, DT>(grid, 0, lds, stream, a);
+        else return 1;
+        break;
+    case 5:
+        if constexpr (DT == 2) launch_attention_nt<5, DT>(grid, 0, lds, stream, a);
+        else return 1;
+        break;
+    case 6:
+        if constexpr (DT == 2) launch_attention_nt<6, DT>(grid, 0, lds, stream, a);
+        else return 1;
+        break;
+    case 12:
+        if constexpr (DT == 2) launch_attention_nt<12, DT>(grid, grid8, lds, stream, a);
+        else return 1;
+        break;
     case 16:
         if constexpr (DT <= 2) launch_attention_nt<16, DT>(grid, grid8, lds, stream, a);
         else return 1;
@@ -532,8 +550,17 @@ extern "C" int a4g_attention_i8(const int8_t* Q, const int8_t* K, const int8_t* 
                 "%s: fused path covers head dimensions that are multiples of 16, up to 64 with up to 512 keys and up to 128 with up "
                 "to 256, got d=%lld sk=%lld", who, (long long)d, (long long)sk);
     const int width = d <= 32 ? 32 : (d <= 64 ? 64 : 128);  // of the kernel: narrower heads run with their missing pieces masked
-    int nt = 1;  // tiles of 32 keys the kernel is instantiated for: the next power of two
-    while (nt * 32 < sk) nt *= 2;
+    // tiles of 32 keys the kernel is instantiated for: the powers of two, and for 64-wide heads also 3, 5, 6 and 12
+    static const int tile_counts_64[] = {1, 2, 3, 4, 5, 6, 8, 12, 16};
+    static const int tile_counts[] = {1, 2, 4, 8, 16};
+    int nt = 16;
+    if (width == 64) {
+        for (int i = 8; i >= 0; --i)
+            if (tile_counts_64[i] * 32 >= sk) nt = tile_counts_64[i];
+    } else {
+        for (int i = 4; i >= 0; --i)
+            if (tile_counts[i] * 32 >= sk) nt = tile_counts[i];
+    }
     const bool ragged = nt * 32 != sk;
     A4G_REQUIRE(batch * heads * ((sq + 127) / 128) <= INT32_MAX && sq <= (1 << 24), A4G_ERR_UNSUPPORTED, "%s: too many rows", who);
     if (batch == 0) return A4G_OK;

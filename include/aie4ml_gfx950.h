@@ -300,9 +300,9 @@ A4G_API int a4g_mlp_add_layernorm_i8(const a4g_mlp_layer* layers, int n_layers, 
  *   use_clb), same parameter rules as the stand-alone entries; probabilities are uint8.
  * Covered shapes: d a multiple of 16, up to 64 with 1 <= sk <= 512 and up to 128 with 1 <= sk <= 256 (head
  * dimensions 16, 48, 80, 96 and 112 run the 32-, 64- and 128-wide kernels with the missing 16-byte pieces of a row
- * masked; any key count: counts off the 32-grid, e.g. 197 tokens, run the kernel of the next power of two with the
- * missing keys masked out), any sq, pointers and strides multiples of 16 bytes, the keys of one head within
- * 2 GiB; anything else returns A4G_ERR_UNSUPPORTED and the caller runs the three operators separately. */
+ * masked; any key count: kernels exist for 1, 2, 4, 8 and 16 tiles of 32 keys, for head dimensions 48 and 64 also for
+ * 3, 5, 6 and 12, and a count in between, e.g. 100 tokens, runs the next of them with the missing keys masked out),
+ * any sq, pointers and strides multiples of 16 bytes, the keys of one head within 2 GiB; anything else returns A4G_ERR_UNSUPPORTED and the caller runs the three operators separately. */
 A4G_API int a4g_attention_i8(const int8_t* Q, const int8_t* K, const int8_t* V, int8_t* O, int64_t batch, int64_t heads,
                      int64_t sq, int64_t sk, int64_t d, const int64_t* strides, int logit_shift,
                      int logit_round_mode, int softmax_kind, int exp_kq, int hccs_B, int hccs_S, int hccs_Dmax,

@@ -29,10 +29,11 @@ def qkv(seed, shape_q, shape_k, sigma=24.0):
     return g(shape_q), g(shape_k), g(shape_k)
 
 
-HCCS = {32: (255, 4, 60), 64: (255, 3, 80), 128: (255, 2, 126), 256: (127, 1, 126), 512: (60, 1, 59)}
+HCCS = {32: (255, 4, 60), 64: (255, 3, 80), 96: (255, 3, 80), 128: (255, 2, 126), 160: (200, 2, 90), 192: (170, 1, 126),
+        256: (127, 1, 126), 384: (85, 1, 80), 512: (60, 1, 59)}
 
 
-@pytest.mark.parametrize('sk', [32, 64, 128, 256, 512])
+@pytest.mark.parametrize('sk', [32, 64, 96, 128, 160, 192, 256, 384, 512])
 @pytest.mark.parametrize('kind', ['exp', 'hccs'])
 def test_attention_matches_three_operators(oracle, sk, kind):
     q, k, v = qkv(sk, (2, 3, sk, 64), (2, 3, sk, 64))
@@ -64,10 +65,10 @@ def test_attention_ragged_query_count(oracle, sq):
     np.testing.assert_array_equal(got, reference(oracle, q, k, v, 6, 'symmetric_inf', sm, 8, 'floor'))
 
 
-@pytest.mark.parametrize('sk', [1, 5, 31, 33, 96, 100, 197, 250, 300, 511])
+@pytest.mark.parametrize('sk', [1, 5, 31, 33, 90, 96, 100, 150, 180, 197, 250, 300, 370, 511])
 @pytest.mark.parametrize('kind', ['exp', 'hccs'])
 def test_attention_key_count_off_the_tile_grid(oracle, sk, kind):
-    """Any number of keys up to 512: the kernel of the next power of two runs with the missing keys masked (they
+    """Any number of keys up to 512: the kernel of the next tile count that has one runs with the missing keys masked (they
     must neither raise a row's maximum, nor add to its sum, nor to the output). Self-attention shapes (sq == sk, as
     a 197-token ViT block has them), plus a query count of its own; both forms of the logit requantisation."""
     for sq in (sk, 70):
@@ -138,7 +139,7 @@ def test_attention_masked_keys_do_not_leak(oracle):
     np.testing.assert_array_equal(got, want)
 
 
-@pytest.mark.parametrize('sq,sk', [(512, 512), (300, 256), (256, 512)])
+@pytest.mark.parametrize('sq,sk', [(512, 512), (300, 256), (256, 512), (512, 384), (300, 384)])
 @pytest.mark.parametrize('mode', ['conv_even', 'symmetric_inf', 'floor'])
 def test_attention_with_256_row_workgroups(oracle, sq, sk, mode):
     # at least 256 workgroups of 256 query rows and 256 or more keys: the eight-wave form with the score table
@@ -150,6 +151,17 @@ def test_attention_with_256_row_workgroups(oracle, sq, sk, mode):
                {'kind': 'exp', 'exp_kq': 23, 'inv_shift': 17}):
         got = ops.attention(dev(q), dev(k), dev(v), 6, mode, sm, 7, mode).cpu().numpy()
         np.testing.assert_array_equal(got, reference(oracle, q, k, v, 6, mode, sm, 7, mode))
+
+
+@pytest.mark.parametrize('sk', [96, 160, 192, 384])
+@pytest.mark.parametrize('mode', ['floor', 'symmetric_inf', 'symmetric_zero', 'conv_even', 'conv_odd'])
+def test_attention_tile_counts_between_the_powers_of_two(oracle, sk, mode):
+    """3, 5, 6 and 12 key tiles have kernels of their own for 64-wide heads: every form of the logit requantisation, both
+    forms of the probability (the shift of 17 needs the clamp), a ragged query count."""
+    q, k, v = qkv(4000 + sk, (2, 3, sk - 7, 64), (2, 3, sk, 64), sigma=36.0)
+    for sm in ({'kind': 'exp', 'exp_kq': 31}, {'kind': 'exp', 'exp_kq': 23, 'inv_shift': 17}):
+        got = ops.attention(dev(q), dev(k), dev(v), 5, mode, sm, 7, mode).cpu().numpy()
+        np.testing.assert_array_equal(got, reference(oracle, q, k, v, 5, mode, sm, 7, mode))
 
 
 def test_attention_zero_shift_and_saturation(oracle):
