@@ -28,13 +28,17 @@ __device__ __forceinline__ unsigned sat_add_u8x4(unsigned a, unsigned b) {
     return se | (so << 8);
 }
 
+// The row kernels of this file load with the default cache policy and store non-temporally. An operand that the launch
+// before has written, or read, is then found in the 256 MB memory-side cache where it fits; loads marked non-temporal
+// never are (measured on 16384 x 1024: LayerNorm 8.1 -> 6.5 us, Add 7.0 -> 6.5 us, Softmax on 134 MB 44.6 -> 39.8 us),
+// while results that leave without allocating there do not push the operands out (Add with plain stores: 8.7 us).
 template <bool UNSIGNED>
 __global__ __launch_bounds__(256) void add_sat8_kernel(const v4i* __restrict__ a, const v4i* __restrict__ b,
                                                         v4i* __restrict__ out, int64_t nvec) {
     const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec; i += stride) {
-        const v4i va = __builtin_nontemporal_load(a + i);
-        const v4i vb = __builtin_nontemporal_load(b + i);
+        const v4i va = a[i];
+        const v4i vb = b[i];
         v4i r;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -52,8 +56,8 @@ __global__ __launch_bounds__(256) void add_vec_kernel(const v4i* __restrict__ a,
                                                        int64_t nvec, FastRound fr, int lo, int hi) {
     const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
     for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec; i += stride) {
-        const v4i va = __builtin_nontemporal_load(a + i);
-        const v4i vb = __builtin_nontemporal_load(b + i);
+        const v4i va = a[i];
+        const v4i vb = b[i];
         v4i r;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
@@ -241,7 +245,8 @@ __global__ __launch_bounds__(256, 2) void layernorm_rows_kernel(const int8_t* __
     const auto rsrc_x2 = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(x2), 0, FUSE_ADD ? tensor_bytes : 0, 0x00020000);
     const auto rsrc_sum = __builtin_amdgcn_make_buffer_rsrc(sum_out, 0, sum_out ? tensor_bytes : 0, 0x00020000);
     const auto rsrc_out = __builtin_amdgcn_make_buffer_rsrc(out, 0, tensor_bytes, 0x00020000);
-    constexpr int NT = 2;  // non-temporal
+    constexpr int NT = 2;     // stores: non-temporal
+    constexpr int CACHED = 0;  // loads: default policy (see add_sat8_kernel)
     auto offset_of = [&](int row, int i) {
         return row < rows && valid[i] ? static_cast<unsigned>(row) * static_cast<unsigned>(cols) + chunk_of[i] * 16 : NOWHERE;
     };
@@ -249,8 +254,8 @@ __global__ __launch_bounds__(256, 2) void layernorm_rows_kernel(const int8_t* __
     auto fetch = [&](int row) {
 #pragma unroll
         for (int i = 0; i < NCH; ++i) {
-            nx[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, offset_of(row, i), 0, NT));
-            if (FUSE_ADD) nx2[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_x2, offset_of(row, i), 0, NT));
+            nx[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_x, offset_of(row, i), 0, CACHED));
+            if (FUSE_ADD) nx2[i] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_x2, offset_of(row, i), 0, CACHED));
         }
     };
     auto put = [&](__amdgpu_buffer_rsrc_t rsrc, const v4i& v, int row, int i) {
@@ -658,7 +663,7 @@ __global__ __launch_bounds__(256) void softmax_lut_kernel(const int8_t* __restri
                     }
                 }
             } else {
-                if (valid[i]) xv[i] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(x + base + col0));
+                if (valid[i]) xv[i] = *reinterpret_cast<const v4i*>(x + base + col0);
             }
 #pragma unroll
             for (int j = 0; j < 4; ++j) m = max(m, max_i8x4(xv[i][j]));

@@ -9,6 +9,9 @@ inputs already resident in HBM. Prints ONE JSON line.
 The default run also times, after the headline workload, the matrix-core calibration loop (`roofline.calibrated_peak`,
 `frac_of_calibrated`, the clock under matrix load) and every other baseline configuration with the same method
 (`workloads`: value, ms_per_step, bit_exact, roofline per configuration; no CPU leg). `--only` skips both.
+The HBM-bound workloads are timed twice: on one set of buffers like every other workload (`value`, `roofline.frac`:
+operands that fit the 256 MB memory-side cache are found there by the next launch), and over a ring of operand copies
+of 1 GiB (`roofline.frac_operands_from_hbm`: every operand comes from HBM).
 
 Other workloads (--workload c2_dense_i16 | c2_dense_i16x16 | c2_dense_bf16 | c2_dense_fp8 | c1_mlp | c1_mlp_stream | c3_softmax_exp | c3_softmax_hccs | c3_qk | c3_pv |
 c3_attention_exp | c3_attention_hccs | c4_add_layernorm | c4_layernorm | c4_add | c5_encoder) print the same line for that operator or graph;
@@ -34,6 +37,7 @@ PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, TOP/s
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, TFLOP/s
 PEAK_FP8_TFLOPS = 5000.0   # MI355X dense fp8 MFMA, TFLOP/s
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
+COLD_RING_BYTES = 1 << 30  # operand copies the cold leg of the HBM-bound workloads cycles through: 4 x the 256 MB memory-side cache
 
 # HBM bytes per launch of each workload's dominant kernel come from hardware counters (FETCH_SIZE and WRITE_SIZE, one
 # counter run each, scaled by what the same counter reads for calib_copy). The summaries of those runs are the text
@@ -124,6 +128,24 @@ def prepare(wl, torch):
 
     dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).cuda()  # noqa: E731
     extra = {}
+    fn_cold = None
+
+    def rotating(call, tensors, bytes_per_launch):
+        """`call(*tensors)` over a ring of copies of the tensors that holds COLD_RING_BYTES in all: by the time a copy's
+        turn comes again, four times the memory-side cache's capacity has passed through it, so every launch fetches its
+        operands from HBM. The plain step function works on one set of buffers, which a replayed graph finds in that
+        cache again where they fit (the C4 tensors do)."""
+        nsets = max(2, -(-COLD_RING_BYTES // int(bytes_per_launch)))
+        ring = [tuple(t.clone() for t in tensors) for _ in range(nsets)]
+        turn = [0]
+
+        def step():
+            ts = ring[turn[0] % nsets]
+            turn[0] += 1
+            call(*ts)
+
+        step.bytes_per_launch = int(bytes_per_launch)
+        return step
     cpu_fn = None
     cpu_samples = None
     cpu_work = cpu_desc = None
@@ -331,6 +353,8 @@ def prepare(wl, torch):
             work = 3.0 * rows * cols
             cpu_fn = lambda: oracle.add_layernorm(a, b, gamma, beta, prm['out_shift'], 'conv_even')  # noqa: E731
             kernel = 'layernorm_rows_kernel'
+            fn_cold = rotating(lambda a_, b_, o_: ops.add_layernorm(a_, b_, dg, dbt, prm['out_shift'], 'conv_even', out=o_),
+                               (da, db, dout), work)
         elif wl == 'c4_layernorm':
             fn = lambda: ops.layernorm(da, dg, dbt, prm['out_shift'], 'conv_even', out=dout)  # noqa: E731
             got = fn()
@@ -338,6 +362,7 @@ def prepare(wl, torch):
             work = 2.0 * rows * cols
             cpu_fn = lambda: oracle.layernorm(a, gamma, beta, prm['out_shift'], 'conv_even')  # noqa: E731
             kernel = 'layernorm_rows_kernel'
+            fn_cold = rotating(lambda a_, o_: ops.layernorm(a_, dg, dbt, prm['out_shift'], 'conv_even', out=o_), (da, dout), work)
         else:
             fn = lambda: ops.add(da, db, out=dout)  # noqa: E731
             got = fn()
@@ -345,6 +370,7 @@ def prepare(wl, torch):
             work = 3.0 * rows * cols
             cpu_fn = lambda: oracle.add(a, b)  # noqa: E731
             kernel = 'add_sat8_kernel'
+            fn_cold = rotating(lambda a_, b_, o_: ops.add(a_, b_, out=o_), (da, db, dout), work)
         torch.cuda.synchronize()
         bit_exact = bool(np.array_equal(got[sub].cpu().numpy(), exp))
         bound, samples = 'hbm', rows
@@ -375,6 +401,8 @@ def prepare(wl, torch):
             cpu_desc = 'oracle MatMul on 4 of 512 (batch, head) slices'
             work = float(bytes_)
             kernel = 'matmul_lean_nt_kernel'
+            fn_cold = rotating(lambda q_, k_, o_: ops.matmul(q_, k_, prm['logit_shift'], 'conv_even', trans_b=True, out=o_),
+                               (dq, dk, out), bytes_)
         elif wl == 'c3_pv':
             ws = torch.empty((ops._lib.load().a4g_matmul_i8_workspace_bytes(Bt * H, S, D, S, 0, 1),), dtype=torch.uint8,
                              device='cuda')
@@ -391,15 +419,20 @@ def prepare(wl, torch):
             cpu_work = bytes_ * 4 / (Bt * H)
             cpu_desc = 'oracle MatMul (uint8 x int8) on 4 of 512 (batch, head) slices'
             kernel = 'matmul_lean_nn_kernel'
+            fn_cold = rotating(lambda p_, v_, o_: ops.matmul(p_, v_, prm['pv_shift'], 'conv_even', out=o_, workspace=ws),
+                               (probs, dv, out), bytes_)
         else:
             out = torch.empty(logits.shape, dtype=torch.uint8, device='cuda')
             hc = prm['hccs']
             if wl == 'c3_softmax_exp':
                 fn = lambda: ops.softmax_exp(logits, prm['exp_kq'], out=out)  # noqa: E731
+                fn_cold = rotating(lambda x_, o_: ops.softmax_exp(x_, prm['exp_kq'], out=o_), (logits, out), 2.0 * Bt * H * S * S)
                 ref = oracle.softmax_exp(l_ref, prm['exp_kq'])
                 cpu1 = lambda x_: oracle.softmax_exp(x_, prm['exp_kq'])  # noqa: E731
             else:
                 fn = lambda: ops.softmax_hccs(logits, hc['B'], hc['S'], hc['Dmax'], out=out)  # noqa: E731
+                fn_cold = rotating(lambda x_, o_: ops.softmax_hccs(x_, hc['B'], hc['S'], hc['Dmax'], out=o_), (logits, out),
+                                   2.0 * Bt * H * S * S)
                 ref = oracle.softmax_hccs(l_ref, hc['B'], hc['S'], hc['Dmax'])
                 cpu1 = lambda x_: oracle.softmax_hccs(x_, hc['B'], hc['S'], hc['Dmax'])  # noqa: E731
             fn()
@@ -492,7 +525,7 @@ def prepare(wl, torch):
         sys.exit(f'unknown workload {wl}')
 
 
-    return dict(wl=wl, fn=fn, bit_exact=bit_exact, work=work, bound=bound, samples=samples, config=config, metric=metric,
+    return dict(wl=wl, fn=fn, fn_cold=fn_cold, bit_exact=bit_exact, work=work, bound=bound, samples=samples, config=config, metric=metric,
                 unit=unit, kernel=kernel, extra=extra, cpu_fn=cpu_fn, cpu_work=cpu_work, cpu_desc=cpu_desc,
                 cpu_samples=cpu_samples, peak_mfma=peak_mfma, mfma_unit=mfma_unit)
 
@@ -515,6 +548,13 @@ def measure(torch, w, steps, warmup, eager=False):
         roof = {'bound': 'hbm', 'achieved': round(achieved, 2), 'peak': PEAK_HBM_GBS, 'unit': 'GB/s',
                 'frac': round(achieved / PEAK_HBM_GBS, 4)}
     roof.update({'traffic': traffic, 'traffic_source': source, 'kernel': w['kernel'], 'kernel_ms': round(ms_ev, 5)})
+    cold = w.get('fn_cold')
+    if cold is not None and w['bound'] == 'hbm' and steps * cold.bytes_per_launch >= COLD_RING_BYTES // 2:
+        # the same launches over a ring of operand copies four times the size of the memory-side cache: nothing is found there
+        _, ms_cold, _ = _time_gpu(torch, cold, steps, warmup, use_graph=not eager)
+        roof.update({'achieved_operands_from_hbm': round(work / (ms_cold * 1e-3) / 1e9, 2),
+                     'frac_operands_from_hbm': round(work / (ms_cold * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                     'kernel_ms_operands_from_hbm': round(ms_cold, 5)})
     if unit in ('TOP/s', 'TFLOP/s'):
         value = work / (ms * 1e-3) / 1e12
     elif unit == 'GB/s':
@@ -663,7 +703,9 @@ def main():
                 o = prepare(name, torch)
                 o_ms, o_value, o_roof, _ = measure(torch, o, args.steps, args.warmup, args.eager)
                 others[name] = {'value': float(f'{o_value:.6g}'), 'unit': o['unit'], 'ms_per_step': round(o_ms, 5),
-                                'bit_exact': o['bit_exact'], 'roofline': {k: o_roof[k] for k in ('bound', 'achieved', 'peak', 'unit', 'frac', 'traffic', 'traffic_source', 'kernel')}}
+                                'bit_exact': o['bit_exact'], 'roofline': {k: o_roof[k] for k in ('bound', 'achieved', 'peak', 'unit', 'frac', 'traffic', 'traffic_source', 'kernel',
+                                                                   'achieved_operands_from_hbm', 'frac_operands_from_hbm',
+                                                                   'kernel_ms_operands_from_hbm') if k in o_roof}}
                 all_exact = all_exact and o['bit_exact']
                 del o
             except Exception as exc:  # noqa: BLE001
