@@ -533,7 +533,7 @@ def prepare(wl, torch):
 KERNEL_FILE = {'whole graph (GEMM kernels dominate)': 'graph_executor'}
 
 
-def measure(torch, w, steps, warmup, eager=False):
+def measure(torch, w, steps, warmup, eager=False, cold_leg=True):
     """Times `steps` launches of a prepared workload; returns (ms per step, value in the workload's unit, roofline)."""
     ms_wall, ms_ev, graphed = _time_gpu(torch, w['fn'], steps, warmup, use_graph=not eager)
     ms = max(ms_wall, ms_ev)
@@ -549,7 +549,7 @@ def measure(torch, w, steps, warmup, eager=False):
                 'frac': round(achieved / PEAK_HBM_GBS, 4)}
     roof.update({'traffic': traffic, 'traffic_source': source, 'kernel': w['kernel'], 'kernel_ms': round(ms_ev, 5)})
     cold = w.get('fn_cold')
-    if cold is not None and w['bound'] == 'hbm' and steps * cold.bytes_per_launch >= COLD_RING_BYTES // 2:
+    if cold_leg and cold is not None and w['bound'] == 'hbm' and steps * cold.bytes_per_launch >= COLD_RING_BYTES // 2:
         # the same launches over a ring of operand copies four times the size of the memory-side cache: nothing is found there
         _, ms_cold, _ = _time_gpu(torch, cold, steps, warmup, use_graph=not eager)
         roof.update({'achieved_operands_from_hbm': round(work / (ms_cold * 1e-3) / 1e9, 2),
@@ -623,6 +623,8 @@ def main():
     ap.add_argument('--only', action='store_true', help='time the named workload alone (the default run of c2_dense '
                     'also times the other configurations and the matrix-core calibration loop)')
     ap.add_argument('--eager', action='store_true', help='time eager launches instead of a replayed HIP graph')
+    ap.add_argument('--one-buffer-set', action='store_true', help='skip the second timing of the HBM-bound workloads over a ring '
+                    'of operand copies (for a profiler run, whose kernel table should hold one kind of launch)')
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit('bench.py: this build runs on exactly one GPU (every operator is row-independent, so more GPUs '
@@ -650,7 +652,7 @@ def main():
         return
 
     w = prepare(wl, torch)
-    ms, value, roof, graphed = measure(torch, w, args.steps, args.warmup, args.eager)
+    ms, value, roof, graphed = measure(torch, w, args.steps, args.warmup, args.eager, not args.one_buffer_set)
     unit, samples, bit_exact = w['unit'], w['samples'], w['bit_exact']
 
     cpu = None
@@ -701,7 +703,7 @@ def main():
             torch.cuda.empty_cache()
             try:
                 o = prepare(name, torch)
-                o_ms, o_value, o_roof, _ = measure(torch, o, args.steps, args.warmup, args.eager)
+                o_ms, o_value, o_roof, _ = measure(torch, o, args.steps, args.warmup, args.eager, not args.one_buffer_set)
                 others[name] = {'value': float(f'{o_value:.6g}'), 'unit': o['unit'], 'ms_per_step': round(o_ms, 5),
                                 'bit_exact': o['bit_exact'], 'roofline': {k: o_roof[k] for k in ('bound', 'achieved', 'peak', 'unit', 'frac', 'traffic', 'traffic_source', 'kernel',
                                                                    'achieved_operands_from_hbm', 'frac_operands_from_hbm',
