@@ -275,6 +275,15 @@ __global__ __launch_bounds__(WS_NT, 1) void gemm_wrow_kernel(GemmArgs g, int pie
     // MFMA from the third MFMA on (its last MFMAs have left the pipe by then), and stored.
     // GEN: the column block takes the general requantisation, done right behind each row block, and its weight
     // fragments come from memory one K step at a time.
+    // GEN keeps no weights in registers: fragment (column group, K step) of MFMA Z is fetched WD MFMAs ahead into a ring
+    // (both row blocks of every piece of the column block take the same 2 * NKS fragments in the same order, so the
+    // ring runs on across pieces; fetched at the MFMA that uses it, every MFMA waited for its own load from L2)
+    constexpr int WD = 8;
+    typedef unsigned v4u_w __attribute__((ext_vector_type(4)));
+    v4u_w wq[WD];
+    auto fetch_gen_weight = [&](int Zm) WS_INLINE {  // Zm: MFMA number within a row block, 0 .. NM - 1
+        return __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, woff + ((Zm & 1) * NKS + (Zm >> 1)) * 1024, 0, 0);
+    };
     auto do_piece = [&](auto gen_tag, auto first_tag) WS_INLINE {
         constexpr bool GEN = decltype(gen_tag)::value;
         piece_sync(first_tag);
@@ -292,7 +301,8 @@ __global__ __launch_bounds__(WS_NT, 1) void gemm_wrow_kernel(GemmArgs g, int pie
             v4i a_op = af[F % AFS];
             if (A_UNSIGNED) a_op ^= static_cast<int>(0x80808080u);  // uint8 -> int8; 128 * colsum is in the start value
             if constexpr (GEN) {
-                const auto w = __builtin_amdgcn_raw_buffer_load_b128(rsrc_w, woff + (c * NKS + s) * 1024, 0, 0);
+                const v4u_w w = wq[Z % WD];
+                wq[Z % WD] = fetch_gen_weight((z + WD) % NM);
                 const v4i w_op = v4i{static_cast<int>(w[0]), static_cast<int>(w[1]), static_cast<int>(w[2]), static_cast<int>(w[3])};
                 if constexpr (s == 0) acc[i][c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w_op, a_op, v16i{}, 0, 0, 0);
                 else acc[i][c] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w_op, a_op, acc[i][c], 0, 0, 0);
@@ -352,6 +362,8 @@ __global__ __launch_bounds__(WS_NT, 1) void gemm_wrow_kernel(GemmArgs g, int pie
         if (general) {
             // no weights stay in registers here: the general requantisation needs the room
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int q = 0; q < WD; ++q) wq[q] = fetch_gen_weight(q);
             while (it < it_end) do_piece(std::true_type{}, std::false_type{});
         } else {
             load_column_registers();

@@ -151,6 +151,8 @@ class PackedDense:
     shift0: Optional[int] = None          # the shift as a host integer when there is one for every column
     wf: Optional[torch.Tensor] = None     # int8 weights in fragment order (short reductions: at pack time; else on
                                           # first use by dense_add_layernorm)
+    quick_shifts: bool = True             # every shift lies in 1..15: the requantisation that the kernel fed by `wf`
+                                          # overlaps with its matrix work covers exactly those
 
     @property
     def ldwt(self) -> int:
@@ -185,8 +187,8 @@ def pack_dense(weight: torch.Tensor, bias: Optional[torch.Tensor], shifts) -> Pa
     if int(sh.min()) < 0 or int(sh.max()) > top:
         raise ValueError(f'dense accumulator output shift must be in [0, {top}], got [{int(sh.min())}, {int(sh.max())}].')
     p = PackedDense(wt=wt, colsum=colsum, bias=bias, shifts=sh.to(weight.device), K=K, N=N, wt_lo=wt_lo,
-                    shift0=int(sh[0]) if sh.numel() == 1 else None)
-    if wt_lo is None and K <= 768 and K % 16 == 0:
+                    shift0=int(sh[0]) if sh.numel() == 1 else None, quick_shifts=bool(int(sh.min()) >= 1 and int(sh.max()) <= 15))
+    if wt_lo is None and K <= 768 and K % 16 == 0 and p.quick_shifts:
         _rowpack(p)  # the Dense kernel for short reductions fetches its weights in this order
     return p
 
@@ -262,8 +264,10 @@ def dense(x: torch.Tensor, p: PackedDense, rounding='floor', relu: bool = False,
         # of layers over 32 samples per wave does a chain of one at 3-5 TB/s (1 Mi x 16 -> 64: 23 us against 151 us)
         mlp(x2, [MlpLayerSpec(p, int(p.shift0), bool(relu), 'uint8' if ok == 1 else 'int8')], rounding, out=y2)
         return out
+    # A shift of 0 or above 15 sends a column block of the kernel that takes `wf` through its general requantisation, which
+    # keeps no weights in registers (8192 x 768 -> 3072: 50 us against 26 us); the kernel without `wf` does such layers in 33 us.
     check(_lib.load().a4g_dense_i8_wf(_ptr(x2), _TORCH_KIND[x2.dtype], 0, x2.stride(0) if M > 0 else p.K, _ptr(p.wt), p.ldwt,
-                                      _ptr(p.wf), _ptr(p.colsum), _ptr(p.bias), _ptr(p.shifts), int(p.shifts.numel()),
+                                      _ptr(p.wf if p.quick_shifts else None), _ptr(p.colsum), _ptr(p.bias), _ptr(p.shifts), int(p.shifts.numel()),
                                       _mode(rounding), int(bool(relu)), ok, _ptr(y2), y2.stride(0) if M > 0 else p.N, M, p.N,
                                       p.K, _stream()))
     return out

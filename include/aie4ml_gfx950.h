@@ -123,7 +123,10 @@ A4G_API int a4g_dense_i8(const void* A, int a_kind, int trans_a, int64_t lda, co
  *   Wf      a4g_rowpack_weights_i8 applied to Wt (a4g_rowpacked_bytes(N, K) bytes, 16-byte aligned), or NULL
  * With Wf, reductions of up to 768 with 16-byte aligned rows on both sides take a kernel that keeps a column block's
  * weights in registers and fetches them with whole-line loads (csrc/gemm_wrow.hip); every other shape, and a NULL Wf,
- * runs exactly as a4g_dense_i8. */
+ * runs exactly as a4g_dense_i8. That kernel overlaps the requantisation with its matrix work where a block of 256
+ * columns has every shift in 1..15 and every bias + 128 * colsum within +-2^30; other blocks take a form that refetches
+ * the weights per row block and runs at about half the rate, below that of a4g_dense_i8: a caller that knows a layer's
+ * shifts to lie outside 1..15 passes NULL. */
 A4G_API int a4g_dense_i8_wf(const void* A, int a_kind, int trans_a, int64_t lda, const int8_t* Wt, int64_t ldwt,
                     const int8_t* Wf, const int32_t* colsum, const int32_t* bias, const int32_t* shifts, int n_shift,
                     int round_mode, int relu, int out_kind, void* Y, int64_t ldy, int64_t M, int64_t N,

@@ -329,13 +329,23 @@ def test_dense_short_reduction_with_and_without_fragment_order_weights(ops, orac
             bias[540], bias[541] = 2**31 - 5, -2**31 + 7
         bias = bias.astype(np.int32)
         p = ops.pack_dense(dev(W), dev(bias), shifts)
-        assert p.wf is not None
+        # a layer with a shift outside 1..15 is packed without the fragment-order copy (the other kernel does its general
+        # requantisation faster); the copy is made here and forced on the call, which is what a C caller may do
+        assert p.wf is None and not p.quick_shifts
+        from aie4ml_amd.ops import _rowpack
+        _rowpack(p)
+        forced = dataclasses.replace(p, quick_shifts=True)
         exp = oracle.dense(A, W, bias, shifts, mode, relu=False, out='int8')
-        got = host(ops.dense(dev(A), p, mode, relu=False, out_kind='int8'))
+        got = host(ops.dense(dev(A), forced, mode, relu=False, out_kind='int8'))
         assert np.array_equal(got, exp), (M, K, N, np.argwhere(got != exp)[:5])
-        plain = dataclasses.replace(p, wf=None)
-        got = host(ops.dense(dev(A), plain, mode, relu=False, out_kind='int8'))
+        got = host(ops.dense(dev(A), p, mode, relu=False, out_kind='int8'))
         assert np.array_equal(got, exp), ('row-major weights', M, K, N, np.argwhere(got != exp)[:5])
+    # shifts within 1..15: the copy is made at pack time and used
+    shifts = r.integers(1, 16, 1024).astype(np.int32)
+    W, A = gauss8(r, 30, (256, 1024)), gauss8(r, 40, (300, 256))
+    p = ops.pack_dense(dev(W), None, shifts)
+    assert p.wf is not None and p.quick_shifts
+    assert np.array_equal(host(ops.dense(dev(A), p, 'conv_even', out_kind='int8')), oracle.dense(A, W, None, shifts, 'conv_even', out='int8'))
 
 
 # Longer reductions on at most 256 tiles of 128 x 192 take the kernel that splits the reduction inside the workgroup.
