@@ -4,7 +4,7 @@
 //
 //   acc_t                        16 accumulators of one 32 x 32 block (v16i or v16f)
 //   MMAS                         MFMA instructions issued per pair of fragments
-//   FIX_A, fix_a(v4i&)           optional fix-up of an A fragment before use
+//   FIX_A, fix_a(v4i&)           optional fix-up of a 16-byte chunk of A before it is staged
 //   mma(b, a, acc)               acc += the 32 x 32 block product of two fragments
 //   KSTEP_BYTES                  bytes of K one mma() call consumes per operand row: 32 (one 16-byte fragment per lane)
 //                                or 64 (two fragments per lane; the K tile then has two steps instead of four)
@@ -288,6 +288,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
             if (idx < Cfg::A_LOADS && (idx & 1) == 0)
                 P::split_a(ra[idx], ra[idx + 1 < Cfg::A_LOADS ? idx + 1 : idx], extra, idx >> 1, split_live);
         }
+        // the operand fix-up (uint8 -> int8) is made here, once per staged chunk: at the fragments every chunk would be
+        // fixed again by each of the WAVES_N waves that read it
+        if (P::FIX_A && idx < Cfg::A_LOADS) P::fix_a(ra[idx]);
         if (idx < Cfg::A_LOADS) *reinterpret_cast<v4i*>(stage + st_off + idx * Cfg::ROWS_PER_PASS * BK) = ra[idx];
         else *reinterpret_cast<v4i*>(stage + BM * BK + st_off + (idx - Cfg::A_LOADS) * Cfg::ROWS_PER_PASS * BK) = rb[idx - Cfg::A_LOADS];
     };
@@ -352,10 +355,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
 #pragma unroll
         for (int m = 0; m < NM; ++m) {
             const int i = m / Cfg::TN, j = m % Cfg::TN;
-            if (P::FIX_A && j == 0) {
-#pragma unroll
-                for (int f = 0; f < FR; ++f) P::fix_a(af[cur][i][f]);
-            }
             // operands swapped: the block's first index (registers) runs over n, lanes over m
             acc[i][j] = P::mma(bf[cur][j], af[cur][i], acc[i][j]);
             if (m < NR) read_one(nxt, next_base, next_kk, m);
@@ -367,11 +366,11 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
         }
 #pragma unroll
         for (int m = 0; m < NM; ++m) {
-            if (P::FIX_A && m % Cfg::TN == 0) __builtin_amdgcn_sched_group_barrier(0x002, 4 * FR, 0);  // operand fix-up
             __builtin_amdgcn_sched_group_barrier(0x008, P::MMAS, 0);                              // one fragment pair
             if (m < NR) __builtin_amdgcn_sched_group_barrier(0x100, FR, 0);                         // one fragment's LDS reads
 #pragma unroll
             for (int e = m * Cfg::EPM; e < (m + 1) * Cfg::EPM && e < Cfg::LOADS; ++e) {
+                if (P::FIX_A && (EXTRA == 1 || EXTRA == 3) && e < Cfg::A_LOADS) __builtin_amdgcn_sched_group_barrier(0x002, 4, 0);  // its fix-up
                 if (EXTRA == 1 || EXTRA == 3) __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // one LDS write
                 if (EXTRA == 2 || EXTRA == 3) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // one global load
             }
