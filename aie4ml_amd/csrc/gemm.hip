@@ -1023,8 +1023,9 @@ static int matmul_i8_impl(const char* who, bool own_scratch, const void* A, int 
     A4G_REQUIRE(A && B && C, A4G_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
 
     // the two attention shapes have kernels of their own that need neither workspace nor K-loop barriers
-    if (out_kind != A4G_I16 && env_variant() == 0 && !trans_a) {
-        LeanArgs la{};
+    LeanArgs la{};
+    const bool lean_shape = out_kind != A4G_I16 && env_variant() == 0 && !trans_a;
+    if (lean_shape) {
         la.A = static_cast<const int8_t*>(A);
         la.B = B;
         la.C = static_cast<int8_t*>(C);
@@ -1107,6 +1108,12 @@ static int matmul_i8_impl(const char* who, bool own_scratch, const void* A, int 
         g.Bt = ws;
         g.ldb = ldt;
         g.stride_b = N * ldt;
+        if (lean_shape) {  // a short reduction against a wide right operand given as [K][N]: its transpose takes the lean kernel
+            la.B = ws;
+            la.ldb = ldt;
+            la.stride_b = N * ldt;
+            if (lean_nt_applicable(la)) return check_hip(launch_lean_nt(la, stream), who);
+        }
         e = trans_a ? launch_trans_a(g, static_cast<int>(batch), stream)
             : a_ok  ? launch_aligned()
                     : launch_ragged(g, static_cast<int>(batch), stream);
