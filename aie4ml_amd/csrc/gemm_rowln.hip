@@ -53,6 +53,7 @@ struct RowLnArgs {
     int lo, hi;
     int log2c, eps_q0, ln_mode, gamma_shift, final_shift;
     LnFloat lf;
+    FastRound ln_rg, ln_ro;  // the integer form's two roundings (inv * gamma, then vd * fscale + beta) as data: one path for all modes
 };
 
 // FR: the float form of the normalisation (0 nearest even, 1 floor family, 2 ceil family), -1: integer form only.
@@ -311,8 +312,10 @@ __global__ __launch_bounds__(RL_NT, 2) void gemm_rowln_kernel(RowLnArgs g) {
 #pragma unroll
                     for (int t = 0; t < 4; ++t) {
                         const int vd = sext8(sword, t) - st.mu;
-                        const int fs = clamp_i(round_shift_rt(st.inv * g4[t], g.gamma_shift, g.ln_mode), -32768, 32767);
-                        y4[t] = clamp_i(round_shift_rt(vd * fs + b4[t], g.final_shift, g.ln_mode), -128, 127);
+                        // inv * gamma < 2^30 and |vd * fscale + beta| < 2^24: the short form of the rounding applies (the
+                        // switch over the eight modes per element cost 10 us of the launch's 24)
+                        const int fs = clamp_i(fast_round(st.inv * g4[t], g.ln_rg), -32768, 32767);
+                        y4[t] = clamp_i(fast_round(vd * fs + b4[t], g.ln_ro), -128, 127);
                     }
                     o[q] = static_cast<int>(pack4_bytes(y4[0], y4[1], y4[2], y4[3]));
                 }
@@ -454,6 +457,8 @@ extern "C" int a4g_dense_add_layernorm_i8(const void* A, int a_kind, int64_t lda
     g.final_shift = 15 - out_shift;
     int fr = -1;
     g.lf = make_ln_float(ln_round_mode, gamma_shift, g.final_shift, &fr);
+    g.ln_rg = make_fast_round(ln_round_mode, gamma_shift);
+    g.ln_ro = make_fast_round(ln_round_mode, g.final_shift);
 
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     // 64 rows per workgroup halve the weight traffic and double the epilogue's arithmetic per CU: taken when the

@@ -279,7 +279,7 @@ class GPUModel:
         x = values[input_tensor_for_role(d_inst.node, 'lhs').name]
         packed = d_inst.artifacts['packed_weights']
         rows = x.numel() // int(x.shape[-1]) if x.numel() else 0
-        if ops.dense_add_layernorm_applicable(x, packed) and ops.dense_add_layernorm_pays(rows, packed, cfg.rounding_mode):
+        if ops.dense_add_layernorm_applicable(x, packed) and ops.dense_add_layernorm_pays(rows, packed):
             values[ln_inst.node.outputs[0].name] = ops.dense_add_layernorm(
                 x, packed, values[info['residual']], ln_inst.artifacts['packed_gamma'], ln_inst.artifacts['packed_beta'],
                 cfg.out_shift, dense_rounding=dcfg.rounding_mode, relu=dcfg.flags.use_relu, rounding=cfg.rounding_mode,

@@ -393,21 +393,16 @@ def dense_add_layernorm_applicable(x: torch.Tensor, p: PackedDense) -> bool:
             and x.dtype in (torch.int8, torch.uint8) and x.dim() >= 1 and int(x.shape[-1]) == p.K)
 
 
-# rounding modes whose LayerNorm normalisation has a float form in the kernels (the others restate the integer recipe)
-_LN_FLOAT_FORM_MODES = frozenset(ROUNDING[m] for m in ('floor', 'ceil', 'positive_inf', 'negative_inf', 'conv_even'))
-
-
-def dense_add_layernorm_pays(rows: int, p: PackedDense, rounding='conv_even') -> bool:
+def dense_add_layernorm_pays(rows: int, p: PackedDense) -> bool:
     """Whether the one-launch form is the faster one. Every workgroup of that kernel streams the whole weight matrix,
     one per 32 rows, and a single round of workgroups has nothing to hide its first loads and its normalisation behind;
     measured against dense() + add_layernorm() at 768 outputs: 768 inputs 12.2 / 14.1 / 23.1 us against 14.2 / 19.6 /
     28.7 us at 4096 / 8192 / 16384 rows, but 11.6 against 11.3 us at 2048 rows and 45.4 against 46.3 us at 32768;
     1024 inputs 16.1 against 22.1 us, 1536 inputs 20.2 against 25.2 us, 2048 inputs 26.1 against 27.9 us, 3072 inputs
     35.2 against 34.2 us (8192 rows); 512 -> 512: 11.0 against 13.7 us; 256 outputs (one 32-column block per wave) 8.8
-    against 10.0 us at 8192 rows, 26.5 against 17.7 us at 32768. ``rounding`` is the LayerNorm's: the three modes whose
-    normalisation has no float form (symmetric_inf, symmetric_zero, conv_odd) take 24-25 us in the one-launch form at
-    8192 x 768 -> 768 where the two launches take 19."""
-    return 4096 <= rows <= 16384 and p.K <= 1536 and p.N >= 384 and _mode(rounding) in _LN_FLOAT_FORM_MODES
+    against 10.0 us at 8192 rows, 26.5 against 17.7 us at 32768. The LayerNorm's rounding mode does not matter: 13.3-14.9 us for
+    every pair of modes at 8192 x 768 -> 768 against 17.7-19.0 us for the two launches."""
+    return 4096 <= rows <= 16384 and p.K <= 1536 and p.N >= 384
 
 
 def dense_add_layernorm(x: torch.Tensor, p: PackedDense, residual: Optional[torch.Tensor], gamma_q7: torch.Tensor,
