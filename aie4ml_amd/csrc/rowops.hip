@@ -411,7 +411,8 @@ __global__ __launch_bounds__(256, 2) void layernorm_rows_kernel(const int8_t* __
                 put(rsrc_out, o, row, i);
             }
             };
-            if (!AS_FLOAT || __builtin_amdgcn_ballot_w64(may_clip) != 0) normalise(std::true_type{});
+            // (rows of sixteen chunks keep the one copy with the clamp: two copies of the loop cost them 42 spilled registers)
+            if (!AS_FLOAT || NCH > 8 || __builtin_amdgcn_ballot_w64(may_clip) != 0) normalise(std::true_type{});
             else normalise(std::false_type{});
         }
     };
