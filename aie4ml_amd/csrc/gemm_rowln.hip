@@ -464,7 +464,9 @@ extern "C" int a4g_dense_add_layernorm_i8(const void* A, int a_kind, int64_t lda
     // 64 rows per workgroup halve the weight traffic and double the epilogue's arithmetic per CU: taken when the
     // activations fit LDS and there are still enough workgroups for every CU (with 8192 rows, 128 workgroups of 64 rows
     // measured 20.9 us against 16.2 us for 256 of 32)
-    const bool two = K <= RL_MAX_K2 && (M + 63) / 64 >= 256;
+    // ... and also as soon as workgroups of 32 rows would need a second round on 256 CUs: 9216 / 12 288 rows measured
+    // 23.3 / 24.2 us in two rounds of 32-row workgroups
+    const bool two = K <= RL_MAX_K2 && (M + 31) / 32 > 256;
     const hipError_t e = two ? launch_rowln_rb<2>(g, fr, stream) : launch_rowln_rb<1>(g, fr, stream);
     return check_hip(e, who);
 }

@@ -884,7 +884,9 @@ def run_dense_add_layernorm(ops, oracle, M, K, N, seed, dmode='conv_even', lmode
 
 
 @pytest.mark.parametrize('case', [(1, 128, 32), (31, 128, 768), (33, 256, 256), (100, 768, 768), (64, 384, 512),
-                                  (257, 512, 384), (96, 640, 160), (40, 3072, 768), (700, 1024, 64), (65, 4096, 96)])
+                                  (257, 512, 384), (96, 640, 160), (40, 3072, 768), (700, 1024, 64), (65, 4096, 96),
+                                  # more than 256 workgroups of 32 rows: workgroups of 64 rows, the last one ragged
+                                  (8200, 256, 128), (16390, 128, 64), (9216, 768, 768)])
 def test_dense_add_layernorm_shapes(ops, oracle, case):
     M, K, N = case
     run_dense_add_layernorm(ops, oracle, M, K, N, seed=sum(case))
