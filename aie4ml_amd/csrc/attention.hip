@@ -62,9 +62,9 @@ __device__ __forceinline__ void transpose4x4(const unsigned a[4], unsigned c[4])
 // (d << 8) | (c << 2) built by one v_perm): with a single copy, lanes that gather different gaps from one bank
 // serialise, and those conflicts were two thirds of this kernel's LDS cycles.
 template <int NT, int DT, int BIT, bool FASTP, int NW = 4, bool RAGGED = false>
-__global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(AttnArgs a) {
+__global__ __launch_bounds__(NW * 64, (NW == 8 || NW == 6) ? 1 : 2) void attention_kernel(AttnArgs a) {
     constexpr int SK = NT * 32, D = DT * 32, PITCH = SK + 16;
-    constexpr bool BANKED = NW == 8;
+    constexpr bool BANKED = NW == 8 || NW == 6;  // 6: the same form on 192 query rows (384 queries are two such blocks)
     constexpr int THREADS = NW * 64, ROWS = NW * 32;
     // The score table is a static array: its LDS address is then a compile-time constant that folds into the
     // offset field of the gathers (an array inside the dynamic block costs one address add per gather).
@@ -428,21 +428,22 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attention_kernel(Att
 
 constexpr int ATTN_CUS = 256;
 
-template <int NT, int DT, int BIT, bool FASTP>
+template <int NT, int DT, int BIT, bool FASTP, int NW = 8>
 static void launch_attention_wide(int grid8, size_t lds, hipStream_t stream, const AttnArgs& a) {
-    auto kern = attention_kernel<NT, DT, BIT, FASTP, 8>;
+    auto kern = attention_kernel<NT, DT, BIT, FASTP, NW>;
     static bool attr_set = false;  // benign race: the attribute is idempotent
     if (!attr_set) {
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
                                   static_cast<int>(lds));
         attr_set = true;
     }
-    kern<<<std::min(grid8, ATTN_CUS), 512, lds, stream>>>(a);  // persistent: at most one workgroup per CU
+    kern<<<std::min(grid8, ATTN_CUS), NW * 64, lds, stream>>>(a);  // persistent: at most one workgroup per CU
 }
 
-// grid: workgroups of 128 query rows; grid8: workgroups of 256 (0 = do not use the eight-wave form).
+// grid: workgroups of 128 query rows; grid8: workgroups of 256 (0 = do not use the eight-wave form), or, when
+// `six`, of 192 in the six-wave form.
 template <int NT, int DT>
-static void launch_attention_nt(int grid, int grid8, size_t lds, hipStream_t stream, const AttnArgs& a) {
+static void launch_attention_nt(int grid, int grid8, size_t lds, hipStream_t stream, const AttnArgs& a, bool six = false) {
     const bool fastp = a.noclamp && a.sm.out_shift <= 16;
     const bool ragged = a.sk != NT * 32;  // always in workgroups of four waves (grid8 == 0)
 #define A4G_ATTN(B)                                                                  \
@@ -451,7 +452,10 @@ static void launch_attention_nt(int grid, int grid8, size_t lds, hipStream_t str
         else attention_kernel<NT, DT, B, false, 4, true><<<grid, 256, lds, stream>>>(a);        \
     } else if (NT >= 8 && DT == 2 && grid8 > 0) {                                           \
         if constexpr (NT >= 8 && DT == 2) {                                                     \
-            if (fastp) launch_attention_wide<NT, DT, B, true>(grid8, lds, stream, a); \
+            if (six) {                                                                          \
+                if (fastp) launch_attention_wide<NT, DT, B, true, 6>(grid8, lds, stream, a);    \
+                else launch_attention_wide<NT, DT, B, false, 6>(grid8, lds, stream, a);         \
+            } else if (fastp) launch_attention_wide<NT, DT, B, true>(grid8, lds, stream, a); \
             else launch_attention_wide<NT, DT, B, false>(grid8, lds, stream, a);      \
         }                                                                            \
     } else if (fastp)                                                                \
@@ -484,14 +488,14 @@ static void launch_attention_seven(int grid, hipStream_t stream, const AttnArgs&
 }
 
 template <int DT>
-static int launch_attention(int nt, int grid, int grid8, hipStream_t stream, const AttnArgs& a) {
+static int launch_attention(int nt, int grid, int grid8, hipStream_t stream, const AttnArgs& a, bool six = false) {
     size_t lds = static_cast<size_t>(DT * 32) * (nt * 32 + 16) + DT * 32 * 4;  // V^T + column sums
     if (nt >= 16 && grid8 > 0) lds += 3 * 8 * 512 * sizeof(unsigned);            // + three parked score tiles per thread
     switch (nt) {
     case 1: launch_attention_nt<1, DT>(grid, 0, lds, stream, a); break;
     case 2: launch_attention_nt<2, DT>(grid, 0, lds, stream, a); break;
     case 4: launch_attention_nt<4, DT>(grid, 0, lds, stream, a); break;
-    case 8: launch_attention_nt<8, DT>(grid, grid8, lds, stream, a); break;
+    case 8: launch_attention_nt<8, DT>(grid, grid8, lds, stream, a, six); break;
     // tile counts between the powers of two, for the 64-wide heads only (96, 160, 192 and 384 keys: a kernel of the next
     // power of two would spend a quarter to three eighths of its three passes on keys that do not exist)
     case 3:
@@ -507,11 +511,11 @@ static int launch_attention(int nt, int grid, int grid8, hipStream_t stream, con
         else return 1;
         break;
     case 12:
-        if constexpr (DT == 2) launch_attention_nt<12, DT>(grid, grid8, lds, stream, a);
+        if constexpr (DT == 2) launch_attention_nt<12, DT>(grid, grid8, lds, stream, a, six);
         else return 1;
         break;
     case 16:
-        if constexpr (DT <= 2) launch_attention_nt<16, DT>(grid, grid8, lds, stream, a);
+        if constexpr (DT <= 2) launch_attention_nt<16, DT>(grid, grid8, lds, stream, a, six);
         else return 1;
         break;
     default: return 1;
@@ -590,7 +594,12 @@ extern "C" int a4g_attention_i8(const int8_t* Q, const int8_t* K, const int8_t* 
     const int grid = static_cast<int>(batch * heads * ((sq + 127) / 128));
     // eight waves per workgroup (256 query rows, bank-replicated score table) once every CU gets at least one
     const int64_t wg8 = batch * heads * ((sq + 255) / 256);
-    const int grid8 = (!ragged && d == 64 && sq >= 256 && wg8 >= 256) ? static_cast<int>(wg8) : 0;
+    int grid8 = (!ragged && d == 64 && sq >= 256 && wg8 >= 256) ? static_cast<int>(wg8) : 0;
+    // blocks of 192 rows where they leave fewer rows empty than blocks of 256 (384 queries: two full blocks against one
+    // full and one half)
+    const int64_t wg6 = batch * heads * ((sq + 191) / 192);
+    const bool six = grid8 > 0 && wg6 >= 256 && (sq + 191) / 192 * 192 < (sq + 255) / 256 * 256;
+    if (six) grid8 = static_cast<int>(wg6);
     a.items = grid8 > 0 ? grid8 : grid;
     if (d == 64 && sq > 192 && sq <= 224 && sk > 192 && sk <= 224) {
         // 193 .. 224 queries and keys (the 197 tokens of a vision transformer): seven key tiles instead of eight, and one
@@ -599,7 +608,7 @@ extern "C" int a4g_attention_i8(const int8_t* Q, const int8_t* K, const int8_t* 
         launch_attention_seven(a.items, stream, a);
         return check_hip(hipGetLastError(), who);
     }
-    const int no_kernel = width == 64 ? launch_attention<2>(nt, grid, grid8, stream, a)
+    const int no_kernel = width == 64 ? launch_attention<2>(nt, grid, grid8, stream, a, six)
                           : (width == 32 ? launch_attention<1>(nt, grid, 0, stream, a) : launch_attention<4>(nt, grid, 0, stream, a));
     if (no_kernel) return fail(A4G_ERR_UNSUPPORTED, "%s: no kernel for sk=%lld", who, (long long)sk);
     return check_hip(hipGetLastError(), who);
