@@ -856,20 +856,16 @@ static hipError_t launch_gemm_nt(const GemmArgs& g, int batch, hipStream_t strea
         if (k128) return g.a_unsigned ? launch_rs_u<256, 256, 2, 4, true, true>(g, batch, stream)
                                       : launch_rs_u<256, 256, 2, 4, false, true>(g, batch, stream);
         if (k64) return launch_dtl<256, 256, 64, 2, 4, 4>(g, batch, stream);
-        {  // K in whole 16-byte chunks but not whole tiles: the pipelined kernel with a masked last tile
-            GemmArgs r = g;
-            r.ragged_a = r.ragged_b = 0;
-            return g.a_unsigned ? launch_rs_policy<I8Policy<true>, 256, 256, 2, 4, true, true>(r, batch, stream)
-                                : launch_rs_policy<I8Policy<false>, 256, 256, 2, 4, true, true>(r, batch, stream);
-        }
+        // K in whole 16-byte chunks but not whole tiles: the pipelined kernel with the last tile's missing chunks
+        // fetched from outside the operands' descriptors
+        return g.a_unsigned ? launch_rs_policy<I8Policy<true>, 256, 256, 2, 4, true, false, true>(g, batch, stream)
+                            : launch_rs_policy<I8Policy<false>, 256, 256, 2, 4, true, false, true>(g, batch, stream);
     case 2:  // 128 x 128
         if (k128) return launch_rs<128, 128, 2, 2>(g, batch, stream);
         if (k64) return launch_dtl<128, 128, 64, 2, 2, 4>(g, batch, stream);
-        if (g.K >= 256) {  // K in whole 16-byte chunks but not whole tiles: the pipelined kernel with a masked last tile
-            GemmArgs r = g;
-            r.ragged_a = r.ragged_b = 0;
-            return g.a_unsigned ? launch_rs_policy<I8Policy<true>, 128, 128, 2, 2, false, true>(r, batch, stream)
-                                : launch_rs_policy<I8Policy<false>, 128, 128, 2, 2, false, true>(r, batch, stream);
+        if (g.K >= 256) {  // K in whole 16-byte chunks but not whole tiles: as above
+            return g.a_unsigned ? launch_rs_policy<I8Policy<true>, 128, 128, 2, 2, false, false, true>(g, batch, stream)
+                                : launch_rs_policy<I8Policy<false>, 128, 128, 2, 2, false, false, true>(g, batch, stream);
         }
         return launch_tiled<128, 128, 64, 2, 2>(g, batch, stream);
     case 4:  // 128 x 192

@@ -195,8 +195,13 @@ static inline int ragged_mode(const void* p, int64_t ld, int64_t stride, int64_t
     return 2;
 }
 
-template <class P, int BM, int BN, int WAVES_M, int WAVES_N, bool EARLY = false, bool RAGGED = false>
+// RAGGED: K need not fill its last tile and rows need not be aligned (chunk loads that respect the row ends).
+// KTAIL: aligned rows, K in whole 16-byte chunks but not whole tiles: the aligned form's descriptor loads, with the
+// chunks past K sent to an offset outside the descriptor (they read as zero) - no load sits in a branch, so the waits
+// stay exact, which the ragged loads' branches do not allow (8192 x 784 -> 128: 17 us ragged, 9 us this way).
+template <class P, int BM, int BN, int WAVES_M, int WAVES_N, bool EARLY = false, bool RAGGED = false, bool KTAIL = false>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs g) {
+    static_assert(!KTAIL || (!RAGGED && !P::SPLIT_A && !P::SPLIT_B), "the K tail form serves the unsplit policies");
     using Cfg = RsCfg<P, BM, BN, WAVES_M, WAVES_N>;
     constexpr int BK = Cfg::BK, KSTEPS = Cfg::KSTEPS;
     extern __shared__ __attribute__((aligned(16))) int8_t smem[];
@@ -245,8 +250,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
     // policies, short of registers, reloaded address pairs from scratch inside the loop, each reload waiting for every
     // load in flight.
     constexpr int A_TILE_BYTES = P::SPLIT_A ? 2 * BK : BK;
-    const int64_t a_range = static_cast<int64_t>(g.M - 1 - m0) * g.lda + static_cast<int64_t>(g.K / BK) * A_TILE_BYTES;
-    const int64_t b_range = static_cast<int64_t>(g.N - 1 - n0) * g.ldb + static_cast<int64_t>(g.K / BK) * BK;
+    const int64_t a_range = static_cast<int64_t>(g.M - 1 - m0) * g.lda + (KTAIL ? g.K : static_cast<int64_t>(g.K / BK) * A_TILE_BYTES);
+    const int64_t b_range = static_cast<int64_t>(g.N - 1 - n0) * g.ldb + (KTAIL ? g.K : static_cast<int64_t>(g.K / BK) * BK);
     const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<int8_t*>(Abase), 0, static_cast<int>(a_range < 0x7fffffff ? a_range : 0x7fffffff), 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrc_b =
@@ -255,6 +260,18 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
     const int voff_a = lrow * static_cast<int>(g.lda) + lchunk * (P::SPLIT_A ? 32 : 16);
     const int voff_b = lrow * static_cast<int>(g.ldb) + lchunk * 16;
     auto load_one = [&](int kt, int idx) {
+        if constexpr (KTAIL) {
+            constexpr unsigned NOWHERE = 0xfffffff0u;  // beyond every descriptor: reads as zero
+            const bool inside = kt * BK + lchunk * 16 < g.K;
+            if (idx < Cfg::A_LOADS) {
+                const unsigned off = voff_a + kt * BK + idx * Cfg::ROWS_PER_PASS * static_cast<int>(g.lda);
+                ra[idx] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, inside ? off : NOWHERE, 0, 0));
+            } else {
+                const unsigned off = voff_b + kt * BK + (idx - Cfg::A_LOADS) * Cfg::ROWS_PER_PASS * static_cast<int>(g.ldb);
+                rb[idx - Cfg::A_LOADS] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, inside ? off : NOWHERE, 0, 0));
+            }
+            return;
+        }
         if constexpr (RAGGED) {
             // K (bytes here) need not fill its last tile and rows need not be aligned: bytes past K read as zero
             static_assert(!RAGGED || (!P::SPLIT_A && !P::SPLIT_B), "the ragged loads serve the unsplit policies");
@@ -295,7 +312,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
         else *reinterpret_cast<v4i*>(stage + BM * BK + st_off + (idx - Cfg::A_LOADS) * Cfg::ROWS_PER_PASS * BK) = rb[idx - Cfg::A_LOADS];
     };
 
-    const int ktiles = RAGGED ? (g.K + BK - 1) / BK : g.K / BK;
+    const int ktiles = (RAGGED || KTAIL) ? (g.K + BK - 1) / BK : g.K / BK;
 #pragma unroll
     for (int i = 0; i < Cfg::LOADS; ++i) load_one(0, i);
 
@@ -440,10 +457,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
 }
 
 // Launches one workgroup per tile (padded to whole ranges for the 8 XCDs; surplus workgroups exit at once).
-template <class P, int BM, int BN, int WAVES_M, int WAVES_N, bool EARLY = false, bool RAGGED = false>
+template <class P, int BM, int BN, int WAVES_M, int WAVES_N, bool EARLY = false, bool RAGGED = false, bool KTAIL = false>
 static hipError_t launch_rs_policy(const GemmArgs& g, int batch, hipStream_t stream) {
     using Cfg = RsCfg<P, BM, BN, WAVES_M, WAVES_N>;
-    auto kern = gemm_rs_kernel<P, BM, BN, WAVES_M, WAVES_N, EARLY, RAGGED>;
+    auto kern = gemm_rs_kernel<P, BM, BN, WAVES_M, WAVES_N, EARLY, RAGGED, KTAIL>;
     static bool attr_set = false;  // benign race: the attribute is idempotent
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,

@@ -666,6 +666,29 @@ def test_dense_ragged_reduction_and_unaligned_rows(ops, oracle, kind, case):
         assert np.array_equal(got, oracle.dense(A, W, bias, shifts, mode, relu=relu, out=out)), (mode, relu)
 
 
+@pytest.mark.parametrize('case', [(300, 200, 784, 16), (1, 128, 784, 0), (1000, 130, 800, 240), (700, 520, 272, 112),
+                                  (4096, 4096, 1040, 0), (4100, 4096, 528, 16)])
+@pytest.mark.parametrize('a_dtype', [np.int8, np.uint8])
+def test_dense_reduction_in_whole_chunks_but_not_whole_tiles(ops, oracle, case, a_dtype):
+    """Aligned rows, K a multiple of 16 but not of 128, from two K tiles on (a 784-input classifier): the pipelined
+    kernel fetches the last tile's missing chunks from outside the operands' descriptors. What lies behind K in a row
+    (the rest of a wider matrix, extreme values) and behind the last row must count as zero; 128 x 128 and 256 x 256 tiles."""
+    M, N, K, extra = case
+    r = rng(M + N + K)
+    info = np.iinfo(a_dtype)
+    wide = np.full((M, K + extra), info.max, dtype=a_dtype)
+    A = r.integers(info.min, info.max + 1, (M, K)).astype(a_dtype)
+    wide[:, :K] = A
+    W = gauss8(r, 40, (K, N))
+    bias = r.integers(-2**15, 2**15, N).astype(np.int32)
+    shifts = r.integers(7, 13, N).astype(np.int32)
+    p = ops.pack_dense(dev(W), dev(bias), shifts)
+    x = dev(wide)[:, :K]
+    for mode, relu in (('conv_even', True), ('symmetric_inf', False)):
+        got = host(ops.dense(x, p, mode, relu=relu, out_kind='int8'))
+        assert np.array_equal(got, oracle.dense(A, W, bias, shifts, mode, relu=relu, out='int8')), (mode, relu)
+
+
 @pytest.mark.parametrize('trans_b', [True, False])
 @pytest.mark.parametrize('a_dtype,b_dtype', [(np.int8, np.int8), (np.uint8, np.int8), (np.int16, np.int8), (np.int16, np.int16)])
 @pytest.mark.parametrize('shape', [((2,), 130, 70, 100), ((3,), 64, 129, 37), ((), 257, 200, 1001), ((2, 2), 33, 17, 7)])
