@@ -271,6 +271,13 @@ static hipError_t launch_float_nt(const void* A, int trans_a, int64_t lda, int64
         g.ragged_a = ragged_mode(g.A, g.lda, g.stride_a, g.K);
         g.ragged_b = ragged_mode(g.Bt, g.ldb, g.stride_b, g.K);
         g.trans_a_es = trans_a ? es : 0;  // A stored transposed: its chunks are gathered element by element
+        if (!trans_a && g.K >= 256 && g.ragged_a <= 1 && g.ragged_b == 0 && g.lda >= (g.K + 3) / 4 * 4) {
+            // 4-byte aligned activation rows, 16-byte aligned rows of the other operand that hold K rounded up to 16: the
+            // descriptor loads without branches (K off the 16-byte grid; the bytes past K are cleared at the staging)
+            if (fmt == A4G_F32) return launch_rs_policy<FloatPolicy<A4G_F32>, 128, 128, 2, 2, false, false, 2>(g, batch, stream);
+            if (fmt == A4G_FP8) return launch_rs_policy<FloatPolicy<A4G_FP8>, 128, 128, 2, 2, false, false, 2>(g, batch, stream);
+            return launch_rs_policy<FloatPolicy<A4G_BF16>, 128, 128, 2, 2, false, false, 2>(g, batch, stream);
+        }
         if (fmt == A4G_F32) return launch_rs_policy<FloatPolicy<A4G_F32>, 128, 128, 2, 2, false, true>(g, batch, stream);
         if (fmt == A4G_FP8) return launch_rs_policy<FloatPolicy<A4G_FP8>, 128, 128, 2, 2, false, true>(g, batch, stream);
         return launch_rs_policy<FloatPolicy<A4G_BF16>, 128, 128, 2, 2, false, true>(g, batch, stream);

@@ -199,9 +199,12 @@ static inline int ragged_mode(const void* p, int64_t ld, int64_t stride, int64_t
 // KTAIL: aligned rows, K in whole 16-byte chunks but not whole tiles: the aligned form's descriptor loads, with the
 // chunks past K sent to an offset outside the descriptor (they read as zero) - no load sits in a branch, so the waits
 // stay exact, which the ragged loads' branches do not allow (8192 x 784 -> 128: 17 us ragged, 9 us this way).
-template <class P, int BM, int BN, int WAVES_M, int WAVES_N, bool EARLY = false, bool RAGGED = false, bool KTAIL = false>
+// KTAIL 2: the same for K off the 16-byte grid: rows of A 4-byte aligned (four dword loads per chunk, each inside K or
+// sent outside the descriptor), rows of B 16-byte aligned with a pitch that holds K rounded up to 16; the bytes past K
+// of the one dword or chunk that straddles it are cleared where the last K tile is staged.
+template <class P, int BM, int BN, int WAVES_M, int WAVES_N, bool EARLY = false, bool RAGGED = false, int KTAIL = 0>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs g) {
-    static_assert(!KTAIL || (!RAGGED && !P::SPLIT_A && !P::SPLIT_B), "the K tail form serves the unsplit policies");
+    static_assert(KTAIL == 0 || (!RAGGED && !P::SPLIT_A && !P::SPLIT_B), "the K tail form serves the unsplit policies");
     using Cfg = RsCfg<P, BM, BN, WAVES_M, WAVES_N>;
     constexpr int BK = Cfg::BK, KSTEPS = Cfg::KSTEPS;
     extern __shared__ __attribute__((aligned(16))) int8_t smem[];
@@ -250,8 +253,11 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
     // policies, short of registers, reloaded address pairs from scratch inside the loop, each reload waiting for every
     // load in flight.
     constexpr int A_TILE_BYTES = P::SPLIT_A ? 2 * BK : BK;
-    const int64_t a_range = static_cast<int64_t>(g.M - 1 - m0) * g.lda + (KTAIL ? g.K : static_cast<int64_t>(g.K / BK) * A_TILE_BYTES);
-    const int64_t b_range = static_cast<int64_t>(g.N - 1 - n0) * g.ldb + (KTAIL ? g.K : static_cast<int64_t>(g.K / BK) * BK);
+    // KTAIL 2 reads the dword (A) or chunk (B) that straddles K whole: inside the row's pitch, which the host has checked
+    const int64_t a_range = static_cast<int64_t>(g.M - 1 - m0) * g.lda +
+                            (KTAIL == 2 ? (g.K + 3) / 4 * 4 : KTAIL ? g.K : static_cast<int64_t>(g.K / BK) * A_TILE_BYTES);
+    const int64_t b_range = static_cast<int64_t>(g.N - 1 - n0) * g.ldb +
+                            (KTAIL == 2 ? (g.K + 15) / 16 * 16 : KTAIL ? g.K : static_cast<int64_t>(g.K / BK) * BK);
     const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<int8_t*>(Abase), 0, static_cast<int>(a_range < 0x7fffffff ? a_range : 0x7fffffff), 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrc_b =
@@ -260,11 +266,18 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
     const int voff_a = lrow * static_cast<int>(g.lda) + lchunk * (P::SPLIT_A ? 32 : 16);
     const int voff_b = lrow * static_cast<int>(g.ldb) + lchunk * 16;
     auto load_one = [&](int kt, int idx) {
-        if constexpr (KTAIL) {
+        if constexpr (KTAIL != 0) {
             constexpr unsigned NOWHERE = 0xfffffff0u;  // beyond every descriptor: reads as zero
             const bool inside = kt * BK + lchunk * 16 < g.K;
             if (idx < Cfg::A_LOADS) {
                 const unsigned off = voff_a + kt * BK + idx * Cfg::ROWS_PER_PASS * static_cast<int>(g.lda);
+                if constexpr (KTAIL == 2) {
+                    const int rem = g.K - (kt * BK + lchunk * 16);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        ra[idx][j] = static_cast<int>(__builtin_amdgcn_raw_buffer_load_b32(rsrc_a, 4 * j < rem ? off + 4 * j : NOWHERE, 0, 0));
+                    return;
+                }
                 ra[idx] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, inside ? off : NOWHERE, 0, 0));
             } else {
                 const unsigned off = voff_b + kt * BK + (idx - Cfg::A_LOADS) * Cfg::ROWS_PER_PASS * static_cast<int>(g.ldb);
@@ -300,7 +313,21 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
             rb[idx - Cfg::A_LOADS] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, voff_b, kt * BK + pass, 0));
         }
     };
+    const int ktiles = (RAGGED || KTAIL != 0) ? (g.K + BK - 1) / BK : g.K / BK;
+    int stage_kt = 0;  // the K tile that the staging registers hold (KTAIL 2: its last tile is cleared past K)
     auto store_one = [&](int8_t* stage, int idx) {
+        if constexpr (KTAIL == 2) {
+            if (stage_kt == ktiles - 1) {  // workgroup-uniform, and no load inside
+                const int rem = g.K - (stage_kt * BK + lchunk * 16);
+                v4i& r = idx < Cfg::A_LOADS ? ra[idx] : rb[idx - Cfg::A_LOADS];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int v = rem - 4 * j;  // bytes of this dword that belong to K
+                    if (v <= 0) r[j] = 0;
+                    else if (v < 4) r[j] &= static_cast<int>((1u << (8 * v)) - 1u);
+                }
+            }
+        }
         if constexpr (P::SPLIT_A) {
             if (idx < Cfg::A_LOADS && (idx & 1) == 0)
                 P::split_a(ra[idx], ra[idx + 1 < Cfg::A_LOADS ? idx + 1 : idx], extra, idx >> 1, split_live);
@@ -312,7 +339,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
         else *reinterpret_cast<v4i*>(stage + BM * BK + st_off + (idx - Cfg::A_LOADS) * Cfg::ROWS_PER_PASS * BK) = rb[idx - Cfg::A_LOADS];
     };
 
-    const int ktiles = (RAGGED || KTAIL) ? (g.K + BK - 1) / BK : g.K / BK;
 #pragma unroll
     for (int i = 0; i < Cfg::LOADS; ++i) load_one(0, i);
 
@@ -412,6 +438,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
         int8_t* cur_base = smem + (kt & 1) * Cfg::STAGE_BYTES;
         int8_t* nxt_base = smem + ((kt + 1) & 1) * Cfg::STAGE_BYTES;
         split_live = kt + 1 < ktiles;
+        stage_kt = min(kt + 1, ktiles - 1);
         if constexpr (KSTEPS == 2) {
             // two 64-byte steps per K tile: step 0 carries all the memory work, the barrier sits between the two
             if (EARLY) {
@@ -457,7 +484,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
 }
 
 // Launches one workgroup per tile (padded to whole ranges for the 8 XCDs; surplus workgroups exit at once).
-template <class P, int BM, int BN, int WAVES_M, int WAVES_N, bool EARLY = false, bool RAGGED = false, bool KTAIL = false>
+template <class P, int BM, int BN, int WAVES_M, int WAVES_N, bool EARLY = false, bool RAGGED = false, int KTAIL = 0>
 static hipError_t launch_rs_policy(const GemmArgs& g, int batch, hipStream_t stream) {
     using Cfg = RsCfg<P, BM, BN, WAVES_M, WAVES_N>;
     auto kern = gemm_rs_kernel<P, BM, BN, WAVES_M, WAVES_N, EARLY, RAGGED, KTAIL>;
