@@ -902,9 +902,16 @@ static hipError_t launch_ragged(GemmArgs g, int batch, hipStream_t stream) {
     // from two K tiles on, the pipelined kernel is ahead (25 us against 31 us at 8192 x 1024 x 1008): with descriptor loads
     // and no branches where the activations' rows are 4-byte aligned and the other operand's 16-byte aligned rows hold
     // K rounded up to 16 (packed weights always do) ...
-    if (g.K >= 256 && g.ragged_a <= 1 && g.ragged_b == 0 && !g.trans_a_es && static_cast<int64_t>(g.lda) >= (g.K + 3) / 4 * 4)
+    if (g.K >= 256 && g.ragged_a <= 1 && g.ragged_b == 0 && !g.trans_a_es && static_cast<int64_t>(g.lda) >= (g.K + 3) / 4 * 4) {
+        // (8-byte aligned rows, a pitch of 1000 bytes: two loads per chunk instead of four)
+        const bool by8 = g.lda % 8 == 0 && g.stride_a % 8 == 0 && (reinterpret_cast<uintptr_t>(g.A) & 7) == 0 &&
+                         static_cast<int64_t>(g.lda) >= (g.K + 7) / 8 * 8;
+        if (by8)
+            return g.a_unsigned ? launch_rs_policy<I8Policy<true>, 128, 128, 2, 2, false, false, 3>(g, batch, stream)
+                                : launch_rs_policy<I8Policy<false>, 128, 128, 2, 2, false, false, 3>(g, batch, stream);
         return g.a_unsigned ? launch_rs_policy<I8Policy<true>, 128, 128, 2, 2, false, false, 2>(g, batch, stream)
                             : launch_rs_policy<I8Policy<false>, 128, 128, 2, 2, false, false, 2>(g, batch, stream);
+    }
     // ... else with chunk loads that respect the row ends
     if (g.K >= 256)
         return g.a_unsigned ? launch_rs_policy<I8Policy<true>, 128, 128, 2, 2, false, true>(g, batch, stream)

@@ -201,7 +201,8 @@ static inline int ragged_mode(const void* p, int64_t ld, int64_t stride, int64_t
 // stay exact, which the ragged loads' branches do not allow (8192 x 784 -> 128: 17 us ragged, 9 us this way).
 // KTAIL 2: the same for K off the 16-byte grid: rows of A 4-byte aligned (four dword loads per chunk, each inside K or
 // sent outside the descriptor), rows of B 16-byte aligned with a pitch that holds K rounded up to 16; the bytes past K
-// of the one dword or chunk that straddles it are cleared where the last K tile is staged.
+// of the one dword or chunk that straddles it are cleared where the last K tile is staged. KTAIL 3: the same with rows
+// of A 8-byte aligned, two 8-byte loads per chunk.
 template <class P, int BM, int BN, int WAVES_M, int WAVES_N, bool EARLY = false, bool RAGGED = false, int KTAIL = 0>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs g) {
     static_assert(KTAIL == 0 || (!RAGGED && !P::SPLIT_A && !P::SPLIT_B), "the K tail form serves the unsplit policies");
@@ -255,9 +256,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
     constexpr int A_TILE_BYTES = P::SPLIT_A ? 2 * BK : BK;
     // KTAIL 2 reads the dword (A) or chunk (B) that straddles K whole: inside the row's pitch, which the host has checked
     const int64_t a_range = static_cast<int64_t>(g.M - 1 - m0) * g.lda +
-                            (KTAIL == 2 ? (g.K + 3) / 4 * 4 : KTAIL ? g.K : static_cast<int64_t>(g.K / BK) * A_TILE_BYTES);
+                            (KTAIL == 3 ? (g.K + 7) / 8 * 8 : KTAIL == 2 ? (g.K + 3) / 4 * 4 : KTAIL ? g.K : static_cast<int64_t>(g.K / BK) * A_TILE_BYTES);
     const int64_t b_range = static_cast<int64_t>(g.N - 1 - n0) * g.ldb +
-                            (KTAIL == 2 ? (g.K + 15) / 16 * 16 : KTAIL ? g.K : static_cast<int64_t>(g.K / BK) * BK);
+                            (KTAIL >= 2 ? (g.K + 15) / 16 * 16 : KTAIL ? g.K : static_cast<int64_t>(g.K / BK) * BK);
     const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<int8_t*>(Abase), 0, static_cast<int>(a_range < 0x7fffffff ? a_range : 0x7fffffff), 0x00020000);
     const __amdgpu_buffer_rsrc_t rsrc_b =
@@ -271,6 +272,17 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
             const bool inside = kt * BK + lchunk * 16 < g.K;
             if (idx < Cfg::A_LOADS) {
                 const unsigned off = voff_a + kt * BK + idx * Cfg::ROWS_PER_PASS * static_cast<int>(g.lda);
+                if constexpr (KTAIL == 3) {
+                    typedef unsigned v2u_t __attribute__((ext_vector_type(2)));
+                    const int rem = g.K - (kt * BK + lchunk * 16);
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        const v2u_t w = __builtin_amdgcn_raw_buffer_load_b64(rsrc_a, 8 * j < rem ? off + 8 * j : NOWHERE, 0, 0);
+                        ra[idx][2 * j] = static_cast<int>(w[0]);
+                        ra[idx][2 * j + 1] = static_cast<int>(w[1]);
+                    }
+                    return;
+                }
                 if constexpr (KTAIL == 2) {
                     const int rem = g.K - (kt * BK + lchunk * 16);
 #pragma unroll
@@ -316,7 +328,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void gemm_rs_kernel(GemmArgs
     const int ktiles = (RAGGED || KTAIL != 0) ? (g.K + BK - 1) / BK : g.K / BK;
     int stage_kt = 0;  // the K tile that the staging registers hold (KTAIL 2: its last tile is cleared past K)
     auto store_one = [&](int8_t* stage, int idx) {
-        if constexpr (KTAIL == 2) {
+        if constexpr (KTAIL >= 2) {
             if (stage_kt == ktiles - 1) {  // workgroup-uniform, and no load inside
                 const int rem = g.K - (stage_kt * BK + lchunk * 16);
                 v4i& r = idx < Cfg::A_LOADS ? ra[idx] : rb[idx - Cfg::A_LOADS];

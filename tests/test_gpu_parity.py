@@ -637,7 +637,9 @@ def test_matmul_int16_left_operand(ops, oracle, shape, trans_b, b_dtype):
 
 
 RAGGED = [(300, 200, 100, 0, 0), (257, 130, 1000, 0, 0), (129, 70, 37, 3, 1), (64, 33, 7, 5, 3), (500, 256, 1030, 2, 2),
-          (1, 1, 1, 0, 0), (140, 128, 200, 56, 8)]
+          (1, 1, 1, 0, 0), (140, 128, 200, 56, 8),
+          # from two K tiles on, rows 4- or 8-byte aligned: descriptor loads by dwords / by 8 bytes, the bytes past K cleared
+          (300, 144, 1004, 0, 0), (200, 256, 300, 4, 4), (130, 200, 1001, 7, 0), (260, 130, 2042, 6, 8)]
 
 
 @pytest.mark.parametrize('case', RAGGED)
